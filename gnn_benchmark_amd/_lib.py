@@ -1,0 +1,103 @@
+"""ctypes binding of ``csrc/libgnnagg.so`` (the C ABI declared in ``include/gnn_agg.h``).
+
+There is no fallback: if the library has not been built, or a tensor is not on a HIP
+device, the callers in this package raise.
+"""
+import ctypes
+import os
+import subprocess
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_CSRC = os.path.join(_HERE, "csrc")
+LIB_PATH = os.path.join(_CSRC, "libgnnagg.so")
+
+OK, ERR_INVALID, ERR_HIP, ERR_UNSUPPORTED = 0, 1, 2, 3
+ABI_VERSION = 1
+
+EXPORTS = (
+    "gnnagg_abi_version",
+    "gnnagg_last_error",
+    "gnnagg_spmm_csr_f32",
+    "gnnagg_plan_create",
+    "gnnagg_plan_destroy",
+    "gnnagg_plan_spmm_f32",
+    "gnnagg_plan_info",
+    "gnnagg_plan_profile",
+    "gnnagg_plan_profile_read",
+    "gnnagg_csr_transpose",
+    "gnnagg_coo_to_csr",
+    "gnnagg_gather_rows_f32",
+)
+
+_lib = None
+
+
+class GnnAggError(RuntimeError):
+    """A libgnnagg entry point returned an error code."""
+
+    def __init__(self, code: int, message: str):
+        super().__init__(f"libgnnagg error {code}: {message}")
+        self.code = code
+
+
+def build(verbose: bool = False) -> str:
+    """Compile libgnnagg.so for gfx950 with hipcc (cross-compiles without a GPU)."""
+    out = None if verbose else subprocess.DEVNULL
+    subprocess.check_call(["make", "-C", _CSRC, "-B", "-j4", "libgnnagg.so"], stdout=out, stderr=out)
+    return LIB_PATH
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it first (python -c 'import __graft_entry__ as g; g.build()' "
+            "or make -C gnn_benchmark_amd/csrc). There is no CPU fallback.")
+    L = ctypes.CDLL(LIB_PATH)
+    vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+    L.gnnagg_abi_version.restype = i32
+    L.gnnagg_abi_version.argtypes = []
+    L.gnnagg_last_error.restype = ctypes.c_char_p
+    L.gnnagg_last_error.argtypes = []
+    L.gnnagg_spmm_csr_f32.restype = i32
+    L.gnnagg_spmm_csr_f32.argtypes = [vp, vp, vp, vp, vp, i64, i64, vp]
+    L.gnnagg_plan_create.restype = i32
+    L.gnnagg_plan_create.argtypes = [vp, vp, i64, i64, i64, vp, ctypes.POINTER(vp)]
+    L.gnnagg_plan_destroy.restype = i32
+    L.gnnagg_plan_destroy.argtypes = [vp]
+    L.gnnagg_plan_spmm_f32.restype = i32
+    L.gnnagg_plan_spmm_f32.argtypes = [vp, vp, vp, vp, i64, i32, vp]
+    L.gnnagg_plan_info.restype = i32
+    L.gnnagg_plan_info.argtypes = [vp, ctypes.POINTER(i64)]
+    L.gnnagg_plan_profile.restype = i32
+    L.gnnagg_plan_profile.argtypes = [vp, i32]
+    L.gnnagg_plan_profile_read.restype = i32
+    L.gnnagg_plan_profile_read.argtypes = [vp, ctypes.POINTER(ctypes.c_double)]
+    L.gnnagg_csr_transpose.restype = i32
+    L.gnnagg_csr_transpose.argtypes = [vp, vp, vp, i64, i64, i64, vp, vp, vp, vp]
+    L.gnnagg_coo_to_csr.restype = i32
+    L.gnnagg_coo_to_csr.argtypes = [vp, vp, vp, i64, i64, i64, vp, vp, vp, vp]
+    L.gnnagg_gather_rows_f32.restype = i32
+    L.gnnagg_gather_rows_f32.argtypes = [vp, vp, vp, i64, i64, vp]
+    if L.gnnagg_abi_version() != ABI_VERSION:
+        raise RuntimeError("libgnnagg.so was built from a different include/gnn_agg.h; rebuild it")
+    _lib = L
+    return L
+
+
+def check(rc: int) -> None:
+    if rc != OK:
+        raise GnnAggError(rc, lib().gnnagg_last_error().decode("utf-8", "replace"))
+
+
+def ptr(t):
+    """Device address of a tensor (None -> NULL)."""
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def current_stream(device):
+    import torch
+
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)

@@ -1,0 +1,128 @@
+"""The aggregation autograd.Function of one graph partition.
+
+Reference: self_benchmark/a64fx/model/layers/aggregator.py:15-119 (forward), :121-208
+(backward).  Same ``apply`` signature ``(graph, local_nodes_feat, layer, num_bits,
+is_pre_delay, is_training)`` and the same backward arity ``(None, grad, None, None,
+None, None)``.
+
+Per direction: (1) fill the outgoing boundary buffer -- pre-aggregation SpMM or row
+gather; (2) hand the buffers to the exchange; (3) local SpMM; (4) wait for the
+exchange; (5) accumulate the received halo rows into the same output
+(post-aggregation).  Backward runs the same pipeline on the transposed matrices with
+the two buffers swapping roles (aggregator.py:141, :186).
+
+What differs from the reference, on purpose:
+* The boundary all-to-all (communicator.py:55-109) is ``graph.exchange``, a callable
+  ``exchange(comm_splits, comm_buf, tag, direction) -> handle | None``: on "forward" it
+  must leave the received halo rows in ``comm_buf.recv_buf``, on "backward" the received
+  gradient rows in ``comm_buf.send_buf``.  A returned handle's ``wait()`` is called after
+  the local SpMM, where the reference waits (aggregator.py:78, :175).  ``exchange is
+  None`` is the single-rank world: pre/post steps are skipped (aggregator.py:47, :100).
+* No process group, timers or quantiser singletons are touched.
+* ``torch.zeros`` + accumulate (aggregator.py:67-70, :167-170) and ``zero_()`` +
+  accumulate (:44-49, :144-149) run as one overwriting SpMM; the values are identical
+  because an FMA chain started from a stored 0 equals one started from a register 0.
+* The backward ``index_add_`` (:197-199) runs as a deterministic SpMM with the
+  selection matrix of ``idx_nodes_send_to_others``.
+"""
+import torch
+
+from . import _lib
+from .spmm_kernel import SPMM_backward, SPMM_forward
+
+
+def _gather_rows(src: torch.Tensor, index: torch.Tensor, out: torch.Tensor) -> None:
+    # torch.index_select(local_nodes_feat, 0, idx, out=send_buf)   (aggregator.py:51)
+    if not (src.is_cuda and index.is_cuda and out.is_cuda):
+        raise RuntimeError("gather operands must be GPU (HIP) tensors; there is no CPU path")
+    if src.dtype != torch.float32 or out.dtype != torch.float32 or index.dtype != torch.int64:
+        raise RuntimeError("Input mismatch: gather needs float32 rows and int64 indices")
+    if out.size(0) != index.numel() or out.size(1) != src.size(1) or not out.is_contiguous():
+        raise RuntimeError("Input mismatch: gather output shape")
+    src = src.contiguous()
+    with torch.cuda.device(src.device):
+        _lib.check(_lib.lib().gnnagg_gather_rows_f32(_lib.ptr(src), _lib.ptr(index), _lib.ptr(out), index.numel(),
+                                                     src.size(1), _lib.current_stream(src.device)))
+
+
+def _check_bits(num_bits: int) -> None:
+    if num_bits not in (32, 16):
+        raise NotImplementedError("quantised boundary exchange (num_bits=%r) is outside this build" % (num_bits,))
+
+
+class Aggregator(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, graph, local_nodes_feat, layer, num_bits: int, is_pre_delay: bool, is_training: bool):
+        _check_bits(num_bits)
+        ctx.graph = graph
+        ctx.num_bits = num_bits
+        ctx.is_pre_delay = is_pre_delay
+        ctx.layer = layer
+
+        feat_len = local_nodes_feat.size(-1)
+        local_nodes_feat = local_nodes_feat.contiguous()
+        graph.comm_buf.resize_buffer(graph.comm_splits, feat_len, num_bits)
+        exchange = getattr(graph, "exchange", None)
+        comm_handle = None
+        send_buf = graph.comm_buf.send_buf
+
+        if exchange is not None:
+            if is_pre_delay:  # pre-aggregation: send_buf = A_to @ X
+                SPMM_forward(graph.adj_t_pre_post_aggr_to, local_nodes_feat, send_buf, accumulate=False)
+            else:  # raw boundary rows
+                _gather_rows(local_nodes_feat, graph.idx_nodes_send_to_others, send_buf)
+            comm_handle = exchange(graph.comm_splits, graph.comm_buf, f"forward{layer}", "forward")
+
+        out = torch.empty([graph.local_adj_t.sparse_size(0), feat_len], dtype=torch.float32,
+                          device=local_nodes_feat.device)
+        SPMM_forward(graph.local_adj_t, local_nodes_feat, out, accumulate=False)
+
+        if comm_handle is not None:
+            comm_handle.wait()
+
+        remote_nodes_feat = graph.comm_buf.recv_buf
+        if exchange is not None and remote_nodes_feat.size(0) != 0:
+            if is_pre_delay:  # post-aggregation
+                SPMM_forward(graph.adj_t_pre_post_aggr_from, remote_nodes_feat, out)
+            else:
+                SPMM_forward(graph.remote_adj_t, remote_nodes_feat, out)
+        return out
+
+    @staticmethod
+    def backward(ctx, local_out_grad):
+        graph = ctx.graph
+        num_bits = ctx.num_bits
+        is_pre_delay = ctx.is_pre_delay
+        layer = f"backward{ctx.layer}"
+
+        local_out_grad = local_out_grad.contiguous()
+        feat_len = local_out_grad.size(-1)
+        graph.comm_buf.resize_buffer(graph.comm_splits, feat_len, num_bits)
+        exchange = getattr(graph, "exchange", None)
+
+        # the receive buffer carries the outgoing halo gradients on the way back
+        remote_nodes_grad_buf = graph.comm_buf.recv_buf
+        if remote_nodes_grad_buf.size(0) != 0:
+            if is_pre_delay:
+                SPMM_backward(graph.adj_t_pre_post_aggr_from, local_out_grad, remote_nodes_grad_buf, accumulate=False)
+            else:
+                SPMM_backward(graph.remote_adj_t, local_out_grad, remote_nodes_grad_buf, accumulate=False)
+
+        comm_handle = None
+        if exchange is not None:
+            comm_handle = exchange(graph.comm_splits, graph.comm_buf, layer, "backward")
+
+        local_nodes_grad = torch.empty([graph.local_adj_t.sparse_size(-1), feat_len], dtype=torch.float32,
+                                       device=local_out_grad.device)
+        SPMM_backward(graph.local_adj_t, local_out_grad, local_nodes_grad, accumulate=False)
+
+        if comm_handle is not None:
+            comm_handle.wait()
+
+        local_nodes_grad_buf = graph.comm_buf.send_buf
+        if exchange is not None and local_nodes_grad_buf.size(0) != 0:
+            if is_pre_delay:
+                SPMM_backward(graph.adj_t_pre_post_aggr_to, local_nodes_grad_buf, local_nodes_grad)
+            else:
+                SPMM_forward(graph.send_scatter_adj_t(), local_nodes_grad_buf, local_nodes_grad)
+        return None, local_nodes_grad, None, None, None, None

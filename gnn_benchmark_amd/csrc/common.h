@@ -1,0 +1,77 @@
+// Shared host-side helpers of libgnnagg.so (error reporting, HIP call checking,
+// owned device buffers).  gfx950 only; no other backend is supported.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <string>
+
+#include "gnn_agg.h"
+
+namespace gnnagg {
+
+std::string &last_error_slot();
+
+inline int fail(int code, const char *fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    last_error_slot() = buf;
+    return code;
+}
+
+#define GNNAGG_HIP(expr)                                                                           \
+    do {                                                                                           \
+        hipError_t e__ = (expr);                                                                   \
+        if (e__ != hipSuccess)                                                                     \
+            return ::gnnagg::fail(GNNAGG_ERR_HIP, "%s failed: %s (%s:%d)", #expr,                  \
+                                  hipGetErrorString(e__), __FILE__, __LINE__);                     \
+    } while (0)
+
+#define GNNAGG_REQUIRE(cond, ...)                                                                  \
+    do {                                                                                           \
+        if (!(cond)) return ::gnnagg::fail(GNNAGG_ERR_INVALID, __VA_ARGS__);                       \
+    } while (0)
+
+// Device allocation released on scope exit (setup-time paths only).
+template <typename T>
+struct DevBuf {
+    T *p = nullptr;
+    size_t n = 0;
+    DevBuf() = default;
+    DevBuf(const DevBuf &) = delete;
+    DevBuf &operator=(const DevBuf &) = delete;
+    ~DevBuf() { reset(); }
+    hipError_t alloc(size_t count) {
+        reset();
+        n = count;
+        if (count == 0) return hipSuccess;
+        return hipMalloc(reinterpret_cast<void **>(&p), count * sizeof(T));
+    }
+    void reset() {
+        if (p) (void)hipFree(p);
+        p = nullptr;
+        n = 0;
+    }
+    T *release() {
+        T *r = p;
+        p = nullptr;
+        n = 0;
+        return r;
+    }
+};
+
+inline int ceil_log2_u64(uint64_t x) {  // smallest b with 2^b >= x (x >= 1)
+    int b = 0;
+    while ((uint64_t(1) << b) < x) ++b;
+    return b;
+}
+
+inline unsigned grid_for(int64_t n, int block) { return (unsigned)((n + block - 1) / block); }
+
+}  // namespace gnnagg

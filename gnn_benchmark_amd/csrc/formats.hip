@@ -1,0 +1,227 @@
+// Sparse-format construction on the device (setup-time): COO -> CSR, CSR -> transposed
+// CSR, and the boundary-row gather.  gfx950 only.
+#include <hipcub/hipcub.hpp>
+
+#include <algorithm>
+
+#include "common.h"
+
+namespace gnnagg {
+namespace {
+
+// key = row << col_bits | col ; idx = position
+__global__ __launch_bounds__(256) void pack_keys_kernel(const int64_t *__restrict__ row,
+                                                        const int64_t *__restrict__ col, int64_t nnz, int64_t rows,
+                                                        int64_t cols, int col_bits, uint64_t *__restrict__ key,
+                                                        uint32_t *__restrict__ idx, unsigned int *__restrict__ bad) {
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= nnz) return;
+    const int64_t r = row[e], c = col[e];
+    if (r < 0 || r >= rows || c < 0 || c >= cols) {
+        atomicOr(bad, 1u);
+        key[e] = 0;
+    } else {
+        key[e] = ((uint64_t)r << col_bits) | (uint64_t)c;
+    }
+    idx[e] = (uint32_t)e;
+}
+
+__global__ __launch_bounds__(256) void unpack_sorted_kernel(const uint64_t *__restrict__ key,
+                                                            const uint32_t *__restrict__ idx,
+                                                            const float *__restrict__ value, int64_t nnz,
+                                                            int col_bits, int64_t *__restrict__ col_out,
+                                                            float *__restrict__ value_out) {
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= nnz) return;
+    col_out[e] = (int64_t)(key[e] & ((uint64_t(1) << col_bits) - 1));
+    if (value_out) value_out[e] = value[idx[e]];
+}
+
+// ptr[r] = number of sorted keys whose major index (key >> shift) is < r, r in [0, n]
+__global__ __launch_bounds__(256) void major_ptr_kernel(const uint64_t *__restrict__ key, int64_t nnz, int shift,
+                                                        int64_t n, int64_t *__restrict__ ptr) {
+    const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (r > n) return;
+    int64_t lo = 0, hi = nnz;  // first position with major >= r
+    while (lo < hi) {
+        const int64_t mid = (lo + hi) >> 1;
+        if ((int64_t)(key[mid] >> shift) < r) lo = mid + 1; else hi = mid;
+    }
+    ptr[r] = lo;
+}
+
+// key = col << row_bits | row for every stored element of a CSR matrix (row found by
+// binary search in rowptr); idx = position.
+__global__ __launch_bounds__(256) void pack_transposed_keys_kernel(const int64_t *__restrict__ rowptr,
+                                                                   const int64_t *__restrict__ col, int64_t rows,
+                                                                   int64_t cols, int64_t nnz, int row_bits,
+                                                                   uint64_t *__restrict__ key,
+                                                                   uint32_t *__restrict__ idx,
+                                                                   unsigned int *__restrict__ bad) {
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= nnz) return;
+    int64_t lo = 0, hi = rows;  // last row with rowptr[row] <= e
+    while (hi - lo > 1) {
+        const int64_t mid = (lo + hi) >> 1;
+        if (rowptr[mid] <= e) lo = mid; else hi = mid;
+    }
+    const int64_t c = col[e];
+    if (c < 0 || c >= cols) {
+        atomicOr(bad, 1u);
+        key[e] = 0;
+    } else {
+        key[e] = ((uint64_t)c << row_bits) | (uint64_t)lo;
+    }
+    idx[e] = (uint32_t)e;
+}
+
+template <int VEC>
+__global__ __launch_bounds__(256) void gather_rows_kernel(const float *__restrict__ src,
+                                                          const int64_t *__restrict__ index,
+                                                          float *__restrict__ out, int64_t n_index, int feat_vec) {
+    typedef float vec_t __attribute__((ext_vector_type(VEC)));
+    // one wavefront per output row, lanes along the feature dimension
+    const int64_t i = (int64_t)blockIdx.x * 4 + ((int)threadIdx.x >> 6);
+    if (i >= n_index) return;
+    const int lane = (int)threadIdx.x & 63;
+    const size_t r = (size_t)index[i];
+    const vec_t *s = reinterpret_cast<const vec_t *>(src) + r * (size_t)feat_vec;
+    vec_t *d = reinterpret_cast<vec_t *>(out) + (size_t)i * (size_t)feat_vec;
+    for (int f = lane; f < feat_vec; f += 64) d[f] = s[f];
+}
+
+int sort_keys(uint64_t *key_in, uint64_t *key_out, uint32_t *idx_in, uint32_t *idx_out, int64_t n, int bits,
+              hipStream_t st) {
+    size_t tmp_bytes = 0;
+    GNNAGG_HIP(hipcub::DeviceRadixSort::SortPairs(nullptr, tmp_bytes, key_in, key_out, idx_in, idx_out, (int)n, 0,
+                                                  bits, st));
+    DevBuf<char> tmp;
+    GNNAGG_HIP(tmp.alloc(std::max<size_t>(tmp_bytes, 1)));
+    GNNAGG_HIP(hipcub::DeviceRadixSort::SortPairs(tmp.p, tmp_bytes, key_in, key_out, idx_in, idx_out, (int)n, 0, bits,
+                                                  st));
+    GNNAGG_HIP(hipStreamSynchronize(st));
+    return GNNAGG_OK;
+}
+
+}  // namespace
+}  // namespace gnnagg
+
+using namespace gnnagg;
+
+static int check_format_sizes(int64_t rows, int64_t cols, int64_t nnz) {
+    GNNAGG_REQUIRE(rows >= 0 && cols >= 0 && nnz >= 0, "negative size");
+    if (rows >= (int64_t(1) << 31) - 1 || cols >= (int64_t(1) << 31) - 1 || nnz >= (int64_t(1) << 31) - 1)
+        return fail(GNNAGG_ERR_UNSUPPORTED, "format limits: rows, cols, nnz < 2^31-1 (got %lld, %lld, %lld)",
+                    (long long)rows, (long long)cols, (long long)nnz);
+    return GNNAGG_OK;
+}
+
+extern "C" int gnnagg_coo_to_csr(const int64_t *row, const int64_t *col, const float *value, int64_t nnz, int64_t rows,
+                                 int64_t cols, int64_t *rowptr, int64_t *col_out, float *value_out, void *stream) {
+    if (int rc = check_format_sizes(rows, cols, nnz)) return rc;
+    GNNAGG_REQUIRE(rowptr, "null rowptr");
+    GNNAGG_REQUIRE(nnz == 0 || (row && col && col_out), "null row/col/col_out");
+    GNNAGG_REQUIRE((value == nullptr) == (value_out == nullptr), "value and value_out must both be given or both be null");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (nnz == 0) {
+        GNNAGG_HIP(hipMemsetAsync(rowptr, 0, sizeof(int64_t) * (size_t)(rows + 1), st));
+        GNNAGG_HIP(hipStreamSynchronize(st));
+        return GNNAGG_OK;
+    }
+    const int col_bits = std::max(1, ceil_log2_u64((uint64_t)std::max<int64_t>(cols, 1)));
+    const int row_bits = std::max(1, ceil_log2_u64((uint64_t)std::max<int64_t>(rows, 1)));
+    DevBuf<uint64_t> key_in, key_out;
+    DevBuf<uint32_t> idx_in, idx_out;
+    DevBuf<unsigned int> bad;
+    GNNAGG_HIP(key_in.alloc((size_t)nnz));
+    GNNAGG_HIP(key_out.alloc((size_t)nnz));
+    GNNAGG_HIP(idx_in.alloc((size_t)nnz));
+    GNNAGG_HIP(idx_out.alloc((size_t)nnz));
+    GNNAGG_HIP(bad.alloc(1));
+    GNNAGG_HIP(hipMemsetAsync(bad.p, 0, sizeof(unsigned int), st));
+    hipLaunchKernelGGL(pack_keys_kernel, dim3(grid_for(nnz, 256)), dim3(256), 0, st, row, col, nnz, rows, cols, col_bits,
+                       key_in.p, idx_in.p, bad.p);
+    GNNAGG_HIP(hipGetLastError());
+    unsigned int h_bad = 0;
+    GNNAGG_HIP(hipMemcpyAsync(&h_bad, bad.p, sizeof(unsigned int), hipMemcpyDeviceToHost, st));
+    GNNAGG_HIP(hipStreamSynchronize(st));
+    GNNAGG_REQUIRE(!h_bad, "a row/col index lies outside [0,%lld) x [0,%lld)", (long long)rows, (long long)cols);
+    if (int rc = sort_keys(key_in.p, key_out.p, idx_in.p, idx_out.p, nnz, col_bits + row_bits, st)) return rc;
+    hipLaunchKernelGGL(unpack_sorted_kernel, dim3(grid_for(nnz, 256)), dim3(256), 0, st, key_out.p, idx_out.p, value,
+                       nnz, col_bits, col_out, value_out);
+    GNNAGG_HIP(hipGetLastError());
+    hipLaunchKernelGGL(major_ptr_kernel, dim3(grid_for(rows + 1, 256)), dim3(256), 0, st, key_out.p, nnz, col_bits, rows,
+                       rowptr);
+    GNNAGG_HIP(hipGetLastError());
+    GNNAGG_HIP(hipStreamSynchronize(st));
+    return GNNAGG_OK;
+}
+
+extern "C" int gnnagg_csr_transpose(const int64_t *rowptr, const int64_t *col, const float *value, int64_t rows,
+                                    int64_t cols, int64_t nnz, int64_t *colptr, int64_t *row_t, float *value_t,
+                                    void *stream) {
+    if (int rc = check_format_sizes(rows, cols, nnz)) return rc;
+    GNNAGG_REQUIRE(rowptr && colptr, "null rowptr/colptr");
+    GNNAGG_REQUIRE(nnz == 0 || (col && row_t), "null col/row_t");
+    GNNAGG_REQUIRE((value == nullptr) == (value_t == nullptr), "value and value_t must both be given or both be null");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (nnz == 0) {
+        GNNAGG_HIP(hipMemsetAsync(colptr, 0, sizeof(int64_t) * (size_t)(cols + 1), st));
+        GNNAGG_HIP(hipStreamSynchronize(st));
+        return GNNAGG_OK;
+    }
+    int64_t ends[2] = {0, 0};
+    GNNAGG_HIP(hipMemcpyAsync(&ends[0], rowptr, sizeof(int64_t), hipMemcpyDeviceToHost, st));
+    GNNAGG_HIP(hipMemcpyAsync(&ends[1], rowptr + rows, sizeof(int64_t), hipMemcpyDeviceToHost, st));
+    GNNAGG_HIP(hipStreamSynchronize(st));
+    GNNAGG_REQUIRE(ends[0] == 0 && ends[1] == nnz, "rowptr[0]=%lld, rowptr[rows]=%lld do not match nnz=%lld",
+                   (long long)ends[0], (long long)ends[1], (long long)nnz);
+    const int col_bits = std::max(1, ceil_log2_u64((uint64_t)std::max<int64_t>(cols, 1)));
+    const int row_bits = std::max(1, ceil_log2_u64((uint64_t)std::max<int64_t>(rows, 1)));
+    DevBuf<uint64_t> key_in, key_out;
+    DevBuf<uint32_t> idx_in, idx_out;
+    DevBuf<unsigned int> bad;
+    GNNAGG_HIP(key_in.alloc((size_t)nnz));
+    GNNAGG_HIP(key_out.alloc((size_t)nnz));
+    GNNAGG_HIP(idx_in.alloc((size_t)nnz));
+    GNNAGG_HIP(idx_out.alloc((size_t)nnz));
+    GNNAGG_HIP(bad.alloc(1));
+    GNNAGG_HIP(hipMemsetAsync(bad.p, 0, sizeof(unsigned int), st));
+    hipLaunchKernelGGL(pack_transposed_keys_kernel, dim3(grid_for(nnz, 256)), dim3(256), 0, st, rowptr, col, rows, cols,
+                       nnz, row_bits, key_in.p, idx_in.p, bad.p);
+    GNNAGG_HIP(hipGetLastError());
+    unsigned int h_bad = 0;
+    GNNAGG_HIP(hipMemcpyAsync(&h_bad, bad.p, sizeof(unsigned int), hipMemcpyDeviceToHost, st));
+    GNNAGG_HIP(hipStreamSynchronize(st));
+    GNNAGG_REQUIRE(!h_bad, "a column index lies outside [0,%lld)", (long long)cols);
+    // (col, row) keys are unique per stored position up to repeated entries; the radix
+    // sort is stable, so repeated (row, col) pairs keep their CSR order.
+    if (int rc = sort_keys(key_in.p, key_out.p, idx_in.p, idx_out.p, nnz, col_bits + row_bits, st)) return rc;
+    hipLaunchKernelGGL(unpack_sorted_kernel, dim3(grid_for(nnz, 256)), dim3(256), 0, st, key_out.p, idx_out.p, value,
+                       nnz, row_bits, row_t, value_t);
+    GNNAGG_HIP(hipGetLastError());
+    hipLaunchKernelGGL(major_ptr_kernel, dim3(grid_for(cols + 1, 256)), dim3(256), 0, st, key_out.p, nnz, row_bits, cols,
+                       colptr);
+    GNNAGG_HIP(hipGetLastError());
+    GNNAGG_HIP(hipStreamSynchronize(st));
+    return GNNAGG_OK;
+}
+
+extern "C" int gnnagg_gather_rows_f32(const float *src, const int64_t *index, float *out, int64_t n_index, int64_t feat,
+                                      void *stream) {
+    GNNAGG_REQUIRE(n_index >= 0 && feat >= 0, "negative size");
+    if (n_index == 0 || feat == 0) return GNNAGG_OK;
+    GNNAGG_REQUIRE(src && index && out, "null src/index/out");
+    if (feat > (1 << 20)) return fail(GNNAGG_ERR_UNSUPPORTED, "feature width %lld above 2^20", (long long)feat);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(out);
+    const unsigned grid = grid_for(n_index, 4);
+    if (feat % 4 == 0 && bits % 16 == 0)
+        hipLaunchKernelGGL(gather_rows_kernel<4>, dim3(grid), dim3(256), 0, st, src, index, out, n_index, (int)(feat / 4));
+    else if (feat % 2 == 0 && bits % 8 == 0)
+        hipLaunchKernelGGL(gather_rows_kernel<2>, dim3(grid), dim3(256), 0, st, src, index, out, n_index, (int)(feat / 2));
+    else
+        hipLaunchKernelGGL(gather_rows_kernel<1>, dim3(grid), dim3(256), 0, st, src, index, out, n_index, (int)feat);
+    GNNAGG_HIP(hipGetLastError());
+    return GNNAGG_OK;
+}

@@ -1,0 +1,282 @@
+// Device kernels of the CSR SpMM (out (+)= A @ X, fp32) for gfx950.
+//
+// Work decomposition.  A "task" is one sparse row, or one fixed-length segment of a
+// long row.  A wavefront (64 lanes) is cut into groups of LPR lanes; one group owns one
+// task at a time.  Inside a group the lanes lie ALONG THE FEATURE DIMENSION: lane l
+// holds features [(k*LPR + l)*VEC, +VEC) for k < NCH, so every gather of a dense row
+// X[col,:] is one contiguous, fully coalesced run of LPR*VEC*4 bytes per k.
+//
+// Column indices / values of a task are fetched LPR at a time by the group's lanes
+// (one coalesced, non-temporal load each), then handed round lane by lane:
+// v_readlane for a whole-wave group (the index lands in a scalar register and the
+// row address is scalar+lane), ds_bpermute for sub-wavefront groups.  UNROLL gathers
+// are issued back to back before their FMAs so that each group keeps UNROLL*NCH
+// vector loads in flight -- the kernel is bound by HBM latency/bandwidth, not issue.
+//
+// Arithmetic.  A row is one fp32 FMA chain in CSR order starting from the value in
+// `out` (or 0), i.e. the recurrence of the reference's kernel_1xN
+// (self_benchmark/a64fx/model/ops/src/spmm.cpp:37-53).  Rows cut into segments add
+// their segment sums in segment order afterwards (fixed order, no atomics).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace gnnagg {
+
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+template <int VEC>
+struct FVec;
+
+template <>
+struct FVec<1> {
+    float d;
+    __device__ __forceinline__ static FVec zero() { return FVec{0.0f}; }
+    __device__ __forceinline__ static FVec load(const float *p) { return FVec{*p}; }
+    __device__ __forceinline__ void store(float *p) const { *p = d; }
+    __device__ __forceinline__ void fma(float a, const FVec &x) { d = __builtin_fmaf(a, x.d, d); }
+    __device__ __forceinline__ void add(const FVec &x) { d += x.d; }
+};
+
+template <>
+struct FVec<2> {
+    f32x2 d;
+    __device__ __forceinline__ static FVec zero() { return FVec{f32x2{0.0f, 0.0f}}; }
+    __device__ __forceinline__ static FVec load(const float *p) {
+        return FVec{*reinterpret_cast<const f32x2 *>(p)};
+    }
+    __device__ __forceinline__ void store(float *p) const { *reinterpret_cast<f32x2 *>(p) = d; }
+    __device__ __forceinline__ void fma(float a, const FVec &x) {
+        d.x = __builtin_fmaf(a, x.d.x, d.x);
+        d.y = __builtin_fmaf(a, x.d.y, d.y);
+    }
+    __device__ __forceinline__ void add(const FVec &x) {
+        d.x += x.d.x;
+        d.y += x.d.y;
+    }
+};
+
+template <>
+struct FVec<4> {
+    f32x4 d;
+    __device__ __forceinline__ static FVec zero() { return FVec{f32x4{0.0f, 0.0f, 0.0f, 0.0f}}; }
+    __device__ __forceinline__ static FVec load(const float *p) {
+        return FVec{*reinterpret_cast<const f32x4 *>(p)};
+    }
+    __device__ __forceinline__ void store(float *p) const { *reinterpret_cast<f32x4 *>(p) = d; }
+    __device__ __forceinline__ void fma(float a, const FVec &x) {
+        d.x = __builtin_fmaf(a, x.d.x, d.x);
+        d.y = __builtin_fmaf(a, x.d.y, d.y);
+        d.z = __builtin_fmaf(a, x.d.z, d.z);
+        d.w = __builtin_fmaf(a, x.d.w, d.w);
+    }
+    __device__ __forceinline__ void add(const FVec &x) {
+        d.x += x.d.x;
+        d.y += x.d.y;
+        d.z += x.d.z;
+        d.w += x.d.w;
+    }
+};
+
+// Lane-to-lane hand-over of a 32-bit word inside a group of LPR lanes.  For LPR == 64
+// the source lane index must be wave-uniform.
+template <int LPR>
+__device__ __forceinline__ int group_bcast(int v, int src) {
+    if constexpr (LPR == 64) {
+        return __builtin_amdgcn_readlane(v, src);
+    } else {
+        const int self = (int)__lane_id();
+        const int idx = (self & ~(LPR - 1)) | (src & (LPR - 1));
+        return __builtin_amdgcn_ds_bpermute(idx << 2, v);
+    }
+}
+
+template <int LPR>
+__device__ __forceinline__ int64_t group_bcast_idx(int64_t v, int src) {
+    const int lo = group_bcast<LPR>((int)(uint32_t)(v & 0xffffffffll), src);
+    const int hi = group_bcast<LPR>((int)(v >> 32), src);
+    return ((int64_t)hi << 32) | (uint32_t)lo;
+}
+template <int LPR>
+__device__ __forceinline__ int64_t group_bcast_idx(int32_t v, int src) {
+    return (int64_t)group_bcast<LPR>(v, src);
+}
+
+__device__ __forceinline__ int64_t uniform_i64(int64_t v) {
+    const int lo = __builtin_amdgcn_readfirstlane((int)(uint32_t)(v & 0xffffffffll));
+    const int hi = __builtin_amdgcn_readfirstlane((int)(v >> 32));
+    return ((int64_t)hi << 32) | (uint32_t)lo;
+}
+
+enum TaskMode : int {
+    kRowsNatural = 0,  // task t is row t
+    kRowsPermuted = 1, // task t is row perm[t]
+    kSegments = 2      // task t is nnz range [seg_start[t], +seg_len[t]) -> partial[t,:]
+};
+
+struct SpmmArgs {
+    const int64_t *rowptr;    // [rows+1]                      (row modes)
+    const int32_t *perm;      // [ntasks] row of task t        (kRowsPermuted)
+    const int64_t *seg_start; // [ntasks] first nnz of segment (kSegments)
+    const int32_t *seg_len;   // [ntasks] nnz in segment       (kSegments)
+    const void *col;          // IdxT [nnz]
+    const float *val;         // [nnz]
+    const float *x;           // dense operand [K, F]
+    float *dst;               // out [rows, F], or partial [ntasks, F] for kSegments
+    int64_t ntasks;
+    int feat;                 // F (row stride of x and dst, in floats)
+    int f_base;               // first feature handled by this launch
+    int accumulate;           // row modes: start from dst (1) or from 0 (0)
+    int tasks_per_block;
+};
+
+template <int VEC, int NCH>
+struct UnrollFor {
+    static constexpr int regs = VEC * NCH;
+    static constexpr int value = regs <= 4 ? 8 : (regs <= 8 ? 4 : (regs <= 20 ? 2 : 1));
+};
+
+template <int VEC, int LPR, int NCH, typename IdxT, int MODE>
+__global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
+    constexpr int GPB = 256 / LPR;  // groups per 256-thread block
+    constexpr int U = UnrollFor<VEC, NCH>::value;
+    typedef FVec<VEC> V;
+
+    const int lane = (int)threadIdx.x & 63;
+    const int lig = lane & (LPR - 1);  // lane in group
+    int group = (int)threadIdx.x / LPR;
+    if constexpr (LPR == 64) group = __builtin_amdgcn_readfirstlane(group);
+
+    const IdxT *__restrict__ col = static_cast<const IdxT *>(a.col);
+    const float *__restrict__ val = a.val;
+    const float *__restrict__ x = a.x;
+    const int F = a.feat;
+
+    // Lanes past the end of the feature row keep a valid address (the first feature of
+    // this launch) so that gathers need no predication; only their loads of / stores to
+    // `dst` are masked.  The host guarantees f_base < F and F % VEC == 0.
+    int foff[NCH];
+    bool fok[NCH];
+#pragma unroll
+    for (int k = 0; k < NCH; ++k) {
+        const int f = a.f_base + (k * LPR + lig) * VEC;
+        fok[k] = f < F;
+        foff[k] = fok[k] ? f : a.f_base;
+    }
+
+    const int64_t t0 = (int64_t)blockIdx.x * a.tasks_per_block;
+    int64_t t1 = t0 + a.tasks_per_block;
+    if (t1 > a.ntasks) t1 = a.ntasks;
+
+    for (int64_t t = t0 + group; t < t1; t += GPB) {
+        int64_t start, end;
+        float *dst;
+        bool from_dst;
+        if constexpr (MODE == kSegments) {
+            start = a.seg_start[t];
+            end = start + a.seg_len[t];
+            dst = a.dst + (size_t)t * (size_t)F;
+            from_dst = false;
+        } else {
+            int64_t row = t;
+            if constexpr (MODE == kRowsPermuted) row = a.perm[t];
+            start = a.rowptr[row];
+            end = a.rowptr[row + 1];
+            dst = a.dst + (size_t)row * (size_t)F;
+            from_dst = a.accumulate != 0;
+        }
+        if constexpr (LPR == 64) {
+            start = uniform_i64(start);
+            end = uniform_i64(end);
+        }
+
+        V acc[NCH];
+#pragma unroll
+        for (int k = 0; k < NCH; ++k) {
+            acc[k] = V::zero();
+            if (from_dst && fok[k]) acc[k] = V::load(dst + foff[k]);
+        }
+
+        for (int64_t base = start; base < end; base += LPR) {
+            const int64_t left = end - base;
+            const int cnt = left < LPR ? (int)left : LPR;
+            IdxT c_l = 0;
+            float v_l = 0.0f;
+            if (lig < cnt) {
+                c_l = __builtin_nontemporal_load(col + base + lig);
+                v_l = __builtin_nontemporal_load(val + base + lig);
+            }
+            int j = 0;
+            for (; j + U <= cnt; j += U) {
+                const float *xr[U];
+                float vv[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int64_t c = group_bcast_idx<LPR>(c_l, j + u);
+                    vv[u] = __int_as_float(group_bcast<LPR>(__float_as_int(v_l), j + u));
+                    xr[u] = x + (size_t)c * (size_t)F;
+                }
+                V xv[U][NCH];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+#pragma unroll
+                    for (int k = 0; k < NCH; ++k) xv[u][k] = V::load(xr[u] + foff[k]);
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+#pragma unroll
+                    for (int k = 0; k < NCH; ++k) acc[k].fma(vv[u], xv[u][k]);
+                }
+            }
+            for (; j < cnt; ++j) {
+                const int64_t c = group_bcast_idx<LPR>(c_l, j);
+                const float v = __int_as_float(group_bcast<LPR>(__float_as_int(v_l), j));
+                const float *xr = x + (size_t)c * (size_t)F;
+#pragma unroll
+                for (int k = 0; k < NCH; ++k) acc[k].fma(v, V::load(xr + foff[k]));
+            }
+        }
+
+#pragma unroll
+        for (int k = 0; k < NCH; ++k) {
+            if (fok[k]) acc[k].store(dst + foff[k]);
+        }
+    }
+}
+
+// out[row,:] (+)= sum over the row's segment partial sums, in segment order.
+struct ReduceArgs {
+    const int32_t *heavy_row;     // [nheavy]
+    const int64_t *heavy_segbase; // [nheavy+1]
+    const float *partial;         // [nseg, F]
+    float *out;
+    int nheavy;
+    int feat;
+    int f_base;
+    int accumulate;
+};
+
+template <int VEC, int LPR, int NCH>
+__global__ __launch_bounds__(256) void heavy_reduce_kernel(const ReduceArgs a) {
+    constexpr int GPB = 256 / LPR;
+    typedef FVec<VEC> V;
+    const int lig = (int)threadIdx.x & (LPR - 1);
+    const int group = (int)threadIdx.x / LPR;
+    const int h = (int)blockIdx.x * GPB + group;
+    if (h >= a.nheavy) return;
+    const int F = a.feat;
+    const int64_t s0 = a.heavy_segbase[h], s1 = a.heavy_segbase[h + 1];
+    float *dst = a.out + (size_t)a.heavy_row[h] * (size_t)F;
+#pragma unroll
+    for (int k = 0; k < NCH; ++k) {
+        const int f = a.f_base + (k * LPR + lig) * VEC;
+        if (f >= F) continue;
+        V acc = a.accumulate ? V::load(dst + f) : V::zero();
+        for (int64_t s = s0; s < s1; ++s) acc.add(V::load(a.partial + (size_t)s * (size_t)F + f));
+        acc.store(dst + f);
+    }
+}
+
+}  // namespace gnnagg

@@ -1,0 +1,9 @@
+from .CommBuffer import CommBuffer
+from .CommSplits import CommSplits
+from .DataLoader import get_distributed_graph, get_distributed_graph_for_pre_aggressive, load_graph_structures
+from .DataProcessor import DataProcessor, DataProcessorForPreAggresive
+from .DistributedGraph import DistributedGraph, DistributedGraphForPre
+
+__all__ = ["CommBuffer", "CommSplits", "DataProcessor", "DataProcessorForPreAggresive", "DistributedGraph",
+           "DistributedGraphForPre", "get_distributed_graph", "get_distributed_graph_for_pre_aggressive",
+           "load_graph_structures"]

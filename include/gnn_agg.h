@@ -1,0 +1,141 @@
+/*
+ * gnn_agg.h -- C ABI of libgnnagg.so: the aggregation hot path of a full-batch,
+ * graph-partitioned GCN/GraphSAGE trainer, written for AMD MI355X (gfx950).
+ *
+ * Every pointer is a DEVICE pointer unless its comment says "host".  `stream` is a
+ * hipStream_t passed as void* (NULL = the default stream).  All entry points only
+ * enqueue work on `stream` unless their comment says they synchronise.  They return
+ * GNNAGG_OK or an error code; gnnagg_last_error() gives the message of the calling
+ * thread's last failure.  Results are deterministic: no floating-point atomics are
+ * used anywhere, so two runs on the same inputs are bit-identical.
+ *
+ * Reference paths cited below are relative to self_benchmark/a64fx/ of
+ * zhuangbility111/GNN_benchmark.
+ */
+#ifndef GNN_AGG_H
+#define GNN_AGG_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GNNAGG_OK 0
+#define GNNAGG_ERR_INVALID 1     /* bad argument (null pointer, negative size, bad alignment, index out of range) */
+#define GNNAGG_ERR_HIP 2         /* a HIP runtime call failed */
+#define GNNAGG_ERR_UNSUPPORTED 3 /* sizes beyond what the kernels address (see each function) */
+
+#define GNNAGG_ABI_VERSION 1
+
+/* Version of this ABI (GNNAGG_ABI_VERSION of the built library).  No reference counterpart. */
+int gnnagg_abi_version(void);
+
+/* Message of the calling thread's most recent failure ("" if none).  Host string,
+ * valid until the next failing call on the same thread.  Replaces the c10::Error text
+ * raised by CHECK_CPU / CHECK_INPUT (model/ops/src/utils.h:12-13). */
+const char *gnnagg_last_error(void);
+
+/* ---------------------------------------------------------------------------------
+ * CSR SpMM, out[m,:] += sum_{e in row m} value[e] * mat[col[e],:]  for m < sparse_rows.
+ *
+ * Replaces `computation_ops.spmm(rowptr, col, value, mat, out, sparse_rows,
+ * parallel_row_split, parallel_col_split)` = spmm_cpu_optimized_no_tile_v1
+ * (model/ops/src/spmm.h:3-6, model/ops/src/spmm.cpp:327-507, bound at
+ * model/ops/src/ops.cpp:23).  Same accumulate-into-`out` semantics (spmm.cpp:32-35,
+ * :78-95) and the same int64/int64/fp32 CSR arrays.  The two CPU thread-split
+ * arguments have no meaning on a GPU and are not part of this signature.
+ *   rowptr int64 [sparse_rows+1], col int64 [nnz], value fp32 [nnz]
+ *   mat    fp32 row-major [dense_rows, feat] (contiguous), out fp32 [sparse_rows, feat]
+ * Each row is one fp32 FMA chain in CSR order starting from out[m,:], exactly the
+ * recurrence of kernel_1xN (spmm.cpp:37-53).  Column indices are NOT range-checked
+ * here (the reference does not check them either); use a plan for checked inputs.
+ * ------------------------------------------------------------------------------- */
+int gnnagg_spmm_csr_f32(const int64_t *rowptr, const int64_t *col, const float *value, const float *mat,
+                        float *out, int64_t sparse_rows, int64_t feat, void *stream);
+
+/* ---------------------------------------------------------------------------------
+ * Cached schedule ("plan") of one sparse matrix.
+ *
+ * Replaces the per-matrix CPU work split the reference computes once and caches on
+ * the sparse object: distribute_work_for_row + get/set_work_range[_for_transpose]
+ * (model/ops/spmm_kernel.py:7-28, :48-57, :80-87).  On the GPU the cached object is a
+ * degree-binned row schedule: rows ordered by degree class, rows longer than a
+ * threshold cut into fixed-length segments whose partial sums are combined in a fixed
+ * order, and column indices narrowed to int32.
+ *
+ * gnnagg_plan_create reads rowptr/col on `stream`, validates them (rowptr[0]==0,
+ * non-decreasing, rowptr[rows]==nnz, 0 <= col < cols) and SYNCHRONISES the stream; it
+ * allocates device memory it owns.  The plan keeps no reference to rowptr/col after
+ * it returns.  rows, cols < 2^31 and nnz < 2^40 (GNNAGG_ERR_UNSUPPORTED otherwise).
+ * ------------------------------------------------------------------------------- */
+typedef struct gnnagg_plan gnnagg_plan;
+
+int gnnagg_plan_create(const int64_t *rowptr, const int64_t *col, int64_t rows, int64_t cols, int64_t nnz,
+                       void *stream, gnnagg_plan **plan_out);
+
+/* Frees a plan (synchronises the device; NULL is accepted). */
+int gnnagg_plan_destroy(gnnagg_plan *plan);
+
+/* out (+)= A @ mat through a plan.  `value` is the fp32 [nnz] array in the CSR order
+ * the plan was built from.  accumulate != 0: out += A@mat (the reference semantics,
+ * spmm.cpp:32-35).  accumulate == 0: out = A@mat, every row written (fuses the
+ * `torch.zeros` the reference allocates before the local aggregation,
+ * model/layers/aggregator.py:67-70, :167-170).  May grow a plan-owned scratch buffer
+ * (hipMalloc, synchronising) the first time a larger `feat` is seen.  Calls sharing a
+ * plan must be on one stream or otherwise ordered. */
+int gnnagg_plan_spmm_f32(gnnagg_plan *plan, const float *value, const float *mat, float *out, int64_t feat,
+                         int accumulate, void *stream);
+
+/* Host-side description of a plan, info[0..7] (host pointer):
+ * rows, cols, nnz, rows cut into segments, segments, segment length,
+ * rows with no stored element, largest row length. */
+int gnnagg_plan_info(const gnnagg_plan *plan, int64_t *info);
+
+/* Kernel timing of a plan, for benchmarks.  After gnnagg_plan_profile(plan, 1) every
+ * gnnagg_plan_spmm_f32 call records HIP events on its stream around the whole call and
+ * around its dominant kernel (the one that walks the rows that are not cut).
+ * gnnagg_plan_profile_read SYNCHRONISES on the last recorded events and returns, in
+ * milliseconds, ms[0] = that kernel, ms[1] = the whole call (all kernels), of the most
+ * recent call (host pointer; -1 when nothing was recorded).  Replaces the std::chrono
+ * prints the reference compiles in under `#define PROFILE` (spmm.cpp:12, :411-413,
+ * :486-491). */
+int gnnagg_plan_profile(gnnagg_plan *plan, int enable);
+int gnnagg_plan_profile_read(gnnagg_plan *plan, double *ms);
+
+/* ---------------------------------------------------------------------------------
+ * Transposed CSR arrays (colptr, row_T, value_T) of a CSR matrix: entries grouped by
+ * column, rows ascending inside a column.  Replaces the torch_sparse storage accessors
+ * the backward wrapper reads (model/ops/spmm_kernel.py:76-78: storage.colptr(),
+ * storage.row_T(), storage.value_T()), so that `A^T @ G` runs through the same SpMM.
+ * Outputs: colptr int64 [cols+1], row_t int64 [nnz], value_t fp32 [nnz].
+ * `value`/`value_t` may both be NULL (structure only).  Allocates temporaries and
+ * SYNCHRONISES the stream.  rows, cols < 2^31.
+ * ------------------------------------------------------------------------------- */
+int gnnagg_csr_transpose(const int64_t *rowptr, const int64_t *col, const float *value, int64_t rows,
+                         int64_t cols, int64_t nnz, int64_t *colptr, int64_t *row_t, float *value_t,
+                         void *stream);
+
+/* ---------------------------------------------------------------------------------
+ * COO -> CSR: entries ordered by (row, col), repeated (row, col) pairs KEPT, rowptr by
+ * counting.  Replaces `SparseTensor(row=, col=, value=, sparse_sizes=)` at the call
+ * sites data_manager/DataProcessor.py:104-116, :458-502 (torch_sparse, third party).
+ * Outputs: rowptr int64 [rows+1], col_out int64 [nnz], value_out fp32 [nnz] (value and
+ * value_out may both be NULL).  Validates 0 <= row < rows, 0 <= col < cols.  Allocates
+ * temporaries and SYNCHRONISES the stream.  rows, cols < 2^31.
+ * ------------------------------------------------------------------------------- */
+int gnnagg_coo_to_csr(const int64_t *row, const int64_t *col, const float *value, int64_t nnz, int64_t rows,
+                      int64_t cols, int64_t *rowptr, int64_t *col_out, float *value_out, void *stream);
+
+/* ---------------------------------------------------------------------------------
+ * Boundary-row gather, out[i,:] = src[index[i],:].  Replaces
+ * `torch.index_select(local_nodes_feat, 0, idx_nodes_send_to_others, out=send_buf)`
+ * (model/layers/aggregator.py:51).  index int64 [n_index]; not range-checked.
+ * ------------------------------------------------------------------------------- */
+int gnnagg_gather_rows_f32(const float *src, const int64_t *index, float *out, int64_t n_index, int64_t feat,
+                           void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GNN_AGG_H */

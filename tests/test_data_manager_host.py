@@ -1,0 +1,216 @@
+"""Host logic: the vectorised index-map builders of gnn_benchmark_amd.data_manager must
+reproduce (a) the reference's known-answer vectors and (b) the loop-faithful oracle on
+seeded random partitions, bit for bit (int64 maps)."""
+import numpy as np
+import pytest
+import torch
+
+from gnn_benchmark_amd.data_manager import DataProcessor, DataProcessorForPreAggresive
+from oracle import index_maps as om
+
+
+def T(x):
+    return torch.tensor(x, dtype=torch.int64)
+
+
+def N(x):
+    return np.asarray(x, dtype=np.int64)
+
+
+# ------------------------------------------------------------------ reference vectors
+def test_sort_remote_edges(golden):
+    for c in golden["sort_remote_edges"]:
+        out = DataProcessor.sort_remote_edges_list_based_on_remote_nodes(T(c["edges"]))
+        assert torch.equal(out, T(c["expected"]))
+
+
+def test_obtain_remote_nodes_list(golden):
+    for c in golden["obtain_remote_nodes_list"]:
+        edges = DataProcessor.sort_remote_edges_list_based_on_remote_nodes(T(c["edges"]))
+        nodes, ranges, counts = DataProcessor.obtain_remote_nodes_list(edges, c["num_local_nodes"], T(c["begins"]),
+                                                                       c["world_size"])
+        assert torch.equal(edges, T(c["expected_edges"]))
+        assert torch.equal(nodes, T(c["expected_remote_nodes"]))
+        assert torch.equal(ranges, T(c["expected_ranges"])) and torch.equal(counts, T(c["expected_counts"]))
+
+
+def test_transform_edge_index_to_sparse_tensor(golden):
+    for c in golden["transform_edge_index_to_sparse_tensor"]:
+        local, remote = DataProcessor.transform_edge_index_to_sparse_tensor(
+            [T(c["local_edges"][0]), T(c["local_edges"][1])], [T(c["remote_edges"][0]), T(c["remote_edges"][1])],
+            c["num_local_nodes"], c["num_remote_nodes"])
+        for got, key, edges in ((local, "expected_local_coo", c["local_edges"]),
+                                (remote, "expected_remote_coo", c["remote_edges"])):
+            coo = c[key]
+            expect = torch.zeros(coo["size"])
+            expect[coo["row"], coo["col"]] = torch.tensor(coo["val"])
+            assert list(got.sparse_sizes()) == coo["size"]
+            assert torch.equal(got.to_dense() > 0, expect > 0)
+            assert got.nnz() == len(edges[0]) and float(got.to_dense().sum()) == len(edges[0])
+
+
+def test_get_in_degrees(golden):
+    for c in golden["get_in_degrees"]:
+        got = DataProcessor.get_in_degrees([T(x) for x in c["local_edges"]], [T(x) for x in c["remote_edges"]],
+                                           c["num_local_nodes"])
+        assert got.dtype == torch.float32 and torch.equal(got, torch.tensor(c["expected"]))
+
+
+def test_get_degrees(golden):
+    for c in golden["get_degrees"]:
+        assert DataProcessorForPreAggresive.get_degrees(T(c["nodes"])) == {int(k): v for k, v in c["expected"].items()}
+
+
+def test_decide_pre_or_post_aggr(golden):
+    for c in golden["decide_pre_or_post_aggr"]:
+        got = DataProcessorForPreAggresive.decide_pre_or_post_aggr(T(c["src"]), T(c["dst"]), c["is_pre"], c["is_post"])
+        assert got.dtype == torch.int64 and torch.equal(got, T(c["expected"])), c["source"]
+
+
+def test_collect_edges_sent_to_other_subgraphs(golden):
+    for c in golden["collect_edges_sent_to_other_subgraphs"]:
+        sent = []
+        DataProcessorForPreAggresive.collect_edges_sent_to_other_subgraphs(
+            T(c["src"]), T(c["dst"]), T(c["pre_idx"]), T(c["post_idx"]), sent)
+        n = len(c["expected_src_to_send"])
+        assert torch.equal(sent[0][:n], T(c["expected_src_to_send"])), c["source"]
+        assert torch.equal(sent[0][n:], T(c["expected_dst_to_send"])), c["source"]
+
+
+def test_collect_edges_for_aggregation(golden):
+    for c in golden["collect_edges_for_aggregation"]:
+        lists, splits, begin = [T([]), T([])], [], torch.zeros(2, dtype=torch.int64)
+        DataProcessorForPreAggresive.collect_edges_for_aggregation(
+            T(c["src"]), T(c["dst"]), T(c["pre_idx"]), T(c["post_idx"]), lists, splits, begin, 0)
+        assert torch.equal(lists[0], T(c["expected_src"])) and torch.equal(lists[1], T(c["expected_dst"]))
+        assert splits == c["expected_splits"] and torch.equal(begin, T(c["expected_begin_edge"]))
+
+
+def test_split_remote_edges_for_aggr_and_graph_exchange(golden):
+    for c in golden["split_remote_edges_for_aggr_and_graph_exchange"]:
+        sent, aggr, begin_from, recv_splits = (
+            DataProcessorForPreAggresive.split_remote_edges_for_aggr_and_graph_exchange(
+                T(c["begins"]), [T(c["edges"][0]), T(c["edges"][1])], c["world_size"]))
+        for got, exp in zip(sent, c["expected_sent"]):
+            assert torch.equal(got, T(exp))
+        assert torch.equal(aggr[0], T(c["expected_aggr_on_recv"][0]))
+        assert torch.equal(aggr[1], T(c["expected_aggr_on_recv"][1]))
+        assert torch.equal(begin_from, T(c["expected_begin_edge_from"])) and recv_splits == c["expected_recv_splits"]
+
+
+def test_split_remote_edges_recv_from_graph_exchange(golden):
+    for c in golden["split_remote_edges_recv_from_graph_exchange"]:
+        lists, begin_to, splits = DataProcessorForPreAggresive.split_remote_edges_recv_from_graph_exchange(
+            [T(x) for x in c["recv_lists"]], c["world_size"])
+        assert torch.equal(lists[0], T(c["expected_lists"][0])) and torch.equal(lists[1], T(c["expected_lists"][1]))
+        assert torch.equal(begin_to, T(c["expected_begin_edge_to"])) and splits == c["expected_send_splits"]
+
+
+def test_remap_remote_nodes_id(golden):
+    for c in golden["remap_remote_nodes_id"]:
+        nodes = T(c["nodes"])
+        assert DataProcessorForPreAggresive.remap_remote_nodes_id(nodes, T(c["begins"])) == c["expected_count"]
+        assert torch.equal(nodes, T(c["expected_nodes"])), c["source"]
+
+
+# ------------------------------------------------------------------ vs. the oracle on random partitions
+def _random_partition(seed, world=5, n_local=40, e_local=300, e_remote=260, rank=2):
+    rng = np.random.default_rng(seed)
+    sizes = rng.integers(0, 60, world)
+    sizes[rank] = n_local
+    begins = np.concatenate(([0], np.cumsum(sizes))).astype(np.int64)
+    local = np.stack([rng.integers(0, n_local, e_local), rng.integers(0, n_local, e_local)]).astype(np.int64)
+    others = np.concatenate([np.arange(begins[i], begins[i + 1]) for i in range(world) if i != rank])
+    # skewed choice of remote sources so that both PRE and POST edges occur
+    p = 1.0 / (1.0 + np.arange(others.size)) if others.size else None
+    src = rng.choice(others, e_remote, p=None if p is None else p / p.sum()) if others.size else np.zeros(0, np.int64)
+    dst = rng.integers(0, max(n_local // 3, 1), src.size)
+    remote = np.stack([src, dst]).astype(np.int64)
+    return begins, local, remote
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_non_pre_maps_equal_oracle(seed):
+    begins, local, remote = _random_partition(seed)
+    world, n_local = len(begins) - 1, 40
+    o_edges = [remote[0].copy(), remote[1].copy()]
+    om.sort_remote_edges_list_based_on_remote_nodes(o_edges)
+    o_nodes, o_ranges, o_counts = om.obtain_remote_nodes_list(o_edges, n_local, begins, world)
+
+    t_edges = torch.from_numpy(remote.copy())
+    DataProcessor.sort_remote_edges_list_based_on_remote_nodes(t_edges)
+    nodes, ranges, counts = DataProcessor.obtain_remote_nodes_list(t_edges, n_local, torch.from_numpy(begins), world)
+    assert np.array_equal(t_edges.numpy(), np.stack(o_edges))
+    assert np.array_equal(nodes.numpy(), o_nodes) and np.array_equal(ranges.numpy(), o_ranges)
+    assert np.array_equal(counts.numpy(), o_counts)
+
+    o_local, o_remote = om.transform_edge_index_to_sparse_tensor(local, o_edges, n_local, len(o_nodes))
+    t_local, t_remote = DataProcessor.transform_edge_index_to_sparse_tensor(torch.from_numpy(local), t_edges, n_local,
+                                                                            int(nodes.numel()))
+    for got, exp in ((t_local, o_local), (t_remote, o_remote)):
+        rowptr, col, val = got.csr()
+        assert np.array_equal(rowptr.numpy(), exp[0]) and np.array_equal(col.numpy(), exp[1])
+        assert np.array_equal(val.numpy(), exp[2]) and tuple(got.sparse_sizes()) == tuple(exp[3])
+    assert np.array_equal(DataProcessor.get_in_degrees(torch.from_numpy(local), torch.from_numpy(remote), n_local).numpy(),
+                          om.get_in_degrees(local, remote, n_local))
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_pre_post_maps_equal_oracle(seed):
+    rank = 2
+    begins, local, remote = _random_partition(100 + seed, rank=rank)
+    world, n_local = len(begins) - 1, 40
+    remote_g = remote.copy()
+    remote_g[1] += begins[rank]  # DataLoader.py:139
+    o = om.split_remote_edges_for_aggr_and_graph_exchange(begins, [remote_g[0], remote_g[1]], world)
+    t = DataProcessorForPreAggresive.split_remote_edges_for_aggr_and_graph_exchange(
+        torch.from_numpy(begins), [torch.from_numpy(remote_g[0]), torch.from_numpy(remote_g[1])], world)
+    for a, b in zip(t[0], o[0]):
+        assert np.array_equal(a.numpy(), b)
+    assert np.array_equal(t[1][0].numpy(), o[1][0]) and np.array_equal(t[1][1].numpy(), o[1][1])
+    assert np.array_equal(t[2].numpy(), o[2]) and t[3] == o[3]
+
+    # what the peers would send here: seeded packed lists (sorted by second half)
+    rng = np.random.default_rng(seed)
+    recv = []
+    for i in range(world):
+        if i == rank or begins[i + 1] == begins[i]:
+            recv.append(np.zeros(0, dtype=np.int64))
+            continue
+        n = int(rng.integers(0, 50))
+        dst = np.sort(rng.integers(begins[i], begins[i + 1], n))
+        src = rng.integers(begins[rank], begins[rank + 1], n)
+        recv.append(np.concatenate([src, dst]).astype(np.int64))
+    o_send, o_begin_to, o_splits = om.split_remote_edges_recv_from_graph_exchange(recv, world)
+    t_send, t_begin_to, t_splits = DataProcessorForPreAggresive.split_remote_edges_recv_from_graph_exchange(
+        [torch.from_numpy(x) for x in recv], world)
+    assert np.array_equal(t_send[0].numpy(), o_send[0]) and np.array_equal(t_send[1].numpy(), o_send[1])
+    assert np.array_equal(t_begin_to.numpy(), o_begin_to) and t_splits == o_splits
+
+    o_mats = om.transform_edge_index_to_sparse_tensor_for_pre(
+        local, [o[1][0].copy(), o[1][1].copy()], [o_send[0].copy(), o_send[1].copy()], o[2], o_begin_to, n_local,
+        begins[rank])
+    t_mats = DataProcessorForPreAggresive.transform_edge_index_to_sparse_tensor(
+        torch.from_numpy(local), [t[1][0].clone(), t[1][1].clone()], [t_send[0].clone(), t_send[1].clone()], t[2],
+        t_begin_to, n_local, int(begins[rank]))
+    for got, exp in zip(t_mats, o_mats):
+        rowptr, col, val = got.csr()
+        assert tuple(got.sparse_sizes()) == tuple(exp[3])
+        assert np.array_equal(rowptr.numpy(), exp[0]) and np.array_equal(col.numpy(), exp[1])
+        assert np.array_equal(val.numpy(), exp[2])
+    # buffer rows line up with the split lists
+    assert t_mats[1].sparse_size(1) == sum(t[3]) and t_mats[2].sparse_size(0) == sum(t_splits)
+
+
+def test_remap_random_equals_oracle():
+    rng = np.random.default_rng(5)
+    for _ in range(20):
+        w = int(rng.integers(1, 6))
+        lens = rng.integers(0, 8, w)
+        begins = np.concatenate(([0], np.cumsum(lens))).astype(np.int64)
+        nodes = np.concatenate([np.sort(rng.integers(0, 6, l)) for l in lens] + [np.zeros(0, np.int64)]).astype(np.int64)
+        o_nodes = nodes.copy()
+        t_nodes = torch.from_numpy(nodes.copy())
+        assert om.remap_remote_nodes_id(o_nodes, begins) == DataProcessorForPreAggresive.remap_remote_nodes_id(
+            t_nodes, torch.from_numpy(begins))
+        assert np.array_equal(o_nodes, t_nodes.numpy())

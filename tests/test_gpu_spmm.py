@@ -1,0 +1,212 @@
+"""GPU parity of the SpMM path (through the C ABI of libgnnagg.so) against the CPU
+oracle on the same seeded inputs.  Tolerance: rel 1e-5 / abs 1e-6 (tests/gpu_util.py);
+where a row is not cut into segments the FMA chain is the oracle's, so those cases
+are additionally required to be bit-identical."""
+import numpy as np
+import pytest
+import torch
+
+from gnn_benchmark_amd import SPMM_backward, SPMM_forward, SparseTensor, computation_ops
+from gnn_benchmark_amd.sparse_tensor import SpmmPlan
+from oracle import index_maps as om
+from oracle import spmm as ospmm
+from tests.gpu_util import assert_close, dev, random_csr, skewed_csr
+
+pytestmark = pytest.mark.gpu
+
+EMPTY_I32 = torch.empty(0, dtype=torch.int32)
+
+
+def _oracle(rowptr, col, val, x, out0=None):
+    out = np.zeros((rowptr.shape[0] - 1, x.shape[1]), dtype=np.float32) if out0 is None else out0.copy()
+    return ospmm.spmm(rowptr, col, val, x, out)
+
+
+def test_reference_recipe_forward_and_backward():
+    # the reference's own test: 20020 x 1020, density 7e-4, F=128 (tests/test_spmm.py:70-115)
+    a = random_csr(20020, 1020, 0.0007, seed=0)
+    rng = np.random.default_rng(0)
+    x = rng.random((1020, 128), dtype=np.float32)
+    g = rng.standard_normal((20020, 128)).astype(np.float32)
+    src = SparseTensor.from_scipy(a).cuda()
+
+    out = torch.zeros(20020, 128, device="cuda")
+    assert SPMM_forward(src, dev(x), out) is None
+    want = _oracle(a.indptr, a.indices, a.data, x)
+    assert_close(out, want, "forward")
+    assert np.array_equal(out.cpu().numpy(), want)  # no row is cut here: same FMA chain as the oracle
+    assert torch.allclose(out.cpu(), torch.from_numpy(a.toarray()) @ torch.from_numpy(x), atol=1e-5)
+
+    grad = torch.zeros(1020, 128, device="cuda")
+    ret = SPMM_backward(src, dev(g), grad)
+    assert ret[0] is grad and ret[1] is None
+    want_g = np.zeros((1020, 128), dtype=np.float32)
+    ospmm.spmm_transposed(a.indptr, a.indices, a.data, g, want_g, 1020)
+    assert_close(grad, want_g, "backward")
+
+
+@pytest.mark.parametrize("feat", [1, 2, 15, 16, 17, 40, 47, 63, 64, 65, 100, 128, 130, 172, 256, 258, 602, 1030, 2052])
+def test_native_op_accumulates_for_every_width(feat):
+    rowptr, col, val = skewed_csr(700, 333, seed=feat, heavy_rows=(900, 300))
+    rng = np.random.default_rng(feat)
+    x = rng.standard_normal((333, feat)).astype(np.float32)
+    out0 = rng.standard_normal((700, feat)).astype(np.float32)
+    out = dev(out0)
+    ret = computation_ops.spmm(dev(rowptr), dev(col), dev(val), dev(x), out, 700, EMPTY_I32, EMPTY_I32)
+    assert ret[0] is out and ret[1] is None
+    want = _oracle(rowptr, col, val, x, out0)
+    assert_close(out, want, f"native op F={feat}")
+    assert np.array_equal(out.cpu().numpy(), want)  # plan-less path: one chain per row, CSR order
+
+
+@pytest.mark.parametrize("feat", [1, 16, 47, 64, 100, 128, 256, 602, 1030])
+@pytest.mark.parametrize("accumulate", [True, False])
+def test_plan_path_with_cut_rows_and_empty_rows(feat, accumulate):
+    rowptr, col, val = skewed_csr(900, 450, seed=1000 + feat)
+    rng = np.random.default_rng(feat)
+    x = rng.standard_normal((450, feat)).astype(np.float32)
+    out0 = rng.standard_normal((900, feat)).astype(np.float32)
+    plan = SpmmPlan(dev(rowptr), dev(col), 900, 450)
+    info = plan.info()
+    assert info["cut_rows"] == 3 and info["max_row_len"] == 5000 and info["empty_rows"] > 0
+    assert info["segments"] == sum(-(-h // info["segment_len"]) for h in (5000, 1300, 700))
+    out = dev(out0)
+    plan.spmm(dev(val), dev(x), out, accumulate=accumulate)
+    want = _oracle(rowptr, col, val, x, out0 if accumulate else None)
+    assert_close(out, want, f"plan F={feat} acc={accumulate}")
+    # rows that are not cut keep the oracle's exact chain
+    deg = np.diff(rowptr)
+    keep = deg <= 2 * info["segment_len"]
+    assert np.array_equal(out.cpu().numpy()[keep], want[keep])
+
+
+def test_results_are_deterministic():
+    rowptr, col, val = skewed_csr(2000, 800, seed=5)
+    x = dev(np.random.default_rng(5).standard_normal((800, 128)).astype(np.float32))
+    plan = SpmmPlan(dev(rowptr), dev(col), 2000, 800)
+    outs = []
+    for _ in range(3):
+        out = torch.empty(2000, 128, device="cuda")
+        plan.spmm(dev(val), x, out, accumulate=False)
+        outs.append(out.cpu())
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+
+
+def test_unaligned_operands_fall_back_to_narrower_loads():
+    rowptr, col, val = skewed_csr(300, 120, seed=9, heavy_rows=(600,))
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((120, 64)).astype(np.float32)
+    base = torch.zeros(120 * 64 + 1, device="cuda")
+    x_un = base[1:].view(120, 64)  # 4-byte aligned only
+    x_un.copy_(dev(x))
+    out = torch.zeros(300, 64, device="cuda")
+    computation_ops.spmm(dev(rowptr), dev(col), dev(val), x_un, out, 300, EMPTY_I32, EMPTY_I32)
+    assert_close(out, _oracle(rowptr, col, val, x), "unaligned")
+
+
+def test_edge_shapes():
+    # empty matrix, single row, matrix with only empty rows
+    x = torch.ones(5, 8, device="cuda")
+    out = torch.full((4, 8), 2.0, device="cuda")
+    rowptr = torch.zeros(5, dtype=torch.int64, device="cuda")
+    empty = torch.empty(0, dtype=torch.int64, device="cuda")
+    computation_ops.spmm(rowptr, empty, torch.empty(0, device="cuda"), x, out, 4, EMPTY_I32, EMPTY_I32)
+    assert torch.equal(out.cpu(), torch.full((4, 8), 2.0))
+    plan = SpmmPlan(rowptr, empty, 4, 5)
+    plan.spmm(torch.empty(0, device="cuda"), x, out, accumulate=True)
+    assert torch.equal(out.cpu(), torch.full((4, 8), 2.0))
+    plan.spmm(torch.empty(0, device="cuda"), x, out, accumulate=False)
+    assert torch.equal(out.cpu(), torch.zeros(4, 8))
+    src = SparseTensor(row=torch.tensor([0]).cuda(), col=torch.tensor([3]).cuda(), value=torch.tensor([2.5]).cuda(),
+                       sparse_sizes=(1, 5))
+    out = torch.zeros(1, 8, device="cuda")
+    SPMM_forward(src, x, out)
+    assert torch.equal(out.cpu(), torch.full((1, 8), 2.5))
+
+
+def test_error_behaviour():
+    rowptr, col, val = skewed_csr(50, 20, seed=1, heavy_rows=())
+    x = torch.ones(20, 8, device="cuda")
+    out = torch.zeros(50, 8, device="cuda")
+    with pytest.raises(RuntimeError, match="Input mismatch"):
+        computation_ops.spmm(dev(rowptr), dev(col), dev(val)[:-1], x, out, 50, EMPTY_I32, EMPTY_I32)
+    with pytest.raises(RuntimeError, match="Input mismatch"):
+        computation_ops.spmm(dev(rowptr), dev(col), dev(val), x.view(-1), out, 50, EMPTY_I32, EMPTY_I32)
+    with pytest.raises(RuntimeError, match="float32"):
+        computation_ops.spmm(dev(rowptr), dev(col), dev(val).double(), x, out, 50, EMPTY_I32, EMPTY_I32)
+    with pytest.raises(RuntimeError, match="GPU"):
+        computation_ops.spmm(dev(rowptr), dev(col), dev(val), x.cpu(), out, 50, EMPTY_I32, EMPTY_I32)
+    assert torch.equal(out.cpu(), torch.zeros(50, 8))
+    bad_col = col.copy()
+    bad_col[3] = 20
+    with pytest.raises(RuntimeError, match="column index"):
+        SpmmPlan(dev(rowptr), dev(bad_col), 50, 20)
+    bad_ptr = rowptr.copy()
+    bad_ptr[5], bad_ptr[6] = bad_ptr[6], bad_ptr[5] - 1
+    with pytest.raises(RuntimeError, match="rowptr"):
+        SpmmPlan(dev(bad_ptr), dev(col), 50, 20)
+
+
+def test_transposed_arrays_and_csr_build_are_bit_exact():
+    rowptr, col, val = skewed_csr(400, 260, seed=11, heavy_rows=(800,))
+    src = SparseTensor(rowptr=dev(rowptr), col=dev(col), value=dev(val), sparse_sizes=(400, 260), is_sorted=True)
+    colptr, row_t, val_t = ospmm.csr_transpose(rowptr, col, val, 260)
+    assert np.array_equal(src.storage.colptr().cpu().numpy(), colptr)
+    assert np.array_equal(src.storage.row_T().cpu().numpy(), row_t)
+    assert np.array_equal(src.storage.value_T().cpu().numpy(), val_t)
+
+    rng = np.random.default_rng(12)
+    n = 5000
+    row = rng.integers(0, 300, n).astype(np.int64)
+    c = rng.integers(0, 40, n).astype(np.int64)  # few columns: many repeated (row, col) pairs
+    v = rng.standard_normal(n).astype(np.float32)
+    got = SparseTensor(row=dev(row), col=dev(c), value=dev(v), sparse_sizes=(300, 40))
+    o_rowptr, o_col, o_val = om.build_csr(row, c, v, 300)
+    g_rowptr, g_col, g_val = got.csr()
+    assert np.array_equal(g_rowptr.cpu().numpy(), o_rowptr) and np.array_equal(g_col.cpu().numpy(), o_col)
+    assert np.array_equal(g_val.cpu().numpy(), o_val)  # repeated pairs keep their input order
+    with pytest.raises(RuntimeError, match="outside"):
+        SparseTensor(row=dev(row), col=dev(c), value=dev(v), sparse_sizes=(300, 39))
+    # host (CPU tensor) construction gives the same arrays
+    host = SparseTensor(row=torch.from_numpy(row), col=torch.from_numpy(c), value=torch.from_numpy(v), sparse_sizes=(300, 40))
+    assert all(torch.equal(a.cpu(), b) for a, b in zip(got.csr(), host.csr()))
+
+
+def test_full_size_properties_power_law():
+    """Size-independent checks on a graph too large for the oracle to sweep fully:
+    linearity in the dense operand, agreement of the plan and plan-less paths, the
+    adjoint identity <A x, y> == <x, A^T y>, and oracle parity on a row sample."""
+    from gnn_benchmark_amd.synthetic import power_law_graph
+
+    g = power_law_graph(num_nodes=300_000, mean_out_degree=12, zipf_s=1.8, max_degree=15000, seed=3, device="cuda")
+    src, n = g.adj, g.num_nodes
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    x1 = torch.randn(n, 128, device="cuda", generator=gen)
+    x2 = torch.randn(n, 128, device="cuda", generator=gen)
+    y = torch.randn(n, 128, device="cuda", generator=gen)
+
+    def fwd(x):
+        out = torch.empty(n, 128, device="cuda")
+        SPMM_forward(src, x, out, accumulate=False)
+        return out
+
+    o1, o2, o12 = fwd(x1), fwd(x2), fwd(x1 + 2.0 * x2)
+    scale = float(o12.abs().max())
+    assert float((o12 - (o1 + 2.0 * o2)).abs().max()) <= 2e-5 * scale
+    rowptr, col, val = src.csr()
+    direct = torch.zeros(n, 128, device="cuda")
+    computation_ops.spmm(rowptr, col, val, x1, direct, n, EMPTY_I32, EMPTY_I32)
+    assert float((direct - o1).abs().max()) <= 2e-5 * scale
+    gt = torch.empty(n, 128, device="cuda")
+    SPMM_backward(src, y, gt, accumulate=False)
+    lhs = float((o1.double() * y.double()).sum())
+    rhs = float((x1.double() * gt.double()).sum())
+    assert abs(lhs - rhs) <= 1e-6 * max(abs(lhs), abs(rhs), 1.0) + 1e-3
+    # oracle parity on 4096 sampled rows (heaviest rows included)
+    deg = (rowptr[1:] - rowptr[:-1]).cpu().numpy()
+    rows = np.unique(np.concatenate([np.argsort(deg)[-64:], np.random.default_rng(0).integers(0, n, 4032)]))
+    rp, c, v = rowptr.cpu().numpy(), col.cpu().numpy(), val.cpu().numpy()
+    sub_ptr = np.concatenate(([0], np.cumsum(deg[rows]))).astype(np.int64)
+    take = np.concatenate([np.arange(rp[r], rp[r + 1]) for r in rows])
+    want = _oracle(sub_ptr, c[take], v[take], x1.cpu().numpy())
+    assert_close(o1[torch.from_numpy(rows).cuda()], want, "row sample vs oracle")

@@ -1,0 +1,64 @@
+"""CPU-only: the C-ABI library loads and exports every entry point include/gnn_agg.h
+declares; argument checks that need no GPU work are exercised (no compute calls)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from gnn_benchmark_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    with open(os.path.join(ROOT, "include", "gnn_agg.h")) as f:
+        text = f.read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(gnnagg_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_binding_agree():
+    assert _declared() == sorted(_lib.EXPORTS)
+
+
+def test_library_exports_every_declared_symbol():
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("libgnnagg.so not built yet (python -c 'import __graft_entry__ as g; g.build()')")
+    cdll = ctypes.CDLL(_lib.LIB_PATH)
+    for name in _declared():
+        assert hasattr(cdll, name), name
+    assert _lib.lib().gnnagg_abi_version() == _lib.ABI_VERSION
+
+
+def test_argument_errors_without_gpu_work():
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("libgnnagg.so not built yet")
+    L = _lib.lib()
+    assert L.gnnagg_spmm_csr_f32(None, None, None, None, None, -1, 4, None) == _lib.ERR_INVALID
+    assert b"negative" in L.gnnagg_last_error()
+    assert L.gnnagg_spmm_csr_f32(None, None, None, None, None, 0, 4, None) == _lib.OK  # empty problem
+    assert L.gnnagg_spmm_csr_f32(None, None, None, None, None, 3, 4, None) == _lib.ERR_INVALID
+    assert L.gnnagg_plan_create(None, None, 1, 1, 0, None, None) == _lib.ERR_INVALID
+    assert L.gnnagg_plan_destroy(None) == _lib.OK
+    assert L.gnnagg_gather_rows_f32(None, None, None, 0, 8, None) == _lib.OK
+    with pytest.raises(_lib.GnnAggError):
+        _lib.check(L.gnnagg_gather_rows_f32(None, None, None, 5, 8, None))
+
+
+def test_product_refuses_cpu_tensors():
+    import torch
+
+    from gnn_benchmark_amd import SPMM_forward, SparseTensor, computation_ops
+
+    rowptr = torch.tensor([0, 1, 2])
+    col = torch.tensor([0, 1])
+    val = torch.ones(2)
+    x = torch.ones(2, 4)
+    out = torch.zeros(2, 4)
+    with pytest.raises(RuntimeError, match="GPU"):
+        computation_ops.spmm(rowptr, col, val, x, out, 2, torch.empty(0, dtype=torch.int32), torch.tensor([0, 4], dtype=torch.int32))
+    src = SparseTensor(rowptr=rowptr, col=col, value=val, sparse_sizes=(2, 2), is_sorted=True)
+    with pytest.raises(RuntimeError, match="GPU"):
+        SPMM_forward(src, x, out)
+    assert torch.equal(out, torch.zeros(2, 4))
