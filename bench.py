@@ -39,16 +39,10 @@ def b_min(nnz: int, rows: int, cols: int, feat: int) -> float:
 
 
 def rows_kernel_cover(src, plan_info):
-    """(rows, nnz) covered by the dominant (row) kernel with accumulate=1: rows that are
-    neither cut into segments nor empty."""
-    import torch
-
+    """(rows, nnz) covered by the dominant kernel launch with accumulate=1: every row
+    that has a stored element (empty rows are not visited)."""
     rowptr = src.csr()[0]
-    deg = rowptr[1:] - rowptr[:-1]
-    cut = deg > 2 * plan_info["segment_len"]
-    nnz_cut = int(deg[cut].sum())
-    rows = int(deg.numel()) - plan_info["cut_rows"] - plan_info["empty_rows"]
-    return rows, int(rowptr[-1]) - nnz_cut
+    return plan_info["rows"] - plan_info["empty_rows"], int(rowptr[-1])
 
 
 def time_spmm(plan, value, x, out, steps, warmup):
@@ -194,12 +188,12 @@ def run_c2(args):
         "config": {"workload": f"c2: CSR SpMM forward A@X + transposed backward A^T@G, power-law graph "
                                f"{n} nodes / {nnz} nnz (Zipf s=1.8, max row {g.max_degree}), GCN-normalised fp32, "
                                f"dense operand {n}x{feat} fp32",
-                   "nodes": n, "nnz": nnz, "feat": feat, "seed": args.seed, "cut_rows": info["cut_rows"],
-                   "segments": info["segments"], "setup_s": round(setup_s, 2)},
+                   "nodes": n, "nnz": nnz, "feat": feat, "seed": args.seed, "long_rows": info["long_rows"],
+                   "max_row_len": info["max_row_len"], "setup_s": round(setup_s, 2)},
         "roofline": {"bound": "hbm", "achieved": round(r["kernel_bytes"] / (r["kernel_ms"] * 1e-3) / 1e9, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(r["kernel_bytes"] / (r["kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                     "traffic": None, "kernel": "spmm_tasks_kernel (forward, rows not cut)",
+                     "traffic": None, "kernel": "spmm_tasks_kernel (forward A@X, all rows)",
                      "kernel_ms": r["kernel_ms"], "bytes_per_launch": r["kernel_bytes"]},
         "extra": {"c2": [results[f] for f in feats]},
     }
@@ -222,6 +216,9 @@ def main():
     ap.add_argument("--mean-out-degree", type=float, default=25.0)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 1 GiB device copy 3 times (a kernel of known traffic for scaling "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU's share of the partitioned graph; --gpus must be 1 "
@@ -232,6 +229,13 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU (there is no CPU path)", file=sys.stderr)
         sys.exit(3)
+    if args.copy_calibration:
+        a = torch.ones(1 << 28, dtype=torch.float32, device="cuda:0")  # 1 GiB
+        b = torch.empty_like(a)
+        for _ in range(3):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        del a, b
     line = run_c2(args)
     print(json.dumps(line), flush=True)
 

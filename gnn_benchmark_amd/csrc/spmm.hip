@@ -50,11 +50,15 @@ hipError_t launch_tasks(const SpmmArgs &a, int rows_per_group, hipStream_t strea
     constexpr int GPB = 256 / LPR;
     SpmmArgs args = a;
     args.tasks_per_block = GPB * rows_per_group;
-    const int64_t nblocks = (a.ntasks + args.tasks_per_block - 1) / args.tasks_per_block;
+    if (args.head_tasks > args.ntasks) args.head_tasks = args.ntasks;
+    const int64_t head_blocks = (args.head_tasks + GPB - 1) / GPB;
+    const int64_t nblocks =
+        head_blocks + (args.ntasks - args.head_tasks + args.tasks_per_block - 1) / args.tasks_per_block;
     if (nblocks == 0) return hipSuccess;
+    args.head_blocks = (int)head_blocks;
     if (nblocks > 0x7fffffffll) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((spmm_tasks_kernel<VEC, LPR, NCH, IdxT, MODE>), dim3((unsigned)nblocks), dim3(256), 0, stream,
-                       args);
+    hipLaunchKernelGGL((spmm_tasks_kernel<VEC, LPR, NCH, IdxT, MODE>), dim3((unsigned)nblocks), dim3(256), 0,
+                       stream, args);
     return hipGetLastError();
 }
 
@@ -82,61 +86,34 @@ hipError_t dispatch_tasks(const Shape &s, const SpmmArgs &a, int rpg, hipStream_
     return dispatch_shape<1, IdxT, MODE>(s, a, rpg, st);
 }
 
-template <int VEC>
-hipError_t dispatch_reduce_vec(const Shape &s, const ReduceArgs &a, hipStream_t st) {
-#define GNNAGG_CASE(L, N)                                                                               \
-    if (s.lpr == L && s.nch == N) {                                                                     \
-        constexpr int GPB = 256 / L;                                                                    \
-        hipLaunchKernelGGL((heavy_reduce_kernel<VEC, L, N>), dim3((unsigned)((a.nheavy + GPB - 1) / GPB)), \
-                           dim3(256), 0, st, a);                                                        \
-        return hipGetLastError();                                                                       \
-    }
-    GNNAGG_CASE(16, 1)
-    GNNAGG_CASE(32, 1)
-    GNNAGG_CASE(64, 1)
-    GNNAGG_CASE(64, 2)
-    GNNAGG_CASE(64, 3)
-    GNNAGG_CASE(64, 4)
-    GNNAGG_CASE(64, 5)
-    GNNAGG_CASE(64, 6)
-    GNNAGG_CASE(64, 8)
-#undef GNNAGG_CASE
-    return hipErrorInvalidValue;
-}
-
-hipError_t dispatch_reduce(const Shape &s, const ReduceArgs &a, hipStream_t st) {
-    if (a.nheavy == 0) return hipSuccess;
-    if (s.vec == 4) return dispatch_reduce_vec<4>(s, a, st);
-    if (s.vec == 2) return dispatch_reduce_vec<2>(s, a, st);
-    return dispatch_reduce_vec<1>(s, a, st);
-}
-
 // ------------------------------------------------------------------ plan kernels
-constexpr int kMaxClasses = 40;
+// Degree class of a row: class c (c < kEmptyClass) holds the rows with
+// ceil(log2(length)) == kEmptyClass - 1 - c, i.e. classes run from the LONGEST rows
+// (small c) to single-element rows; the last class holds the empty rows.
+constexpr int kEmptyClass = 41;
+constexpr int kNumClasses = kEmptyClass + 1;
+constexpr int kClassBits = 6;
 
 struct ClassifyOut {
-    unsigned long long class_count[kMaxClasses];
+    unsigned long long class_count[kNumClasses];
     unsigned long long max_deg;
     unsigned int bad_rowptr;  // rowptr decreasing somewhere
     unsigned int bad_col;     // a column index outside [0, cols)
 };
 
-// Degree class of a row: 0 = cut into segments (deg > heavy_thresh); then one class per
-// power-of-two degree bucket in DESCENDING degree order; the last class holds empty rows.
-__device__ __forceinline__ int degree_class(int64_t deg, int heavy_thresh, int heavy_log) {
-    if (deg > heavy_thresh) return 0;
-    if (deg == 0) return heavy_log + 2;
-    const int clog = deg <= 1 ? 0 : 64 - __builtin_clzll((unsigned long long)(deg - 1));  // ceil(log2(deg))
-    return 1 + (heavy_log - clog);
+__host__ __device__ __forceinline__ int degree_class(int64_t deg) {
+    if (deg <= 0) return kEmptyClass;
+    int clog = 0;  // ceil(log2(deg))
+    while ((int64_t(1) << clog) < deg) ++clog;
+    return kEmptyClass - 1 - clog;
 }
 
 __global__ __launch_bounds__(256) void classify_rows_kernel(const int64_t *__restrict__ rowptr, int rows,
-                                                            int heavy_thresh, int heavy_log,
                                                             uint32_t *__restrict__ key, int32_t *__restrict__ rowid,
                                                             ClassifyOut *__restrict__ out) {
-    __shared__ unsigned int hist[kMaxClasses];
+    __shared__ unsigned int hist[kNumClasses];
     __shared__ unsigned long long smax;
-    if (threadIdx.x < kMaxClasses) hist[threadIdx.x] = 0;
+    if (threadIdx.x < kNumClasses) hist[threadIdx.x] = 0;
     if (threadIdx.x == 0) smax = 0;
     __syncthreads();
     const int r = (int)blockIdx.x * 256 + (int)threadIdx.x;
@@ -144,9 +121,9 @@ __global__ __launch_bounds__(256) void classify_rows_kernel(const int64_t *__res
         const int64_t d = rowptr[r + 1] - rowptr[r];
         if (d < 0) {
             atomicOr(&out->bad_rowptr, 1u);
-            key[r] = (uint32_t)(heavy_log + 2);
+            key[r] = (uint32_t)kEmptyClass;
         } else {
-            const int c = degree_class(d, heavy_thresh, heavy_log);
+            const int c = degree_class(d);
             key[r] = (uint32_t)c;
             atomicAdd(&hist[c], 1u);
             atomicMax(&smax, (unsigned long long)d);
@@ -154,7 +131,7 @@ __global__ __launch_bounds__(256) void classify_rows_kernel(const int64_t *__res
         rowid[r] = r;
     }
     __syncthreads();
-    if (threadIdx.x < kMaxClasses && hist[threadIdx.x])
+    if (threadIdx.x < kNumClasses && hist[threadIdx.x])
         atomicAdd(&out->class_count[threadIdx.x], (unsigned long long)hist[threadIdx.x]);
     if (threadIdx.x == 0 && smax) atomicMax(&out->max_deg, smax);
 }
@@ -169,39 +146,6 @@ __global__ __launch_bounds__(256) void narrow_cols_kernel(const int64_t *__restr
         col32[e] = (int32_t)c;
     }
     if (bad) atomicOr(&out->bad_col, 1u);
-}
-
-// nseg[h] for the rows cut into segments (the first nheavy entries of perm).
-__global__ __launch_bounds__(256) void heavy_count_kernel(const int64_t *__restrict__ rowptr,
-                                                          const int32_t *__restrict__ perm, int nheavy, int seg_len,
-                                                          int64_t *__restrict__ nseg) {
-    const int h = (int)blockIdx.x * 256 + (int)threadIdx.x;
-    if (h >= nheavy) return;
-    const int r = perm[h];
-    const int64_t d = rowptr[r + 1] - rowptr[r];
-    nseg[h] = (d + seg_len - 1) / seg_len;
-}
-
-// One thread per segment: find its row by binary search in segbase, write (start, len).
-__global__ __launch_bounds__(256) void heavy_expand_kernel(const int64_t *__restrict__ rowptr,
-                                                           const int32_t *__restrict__ perm,
-                                                           const int64_t *__restrict__ segbase, int nheavy,
-                                                           int64_t nseg_total, int seg_len,
-                                                           int64_t *__restrict__ seg_start,
-                                                           int32_t *__restrict__ seg_n) {
-    const int64_t s = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (s >= nseg_total) return;
-    int lo = 0, hi = nheavy;  // last h with segbase[h] <= s
-    while (hi - lo > 1) {
-        const int mid = (lo + hi) >> 1;
-        if (segbase[mid] <= s) lo = mid; else hi = mid;
-    }
-    const int r = perm[lo];
-    const int64_t k = s - segbase[lo];
-    const int64_t b = rowptr[r] + k * seg_len;
-    const int64_t e = rowptr[r + 1];
-    seg_start[s] = b;
-    seg_n[s] = (int32_t)((e - b) < seg_len ? (e - b) : seg_len);
 }
 
 int env_int(const char *name, int dflt, int lo, int hi) {
@@ -219,25 +163,18 @@ using namespace gnnagg;
 
 struct gnnagg_plan {
     int64_t rows = 0, cols = 0, nnz = 0;
-    int seg_len = 0;          // nnz per segment of a cut row
-    int heavy_thresh = 0;     // rows longer than this are cut
-    int64_t nheavy = 0;       // rows cut into segments
-    int64_t nseg = 0;         // segments
-    int64_t nempty = 0;       // rows with no stored element
+    int long_thresh = 0;      // rows longer than this get a lane group of their own (head region)
+    int64_t nlong = 0;        // such rows (the first nlong entries of perm)
+    int64_t nempty = 0;       // rows with no stored element (the last nempty entries of perm)
     int64_t max_deg = 0;
     int device = 0;
-    int64_t *rowptr = nullptr;     // [rows+1] own copy
-    int32_t *col32 = nullptr;      // [nnz]
-    int32_t *perm = nullptr;       // [rows] rows by class: cut rows, then descending degree, then empty
-    int64_t *segbase = nullptr;    // [nheavy+1]
-    int64_t *seg_start = nullptr;  // [nseg]
-    int32_t *seg_n = nullptr;      // [nseg]
-    float *partial = nullptr;      // [nseg, partial_feat] scratch of segment sums
-    int64_t partial_feat = 0;
+    int64_t *rowptr = nullptr;  // [rows+1] own copy
+    int32_t *col32 = nullptr;   // [nnz]
+    int32_t *perm = nullptr;    // [rows] rows by degree class, longest first; ascending row id inside a class
     int rows_per_group = 4;
     bool profile = false;
     bool profile_valid = false;
-    hipEvent_t ev[4] = {nullptr, nullptr, nullptr, nullptr};  // call begin, rows-kernel begin/end, call end
+    hipEvent_t ev[4] = {nullptr, nullptr, nullptr, nullptr};  // call begin, main-kernel begin/end, call end
 };
 
 extern "C" int gnnagg_abi_version(void) { return GNNAGG_ABI_VERSION; }
@@ -256,7 +193,8 @@ extern "C" int gnnagg_spmm_csr_f32(const int64_t *rowptr, const int64_t *col, co
                    (long long)feat);
     if (sparse_rows == 0 || feat == 0) return GNNAGG_OK;
     GNNAGG_REQUIRE(rowptr && out, "null rowptr/out");
-    GNNAGG_REQUIRE(col && value && mat, "null col/value/mat");
+    // col/value/mat may be null only for a matrix without stored elements, which this
+    // entry point cannot tell (nnz is not an argument); they are not dereferenced then
     if (int rc = check_feat(feat)) return rc;
     if (sparse_rows >= (int64_t(1) << 31))
         return fail(GNNAGG_ERR_UNSUPPORTED, "more than 2^31-1 sparse rows (%lld)", (long long)sparse_rows);
@@ -285,10 +223,6 @@ static void plan_free(gnnagg_plan *p) {
     (void)hipFree(p->rowptr);
     (void)hipFree(p->col32);
     (void)hipFree(p->perm);
-    (void)hipFree(p->segbase);
-    (void)hipFree(p->seg_start);
-    (void)hipFree(p->seg_n);
-    (void)hipFree(p->partial);
     for (hipEvent_t e : p->ev)
         if (e) (void)hipEventDestroy(e);
     delete p;
@@ -316,13 +250,9 @@ extern "C" int gnnagg_plan_create(const int64_t *rowptr, const int64_t *col, int
     p->rows = rows;
     p->cols = cols;
     p->nnz = nnz;
-    p->seg_len = env_int("GNNAGG_SEG_LEN", 256, 32, 1 << 20);
-    p->heavy_thresh = env_int("GNNAGG_HEAVY_THRESH", 2 * p->seg_len, p->seg_len, 1 << 24);
+    p->long_thresh = env_int("GNNAGG_LONG_THRESH", 256, 1, 1 << 30);
     p->rows_per_group = env_int("GNNAGG_ROWS_PER_GROUP", 4, 1, 1024);
     GNNAGG_HIP(hipGetDevice(&p->device));
-    const int heavy_log = ceil_log2_u64((uint64_t)p->heavy_thresh);
-    const int nclasses = heavy_log + 3;
-    GNNAGG_REQUIRE(nclasses <= kMaxClasses, "heavy threshold too large");
 
     // rowptr end points (host check; also forces the inputs to be ready)
     int64_t ends[2] = {0, 0};
@@ -349,7 +279,7 @@ extern "C" int gnnagg_plan_create(const int64_t *rowptr, const int64_t *col, int
         GNNAGG_HIP(key_out.alloc((size_t)rows));
         GNNAGG_HIP(row_in.alloc((size_t)rows));
         hipLaunchKernelGGL(classify_rows_kernel, dim3(grid_for(rows, 256)), dim3(256), 0, st, p->rowptr, (int)rows,
-                           p->heavy_thresh, heavy_log, key_in.p, row_in.p, d_out.p);
+                           key_in.p, row_in.p, d_out.p);
         GNNAGG_HIP(hipGetLastError());
         if (nnz > 0) {
             const unsigned g = (unsigned)std::min<int64_t>((nnz + 255) / 256, 1 << 20);
@@ -358,44 +288,23 @@ extern "C" int gnnagg_plan_create(const int64_t *rowptr, const int64_t *col, int
         }
         // stable sort of the rows by class: ascending row id inside a class
         size_t tmp_bytes = 0;
-        const int end_bit = std::max(1, ceil_log2_u64((uint64_t)nclasses));
         GNNAGG_HIP(hipcub::DeviceRadixSort::SortPairs(nullptr, tmp_bytes, key_in.p, key_out.p, row_in.p, p->perm,
-                                                      (int)rows, 0, end_bit, st));
+                                                      (int)rows, 0, kClassBits, st));
         DevBuf<char> tmp;
         GNNAGG_HIP(tmp.alloc(std::max<size_t>(tmp_bytes, 1)));
         GNNAGG_HIP(hipcub::DeviceRadixSort::SortPairs(tmp.p, tmp_bytes, key_in.p, key_out.p, row_in.p, p->perm,
-                                                      (int)rows, 0, end_bit, st));
+                                                      (int)rows, 0, kClassBits, st));
         GNNAGG_HIP(hipMemcpyAsync(&h_out, d_out.p, sizeof(ClassifyOut), hipMemcpyDeviceToHost, st));
         GNNAGG_HIP(hipStreamSynchronize(st));
     }
     GNNAGG_REQUIRE(!h_out.bad_rowptr, "rowptr is not non-decreasing");
     GNNAGG_REQUIRE(!h_out.bad_col, "a column index lies outside [0, %lld)", (long long)cols);
-    p->nheavy = (int64_t)h_out.class_count[0];
-    p->nempty = (int64_t)h_out.class_count[nclasses - 1];
+    p->nempty = (int64_t)h_out.class_count[kEmptyClass];
     p->max_deg = (int64_t)h_out.max_deg;
+    // rows strictly longer than long_thresh: whole classes above the threshold's class
+    const int thresh_class = degree_class(p->long_thresh);
+    for (int c = 0; c < thresh_class; ++c) p->nlong += (int64_t)h_out.class_count[c];
 
-    if (p->nheavy > 0) {
-        DevBuf<int64_t> nseg;
-        GNNAGG_HIP(nseg.alloc((size_t)p->nheavy + 1));
-        GNNAGG_HIP(hipMemsetAsync(nseg.p, 0, sizeof(int64_t) * ((size_t)p->nheavy + 1), st));
-        hipLaunchKernelGGL(heavy_count_kernel, dim3(grid_for(p->nheavy, 256)), dim3(256), 0, st, p->rowptr, p->perm,
-                           (int)p->nheavy, p->seg_len, nseg.p);
-        GNNAGG_HIP(hipGetLastError());
-        GNNAGG_HIP(hipMalloc((void **)&p->segbase, sizeof(int64_t) * ((size_t)p->nheavy + 1)));
-        size_t tmp_bytes = 0;
-        GNNAGG_HIP(hipcub::DeviceScan::ExclusiveSum(nullptr, tmp_bytes, nseg.p, p->segbase, (int)p->nheavy + 1, st));
-        DevBuf<char> tmp;
-        GNNAGG_HIP(tmp.alloc(std::max<size_t>(tmp_bytes, 1)));
-        GNNAGG_HIP(hipcub::DeviceScan::ExclusiveSum(tmp.p, tmp_bytes, nseg.p, p->segbase, (int)p->nheavy + 1, st));
-        GNNAGG_HIP(hipMemcpyAsync(&p->nseg, p->segbase + p->nheavy, sizeof(int64_t), hipMemcpyDeviceToHost, st));
-        GNNAGG_HIP(hipStreamSynchronize(st));
-        GNNAGG_HIP(hipMalloc((void **)&p->seg_start, sizeof(int64_t) * (size_t)p->nseg));
-        GNNAGG_HIP(hipMalloc((void **)&p->seg_n, sizeof(int32_t) * (size_t)p->nseg));
-        hipLaunchKernelGGL(heavy_expand_kernel, dim3(grid_for(p->nseg, 256)), dim3(256), 0, st, p->rowptr, p->perm,
-                           p->segbase, (int)p->nheavy, p->nseg, p->seg_len, p->seg_start, p->seg_n);
-        GNNAGG_HIP(hipGetLastError());
-        GNNAGG_HIP(hipStreamSynchronize(st));
-    }
     guard.p = nullptr;
     *plan_out = p;
     return GNNAGG_OK;
@@ -413,11 +322,11 @@ extern "C" int gnnagg_plan_info(const gnnagg_plan *plan, int64_t *info) {
     info[0] = plan->rows;
     info[1] = plan->cols;
     info[2] = plan->nnz;
-    info[3] = plan->nheavy;
-    info[4] = plan->nseg;
-    info[5] = plan->seg_len;
-    info[6] = plan->nempty;
-    info[7] = plan->max_deg;
+    info[3] = plan->nlong;
+    info[4] = plan->long_thresh;
+    info[5] = plan->nempty;
+    info[6] = plan->max_deg;
+    info[7] = plan->rows_per_group;
     return GNNAGG_OK;
 }
 
@@ -431,19 +340,9 @@ extern "C" int gnnagg_plan_spmm_f32(gnnagg_plan *plan, const float *value, const
     if (int rc = check_feat(feat)) return rc;
     hipStream_t st = static_cast<hipStream_t>(stream);
 
-    if (plan->nseg > 0 && plan->partial_feat < feat) {
-        GNNAGG_HIP(hipDeviceSynchronize());
-        (void)hipFree(plan->partial);
-        plan->partial = nullptr;
-        plan->partial_feat = 0;
-        GNNAGG_HIP(hipMalloc((void **)&plan->partial, sizeof(float) * (size_t)plan->nseg * (size_t)feat));
-        plan->partial_feat = feat;
-    }
-
-    // the scratch of segment sums comes from hipMalloc (256-byte aligned) and has row
-    // stride `feat`, so it never lowers the vector width chosen for mat/out
     const int vec = pick_vec(feat, mat, out);
-    const int64_t nrow_tasks = plan->rows - plan->nheavy - (accumulate ? plan->nempty : 0);
+    // accumulate: empty rows keep their value, so they are not visited at all
+    const int64_t nshort = plan->rows - plan->nlong - (accumulate ? plan->nempty : 0);
     const bool prof = plan->profile;
     if (prof) {
         plan->profile_valid = false;
@@ -451,45 +350,25 @@ extern "C" int gnnagg_plan_spmm_f32(gnnagg_plan *plan, const float *value, const
     }
     for (int64_t f_base = 0; f_base < feat;) {
         const Shape s = pick_shape(vec, feat - f_base);
-        if (plan->nseg > 0) {
-            SpmmArgs a{};
-            a.seg_start = plan->seg_start;
-            a.seg_len = plan->seg_n;
-            a.col = plan->col32;
-            a.val = value;
-            a.x = mat;
-            a.dst = plan->partial;
-            a.ntasks = plan->nseg;
-            a.feat = (int)feat;
-            a.f_base = (int)f_base;
-            GNNAGG_HIP((dispatch_tasks<int32_t, kSegments>(s, a, 1, st)));
-            ReduceArgs r{};
-            r.heavy_row = plan->perm;
-            r.heavy_segbase = plan->segbase;
-            r.partial = plan->partial;
-            r.out = out;
-            r.nheavy = (int)plan->nheavy;
-            r.feat = (int)feat;
-            r.f_base = (int)f_base;
-            r.accumulate = accumulate;
-            GNNAGG_HIP(dispatch_reduce(s, r, st));
-        }
-        if (nrow_tasks > 0) {
-            SpmmArgs a{};
-            a.rowptr = plan->rowptr;
-            a.perm = plan->perm + plan->nheavy;
-            a.col = plan->col32;
-            a.val = value;
-            a.x = mat;
-            a.dst = out;
-            a.ntasks = nrow_tasks;
-            a.feat = (int)feat;
-            a.f_base = (int)f_base;
-            a.accumulate = accumulate;
-            const bool first_tile = prof && f_base == 0;
-            if (first_tile) GNNAGG_HIP(hipEventRecord(plan->ev[1], st));
+        SpmmArgs a{};
+        a.rowptr = plan->rowptr;
+        a.col = plan->col32;
+        a.val = value;
+        a.x = mat;
+        a.dst = out;
+        a.feat = (int)feat;
+        a.f_base = (int)f_base;
+        a.accumulate = accumulate;
+        // one launch over every row, longest first; the rows above the long-row threshold
+        // form the head region (one lane group per row)
+        if (plan->nlong + nshort > 0) {
+            const bool timed = prof && f_base == 0;
+            a.perm = plan->perm;
+            a.ntasks = plan->nlong + nshort;
+            a.head_tasks = plan->nlong;
+            if (timed) GNNAGG_HIP(hipEventRecord(plan->ev[1], st));
             GNNAGG_HIP((dispatch_tasks<int32_t, kRowsPermuted>(s, a, plan->rows_per_group, st)));
-            if (first_tile) {
+            if (timed) {
                 GNNAGG_HIP(hipEventRecord(plan->ev[2], st));
                 plan->profile_valid = true;
             }

@@ -1,8 +1,7 @@
 // Device kernels of the CSR SpMM (out (+)= A @ X, fp32) for gfx950.
 //
-// Work decomposition.  A "task" is one sparse row, or one fixed-length segment of a
-// long row.  A wavefront (64 lanes) is cut into groups of LPR lanes; one group owns one
-// task at a time.  Inside a group the lanes lie ALONG THE FEATURE DIMENSION: lane l
+// Work decomposition.  A "task" is one sparse row.  A wavefront (64 lanes) is cut into
+// groups of LPR lanes; one group owns one task at a time.  Inside a group the lanes lie ALONG THE FEATURE DIMENSION: lane l
 // holds features [(k*LPR + l)*VEC, +VEC) for k < NCH, so every gather of a dense row
 // X[col,:] is one contiguous, fully coalesced run of LPR*VEC*4 bytes per k.
 //
@@ -13,10 +12,12 @@
 // are issued back to back before their FMAs so that each group keeps UNROLL*NCH
 // vector loads in flight -- the kernel is bound by HBM latency/bandwidth, not issue.
 //
-// Arithmetic.  A row is one fp32 FMA chain in CSR order starting from the value in
-// `out` (or 0), i.e. the recurrence of the reference's kernel_1xN
-// (self_benchmark/a64fx/model/ops/src/spmm.cpp:37-53).  Rows cut into segments add
-// their segment sums in segment order afterwards (fixed order, no atomics).
+// Arithmetic.  EVERY row, whatever its length, is one fp32 FMA chain in CSR order
+// starting from the value in `out` (or 0), i.e. the recurrence of the reference's
+// kernel_1xN (self_benchmark/a64fx/model/ops/src/spmm.cpp:37-53): results are
+// bit-identical to the reference's CPU operator.  Long rows are therefore not split over
+// their stored elements; the plan schedules them first, one lane group each, and the
+// short rows fill in behind them.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -110,32 +111,61 @@ __device__ __forceinline__ int64_t uniform_i64(int64_t v) {
     return ((int64_t)hi << 32) | (uint32_t)lo;
 }
 
+// UU gathers issued back to back, then their FMAs in CSR order: elements j .. j+UU-1 of
+// the chunk held in (c_l, v_l) across the group's lanes.
+template <int UU, int VEC, int LPR, int NCH, typename IdxT>
+__device__ __forceinline__ void gather_fma(FVec<VEC> (&acc)[NCH], IdxT c_l, float v_l, int j,
+                                           const float *__restrict__ x, int F, const int (&foff)[NCH]) {
+    const float *xr[UU];
+    float vv[UU];
+#pragma unroll
+    for (int u = 0; u < UU; ++u) {
+        const int64_t c = group_bcast_idx<LPR>(c_l, j + u);
+        vv[u] = __int_as_float(group_bcast<LPR>(__float_as_int(v_l), j + u));
+        xr[u] = x + (size_t)c * (size_t)F;
+    }
+    FVec<VEC> xv[UU][NCH];
+#pragma unroll
+    for (int u = 0; u < UU; ++u) {
+#pragma unroll
+        for (int k = 0; k < NCH; ++k) xv[u][k] = FVec<VEC>::load(xr[u] + foff[k]);
+    }
+#pragma unroll
+    for (int u = 0; u < UU; ++u) {
+#pragma unroll
+        for (int k = 0; k < NCH; ++k) acc[k].fma(vv[u], xv[u][k]);
+    }
+}
+
 enum TaskMode : int {
     kRowsNatural = 0,  // task t is row t
-    kRowsPermuted = 1, // task t is row perm[t]
-    kSegments = 2      // task t is nnz range [seg_start[t], +seg_len[t]) -> partial[t,:]
+    kRowsPermuted = 1  // task t is row perm[t]
 };
 
 struct SpmmArgs {
-    const int64_t *rowptr;    // [rows+1]                      (row modes)
+    const int64_t *rowptr;    // [rows+1]
     const int32_t *perm;      // [ntasks] row of task t        (kRowsPermuted)
-    const int64_t *seg_start; // [ntasks] first nnz of segment (kSegments)
-    const int32_t *seg_len;   // [ntasks] nnz in segment       (kSegments)
     const void *col;          // IdxT [nnz]
     const float *val;         // [nnz]
     const float *x;           // dense operand [K, F]
-    float *dst;               // out [rows, F], or partial [ntasks, F] for kSegments
+    float *dst;               // out [rows, F]
     int64_t ntasks;
     int feat;                 // F (row stride of x and dst, in floats)
     int f_base;               // first feature handled by this launch
-    int accumulate;           // row modes: start from dst (1) or from 0 (0)
-    int tasks_per_block;
+    int accumulate;           // start every row from dst (1) or from 0 (0)
+    int tasks_per_block;      // tasks handled by one block past the head region
+    int64_t head_tasks;       // the first head_tasks tasks (the longest rows) get one lane group each
+    int head_blocks;          // = ceil(head_tasks / groups per block)
 };
 
+// Gathers kept in flight per lane group, sized so that a wave stays near 64-90 VGPRs:
+// measured on MI355X, deeper unrolls (fewer waves per SIMD) bring nothing -- the
+// kernel already saturates the memory system.
 template <int VEC, int NCH>
 struct UnrollFor {
-    static constexpr int regs = VEC * NCH;
-    static constexpr int value = regs <= 4 ? 8 : (regs <= 8 ? 4 : (regs <= 20 ? 2 : 1));
+    static constexpr int regs = VEC * NCH;  // VGPRs per gathered row per lane
+    static constexpr int raw = 32 / regs;
+    static constexpr int value = raw >= 8 ? 8 : (raw >= 4 ? 4 : (raw >= 2 ? 2 : 1));
 };
 
 template <int VEC, int LPR, int NCH, typename IdxT, int MODE>
@@ -166,27 +196,27 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
         foff[k] = fok[k] ? f : a.f_base;
     }
 
-    const int64_t t0 = (int64_t)blockIdx.x * a.tasks_per_block;
-    int64_t t1 = t0 + a.tasks_per_block;
-    if (t1 > a.ntasks) t1 = a.ntasks;
+    // Head region: one task per lane group, so that no group queues several of the
+    // longest rows behind each other.  Blocks are dispatched in index order, hence the
+    // longest rows start first and the short ones fill in behind them.
+    int64_t t0, t1;
+    if ((int)blockIdx.x < a.head_blocks) {
+        t0 = (int64_t)blockIdx.x * GPB;
+        t1 = t0 + GPB;
+        if (t1 > a.head_tasks) t1 = a.head_tasks;
+    } else {
+        t0 = a.head_tasks + (int64_t)((int)blockIdx.x - a.head_blocks) * a.tasks_per_block;
+        t1 = t0 + a.tasks_per_block;
+        if (t1 > a.ntasks) t1 = a.ntasks;
+    }
 
     for (int64_t t = t0 + group; t < t1; t += GPB) {
-        int64_t start, end;
-        float *dst;
-        bool from_dst;
-        if constexpr (MODE == kSegments) {
-            start = a.seg_start[t];
-            end = start + a.seg_len[t];
-            dst = a.dst + (size_t)t * (size_t)F;
-            from_dst = false;
-        } else {
-            int64_t row = t;
-            if constexpr (MODE == kRowsPermuted) row = a.perm[t];
-            start = a.rowptr[row];
-            end = a.rowptr[row + 1];
-            dst = a.dst + (size_t)row * (size_t)F;
-            from_dst = a.accumulate != 0;
-        }
+        int64_t row = t;
+        if constexpr (MODE == kRowsPermuted) row = a.perm[t];
+        int64_t start = a.rowptr[row];
+        int64_t end = a.rowptr[row + 1];
+        float *dst = a.dst + (size_t)row * (size_t)F;
+        const bool from_dst = a.accumulate != 0;
         if constexpr (LPR == 64) {
             start = uniform_i64(start);
             end = uniform_i64(end);
@@ -208,34 +238,18 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
                 c_l = __builtin_nontemporal_load(col + base + lig);
                 v_l = __builtin_nontemporal_load(val + base + lig);
             }
+            // full blocks of U gathers, then a halving cascade for what is left, so that a
+            // chunk of cnt elements costs at most cnt/U + log2(U) dependent round trips
             int j = 0;
-            for (; j + U <= cnt; j += U) {
-                const float *xr[U];
-                float vv[U];
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const int64_t c = group_bcast_idx<LPR>(c_l, j + u);
-                    vv[u] = __int_as_float(group_bcast<LPR>(__float_as_int(v_l), j + u));
-                    xr[u] = x + (size_t)c * (size_t)F;
-                }
-                V xv[U][NCH];
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-#pragma unroll
-                    for (int k = 0; k < NCH; ++k) xv[u][k] = V::load(xr[u] + foff[k]);
-                }
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-#pragma unroll
-                    for (int k = 0; k < NCH; ++k) acc[k].fma(vv[u], xv[u][k]);
-                }
+            for (; j + U <= cnt; j += U) gather_fma<U, VEC, LPR, NCH>(acc, c_l, v_l, j, x, F, foff);
+            if constexpr (U > 4) {
+                if (j + 4 <= cnt) { gather_fma<4, VEC, LPR, NCH>(acc, c_l, v_l, j, x, F, foff); j += 4; }
             }
-            for (; j < cnt; ++j) {
-                const int64_t c = group_bcast_idx<LPR>(c_l, j);
-                const float v = __int_as_float(group_bcast<LPR>(__float_as_int(v_l), j));
-                const float *xr = x + (size_t)c * (size_t)F;
-#pragma unroll
-                for (int k = 0; k < NCH; ++k) acc[k].fma(v, V::load(xr + foff[k]));
+            if constexpr (U > 2) {
+                if (j + 2 <= cnt) { gather_fma<2, VEC, LPR, NCH>(acc, c_l, v_l, j, x, F, foff); j += 2; }
+            }
+            if constexpr (U > 1) {
+                if (j + 1 <= cnt) { gather_fma<1, VEC, LPR, NCH>(acc, c_l, v_l, j, x, F, foff); j += 1; }
             }
         }
 
@@ -243,39 +257,6 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
         for (int k = 0; k < NCH; ++k) {
             if (fok[k]) acc[k].store(dst + foff[k]);
         }
-    }
-}
-
-// out[row,:] (+)= sum over the row's segment partial sums, in segment order.
-struct ReduceArgs {
-    const int32_t *heavy_row;     // [nheavy]
-    const int64_t *heavy_segbase; // [nheavy+1]
-    const float *partial;         // [nseg, F]
-    float *out;
-    int nheavy;
-    int feat;
-    int f_base;
-    int accumulate;
-};
-
-template <int VEC, int LPR, int NCH>
-__global__ __launch_bounds__(256) void heavy_reduce_kernel(const ReduceArgs a) {
-    constexpr int GPB = 256 / LPR;
-    typedef FVec<VEC> V;
-    const int lig = (int)threadIdx.x & (LPR - 1);
-    const int group = (int)threadIdx.x / LPR;
-    const int h = (int)blockIdx.x * GPB + group;
-    if (h >= a.nheavy) return;
-    const int F = a.feat;
-    const int64_t s0 = a.heavy_segbase[h], s1 = a.heavy_segbase[h + 1];
-    float *dst = a.out + (size_t)a.heavy_row[h] * (size_t)F;
-#pragma unroll
-    for (int k = 0; k < NCH; ++k) {
-        const int f = a.f_base + (k * LPR + lig) * VEC;
-        if (f >= F) continue;
-        V acc = a.accumulate ? V::load(dst + f) : V::zero();
-        for (int64_t s = s0; s < s1; ++s) acc.add(V::load(a.partial + (size_t)s * (size_t)F + f));
-        acc.store(dst + f);
     }
 }
 

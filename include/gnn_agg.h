@@ -60,9 +60,10 @@ int gnnagg_spmm_csr_f32(const int64_t *rowptr, const int64_t *col, const float *
  * Replaces the per-matrix CPU work split the reference computes once and caches on
  * the sparse object: distribute_work_for_row + get/set_work_range[_for_transpose]
  * (model/ops/spmm_kernel.py:7-28, :48-57, :80-87).  On the GPU the cached object is a
- * degree-binned row schedule: rows ordered by degree class, rows longer than a
- * threshold cut into fixed-length segments whose partial sums are combined in a fixed
- * order, and column indices narrowed to int32.
+ * degree-binned row schedule: rows ordered by degree class (powers of two of the row
+ * length), longest rows first, and column indices narrowed to int32.  Every row is
+ * still one fp32 FMA chain in CSR order, so results are bit-identical to
+ * gnnagg_spmm_csr_f32 and to the reference's CPU operator.
  *
  * gnnagg_plan_create reads rowptr/col on `stream`, validates them (rowptr[0]==0,
  * non-decreasing, rowptr[rows]==nnz, 0 <= col < cols) and SYNCHRONISES the stream; it
@@ -81,20 +82,20 @@ int gnnagg_plan_destroy(gnnagg_plan *plan);
  * the plan was built from.  accumulate != 0: out += A@mat (the reference semantics,
  * spmm.cpp:32-35).  accumulate == 0: out = A@mat, every row written (fuses the
  * `torch.zeros` the reference allocates before the local aggregation,
- * model/layers/aggregator.py:67-70, :167-170).  May grow a plan-owned scratch buffer
- * (hipMalloc, synchronising) the first time a larger `feat` is seen.  Calls sharing a
- * plan must be on one stream or otherwise ordered. */
+ * model/layers/aggregator.py:67-70, :167-170).  Allocates nothing and does not
+ * synchronise. */
 int gnnagg_plan_spmm_f32(gnnagg_plan *plan, const float *value, const float *mat, float *out, int64_t feat,
                          int accumulate, void *stream);
 
 /* Host-side description of a plan, info[0..7] (host pointer):
- * rows, cols, nnz, rows cut into segments, segments, segment length,
- * rows with no stored element, largest row length. */
+ * rows, cols, nnz, rows above the long-row threshold, that threshold,
+ * rows with no stored element, largest row length, rows handled per lane group. */
 int gnnagg_plan_info(const gnnagg_plan *plan, int64_t *info);
 
 /* Kernel timing of a plan, for benchmarks.  After gnnagg_plan_profile(plan, 1) every
  * gnnagg_plan_spmm_f32 call records HIP events on its stream around the whole call and
- * around its dominant kernel (the one that walks the rows that are not cut).
+ * around its dominant kernel (the launch that walks the rows of the first feature tile;
+ * the only launch unless the feature row is wider than one tile).
  * gnnagg_plan_profile_read SYNCHRONISES on the last recorded events and returns, in
  * milliseconds, ms[0] = that kernel, ms[1] = the whole call (all kernels), of the most
  * recent call (host pointer; -1 when nothing was recorded).  Replaces the std::chrono

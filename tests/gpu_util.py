@@ -15,6 +15,15 @@ def assert_close(got: torch.Tensor, want: np.ndarray, what: str = ""):
     assert err.max(initial=-1.0) <= 0.0, f"{what}: worst excess {err.max():.3e} at {np.unravel_index(err.argmax(), err.shape)}"
 
 
+def assert_math_close(got: torch.Tensor, want_fp64: np.ndarray, what: str = ""):
+    """Against an exact (fp64, differently associated) product: only fp32 rounding of sums
+    with cancellation separates the two, so this is a looser, independent sanity bound --
+    the parity gate proper is assert_close against the oracle."""
+    got = got.detach().cpu().numpy().astype(np.float64)
+    assert got.shape == want_fp64.shape, (what, got.shape, want_fp64.shape)
+    assert np.allclose(got, want_fp64, rtol=1e-4, atol=1e-4), f"{what}: max abs diff {np.abs(got - want_fp64).max():.3e}"
+
+
 def random_csr(rows, cols, density, seed, dtype=np.float32):
     a = sp.rand(rows, cols, density=density, format="csr", dtype=dtype, random_state=seed)
     a.sort_indices()

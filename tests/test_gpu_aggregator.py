@@ -1,0 +1,197 @@
+"""GPU parity of the aggregation pipeline (pre-aggregation, local SpMM, post-aggregation
+and their transposes behind the ``Aggregator`` autograd.Function) and of the index maps
+built on the device, against the CPU oracle.
+
+A small partitioned world is held on one GPU: every rank's graph is built with the
+product's own builders, the setup-time and per-layer exchanges are played by moving
+buffers between the simulated ranks.  Checks: (1) int64 maps / CSR arrays bit-identical
+to the oracle's; (2) forward output and input gradient bit-identical to the oracle
+pipeline (same FMA chains) and equal to the plain global product within rel 1e-5 /
+abs 1e-6; (3) the autograd contract of the reference (6-argument apply, gradient only
+for the features)."""
+import numpy as np
+import pytest
+import torch
+
+from gnn_benchmark_amd import Aggregator, SPMM_backward, SPMM_forward
+from gnn_benchmark_amd.data_manager import (DataProcessor, DataProcessorForPreAggresive, get_distributed_graph,
+                                            get_distributed_graph_for_pre_aggressive)
+from oracle import aggregator as oagg
+from oracle import index_maps as om
+from tests.gpu_util import assert_close, assert_math_close, dev
+from tests.test_pipeline_invariant import build_pre_world, exchange as host_exchange
+from tests.world_sim import World
+
+pytestmark = pytest.mark.gpu
+
+
+def _csr_np(m):
+    return [t.cpu().numpy() for t in m.csr()]
+
+
+def _same_matrix(got, want):
+    rowptr, col, val = _csr_np(got)
+    assert tuple(got.sparse_sizes()) == tuple(want[3])
+    assert np.array_equal(rowptr, want[0]) and np.array_equal(col, want[1]) and np.array_equal(val, want[2])
+
+
+class PlayedExchange:
+    """Per-layer exchange of one simulated rank: the rows the peers would deliver were
+    computed beforehand; this copies them into the buffer the aggregator reads next."""
+
+    def __init__(self, forward_rows, backward_rows):
+        self.forward_rows, self.backward_rows = forward_rows, backward_rows
+        self.log = []
+
+    def __call__(self, comm_splits, comm_buf, tag, direction):
+        self.log.append((tag, direction))
+        if direction == "forward":
+            comm_buf.recv_buf.copy_(self.forward_rows)
+        else:
+            comm_buf.send_buf.copy_(self.backward_rows)
+        return None
+
+
+def _build_pre_graphs(w: World, feat):
+    W = w.world
+    parts = [w.partition(r) for r in range(W)]
+    sent = []
+    for r in range(W):
+        remote_g = [dev(parts[r][1][0]), dev(parts[r][1][1] + w.begins[r])]
+        sent.append(DataProcessorForPreAggresive.split_remote_edges_for_aggr_and_graph_exchange(
+            torch.from_numpy(w.begins), remote_g, W)[0])
+    graphs = []
+    for r in range(W):
+        graphs.append(get_distributed_graph_for_pre_aggressive(
+            torch.from_numpy(parts[r][0].copy()), torch.from_numpy(parts[r][1].copy()), torch.from_numpy(w.begins),
+            int(w.sizes[r]), feat, r, W, 32, graph_exchange=lambda _s, r=r: [sent[i][r] for i in range(W)],
+            device="cuda"))
+    return graphs
+
+
+@pytest.mark.parametrize("seed,sizes", [(0, (300, 450, 250)), (1, (600, 1, 400, 330)), (2, (500, 0, 500))])
+def test_pre_post_world_matches_oracle_and_global_product(seed, sizes):
+    w = World(seed, sizes, mean_deg=8.0)
+    W, F = w.world, 48
+    graphs = _build_pre_graphs(w, F)
+    oracle_ranks = build_pre_world(w)
+    for r in range(W):
+        _same_matrix(graphs[r].local_adj_t, oracle_ranks[r]["local"])
+        _same_matrix(graphs[r].adj_t_pre_post_aggr_from, oracle_ranks[r]["a_from"])
+        _same_matrix(graphs[r].adj_t_pre_post_aggr_to, oracle_ranks[r]["a_to"])
+        assert graphs[r].comm_splits.recv_splits == oracle_ranks[r]["recv_splits"]
+        assert graphs[r].comm_splits.send_splits == oracle_ranks[r]["send_splits"]
+        part_local, part_remote = w.partition(r)
+        assert np.array_equal(graphs[r].in_degrees.cpu().numpy(), om.get_in_degrees(part_local, part_remote, int(sizes[r])))
+
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((w.n, F)).astype(np.float32)
+    g = rng.standard_normal((w.n, F)).astype(np.float32)
+    sl = [slice(int(w.begins[r]), int(w.begins[r + 1])) for r in range(W)]
+
+    # what every rank puts on the wire, computed with the product's own operators
+    send, back = [], []
+    for r in range(W):
+        gr = graphs[r]
+        s = torch.zeros(sum(gr.comm_splits.send_splits), F, device="cuda")
+        SPMM_forward(gr.adj_t_pre_post_aggr_to, dev(x[sl[r]]), s)
+        b = torch.zeros(sum(gr.comm_splits.recv_splits), F, device="cuda")
+        SPMM_backward(gr.adj_t_pre_post_aggr_from, dev(g[sl[r]]), b)
+        send.append(s.cpu().numpy())
+        back.append(b.cpu().numpy())
+    recv = host_exchange(send, [gr.comm_splits.send_splits for gr in graphs], [gr.comm_splits.recv_splits for gr in graphs])
+    incoming = host_exchange(back, [gr.comm_splits.recv_splits for gr in graphs], [gr.comm_splits.send_splits for gr in graphs])
+
+    want, want_t = w.global_product(x), w.global_product(g, transposed=True)
+    for r in range(W):
+        gr, o = graphs[r], oracle_ranks[r]
+        gr.exchange = PlayedExchange(dev(recv[r]), dev(incoming[r]))
+        xr = dev(x[sl[r]]).requires_grad_()
+        out = Aggregator.apply(gr, xr, 3, 32, True, True)
+        assert np.array_equal(gr.comm_buf.send_buf.cpu().numpy(), oagg.forward_send(o["a_to"], np.ascontiguousarray(x[sl[r]])))
+        out.backward(dev(g[sl[r]]))
+        assert gr.exchange.log == [("forward3", "forward"), ("backward3", "backward")]
+        assert np.array_equal(gr.comm_buf.recv_buf.cpu().numpy(), oagg.backward_recv(o["a_from"], np.ascontiguousarray(g[sl[r]])))
+        o_out = oagg.forward_out(o["local"], o["a_from"], np.ascontiguousarray(x[sl[r]]), recv[r])
+        o_dx = oagg.backward_out(o["local"], o["a_to"], np.ascontiguousarray(g[sl[r]]), incoming[r])
+        assert np.array_equal(out.detach().cpu().numpy(), o_out)
+        assert np.array_equal(xr.grad.cpu().numpy(), o_dx)
+        assert_close(out, o_out, "forward vs oracle pipeline")
+        assert_close(xr.grad, o_dx, "gradient vs oracle pipeline")
+        assert_math_close(out, want[sl[r]], "forward vs global product")
+        assert_math_close(xr.grad, want_t[sl[r]], "gradient vs global transposed product")
+
+
+@pytest.mark.parametrize("seed,sizes", [(4, (300, 450, 250)), (5, (600, 1, 400, 330))])
+def test_raw_halo_world_matches_oracle_and_global_product(seed, sizes):
+    w = World(seed, sizes, mean_deg=8.0)
+    W, F = w.world, 40
+    parts = [w.partition(r) for r in range(W)]
+    # pass 1: halo id lists of every rank (what the id exchange moves)
+    halo = []
+    for r in range(W):
+        e = DataProcessor.sort_remote_edges_list_based_on_remote_nodes(dev(parts[r][1].copy()))
+        nodes, ranges, _ = DataProcessor.obtain_remote_nodes_list(e, int(sizes[r]), torch.from_numpy(w.begins), W)
+        halo.append((nodes, ranges))
+    graphs = []
+    for r in range(W):
+        begin = int(w.begins[r])
+        local_nodes_list = torch.stack((torch.arange(begin, begin + int(sizes[r])),) * 2, dim=1) if sizes[r] else torch.zeros((1, 2), dtype=torch.int64)
+        asked = lambda _s, r=r: [halo[i][0][int(halo[i][1][r]):int(halo[i][1][r + 1])] for i in range(W)]
+        graphs.append(get_distributed_graph(torch.from_numpy(parts[r][0].copy()), torch.from_numpy(parts[r][1].copy()),
+                                            local_nodes_list, torch.from_numpy(w.begins), int(sizes[r]), F, W, 32,
+                                            halo_id_exchange=asked, device="cuda"))
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((w.n, F)).astype(np.float32)
+    g = rng.standard_normal((w.n, F)).astype(np.float32)
+    sl = [slice(int(w.begins[r]), int(w.begins[r + 1])) for r in range(W)]
+    send = [x[sl[r]][graphs[r].idx_nodes_send_to_others.cpu().numpy()] for r in range(W)]
+    back = []
+    for r in range(W):
+        b = torch.zeros(sum(graphs[r].comm_splits.recv_splits), F, device="cuda")
+        SPMM_backward(graphs[r].remote_adj_t, dev(g[sl[r]]), b)
+        back.append(b.cpu().numpy())
+    send_splits = [gr.comm_splits.send_splits for gr in graphs]
+    recv_splits = [gr.comm_splits.recv_splits for gr in graphs]
+    recv = host_exchange(send, send_splits, recv_splits)
+    incoming = host_exchange(back, recv_splits, send_splits)
+    want, want_t = w.global_product(x), w.global_product(g, transposed=True)
+    for r in range(W):
+        gr = graphs[r]
+        gr.exchange = PlayedExchange(dev(recv[r]), dev(incoming[r]))
+        xr = dev(x[sl[r]]).requires_grad_()
+        out = Aggregator.apply(gr, xr, 0, 32, False, True)
+        assert np.array_equal(gr.comm_buf.send_buf.cpu().numpy(), send[r])  # the row gather
+        out.backward(dev(g[sl[r]]))
+        assert_math_close(out, want[sl[r]], "raw halo forward")
+        assert_math_close(xr.grad, want_t[sl[r]], "raw halo gradient")
+        local = _csr_np(gr.local_adj_t) + [gr.local_adj_t.sparse_sizes()]
+        remote = _csr_np(gr.remote_adj_t) + [gr.remote_adj_t.sparse_sizes()]
+        o_out = oagg.forward_out(local, remote, np.ascontiguousarray(x[sl[r]]), recv[r])
+        assert_close(out, o_out, "raw halo forward vs oracle")
+        assert np.array_equal(out.detach().cpu().numpy(), o_out)
+        # the oracle adds the incoming rows one by one in index order (index_add_); the
+        # product adds them per destination row in the same order: same chains
+        o_dx = oagg.backward_out_raw(local, gr.idx_nodes_send_to_others.cpu().numpy(), np.ascontiguousarray(g[sl[r]]), incoming[r])
+        assert_close(xr.grad, o_dx, "raw halo gradient vs oracle")
+
+
+def test_single_rank_world_and_autograd_contract():
+    w = World(9, (700,), mean_deg=6.0)
+    local, remote = w.partition(0)
+    gr = get_distributed_graph_for_pre_aggressive(torch.from_numpy(local), torch.from_numpy(remote),
+                                                  torch.from_numpy(w.begins), 700, 32, 0, 1, 32, device="cuda")
+    assert gr.exchange is None and gr.comm_buf.send_buf.shape[0] == 0 and gr.comm_buf.recv_buf.shape[0] == 0
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((700, 32)).astype(np.float32)
+    xr = dev(x).requires_grad_()
+    out = Aggregator.apply(gr, xr, 0, 32, True, True)
+    assert_math_close(out, w.global_product(x), "single rank")
+    g = rng.standard_normal((700, 32)).astype(np.float32)
+    grads = torch.autograd.grad(out, xr, dev(g))
+    assert len(grads) == 1
+    assert_math_close(grads[0], w.global_product(g, transposed=True), "single rank gradient")
+    ret = Aggregator.backward(type("Ctx", (), dict(graph=gr, num_bits=32, is_pre_delay=True, layer=0))(), dev(g))
+    assert len(ret) == 6 and all(ret[i] is None for i in (0, 2, 3, 4, 5))  # aggregator.py:208
+    with pytest.raises(NotImplementedError):
+        Aggregator.apply(gr, xr, 0, 2, True, True)
