@@ -1,19 +1,24 @@
 #!/usr/bin/env python3
 """Benchmark of the aggregation hot path on ONE MI355X.
 
-Default workload ("c2"): standalone CSR SpMM forward A @ X plus the transposed backward
-A^T @ G on a seeded power-law graph of 2.45 M nodes / ~124 M stored elements with
+Headline workload ("c2"): standalone CSR SpMM forward A @ X plus the transposed backward
+A^T @ G on a seeded power-law graph of 2.45 M nodes / ~122 M stored elements with
 GCN-normalised fp32 values and a 2.45 M x 100 fp32 dense operand.  One "step" is one
 forward plus one backward, with every input already resident in HBM.
 
 Prints ONE JSON line.  ``value`` is the FLOP rate of the whole step (2 * nnz * F per
 product).  ``roofline`` prices the dominant kernel (the forward's row kernel) against
-the 8 TB/s HBM peak with the no-reuse gather byte model:
+the 8 TB/s HBM peak with the no-reuse gather byte model
     bytes = nnz*(8+4) + (rows+1)*8 + nnz*F*4 + 2*rows*F*4
-over the rows / stored elements that kernel launch covers, divided by its duration
-measured with HIP events on the launch stream inside the timed region.
-``cpu_baseline`` is the reference's own compiled operator (or the C port of it when
-that is not available on the host) timed on this machine's cores on the same matrices.
+over the rows / stored elements that launch covers, divided by its duration measured
+with HIP events on the launch stream inside the timed region.  ``cpu_baseline`` is the
+reference's own compiled operator (or the C port of it when that cannot run on the
+host) timed on this machine's cores on the same matrices.
+
+``extra`` carries the other workloads, run after the timed headline: c2 at F=128/256,
+c3 (dense-degree mean aggregation, F=602/256), c4 (one partition of a 16-way split:
+pre-aggregation, local SpMM, post-aggregation, F=128) and c5 (3-layer GCN train step on
+the c4 partition).  ``--only headline`` skips them.
 """
 import argparse
 import json
@@ -27,6 +32,12 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak
 
+# HBM-side traffic of ONE forward launch of the headline workload (default arguments),
+# from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE:
+# FETCH_SIZE 27 980 938 KiB x 2.0 (the counter reads 0.5 KiB per KiB on a 1 GiB device copy)
+# + WRITE_SIZE 987 671 KiB x 1.0.  Keyed by (workload, nodes, mean out-degree, F, seed).
+MEASURED_TRAFFIC_BYTES = {("c2", 2_450_000, 25.0, 100, 0): (27_980_938 * 2.0 + 987_671) * 1024.0}
+
 
 def b_alg(nnz: int, rows: int, feat: int) -> float:
     """Algorithmic bytes of one out += A @ X call (no-reuse gather model)."""
@@ -38,27 +49,30 @@ def b_min(nnz: int, rows: int, cols: int, feat: int) -> float:
     return nnz * 12.0 + (rows + 1) * 8.0 + cols * feat * 4.0 + 2.0 * rows * feat * 4.0
 
 
-def rows_kernel_cover(src, plan_info):
-    """(rows, nnz) covered by the dominant kernel launch with accumulate=1: every row
-    that has a stored element (empty rows are not visited)."""
-    rowptr = src.csr()[0]
-    return plan_info["rows"] - plan_info["empty_rows"], int(rowptr[-1])
-
-
-def time_spmm(plan, value, x, out, steps, warmup):
-    """Median/mean of the dominant-kernel and whole-call durations over `steps` calls."""
-    import torch
-
+def time_plan(plan, value, x, out, steps, warmup, accumulate=True):
+    """Mean dominant-kernel and whole-call durations (ms) over `steps` calls, HIP events."""
     plan.profile(True)
     k_ms, c_ms = [], []
     for i in range(warmup + steps):
-        plan.spmm(value, x, out, accumulate=True)
+        plan.spmm(value, x, out, accumulate=accumulate)
         k, c = plan.profile_read()
         if i >= warmup:
             k_ms.append(k)
             c_ms.append(c)
     plan.profile(False)
-    return sum(k_ms) / len(k_ms), sum(c_ms) / len(c_ms), min(c_ms)
+    return sum(k_ms) / len(k_ms), sum(c_ms) / len(c_ms)
+
+
+def op_report(name, nnz, rows, cols, feat, ms, empty_rows=0):
+    """Rates of one accumulate call; rows without stored elements are neither read nor
+    written by the kernel, so they are left out of the byte model."""
+    rows_total, rows = rows, rows - empty_rows
+    gbs = b_alg(nnz, rows, feat) / (ms * 1e-3) / 1e9
+    return {"op": name, "rows": rows_total, "rows_visited": rows, "cols": cols, "nnz": nnz, "feat": feat,
+            "ms": round(ms, 4),
+            "gflops": round(2.0 * nnz * feat / (ms * 1e-3) / 1e9, 1), "gbs_model": round(gbs, 1),
+            "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
+            "gbs_floor": round(b_min(nnz, rows, cols, feat) / (ms * 1e-3) / 1e9, 1)}
 
 
 def cpu_baseline_spmm(src, x_host, g_host, reps=3):
@@ -114,94 +128,201 @@ def cpu_baseline_spmm(src, x_host, g_host, reps=3):
             "ms_per_step": round(sec * 1e3, 2)}
 
 
+def spmm_pair(src, feat, steps, warmup, gen):
+    """Times `steps` (forward + transposed backward) steps; returns (report, x, g)."""
+    import torch
+
+    rows, cols = src.sparse_sizes()
+    nnz = src.nnz()
+    dev = src.device
+    plan_f, plan_b = src.get_plan(), src.get_plan_for_transpose()
+    val, val_t = src.csr()[2], src.storage.value_T()
+    x = torch.randn(cols, feat, device=dev, generator=gen)
+    g = torch.randn(rows, feat, device=dev, generator=gen)
+    out = torch.zeros(rows, feat, device=dev)
+    dx = torch.zeros(cols, feat, device=dev)
+    for _ in range(warmup):
+        plan_f.spmm(val, x, out, True)
+        plan_b.spmm(val_t, g, dx, True)
+    plan_f.profile(True)
+    k_ms = []
+    torch.cuda.synchronize()
+    t_begin = time.perf_counter()
+    for _ in range(steps):
+        plan_f.spmm(val, x, out, True)
+        plan_b.spmm(val_t, g, dx, True)
+        k_ms.append(plan_f.profile_read()[0])
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t_begin) * 1e3 / steps
+    plan_f.profile(False)
+    kern_ms = sum(k_ms) / len(k_ms)
+    info = plan_f.info()
+    bytes_launch = b_alg(nnz, rows - info["empty_rows"], feat)  # empty rows are not visited
+    _, fwd_ms = time_plan(plan_f, val, x, out, max(3, steps // 2), 1)
+    _, bwd_ms = time_plan(plan_b, val_t, g, dx, max(3, steps // 2), 1)
+    r = {"feat": feat, "steps": steps, "ms_per_step": round(ms_step, 4),
+         "gflops": round(2 * 2.0 * nnz * feat / (ms_step * 1e-3) / 1e9, 2),
+         "forward": op_report("A@X", nnz, rows, cols, feat, fwd_ms, info["empty_rows"]),
+         "backward": op_report("A^T@G", nnz, cols, rows, feat, bwd_ms, plan_b.info()["empty_rows"]),
+         "kernel_ms": round(kern_ms, 4), "kernel_bytes": bytes_launch}
+    return r, x, g
+
+
 def run_c2(args):
     import torch
 
     from gnn_benchmark_amd import synthetic
 
     dev = "cuda:0"
-    feat = args.feat
     t0 = time.perf_counter()
     g = synthetic.power_law_graph(num_nodes=args.nodes, mean_out_degree=args.mean_out_degree, zipf_s=1.8,
                                   max_degree=15000, seed=args.seed, device=dev)
     src = g.adj
-    n, nnz = g.num_nodes, g.nnz
-    plan_f = src.get_plan()
-    plan_b = src.get_plan_for_transpose()
+    info = src.get_plan().info()
+    src.get_plan_for_transpose()
     torch.cuda.synchronize()
     setup_s = time.perf_counter() - t0
-    info = plan_f.info()
-    _, _, val = src.csr()
-    val_t = src.storage.value_T()
-
-    results = {}
     gen = torch.Generator(device=dev).manual_seed(args.seed)
-    feats = [feat] + [f for f in args.extra_feats if f != feat]
-    main = None
-    for f in feats:
-        x = torch.randn(n, f, device=dev, generator=gen)
-        gr = torch.randn(n, f, device=dev, generator=gen)
-        out = torch.zeros(n, f, device=dev)
-        dx = torch.zeros(n, f, device=dev)
-        steps, warmup = (args.steps, args.warmup) if f == feat else (max(3, args.steps // 4), 2)
-        # whole-step timing: exactly `steps` steps between two synchronisations
-        for _ in range(warmup):
-            plan_f.spmm(val, x, out, True)
-            plan_b.spmm(val_t, gr, dx, True)
-        plan_f.profile(True)
-        k_ms = []
-        torch.cuda.synchronize()
-        t_begin = time.perf_counter()
-        for _ in range(steps):
-            plan_f.spmm(val, x, out, True)
-            plan_b.spmm(val_t, gr, dx, True)
-            k_ms.append(plan_f.profile_read()[0])
-        torch.cuda.synchronize()
-        ms_step = (time.perf_counter() - t_begin) * 1e3 / steps
-        plan_f.profile(False)
-        kern_ms = sum(k_ms) / len(k_ms)
-        rows_cov, nnz_cov = rows_kernel_cover(src, info)
-        bytes_launch = b_alg(nnz_cov, rows_cov, f)
-        # separate forward / backward whole-call timings
-        _, fwd_ms, _ = time_spmm(plan_f, val, x, out, max(3, steps // 2), 1)
-        _, bwd_ms, _ = time_spmm(plan_b, val_t, gr, dx, max(3, steps // 2), 1)
-        r = {
-            "feat": f, "ms_per_step": round(ms_step, 4), "fwd_ms": round(fwd_ms, 4), "bwd_ms": round(bwd_ms, 4),
-            "gflops": round(2 * 2.0 * nnz * f / (ms_step * 1e-3) / 1e9, 2),
-            "fwd_gbs_model": round(b_alg(nnz, n, f) / (fwd_ms * 1e-3) / 1e9, 1),
-            "fwd_frac_of_hbm_peak": round(b_alg(nnz, n, f) / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-            "bwd_gbs_model": round(b_alg(nnz, n, f) / (bwd_ms * 1e-3) / 1e9, 1),
-            "fwd_gbs_floor": round(b_min(nnz, n, n, f) / (fwd_ms * 1e-3) / 1e9, 1),
-            "kernel_ms": round(kern_ms, 4), "kernel_bytes": bytes_launch, "steps": steps,
-        }
-        results[f] = r
-        if f == feat:
-            main = (r, x, gr)
-        else:
-            del x, gr
-        del out, dx
-    r, x, gr = main
+    r, x, gr = spmm_pair(src, args.feat, args.steps, args.warmup, gen)
+    achieved = r["kernel_bytes"] / (r["kernel_ms"] * 1e-3) / 1e9
+    traffic = MEASURED_TRAFFIC_BYTES.get(("c2", args.nodes, args.mean_out_degree, args.feat, args.seed))
     line = {
         "metric": "spmm_fwd_bwd_gflops", "value": r["gflops"], "unit": "GFLOP/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": r["ms_per_step"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"c2: CSR SpMM forward A@X + transposed backward A^T@G, power-law graph "
-                               f"{n} nodes / {nnz} nnz (Zipf s=1.8, max row {g.max_degree}), GCN-normalised fp32, "
-                               f"dense operand {n}x{feat} fp32",
-                   "nodes": n, "nnz": nnz, "feat": feat, "seed": args.seed, "long_rows": info["long_rows"],
-                   "max_row_len": info["max_row_len"], "setup_s": round(setup_s, 2)},
-        "roofline": {"bound": "hbm", "achieved": round(r["kernel_bytes"] / (r["kernel_ms"] * 1e-3) / 1e9, 1),
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(r["kernel_bytes"] / (r["kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                     "traffic": None, "kernel": "spmm_tasks_kernel (forward A@X, all rows)",
+                               f"{g.num_nodes} nodes / {g.nnz} nnz (Zipf s=1.8, longest row {g.max_degree}), "
+                               f"GCN-normalised fp32, dense operand {g.num_nodes}x{args.feat} fp32",
+                   "nodes": g.num_nodes, "nnz": g.nnz, "feat": args.feat, "seed": args.seed,
+                   "long_rows": info["long_rows"], "max_row_len": info["max_row_len"], "setup_s": round(setup_s, 2)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                     "kernel": "gnnagg::spmm_tasks_kernel<4,32,1,int,1> (forward A@X, one launch over all rows)",
                      "kernel_ms": r["kernel_ms"], "bytes_per_launch": r["kernel_bytes"]},
-        "extra": {"c2": [results[f] for f in feats]},
     }
-    if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline_spmm(src, x.cpu().numpy(), gr.cpu().numpy())
-    else:
-        line["cpu_baseline"] = None
-    return line
+    extra = {"c2": [r]}
+    if "c2" in args.extras:
+        for f in (128, 256):
+            if f != args.feat:
+                extra["c2"].append(spmm_pair(src, f, max(3, args.steps // 4), 2, gen)[0])
+    line["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline_spmm(src, x.cpu().numpy(), gr.cpu().numpy())
+    return line, extra
+
+
+def run_c3(args):
+    import torch
+
+    from gnn_benchmark_amd import synthetic
+
+    dev = "cuda:0"
+    g = synthetic.dense_degree_graph(num_nodes=233_000, mu=5.5, sigma=1.2, seed=args.seed, device=dev)
+    gen = torch.Generator(device=dev).manual_seed(args.seed + 3)
+    out = {"graph": g.description, "nodes": g.num_nodes, "nnz": g.nnz, "max_row_len": g.max_degree, "runs": []}
+    for f in (602, 256):
+        out["runs"].append(spmm_pair(g.adj, f, max(3, args.steps // 4), 2, gen)[0])
+    return out
+
+
+def build_c4(args):
+    import torch
+
+    from gnn_benchmark_amd import synthetic
+
+    dev = "cuda:0"
+    t0 = time.perf_counter()
+    part = synthetic.partition_edges(num_local_nodes=args.c4_nodes, world_size=16, rank=3,
+                                     local_mean_out_degree=6.8, zipf_s=1.8, max_degree=15000,
+                                     num_halo_nodes=int(args.c4_nodes * 3 / 7),
+                                     num_remote_edges=int(args.c4_nodes * 20 / 7), seed=args.seed + 4, device=dev)
+    exchange = synthetic.SeededHaloExchange(args.seed + 4)
+    graph = synthetic.build_partition_graph(part, 256, True, exchange=exchange, device=dev)
+    for m in (graph.local_adj_t, graph.adj_t_pre_post_aggr_from, graph.adj_t_pre_post_aggr_to):
+        m.get_plan()
+        m.get_plan_for_transpose()
+    torch.cuda.synchronize()
+    return part, graph, time.perf_counter() - t0
+
+
+def run_c4(args, graph, setup_s):
+    import torch
+
+    from gnn_benchmark_amd import Aggregator
+
+    dev = "cuda:0"
+    n, feat = graph.local_adj_t.sparse_size(0), 128
+    steps = max(5, args.steps // 2)
+    gen = torch.Generator(device=dev).manual_seed(args.seed + 5)
+    x = torch.randn(n, feat, device=dev, generator=gen)
+    g = torch.randn(n, feat, device=dev, generator=gen)
+    graph.comm_buf.resize_buffer(graph.comm_splits, feat, 32)
+    send_buf, recv_buf = graph.comm_buf.send_buf, graph.comm_buf.recv_buf
+    recv_buf.normal_(generator=gen)
+    out = torch.zeros(n, feat, device=dev)
+    ops = []
+    for name, m, src_x, dst in (("pre-aggregation A_to@X -> send_buf", graph.adj_t_pre_post_aggr_to, x, send_buf),
+                                ("local A_local@X -> out", graph.local_adj_t, x, out),
+                                ("post-aggregation A_from@recv_buf -> out", graph.adj_t_pre_post_aggr_from, recv_buf, out)):
+        rows, cols = m.sparse_sizes()
+        _, ms = time_plan(m.get_plan(), m.csr()[2], src_x, dst, steps, 2, accumulate=True)
+        ops.append(op_report(name, m.nnz(), rows, cols, feat, ms, m.get_plan().info()["empty_rows"]))
+        back = torch.zeros(cols, feat, device=dev)
+        _, ms = time_plan(m.get_plan_for_transpose(), m.storage.value_T(), dst, back, steps, 2, accumulate=True)
+        ops.append(op_report(name.split(" ")[0] + " transposed (gradient direction)", m.nnz(), cols, rows, feat, ms,
+                             m.get_plan_for_transpose().info()["empty_rows"]))
+        del back
+    # the whole autograd.Function, forward and backward, synthetic halo rows generated on the device
+    xr = x.clone().requires_grad_()
+    for _ in range(2):
+        Aggregator.apply(graph, xr, 0, 32, True, True).backward(g)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        o = Aggregator.apply(graph, xr, 0, 32, True, True)
+    torch.cuda.synchronize()
+    fwd_ms = (time.perf_counter() - t0) * 1e3 / steps
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        o = Aggregator.apply(graph, xr, 0, 32, True, True)
+        o.backward(g)
+    torch.cuda.synchronize()
+    both_ms = (time.perf_counter() - t0) * 1e3 / steps
+    return {"partition": f"rank 3 of 16, {n} local nodes", "feat": feat, "setup_s": round(setup_s, 2),
+            "local_nnz": graph.local_adj_t.nnz(), "halo_rows": int(recv_buf.size(0)), "send_rows": int(send_buf.size(0)),
+            "from_nnz": graph.adj_t_pre_post_aggr_from.nnz(), "to_nnz": graph.adj_t_pre_post_aggr_to.nnz(),
+            "ops": ops, "aggregator_forward_ms": round(fwd_ms, 3),
+            "aggregator_forward_backward_ms": round(both_ms, 3)}
+
+
+def run_c5(args, graph):
+    import torch
+
+    from gnn_benchmark_amd import gcn
+
+    dev = "cuda:0"
+    n = graph.local_adj_t.sparse_size(0)
+    dims = [128, 256, 256, 172]
+    gen = torch.Generator(device=dev).manual_seed(args.seed + 6)
+    x = torch.randn(n, dims[0], device=dev, generator=gen)
+    labels = torch.randint(0, dims[-1], (n,), device=dev, generator=gen)
+    train_idx = torch.randperm(n, device=dev, generator=gen)[: n // 10]
+    masks = gcn.make_dropout_masks(n, dims, 0.5, args.seed + 7, dev)
+    steps = max(3, args.steps // 4)
+    out = {"dims": dims, "nodes": n, "labelled": int(train_idx.numel()), "dropout": 0.5, "optimizer": "Adam(lr=0.01)",
+           "steps": steps}
+    for gemm in ("fp32", "bf16"):
+        torch.manual_seed(args.seed)
+        model = gcn.GCN(dims, gemm=gemm).to(dev)
+        opt = torch.optim.Adam(model.parameters(), lr=0.01)
+        losses = [float(gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks)) for _ in range(2)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            loss = gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks)
+        torch.cuda.synchronize()
+        out[f"train_step_ms_{gemm}_gemm"] = round((time.perf_counter() - t0) * 1e3 / steps, 2)
+        out[f"loss_{gemm}"] = [round(v, 5) for v in losses + [float(loss)]]
+        del model, opt
+    return out
 
 
 def main():
@@ -209,17 +330,19 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c2", choices=["c2"])
     ap.add_argument("--feat", type=int, default=100)
-    ap.add_argument("--extra-feats", type=int, nargs="*", default=[128, 256])
     ap.add_argument("--nodes", type=int, default=2_450_000)
     ap.add_argument("--mean-out-degree", type=float, default=25.0)
+    ap.add_argument("--c4-nodes", type=int, default=7_000_000)
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--only", default="", help="'headline' = headline workload only; or a comma list of the extra "
+                                                "workloads to add: c2 (F=128/256), c3, c4, c5.  Default: all of them")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy 3 times (a kernel of known traffic for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
+    args.extras = [s for s in (args.only.split(",") if args.only else ["c2", "c3", "c4", "c5"]) if s and s != "headline"]
     if args.gpus != 1:
         print("bench.py measures one GPU's share of the partitioned graph; --gpus must be 1 "
               "(no multi-GPU path exists in this build)", file=sys.stderr)
@@ -236,7 +359,18 @@ def main():
             b.copy_(a)
         torch.cuda.synchronize()
         del a, b
-    line = run_c2(args)
+    line, extra = run_c2(args)
+    torch.cuda.empty_cache()
+    if "c3" in args.extras:
+        extra["c3"] = run_c3(args)
+        torch.cuda.empty_cache()
+    if "c4" in args.extras or "c5" in args.extras:
+        _part, graph, setup_s = build_c4(args)
+        if "c4" in args.extras:
+            extra["c4"] = run_c4(args, graph, setup_s)
+        if "c5" in args.extras:
+            extra["c5"] = run_c5(args, graph)
+    line["extra"] = extra
     print(json.dumps(line), flush=True)
 
 

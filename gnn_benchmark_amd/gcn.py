@@ -1,0 +1,94 @@
+"""A GCN layer stack around the aggregation path, used for the full train-step workload.
+
+The aggregation is the reference's ``Aggregator`` contract (aggregate-then-transform, the
+order of self_benchmark/a64fx/model/layers/sageconv.py:65-93: ``out = Aggregator(...)``,
+``out /= graph.in_degrees``, then the dense transform).  Everything after the
+aggregation is this build's own definition of the workload: one weight matrix per layer
+(``Z = (A X / deg) W + b``), ReLU, dropout with a precomputed seeded mask, log-softmax +
+NLL on the labelled nodes, Adam.  The dense products run on the matrix cores through
+the BLAS library behind ``torch.mm`` (fp32, or bf16 inputs with fp32 accumulation and
+fp32 output); they are plain library GEMMs, not part of libgnnagg.
+"""
+from typing import List, Optional, Sequence
+
+import torch
+import torch.nn.functional as F
+
+from .aggregator import Aggregator
+
+
+class _Bf16InputLinear(torch.autograd.Function):
+    """y = x @ w with x, w rounded to bf16, products accumulated in fp32, fp32 result;
+    the two gradient products are computed the same way."""
+
+    @staticmethod
+    def _mm(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+        return torch.mm(a.to(torch.bfloat16), b.to(torch.bfloat16), out_dtype=torch.float32)
+
+    @staticmethod
+    def forward(ctx, x, w):
+        ctx.save_for_backward(x, w)
+        return _Bf16InputLinear._mm(x, w)
+
+    @staticmethod
+    def backward(ctx, g):
+        x, w = ctx.saved_tensors
+        gx = _Bf16InputLinear._mm(g, w.t()) if ctx.needs_input_grad[0] else None
+        gw = _Bf16InputLinear._mm(x.t(), g) if ctx.needs_input_grad[1] else None
+        return gx, gw
+
+
+class GCNLayer(torch.nn.Module):
+    def __init__(self, in_channels: int, out_channels: int, gemm: str = "fp32"):
+        super().__init__()
+        if gemm not in ("fp32", "bf16"):
+            raise ValueError("gemm must be 'fp32' or 'bf16'")
+        self.gemm = gemm
+        self.weight = torch.nn.Parameter(torch.empty(in_channels, out_channels))
+        self.bias = torch.nn.Parameter(torch.zeros(out_channels))
+        torch.nn.init.xavier_uniform_(self.weight, gain=torch.nn.init.calculate_gain("relu"))
+
+    def forward(self, graph, x: torch.Tensor, layer: int, is_pre_delay: bool) -> torch.Tensor:
+        agg = Aggregator.apply(graph, x, layer, 32, is_pre_delay, self.training)
+        agg = agg / graph.in_degrees
+        if self.gemm == "bf16":
+            return _Bf16InputLinear.apply(agg, self.weight) + self.bias
+        return torch.mm(agg, self.weight) + self.bias
+
+
+class GCN(torch.nn.Module):
+    def __init__(self, dims: Sequence[int], gemm: str = "fp32", dropout: float = 0.5):
+        super().__init__()
+        self.layers = torch.nn.ModuleList([GCNLayer(dims[i], dims[i + 1], gemm) for i in range(len(dims) - 1)])
+        self.dropout = dropout
+
+    def forward(self, graph, x: torch.Tensor, is_pre_delay: bool,
+                masks: Optional[List[torch.Tensor]] = None) -> torch.Tensor:
+        """``masks[l]``: bool keep-mask [N, dims[l+1]] of the dropout after layer l (training only)."""
+        h = x
+        last = len(self.layers) - 1
+        for l, layer in enumerate(self.layers):
+            h = layer(graph, h, l, is_pre_delay)
+            if l != last:
+                h = torch.relu(h)
+                if self.training and self.dropout > 0.0:
+                    if masks is None:
+                        raise ValueError("training needs the seeded dropout masks")
+                    h = h * masks[l] * (1.0 / (1.0 - self.dropout))
+        return F.log_softmax(h, dim=1)
+
+
+def make_dropout_masks(num_nodes: int, dims: Sequence[int], p: float, seed: int, device) -> List[torch.Tensor]:
+    gen = torch.Generator(device=device).manual_seed(seed)
+    return [torch.rand(num_nodes, dims[l + 1], device=device, generator=gen) >= p for l in range(len(dims) - 2)]
+
+
+def train_step(model: GCN, optimizer, graph, x, labels, train_idx, is_pre_delay: bool, masks) -> torch.Tensor:
+    """forward, NLL loss on the labelled nodes, backward, optimizer update."""
+    model.train()
+    optimizer.zero_grad(set_to_none=True)
+    out = model(graph, x, is_pre_delay, masks)
+    loss = F.nll_loss(out[train_idx], labels[train_idx])
+    loss.backward()
+    optimizer.step()
+    return loss.detach()

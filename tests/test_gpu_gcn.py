@@ -1,0 +1,117 @@
+"""The full train step (3-layer GCN around the aggregation path) on the GPU against an
+independent CPU autograd run: same weights, same seeded dropout masks, same received halo
+rows, aggregation done with torch.sparse.mm on the CPU.  The layer definition after the
+aggregation is this build's own (no reference file holds it), so this is a consistency
+check of forward, backward and the Adam update -- tolerance 1e-4 relative on the loss and
+gradients (fp32 sums in a different order; bf16 variant: 2e-2)."""
+import copy
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from gnn_benchmark_amd import gcn, synthetic
+
+pytestmark = pytest.mark.gpu
+
+
+class ReplayExchange:
+    """Delivers the same seeded rows as SeededHaloExchange and keeps a host copy per tag."""
+
+    def __init__(self, seed):
+        self.inner = synthetic.SeededHaloExchange(seed)
+        self.rows = {}
+
+    def __call__(self, comm_splits, comm_buf, tag, direction):
+        self.inner(comm_splits, comm_buf, tag, direction)
+        buf = comm_buf.recv_buf if direction == "forward" else comm_buf.send_buf
+        self.rows[tag] = buf.detach().cpu().clone()
+        return None
+
+
+def _torch_sparse(m):
+    rowptr, col, val = [t.cpu() for t in m.csr()]
+    return torch.sparse_csr_tensor(rowptr, col, val, size=m.sparse_sizes())
+
+
+class CpuAggregate(torch.autograd.Function):
+    """out = A_local x + A_from recv ; grad = A_local^T g + A_to^T incoming (CPU, torch.sparse)."""
+
+    @staticmethod
+    def forward(ctx, x, a_local, a_from, a_to, recv, incoming):
+        ctx.mats = (a_local, a_to, incoming)
+        return torch.sparse.mm(a_local, x) + torch.sparse.mm(a_from, recv)
+
+    @staticmethod
+    def backward(ctx, g):
+        a_local, a_to, incoming = ctx.mats
+        gx = torch.sparse.mm(a_local.t().to_sparse_csr(), g) + torch.sparse.mm(a_to.t().to_sparse_csr(), incoming)
+        return gx, None, None, None, None, None
+
+
+def _bf16_mm(a, b):
+    return a.to(torch.bfloat16).float() @ b.to(torch.bfloat16).float()
+
+
+class CpuBf16Linear(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, w):
+        ctx.save_for_backward(x, w)
+        return _bf16_mm(x, w)
+
+    @staticmethod
+    def backward(ctx, g):
+        x, w = ctx.saved_tensors
+        return _bf16_mm(g, w.t()), _bf16_mm(x.t(), g)
+
+
+@pytest.mark.parametrize("gemm,tol", [("fp32", 1e-4), ("bf16", 2e-2)])
+def test_train_step_matches_cpu_autograd(gemm, tol):
+    dev = "cuda:0"
+    n, dims = 6000, [32, 64, 64, 12]
+    part = synthetic.partition_edges(n, 4, 2, 6, 1.8, 800, 1500, 9000, seed=3, device=dev)
+    ex = ReplayExchange(5)
+    graph = synthetic.build_partition_graph(part, max(dims), True, exchange=ex, device=dev)
+    torch.manual_seed(0)
+    model = gcn.GCN(dims, gemm=gemm).to(dev)
+    cpu_model = copy.deepcopy(model).cpu()
+    opt = torch.optim.Adam(model.parameters(), lr=0.01)
+    gen = torch.Generator(device=dev).manual_seed(1)
+    x = torch.randn(n, dims[0], device=dev, generator=gen)
+    labels = torch.randint(0, dims[-1], (n,), device=dev, generator=gen)
+    train_idx = torch.randperm(n, device=dev, generator=gen)[: n // 10]
+    masks = gcn.make_dropout_masks(n, dims, 0.5, 7, dev)
+
+    # forward + backward on the GPU (no update yet)
+    model.train()
+    out = model(graph, x, True, masks)
+    loss = F.nll_loss(out[train_idx], labels[train_idx])
+    loss.backward()
+
+    # independent CPU run with the rows the exchange delivered
+    a_local, a_from, a_to = (_torch_sparse(m) for m in (graph.local_adj_t, graph.adj_t_pre_post_aggr_from,
+                                                         graph.adj_t_pre_post_aggr_to))
+    deg = graph.in_degrees.cpu()
+    h = x.cpu()
+    for l, layer in enumerate(cpu_model.layers):
+        # layer 0's input needs no gradient, so its backward exchange never happens
+        incoming = ex.rows.get(f"backward{l}", torch.zeros(a_to.shape[0], dims[l]))
+        agg = CpuAggregate.apply(h, a_local, a_from, a_to, ex.rows[f"forward{l}"], incoming) / deg
+        z = (CpuBf16Linear.apply(agg, layer.weight) if gemm == "bf16" else agg @ layer.weight) + layer.bias
+        h = z if l == len(dims) - 2 else torch.relu(z) * masks[l].cpu() * 2.0
+    cpu_loss = F.nll_loss(F.log_softmax(h, dim=1)[train_idx.cpu()], labels.cpu()[train_idx.cpu()])
+    cpu_loss.backward()
+
+    assert abs(float(loss) - float(cpu_loss)) <= tol * max(1.0, abs(float(cpu_loss)))
+    for (name, p_gpu), p_cpu in zip(model.named_parameters(), cpu_model.parameters()):
+        scale = float(p_cpu.grad.abs().max()) + 1e-12
+        assert float((p_gpu.grad.cpu() - p_cpu.grad).abs().max()) <= 10 * tol * scale, name
+
+    # the full step: loss goes down over a few updates, every Adam update is bounded by lr
+    before = [p.detach().clone() for p in model.parameters()]
+    losses = [float(gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks)) for _ in range(5)]
+    assert all(np.isfinite(losses)) and losses[-1] < losses[0]
+    assert abs(losses[0] - float(cpu_loss)) <= tol * max(1.0, abs(float(cpu_loss)))
+    for b, p in zip(before, model.parameters()):
+        assert float((p.detach() - b).abs().max()) <= 5 * 0.01 * 1.01
