@@ -49,6 +49,8 @@ template <int VEC, int LPR, int NCH, typename IdxT, int MODE>
 hipError_t launch_tasks(const SpmmArgs &a, int rows_per_group, hipStream_t stream) {
     constexpr int GPB = 256 / LPR;
     SpmmArgs args = a;
+    if (rows_per_group > kMaxRowsPerGroup) rows_per_group = kMaxRowsPerGroup;
+    if (rows_per_group < 1) rows_per_group = 1;
     args.tasks_per_block = GPB * rows_per_group;
     if (args.head_tasks > args.ntasks) args.head_tasks = args.ntasks;
     const int64_t head_blocks = (args.head_tasks + GPB - 1) / GPB;
@@ -148,6 +150,21 @@ __global__ __launch_bounds__(256) void narrow_cols_kernel(const int64_t *__restr
     if (bad) atomicOr(&out->bad_col, 1u);
 }
 
+// task[t] = (first element, length, row) of the t-th row of the degree-ordered schedule
+__global__ __launch_bounds__(256) void build_tasks_kernel(const int64_t *__restrict__ rowptr,
+                                                          const int32_t *__restrict__ perm, int rows,
+                                                          RowTask *__restrict__ task) {
+    const int t = (int)blockIdx.x * 256 + (int)threadIdx.x;
+    if (t >= rows) return;
+    const int r = perm[t];
+    const int64_t b = rowptr[r];
+    RowTask d;
+    d.start = b;
+    d.len = (int32_t)(rowptr[r + 1] - b);
+    d.row = r;
+    task[t] = d;
+}
+
 int env_int(const char *name, int dflt, int lo, int hi) {
     const char *v = getenv(name);
     if (!v || !*v) return dflt;
@@ -168,9 +185,8 @@ struct gnnagg_plan {
     int64_t nempty = 0;       // rows with no stored element (the last nempty entries of perm)
     int64_t max_deg = 0;
     int device = 0;
-    int64_t *rowptr = nullptr;  // [rows+1] own copy
     int32_t *col32 = nullptr;   // [nnz]
-    int32_t *perm = nullptr;    // [rows] rows by degree class, longest first; ascending row id inside a class
+    RowTask *task = nullptr;    // [rows] rows by degree class, longest first; ascending row id inside a class
     int rows_per_group = 4;
     bool profile = false;
     bool profile_valid = false;
@@ -220,9 +236,8 @@ extern "C" int gnnagg_spmm_csr_f32(const int64_t *rowptr, const int64_t *col, co
 
 static void plan_free(gnnagg_plan *p) {
     if (!p) return;
-    (void)hipFree(p->rowptr);
     (void)hipFree(p->col32);
-    (void)hipFree(p->perm);
+    (void)hipFree(p->task);
     for (hipEvent_t e : p->ev)
         if (e) (void)hipEventDestroy(e);
     delete p;
@@ -251,7 +266,7 @@ extern "C" int gnnagg_plan_create(const int64_t *rowptr, const int64_t *col, int
     p->cols = cols;
     p->nnz = nnz;
     p->long_thresh = env_int("GNNAGG_LONG_THRESH", 256, 1, 1 << 30);
-    p->rows_per_group = env_int("GNNAGG_ROWS_PER_GROUP", 4, 1, 1024);
+    p->rows_per_group = env_int("GNNAGG_ROWS_PER_GROUP", 4, 1, kMaxRowsPerGroup);
     GNNAGG_HIP(hipGetDevice(&p->device));
 
     // rowptr end points (host check; also forces the inputs to be ready)
@@ -262,10 +277,8 @@ extern "C" int gnnagg_plan_create(const int64_t *rowptr, const int64_t *col, int
     GNNAGG_REQUIRE(ends[0] == 0 && ends[1] == nnz, "rowptr[0]=%lld, rowptr[rows]=%lld do not match nnz=%lld",
                    (long long)ends[0], (long long)ends[1], (long long)nnz);
 
-    GNNAGG_HIP(hipMalloc((void **)&p->rowptr, sizeof(int64_t) * (size_t)(rows + 1)));
-    GNNAGG_HIP(hipMemcpyAsync(p->rowptr, rowptr, sizeof(int64_t) * (size_t)(rows + 1), hipMemcpyDeviceToDevice, st));
     GNNAGG_HIP(hipMalloc((void **)&p->col32, sizeof(int32_t) * (size_t)std::max<int64_t>(nnz, 1)));
-    GNNAGG_HIP(hipMalloc((void **)&p->perm, sizeof(int32_t) * (size_t)std::max<int64_t>(rows, 1)));
+    GNNAGG_HIP(hipMalloc((void **)&p->task, sizeof(RowTask) * (size_t)std::max<int64_t>(rows, 1)));
 
     DevBuf<ClassifyOut> d_out;
     GNNAGG_HIP(d_out.alloc(1));
@@ -274,11 +287,12 @@ extern "C" int gnnagg_plan_create(const int64_t *rowptr, const int64_t *col, int
     ClassifyOut h_out{};
     if (rows > 0) {
         DevBuf<uint32_t> key_in, key_out;
-        DevBuf<int32_t> row_in;
+        DevBuf<int32_t> row_in, perm;
         GNNAGG_HIP(key_in.alloc((size_t)rows));
         GNNAGG_HIP(key_out.alloc((size_t)rows));
         GNNAGG_HIP(row_in.alloc((size_t)rows));
-        hipLaunchKernelGGL(classify_rows_kernel, dim3(grid_for(rows, 256)), dim3(256), 0, st, p->rowptr, (int)rows,
+        GNNAGG_HIP(perm.alloc((size_t)rows));
+        hipLaunchKernelGGL(classify_rows_kernel, dim3(grid_for(rows, 256)), dim3(256), 0, st, rowptr, (int)rows,
                            key_in.p, row_in.p, d_out.p);
         GNNAGG_HIP(hipGetLastError());
         if (nnz > 0) {
@@ -288,19 +302,28 @@ extern "C" int gnnagg_plan_create(const int64_t *rowptr, const int64_t *col, int
         }
         // stable sort of the rows by class: ascending row id inside a class
         size_t tmp_bytes = 0;
-        GNNAGG_HIP(hipcub::DeviceRadixSort::SortPairs(nullptr, tmp_bytes, key_in.p, key_out.p, row_in.p, p->perm,
+        GNNAGG_HIP(hipcub::DeviceRadixSort::SortPairs(nullptr, tmp_bytes, key_in.p, key_out.p, row_in.p, perm.p,
                                                       (int)rows, 0, kClassBits, st));
         DevBuf<char> tmp;
         GNNAGG_HIP(tmp.alloc(std::max<size_t>(tmp_bytes, 1)));
-        GNNAGG_HIP(hipcub::DeviceRadixSort::SortPairs(tmp.p, tmp_bytes, key_in.p, key_out.p, row_in.p, p->perm,
+        GNNAGG_HIP(hipcub::DeviceRadixSort::SortPairs(tmp.p, tmp_bytes, key_in.p, key_out.p, row_in.p, perm.p,
                                                       (int)rows, 0, kClassBits, st));
         GNNAGG_HIP(hipMemcpyAsync(&h_out, d_out.p, sizeof(ClassifyOut), hipMemcpyDeviceToHost, st));
+        GNNAGG_HIP(hipStreamSynchronize(st));
+        if (!h_out.bad_rowptr && h_out.max_deg < (1ull << 31)) {  // row lengths are only meaningful for a monotone rowptr
+            hipLaunchKernelGGL(build_tasks_kernel, dim3(grid_for(rows, 256)), dim3(256), 0, st, rowptr, perm.p,
+                               (int)rows, p->task);
+            GNNAGG_HIP(hipGetLastError());
+            GNNAGG_HIP(hipStreamSynchronize(st));  // perm is released on scope exit
+        }
         GNNAGG_HIP(hipStreamSynchronize(st));
     }
     GNNAGG_REQUIRE(!h_out.bad_rowptr, "rowptr is not non-decreasing");
     GNNAGG_REQUIRE(!h_out.bad_col, "a column index lies outside [0, %lld)", (long long)cols);
     p->nempty = (int64_t)h_out.class_count[kEmptyClass];
     p->max_deg = (int64_t)h_out.max_deg;
+    if (p->max_deg >= (int64_t(1) << 31))
+        return fail(GNNAGG_ERR_UNSUPPORTED, "a row holds %lld stored elements (limit 2^31-1)", (long long)p->max_deg);
     // rows strictly longer than long_thresh: whole classes above the threshold's class
     const int thresh_class = degree_class(p->long_thresh);
     for (int c = 0; c < thresh_class; ++c) p->nlong += (int64_t)h_out.class_count[c];
@@ -351,7 +374,7 @@ extern "C" int gnnagg_plan_spmm_f32(gnnagg_plan *plan, const float *value, const
     for (int64_t f_base = 0; f_base < feat;) {
         const Shape s = pick_shape(vec, feat - f_base);
         SpmmArgs a{};
-        a.rowptr = plan->rowptr;
+        a.task = plan->task;
         a.col = plan->col32;
         a.val = value;
         a.x = mat;
@@ -363,11 +386,10 @@ extern "C" int gnnagg_plan_spmm_f32(gnnagg_plan *plan, const float *value, const
         // form the head region (one lane group per row)
         if (plan->nlong + nshort > 0) {
             const bool timed = prof && f_base == 0;
-            a.perm = plan->perm;
             a.ntasks = plan->nlong + nshort;
             a.head_tasks = plan->nlong;
             if (timed) GNNAGG_HIP(hipEventRecord(plan->ev[1], st));
-            GNNAGG_HIP((dispatch_tasks<int32_t, kRowsPermuted>(s, a, plan->rows_per_group, st)));
+            GNNAGG_HIP((dispatch_tasks<int32_t, kRowsPlanned>(s, a, plan->rows_per_group, st)));
             if (timed) {
                 GNNAGG_HIP(hipEventRecord(plan->ev[2], st));
                 plan->profile_valid = true;

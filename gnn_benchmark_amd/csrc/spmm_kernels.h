@@ -138,13 +138,20 @@ __device__ __forceinline__ void gather_fma(FVec<VEC> (&acc)[NCH], IdxT c_l, floa
 }
 
 enum TaskMode : int {
-    kRowsNatural = 0,  // task t is row t
-    kRowsPermuted = 1  // task t is row perm[t]
+    kRowsNatural = 0,  // task t is row t, described by rowptr        (plan-less entry point)
+    kRowsPlanned = 1   // task t is described by task[t] of a plan    (degree-ordered)
+};
+
+// One row of a plan's schedule: 16 bytes, fetched with a single load.
+struct __attribute__((aligned(16))) RowTask {
+    int64_t start;  // first stored element
+    int32_t len;    // stored elements
+    int32_t row;    // output row
 };
 
 struct SpmmArgs {
-    const int64_t *rowptr;    // [rows+1]
-    const int32_t *perm;      // [ntasks] row of task t        (kRowsPermuted)
+    const int64_t *rowptr;    // [rows+1]                       (kRowsNatural)
+    const RowTask *task;      // [ntasks]                       (kRowsPlanned)
     const void *col;          // IdxT [nnz]
     const float *val;         // [nnz]
     const float *x;           // dense operand [K, F]
@@ -167,6 +174,8 @@ struct UnrollFor {
     static constexpr int raw = 32 / regs;
     static constexpr int value = raw >= 8 ? 8 : (raw >= 4 ? 4 : (raw >= 2 ? 2 : 1));
 };
+
+constexpr int kMaxRowsPerGroup = 16;  // a group's task descriptors live one per lane
 
 template <int VEC, int LPR, int NCH, typename IdxT, int MODE>
 __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
@@ -209,54 +218,111 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
         t1 = t0 + a.tasks_per_block;
         if (t1 > a.ntasks) t1 = a.ntasks;
     }
+    // this group's tasks: t0 + group + i * GPB, i < ntask  (ntask <= kMaxRowsPerGroup <= LPR)
+    const int64_t tfirst = t0 + group;
+    if (tfirst >= t1) return;
+    int ntask = (int)((t1 - tfirst + GPB - 1) / GPB);
+    if constexpr (LPR == 64) ntask = __builtin_amdgcn_readfirstlane(ntask);
 
-    for (int64_t t = t0 + group; t < t1; t += GPB) {
-        int64_t row = t;
-        if constexpr (MODE == kRowsPermuted) row = a.perm[t];
-        int64_t start = a.rowptr[row];
-        int64_t end = a.rowptr[row + 1];
-        float *dst = a.dst + (size_t)row * (size_t)F;
-        const bool from_dst = a.accumulate != 0;
-        if constexpr (LPR == 64) {
-            start = uniform_i64(start);
-            end = uniform_i64(end);
+    // One coalesced fetch brings every descriptor of the group: lane i holds task i.
+    int d_row = 0, d_len = 0;
+    int64_t d_start = 0;
+    if (lig < ntask) {
+        const int64_t t = tfirst + (int64_t)lig * GPB;
+        if constexpr (MODE == kRowsPlanned) {
+            const RowTask d = a.task[t];
+            d_row = d.row;
+            d_len = d.len;
+            d_start = d.start;
+        } else {
+            d_row = (int)t;
+            d_start = a.rowptr[t];
+            d_len = (int)(a.rowptr[t + 1] - d_start);
         }
+    }
 
-        V acc[NCH];
+    // State of the row being accumulated and of the chunk of <= LPR (col, val) pairs held
+    // across the group's lanes.  The NEXT chunk -- of the same row, or the first chunk of
+    // the group's next row -- is always requested before the current chunk's gathers, so
+    // that the index stream never sits on the critical path.
+    int i = 0;
+    int row = group_bcast<LPR>(d_row, 0);
+    int64_t base = group_bcast_idx<LPR>(d_start, 0);
+    int64_t end = base + group_bcast<LPR>(d_len, 0);
+    IdxT c_l = 0;
+    float v_l = 0.0f;
+    if (base + lig < end) {
+        c_l = __builtin_nontemporal_load(col + base + lig);
+        v_l = __builtin_nontemporal_load(val + base + lig);
+    }
+    const bool from_dst = a.accumulate != 0;
+    float *dst = a.dst + (size_t)row * (size_t)F;
+    V acc[NCH];
 #pragma unroll
-        for (int k = 0; k < NCH; ++k) {
-            acc[k] = V::zero();
-            if (from_dst && fok[k]) acc[k] = V::load(dst + foff[k]);
-        }
+    for (int k = 0; k < NCH; ++k) {
+        acc[k] = V::zero();
+        if (from_dst && fok[k]) acc[k] = V::load(dst + foff[k]);
+    }
 
-        for (int64_t base = start; base < end; base += LPR) {
-            const int64_t left = end - base;
-            const int cnt = left < LPR ? (int)left : LPR;
-            IdxT c_l = 0;
-            float v_l = 0.0f;
-            if (lig < cnt) {
-                c_l = __builtin_nontemporal_load(col + base + lig);
-                v_l = __builtin_nontemporal_load(val + base + lig);
-            }
-            // full blocks of U gathers, then a halving cascade for what is left, so that a
-            // chunk of cnt elements costs at most cnt/U + log2(U) dependent round trips
-            int j = 0;
-            for (; j + U <= cnt; j += U) gather_fma<U, VEC, LPR, NCH>(acc, c_l, v_l, j, x, F, foff);
-            if constexpr (U > 4) {
-                if (j + 4 <= cnt) { gather_fma<4, VEC, LPR, NCH>(acc, c_l, v_l, j, x, F, foff); j += 4; }
-            }
-            if constexpr (U > 2) {
-                if (j + 2 <= cnt) { gather_fma<2, VEC, LPR, NCH>(acc, c_l, v_l, j, x, F, foff); j += 2; }
-            }
-            if constexpr (U > 1) {
-                if (j + 1 <= cnt) { gather_fma<1, VEC, LPR, NCH>(acc, c_l, v_l, j, x, F, foff); j += 1; }
+    while (true) {
+        const int64_t left = end - base;
+        const int cnt = left < LPR ? (int)left : LPR;
+
+        // where the next chunk comes from
+        int ni = i;
+        int nrow = row;
+        int64_t nbase = base + LPR, nend = end;
+        bool row_done = nbase >= end;
+        bool more = true;
+        if (row_done) {
+            ni = i + 1;
+            more = ni < ntask;
+            if (more) {
+                nrow = group_bcast<LPR>(d_row, ni);
+                nbase = group_bcast_idx<LPR>(d_start, ni);
+                nend = nbase + group_bcast<LPR>(d_len, ni);
             }
         }
+        IdxT nc = 0;
+        float nv = 0.0f;
+        if (more && nbase + lig < nend) {
+            nc = __builtin_nontemporal_load(col + nbase + lig);
+            nv = __builtin_nontemporal_load(val + nbase + lig);
+        }
 
+        // full blocks of U gathers, then a halving cascade for what is left, so that a
+        // chunk of cnt elements costs at most cnt/U + log2(U) dependent round trips
+        int j = 0;
+        for (; j + U <= cnt; j += U) gather_fma<U, VEC, LPR, NCH>(acc, c_l, v_l, j, x, F, foff);
+        if constexpr (U > 4) {
+            if (j + 4 <= cnt) { gather_fma<4, VEC, LPR, NCH>(acc, c_l, v_l, j, x, F, foff); j += 4; }
+        }
+        if constexpr (U > 2) {
+            if (j + 2 <= cnt) { gather_fma<2, VEC, LPR, NCH>(acc, c_l, v_l, j, x, F, foff); j += 2; }
+        }
+        if constexpr (U > 1) {
+            if (j + 1 <= cnt) { gather_fma<1, VEC, LPR, NCH>(acc, c_l, v_l, j, x, F, foff); j += 1; }
+        }
+
+        if (row_done) {
 #pragma unroll
-        for (int k = 0; k < NCH; ++k) {
-            if (fok[k]) acc[k].store(dst + foff[k]);
+            for (int k = 0; k < NCH; ++k) {
+                if (fok[k]) acc[k].store(dst + foff[k]);
+            }
+            if (!more) break;
+            dst = a.dst + (size_t)nrow * (size_t)F;
+#pragma unroll
+            for (int k = 0; k < NCH; ++k) {
+                acc[k] = V::zero();
+                if (from_dst && fok[k]) acc[k] = V::load(dst + foff[k]);
+            }
         }
+        i = ni;
+        row = nrow;
+        base = nbase;
+        end = nend;
+        c_l = nc;
+        v_l = nv;
     }
 }
 
