@@ -37,6 +37,8 @@ struct FVec<1> {
     __device__ __forceinline__ static FVec zero() { return FVec{0.0f}; }
     __device__ __forceinline__ static FVec load(const float *p) { return FVec{*p}; }
     __device__ __forceinline__ void store(float *p) const { *p = d; }
+    __device__ __forceinline__ static FVec load_stream(const float *p) { return FVec{__builtin_nontemporal_load(p)}; }
+    __device__ __forceinline__ void store_stream(float *p) const { __builtin_nontemporal_store(d, p); }
     __device__ __forceinline__ void fma(float a, const FVec &x) { d = __builtin_fmaf(a, x.d, d); }
     __device__ __forceinline__ void add(const FVec &x) { d += x.d; }
 };
@@ -49,6 +51,12 @@ struct FVec<2> {
         return FVec{*reinterpret_cast<const f32x2 *>(p)};
     }
     __device__ __forceinline__ void store(float *p) const { *reinterpret_cast<f32x2 *>(p) = d; }
+    __device__ __forceinline__ static FVec load_stream(const float *p) {
+        return FVec{__builtin_nontemporal_load(reinterpret_cast<const f32x2 *>(p))};
+    }
+    __device__ __forceinline__ void store_stream(float *p) const {
+        __builtin_nontemporal_store(d, reinterpret_cast<f32x2 *>(p));
+    }
     __device__ __forceinline__ void fma(float a, const FVec &x) {
         d.x = __builtin_fmaf(a, x.d.x, d.x);
         d.y = __builtin_fmaf(a, x.d.y, d.y);
@@ -67,6 +75,12 @@ struct FVec<4> {
         return FVec{*reinterpret_cast<const f32x4 *>(p)};
     }
     __device__ __forceinline__ void store(float *p) const { *reinterpret_cast<f32x4 *>(p) = d; }
+    __device__ __forceinline__ static FVec load_stream(const float *p) {
+        return FVec{__builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p))};
+    }
+    __device__ __forceinline__ void store_stream(float *p) const {
+        __builtin_nontemporal_store(d, reinterpret_cast<f32x4 *>(p));
+    }
     __device__ __forceinline__ void fma(float a, const FVec &x) {
         d.x = __builtin_fmaf(a, x.d.x, d.x);
         d.y = __builtin_fmaf(a, x.d.y, d.y);
@@ -261,7 +275,7 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
 #pragma unroll
     for (int k = 0; k < NCH; ++k) {
         acc[k] = V::zero();
-        if (from_dst && fok[k]) acc[k] = V::load(dst + foff[k]);
+        if (from_dst && fok[k]) acc[k] = V::load_stream(dst + foff[k]);
     }
 
     while (true) {
@@ -307,14 +321,14 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
         if (row_done) {
 #pragma unroll
             for (int k = 0; k < NCH; ++k) {
-                if (fok[k]) acc[k].store(dst + foff[k]);
+                if (fok[k]) acc[k].store_stream(dst + foff[k]);
             }
             if (!more) break;
             dst = a.dst + (size_t)nrow * (size_t)F;
 #pragma unroll
             for (int k = 0; k < NCH; ++k) {
                 acc[k] = V::zero();
-                if (from_dst && fok[k]) acc[k] = V::load(dst + foff[k]);
+                if (from_dst && fok[k]) acc[k] = V::load_stream(dst + foff[k]);
             }
         }
         i = ni;
