@@ -194,7 +194,7 @@ def run_c2(args):
                                f"{g.num_nodes} nodes / {g.nnz} nnz (Zipf s=1.8, longest row {g.max_degree}), "
                                f"GCN-normalised fp32, dense operand {g.num_nodes}x{args.feat} fp32",
                    "nodes": g.num_nodes, "nnz": g.nnz, "feat": args.feat, "seed": args.seed,
-                   "long_rows": info["long_rows"], "max_row_len": info["max_row_len"], "setup_s": round(setup_s, 2)},
+                   "huge_rows": info["huge_rows"], "max_row_len": info["max_row_len"], "setup_s": round(setup_s, 2)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                      "kernel": "gnnagg::spmm_tasks_kernel<4,32,1,int,1> (forward A@X, one launch over all rows)",

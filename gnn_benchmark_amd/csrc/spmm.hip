@@ -81,6 +81,27 @@ hipError_t dispatch_shape(const Shape &s, const SpmmArgs &a, int rpg, hipStream_
     return hipErrorInvalidValue;
 }
 
+template <int VEC>
+hipError_t launch_long_rows(const LongArgs &a, int64_t nrows, hipStream_t st) {
+    static bool configured = false;  // the attribute is per kernel, set once per process
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(spmm_long_rows_kernel<VEC>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLongSmemBytes);
+        if (e != hipSuccess) return e;
+        configured = true;
+    }
+    LongArgs args = a;
+    const int tile = a.feat < kLongFeatTile ? a.feat : kLongFeatTile;
+    const int vpr = tile / VEC;
+    int chunk = kLongMaxChunk;
+    if (chunk * vpr > 256 * kLongLoads) chunk = 256 * kLongLoads / vpr;
+    if (chunk * tile > kLongTileFloats) chunk = kLongTileFloats / tile;
+    args.chunk = chunk;
+    const unsigned tiles = (unsigned)((a.feat + kLongFeatTile - 1) / kLongFeatTile);
+    hipLaunchKernelGGL((spmm_long_rows_kernel<VEC>), dim3((unsigned)nrows, tiles), dim3(256), kLongSmemBytes, st, args);
+    return hipGetLastError();
+}
+
 template <typename IdxT, int MODE>
 hipError_t dispatch_tasks(const Shape &s, const SpmmArgs &a, int rpg, hipStream_t st) {
     if (s.vec == 4) return dispatch_shape<4, IdxT, MODE>(s, a, rpg, st);
@@ -180,14 +201,18 @@ using namespace gnnagg;
 
 struct gnnagg_plan {
     int64_t rows = 0, cols = 0, nnz = 0;
+    int huge_thresh = 0;      // rows longer than this run in the block-per-row kernel
+    int64_t nhuge = 0;        // such rows (the first nhuge tasks)
     int long_thresh = 0;      // rows longer than this get a lane group of their own (head region)
-    int64_t nlong = 0;        // such rows (the first nlong entries of perm)
+    int64_t nlong = 0;        // such rows, the huge ones included (the first nlong tasks)
     int64_t nempty = 0;       // rows with no stored element (the last nempty entries of perm)
     int64_t max_deg = 0;
     int device = 0;
     int32_t *col32 = nullptr;   // [nnz]
     RowTask *task = nullptr;    // [rows] rows by degree class, longest first; ascending row id inside a class
     int rows_per_group = 4;
+    hipStream_t side = nullptr;          // the block-per-row kernel runs here, next to the main launch
+    hipEvent_t fork = nullptr, join = nullptr;
     bool profile = false;
     bool profile_valid = false;
     hipEvent_t ev[4] = {nullptr, nullptr, nullptr, nullptr};  // call begin, main-kernel begin/end, call end
@@ -238,6 +263,9 @@ static void plan_free(gnnagg_plan *p) {
     if (!p) return;
     (void)hipFree(p->col32);
     (void)hipFree(p->task);
+    if (p->fork) (void)hipEventDestroy(p->fork);
+    if (p->join) (void)hipEventDestroy(p->join);
+    if (p->side) (void)hipStreamDestroy(p->side);
     for (hipEvent_t e : p->ev)
         if (e) (void)hipEventDestroy(e);
     delete p;
@@ -266,6 +294,12 @@ extern "C" int gnnagg_plan_create(const int64_t *rowptr, const int64_t *col, int
     p->cols = cols;
     p->nnz = nnz;
     p->long_thresh = env_int("GNNAGG_LONG_THRESH", 256, 1, 1 << 30);
+    // A row is handed to the block-per-row kernel only when its chain, fed by one lane
+    // group (a few elements per microsecond), would outlast the whole launch: that
+    // length grows with the matrix, about nnz / 4096 (measured on MI355X), floor 8192.
+    int64_t huge_default = std::max<int64_t>(8192, nnz / 4096);
+    if (huge_default > (1 << 30)) huge_default = 1 << 30;
+    p->huge_thresh = env_int("GNNAGG_HUGE_THRESH", (int)huge_default, p->long_thresh, 1 << 30);
     p->rows_per_group = env_int("GNNAGG_ROWS_PER_GROUP", 4, 1, kMaxRowsPerGroup);
     GNNAGG_HIP(hipGetDevice(&p->device));
 
@@ -327,6 +361,13 @@ extern "C" int gnnagg_plan_create(const int64_t *rowptr, const int64_t *col, int
     // rows strictly longer than long_thresh: whole classes above the threshold's class
     const int thresh_class = degree_class(p->long_thresh);
     for (int c = 0; c < thresh_class; ++c) p->nlong += (int64_t)h_out.class_count[c];
+    const int huge_class = degree_class(p->huge_thresh);
+    for (int c = 0; c < huge_class; ++c) p->nhuge += (int64_t)h_out.class_count[c];
+    if (p->nhuge > 0) {
+        GNNAGG_HIP(hipStreamCreateWithFlags(&p->side, hipStreamNonBlocking));
+        GNNAGG_HIP(hipEventCreateWithFlags(&p->fork, hipEventDisableTiming));
+        GNNAGG_HIP(hipEventCreateWithFlags(&p->join, hipEventDisableTiming));
+    }
 
     guard.p = nullptr;
     *plan_out = p;
@@ -345,8 +386,8 @@ extern "C" int gnnagg_plan_info(const gnnagg_plan *plan, int64_t *info) {
     info[0] = plan->rows;
     info[1] = plan->cols;
     info[2] = plan->nnz;
-    info[3] = plan->nlong;
-    info[4] = plan->long_thresh;
+    info[3] = plan->nhuge;
+    info[4] = plan->huge_thresh;
     info[5] = plan->nempty;
     info[6] = plan->max_deg;
     info[7] = plan->rows_per_group;
@@ -371,6 +412,24 @@ extern "C" int gnnagg_plan_spmm_f32(gnnagg_plan *plan, const float *value, const
         plan->profile_valid = false;
         GNNAGG_HIP(hipEventRecord(plan->ev[0], st));
     }
+    if (plan->nhuge > 0) {
+        // all feature tiles of the very long rows, one block each, on the plan's side
+        // stream so that they run next to the main launch instead of in front of it
+        GNNAGG_HIP(hipEventRecord(plan->fork, st));
+        GNNAGG_HIP(hipStreamWaitEvent(plan->side, plan->fork, 0));
+        LongArgs la{};
+        la.task = plan->task;
+        la.col = plan->col32;
+        la.val = value;
+        la.x = mat;
+        la.dst = out;
+        la.feat = (int)feat;
+        la.accumulate = accumulate;
+        if (vec == 4) GNNAGG_HIP(launch_long_rows<4>(la, plan->nhuge, plan->side));
+        else if (vec == 2) GNNAGG_HIP(launch_long_rows<2>(la, plan->nhuge, plan->side));
+        else GNNAGG_HIP(launch_long_rows<1>(la, plan->nhuge, plan->side));
+        GNNAGG_HIP(hipEventRecord(plan->join, plan->side));
+    }
     for (int64_t f_base = 0; f_base < feat;) {
         const Shape s = pick_shape(vec, feat - f_base);
         SpmmArgs a{};
@@ -382,12 +441,14 @@ extern "C" int gnnagg_plan_spmm_f32(gnnagg_plan *plan, const float *value, const
         a.feat = (int)feat;
         a.f_base = (int)f_base;
         a.accumulate = accumulate;
-        // one launch over every row, longest first; the rows above the long-row threshold
-        // form the head region (one lane group per row)
-        if (plan->nlong + nshort > 0) {
+        // one launch over the rows, longest first; the rows above the long-row threshold
+        // form the head region (one lane group per row).  The very longest rows went to
+        // the block-per-row kernel above.
+        if (plan->nlong + nshort - plan->nhuge > 0) {
             const bool timed = prof && f_base == 0;
-            a.ntasks = plan->nlong + nshort;
-            a.head_tasks = plan->nlong;
+            a.task = plan->task + plan->nhuge;
+            a.ntasks = plan->nlong + nshort - plan->nhuge;
+            a.head_tasks = plan->nlong - plan->nhuge;
             if (timed) GNNAGG_HIP(hipEventRecord(plan->ev[1], st));
             GNNAGG_HIP((dispatch_tasks<int32_t, kRowsPlanned>(s, a, plan->rows_per_group, st)));
             if (timed) {
@@ -397,6 +458,7 @@ extern "C" int gnnagg_plan_spmm_f32(gnnagg_plan *plan, const float *value, const
         }
         f_base += s.width();
     }
+    if (plan->nhuge > 0) GNNAGG_HIP(hipStreamWaitEvent(st, plan->join, 0));
     if (prof) GNNAGG_HIP(hipEventRecord(plan->ev[3], st));
     return GNNAGG_OK;
 }

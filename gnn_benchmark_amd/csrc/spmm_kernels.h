@@ -340,4 +340,125 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
     }
 }
 
+
+// ---------------------------------------------------------------------------------------
+// Very long rows.  One 256-thread block per (row, feature tile of <= 256 floats).  The
+// row's chain must stay sequential (bit-identical results), so what is parallelised is the
+// FETCH: all four waves gather a chunk of up to 64 dense rows into LDS at once (up to
+// 8 vector loads in flight per thread, 32 KB per block), while the threads that own a
+// feature each run the FMA chain over the previous chunk out of LDS, in CSR order.
+// Chunks are double-buffered; the (col, val) pairs run two chunks ahead.
+// ---------------------------------------------------------------------------------------
+constexpr int kLongTileFloats = 8192;  // floats per LDS tile buffer (32 KB), two buffers
+constexpr int kLongMaxChunk = 64;      // dense rows gathered per chunk
+constexpr int kLongLoads = 8;          // vector loads in flight per thread
+constexpr int kLongFeatTile = 256;     // features per block
+// dynamic LDS: two tile buffers, then three (col, val) chunk buffers
+constexpr size_t kLongSmemBytes =
+    2 * kLongTileFloats * sizeof(float) + 3 * kLongMaxChunk * (sizeof(int) + sizeof(float));
+
+struct LongArgs {
+    const RowTask *task;  // rows handled: task[0 .. gridDim.x)
+    const int32_t *col;
+    const float *val;
+    const float *x;
+    float *dst;
+    int feat;        // F
+    int chunk;       // dense rows per chunk: chunk * min(F, 256) <= kLongTileFloats, chunk * (tile / VEC) <= 2048
+    int accumulate;
+};
+
+template <int VEC>
+__global__ __launch_bounds__(256) void spmm_long_rows_kernel(const LongArgs a) {
+    typedef FVec<VEC> V;
+    extern __shared__ __attribute__((aligned(16))) unsigned char long_smem[];
+    float(*tile)[kLongTileFloats] = reinterpret_cast<float(*)[kLongTileFloats]>(long_smem);
+    int(*s_col)[kLongMaxChunk] =
+        reinterpret_cast<int(*)[kLongMaxChunk]>(long_smem + 2 * kLongTileFloats * sizeof(float));
+    float(*s_val)[kLongMaxChunk] = reinterpret_cast<float(*)[kLongMaxChunk]>(
+        long_smem + 2 * kLongTileFloats * sizeof(float) + 3 * kLongMaxChunk * sizeof(int));
+
+    const int t = (int)threadIdx.x;
+    const RowTask d = a.task[blockIdx.x];
+    const int F = a.feat;
+    const int f0 = (int)blockIdx.y * kLongFeatTile;
+    const int fw = F - f0 < kLongFeatTile ? F - f0 : kLongFeatTile;  // width of this tile (multiple of VEC)
+    const int vpr = fw / VEC;                                        // vectors per gathered row
+    const int C = a.chunk;
+    const int nchunks = (d.len + C - 1) / C;
+    const float *__restrict__ x = a.x + f0;
+    const int32_t *__restrict__ col = a.col + d.start;
+    const float *__restrict__ val = a.val + d.start;
+
+    // fixed (dense row in chunk, vector in row) slots of this thread
+    int sj[kLongLoads], sv[kLongLoads];
+#pragma unroll
+    for (int s = 0; s < kLongLoads; ++s) {
+        const int e = t + s * 256;
+        sj[s] = e / vpr;
+        sv[s] = (e - sj[s] * vpr) * VEC;
+    }
+
+    auto chunk_len = [&](int k) { const int left = d.len - k * C; return left < C ? left : C; };
+
+    // prologue: indices of chunks 0 and 1, dense rows of chunk 0
+    if (t < C) {
+        if (t < chunk_len(0)) { s_col[0][t] = __builtin_nontemporal_load(col + t); s_val[0][t] = __builtin_nontemporal_load(val + t); }
+        if (nchunks > 1 && t < chunk_len(1)) { s_col[1][t] = __builtin_nontemporal_load(col + C + t); s_val[1][t] = __builtin_nontemporal_load(val + C + t); }
+    }
+    __syncthreads();
+    {
+        const int cnt = chunk_len(0);
+#pragma unroll
+        for (int s = 0; s < kLongLoads; ++s) {
+            if (sj[s] < cnt) {
+                const V v = V::load(x + (size_t)s_col[0][sj[s]] * (size_t)F + sv[s]);
+                v.store(&tile[0][sj[s] * fw + sv[s]]);
+            }
+        }
+    }
+    __syncthreads();
+
+    float *dst = a.dst + (size_t)d.row * (size_t)F + f0;
+    float acc = 0.0f;
+    const bool own = t < fw;
+    if (own && a.accumulate) acc = __builtin_nontemporal_load(dst + t);
+
+    for (int k = 0; k < nchunks; ++k) {
+        const int cnt = chunk_len(k);
+        const int ncnt = k + 1 < nchunks ? chunk_len(k + 1) : 0;
+        // (1) request the dense rows of chunk k+1 and the indices of chunk k+2
+        V g[kLongLoads];
+#pragma unroll
+        for (int s = 0; s < kLongLoads; ++s) {
+            if (sj[s] < ncnt) g[s] = V::load(x + (size_t)s_col[(k + 1) % 3][sj[s]] * (size_t)F + sv[s]);
+        }
+        int ci = 0;
+        float vi = 0.0f;
+        const bool idx2 = k + 2 < nchunks && t < chunk_len(k + 2);
+        if (idx2) {
+            ci = __builtin_nontemporal_load(col + (size_t)(k + 2) * C + t);
+            vi = __builtin_nontemporal_load(val + (size_t)(k + 2) * C + t);
+        }
+        // (2) the chain over chunk k, in CSR order, out of LDS
+        if (own) {
+            const float *tb = &tile[k & 1][t];
+            const float *vb = s_val[k % 3];
+#pragma unroll 8
+            for (int j = 0; j < cnt; ++j) acc = __builtin_fmaf(vb[j], tb[j * fw], acc);
+        }
+        // (3) land what was requested in (1)
+#pragma unroll
+        for (int s = 0; s < kLongLoads; ++s) {
+            if (sj[s] < ncnt) g[s].store(&tile[(k + 1) & 1][sj[s] * fw + sv[s]]);
+        }
+        if (idx2) {
+            s_col[(k + 2) % 3][t] = ci;
+            s_val[(k + 2) % 3][t] = vi;
+        }
+        __syncthreads();
+    }
+    if (own) __builtin_nontemporal_store(acc, dst + t);
+}
+
 }  // namespace gnnagg

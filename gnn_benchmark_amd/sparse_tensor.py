@@ -38,7 +38,7 @@ class SpmmPlan:
     def info(self) -> dict:
         buf = (ctypes.c_int64 * 8)()
         _lib.check(_lib.lib().gnnagg_plan_info(self._handle, buf))
-        keys = ("rows", "cols", "nnz", "long_rows", "long_thresh", "empty_rows", "max_row_len", "rows_per_group")
+        keys = ("rows", "cols", "nnz", "huge_rows", "huge_thresh", "empty_rows", "max_row_len", "rows_per_group")
         return dict(zip(keys, [int(x) for x in buf]))
 
     def profile(self, enable: bool = True) -> None:

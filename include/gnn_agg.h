@@ -61,7 +61,9 @@ int gnnagg_spmm_csr_f32(const int64_t *rowptr, const int64_t *col, const float *
  * the sparse object: distribute_work_for_row + get/set_work_range[_for_transpose]
  * (model/ops/spmm_kernel.py:7-28, :48-57, :80-87).  On the GPU the cached object is a
  * degree-binned row schedule: rows ordered by degree class (powers of two of the row
- * length), longest rows first, and column indices narrowed to int32.  Every row is
+ * length), longest rows first, and column indices narrowed to int32.  Rows above a
+ * length threshold are fetched by a whole thread block each (gathers staged through
+ * LDS), the rest by groups of 16-64 lanes.  Every row is
  * still one fp32 FMA chain in CSR order, so results are bit-identical to
  * gnnagg_spmm_csr_f32 and to the reference's CPU operator.
  *
@@ -88,8 +90,9 @@ int gnnagg_plan_spmm_f32(gnnagg_plan *plan, const float *value, const float *mat
                          int accumulate, void *stream);
 
 /* Host-side description of a plan, info[0..7] (host pointer):
- * rows, cols, nnz, rows above the long-row threshold, that threshold,
- * rows with no stored element, largest row length, rows handled per lane group. */
+ * rows, cols, nnz, rows handled by the block-per-row kernel (longer than the next
+ * entry), that length threshold, rows with no stored element, largest row length, rows
+ * handled per lane group. */
 int gnnagg_plan_info(const gnnagg_plan *plan, int64_t *info);
 
 /* Kernel timing of a plan, for benchmarks.  After gnnagg_plan_profile(plan, 1) every

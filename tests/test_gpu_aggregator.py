@@ -18,6 +18,7 @@ from gnn_benchmark_amd.data_manager import (DataProcessor, DataProcessorForPreAg
                                             get_distributed_graph_for_pre_aggressive)
 from oracle import aggregator as oagg
 from oracle import index_maps as om
+from oracle import spmm as ospmm
 from tests.gpu_util import assert_close, assert_math_close, dev
 from tests.test_pipeline_invariant import build_pre_world, exchange as host_exchange
 from tests.world_sim import World
@@ -195,3 +196,43 @@ def test_single_rank_world_and_autograd_contract():
     assert len(ret) == 6 and all(ret[i] is None for i in (0, 2, 3, 4, 5))  # aggregator.py:208
     with pytest.raises(NotImplementedError):
         Aggregator.apply(gr, xr, 0, 2, True, True)
+
+
+def test_synthetic_partition_built_on_device_matches_oracle():
+    """The benchmark's partition builder (index maps computed with device tensors, CSR
+    matrices sorted on the device, peers' lists derived from the mirrored edges) against
+    the loop-faithful oracle run on the same edge lists: every map bit-identical."""
+    from gnn_benchmark_amd import synthetic
+
+    n, W, rank = 20000, 4, 1
+    part = synthetic.partition_edges(n, W, rank, 5, 1.8, 2000, 3000, 20000, seed=11, device="cuda")
+    graph = synthetic.build_partition_graph(part, 32, True, exchange=None, device="cuda")
+    begins = part.begins.numpy()
+    local = part.local_edges.cpu().numpy()
+    remote = part.remote_edges.cpu().numpy()
+    remote_g = [remote[0].copy(), remote[1] + begins[rank]]
+    _sent, aggr_on_recv, begin_from, recv_splits = om.split_remote_edges_for_aggr_and_graph_exchange(begins, remote_g, W)
+    # what each peer addresses to this rank: its own classification of the reversed edges
+    received = []
+    for i in range(W):
+        sel = (remote_g[0] >= begins[i]) & (remote_g[0] < begins[i + 1])
+        p_src, p_dst = remote_g[1][sel], remote_g[0][sel]
+        flags = om.decide_pre_or_post_aggr(p_src, p_dst, 1, 0)
+        out = []
+        om.collect_edges_sent_to_other_subgraphs(p_src, p_dst, flags == 1, flags == 0, out)
+        received.append(out[0])
+    for_send, begin_to, send_splits = om.split_remote_edges_recv_from_graph_exchange(received, W)
+    mats = om.transform_edge_index_to_sparse_tensor_for_pre(
+        local, [aggr_on_recv[0].copy(), aggr_on_recv[1].copy()], [for_send[0].copy(), for_send[1].copy()], begin_from,
+        begin_to, n, int(begins[rank]))
+    _same_matrix(graph.local_adj_t, mats[0])
+    _same_matrix(graph.adj_t_pre_post_aggr_from, mats[1])
+    _same_matrix(graph.adj_t_pre_post_aggr_to, mats[2])
+    assert graph.comm_splits.recv_splits == recv_splits and graph.comm_splits.send_splits == send_splits
+    assert np.array_equal(graph.in_degrees.cpu().numpy(), om.get_in_degrees(local, remote, n))
+    # the transposed arrays the backward uses
+    for m, o in zip((graph.local_adj_t, graph.adj_t_pre_post_aggr_from, graph.adj_t_pre_post_aggr_to), mats):
+        colptr, row_t, val_t = ospmm.csr_transpose(o[0], o[1], o[2], o[3][1])
+        assert np.array_equal(m.storage.colptr().cpu().numpy(), colptr)
+        assert np.array_equal(m.storage.row_T().cpu().numpy(), row_t)
+        assert np.array_equal(m.storage.value_T().cpu().numpy(), val_t)

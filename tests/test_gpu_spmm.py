@@ -15,6 +15,14 @@ from tests.gpu_util import assert_close, dev, random_csr, skewed_csr
 
 pytestmark = pytest.mark.gpu
 
+
+@pytest.fixture
+def low_block_row_threshold(monkeypatch):
+    """Plans read this when they are created: rows longer than 2048 elements then go to
+    the block-per-row kernel, which by default only takes rows that would outlast the
+    whole launch (about nnz / 4096 elements, at least 8192)."""
+    monkeypatch.setenv("GNNAGG_HUGE_THRESH", "2048")
+
 EMPTY_I32 = torch.empty(0, dtype=torch.int32)
 
 
@@ -63,7 +71,7 @@ def test_native_op_accumulates_for_every_width(feat):
 
 @pytest.mark.parametrize("feat", [1, 16, 47, 64, 100, 128, 256, 602, 1030])
 @pytest.mark.parametrize("accumulate", [True, False])
-def test_plan_path_with_long_rows_and_empty_rows(feat, accumulate):
+def test_plan_path_with_long_rows_and_empty_rows(feat, accumulate, low_block_row_threshold):
     rowptr, col, val = skewed_csr(900, 450, seed=1000 + feat)
     rng = np.random.default_rng(feat)
     x = rng.standard_normal((450, feat)).astype(np.float32)
@@ -71,7 +79,7 @@ def test_plan_path_with_long_rows_and_empty_rows(feat, accumulate):
     plan = SpmmPlan(dev(rowptr), dev(col), 900, 450)
     info = plan.info()
     deg = np.diff(rowptr)
-    assert info["long_rows"] == int((deg > info["long_thresh"]).sum()) == 3
+    assert info["huge_rows"] == int((deg > info["huge_thresh"]).sum()) == 1
     assert info["max_row_len"] == 5000 and info["empty_rows"] == int((deg == 0).sum()) > 100
     out = dev(out0)
     plan.spmm(dev(val), dev(x), out, accumulate=accumulate)
@@ -80,7 +88,41 @@ def test_plan_path_with_long_rows_and_empty_rows(feat, accumulate):
     assert np.array_equal(out.cpu().numpy(), want)  # long rows too: one chain per row
 
 
-def test_results_are_deterministic():
+@pytest.mark.parametrize("feat", [4, 33, 100, 128, 256, 300, 602])
+def test_block_per_row_kernel_chunk_edges(feat, low_block_row_threshold):
+    """Rows handled by the block-per-row kernel with lengths on and around its chunk
+    sizes (16/32/64 gathered rows per chunk), several feature tiles (F > 256), odd widths
+    (scalar loads): still the oracle's exact chain."""
+    lens = (2049, 2112, 4096, 4097, 8191, 3000, 2050, 5, 0, 64)
+    rowptr, col, val = skewed_csr(64, 700, seed=77 + feat, heavy_rows=())
+    rng = np.random.default_rng(feat)
+    deg = np.diff(rowptr)
+    deg[: len(lens)] = lens
+    rowptr = np.concatenate(([0], np.cumsum(deg))).astype(np.int64)
+    col = rng.integers(0, 700, rowptr[-1]).astype(np.int64)
+    val = rng.standard_normal(rowptr[-1]).astype(np.float32)
+    x = rng.standard_normal((700, feat)).astype(np.float32)
+    out0 = rng.standard_normal((64, feat)).astype(np.float32)
+    plan = SpmmPlan(dev(rowptr), dev(col), 64, 700)
+    assert plan.info()["huge_rows"] == 7
+    for accumulate in (True, False):
+        out = dev(out0)
+        plan.spmm(dev(val), dev(x), out, accumulate=accumulate)
+        want = _oracle(rowptr, col, val, x, out0 if accumulate else None)
+        assert np.array_equal(out.cpu().numpy(), want), (feat, accumulate)
+
+
+def test_default_threshold_keeps_moderate_rows_in_the_lane_group_kernel():
+    rowptr, col, val = skewed_csr(900, 450, seed=3)  # longest row 5000 < 8192
+    plan = SpmmPlan(dev(rowptr), dev(col), 900, 450)
+    assert plan.info()["huge_rows"] == 0 and plan.info()["huge_thresh"] == 8192
+    x = np.random.default_rng(3).standard_normal((450, 128)).astype(np.float32)
+    out = torch.zeros(900, 128, device="cuda")
+    plan.spmm(dev(val), dev(x), out)
+    assert np.array_equal(out.cpu().numpy(), _oracle(rowptr, col, val, x))
+
+
+def test_results_are_deterministic(low_block_row_threshold):
     rowptr, col, val = skewed_csr(2000, 800, seed=5)
     x = dev(np.random.default_rng(5).standard_normal((800, 128)).astype(np.float32))
     plan = SpmmPlan(dev(rowptr), dev(col), 2000, 800)
