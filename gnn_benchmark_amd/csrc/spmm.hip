@@ -81,15 +81,22 @@ hipError_t dispatch_shape(const Shape &s, const SpmmArgs &a, int rpg, hipStream_
     return hipErrorInvalidValue;
 }
 
+// The block-per-row kernel needs more than the default 64 KB of LDS per block; the limit
+// is a per-device attribute of each instantiation (set when a plan with such rows is made).
+hipError_t enable_long_rows_lds() {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(spmm_long_rows_kernel<4>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLongSmemBytes);
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(spmm_long_rows_kernel<2>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLongSmemBytes);
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(spmm_long_rows_kernel<1>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLongSmemBytes);
+    return e;
+}
+
 template <int VEC>
 hipError_t launch_long_rows(const LongArgs &a, int64_t nrows, hipStream_t st) {
-    static bool configured = false;  // the attribute is per kernel, set once per process
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(spmm_long_rows_kernel<VEC>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLongSmemBytes);
-        if (e != hipSuccess) return e;
-        configured = true;
-    }
     LongArgs args = a;
     const int tile = a.feat < kLongFeatTile ? a.feat : kLongFeatTile;
     const int vpr = tile / VEC;
@@ -364,6 +371,7 @@ extern "C" int gnnagg_plan_create(const int64_t *rowptr, const int64_t *col, int
     const int huge_class = degree_class(p->huge_thresh);
     for (int c = 0; c < huge_class; ++c) p->nhuge += (int64_t)h_out.class_count[c];
     if (p->nhuge > 0) {
+        GNNAGG_HIP(enable_long_rows_lds());
         GNNAGG_HIP(hipStreamCreateWithFlags(&p->side, hipStreamNonBlocking));
         GNNAGG_HIP(hipEventCreateWithFlags(&p->fork, hipEventDisableTiming));
         GNNAGG_HIP(hipEventCreateWithFlags(&p->join, hipEventDisableTiming));

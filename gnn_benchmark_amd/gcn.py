@@ -14,6 +14,7 @@ from typing import List, Optional, Sequence
 import torch
 import torch.nn.functional as F
 
+from . import _lib
 from .aggregator import Aggregator
 
 
@@ -38,6 +39,41 @@ class _Bf16InputLinear(torch.autograd.Function):
         return gx, gw
 
 
+class _BiasReluDropout(torch.autograd.Function):
+    """y = relu(z + bias) * (keep ? scale : 0), one fused pass, written over ``z`` (the GEMM
+    output, which nothing else reads); the gradient needs only ``y``."""
+
+    @staticmethod
+    def forward(ctx, z, bias, keep, scale):
+        if not z.is_cuda:
+            raise RuntimeError("the fused epilogue runs on a GPU (HIP) device only")
+        if z.dtype != torch.float32 or bias.dtype != torch.float32 or not z.is_contiguous() or z.dim() != 2:
+            raise RuntimeError("Input mismatch: z must be contiguous float32 [rows, feat]")
+        if keep is not None and (keep.dtype not in (torch.bool, torch.uint8) or keep.shape != z.shape
+                                 or not keep.is_contiguous()):
+            raise RuntimeError("Input mismatch: keep must be a contiguous bool/uint8 mask shaped like z")
+        with torch.cuda.device(z.device):
+            _lib.check(_lib.lib().gnnagg_bias_relu_dropout_f32(
+                _lib.ptr(z), _lib.ptr(bias.contiguous()), _lib.ptr(keep), float(scale), _lib.ptr(z), z.size(0),
+                z.size(1), _lib.current_stream(z.device)))
+        ctx.mark_dirty(z)
+        ctx.save_for_backward(z)
+        ctx.scale = float(scale)
+        return z
+
+    @staticmethod
+    def backward(ctx, grad_y):
+        (y,) = ctx.saved_tensors
+        grad_y = grad_y.contiguous()
+        grad_z = torch.empty_like(grad_y)
+        with torch.cuda.device(y.device):
+            _lib.check(_lib.lib().gnnagg_relu_dropout_backward_f32(
+                _lib.ptr(grad_y), _lib.ptr(y), ctx.scale, _lib.ptr(grad_z), grad_y.numel(),
+                _lib.current_stream(y.device)))
+        grad_bias = grad_z.sum(dim=0) if ctx.needs_input_grad[1] else None
+        return grad_z, grad_bias, None, None
+
+
 class GCNLayer(torch.nn.Module):
     def __init__(self, in_channels: int, out_channels: int, gemm: str = "fp32"):
         super().__init__()
@@ -48,12 +84,16 @@ class GCNLayer(torch.nn.Module):
         self.bias = torch.nn.Parameter(torch.zeros(out_channels))
         torch.nn.init.xavier_uniform_(self.weight, gain=torch.nn.init.calculate_gain("relu"))
 
-    def forward(self, graph, x: torch.Tensor, layer: int, is_pre_delay: bool) -> torch.Tensor:
+    def transform(self, graph, x: torch.Tensor, layer: int, is_pre_delay: bool) -> torch.Tensor:
+        """(A x / deg) W, without the bias."""
         agg = Aggregator.apply(graph, x, layer, 32, is_pre_delay, self.training)
         agg = agg / graph.in_degrees
         if self.gemm == "bf16":
-            return _Bf16InputLinear.apply(agg, self.weight) + self.bias
-        return torch.mm(agg, self.weight) + self.bias
+            return _Bf16InputLinear.apply(agg, self.weight)
+        return torch.mm(agg, self.weight)
+
+    def forward(self, graph, x: torch.Tensor, layer: int, is_pre_delay: bool) -> torch.Tensor:
+        return self.transform(graph, x, layer, is_pre_delay) + self.bias
 
 
 class GCN(torch.nn.Module):
@@ -68,13 +108,16 @@ class GCN(torch.nn.Module):
         h = x
         last = len(self.layers) - 1
         for l, layer in enumerate(self.layers):
-            h = layer(graph, h, l, is_pre_delay)
-            if l != last:
-                h = torch.relu(h)
-                if self.training and self.dropout > 0.0:
-                    if masks is None:
-                        raise ValueError("training needs the seeded dropout masks")
-                    h = h * masks[l] * (1.0 / (1.0 - self.dropout))
+            if l == last:
+                h = layer(graph, h, l, is_pre_delay)
+                break
+            z = layer.transform(graph, h, l, is_pre_delay)
+            if self.training and self.dropout > 0.0:
+                if masks is None:
+                    raise ValueError("training needs the seeded dropout masks")
+                h = _BiasReluDropout.apply(z, layer.bias, masks[l], 1.0 / (1.0 - self.dropout))
+            else:
+                h = _BiasReluDropout.apply(z, layer.bias, None, 1.0)
         return F.log_softmax(h, dim=1)
 
 

@@ -85,7 +85,10 @@ int gnnagg_plan_destroy(gnnagg_plan *plan);
  * spmm.cpp:32-35).  accumulate == 0: out = A@mat, every row written (fuses the
  * `torch.zeros` the reference allocates before the local aggregation,
  * model/layers/aggregator.py:67-70, :167-170).  Allocates nothing and does not
- * synchronise. */
+ * synchronise the host.  A plan owns a few events (and, when it holds very long rows, a
+ * side stream joined back into `stream` before the call returns), so two calls on the
+ * SAME plan must not overlap: issue them on one stream, or order them yourself.  Calls
+ * on different plans are independent. */
 int gnnagg_plan_spmm_f32(gnnagg_plan *plan, const float *value, const float *mat, float *out, int64_t feat,
                          int accumulate, void *stream);
 
@@ -138,6 +141,20 @@ int gnnagg_coo_to_csr(const int64_t *row, const int64_t *col, const float *value
  * ------------------------------------------------------------------------------- */
 int gnnagg_gather_rows_f32(const float *src, const int64_t *index, float *out, int64_t n_index, int64_t feat,
                            void *stream);
+
+/* ---------------------------------------------------------------------------------
+ * Fused layer epilogue around the aggregation path (the full train-step workload):
+ *   y[i,f] = relu(z[i,f] + bias[f]) * (keep[i,f] ? scale : 0)          forward
+ *   grad_z = y > 0 ? grad_y * scale : 0                                 backward
+ * z, y fp32 [rows, feat] (y may alias z), bias fp32 [feat], keep uint8 [rows, feat] or
+ * NULL (no dropout; pass scale = 1), grad_* fp32 [count] (grad_z may alias grad_y).
+ * The reference runs its epilogue (dropout, LayerNorm, ReLU) as separate torch ops
+ * (model/DistSAGE.py:55-66); this fused form belongs to this build's GCN layer stack.
+ * ------------------------------------------------------------------------------- */
+int gnnagg_bias_relu_dropout_f32(const float *z, const float *bias, const uint8_t *keep, float scale, float *y,
+                                 int64_t rows, int64_t feat, void *stream);
+int gnnagg_relu_dropout_backward_f32(const float *grad_y, const float *y, float scale, float *grad_z, int64_t count,
+                                     void *stream);
 
 #ifdef __cplusplus
 }

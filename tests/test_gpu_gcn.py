@@ -115,3 +115,29 @@ def test_train_step_matches_cpu_autograd(gemm, tol):
     assert abs(losses[0] - float(cpu_loss)) <= tol * max(1.0, abs(float(cpu_loss)))
     for b, p in zip(before, model.parameters()):
         assert float((p.detach() - b).abs().max()) <= 5 * 0.01 * 1.01
+
+
+@pytest.mark.parametrize("rows,feat", [(1000, 256), (333, 47), (64, 4), (1, 1)])
+@pytest.mark.parametrize("with_mask", [True, False])
+def test_fused_epilogue_equals_separate_ops(rows, feat, with_mask):
+    gen = torch.Generator(device="cuda").manual_seed(rows + feat)
+    z = torch.randn(rows, feat, device="cuda", generator=gen)
+    bias = torch.randn(feat, device="cuda", generator=gen)
+    keep = (torch.rand(rows, feat, device="cuda", generator=gen) >= 0.5) if with_mask else None
+    scale = 2.0 if with_mask else 1.0
+    g = torch.randn(rows, feat, device="cuda", generator=gen)
+
+    z_ref = z.clone().requires_grad_()
+    b_ref = bias.clone().requires_grad_()
+    y_ref = torch.relu(z_ref + b_ref)
+    if with_mask:
+        y_ref = y_ref * keep * scale
+    y_ref.backward(g)
+
+    z_in = z.clone().requires_grad_()
+    b_in = bias.clone().requires_grad_()
+    y = gcn._BiasReluDropout.apply(z_in * 1.0, b_in, keep, scale)  # * 1.0: a non-leaf the op may overwrite
+    y.backward(g)
+    assert torch.equal(y.detach(), y_ref.detach())
+    assert torch.equal(z_in.grad, z_ref.grad)
+    assert torch.allclose(b_in.grad, b_ref.grad, rtol=1e-5, atol=1e-5)  # column sums in another order

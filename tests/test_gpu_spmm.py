@@ -252,3 +252,37 @@ def test_full_size_properties_power_law():
     take = np.concatenate([np.arange(rp[r], rp[r + 1]) for r in rows])
     want = _oracle(sub_ptr, c[take], v[take], x1.cpu().numpy())
     assert_close(o1[torch.from_numpy(rows).cuda()], want, "row sample vs oracle")
+
+
+def test_committed_reference_outputs_bit_for_bit():
+    """Outputs of the reference's own compiled operator, committed as fixtures
+    (tests/golden/make_spmm_reference_vectors.py): the HIP paths reproduce them exactly."""
+    from tests.test_oracle_spmm import _golden_cases
+
+    for c in _golden_cases():
+        rows, feat = c["out0"].shape
+        out = dev(c["out0"])
+        computation_ops.spmm(dev(c["rowptr"]), dev(c["col"]), dev(c["val"]), dev(c["x"]), out, rows, EMPTY_I32, EMPTY_I32)
+        assert np.array_equal(out.cpu().numpy(), c["out"])
+        out = dev(c["out0"])
+        SpmmPlan(dev(c["rowptr"]), dev(c["col"]), rows, c["x"].shape[0]).spmm(dev(c["val"]), dev(c["x"]), out)
+        assert np.array_equal(out.cpu().numpy(), c["out"])
+
+
+def test_hip_equals_reference_compiled_op_on_this_host(reference_op):
+    """The reference's compiled operator run on this machine's CPU against the HIP path on
+    the same inputs (skipped where oracle/_ref cannot be loaded)."""
+    a = random_csr(5003, 1777, 0.004, seed=21)
+    rng = np.random.default_rng(21)
+    for feat in (100, 128, 256):
+        x = rng.standard_normal((1777, feat)).astype(np.float32)
+        out0 = rng.standard_normal((5003, feat)).astype(np.float32)
+        theirs = torch.from_numpy(out0.copy())
+        threads = torch.get_num_threads()
+        reference_op.spmm(torch.from_numpy(a.indptr.astype(np.int64)), torch.from_numpy(a.indices.astype(np.int64)),
+                          torch.from_numpy(a.data), torch.from_numpy(x), theirs, 5003,
+                          torch.from_numpy(ospmm.divide_work(5003, threads)), torch.tensor([0, feat], dtype=torch.int32))
+        src = SparseTensor.from_scipy(a).cuda()
+        out = dev(out0)
+        SPMM_forward(src, dev(x), out)
+        assert np.array_equal(out.cpu().numpy(), theirs.numpy())

@@ -153,3 +153,21 @@ def test_oracle_backward_is_bit_identical_to_reference_op(reference_op):
     reference_op.spmm(torch.from_numpy(colptr), torch.from_numpy(row_t), torch.from_numpy(val_t), torch.from_numpy(g),
                       theirs, a.shape[1], rs, torch.tensor([0, 128], dtype=torch.int32))
     assert np.array_equal(mine, theirs.numpy())
+
+
+# ---------------------------------------------------------------- against committed reference outputs
+def _golden_cases():
+    import os
+
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "spmm_reference_op_vectors.npz")
+    z = np.load(path)
+    n = len({k.split("_")[0] for k in z.files})
+    return [{name: z[f"c{i}_{name}"] for name in ("rowptr", "col", "val", "x", "out0", "out")} for i in range(n)]
+
+
+def test_oracle_reproduces_committed_reference_outputs_bit_for_bit():
+    # outputs of the reference's compiled operator (tests/golden/make_spmm_reference_vectors.py)
+    for c in _golden_cases():
+        got = c["out0"].copy()
+        ospmm.spmm(c["rowptr"], c["col"], c["val"], c["x"], got)
+        assert np.array_equal(got, c["out"])
