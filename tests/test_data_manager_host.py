@@ -214,3 +214,79 @@ def test_remap_random_equals_oracle():
         assert om.remap_remote_nodes_id(o_nodes, begins) == DataProcessorForPreAggresive.remap_remote_nodes_id(
             t_nodes, torch.from_numpy(begins))
         assert np.array_equal(o_nodes, t_nodes.numpy())
+
+
+# ------------------------------------------------------------------ the synthetic workload generators (host path)
+def test_synthetic_power_law_graph_is_a_valid_normalised_csr():
+    from gnn_benchmark_amd import synthetic
+
+    g = synthetic.power_law_graph(3000, 8, 1.8, 400, seed=2, device="cpu")
+    rowptr, col, val = [t.numpy() for t in g.adj.csr()]
+    n = g.num_nodes
+    assert rowptr[0] == 0 and rowptr[-1] == col.size == g.nnz and np.all(np.diff(rowptr) >= 1)  # self-loops
+    row = np.repeat(np.arange(n), np.diff(rowptr))
+    keys = row * n + col
+    assert np.all(np.diff(keys) > 0)  # (row, col) sorted, no repeated entry
+    assert np.array_equal(np.sort(col * n + row), keys)  # symmetric pattern
+    deg = np.diff(rowptr).astype(np.float64)
+    assert np.allclose(val, 1.0 / np.sqrt(deg[row] * deg[col]), rtol=1e-6)  # D^-1/2 (A+I) D^-1/2
+    assert g.max_degree == int(deg.max())
+    same = synthetic.power_law_graph(3000, 8, 1.8, 400, seed=2, device="cpu")
+    assert all(torch.equal(a, b) for a, b in zip(g.adj.csr(), same.adj.csr()))  # seeded
+
+
+def test_synthetic_dense_degree_graph_is_row_normalised():
+    from gnn_benchmark_amd import synthetic
+
+    g = synthetic.dense_degree_graph(1500, 3.5, 1.0, seed=4, device="cpu")
+    rowptr, col, val = [t.numpy() for t in g.adj.csr()]
+    sums = np.add.reduceat(val.astype(np.float64), rowptr[:-1])
+    assert np.all(np.diff(rowptr) >= 1) and np.allclose(sums, 1.0, atol=1e-5)
+
+
+def test_synthetic_partition_maps_equal_oracle_on_host():
+    """Same check as the GPU test of the partition builder, on CPU tensors: the maps and
+    CSR matrices of a synthetic partition (peers' lists derived from the mirrored edges)
+    against the loop-faithful oracle."""
+    from gnn_benchmark_amd import synthetic
+
+    n, W, rank = 4000, 4, 2
+    part = synthetic.partition_edges(n, W, rank, 5, 1.8, 500, 700, 4000, seed=9, device="cpu")
+    begins = part.begins.numpy()
+    assert int(part.remote_edges[0].min()) >= 0 and int(part.remote_edges[0].max()) < W * n
+    owner = part.remote_edges[0] // n
+    assert not bool((owner == rank).any())  # remote sources never lie in this rank's range
+    for pre in (True, False):
+        graph = synthetic.build_partition_graph(part, 16, pre, exchange=None, device="cpu")
+        local = part.local_edges.numpy()
+        remote = part.remote_edges.numpy()
+        if pre:
+            remote_g = [remote[0].copy(), remote[1] + begins[rank]]
+            _s, aggr, begin_from, recv_splits = om.split_remote_edges_for_aggr_and_graph_exchange(begins, remote_g, W)
+            received = []
+            for i in range(W):
+                sel = (remote_g[0] >= begins[i]) & (remote_g[0] < begins[i + 1])
+                p_src, p_dst = remote_g[1][sel], remote_g[0][sel]
+                flags = om.decide_pre_or_post_aggr(p_src, p_dst, 1, 0)
+                out = []
+                om.collect_edges_sent_to_other_subgraphs(p_src, p_dst, flags == 1, flags == 0, out)
+                received.append(out[0])
+            for_send, begin_to, send_splits = om.split_remote_edges_recv_from_graph_exchange(received, W)
+            mats = om.transform_edge_index_to_sparse_tensor_for_pre(
+                local, [aggr[0].copy(), aggr[1].copy()], [for_send[0].copy(), for_send[1].copy()], begin_from, begin_to,
+                n, int(begins[rank]))
+            got = (graph.local_adj_t, graph.adj_t_pre_post_aggr_from, graph.adj_t_pre_post_aggr_to)
+            assert graph.comm_splits.recv_splits == recv_splits and graph.comm_splits.send_splits == send_splits
+        else:
+            e = [remote[0].copy(), remote[1].copy()]
+            om.sort_remote_edges_list_based_on_remote_nodes(e)
+            nodes, ranges, counts = om.obtain_remote_nodes_list(e, n, begins, W)
+            mats = om.transform_edge_index_to_sparse_tensor(local, e, n, len(nodes))
+            got = (graph.local_adj_t, graph.remote_adj_t)
+            assert graph.comm_splits.recv_splits == counts.tolist()
+            idx = graph.idx_nodes_send_to_others.numpy()
+            assert idx.size == sum(graph.comm_splits.send_splits) and idx.min() >= 0 and idx.max() < n
+        for m, o in zip(got, mats):
+            rowptr, col, val = [t.numpy() for t in m.csr()]
+            assert tuple(m.sparse_sizes()) == tuple(o[3])
+            assert np.array_equal(rowptr, o[0]) and np.array_equal(col, o[1]) and np.array_equal(val, o[2])
