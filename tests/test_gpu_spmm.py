@@ -286,3 +286,55 @@ def test_hip_equals_reference_compiled_op_on_this_host(reference_op):
         out = dev(out0)
         SPMM_forward(src, dev(x), out)
         assert np.array_equal(out.cpu().numpy(), theirs.numpy())
+
+
+def test_runs_on_the_callers_stream(low_block_row_threshold):
+    """Work is enqueued on torch's CURRENT stream (also the block-per-row kernel, which forks
+    to the plan's side stream and joins back): results are right without any device-wide
+    synchronisation in between, and a later op on the same stream sees them."""
+    rowptr, col, val = skewed_csr(900, 450, seed=31)
+    x = np.random.default_rng(31).standard_normal((450, 128)).astype(np.float32)
+    plan = SpmmPlan(dev(rowptr), dev(col), 900, 450)
+    assert plan.info()["huge_rows"] == 1
+    want = _oracle(rowptr, col, val, x)
+    s = torch.cuda.Stream()
+    d_val, d_x = dev(val), dev(x)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(s):
+        out = torch.zeros(900, 128, device="cuda")
+        for _ in range(3):
+            out.zero_()
+            plan.spmm(d_val, d_x, out)
+        doubled = out * 2.0
+    s.synchronize()
+    assert np.array_equal(out.cpu().numpy(), want)
+    assert np.array_equal(doubled.cpu().numpy(), want * 2.0)
+
+
+@pytest.mark.parametrize("with_block_rows", [False, True])
+def test_plan_spmm_can_be_captured_in_a_hip_graph(monkeypatch, with_block_rows):
+    """The plan call allocates nothing and never synchronises the host, so it can be
+    recorded into a graph; every replay (with fresh operand contents) must equal eager."""
+    if with_block_rows:
+        monkeypatch.setenv("GNNAGG_HUGE_THRESH", "2048")
+    rowptr, col, val = skewed_csr(900, 450, seed=41)
+    plan = SpmmPlan(dev(rowptr), dev(col), 900, 450)
+    assert (plan.info()["huge_rows"] > 0) == with_block_rows
+    rng = np.random.default_rng(41)
+    d_val = dev(val)
+    x = torch.zeros(450, 64, device="cuda")
+    out = torch.zeros(900, 64, device="cuda")
+    x.copy_(dev(rng.standard_normal((450, 64)).astype(np.float32)))
+    plan.spmm(d_val, x, out, accumulate=False)  # warm-up outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        plan.spmm(d_val, x, out, accumulate=False)
+    for _ in range(3):
+        xh = rng.standard_normal((450, 64)).astype(np.float32)
+        x.copy_(dev(xh))
+        out.fill_(7.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(out.cpu().numpy(), _oracle(rowptr, col, val, xh))
