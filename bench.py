@@ -128,6 +128,36 @@ def cpu_baseline_spmm(src, x_host, g_host, reps=3):
             "ms_per_step": round(sec * 1e3, 2)}
 
 
+def cpu_time_product(rowptr, col, val, x_host, rows, reps=2):
+    """Median seconds of one out += A @ x on the host cores (reference's compiled operator if
+    loadable, else the C port), plus which of the two ran and the thread count."""
+    import numpy as np
+    import torch
+
+    from oracle import spmm as ospmm
+
+    threads = ospmm.max_threads()
+    feat = x_host.shape[1]
+    rs = ospmm.distribute_work_for_row(rowptr, np.ones(col.shape[0], np.float32), threads)
+    out = np.zeros((rows, feat), dtype=np.float32)
+    ref = ospmm.load_reference_op()
+    if ref is not None:
+        torch.set_num_threads(threads)
+        args = (torch.from_numpy(rowptr), torch.from_numpy(col), torch.from_numpy(val), torch.from_numpy(x_host),
+                torch.from_numpy(out), rows, torch.from_numpy(rs), torch.tensor([0, feat], dtype=torch.int32))
+        run = lambda: ref.spmm(*args)  # noqa: E731
+    else:
+        run = lambda: ospmm.spmm(rowptr, col, val, x_host, out, rs, threads)  # noqa: E731
+    run()
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    return times[len(times) // 2], ("reference" if ref is not None else "port"), threads
+
+
 def spmm_pair(src, feat, steps, warmup, gen):
     """Times `steps` (forward + transposed backward) steps; returns (report, x, g)."""
     import torch
@@ -219,7 +249,14 @@ def run_c3(args):
     gen = torch.Generator(device=dev).manual_seed(args.seed + 3)
     out = {"graph": g.description, "nodes": g.num_nodes, "nnz": g.nnz, "max_row_len": g.max_degree, "runs": []}
     for f in (602, 256):
-        out["runs"].append(spmm_pair(g.adj, f, max(3, args.steps // 4), 2, gen)[0])
+        r, x, _g = spmm_pair(g.adj, f, max(3, args.steps // 4), 2, gen)
+        if not args.no_cpu_baseline and f == 602:
+            rowptr, col, val = [t.cpu().numpy() for t in g.adj.csr()]
+            sec, kind, threads = cpu_time_product(rowptr, col, val, x.cpu().numpy(), g.num_nodes)
+            r["forward"]["cpu_ms"] = round(sec * 1e3, 1)
+            r["forward"]["cpu"] = f"{kind} operator, {threads} threads"
+        out["runs"].append(r)
+        del x, _g
     return out
 
 
@@ -265,6 +302,11 @@ def run_c4(args, graph, setup_s):
         rows, cols = m.sparse_sizes()
         _, ms = time_plan(m.get_plan(), m.csr()[2], src_x, dst, steps, 2, accumulate=True)
         ops.append(op_report(name, m.nnz(), rows, cols, feat, ms, m.get_plan().info()["empty_rows"]))
+        if not args.no_cpu_baseline:
+            rowptr, col, val = [t.cpu().numpy() for t in m.csr()]
+            sec, kind, threads = cpu_time_product(rowptr, col, val, src_x.cpu().numpy(), rows)
+            ops[-1]["cpu_ms"] = round(sec * 1e3, 1)
+            ops[-1]["cpu"] = f"{kind} operator, {threads} threads"
         back = torch.zeros(cols, feat, device=dev)
         _, ms = time_plan(m.get_plan_for_transpose(), m.storage.value_T(), dst, back, steps, 2, accumulate=True)
         ops.append(op_report(name.split(" ")[0] + " transposed (gradient direction)", m.nnz(), cols, rows, feat, ms,
