@@ -214,21 +214,18 @@ def test_transposed_arrays_and_csr_build_are_bit_exact():
     assert all(torch.equal(a.cpu(), b) for a, b in zip(got.csr(), host.csr()))
 
 
-def test_full_size_properties_power_law():
-    """Size-independent checks on a graph too large for the oracle to sweep fully:
-    linearity in the dense operand, agreement of the plan and plan-less paths, the
-    adjoint identity <A x, y> == <x, A^T y>, and oracle parity on a row sample."""
-    from gnn_benchmark_amd.synthetic import power_law_graph
-
-    g = power_law_graph(num_nodes=300_000, mean_out_degree=12, zipf_s=1.8, max_degree=15000, seed=3, device="cuda")
-    src, n = g.adj, g.num_nodes
-    gen = torch.Generator(device="cuda").manual_seed(0)
-    x1 = torch.randn(n, 128, device="cuda", generator=gen)
-    x2 = torch.randn(n, 128, device="cuda", generator=gen)
-    y = torch.randn(n, 128, device="cuda", generator=gen)
+def _check_properties(src, feat, n_sample, seed):
+    """Size-independent checks of one matrix: linearity in the dense operand, agreement of
+    the plan and plan-less paths, the adjoint identity <A x, y> == <x, A^T y>, and exact
+    oracle parity on a row sample that includes the longest rows."""
+    rows, cols = src.sparse_sizes()
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    x1 = torch.randn(cols, feat, device="cuda", generator=gen)
+    x2 = torch.randn(cols, feat, device="cuda", generator=gen)
+    y = torch.randn(rows, feat, device="cuda", generator=gen)
 
     def fwd(x):
-        out = torch.empty(n, 128, device="cuda")
+        out = torch.empty(rows, feat, device="cuda")
         SPMM_forward(src, x, out, accumulate=False)
         return out
 
@@ -236,22 +233,56 @@ def test_full_size_properties_power_law():
     scale = float(o12.abs().max())
     assert float((o12 - (o1 + 2.0 * o2)).abs().max()) <= 2e-5 * scale
     rowptr, col, val = src.csr()
-    direct = torch.zeros(n, 128, device="cuda")
-    computation_ops.spmm(rowptr, col, val, x1, direct, n, EMPTY_I32, EMPTY_I32)
-    assert float((direct - o1).abs().max()) <= 2e-5 * scale
-    gt = torch.empty(n, 128, device="cuda")
+    direct = torch.zeros(rows, feat, device="cuda")
+    computation_ops.spmm(rowptr, col, val, x1, direct, rows, EMPTY_I32, EMPTY_I32)
+    assert torch.equal(direct, o1)  # both paths run the same chain per row
+    gt = torch.empty(cols, feat, device="cuda")
     SPMM_backward(src, y, gt, accumulate=False)
     lhs = float((o1.double() * y.double()).sum())
     rhs = float((x1.double() * gt.double()).sum())
     assert abs(lhs - rhs) <= 1e-6 * max(abs(lhs), abs(rhs), 1.0) + 1e-3
-    # oracle parity on 4096 sampled rows (heaviest rows included)
     deg = (rowptr[1:] - rowptr[:-1]).cpu().numpy()
-    rows = np.unique(np.concatenate([np.argsort(deg)[-64:], np.random.default_rng(0).integers(0, n, 4032)]))
-    rp, c, v = rowptr.cpu().numpy(), col.cpu().numpy(), val.cpu().numpy()
-    sub_ptr = np.concatenate(([0], np.cumsum(deg[rows]))).astype(np.int64)
-    take = np.concatenate([np.arange(rp[r], rp[r + 1]) for r in rows])
-    want = _oracle(sub_ptr, c[take], v[take], x1.cpu().numpy())
-    assert_close(o1[torch.from_numpy(rows).cuda()], want, "row sample vs oracle")
+    pick = np.unique(np.concatenate([np.argsort(deg)[-64:], np.random.default_rng(seed).integers(0, rows, n_sample)]))
+    rp = rowptr.cpu().numpy()
+    take = torch.from_numpy(np.concatenate([np.arange(rp[r], rp[r + 1]) for r in pick])).cuda()
+    sub_ptr = np.concatenate(([0], np.cumsum(deg[pick]))).astype(np.int64)
+    want = _oracle(sub_ptr, col[take].cpu().numpy(), val[take].cpu().numpy(), x1.cpu().numpy())
+    assert np.array_equal(o1[torch.from_numpy(pick).cuda()].cpu().numpy(), want)
+
+
+def test_full_size_properties_config2():
+    """The headline workload at its full size: 2.45 M nodes, ~122 M stored elements, F=100."""
+    from gnn_benchmark_amd.synthetic import power_law_graph
+
+    g = power_law_graph(num_nodes=2_450_000, mean_out_degree=25.0, zipf_s=1.8, max_degree=15000, seed=0, device="cuda")
+    assert 115_000_000 < g.nnz < 130_000_000 and g.max_degree > 10_000
+    _check_properties(g.adj, 100, 4000, seed=0)
+
+
+def test_full_size_properties_config4_partition():
+    """One partition at full size (7 M local nodes, ~100 M local and ~20 M boundary
+    elements): the three matrices of the pre/post pipeline, F=128, and the pipeline itself
+    against its three products."""
+    from gnn_benchmark_amd import Aggregator, synthetic
+
+    n = 7_000_000
+    part = synthetic.partition_edges(n, 16, 3, 6.8, 1.8, 15000, 3_000_000, 20_000_000, seed=4, device="cuda")
+    graph = synthetic.build_partition_graph(part, 128, True, exchange=synthetic.SeededHaloExchange(4), device="cuda")
+    assert 95_000_000 < graph.local_adj_t.nnz() < 110_000_000
+    assert 2_800_000 < graph.adj_t_pre_post_aggr_from.sparse_size(1) < 3_200_000
+    for i, m in enumerate((graph.local_adj_t, graph.adj_t_pre_post_aggr_from, graph.adj_t_pre_post_aggr_to)):
+        _check_properties(m, 128, 2000, seed=10 + i)
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randn(n, 128, device="cuda", generator=gen)
+    out = Aggregator.apply(graph, x, 0, 32, True, True)
+    send = graph.comm_buf.send_buf.clone()
+    want = torch.zeros(n, 128, device="cuda")
+    SPMM_forward(graph.local_adj_t, x, want)
+    SPMM_forward(graph.adj_t_pre_post_aggr_from, graph.comm_buf.recv_buf, want)
+    assert torch.equal(out, want)
+    want_send = torch.zeros_like(send)
+    SPMM_forward(graph.adj_t_pre_post_aggr_to, x, want_send)
+    assert torch.equal(send, want_send)
 
 
 def test_committed_reference_outputs_bit_for_bit():
