@@ -384,8 +384,16 @@ extern "C" int gnnagg_plan_create(const int64_t *rowptr, const int64_t *col, int
 
 extern "C" int gnnagg_plan_destroy(gnnagg_plan *plan) {
     if (!plan) return GNNAGG_OK;
-    GNNAGG_HIP(hipDeviceSynchronize());
+    // wait for the work of the plan's own device, whichever device is current
+    const int device = plan->device;
+    int current = 0;
+    GNNAGG_HIP(hipGetDevice(&current));
+    if (current != device) GNNAGG_HIP(hipSetDevice(device));
+    const hipError_t sync = hipDeviceSynchronize();
     plan_free(plan);
+    if (current != device) (void)hipSetDevice(current);
+    if (sync != hipSuccess)
+        return fail(GNNAGG_ERR_HIP, "hipDeviceSynchronize failed while destroying a plan: %s", hipGetErrorString(sync));
     return GNNAGG_OK;
 }
 
