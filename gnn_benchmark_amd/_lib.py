@@ -28,6 +28,7 @@ EXPORTS = (
     "gnnagg_coo_to_csr",
     "gnnagg_gather_rows_f32",
     "gnnagg_bias_relu_dropout_f32",
+    "gnnagg_relu_dropout_backward_blocks",
     "gnnagg_relu_dropout_backward_f32",
 )
 
@@ -84,9 +85,11 @@ def lib() -> ctypes.CDLL:
     L.gnnagg_gather_rows_f32.restype = i32
     L.gnnagg_gather_rows_f32.argtypes = [vp, vp, vp, i64, i64, vp]
     L.gnnagg_bias_relu_dropout_f32.restype = i32
-    L.gnnagg_bias_relu_dropout_f32.argtypes = [vp, vp, vp, ctypes.c_float, vp, i64, i64, vp]
+    L.gnnagg_bias_relu_dropout_f32.argtypes = [vp, vp, vp, vp, ctypes.c_float, vp, i64, i64, vp]
     L.gnnagg_relu_dropout_backward_f32.restype = i32
-    L.gnnagg_relu_dropout_backward_f32.argtypes = [vp, vp, ctypes.c_float, vp, i64, vp]
+    L.gnnagg_relu_dropout_backward_f32.argtypes = [vp, vp, vp, ctypes.c_float, vp, vp, i64, i64, vp]
+    L.gnnagg_relu_dropout_backward_blocks.restype = i32
+    L.gnnagg_relu_dropout_backward_blocks.argtypes = [i64, i64]
     if L.gnnagg_abi_version() != ABI_VERSION:
         raise RuntimeError("libgnnagg.so was built from a different include/gnn_agg.h; rebuild it")
     _lib = L

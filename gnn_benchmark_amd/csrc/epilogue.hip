@@ -1,6 +1,8 @@
 // Fused elementwise epilogue of a GCN layer around the aggregation path:
-// y = relu(z + bias) * (keep ? scale : 0) and its gradient.  HBM-bound streaming
-// kernels (one read and one write of the activation instead of four passes).
+// y = relu(z / row_div + bias) * (keep ? scale : 0) and its gradient.  HBM-bound streaming
+// kernels (one read and one write of the activation instead of five passes).  The
+// per-row divisor carries the mean-aggregation normalisation (1/in-degree), moved behind
+// the dense product: D^-1 (A X) W == D^-1 ((A X) W).
 #include "common.h"
 
 namespace gnnagg {
@@ -9,8 +11,8 @@ namespace {
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef unsigned char u8x4 __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ float relu_keep(float z, float b, unsigned char k, float scale) {
-    const float a = z + b;
+__device__ __forceinline__ float relu_keep(float z, float d, float b, unsigned char k, float scale) {
+    const float a = z / d + b;
     const float r = a > 0.0f ? a : 0.0f;
     return k ? r * scale : 0.0f;
 }
@@ -18,56 +20,113 @@ __device__ __forceinline__ float relu_keep(float z, float b, unsigned char k, fl
 // n4 = rows * feat / 4 vectors; feat4 = feat / 4
 __global__ __launch_bounds__(256) void bias_relu_dropout_v4_kernel(const f4 *__restrict__ z,
                                                                    const f4 *__restrict__ bias,
-                                                                   const u8x4 *__restrict__ keep, float scale,
+                                                                   const u8x4 *__restrict__ keep,
+                                                                   const float *__restrict__ row_div, float scale,
                                                                    f4 *__restrict__ y, int64_t n4, int feat4) {
     const int64_t stride = (int64_t)gridDim.x * 256;
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += stride) {
         const f4 v = __builtin_nontemporal_load(z + i);
-        const f4 b = bias[i % feat4];
+        const int64_t row = i / feat4;
+        const f4 b = bias[i - row * feat4];
+        const float d = row_div ? row_div[row] : 1.0f;
         u8x4 k = {1, 1, 1, 1};
         if (keep) k = __builtin_nontemporal_load(keep + i);
         f4 r;
-        r.x = relu_keep(v.x, b.x, k.x, scale);
-        r.y = relu_keep(v.y, b.y, k.y, scale);
-        r.z = relu_keep(v.z, b.z, k.z, scale);
-        r.w = relu_keep(v.w, b.w, k.w, scale);
+        r.x = relu_keep(v.x, d, b.x, k.x, scale);
+        r.y = relu_keep(v.y, d, b.y, k.y, scale);
+        r.z = relu_keep(v.z, d, b.z, k.z, scale);
+        r.w = relu_keep(v.w, d, b.w, k.w, scale);
         __builtin_nontemporal_store(r, y + i);
     }
 }
 
 __global__ __launch_bounds__(256) void bias_relu_dropout_kernel(const float *__restrict__ z,
                                                                 const float *__restrict__ bias,
-                                                                const unsigned char *__restrict__ keep, float scale,
+                                                                const unsigned char *__restrict__ keep,
+                                                                const float *__restrict__ row_div, float scale,
                                                                 float *__restrict__ y, int64_t n, int feat) {
     const int64_t stride = (int64_t)gridDim.x * 256;
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride)
-        y[i] = relu_keep(z[i], bias[i % feat], keep ? keep[i] : (unsigned char)1, scale);
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
+        const int64_t row = i / feat;
+        y[i] = relu_keep(z[i], row_div ? row_div[row] : 1.0f, bias[i - row * feat], keep ? keep[i] : (unsigned char)1,
+                         scale);
+    }
 }
 
-// gz = y > 0 ? g * scale : 0   (y is the OUTPUT of the forward: it is 0 exactly where the
-// unit was inactive or dropped)
+// gz = (y > 0 ? g * scale : 0) / row_div   (y is the OUTPUT of the forward: it is 0 exactly
+// where the unit was inactive or dropped)
 __global__ __launch_bounds__(256) void relu_dropout_backward_v4_kernel(const f4 *__restrict__ g,
-                                                                       const f4 *__restrict__ y, float scale,
-                                                                       f4 *__restrict__ gz, int64_t n4) {
+                                                                       const f4 *__restrict__ y,
+                                                                       const float *__restrict__ row_div, float scale,
+                                                                       f4 *__restrict__ gz, int64_t n4, int feat4) {
     const int64_t stride = (int64_t)gridDim.x * 256;
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += stride) {
         const f4 gv = __builtin_nontemporal_load(g + i);
         const f4 yv = __builtin_nontemporal_load(y + i);
+        const float d = row_div ? row_div[i / feat4] : 1.0f;
         f4 r;
-        r.x = yv.x > 0.0f ? gv.x * scale : 0.0f;
-        r.y = yv.y > 0.0f ? gv.y * scale : 0.0f;
-        r.z = yv.z > 0.0f ? gv.z * scale : 0.0f;
-        r.w = yv.w > 0.0f ? gv.w * scale : 0.0f;
+        r.x = yv.x > 0.0f ? gv.x * scale / d : 0.0f;
+        r.y = yv.y > 0.0f ? gv.y * scale / d : 0.0f;
+        r.z = yv.z > 0.0f ? gv.z * scale / d : 0.0f;
+        r.w = yv.w > 0.0f ? gv.w * scale / d : 0.0f;
         __builtin_nontemporal_store(r, gz + i);
     }
 }
 
 __global__ __launch_bounds__(256) void relu_dropout_backward_kernel(const float *__restrict__ g,
-                                                                    const float *__restrict__ y, float scale,
-                                                                    float *__restrict__ gz, int64_t n) {
+                                                                    const float *__restrict__ y,
+                                                                    const float *__restrict__ row_div, float scale,
+                                                                    float *__restrict__ gz, int64_t n, int feat) {
     const int64_t stride = (int64_t)gridDim.x * 256;
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride)
-        gz[i] = y[i] > 0.0f ? g[i] * scale : 0.0f;
+        gz[i] = y[i] > 0.0f ? g[i] * scale / (row_div ? row_div[i / feat] : 1.0f) : 0.0f;
+}
+
+// Same gradient, organised by rows so that the bias gradient comes out of the same pass:
+// block b owns rows [b*rows_per_block, +rows_per_block); thread t owns the column vector
+// t % feat4 and walks the rows t / feat4, + 256 / feat4, ...  Its running sum of the
+// gradient BEFORE the row division (that is d/d bias) is reduced over the threads of the
+// same column vector in a fixed order and written to bias_partial[b, :].  Needs
+// feat4 <= 256 and 256 % feat4 == 0.
+__global__ __launch_bounds__(256) void relu_dropout_backward_rows_kernel(const f4 *__restrict__ g,
+                                                                         const f4 *__restrict__ y,
+                                                                         const float *__restrict__ row_div, float scale,
+                                                                         f4 *__restrict__ gz,
+                                                                         f4 *__restrict__ bias_partial, int64_t rows,
+                                                                         int feat4, int rows_per_block) {
+    __shared__ f4 sums[256];
+    const int t = (int)threadIdx.x;
+    const int c = t % feat4;
+    const int lanes = 256 / feat4;  // rows in flight per block step
+    const int64_t r_begin = (int64_t)blockIdx.x * rows_per_block;
+    int64_t r_end = r_begin + rows_per_block;
+    if (r_end > rows) r_end = rows;
+    f4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int64_t r = r_begin + t / feat4; r < r_end; r += lanes) {
+        const int64_t i = r * feat4 + c;
+        const f4 gv = __builtin_nontemporal_load(g + i);
+        const f4 yv = __builtin_nontemporal_load(y + i);
+        const float d = row_div ? row_div[r] : 1.0f;
+        f4 pre;
+        pre.x = yv.x > 0.0f ? gv.x * scale : 0.0f;
+        pre.y = yv.y > 0.0f ? gv.y * scale : 0.0f;
+        pre.z = yv.z > 0.0f ? gv.z * scale : 0.0f;
+        pre.w = yv.w > 0.0f ? gv.w * scale : 0.0f;
+        acc += pre;
+        f4 out;
+        out.x = pre.x / d;
+        out.y = pre.y / d;
+        out.z = pre.z / d;
+        out.w = pre.w / d;
+        __builtin_nontemporal_store(out, gz + i);
+    }
+    sums[t] = acc;
+    __syncthreads();
+    if (t < feat4) {
+        f4 total = sums[t];
+        for (int k = 1; k < lanes; ++k) total += sums[t + k * feat4];
+        bias_partial[(int64_t)blockIdx.x * feat4 + t] = total;
+    }
 }
 
 unsigned stream_grid(int64_t n_items) {
@@ -84,8 +143,9 @@ bool aligned16(const void *a, const void *b, const void *c) {
 
 using namespace gnnagg;
 
-extern "C" int gnnagg_bias_relu_dropout_f32(const float *z, const float *bias, const uint8_t *keep, float scale,
-                                            float *y, int64_t rows, int64_t feat, void *stream) {
+extern "C" int gnnagg_bias_relu_dropout_f32(const float *z, const float *bias, const uint8_t *keep,
+                                            const float *row_div, float scale, float *y, int64_t rows, int64_t feat,
+                                            void *stream) {
     GNNAGG_REQUIRE(rows >= 0 && feat >= 0, "negative size");
     if (rows == 0 || feat == 0) return GNNAGG_OK;
     GNNAGG_REQUIRE(z && bias && y, "null z/bias/y");
@@ -95,29 +155,53 @@ extern "C" int gnnagg_bias_relu_dropout_f32(const float *z, const float *bias, c
     if (feat % 4 == 0 && aligned16(z, bias, y) && (reinterpret_cast<uintptr_t>(keep) & 3) == 0) {
         hipLaunchKernelGGL(bias_relu_dropout_v4_kernel, dim3(stream_grid(n / 4)), dim3(256), 0, st,
                            reinterpret_cast<const f4 *>(z), reinterpret_cast<const f4 *>(bias),
-                           reinterpret_cast<const u8x4 *>(keep), scale, reinterpret_cast<f4 *>(y), n / 4,
+                           reinterpret_cast<const u8x4 *>(keep), row_div, scale, reinterpret_cast<f4 *>(y), n / 4,
                            (int)(feat / 4));
     } else {
-        hipLaunchKernelGGL(bias_relu_dropout_kernel, dim3(stream_grid(n)), dim3(256), 0, st, z, bias, keep, scale, y, n,
-                           (int)feat);
+        hipLaunchKernelGGL(bias_relu_dropout_kernel, dim3(stream_grid(n)), dim3(256), 0, st, z, bias, keep, row_div,
+                           scale, y, n, (int)feat);
     }
     GNNAGG_HIP(hipGetLastError());
     return GNNAGG_OK;
 }
 
-extern "C" int gnnagg_relu_dropout_backward_f32(const float *grad_y, const float *y, float scale, float *grad_z,
-                                                int64_t count, void *stream) {
-    GNNAGG_REQUIRE(count >= 0, "negative size");
-    if (count == 0) return GNNAGG_OK;
+extern "C" int gnnagg_relu_dropout_backward_blocks(int64_t rows, int64_t feat) {
+    if (rows <= 0 || feat <= 0 || feat % 4 != 0 || feat / 4 > 256 || 256 % (feat / 4) != 0) return 0;
+    const int64_t target = 256 * 16;  // blocks: enough to fill the chip, few enough to sum cheaply
+    const int64_t rpb = (rows + target - 1) / target;
+    return (int)((rows + rpb - 1) / rpb);
+}
+
+extern "C" int gnnagg_relu_dropout_backward_f32(const float *grad_y, const float *y, const float *row_div, float scale,
+                                                float *grad_z, float *bias_partial, int64_t rows, int64_t feat,
+                                                void *stream) {
+    GNNAGG_REQUIRE(rows >= 0 && feat >= 0, "negative size");
+    if (rows == 0 || feat == 0) return GNNAGG_OK;
     GNNAGG_REQUIRE(grad_y && y && grad_z, "null grad_y/y/grad_z");
+    if (feat > (1 << 20)) return fail(GNNAGG_ERR_UNSUPPORTED, "feature width %lld above 2^20", (long long)feat);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (count % 4 == 0 && aligned16(grad_y, y, grad_z)) {
+    const int64_t count = rows * feat;
+    if (bias_partial) {
+        const int blocks = gnnagg_relu_dropout_backward_blocks(rows, feat);
+        GNNAGG_REQUIRE(blocks > 0, "bias partial sums need feat %% 4 == 0 and 256 %% (feat / 4) == 0 (feat=%lld)",
+                       (long long)feat);
+        GNNAGG_REQUIRE(aligned16(grad_y, y, grad_z) && (reinterpret_cast<uintptr_t>(bias_partial) & 15) == 0,
+                       "bias partial sums need 16-byte aligned operands");
+        const int64_t rpb = (rows + blocks - 1) / blocks;
+        hipLaunchKernelGGL(relu_dropout_backward_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, st,
+                           reinterpret_cast<const f4 *>(grad_y), reinterpret_cast<const f4 *>(y), row_div, scale,
+                           reinterpret_cast<f4 *>(grad_z), reinterpret_cast<f4 *>(bias_partial), rows, (int)(feat / 4),
+                           (int)rpb);
+        GNNAGG_HIP(hipGetLastError());
+        return GNNAGG_OK;
+    }
+    if (feat % 4 == 0 && aligned16(grad_y, y, grad_z)) {
         hipLaunchKernelGGL(relu_dropout_backward_v4_kernel, dim3(stream_grid(count / 4)), dim3(256), 0, st,
-                           reinterpret_cast<const f4 *>(grad_y), reinterpret_cast<const f4 *>(y), scale,
-                           reinterpret_cast<f4 *>(grad_z), count / 4);
+                           reinterpret_cast<const f4 *>(grad_y), reinterpret_cast<const f4 *>(y), row_div, scale,
+                           reinterpret_cast<f4 *>(grad_z), count / 4, (int)(feat / 4));
     } else {
-        hipLaunchKernelGGL(relu_dropout_backward_kernel, dim3(stream_grid(count)), dim3(256), 0, st, grad_y, y, scale,
-                           grad_z, count);
+        hipLaunchKernelGGL(relu_dropout_backward_kernel, dim3(stream_grid(count)), dim3(256), 0, st, grad_y, y, row_div,
+                           scale, grad_z, count, (int)feat);
     }
     GNNAGG_HIP(hipGetLastError());
     return GNNAGG_OK;

@@ -4,8 +4,9 @@ The aggregation is the reference's ``Aggregator`` contract (aggregate-then-trans
 order of self_benchmark/a64fx/model/layers/sageconv.py:65-93: ``out = Aggregator(...)``,
 ``out /= graph.in_degrees``, then the dense transform).  Everything after the
 aggregation is this build's own definition of the workload: one weight matrix per layer
-(``Z = (A X / deg) W + b``), ReLU, dropout with a precomputed seeded mask, log-softmax +
-NLL on the labelled nodes, Adam.  The dense products run on the matrix cores through
+(``Z = ((A X) W) / deg + b`` -- the degree normalisation is applied behind the dense
+product, where it fuses into the epilogue: D^-1 (A X) W == D^-1 ((A X) W)), ReLU, dropout
+with a precomputed seeded mask, log-softmax + NLL on the labelled nodes, Adam.  The dense products run on the matrix cores through
 the BLAS library behind ``torch.mm`` (fp32, or bf16 inputs with fp32 accumulation and
 fp32 output); they are plain library GEMMs, not part of libgnnagg.
 """
@@ -40,11 +41,11 @@ class _Bf16InputLinear(torch.autograd.Function):
 
 
 class _BiasReluDropout(torch.autograd.Function):
-    """y = relu(z + bias) * (keep ? scale : 0), one fused pass, written over ``z`` (the GEMM
-    output, which nothing else reads); the gradient needs only ``y``."""
+    """y = relu(z / row_div + bias) * (keep ? scale : 0), one fused pass, written over ``z``
+    (the GEMM output, which nothing else reads); the gradient needs only ``y``."""
 
     @staticmethod
-    def forward(ctx, z, bias, keep, scale):
+    def forward(ctx, z, bias, keep, scale, row_div):
         if not z.is_cuda:
             raise RuntimeError("the fused epilogue runs on a GPU (HIP) device only")
         if z.dtype != torch.float32 or bias.dtype != torch.float32 or not z.is_contiguous() or z.dim() != 2:
@@ -52,13 +53,17 @@ class _BiasReluDropout(torch.autograd.Function):
         if keep is not None and (keep.dtype not in (torch.bool, torch.uint8) or keep.shape != z.shape
                                  or not keep.is_contiguous()):
             raise RuntimeError("Input mismatch: keep must be a contiguous bool/uint8 mask shaped like z")
+        if row_div is not None and (row_div.dtype != torch.float32 or row_div.numel() != z.size(0)
+                                    or not row_div.is_contiguous()):
+            raise RuntimeError("Input mismatch: row_div must be contiguous float32 with one entry per row")
         with torch.cuda.device(z.device):
             _lib.check(_lib.lib().gnnagg_bias_relu_dropout_f32(
-                _lib.ptr(z), _lib.ptr(bias.contiguous()), _lib.ptr(keep), float(scale), _lib.ptr(z), z.size(0),
-                z.size(1), _lib.current_stream(z.device)))
+                _lib.ptr(z), _lib.ptr(bias.contiguous()), _lib.ptr(keep), _lib.ptr(row_div), float(scale), _lib.ptr(z),
+                z.size(0), z.size(1), _lib.current_stream(z.device)))
         ctx.mark_dirty(z)
         ctx.save_for_backward(z)
         ctx.scale = float(scale)
+        ctx.row_div = row_div
         return z
 
     @staticmethod
@@ -66,12 +71,25 @@ class _BiasReluDropout(torch.autograd.Function):
         (y,) = ctx.saved_tensors
         grad_y = grad_y.contiguous()
         grad_z = torch.empty_like(grad_y)
+        row_div = ctx.row_div
+        L = _lib.lib()
+        # d/d bias sums the gradient BEFORE the per-row division; where the width allows, the
+        # kernel emits per-block partial sums of exactly that in the same pass
+        blocks = int(L.gnnagg_relu_dropout_backward_blocks(y.size(0), y.size(1))) if ctx.needs_input_grad[1] else 0
+        partial = torch.empty(blocks, y.size(1), dtype=torch.float32, device=y.device) if blocks else None
         with torch.cuda.device(y.device):
-            _lib.check(_lib.lib().gnnagg_relu_dropout_backward_f32(
-                _lib.ptr(grad_y), _lib.ptr(y), ctx.scale, _lib.ptr(grad_z), grad_y.numel(),
-                _lib.current_stream(y.device)))
-        grad_bias = grad_z.sum(dim=0) if ctx.needs_input_grad[1] else None
-        return grad_z, grad_bias, None, None
+            _lib.check(L.gnnagg_relu_dropout_backward_f32(
+                _lib.ptr(grad_y), _lib.ptr(y), _lib.ptr(row_div), ctx.scale, _lib.ptr(grad_z), _lib.ptr(partial),
+                y.size(0), y.size(1), _lib.current_stream(y.device)))
+        grad_bias = None
+        if ctx.needs_input_grad[1]:
+            if partial is not None:
+                grad_bias = partial.sum(dim=0)
+            elif row_div is None:
+                grad_bias = grad_z.sum(dim=0)
+            else:
+                grad_bias = (grad_z * row_div.view(-1, 1)).sum(dim=0)
+        return grad_z, grad_bias, None, None, None
 
 
 class GCNLayer(torch.nn.Module):
@@ -85,15 +103,15 @@ class GCNLayer(torch.nn.Module):
         torch.nn.init.xavier_uniform_(self.weight, gain=torch.nn.init.calculate_gain("relu"))
 
     def transform(self, graph, x: torch.Tensor, layer: int, is_pre_delay: bool) -> torch.Tensor:
-        """(A x / deg) W, without the bias."""
+        """(A x) W: neither the degree normalisation nor the bias yet."""
         agg = Aggregator.apply(graph, x, layer, 32, is_pre_delay, self.training)
-        agg = agg / graph.in_degrees
         if self.gemm == "bf16":
             return _Bf16InputLinear.apply(agg, self.weight)
         return torch.mm(agg, self.weight)
 
     def forward(self, graph, x: torch.Tensor, layer: int, is_pre_delay: bool) -> torch.Tensor:
-        return self.transform(graph, x, layer, is_pre_delay) + self.bias
+        """((A x) W) / deg + bias."""
+        return torch.addcdiv(self.bias, self.transform(graph, x, layer, is_pre_delay), graph.in_degrees)
 
 
 class GCN(torch.nn.Module):
@@ -115,9 +133,9 @@ class GCN(torch.nn.Module):
             if self.training and self.dropout > 0.0:
                 if masks is None:
                     raise ValueError("training needs the seeded dropout masks")
-                h = _BiasReluDropout.apply(z, layer.bias, masks[l], 1.0 / (1.0 - self.dropout))
+                h = _BiasReluDropout.apply(z, layer.bias, masks[l], 1.0 / (1.0 - self.dropout), graph.in_degrees)
             else:
-                h = _BiasReluDropout.apply(z, layer.bias, None, 1.0)
+                h = _BiasReluDropout.apply(z, layer.bias, None, 1.0, graph.in_degrees)
         return F.log_softmax(h, dim=1)
 
 

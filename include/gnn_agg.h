@@ -144,17 +144,25 @@ int gnnagg_gather_rows_f32(const float *src, const int64_t *index, float *out, i
 
 /* ---------------------------------------------------------------------------------
  * Fused layer epilogue around the aggregation path (the full train-step workload):
- *   y[i,f] = relu(z[i,f] + bias[f]) * (keep[i,f] ? scale : 0)          forward
- *   grad_z = y > 0 ? grad_y * scale : 0                                 backward
- * z, y fp32 [rows, feat] (y may alias z), bias fp32 [feat], keep uint8 [rows, feat] or
- * NULL (no dropout; pass scale = 1), grad_* fp32 [count] (grad_z may alias grad_y).
- * The reference runs its epilogue (dropout, LayerNorm, ReLU) as separate torch ops
- * (model/DistSAGE.py:55-66); this fused form belongs to this build's GCN layer stack.
+ *   y[i,f]  = relu(z[i,f] / row_div[i] + bias[f]) * (keep[i,f] ? scale : 0)     forward
+ *   grad_z  = (y > 0 ? grad_y * scale : 0) / row_div[i]                          backward
+ *   bias_partial[b, f] = sum over the rows of block b of (y > 0 ? grad_y * scale : 0)
+ * z, y, grad_* fp32 [rows, feat] (y may alias z, grad_z may alias grad_y), bias fp32
+ * [feat], keep uint8 [rows, feat] or NULL (no dropout; pass scale = 1), row_div fp32 [rows]
+ * or NULL (no division).  bias_partial is NULL, or fp32 [blocks, feat] with blocks =
+ * gnnagg_relu_dropout_backward_blocks(rows, feat) (0 = this width cannot use it: needs
+ * feat % 4 == 0 and 256 % (feat / 4) == 0); summing it over its first axis gives the bias
+ * gradient without another pass over the activations (fixed order: deterministic).
+ * row_div carries the reference layer's `out /= graph.in_degrees`
+ * (model/layers/sageconv.py:84) moved behind the dense product, where it costs no pass of
+ * its own.  The reference runs its epilogue (dropout, LayerNorm, ReLU) as separate torch
+ * ops (model/DistSAGE.py:55-66); this fused form belongs to this build's GCN layer stack.
  * ------------------------------------------------------------------------------- */
-int gnnagg_bias_relu_dropout_f32(const float *z, const float *bias, const uint8_t *keep, float scale, float *y,
-                                 int64_t rows, int64_t feat, void *stream);
-int gnnagg_relu_dropout_backward_f32(const float *grad_y, const float *y, float scale, float *grad_z, int64_t count,
-                                     void *stream);
+int gnnagg_bias_relu_dropout_f32(const float *z, const float *bias, const uint8_t *keep, const float *row_div,
+                                 float scale, float *y, int64_t rows, int64_t feat, void *stream);
+int gnnagg_relu_dropout_backward_blocks(int64_t rows, int64_t feat);
+int gnnagg_relu_dropout_backward_f32(const float *grad_y, const float *y, const float *row_div, float scale,
+                                     float *grad_z, float *bias_partial, int64_t rows, int64_t feat, void *stream);
 
 #ifdef __cplusplus
 }

@@ -97,8 +97,8 @@ def test_train_step_matches_cpu_autograd(gemm, tol):
     for l, layer in enumerate(cpu_model.layers):
         # layer 0's input needs no gradient, so its backward exchange never happens
         incoming = ex.rows.get(f"backward{l}", torch.zeros(a_to.shape[0], dims[l]))
-        agg = CpuAggregate.apply(h, a_local, a_from, a_to, ex.rows[f"forward{l}"], incoming) / deg
-        z = (CpuBf16Linear.apply(agg, layer.weight) if gemm == "bf16" else agg @ layer.weight) + layer.bias
+        agg = CpuAggregate.apply(h, a_local, a_from, a_to, ex.rows[f"forward{l}"], incoming)
+        z = (CpuBf16Linear.apply(agg, layer.weight) if gemm == "bf16" else agg @ layer.weight) / deg + layer.bias
         h = z if l == len(dims) - 2 else torch.relu(z) * masks[l].cpu() * 2.0
     cpu_loss = F.nll_loss(F.log_softmax(h, dim=1)[train_idx.cpu()], labels.cpu()[train_idx.cpu()])
     cpu_loss.backward()
@@ -119,25 +119,27 @@ def test_train_step_matches_cpu_autograd(gemm, tol):
 
 @pytest.mark.parametrize("rows,feat", [(1000, 256), (333, 47), (64, 4), (1, 1)])
 @pytest.mark.parametrize("with_mask", [True, False])
-def test_fused_epilogue_equals_separate_ops(rows, feat, with_mask):
+@pytest.mark.parametrize("with_div", [True, False])
+def test_fused_epilogue_equals_separate_ops(rows, feat, with_mask, with_div):
     gen = torch.Generator(device="cuda").manual_seed(rows + feat)
     z = torch.randn(rows, feat, device="cuda", generator=gen)
     bias = torch.randn(feat, device="cuda", generator=gen)
+    div = (torch.randint(1, 9, (rows, 1), device="cuda", generator=gen).float()) if with_div else None
     keep = (torch.rand(rows, feat, device="cuda", generator=gen) >= 0.5) if with_mask else None
     scale = 2.0 if with_mask else 1.0
     g = torch.randn(rows, feat, device="cuda", generator=gen)
 
     z_ref = z.clone().requires_grad_()
     b_ref = bias.clone().requires_grad_()
-    y_ref = torch.relu(z_ref + b_ref)
+    y_ref = torch.relu((z_ref / div if with_div else z_ref) + b_ref)
     if with_mask:
         y_ref = y_ref * keep * scale
     y_ref.backward(g)
 
     z_in = z.clone().requires_grad_()
     b_in = bias.clone().requires_grad_()
-    y = gcn._BiasReluDropout.apply(z_in * 1.0, b_in, keep, scale)  # * 1.0: a non-leaf the op may overwrite
+    y = gcn._BiasReluDropout.apply(z_in * 1.0, b_in, keep, scale, div)  # * 1.0: a non-leaf the op may overwrite
     y.backward(g)
     assert torch.equal(y.detach(), y_ref.detach())
-    assert torch.equal(z_in.grad, z_ref.grad)
+    assert torch.allclose(z_in.grad, z_ref.grad, rtol=2e-7, atol=0)  # (g*scale)/d vs g*(scale/d): last-bit rounding
     assert torch.allclose(b_in.grad, b_ref.grad, rtol=1e-5, atol=1e-5)  # column sums in another order
