@@ -25,6 +25,7 @@ Pinning status (what fixes each function's answers independently of this file):
         (tests/test_data_preprocessor.py:29-40) and it needs a process group:
         PARITY UNPINNED beyond its closed form (ids requested by rank r, minus the
         local begin) and the all-ranks invariant in tests/test_pipeline_invariant.py
+  divide_edges_into_local_and_remote ...... tests/test_postprocess_graph_data.py:10-40 (3 vectors)
   simulate_* helpers ...................... no reference counterpart: they replace the
         setup-time all_to_all calls (DataProcessor.py:76-98, :329-382) by moving the
         lists between simulated ranks in one process
@@ -302,3 +303,22 @@ def simulate_halo_id_exchange(remote_nodes_list_per_rank, ranges_per_rank):
     world = len(remote_nodes_list_per_rank)
     return [[np.asarray(remote_nodes_list_per_rank[i][int(ranges_per_rank[i][r]):int(ranges_per_rank[i][r + 1])],
                         dtype=I64) for i in range(world)] for r in range(world)]
+
+
+# ------------------------------------------------- file contract on the input side
+def divide_edges_into_local_and_remote(edges_list, node_idx_begin, node_idx_end):
+    """graph_partition_scripts/postprocess_graph_multi_proc.py:10-44: edges [E,2] of global
+    (src, dst) whose dst lies in [begin, end] (end inclusive); local edges have both ids
+    localised, remote edges keep the global src.  Pinned by
+    tests/test_postprocess_graph_data.py:10-40 (3 vectors)."""
+    local_s, local_d, remote_s, remote_d = [], [], [], []
+    for s, d in np.asarray(edges_list, dtype=I64).reshape(-1, 2):
+        assert node_idx_begin <= d <= node_idx_end
+        if node_idx_begin <= s <= node_idx_end:
+            local_s.append(s - node_idx_begin)
+            local_d.append(d - node_idx_begin)
+        else:
+            remote_s.append(s)
+            remote_d.append(d - node_idx_begin)
+    return (np.asarray([local_s, local_d], dtype=I64).reshape(2, -1),
+            np.asarray([remote_s, remote_d], dtype=I64).reshape(2, -1))

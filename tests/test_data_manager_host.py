@@ -290,3 +290,41 @@ def test_synthetic_partition_maps_equal_oracle_on_host():
             rowptr, col, val = [t.numpy() for t in m.csr()]
             assert tuple(m.sparse_sizes()) == tuple(o[3])
             assert np.array_equal(rowptr, o[0]) and np.array_equal(col, o[1]) and np.array_equal(val, o[2])
+
+
+# ------------------------------------------------------------------ input-side file contract
+def test_divide_edges_into_local_and_remote(golden):
+    from gnn_benchmark_amd.data_manager import divide_edges_into_local_and_remote
+
+    for c in golden["divide_edges_into_local_and_remote"]:
+        local, remote = divide_edges_into_local_and_remote(T(c["edges"]).t(), c["begin"], c["end"])
+        assert torch.equal(local, T(c["expected_local"]).reshape(2, -1)), c["source"]
+        assert torch.equal(remote, T(c["expected_remote"]).reshape(2, -1)), c["source"]
+    rng = np.random.default_rng(0)
+    edges = np.stack((rng.integers(0, 90, 500), rng.integers(30, 61, 500)), axis=1).astype(np.int64)
+    o_local, o_remote = om.divide_edges_into_local_and_remote(edges, 30, 60)
+    local, remote = divide_edges_into_local_and_remote(torch.from_numpy(edges), 30, 60)
+    assert np.array_equal(local.numpy(), o_local) and np.array_equal(remote.numpy(), o_remote)
+    with pytest.raises(AssertionError):
+        divide_edges_into_local_and_remote(torch.tensor([[0, 99]]), 30, 60)
+
+
+def test_partition_files_round_trip(tmp_path):
+    """A synthetic partition written in the reference's file layout and read back through
+    load_graph_structures feeds the builders unchanged."""
+    from gnn_benchmark_amd import synthetic
+    from gnn_benchmark_amd.data_manager import (get_distributed_graph_for_pre_aggressive, load_graph_structures,
+                                                save_partition_files)
+
+    part = synthetic.partition_edges(1500, 3, 1, 4, 1.8, 200, 300, 1500, seed=5, device="cpu")
+    save_partition_files(str(tmp_path), "toy", part.rank, part.begins, part.local_edges, part.remote_edges)
+    nodes, local, remote, begins, n = load_graph_structures(str(tmp_path), "toy", part.rank)
+    assert n == 1500 and nodes.shape == (1500, 2) and int(nodes[0][0]) == int(part.begins[part.rank])
+    assert torch.equal(local, part.local_edges) and torch.equal(remote, part.remote_edges)
+    assert torch.equal(begins, part.begins)
+    a = get_distributed_graph_for_pre_aggressive(local, remote, begins, n, 8, part.rank, 3, 32,
+                                                 graph_exchange=synthetic.mirrored_graph_exchange(part))
+    b = synthetic.build_partition_graph(part, 8, True, device="cpu")
+    for m1, m2 in ((a.local_adj_t, b.local_adj_t), (a.adj_t_pre_post_aggr_from, b.adj_t_pre_post_aggr_from),
+                   (a.adj_t_pre_post_aggr_to, b.adj_t_pre_post_aggr_to)):
+        assert all(torch.equal(x, y) for x, y in zip(m1.csr(), m2.csr()))

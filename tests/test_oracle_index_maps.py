@@ -128,3 +128,10 @@ def test_remap_remote_nodes_id(golden):
         nodes = A(c["nodes"]).copy()
         assert om.remap_remote_nodes_id(nodes, A(c["begins"])) == c["expected_count"], c["source"]
         assert np.array_equal(nodes, A(c["expected_nodes"])), c["source"]
+
+
+def test_divide_edges_into_local_and_remote(golden):
+    for c in golden["divide_edges_into_local_and_remote"]:
+        local, remote = om.divide_edges_into_local_and_remote(A(c["edges"]).T, c["begin"], c["end"])
+        assert np.array_equal(local, A(c["expected_local"]).reshape(2, -1)), c["source"]
+        assert np.array_equal(remote, A(c["expected_remote"]).reshape(2, -1)), c["source"]
