@@ -62,3 +62,11 @@ def test_product_refuses_cpu_tensors():
     with pytest.raises(RuntimeError, match="GPU"):
         SPMM_forward(src, x, out)
     assert torch.equal(out, torch.zeros(2, 4))
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    """No fallback: with the shared library absent the binding raises, naming the file."""
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libgnnagg.so"))
+    with pytest.raises(RuntimeError, match="libgnnagg.so is missing"):
+        _lib.lib()
