@@ -30,6 +30,8 @@ EXPORTS = (
     "gnnagg_bias_relu_dropout_f32",
     "gnnagg_relu_dropout_backward_blocks",
     "gnnagg_relu_dropout_backward_f32",
+    "gnnagg_wgrad_workspace_bytes",
+    "gnnagg_wgrad_f32",
 )
 
 _lib = None
@@ -90,6 +92,10 @@ def lib() -> ctypes.CDLL:
     L.gnnagg_relu_dropout_backward_f32.argtypes = [vp, vp, vp, ctypes.c_float, vp, vp, i64, i64, vp]
     L.gnnagg_relu_dropout_backward_blocks.restype = i32
     L.gnnagg_relu_dropout_backward_blocks.argtypes = [i64, i64]
+    L.gnnagg_wgrad_workspace_bytes.restype = i64
+    L.gnnagg_wgrad_workspace_bytes.argtypes = [i64, i64, i64]
+    L.gnnagg_wgrad_f32.restype = i32
+    L.gnnagg_wgrad_f32.argtypes = [vp, vp, vp, vp, i64, i64, i64, vp]
     if L.gnnagg_abi_version() != ABI_VERSION:
         raise RuntimeError("libgnnagg.so was built from a different include/gnn_agg.h; rebuild it")
     _lib = L

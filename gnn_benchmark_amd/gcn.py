@@ -6,9 +6,11 @@ order of self_benchmark/a64fx/model/layers/sageconv.py:65-93: ``out = Aggregator
 aggregation is this build's own definition of the workload: one weight matrix per layer
 (``Z = ((A X) W) / deg + b`` -- the degree normalisation is applied behind the dense
 product, where it fuses into the epilogue: D^-1 (A X) W == D^-1 ((A X) W)), ReLU, dropout
-with a precomputed seeded mask, log-softmax + NLL on the labelled nodes, Adam.  The dense products run on the matrix cores through
-the BLAS library behind ``torch.mm`` (fp32, or bf16 inputs with fp32 accumulation and
-fp32 output); they are plain library GEMMs, not part of libgnnagg.
+with a precomputed seeded mask, log-softmax + NLL on the labelled nodes, Adam.  The
+forward and input-gradient products run on the matrix cores through the BLAS library
+behind ``torch.mm`` (fp32, or bf16 inputs with fp32 accumulation and fp32 output); the
+weight gradient -- a reduction over millions of rows into at most 256 x 256 outputs, the
+library's weakest shape -- runs in libgnnagg's own fp32 MFMA kernel.
 """
 from typing import List, Optional, Sequence
 
@@ -20,8 +22,10 @@ from .aggregator import Aggregator
 
 
 class _Bf16InputLinear(torch.autograd.Function):
-    """y = x @ w with x, w rounded to bf16, products accumulated in fp32, fp32 result;
-    the two gradient products are computed the same way."""
+    """y = x @ w with x, w rounded to bf16, products accumulated in fp32, fp32 result; the
+    input gradient is computed the same way.  The weight gradient stays in fp32: the
+    hand-written kernel reads the fp32 operands as they are, which is faster than rounding
+    7 M-row operands to bf16 for the library's product, and more exact."""
 
     @staticmethod
     def _mm(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
@@ -36,7 +40,41 @@ class _Bf16InputLinear(torch.autograd.Function):
     def backward(ctx, g):
         x, w = ctx.saved_tensors
         gx = _Bf16InputLinear._mm(g, w.t()) if ctx.needs_input_grad[0] else None
-        gw = _Bf16InputLinear._mm(x.t(), g) if ctx.needs_input_grad[1] else None
+        gw = weight_gradient(x, g) if ctx.needs_input_grad[1] else None
+        return gx, gw
+
+
+def weight_gradient(x: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
+    """x^T @ g for tall-skinny fp32 operands through the library's MFMA kernel; falls back to
+    the BLAS library for shapes that kernel does not take (more than 256 columns)."""
+    x, g = x.contiguous(), g.contiguous()
+    rows, fi, fo = x.size(0), x.size(1), g.size(1)
+    L = _lib.lib()
+    nbytes = int(L.gnnagg_wgrad_workspace_bytes(rows, fi, fo)) if x.is_cuda and x.dtype == torch.float32 else 0
+    if nbytes == 0:
+        return torch.mm(x.t(), g)
+    out = torch.empty(fi, fo, dtype=torch.float32, device=x.device)
+    workspace = torch.empty(nbytes // 4, dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        _lib.check(L.gnnagg_wgrad_f32(_lib.ptr(x), _lib.ptr(g), _lib.ptr(out), _lib.ptr(workspace), rows, fi, fo,
+                                      _lib.current_stream(x.device)))
+    return out
+
+
+class _Fp32Linear(torch.autograd.Function):
+    """y = x @ w in fp32; the weight gradient (a reduction over millions of rows) runs in
+    the hand-written MFMA kernel, the two other products in the BLAS library."""
+
+    @staticmethod
+    def forward(ctx, x, w):
+        ctx.save_for_backward(x, w)
+        return torch.mm(x, w)
+
+    @staticmethod
+    def backward(ctx, g):
+        x, w = ctx.saved_tensors
+        gx = torch.mm(g, w.t()) if ctx.needs_input_grad[0] else None
+        gw = weight_gradient(x, g) if ctx.needs_input_grad[1] else None
         return gx, gw
 
 
@@ -107,7 +145,7 @@ class GCNLayer(torch.nn.Module):
         agg = Aggregator.apply(graph, x, layer, 32, is_pre_delay, self.training)
         if self.gemm == "bf16":
             return _Bf16InputLinear.apply(agg, self.weight)
-        return torch.mm(agg, self.weight)
+        return _Fp32Linear.apply(agg, self.weight)
 
     def forward(self, graph, x: torch.Tensor, layer: int, is_pre_delay: bool) -> torch.Tensor:
         """((A x) W) / deg + bias."""

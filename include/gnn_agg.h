@@ -164,6 +164,19 @@ int gnnagg_relu_dropout_backward_blocks(int64_t rows, int64_t feat);
 int gnnagg_relu_dropout_backward_f32(const float *grad_y, const float *y, const float *row_div, float scale,
                                      float *grad_z, float *bias_partial, int64_t rows, int64_t feat, void *stream);
 
+/* ---------------------------------------------------------------------------------
+ * Weight gradient of a dense layer, w_grad[fi, fo] = x^T @ g, with x fp32 [rows, fi] and
+ * g fp32 [rows, fo] row-major, rows in the millions, fi, fo <= 256 (GNNAGG_ERR_UNSUPPORTED
+ * otherwise).  Hand-written fp32 MFMA kernel plus a fixed-order reduction of per-slice
+ * partial results: deterministic.  `workspace` is caller-provided device memory of
+ * gnnagg_wgrad_workspace_bytes(rows, fi, fo) bytes (0 = unsupported shape); nothing is
+ * allocated here.  Part of this build's GCN layer stack (the reference leaves this product
+ * to torch's Linear backward, model/layers/sageconv.py:87-88).
+ * ------------------------------------------------------------------------------- */
+int64_t gnnagg_wgrad_workspace_bytes(int64_t rows, int64_t fi, int64_t fo);
+int gnnagg_wgrad_f32(const float *x, const float *g, float *w_grad, void *workspace, int64_t rows, int64_t fi,
+                     int64_t fo, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -143,3 +143,21 @@ def test_fused_epilogue_equals_separate_ops(rows, feat, with_mask, with_div):
     assert torch.equal(y.detach(), y_ref.detach())
     assert torch.allclose(z_in.grad, z_ref.grad, rtol=2e-7, atol=0)  # (g*scale)/d vs g*(scale/d): last-bit rounding
     assert torch.allclose(b_in.grad, b_ref.grad, rtol=1e-5, atol=1e-5)  # column sums in another order
+
+
+@pytest.mark.parametrize("rows,fi,fo", [(100_003, 256, 256), (65_536, 128, 256), (70_001, 256, 172), (999, 40, 47),
+                                        (7, 1, 1), (128, 64, 64), (1, 256, 256), (513, 33, 250)])
+def test_weight_gradient_kernel_matches_fp64(rows, fi, fo):
+    """The hand-written MFMA product x^T @ g against an fp64 product: the error must stay
+    within what fp32 accumulation over `rows` terms allows, and equal runs give equal bits."""
+    gen = torch.Generator(device="cuda").manual_seed(rows + fi + fo)
+    x = torch.randn(rows, fi, device="cuda", generator=gen)
+    g = torch.randn(rows, fo, device="cuda", generator=gen)
+    got = gcn.weight_gradient(x, g)
+    want = x.double().t() @ g.double()
+    bound = 4e-7 * (x.double().abs().t() @ g.double().abs())  # |error| <= c * eps * sum |x||g|
+    assert got.shape == (fi, fo)
+    assert bool(((got.double() - want).abs() <= bound + 1e-6).all()), float((got.double() - want).abs().max())
+    assert torch.equal(got, gcn.weight_gradient(x, g))
+    blas = x.t() @ g
+    assert torch.allclose(got, blas, rtol=1e-4, atol=1e-3 * float(rows) ** 0.5)
