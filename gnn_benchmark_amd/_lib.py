@@ -32,6 +32,10 @@ EXPORTS = (
     "gnnagg_relu_dropout_backward_f32",
     "gnnagg_wgrad_workspace_bytes",
     "gnnagg_wgrad_f32",
+    "gnnagg_quantize_segments_f32",
+    "gnnagg_dequantize_segments_f32",
+    "gnnagg_quantize_mixed_f32",
+    "gnnagg_dequantize_mixed_f32",
 )
 
 _lib = None
@@ -96,6 +100,14 @@ def lib() -> ctypes.CDLL:
     L.gnnagg_wgrad_workspace_bytes.argtypes = [i64, i64, i64]
     L.gnnagg_wgrad_f32.restype = i32
     L.gnnagg_wgrad_f32.argtypes = [vp, vp, vp, vp, i64, i64, i64, vp]
+    L.gnnagg_quantize_segments_f32.restype = i32
+    L.gnnagg_quantize_segments_f32.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp]
+    L.gnnagg_dequantize_segments_f32.restype = i32
+    L.gnnagg_dequantize_segments_f32.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp]
+    L.gnnagg_quantize_mixed_f32.restype = i32
+    L.gnnagg_quantize_mixed_f32.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp]
+    L.gnnagg_dequantize_mixed_f32.restype = i32
+    L.gnnagg_dequantize_mixed_f32.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp]
     if L.gnnagg_abi_version() != ABI_VERSION:
         raise RuntimeError("libgnnagg.so was built from a different include/gnn_agg.h; rebuild it")
     _lib = L

@@ -1,9 +1,13 @@
-"""Drop-in for the reference's native module ``computation_ops`` (only ``spmm``; the
-quantisation ops of that module serve the MPI exchange, which this build leaves out).
+"""Drop-in for the reference's native module ``computation_ops``.
 
-Reference: self_benchmark/a64fx/model/ops/src/spmm.h:3-6, spmm.cpp:327-507, bound at
+``spmm``: self_benchmark/a64fx/model/ops/src/spmm.h:3-6, spmm.cpp:327-507, bound at
 ops.cpp:23.  Same name, positional order, dtypes and ``(out, None)`` return; ``out`` is
 accumulated into in place and returned as the same tensor.
+
+Boundary-buffer codec (ops.cpp:12-18): ``quantize_tensor`` / ``dequantize_tensor`` and
+``*_for_all_procs`` with the signatures of the SVE build (quantization_arm.h:5-8, the one
+the reference's Python calls, quantizer.py:17, :44, :83-90), ``quantize_tensor_v1`` /
+``dequantize_tensor_v1`` (quantization_x86.h:7-8).  All operands are GPU tensors.
 """
 from typing import Optional, Tuple
 
@@ -65,3 +69,146 @@ def spmm(rowptr: torch.Tensor, col: torch.Tensor, value: Optional[torch.Tensor],
         _lib.check(_lib.lib().gnnagg_spmm_csr_f32(_lib.ptr(rowptr), _lib.ptr(col), _lib.ptr(value), _lib.ptr(mat),
                                                   _lib.ptr(out), sparse_rows, mat.size(1), _lib.current_stream(dev)))
     return out, None
+
+
+# ---------------------------------------------------------------- boundary-buffer codec
+
+_PACKED_RANGE_CACHE = {}
+
+
+def _packed_range(work_range_per_proc: torch.Tensor, bits: int, device) -> Tuple[torch.Tensor, torch.Tensor, int]:
+    """Device copies of the per-rank row prefix and of the packed-row prefix derived from it
+    (divide_work_v1, quantization_arm.cpp:21-31), cached per range tensor.  The cache entry
+    keeps the range tensor alive, so its address cannot be handed to another tensor while the
+    entry exists; an in-place change bumps ``_version``."""
+    key = (work_range_per_proc.data_ptr(), work_range_per_proc._version, int(work_range_per_proc.numel()), bits,
+           str(device))
+    hit = _PACKED_RANGE_CACHE.get(key)
+    if hit is None:
+        host = work_range_per_proc.detach().to("cpu", torch.int64)
+        _require(host.dim() == 1 and host.numel() >= 2, "work range must hold num_procs + 1 entries")
+        _require(bool((host[1:] >= host[:-1]).all()) and int(host[0]) == 0, "work range must be a prefix sum from 0")
+        epb = 8 // bits
+        packed = torch.zeros_like(host)
+        packed[1:] = torch.cumsum((host[1:] - host[:-1] + epb - 1) // epb, 0)
+        hit = (host.to(device, torch.int32), packed.to(device, torch.int32), int(packed[-1]), int(host[-1]),
+               work_range_per_proc)
+        if len(_PACKED_RANGE_CACHE) > 64:
+            _PACKED_RANGE_CACHE.clear()
+        _PACKED_RANGE_CACHE[key] = hit
+    return hit[:4]
+
+
+def _check_codec_operands(data_fp32, data_int8, params, bits, params_cols):
+    _require(bits in (2, 4, 8), "bits must be 2, 4 or 8")
+    _require_hip(data_fp32, "fp32 buffer")
+    dev = data_fp32.device
+    _require_hip(data_int8, "packed buffer", dev)
+    _require_hip(params, "quantisation parameters", dev)
+    _require(data_fp32.dtype == torch.float32 and data_fp32.dim() == 2 and data_fp32.is_contiguous(),
+             "fp32 buffer must be contiguous float32 2-D")
+    _require(data_int8.dtype == torch.uint8 and data_int8.is_contiguous(), "packed buffer must be contiguous uint8")
+    _require(params.dtype == torch.float32 and params.is_contiguous() and params.dim() == 2
+             and params.size(0) >= data_fp32.size(0) and params.size(1) == params_cols,
+             f"parameters must be contiguous float32 [rows, {params_cols}]")
+    return dev
+
+
+def quantize_tensor_for_all_procs(input: torch.Tensor, output: torch.Tensor, quantized_params: torch.Tensor,
+                                  work_range_per_proc: torch.Tensor, num_procs: int, bits: int) -> None:
+    """Row-packed quantisation of a boundary buffer, every rank's segment on its own
+    (quantization_arm.cpp:364-435).  ``quantized_params`` [rows, 2] receives (zero_point,
+    scale) per row.  The reference packs 2 bits whatever ``bits`` says (:380-381); here
+    ``bits`` is honoured (2, 4 or 8)."""
+    dev = _check_codec_operands(input, output, quantized_params, bits, 2)
+    _require(work_range_per_proc.numel() == num_procs + 1, "work range must hold num_procs + 1 entries")
+    rows_d, packed_d, packed_rows, rows = _packed_range(work_range_per_proc, bits, dev)
+    _require(rows == input.size(0), "work range does not cover the buffer's rows")
+    _require(output.numel() >= packed_rows * input.size(1), "packed buffer too small")
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().gnnagg_quantize_segments_f32(
+            _lib.ptr(input), _lib.ptr(output), _lib.ptr(quantized_params), _lib.ptr(rows_d), _lib.ptr(packed_d),
+            num_procs, rows, packed_rows, input.size(1), bits, _lib.current_stream(dev)))
+
+
+def dequantize_tensor_for_all_procs(input: torch.Tensor, output: torch.Tensor, dequantized_params: torch.Tensor,
+                                    work_range_per_proc: torch.Tensor, num_procs: int, bits: int) -> None:
+    """Inverse of ``quantize_tensor_for_all_procs`` (quantization_arm.cpp:437-479):
+    ``output = q * scale + zero_point`` with one rounding."""
+    dev = _check_codec_operands(output, input, dequantized_params, bits, 2)
+    _require(work_range_per_proc.numel() == num_procs + 1, "work range must hold num_procs + 1 entries")
+    rows_d, packed_d, packed_rows, rows = _packed_range(work_range_per_proc, bits, dev)
+    _require(rows == output.size(0), "work range does not cover the buffer's rows")
+    _require(input.numel() >= packed_rows * output.size(1), "packed buffer too small")
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().gnnagg_dequantize_segments_f32(
+            _lib.ptr(input), _lib.ptr(dequantized_params), _lib.ptr(output), _lib.ptr(rows_d), _lib.ptr(packed_d),
+            num_procs, rows, packed_rows, output.size(1), bits, _lib.current_stream(dev)))
+
+
+def _one_segment(rows: int) -> torch.Tensor:
+    return torch.tensor([0, rows], dtype=torch.int32)
+
+
+def quantize_tensor(input: torch.Tensor, output: torch.Tensor, quantized_params: torch.Tensor, bits: int) -> None:
+    """The whole buffer as one segment (quantization_arm.cpp:302-331)."""
+    quantize_tensor_for_all_procs(input, output, quantized_params, _one_segment(input.size(0)), 1, bits)
+
+
+def dequantize_tensor(input: torch.Tensor, output: torch.Tensor, dequantized_params: torch.Tensor, bits: int) -> None:
+    """quantization_arm.cpp:333-362."""
+    dequantize_tensor_for_all_procs(input, output, dequantized_params, _one_segment(output.size(0)), 1, bits)
+
+
+def _raise_on_bad_width(flag: torch.Tensor) -> None:
+    if int(flag.item()) != 0:  # the reference prints "Error: unsupported num_bits" and goes on
+        raise RuntimeError("Input mismatch: a row's bit width is not 2, 4 or 8")
+
+
+def quantize_tensor_v1(input: torch.Tensor, output: torch.Tensor, quantized_nodes_feat_range: torch.Tensor,
+                       quantized_params: torch.Tensor) -> None:
+    """Feature-packed quantisation with a width per row (quantization_x86.cpp:164-243):
+    ``quantized_params`` [rows, 3] holds the width in column 0 and receives (zero_point,
+    scale) in columns 1-2; row i owns bytes ``range[i]..range[i+1]`` of ``output``.
+    Synchronises (the width check is read back)."""
+    _require_hip(input, "fp32 buffer")
+    dev = input.device
+    for t, name in ((output, "packed buffer"), (quantized_nodes_feat_range, "feature range"),
+                    (quantized_params, "quantisation parameters")):
+        _require_hip(t, name, dev)
+    _require(input.dtype == torch.float32 and input.dim() == 2 and input.is_contiguous(),
+             "fp32 buffer must be contiguous float32 2-D")
+    _require(output.dtype == torch.uint8 and output.is_contiguous(), "packed buffer must be contiguous uint8")
+    _require(quantized_nodes_feat_range.dtype == torch.int64 and quantized_nodes_feat_range.is_contiguous()
+             and quantized_nodes_feat_range.numel() == input.size(0) + 1, "feature range must be int64 [rows + 1]")
+    _require(quantized_params.dtype == torch.float32 and quantized_params.is_contiguous()
+             and tuple(quantized_params.shape) == (input.size(0), 3), "parameters must be contiguous float32 [rows, 3]")
+    flag = torch.zeros(1, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().gnnagg_quantize_mixed_f32(
+            _lib.ptr(input), _lib.ptr(output), _lib.ptr(quantized_nodes_feat_range), _lib.ptr(quantized_params),
+            input.size(0), input.size(1), _lib.ptr(flag), _lib.current_stream(dev)))
+    _raise_on_bad_width(flag)
+
+
+def dequantize_tensor_v1(input: torch.Tensor, output: torch.Tensor, quantized_nodes_feat_range: torch.Tensor,
+                         quantized_params: torch.Tensor) -> None:
+    """quantization_x86.cpp:245-305."""
+    _require_hip(output, "fp32 buffer")
+    dev = output.device
+    for t, name in ((input, "packed buffer"), (quantized_nodes_feat_range, "feature range"),
+                    (quantized_params, "quantisation parameters")):
+        _require_hip(t, name, dev)
+    _require(output.dtype == torch.float32 and output.dim() == 2 and output.is_contiguous(),
+             "fp32 buffer must be contiguous float32 2-D")
+    _require(input.dtype == torch.uint8 and input.is_contiguous(), "packed buffer must be contiguous uint8")
+    _require(quantized_nodes_feat_range.dtype == torch.int64 and quantized_nodes_feat_range.is_contiguous()
+             and quantized_nodes_feat_range.numel() == output.size(0) + 1, "feature range must be int64 [rows + 1]")
+    _require(quantized_params.dtype == torch.float32 and quantized_params.is_contiguous()
+             and tuple(quantized_params.shape) == (output.size(0), 3), "parameters must be contiguous float32 [rows, 3]")
+    flag = torch.zeros(1, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().gnnagg_dequantize_mixed_f32(
+            _lib.ptr(input), _lib.ptr(quantized_nodes_feat_range), _lib.ptr(quantized_params), _lib.ptr(output),
+            output.size(0), output.size(1), _lib.ptr(flag), _lib.current_stream(dev)))
+    _raise_on_bad_width(flag)

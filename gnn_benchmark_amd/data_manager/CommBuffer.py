@@ -1,7 +1,7 @@
 """Send / receive boundary buffers of one partition, allocated once at the widest layer and
 re-shaped per layer (``resize_`` keeps the storage).  Counterpart of
-self_benchmark/a64fx/data_manager/CommBuffer.py:4-25; the int2 buffers of :27-49 belong to
-the quantised exchange and are not built."""
+self_benchmark/a64fx/data_manager/CommBuffer.py:4-25 (fp32 / bf16 rows) and :27-49 (the
+packed buffers, per-row parameters and per-rank work ranges of the quantised exchange)."""
 import torch
 
 from .CommSplits import CommSplits
@@ -27,3 +27,36 @@ class CommBuffer(object):
         if bits == 16 and self.send_buf_fp16 is not None:
             self.send_buf_fp16.resize_(send_shape)
             self.recv_buf_fp16.resize_(recv_shape)
+
+
+def _prefix(splits, device) -> torch.Tensor:
+    out = torch.zeros(len(splits) + 1, dtype=torch.int32)
+    out[1:] = torch.tensor(splits, dtype=torch.int32).cumsum(0)
+    return out.to(device) if device is not None else out
+
+
+class CommBufferForQuantization(object):
+    """Packed data, (zero_point, scale) per row in fp32 and in the bf16 that travels, and the
+    row prefix per peer rank for both directions (CommBuffer.py:27-49).  The reference builds
+    these for ``bits == 2`` only; 4 and 8 use the same layout here."""
+
+    def __init__(self, comm_splits: CommSplits, feat_len: int, bits: int, device=None) -> None:
+        if bits not in (2, 4, 8):
+            raise ValueError("quantised buffers exist for 2, 4 or 8 bits")
+        self.bits = bits
+        send_rows, recv_rows = sum(comm_splits.send_splits), sum(comm_splits.recv_splits)
+        self.quantized_send_data_buf = torch.zeros((sum(comm_splits.send_splits_int2), feat_len), dtype=torch.uint8,
+                                                   device=device)
+        self.quantized_recv_data_buf = torch.zeros((sum(comm_splits.recv_splits_int2), feat_len), dtype=torch.uint8,
+                                                   device=device)
+        self.quantized_send_params_buf_fp32 = torch.zeros((send_rows, 2), dtype=torch.float32, device=device)
+        self.quantized_recv_params_buf_fp32 = torch.zeros((recv_rows, 2), dtype=torch.float32, device=device)
+        self.quantized_send_params_buf_bf16 = torch.zeros((send_rows, 2), dtype=torch.bfloat16, device=device)
+        self.quantized_recv_params_buf_bf16 = torch.zeros((recv_rows, 2), dtype=torch.bfloat16, device=device)
+        self.quantized_work_range_per_proc = _prefix(comm_splits.send_splits, device)
+        self.dequantized_work_range_per_proc = _prefix(comm_splits.recv_splits, device)
+
+    def resize_buffer(self, comm_splits: CommSplits, feat_len: int, bits: int) -> None:
+        if bits == self.bits:
+            self.quantized_send_data_buf.resize_((sum(comm_splits.send_splits_int2), feat_len))
+            self.quantized_recv_data_buf.resize_((sum(comm_splits.recv_splits_int2), feat_len))

@@ -17,7 +17,7 @@ from typing import Callable, Optional
 import numpy as np
 import torch
 
-from .CommBuffer import CommBuffer
+from .CommBuffer import CommBuffer, CommBufferForQuantization
 from .CommSplits import CommSplits
 from .DataProcessor import DataProcessor, DataProcessorForPreAggresive
 from .DistributedGraph import DistributedGraph, DistributedGraphForPre
@@ -49,6 +49,11 @@ def _to_device(edges, device):
     return edges.to(device)
 
 
+def _quantization_buffers(comm_splits, max_feat_len, bits, device):
+    # DataLoader.py:105-108, :168-171 (there for bits == 2 only)
+    return CommBufferForQuantization(comm_splits, max_feat_len, bits, device=device) if bits in (2, 4, 8) else None
+
+
 def get_distributed_graph(local_edges_list, remote_edges_list, local_nodes_list, nodes_range_on_each_subgraph,
                           num_local_nodes: int, max_feat_len: int, world_size: int, bits: int, *,
                           halo_id_exchange: Optional[Callable] = None, exchange: Optional[Callable] = None,
@@ -71,7 +76,9 @@ def get_distributed_graph(local_edges_list, remote_edges_list, local_nodes_list,
     comm_buf = CommBuffer(comm_splits, max_feat_len, bits, device=local_adj_t.device)
     return DistributedGraph(local_adj_t, remote_adj_t, local_nodes_required_by_other,
                             num_local_nodes_required_by_other.tolist(), remote_nodes_num_from_each_subgraph.tolist(),
-                            in_degrees, comm_splits, comm_buf, None, exchange=exchange)
+                            in_degrees, comm_splits, comm_buf,
+                            _quantization_buffers(comm_splits, max_feat_len, bits, local_adj_t.device),
+                            exchange=exchange)
 
 
 def get_distributed_graph_for_pre_aggressive(local_edges_list, remote_edges_list, nodes_range_on_each_subgraph,
@@ -95,4 +102,6 @@ def get_distributed_graph_for_pre_aggressive(local_edges_list, remote_edges_list
     comm_splits = CommSplits(from_splits, to_splits, world_size, bits)
     comm_buf = CommBuffer(comm_splits, max_feat_len, bits, device=local_adj_t.device)
     return DistributedGraphForPre(local_adj_t, adj_t_pre_post_aggr_from, adj_t_pre_post_aggr_to, from_splits,
-                                  to_splits, in_degrees, comm_splits, comm_buf, None, exchange=exchange)
+                                  to_splits, in_degrees, comm_splits, comm_buf,
+                                  _quantization_buffers(comm_splits, max_feat_len, bits, local_adj_t.device),
+                                  exchange=exchange)

@@ -177,6 +177,46 @@ int64_t gnnagg_wgrad_workspace_bytes(int64_t rows, int64_t fi, int64_t fo);
 int gnnagg_wgrad_f32(const float *x, const float *g, float *w_grad, void *workspace, int64_t rows, int64_t fi,
                      int64_t fo, void *stream);
 
+/* ---------------------------------------------------------------------------------
+ * Codec of the boundary buffers: fp32 rows <-> int2 / int4 / int8 (bits = 2, 4, 8).
+ *
+ * Row-packed layout, one segment per destination rank.  Replaces
+ * `quantize_tensor_for_all_procs` / `dequantize_tensor_for_all_procs`
+ * (model/ops/src/quantization_arm.cpp:364-479, called from quantizer.py:80-90) and, with a
+ * single segment, `quantize_tensor` / `dequantize_tensor` (quantization_arm.cpp:302-362,
+ * quantization_x86.cpp:17-162).  x / out fp32 [rows, feat]; params fp32 [rows, 2] =
+ * (zero_point, scale) per row -- written by quantize (zero_point = row minimum, scale =
+ * (max - min) / (2^bits - 1), 1 when that is 0), read by dequantize; packed uint8
+ * [packed_rows, feat]: 8/bits consecutive rows of a segment share one byte per column, row
+ * k of a group at bit (8/bits - k - 1) * bits, and every segment starts a new group.
+ * row_range / packed_range: int32 [segments + 1] in DEVICE memory, prefix sums of the rows
+ * and of the packed rows (ceil(rows_p * bits / 8)) per segment -- the reference's
+ * `quantized_work_range_per_proc` (data_manager/CommBuffer.py:37-43) and what its
+ * divide_work_v1 derives from it (quantization_arm.cpp:21-31).  q = rint((x - zero_point)
+ * / scale) to nearest even; x' = fma(q, scale, zero_point).  The reference hard-codes 2
+ * bits in the per-rank variant; 4 and 8 follow the same rule as its x86 kernels.
+ * No allocation, no host synchronisation.
+ *
+ * Feature-packed layout with a width per row ("mixed bits").  Replaces
+ * `quantize_tensor_v1` / `dequantize_tensor_v1` (quantization_x86.cpp:164-305, called from
+ * quantizer.py:52-66).  params fp32 [rows, 3] = (bits, zero_point, scale): column 0 is read
+ * (2, 4 or 8 per row), columns 1-2 written by quantize; feat_range int64 [rows + 1] in
+ * device memory = byte offset of every row in `data`
+ * (quantizer.py:69-77); 8/bits consecutive features share a byte, same shift rule.  A row
+ * whose width is not 2, 4 or 8 is left alone and sets *bad_width (device int32, zeroed by
+ * the caller) to 1 -- the reference prints an error for it (quantization_x86.cpp:241).
+ * ------------------------------------------------------------------------------- */
+int gnnagg_quantize_segments_f32(const float *x, uint8_t *packed, float *params, const int32_t *row_range,
+                                 const int32_t *packed_range, int64_t segments, int64_t rows, int64_t packed_rows,
+                                 int64_t feat, int bits, void *stream);
+int gnnagg_dequantize_segments_f32(const uint8_t *packed, const float *params, float *out, const int32_t *row_range,
+                                   const int32_t *packed_range, int64_t segments, int64_t rows, int64_t packed_rows,
+                                   int64_t feat, int bits, void *stream);
+int gnnagg_quantize_mixed_f32(const float *x, uint8_t *data, const int64_t *feat_range, float *params, int64_t rows,
+                              int64_t feat, int32_t *bad_width, void *stream);
+int gnnagg_dequantize_mixed_f32(const uint8_t *data, const int64_t *feat_range, const float *params, float *out,
+                                int64_t rows, int64_t feat, int32_t *bad_width, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -43,12 +43,27 @@ def _lib():
                                         ctypes.c_int32]
         lib.oracle_spmm_f32.restype = ctypes.c_int
         lib.oracle_max_threads.restype = ctypes.c_int
+        lib.oracle_fma_rows_f32.argtypes = [f32p, f32p, f32p, f32p, ctypes.c_int64, ctypes.c_int64]
+        lib.oracle_fma_rows_f32.restype = None
         _LIB = lib
     return _LIB
 
 
 def _p(a, ct):
     return a.ctypes.data_as(ctypes.POINTER(ct))
+
+
+def fma_rows(q: np.ndarray, scale: np.ndarray, zero_point: np.ndarray) -> np.ndarray:
+    """``fmaf(q[r, j], scale[r], zero_point[r])`` for every element, one rounding each."""
+    q = np.ascontiguousarray(q, dtype=np.float32)
+    scale = np.ascontiguousarray(scale, dtype=np.float32)
+    zero_point = np.ascontiguousarray(zero_point, dtype=np.float32)
+    rows, feat = q.shape
+    assert scale.shape == (rows,) and zero_point.shape == (rows,)
+    out = np.empty_like(q)
+    _lib().oracle_fma_rows_f32(_p(q, ctypes.c_float), _p(scale, ctypes.c_float), _p(zero_point, ctypes.c_float),
+                               _p(out, ctypes.c_float), rows, feat)
+    return out
 
 
 def max_threads() -> int:

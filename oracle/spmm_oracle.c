@@ -133,3 +133,14 @@ int oracle_max_threads(void) {
     return 1;
 #endif
 }
+
+/* out[r][j] = fmaf(q[r][j], scale[r], zero_point[r]): the single-rounding multiply-add the
+ * reference's dequantisation kernels use (svmla, quantization_arm.cpp:263-266).  Exact fmaf
+ * from libm / the FMA unit; numpy has no fused multiply-add. */
+void oracle_fma_rows_f32(const float *q, const float *scale, const float *zero_point, float *out,
+                         int64_t rows, int64_t feat) {
+    for (int64_t r = 0; r < rows; r++) {
+        const float s = scale[r], z = zero_point[r];
+        for (int64_t j = 0; j < feat; j++) out[r * feat + j] = fmaf(q[r * feat + j], s, z);
+    }
+}

@@ -1,0 +1,196 @@
+"""GPU parity of the boundary-buffer codec against the oracle (oracle/quantization.py,
+itself pinned to the reference's golden bytes and compiled kernels): packed bytes and
+parameters bit-exact, dequantised rows bit-exact (one fused multiply-add per element)."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import quantization as oq
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "quantization_reference_op_vectors.npz")
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _rows(rng, rows, feat):
+    x = (rng.standard_normal((rows, feat)) * rng.uniform(0.01, 50.0, (rows, 1))).astype(np.float32)
+    if rows > 3:
+        x[3] = -4.5  # constant row: scale 0 -> 1
+    return x
+
+
+@pytest.mark.parametrize("bits", [2, 4, 8])
+@pytest.mark.parametrize("feat", [1, 3, 16, 47, 64, 100, 128, 130, 256, 260, 602, 1024, 1028, 2052])
+def test_segments_codec_matches_oracle(bits, feat):
+    from gnn_benchmark_amd import computation_ops as ops
+
+    rng = np.random.default_rng(1000 * bits + feat)
+    splits = [5, 0, 13, 1, 8, 0, 4, 7]
+    rows = sum(splits)
+    x = _rows(rng, rows, feat)
+    want_packed, want_params = oq.quantize_segments(x, splits, bits)
+    work_range = torch.tensor(np.concatenate(([0], np.cumsum(splits))), dtype=torch.int32)
+    packed = torch.full(want_packed.shape, 0xAB, dtype=torch.uint8, device="cuda")
+    params = torch.full((rows, 2), -7.0, device="cuda")
+    ops.quantize_tensor_for_all_procs(dev(x), packed, params, work_range, len(splits), bits)
+    assert np.array_equal(params.cpu().numpy(), want_params)
+    assert np.array_equal(packed.cpu().numpy(), want_packed)
+
+    wire = oq.params_over_the_wire(want_params)  # the receiver sees bf16-rounded parameters
+    for p in (want_params, wire):
+        want_back = oq.dequantize_segments(want_packed, p, splits, bits)
+        back = torch.full((rows, feat), 9.0, device="cuda")
+        ops.dequantize_tensor_for_all_procs(packed, back, dev(p), work_range.cuda(), len(splits), bits)
+        assert np.array_equal(back.cpu().numpy().view(np.uint32), want_back.view(np.uint32))
+
+
+@pytest.mark.parametrize("bits", [2, 4, 8])
+def test_whole_buffer_as_one_segment_and_ragged_tail(bits):
+    from gnn_benchmark_amd.quantizer import QuantizerForPureBits
+
+    epb = 8 // bits
+    rng = np.random.default_rng(bits)
+    for rows in (1, epb, epb + 1, 4 * epb - 1, 1001):
+        x = _rows(rng, rows, 100)
+        want_packed, want_params = oq.quantize_segments(x, [rows], bits)
+        packed = torch.zeros(want_packed.shape, dtype=torch.uint8, device="cuda")
+        assert packed.numel() == QuantizerForPureBits.get_quantized_buffer_size(rows, bits, 100)
+        params = torch.zeros((rows, 2), device="cuda")
+        QuantizerForPureBits.quantize_fp32_to_intX(dev(x), packed, params, bits)
+        assert np.array_equal(packed.cpu().numpy(), want_packed)
+        assert np.array_equal(params.cpu().numpy(), want_params)
+        back = torch.zeros((rows, 100), device="cuda")
+        QuantizerForPureBits.dequantize_intX_to_fp32(packed, back, params, bits)
+        assert np.array_equal(back.cpu().numpy(), oq.dequantize_segments(want_packed, want_params, [rows], bits))
+
+
+def test_committed_outputs_of_the_reference_kernels_bit_for_bit():
+    """Row-packed cases: the reference's x86 kernel takes the parameters as inputs; they are
+    the row's own min / range here, so the bytes must agree.  Mixed-bits cases as they are."""
+    from gnn_benchmark_amd import computation_ops as ops
+
+    z = np.load(GOLDEN)
+    for c in range(int(z["rows_cases"])):
+        x, bits = z[f"rows{c}_x"], int(z[f"rows{c}_bits"])
+        packed = torch.zeros(z[f"rows{c}_packed"].shape, dtype=torch.uint8, device="cuda")
+        params = torch.zeros((x.shape[0], 2), device="cuda")
+        ops.quantize_tensor(dev(x), packed, params, bits)
+        assert np.array_equal(params.cpu().numpy(), z[f"rows{c}_params"])
+        assert np.array_equal(packed.cpu().numpy(), z[f"rows{c}_packed"]), c
+        back = torch.zeros(x.shape, device="cuda")
+        ops.dequantize_tensor(packed, back, params, bits)
+        assert np.array_equal(back.cpu().numpy(), z[f"rows{c}_back"]), c
+    for c in range(int(z["mixed_cases"])):
+        x = z[f"mixed{c}_x"]
+        params = torch.zeros((x.shape[0], 3), device="cuda")
+        params[:, 0] = dev(z[f"mixed{c}_bits"])
+        feat_range = dev(z[f"mixed{c}_range"])
+        data = torch.zeros(int(z[f"mixed{c}_range"][-1]), dtype=torch.uint8, device="cuda")
+        ops.quantize_tensor_v1(dev(x), data, feat_range, params)
+        assert np.array_equal(data.cpu().numpy(), z[f"mixed{c}_data"]), c
+        assert np.array_equal(params.cpu().numpy(), z[f"mixed{c}_params"]), c
+        back = torch.zeros(x.shape, device="cuda")
+        ops.dequantize_tensor_v1(data, back, feat_range, params)
+        assert np.array_equal(back.cpu().numpy(), z[f"mixed{c}_back"]), c
+
+
+def test_mixed_bits_golden_bytes_of_the_reference():
+    """self_benchmark/a64fx/tests/test_quantizer.py:58-84 through the reference's class names."""
+    from gnn_benchmark_amd.quantizer import QuantizerForMixedBits
+
+    x = torch.tensor([[0.2, 0.1, 0.3], [0.4, 0.5, 0.6], [0.7, 0.8, 0.9], [1.0, 1.1, 1.2], [0.3, 0.1, 0.7]],
+                     device="cuda")
+    bits = torch.tensor([8, 4, 2, 4, 4], device="cuda")
+    params = torch.empty((5, 3), device="cuda")
+    params[:, 0] = bits
+    feat_range = QuantizerForMixedBits.get_quantized_nodes_feat_range(5, 3, bits)
+    assert feat_range.tolist() == [0, 3, 5, 6, 8, 10]
+    data = torch.empty(int(feat_range[-1]), dtype=torch.uint8, device="cuda")
+    QuantizerForMixedBits.quantize_fp32_to_intX(x, data, feat_range, params)
+    assert data.tolist() == [127, 0, 255, 7, 240, 44, 8, 240, 80, 240]
+    lo = x.min(dim=1)[0]
+    assert torch.allclose(params[:, 1], lo) and torch.allclose(params[:, 2], (x.max(dim=1)[0] - lo) / (2.0 ** bits - 1))
+    back = torch.empty_like(x)
+    QuantizerForMixedBits.dequantize_intX_to_fp32(data, back, feat_range, params)
+    assert bool(((back - x).abs() <= params[:, 2:3] * 0.5 + 1e-6).all())
+
+
+def test_mixed_bits_wide_rows_match_oracle():
+    from gnn_benchmark_amd import computation_ops as ops
+
+    rng = np.random.default_rng(77)
+    for rows, feat in ((300, 100), (64, 602), (17, 1)):
+        x = _rows(rng, rows, feat)
+        bits = rng.choice([2, 4, 8], rows).astype(np.float32)
+        want_data, want_params = oq.quantize_mixed(x, bits)
+        feat_range = oq.get_quantized_nodes_feat_range(rows, feat, bits)
+        params = torch.zeros((rows, 3), device="cuda")
+        params[:, 0] = dev(bits)
+        data = torch.zeros(int(feat_range[-1]), dtype=torch.uint8, device="cuda")
+        ops.quantize_tensor_v1(dev(x), data, dev(feat_range), params)
+        assert np.array_equal(data.cpu().numpy(), want_data)
+        assert np.array_equal(params.cpu().numpy(), want_params)
+        back = torch.zeros((rows, feat), device="cuda")
+        ops.dequantize_tensor_v1(data, back, dev(feat_range), params)
+        assert np.array_equal(back.cpu().numpy(), oq.dequantize_mixed(want_data, want_params, feat))
+
+
+def test_error_behaviour():
+    from gnn_benchmark_amd import computation_ops as ops
+
+    x = torch.zeros((8, 16), device="cuda")
+    packed = torch.zeros((2, 16), dtype=torch.uint8, device="cuda")
+    params = torch.zeros((8, 2), device="cuda")
+    with pytest.raises(RuntimeError, match="bits"):
+        ops.quantize_tensor(x, packed, params, 3)
+    with pytest.raises(RuntimeError, match="GPU"):
+        ops.quantize_tensor(x.cpu(), packed, params, 2)
+    with pytest.raises(RuntimeError, match="too small"):
+        ops.quantize_tensor(x, packed[:1], params, 2)
+    with pytest.raises(RuntimeError, match="work range"):
+        ops.quantize_tensor_for_all_procs(x, packed, params, torch.tensor([0, 4, 7], dtype=torch.int32), 2, 2)
+    p3 = torch.zeros((8, 3), device="cuda")
+    p3[:, 0] = 3
+    with pytest.raises(RuntimeError, match="bit width"):
+        ops.quantize_tensor_v1(x, torch.zeros(64, dtype=torch.uint8, device="cuda"),
+                               torch.arange(9, dtype=torch.int64, device="cuda") * 6, p3)
+    # empty buffers are fine
+    ops.quantize_tensor(x[:0], packed[:0], params[:0], 2)
+    ops.dequantize_tensor(packed[:0], x[:0], params[:0], 2)
+
+
+def test_full_size_round_trip_properties():
+    """3 M boundary rows x 128 (config 4's receive buffer): idempotence of the codec -- what was
+    dequantised quantises back to the same bytes -- and the half-step error bound."""
+    from gnn_benchmark_amd import computation_ops as ops
+
+    rows, feat, bits = 3_000_003, 128, 2
+    gen = torch.Generator(device="cuda").manual_seed(1)
+    x = torch.randn(rows, feat, device="cuda", generator=gen)
+    splits = [rows // 15] * 15
+    splits[-1] += rows - sum(splits)
+    splits.insert(3, 0)
+    work_range = torch.tensor(np.concatenate(([0], np.cumsum(splits))), dtype=torch.int32)
+    packed_rows = sum(-(-s // 4) for s in splits)
+    packed = torch.zeros((packed_rows, feat), dtype=torch.uint8, device="cuda")
+    params = torch.zeros((rows, 2), device="cuda")
+    ops.quantize_tensor_for_all_procs(x, packed, params, work_range, 16, bits)
+    back = torch.empty_like(x)
+    ops.dequantize_tensor_for_all_procs(packed, back, params, work_range, 16, bits)
+    assert bool(((back - x).abs() <= params[:, 1:2] * 0.5 * (1 + 1e-5) + 1e-6).all())
+    assert torch.equal(params[:, 0], x.min(dim=1)[0])
+    packed2 = torch.zeros_like(packed)
+    params2 = torch.zeros_like(params)
+    ops.quantize_tensor_for_all_procs(back, packed2, params2, work_range, 16, bits)
+    assert torch.equal(packed2, packed)
+    # a sample of rows against the oracle
+    sel = slice(splits[0] - 5, splits[0] + 9)  # straddles the first segment boundary
+    xs = x[sel].cpu().numpy()
+    want = oq.row_params(xs, bits)
+    assert np.array_equal(params[sel].cpu().numpy(), want)
