@@ -18,7 +18,19 @@ What differs from the reference, on purpose:
   gradient rows in ``comm_buf.send_buf``.  A returned handle's ``wait()`` is called after
   the local SpMM, where the reference waits (aggregator.py:78, :175).  ``exchange is
   None`` is the single-rank world: pre/post steps are skipped (aggregator.py:47, :100).
-* No process group, timers or quantiser singletons are touched.
+* With ``num_bits`` 2 (the reference's int2 exchange, communicator.py:231-325; 4 and 8 are
+  accepted with the same layout) the outgoing buffer is quantised here, per peer rank,
+  into ``graph.comm_buf_for_quantization`` -- the reference does that inside its
+  communicator (:281-284) -- and the byte exchange is ``graph.exchange_quantized``, a
+  callable ``(comm_splits, comm_buf_for_quantization, tag, direction) -> handle | None``:
+  on "forward" it must leave the peers' packed rows in ``quantized_recv_data_buf`` and
+  their (zero_point, scale) rows, rounded through bf16 as on the reference's wire
+  (:297-303), in ``quantized_recv_params_buf_fp32``; on "backward" the same with the
+  roles of the send and receive buffers swapped (:266-276).  The received rows are
+  dequantised after the wait, where the reference does it (aggregator.py:83-88,
+  :180-187).  Outside training the forward exchange stays fp32 (communicator.py:64-65).
+* No process group or timers are touched; the quantiser is built from the buffers' width,
+  not looked up as a singleton.
 * ``torch.zeros`` + accumulate (aggregator.py:67-70, :167-170) and ``zero_()`` +
   accumulate (:44-49, :144-149) run as one overwriting SpMM; the values are identical
   because an FMA chain started from a stored 0 equals one started from a register 0.
@@ -27,7 +39,7 @@ What differs from the reference, on purpose:
 """
 import torch
 
-from . import _lib
+from . import _lib, computation_ops
 from .spmm_kernel import SPMM_backward, SPMM_forward
 
 
@@ -46,8 +58,52 @@ def _gather_rows(src: torch.Tensor, index: torch.Tensor, out: torch.Tensor) -> N
 
 
 def _check_bits(num_bits: int) -> None:
-    if num_bits not in (32, 16):
-        raise NotImplementedError("quantised boundary exchange (num_bits=%r) is outside this build" % (num_bits,))
+    if num_bits not in (32, 16, 8, 4, 2):
+        raise NotImplementedError("boundary exchange with num_bits=%r is not defined" % (num_bits,))
+
+
+def _quantized(graph, num_bits: int) -> bool:
+    # aggregator.py:35, :83, :136, :180: quantised buffers are used for widths other than 32 / 16
+    if num_bits in (32, 16):
+        return False
+    qbuf = getattr(graph, "comm_buf_for_quantization", None)
+    if qbuf is None or qbuf.bits != num_bits:
+        raise RuntimeError("Input mismatch: the graph holds no %d-bit quantisation buffers "
+                           "(build it with bits=%d)" % (num_bits, num_bits))
+    if getattr(graph, "exchange_quantized", None) is None:
+        raise RuntimeError("graph.exchange_quantized is required for a %d-bit boundary exchange" % num_bits)
+    return True
+
+
+def _quantize_and_exchange(graph, num_bits: int, tag: str, direction: str):
+    """Pack the outgoing rows per peer rank and hand the bytes to the exchange
+    (communicator.py:241-311)."""
+    qbuf = graph.comm_buf_for_quantization
+    world = len(graph.comm_splits.send_splits)
+    if direction == "forward":
+        outgoing, data, params, work_range = (graph.comm_buf.send_buf, qbuf.quantized_send_data_buf,
+                                              qbuf.quantized_send_params_buf_fp32, qbuf.quantized_work_range_per_proc)
+    else:
+        outgoing, data, params, work_range = (graph.comm_buf.recv_buf, qbuf.quantized_recv_data_buf,
+                                              qbuf.quantized_recv_params_buf_fp32,
+                                              qbuf.dequantized_work_range_per_proc)
+    if outgoing.size(0) != 0:
+        computation_ops.quantize_tensor_for_all_procs(outgoing, data, params, work_range, world, num_bits)
+    return graph.exchange_quantized(graph.comm_splits, qbuf, tag, direction)
+
+
+def _dequantize_received(graph, num_bits: int, direction: str) -> None:
+    qbuf = graph.comm_buf_for_quantization
+    world = len(graph.comm_splits.send_splits)
+    if direction == "forward":  # aggregator.py:85-88
+        incoming, data, params, work_range = (graph.comm_buf.recv_buf, qbuf.quantized_recv_data_buf,
+                                              qbuf.quantized_recv_params_buf_fp32,
+                                              qbuf.dequantized_work_range_per_proc)
+    else:  # aggregator.py:182-187
+        incoming, data, params, work_range = (graph.comm_buf.send_buf, qbuf.quantized_send_data_buf,
+                                              qbuf.quantized_send_params_buf_fp32, qbuf.quantized_work_range_per_proc)
+    if incoming.size(0) != 0:
+        computation_ops.dequantize_tensor_for_all_procs(data, incoming, params, work_range, world, num_bits)
 
 
 class Aggregator(torch.autograd.Function):
@@ -63,6 +119,10 @@ class Aggregator(torch.autograd.Function):
         local_nodes_feat = local_nodes_feat.contiguous()
         graph.comm_buf.resize_buffer(graph.comm_splits, feat_len, num_bits)
         exchange = getattr(graph, "exchange", None)
+        quantized = exchange is not None and _quantized(graph, num_bits)
+        if quantized:
+            graph.comm_buf_for_quantization.resize_buffer(graph.comm_splits, feat_len, num_bits)
+        quantized = quantized and is_training  # communicator.py:64-65: fp32 rows outside training
         comm_handle = None
         send_buf = graph.comm_buf.send_buf
 
@@ -71,7 +131,10 @@ class Aggregator(torch.autograd.Function):
                 SPMM_forward(graph.adj_t_pre_post_aggr_to, local_nodes_feat, send_buf, accumulate=False)
             else:  # raw boundary rows
                 _gather_rows(local_nodes_feat, graph.idx_nodes_send_to_others, send_buf)
-            comm_handle = exchange(graph.comm_splits, graph.comm_buf, f"forward{layer}", "forward")
+            if quantized:
+                comm_handle = _quantize_and_exchange(graph, num_bits, f"forward{layer}", "forward")
+            else:
+                comm_handle = exchange(graph.comm_splits, graph.comm_buf, f"forward{layer}", "forward")
 
         out = torch.empty([graph.local_adj_t.sparse_size(0), feat_len], dtype=torch.float32,
                           device=local_nodes_feat.device)
@@ -79,6 +142,8 @@ class Aggregator(torch.autograd.Function):
 
         if comm_handle is not None:
             comm_handle.wait()
+        if quantized:
+            _dequantize_received(graph, num_bits, "forward")
 
         remote_nodes_feat = graph.comm_buf.recv_buf
         if exchange is not None and remote_nodes_feat.size(0) != 0:
@@ -99,6 +164,9 @@ class Aggregator(torch.autograd.Function):
         feat_len = local_out_grad.size(-1)
         graph.comm_buf.resize_buffer(graph.comm_splits, feat_len, num_bits)
         exchange = getattr(graph, "exchange", None)
+        quantized = exchange is not None and _quantized(graph, num_bits)
+        if quantized:
+            graph.comm_buf_for_quantization.resize_buffer(graph.comm_splits, feat_len, num_bits)
 
         # the receive buffer carries the outgoing halo gradients on the way back
         remote_nodes_grad_buf = graph.comm_buf.recv_buf
@@ -109,7 +177,9 @@ class Aggregator(torch.autograd.Function):
                 SPMM_backward(graph.remote_adj_t, local_out_grad, remote_nodes_grad_buf, accumulate=False)
 
         comm_handle = None
-        if exchange is not None:
+        if quantized:
+            comm_handle = _quantize_and_exchange(graph, num_bits, layer, "backward")
+        elif exchange is not None:
             comm_handle = exchange(graph.comm_splits, graph.comm_buf, layer, "backward")
 
         local_nodes_grad = torch.empty([graph.local_adj_t.sparse_size(-1), feat_len], dtype=torch.float32,
@@ -118,6 +188,8 @@ class Aggregator(torch.autograd.Function):
 
         if comm_handle is not None:
             comm_handle.wait()
+        if quantized:
+            _dequantize_received(graph, num_bits, "backward")
 
         local_nodes_grad_buf = graph.comm_buf.send_buf
         if exchange is not None and local_nodes_grad_buf.size(0) != 0:

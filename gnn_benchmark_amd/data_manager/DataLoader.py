@@ -57,7 +57,7 @@ def _quantization_buffers(comm_splits, max_feat_len, bits, device):
 def get_distributed_graph(local_edges_list, remote_edges_list, local_nodes_list, nodes_range_on_each_subgraph,
                           num_local_nodes: int, max_feat_len: int, world_size: int, bits: int, *,
                           halo_id_exchange: Optional[Callable] = None, exchange: Optional[Callable] = None,
-                          device=None) -> DistributedGraph:
+                          exchange_quantized: Optional[Callable] = None, device=None) -> DistributedGraph:
     local_edges_list = _to_device(local_edges_list, device)
     remote_edges_list = _to_device(remote_edges_list, device)
     in_degrees = DataProcessor.get_in_degrees(local_edges_list, remote_edges_list, num_local_nodes)
@@ -78,13 +78,14 @@ def get_distributed_graph(local_edges_list, remote_edges_list, local_nodes_list,
                             num_local_nodes_required_by_other.tolist(), remote_nodes_num_from_each_subgraph.tolist(),
                             in_degrees, comm_splits, comm_buf,
                             _quantization_buffers(comm_splits, max_feat_len, bits, local_adj_t.device),
-                            exchange=exchange)
+                            exchange=exchange, exchange_quantized=exchange_quantized)
 
 
 def get_distributed_graph_for_pre_aggressive(local_edges_list, remote_edges_list, nodes_range_on_each_subgraph,
                                              num_local_nodes, max_feat_len, rank, world_size, bits, *,
                                              graph_exchange: Optional[Callable] = None,
                                              exchange: Optional[Callable] = None,
+                                             exchange_quantized: Optional[Callable] = None,
                                              device=None) -> DistributedGraphForPre:
     local_edges_list = _to_device(local_edges_list, device)
     remote_edges_list = _to_device(remote_edges_list, device)
@@ -104,4 +105,4 @@ def get_distributed_graph_for_pre_aggressive(local_edges_list, remote_edges_list
     return DistributedGraphForPre(local_adj_t, adj_t_pre_post_aggr_from, adj_t_pre_post_aggr_to, from_splits,
                                   to_splits, in_degrees, comm_splits, comm_buf,
                                   _quantization_buffers(comm_splits, max_feat_len, bits, local_adj_t.device),
-                                  exchange=exchange)
+                                  exchange=exchange, exchange_quantized=exchange_quantized)

@@ -3,10 +3,12 @@ split lists and the boundary buffers.  Field names and constructor order are the
 reference's (self_benchmark/a64fx/data_manager/DistributedGraph.py:8-33, :35-59), because
 ``Aggregator`` and the layers address them by name.
 
-One field is added to both: ``exchange``, the callable that stands in for the boundary
-all-to-all (model/layers/aggregator.py:54-61, :156-163).  ``None`` means a single-rank
+Two fields are added to both: ``exchange``, the callable that stands in for the boundary
+all-to-all (model/layers/aggregator.py:54-61, :156-163) -- ``None`` means a single-rank
 world: the aggregator then skips pre-/post-aggregation exactly like the reference does for
-``world_size == 1`` (aggregator.py:47, :100).
+``world_size == 1`` (aggregator.py:47, :100) -- and ``exchange_quantized``, its counterpart
+for the packed bytes and per-row parameters of a quantised exchange
+(communicator.py:231-325).
 """
 from dataclasses import dataclass, field
 from typing import Any, Callable, List, Optional
@@ -29,8 +31,9 @@ class DistributedGraph:
     in_degrees: torch.Tensor                   # fp32 [N, 1]
     comm_splits: CommSplits
     comm_buf: CommBuffer
-    comm_buf_for_quantization: Any = None      # quantised exchange: not built
+    comm_buf_for_quantization: Any = None      # CommBufferForQuantization for bits 2 / 4 / 8
     exchange: Optional[Callable] = None
+    exchange_quantized: Optional[Callable] = None
     _scatter: Optional[SparseTensor] = field(default=None, repr=False)
 
     def send_scatter_adj_t(self) -> SparseTensor:
@@ -59,3 +62,4 @@ class DistributedGraphForPre:
     comm_buf: CommBuffer
     comm_buf_for_quantization: Any = None
     exchange: Optional[Callable] = None
+    exchange_quantized: Optional[Callable] = None

@@ -12,6 +12,7 @@ product ``A X`` on every rank, and likewise for the transposed (gradient) direct
 """
 import numpy as np
 
+from . import quantization as oquant
 from . import spmm as ospmm
 
 
@@ -67,3 +68,14 @@ def backward_out_raw(local_adj, idx_nodes_send_to_others, grad, send_buf_in):
     for i, r in enumerate(np.asarray(idx_nodes_send_to_others, dtype=np.int64)):
         dx[r] += send_buf_in[i]
     return dx
+
+
+def quantized_wire(outgoing, splits, bits):
+    """What the peers see of an outgoing boundary buffer in a quantised exchange
+    (communicator.py:281-311, aggregator.py:83-88): every peer's segment packed on its own,
+    parameters rounded through bf16 on the wire, dequantised with those.  Row i of the result
+    is what the owner of row i's segment receives for it."""
+    if outgoing.shape[0] == 0:
+        return outgoing.copy()
+    packed, params = oquant.quantize_segments(outgoing, splits, bits)
+    return oquant.dequantize_segments(packed, oquant.params_over_the_wire(params), splits, bits)

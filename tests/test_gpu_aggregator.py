@@ -53,7 +53,7 @@ class PlayedExchange:
         return None
 
 
-def _build_pre_graphs(w: World, feat):
+def _build_pre_graphs(w: World, feat, bits=32):
     W = w.world
     parts = [w.partition(r) for r in range(W)]
     sent = []
@@ -65,7 +65,7 @@ def _build_pre_graphs(w: World, feat):
     for r in range(W):
         graphs.append(get_distributed_graph_for_pre_aggressive(
             torch.from_numpy(parts[r][0].copy()), torch.from_numpy(parts[r][1].copy()), torch.from_numpy(w.begins),
-            int(w.sizes[r]), feat, r, W, 32, graph_exchange=lambda _s, r=r: [sent[i][r] for i in range(W)],
+            int(w.sizes[r]), feat, r, W, bits, graph_exchange=lambda _s, r=r: [sent[i][r] for i in range(W)],
             device="cuda"))
     return graphs
 
@@ -195,7 +195,9 @@ def test_single_rank_world_and_autograd_contract():
     ret = Aggregator.backward(type("Ctx", (), dict(graph=gr, num_bits=32, is_pre_delay=True, layer=0))(), dev(g))
     assert len(ret) == 6 and all(ret[i] is None for i in (0, 2, 3, 4, 5))  # aggregator.py:208
     with pytest.raises(NotImplementedError):
-        Aggregator.apply(gr, xr, 0, 2, True, True)
+        Aggregator.apply(gr, xr, 0, 3, True, True)
+    # a single rank exchanges nothing, so a quantised width changes nothing (aggregator.py:47, :83)
+    assert torch.equal(Aggregator.apply(gr, xr, 0, 2, True, True), out)
 
 
 def test_synthetic_partition_built_on_device_matches_oracle():
@@ -236,3 +238,107 @@ def test_synthetic_partition_built_on_device_matches_oracle():
         assert np.array_equal(m.storage.colptr().cpu().numpy(), colptr)
         assert np.array_equal(m.storage.row_T().cpu().numpy(), row_t)
         assert np.array_equal(m.storage.value_T().cpu().numpy(), val_t)
+
+
+class PlayedQuantizedExchange:
+    """Quantised counterpart of PlayedExchange: delivers the peers' packed rows and their
+    bf16-rounded parameters into the buffers the aggregator dequantises from."""
+
+    def __init__(self, forward, backward):
+        self.forward, self.backward = forward, backward  # (packed rows, params) each
+        self.log = []
+
+    def __call__(self, comm_splits, qbuf, tag, direction):
+        self.log.append((tag, direction))
+        if direction == "forward":
+            qbuf.quantized_recv_data_buf.copy_(self.forward[0])
+            qbuf.quantized_recv_params_buf_fp32.copy_(self.forward[1])
+        else:
+            qbuf.quantized_send_data_buf.copy_(self.backward[0])
+            qbuf.quantized_send_params_buf_fp32.copy_(self.backward[1])
+        return None
+
+
+@pytest.mark.parametrize("bits", [2, 4, 8])
+@pytest.mark.parametrize("seed,sizes", [(0, (300, 450, 250)), (1, (600, 1, 400, 330))])
+def test_quantised_exchange_world_matches_oracle(seed, sizes, bits):
+    """Pre/post-aggregation with the boundary rows travelling as packed int2 / int4 / int8: every
+    rank's buffers, output and gradient are bit-identical to the oracle pipeline (oracle codec
+    between oracle SpMMs), and the result stays within the codec's error of the exact product."""
+    from oracle import quantization as oq
+
+    w = World(seed, sizes, mean_deg=8.0)
+    W, F = w.world, 48
+    graphs = _build_pre_graphs(w, F, bits=bits)
+    oracle_ranks = build_pre_world(w)
+    rng = np.random.default_rng(seed + 100)
+    x = rng.standard_normal((w.n, F)).astype(np.float32)
+    g = rng.standard_normal((w.n, F)).astype(np.float32)
+    sl = [slice(int(w.begins[r]), int(w.begins[r + 1])) for r in range(W)]
+    send_splits = [gr.comm_splits.send_splits for gr in graphs]
+    recv_splits = [gr.comm_splits.recv_splits for gr in graphs]
+    send_packed = [gr.comm_splits.send_splits_int2 for gr in graphs]
+    recv_packed = [gr.comm_splits.recv_splits_int2 for gr in graphs]
+
+    # oracle: what every rank sends, packed, in both directions
+    o_send = [oagg.forward_send(oracle_ranks[r]["a_to"], np.ascontiguousarray(x[sl[r]])) for r in range(W)]
+    o_back = [oagg.backward_recv(oracle_ranks[r]["a_from"], np.ascontiguousarray(g[sl[r]])) for r in range(W)]
+    q_send = [oq.quantize_segments(o_send[r], send_splits[r], bits) for r in range(W)]
+    q_back = [oq.quantize_segments(o_back[r], recv_splits[r], bits) for r in range(W)]
+    fwd_data = host_exchange([q[0] for q in q_send], send_packed, recv_packed)
+    fwd_params = host_exchange([oq.params_over_the_wire(q[1]) for q in q_send], send_splits, recv_splits)
+    bwd_data = host_exchange([q[0] for q in q_back], recv_packed, send_packed)
+    bwd_params = host_exchange([oq.params_over_the_wire(q[1]) for q in q_back], recv_splits, send_splits)
+    # the same rows, as the oracle's receiver decodes them
+    recv = host_exchange([oagg.quantized_wire(o_send[r], send_splits[r], bits) for r in range(W)], send_splits, recv_splits)
+    incoming = host_exchange([oagg.quantized_wire(o_back[r], recv_splits[r], bits) for r in range(W)], recv_splits,
+                             send_splits)
+
+    want, want_t = w.global_product(x), w.global_product(g, transposed=True)
+    for r in range(W):
+        gr, o = graphs[r], oracle_ranks[r]
+        gr.exchange = lambda *a: (_ for _ in ()).throw(AssertionError("fp32 exchange used in a quantised run"))
+        gr.exchange_quantized = PlayedQuantizedExchange((dev(fwd_data[r]), dev(fwd_params[r])),
+                                                        (dev(bwd_data[r]), dev(bwd_params[r])))
+        xr = dev(x[sl[r]]).requires_grad_()
+        out = Aggregator.apply(gr, xr, 1, bits, True, True)
+        qb = gr.comm_buf_for_quantization
+        assert np.array_equal(qb.quantized_send_data_buf.cpu().numpy(), q_send[r][0])
+        assert np.array_equal(qb.quantized_send_params_buf_fp32.cpu().numpy(), q_send[r][1])
+        assert np.array_equal(gr.comm_buf.recv_buf.cpu().numpy(), recv[r])
+        o_out = oagg.forward_out(o["local"], o["a_from"], np.ascontiguousarray(x[sl[r]]), recv[r])
+        assert np.array_equal(out.detach().cpu().numpy(), o_out)
+        out.backward(dev(g[sl[r]]))
+        assert gr.exchange_quantized.log == [("forward1", "forward"), ("backward1", "backward")]
+        assert np.array_equal(qb.quantized_recv_data_buf.cpu().numpy(), q_back[r][0])
+        assert np.array_equal(gr.comm_buf.send_buf.cpu().numpy(), incoming[r])
+        o_dx = oagg.backward_out(o["local"], o["a_to"], np.ascontiguousarray(g[sl[r]]), incoming[r])
+        assert np.array_equal(xr.grad.cpu().numpy(), o_dx)
+        # 8-bit rows: within a few 1e-2 of the exact product (sum of <= half-step errors)
+        if bits == 8:
+            assert np.abs(out.detach().cpu().numpy() - want[sl[r]]).max() < 0.5
+            assert np.abs(xr.grad.cpu().numpy() - want_t[sl[r]]).max() < 0.5
+
+    # outside training the forward exchange carries fp32 rows (communicator.py:64-65)
+    gr = graphs[0]
+    exact = host_exchange(o_send, send_splits, recv_splits)
+    gr.exchange = PlayedExchange(dev(exact[0]), None)
+    gr.exchange_quantized = lambda *a: (_ for _ in ()).throw(AssertionError("quantised exchange used outside training"))
+    out = Aggregator.apply(gr, dev(x[sl[0]]), 1, bits, True, False)
+    assert np.array_equal(out.cpu().numpy(), oagg.forward_out(oracle_ranks[0]["local"], oracle_ranks[0]["a_from"],
+                                                              np.ascontiguousarray(x[sl[0]]), exact[0]))
+
+
+def test_quantised_run_needs_its_buffers_and_hook():
+    w = World(7, (40, 50), mean_deg=4.0)
+    graphs = _build_pre_graphs(w, 8)
+    graphs[0].exchange = PlayedExchange(None, None)
+    x = torch.zeros(40, 8, device="cuda")
+    with pytest.raises(RuntimeError, match="quantisation buffers"):
+        Aggregator.apply(graphs[0], x, 0, 2, True, True)
+    graphs2 = _build_pre_graphs(w, 8, bits=2)
+    graphs2[0].exchange = PlayedExchange(None, None)
+    with pytest.raises(RuntimeError, match="exchange_quantized"):
+        Aggregator.apply(graphs2[0], x, 0, 2, True, True)
+    with pytest.raises(NotImplementedError):
+        Aggregator.apply(graphs2[0], x, 0, 3, True, True)
