@@ -328,11 +328,77 @@ def run_c4(args, graph, setup_s):
         o.backward(g)
     torch.cuda.synchronize()
     both_ms = (time.perf_counter() - t0) * 1e3 / steps
-    return {"partition": f"rank 3 of 16, {n} local nodes", "feat": feat, "setup_s": round(setup_s, 2),
+    codec = run_c4_codec(graph, feat, steps, gen)
+    # the same autograd.Function with the boundary rows travelling as int2 (seeded packed rows)
+    from gnn_benchmark_amd import synthetic
+    from gnn_benchmark_amd.data_manager import CommBufferForQuantization, CommSplits
+
+    world = len(graph.comm_splits.send_splits)
+    fp32_splits = graph.comm_splits
+    graph.comm_splits = CommSplits(fp32_splits.recv_splits, fp32_splits.send_splits, world, 2)
+    graph.comm_buf_for_quantization = CommBufferForQuantization(graph.comm_splits, feat, 2, device=dev)
+    graph.exchange_quantized = synthetic.SeededQuantizedHaloExchange(args.seed + 6)
+    for _ in range(2):
+        Aggregator.apply(graph, xr, 0, 2, True, True).backward(g)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        o = Aggregator.apply(graph, xr, 0, 2, True, True)
+        o.backward(g)
+    torch.cuda.synchronize()
+    int2_both_ms = (time.perf_counter() - t0) * 1e3 / steps
+    graph.comm_splits, graph.comm_buf_for_quantization, graph.exchange_quantized = fp32_splits, None, None
+    return {"partition": f"rank 3 of 16, {n} local nodes", "feat": feat, "setup_s": round(setup_s, 2), "codec": codec,
             "local_nnz": graph.local_adj_t.nnz(), "halo_rows": int(recv_buf.size(0)), "send_rows": int(send_buf.size(0)),
             "from_nnz": graph.adj_t_pre_post_aggr_from.nnz(), "to_nnz": graph.adj_t_pre_post_aggr_to.nnz(),
             "ops": ops, "aggregator_forward_ms": round(fwd_ms, 3),
-            "aggregator_forward_backward_ms": round(both_ms, 3)}
+            "aggregator_forward_backward_ms": round(both_ms, 3),
+            "aggregator_forward_backward_ms_int2_exchange": round(int2_both_ms, 3)}
+
+
+def run_c4_codec(graph, feat, steps, gen):
+    """int2 codec of the partition's boundary buffers (one segment per peer rank): quantise the
+    send buffer, dequantise into the receive buffer.  Bytes: fp32 rows + packed rows + 8 B of
+    parameters per row, each moved once."""
+    import torch
+
+    from gnn_benchmark_amd import computation_ops as ops
+    from gnn_benchmark_amd.data_manager import CommBufferForQuantization, CommSplits
+
+    world = len(graph.comm_splits.send_splits)
+    out = []
+    for bits in (2, 8):
+        splits = CommSplits(graph.comm_splits.recv_splits, graph.comm_splits.send_splits, world, bits)
+        q = CommBufferForQuantization(splits, feat, bits, device=graph.comm_buf.send_buf.device)
+        send_buf, recv_buf = graph.comm_buf.send_buf, graph.comm_buf.recv_buf
+        send_buf.normal_(generator=gen)
+
+        def quantize():
+            ops.quantize_tensor_for_all_procs(send_buf, q.quantized_send_data_buf, q.quantized_send_params_buf_fp32,
+                                              q.quantized_work_range_per_proc, world, bits)
+
+        def dequantize():
+            ops.dequantize_tensor_for_all_procs(q.quantized_recv_data_buf, recv_buf, q.quantized_recv_params_buf_fp32,
+                                                q.dequantized_work_range_per_proc, world, bits)
+
+        for name, fn, rows, packed_rows in (("quantize send_buf", quantize, send_buf.size(0), q.quantized_send_data_buf.size(0)),
+                                            ("dequantize into recv_buf", dequantize, recv_buf.size(0),
+                                             q.quantized_recv_data_buf.size(0))):
+            for _ in range(2):
+                fn()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(steps):
+                fn()
+            e1.record()
+            e1.synchronize()
+            ms = e0.elapsed_time(e1) / steps
+            nbytes = rows * feat * 4.0 + packed_rows * feat + rows * 8.0
+            out.append({"op": name, "bits": bits, "rows": int(rows), "packed_rows": int(packed_rows), "feat": feat,
+                        "ms": round(ms, 4), "bytes": nbytes, "gbs": round(nbytes / ms / 1e6, 1),
+                        "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)})
+        del q
+    return out
 
 
 def run_c5(args, graph):

@@ -11,10 +11,11 @@
 // (1 when that is 0), q = rint((x - zero_point) / scale) to nearest even with an IEEE
 // division, x' = fma(q, scale, zero_point).
 //
-// All kernels stream: HBM-bound.  One lane group (16, 32 or 64 lanes, by row width) owns
-// one group of rows that share bytes; the rows are held in registers between the min/max
-// pass and the packing pass when they fit (F <= 1024), so the fp32 rows are read from
-// memory once.
+// All kernels stream: HBM-bound (quantise reads 4F + writes F*bits/8 + 8 bytes per row,
+// dequantise the reverse).  One lane group (16, 32 or 64 lanes, by row width) owns four fp32
+// rows at a time -- one, two or four groups of rows that share bytes; the rows are held in
+// registers between the min/max pass and the packing pass when they fit (F <= 1024), so the
+// fp32 rows are read from memory once.  The per-rank prefix arrays are staged in LDS.
 #include "common.h"
 
 namespace gnnagg {
@@ -71,6 +72,20 @@ __device__ __forceinline__ uint32_t quantize_one(float x, float zp, float scale)
     return (uint32_t)__float2int_rn(__fdiv_rn(__fsub_rn(x, zp), scale));
 }
 
+// The same value without an IEEE division per element.  t = d * rcp(scale) lies within 2.4e-7 * |t|
+// of the correctly rounded quotient fl(d / scale) (v_rcp_f32 is good to 1 ulp, the product adds
+// half an ulp, fl() itself another half).  Unless t comes closer than that to a half-integer, t
+// and fl(d / scale) round to the same integer; the rare close calls (and anything huge or not
+// finite) take the exact division.
+__device__ __forceinline__ uint32_t quantize_one_fast(float x, float zp, float scale, float inv_scale) {
+    const float d = __fsub_rn(x, zp);
+    const float t = __fmul_rn(d, inv_scale);
+    float k = rintf(t);
+    const float gap = 0.5f - fabsf(__fsub_rn(t, k));
+    if (!(fabsf(t) < 1.0e6f) || gap <= 4.0e-7f * fabsf(t) + 1.0e-30f) k = rintf(__fdiv_rn(d, scale));
+    return (uint32_t)(int)k;
+}
+
 __device__ __forceinline__ void params_of(float lo, float hi, int bits, float &zp, float &scale) {
     zp = lo;
     scale = __fdiv_rn(__fsub_rn(hi, lo), (float)((1 << bits) - 1));
@@ -78,7 +93,7 @@ __device__ __forceinline__ void params_of(float lo, float hi, int bits, float &z
 }
 
 // Which segment a packed row belongs to: the last p with packed_range[p] <= g.
-__device__ __forceinline__ int segment_of(const int32_t *__restrict__ packed_range, int segments, int g) {
+__device__ __forceinline__ int segment_of(const int32_t *packed_range, int segments, int g) {
     int lo = 0, hi = segments;  // invariant: packed_range[lo] <= g < packed_range[hi]
     while (hi - lo > 1) {
         const int mid = (lo + hi) >> 1;
@@ -94,9 +109,9 @@ struct RowGroup {
 };
 
 template <int EPB>
-__device__ __forceinline__ RowGroup locate_group(const int32_t *__restrict__ row_range,
-                                                 const int32_t *__restrict__ packed_range, int segments, int g,
-                                                 int rows) {
+__device__ __forceinline__ RowGroup locate_group(const int32_t *row_range, const int32_t *packed_range, int segments,
+                                                 int g, int rows, int packed_rows) {
+    if (g >= packed_rows) return RowGroup{0, 0};
     const int p = segment_of(packed_range, segments, g);
     const int first = row_range[p] + (g - packed_range[p]) * EPB;
     int end = row_range[p + 1];
@@ -107,7 +122,35 @@ __device__ __forceinline__ RowGroup locate_group(const int32_t *__restrict__ row
     return RowGroup{first, count};
 }
 
-// NV = float vectors a lane keeps per row between the two passes (0: rows are read twice).
+constexpr int kCodecIters = 8;         // slices a lane group walks per launch
+constexpr int kRowsPerLaneGroup = 4;   // fp32 rows one lane group handles, whatever the width
+constexpr int kMaxLdsSegments = 4095;  // both prefix arrays of up to this many segments are staged in LDS
+
+// The per-rank prefix arrays are searched by every lane group; a block copies them into LDS
+// once (when they fit) so that the search costs no chain of global-memory round trips.
+__device__ __forceinline__ void stage_ranges(const int32_t *__restrict__ row_range,
+                                             const int32_t *__restrict__ packed_range, int segments, int32_t *lds,
+                                             const int32_t *&rr, const int32_t *&pr) {
+    if (segments <= kMaxLdsSegments) {
+        for (int i = (int)threadIdx.x; i <= segments; i += 256) {
+            lds[i] = row_range[i];
+            lds[segments + 1 + i] = packed_range[i];
+        }
+        __syncthreads();
+        rr = lds;
+        pr = lds + segments + 1;
+    } else {
+        rr = row_range;
+        pr = packed_range;
+    }
+}
+
+// One lane group of G lanes handles GPL = kRowsPerLaneGroup / EPB consecutive packed rows at a
+// time, i.e. the same number of fp32 rows whatever the width, and walks kCodecIters such slices of
+// its block's share: the rows of the next slice are loaded before the current slice is reduced,
+// packed and stored, so loads stay in flight throughout.
+// NV = float vectors a lane keeps per row between the two passes (0: rows are read twice, no
+// prefetch).
 template <int BITS, int VEC, int G, int NV>
 __global__ __launch_bounds__(256) void quantize_segments_kernel(const float *__restrict__ x, uint8_t *__restrict__ packed,
                                                                 float *__restrict__ params,
@@ -115,79 +158,140 @@ __global__ __launch_bounds__(256) void quantize_segments_kernel(const float *__r
                                                                 const int32_t *__restrict__ packed_range, int segments,
                                                                 int rows, int packed_rows, int feat) {
     constexpr int EPB = 8 / BITS;
+    constexpr int GPL = kRowsPerLaneGroup / EPB;
     constexpr int KEEP = NV > 0 ? NV : 1;
-    const int g = (int)(((int64_t)blockIdx.x * 256 + threadIdx.x) / G);
-    if (g >= packed_rows) return;  // whole lane groups leave together
+    constexpr int kLaneGroups = 256 / G;
+    constexpr bool kPrefetch = NV == 1;  // two slices of rows in registers
+    extern __shared__ int32_t range_lds[];
+    const int32_t *rr, *pr;
+    stage_ranges(row_range, packed_range, segments, range_lds, rr, pr);
+
     const int l = (int)threadIdx.x & (G - 1);
-    const RowGroup rg = locate_group<EPB>(row_range, packed_range, segments, g, rows);
     const int nvec = (feat + VEC - 1) / VEC;  // VEC == 4 implies feat % 4 == 0
 
-    QVec<VEC> held[EPB][KEEP];
-    float zp[EPB], scale[EPB];
+    struct Slice {
+        int g0;
+        RowGroup rg[GPL];
+        QVec<VEC> held[GPL][EPB][KEEP];
+    };
+    auto slice_start = [&](int it) {
+        return (int)((((int64_t)blockIdx.x * kCodecIters + it) * kLaneGroups + (int)threadIdx.x / G) * GPL);
+    };
+    // locate the slice's rows and (NV > 0) issue their loads
+    auto fetch = [&](int it, Slice &sl) {
+        sl.g0 = slice_start(it);
 #pragma unroll
-    for (int k = 0; k < EPB; ++k) {
-        zp[k] = 0.0f;
-        scale[k] = 1.0f;
-        if (k < rg.count) {
-            const float *row = x + (size_t)(rg.first + k) * (size_t)feat;
-            float lo = INFINITY, hi = -INFINITY;
+        for (int u = 0; u < GPL; ++u) sl.rg[u] = locate_group<EPB>(rr, pr, segments, sl.g0 + u, rows, packed_rows);
+        if (NV > 0) {
+#pragma unroll
+            for (int u = 0; u < GPL; ++u)
+#pragma unroll
+                for (int k = 0; k < EPB; ++k)
+                    if (k < sl.rg[u].count) {
+                        const float *row = x + (size_t)(sl.rg[u].first + k) * (size_t)feat;
+#pragma unroll
+                        for (int j = 0; j < KEEP; ++j) {
+                            const int v = l + G * j;
+                            if (v < nvec) sl.held[u][k][j] = QVec<VEC>::load(row + (size_t)v * VEC);
+                        }
+                    }
+        }
+    };
+    auto process = [&](const Slice &sl) {
+        float zp[GPL][EPB], scale[GPL][EPB], inv[GPL][EPB];
+#pragma unroll
+        for (int u = 0; u < GPL; ++u)
+#pragma unroll
+            for (int k = 0; k < EPB; ++k) {
+                zp[u][k] = 0.0f;
+                scale[u][k] = 1.0f;
+                inv[u][k] = 1.0f;
+                if (k < sl.rg[u].count) {
+                    float lo = INFINITY, hi = -INFINITY;
+                    if (NV > 0) {
+#pragma unroll
+                        for (int j = 0; j < KEEP; ++j) {
+                            if (l + G * j < nvec) {
+#pragma unroll
+                                for (int e = 0; e < VEC; ++e) {
+                                    lo = fminf(lo, sl.held[u][k][j].get(e));
+                                    hi = fmaxf(hi, sl.held[u][k][j].get(e));
+                                }
+                            }
+                        }
+                    } else {
+                        const float *row = x + (size_t)(sl.rg[u].first + k) * (size_t)feat;
+                        for (int v = l; v < nvec; v += G) {
+                            const QVec<VEC> t = QVec<VEC>::load(row + (size_t)v * VEC);
+#pragma unroll
+                            for (int e = 0; e < VEC; ++e) {
+                                lo = fminf(lo, t.get(e));
+                                hi = fmaxf(hi, t.get(e));
+                            }
+                        }
+                    }
+                    group_min_max<G>(lo, hi);
+                    params_of(lo, hi, BITS, zp[u][k], scale[u][k]);
+                    inv[u][k] = __builtin_amdgcn_rcpf(scale[u][k]);
+                    if (l == 0) {
+                        const float2 zs = make_float2(zp[u][k], scale[u][k]);
+                        *reinterpret_cast<float2 *>(params + (size_t)(sl.rg[u].first + k) * 2) = zs;
+                    }
+                }
+            }
+#pragma unroll
+        for (int u = 0; u < GPL; ++u) {
+            if (sl.g0 + u >= packed_rows) continue;
+            uint8_t *dst = packed + (size_t)(sl.g0 + u) * (size_t)feat;
+            auto pack = [&](int v, int j) {
+                uint32_t byte[VEC];
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) byte[e] = 0;
+#pragma unroll
+                for (int k = 0; k < EPB; ++k) {
+                    if (k < sl.rg[u].count) {
+                        QVec<VEC> t;
+                        if (NV > 0) t = sl.held[u][k][j];
+                        else t = QVec<VEC>::load(x + (size_t)(sl.rg[u].first + k) * (size_t)feat + (size_t)v * VEC);
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e)
+                            byte[e] |= quantize_one_fast(t.get(e), zp[u][k], scale[u][k], inv[u][k])
+                                       << ((EPB - k - 1) * BITS);
+                    }
+                }
+                QVec<VEC>::store_bytes(dst + (size_t)v * VEC, byte);
+            };
             if (NV > 0) {
 #pragma unroll
                 for (int j = 0; j < KEEP; ++j) {
                     const int v = l + G * j;
-                    if (v < nvec) {
-                        held[k][j] = QVec<VEC>::load(row + (size_t)v * VEC);
-#pragma unroll
-                        for (int e = 0; e < VEC; ++e) {
-                            lo = fminf(lo, held[k][j].get(e));
-                            hi = fmaxf(hi, held[k][j].get(e));
-                        }
-                    }
+                    if (v < nvec) pack(v, j);
                 }
             } else {
-                for (int v = l; v < nvec; v += G) {
-                    const QVec<VEC> t = QVec<VEC>::load(row + (size_t)v * VEC);
-#pragma unroll
-                    for (int e = 0; e < VEC; ++e) {
-                        lo = fminf(lo, t.get(e));
-                        hi = fmaxf(hi, t.get(e));
-                    }
-                }
-            }
-            group_min_max<G>(lo, hi);
-            params_of(lo, hi, BITS, zp[k], scale[k]);
-            if (l == 0) {
-                params[(size_t)(rg.first + k) * 2 + 0] = zp[k];
-                params[(size_t)(rg.first + k) * 2 + 1] = scale[k];
+                for (int v = l; v < nvec; v += G) pack(v, 0);
             }
         }
-    }
-
-    uint8_t *dst = packed + (size_t)g * (size_t)feat;
-    auto pack = [&](int v, int j) {
-        uint32_t byte[VEC];
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) byte[e] = 0;
-#pragma unroll
-        for (int k = 0; k < EPB; ++k) {
-            if (k < rg.count) {
-                QVec<VEC> t;
-                if (NV > 0) t = held[k][j];
-                else t = QVec<VEC>::load(x + (size_t)(rg.first + k) * (size_t)feat + (size_t)v * VEC);
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) byte[e] |= quantize_one(t.get(e), zp[k], scale[k]) << ((EPB - k - 1) * BITS);
-            }
-        }
-        QVec<VEC>::store_bytes(dst + (size_t)v * VEC, byte);
     };
-    if (NV > 0) {
-#pragma unroll
-        for (int j = 0; j < KEEP; ++j) {
-            const int v = l + G * j;
-            if (v < nvec) pack(v, j);
+
+    // Whole lane groups leave together, and no barrier follows the staging above.
+    if (kPrefetch) {
+        Slice cur, nxt;
+        if (slice_start(0) >= packed_rows) return;
+        fetch(0, cur);
+        for (int it = 0; it < kCodecIters; ++it) {
+            const bool more = it + 1 < kCodecIters && slice_start(it + 1) < packed_rows;
+            if (more) fetch(it + 1, nxt);
+            process(cur);
+            if (!more) break;
+            cur = nxt;
         }
     } else {
-        for (int v = l; v < nvec; v += G) pack(v, 0);
+        for (int it = 0; it < kCodecIters; ++it) {
+            if (slice_start(it) >= packed_rows) break;
+            Slice cur;
+            fetch(it, cur);
+            process(cur);
+        }
     }
 }
 
@@ -199,36 +303,53 @@ __global__ __launch_bounds__(256) void dequantize_segments_kernel(const uint8_t 
                                                                   const int32_t *__restrict__ packed_range,
                                                                   int segments, int rows, int packed_rows, int feat) {
     constexpr int EPB = 8 / BITS;
+    constexpr int GPL = kRowsPerLaneGroup / EPB;
     constexpr uint32_t kMask = (1u << BITS) - 1u;
-    const int g = (int)(((int64_t)blockIdx.x * 256 + threadIdx.x) / G);
-    if (g >= packed_rows) return;
+    extern __shared__ int32_t range_lds[];
+    const int32_t *rr, *pr;
+    stage_ranges(row_range, packed_range, segments, range_lds, rr, pr);
+
+    // a lane group walks kCodecIters slices of the block's share, so that the staging above is paid once
+    constexpr int kLaneGroups = 256 / G;
+    for (int it = 0; it < kCodecIters; ++it) {
+    const int g0 = (int)((((int64_t)blockIdx.x * kCodecIters + it) * kLaneGroups + (int)threadIdx.x / G) * GPL);
+    if (g0 >= packed_rows) break;  // whole lane groups leave together; no barrier follows
     const int l = (int)threadIdx.x & (G - 1);
-    const RowGroup rg = locate_group<EPB>(row_range, packed_range, segments, g, rows);
     const int nvec = (feat + VEC - 1) / VEC;
-    float zp[EPB], scale[EPB];
+    RowGroup rg[GPL];
+    float zp[GPL][EPB], scale[GPL][EPB];
 #pragma unroll
-    for (int k = 0; k < EPB; ++k) {
-        zp[k] = 0.0f;
-        scale[k] = 0.0f;
-        if (k < rg.count) {
-            zp[k] = params[(size_t)(rg.first + k) * 2 + 0];
-            scale[k] = params[(size_t)(rg.first + k) * 2 + 1];
-        }
-    }
-    const uint8_t *src = packed + (size_t)g * (size_t)feat;
-    for (int v = l; v < nvec; v += G) {
-        uint32_t byte[VEC];
-        QVec<VEC>::load_bytes(src + (size_t)v * VEC, byte);
+    for (int u = 0; u < GPL; ++u) {
+        rg[u] = locate_group<EPB>(rr, pr, segments, g0 + u, rows, packed_rows);
 #pragma unroll
         for (int k = 0; k < EPB; ++k) {
-            if (k < rg.count) {
-                float o[VEC];
-#pragma unroll
-                for (int e = 0; e < VEC; ++e)
-                    o[e] = __fmaf_rn((float)((byte[e] >> ((EPB - k - 1) * BITS)) & kMask), scale[k], zp[k]);
-                QVec<VEC>::store(out + (size_t)(rg.first + k) * (size_t)feat + (size_t)v * VEC, o);
+            zp[u][k] = 0.0f;
+            scale[u][k] = 0.0f;
+            if (k < rg[u].count) {
+                const float2 zs = *reinterpret_cast<const float2 *>(params + (size_t)(rg[u].first + k) * 2);
+                zp[u][k] = zs.x;
+                scale[u][k] = zs.y;
             }
         }
+    }
+    for (int v = l; v < nvec; v += G) {
+        uint32_t byte[GPL][VEC];
+#pragma unroll
+        for (int u = 0; u < GPL; ++u)
+            if (rg[u].count > 0) QVec<VEC>::load_bytes(packed + (size_t)(g0 + u) * (size_t)feat + (size_t)v * VEC, byte[u]);
+#pragma unroll
+        for (int u = 0; u < GPL; ++u)
+#pragma unroll
+            for (int k = 0; k < EPB; ++k) {
+                if (k < rg[u].count) {
+                    float o[VEC];
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e)
+                        o[e] = __fmaf_rn((float)((byte[u][e] >> ((EPB - k - 1) * BITS)) & kMask), scale[u][k], zp[u][k]);
+                    QVec<VEC>::store(out + (size_t)(rg[u].first + k) * (size_t)feat + (size_t)v * VEC, o);
+                }
+            }
+    }
     }
 }
 
@@ -307,19 +428,28 @@ struct SegArgs {
     hipStream_t st;
 };
 
+// packed rows handled by one lane group
+constexpr int groups_per_lane_group(int bits) { return kRowsPerLaneGroup / (8 / bits); }
+
+size_t range_lds_bytes(int segments) {
+    return segments <= kMaxLdsSegments ? 2 * (size_t)(segments + 1) * sizeof(int32_t) : 0;
+}
+
 template <int BITS, int VEC, int G>
 void launch_quantize(const float *x, uint8_t *packed, float *params, const SegArgs &a) {
     const int nvec = (a.feat + VEC - 1) / VEC;
-    const unsigned blocks = grid_for((int64_t)a.packed_rows * G, 256);
+    constexpr int gpl = groups_per_lane_group(BITS);
+    const unsigned blocks = grid_for(((int64_t)a.packed_rows + gpl - 1) / gpl * G, 256 * kCodecIters);
+    const size_t lds = range_lds_bytes(a.segments);
     if (nvec <= G)
-        hipLaunchKernelGGL((quantize_segments_kernel<BITS, VEC, G, 1>), dim3(blocks), dim3(256), 0, a.st, x, packed, params,
-                           a.row_range, a.packed_range, a.segments, a.rows, a.packed_rows, a.feat);
+        hipLaunchKernelGGL((quantize_segments_kernel<BITS, VEC, G, 1>), dim3(blocks), dim3(256), lds, a.st, x, packed,
+                           params, a.row_range, a.packed_range, a.segments, a.rows, a.packed_rows, a.feat);
     else if (nvec <= 4 * G)
-        hipLaunchKernelGGL((quantize_segments_kernel<BITS, VEC, G, 4>), dim3(blocks), dim3(256), 0, a.st, x, packed, params,
-                           a.row_range, a.packed_range, a.segments, a.rows, a.packed_rows, a.feat);
+        hipLaunchKernelGGL((quantize_segments_kernel<BITS, VEC, G, 4>), dim3(blocks), dim3(256), lds, a.st, x, packed,
+                           params, a.row_range, a.packed_range, a.segments, a.rows, a.packed_rows, a.feat);
     else
-        hipLaunchKernelGGL((quantize_segments_kernel<BITS, VEC, G, 0>), dim3(blocks), dim3(256), 0, a.st, x, packed, params,
-                           a.row_range, a.packed_range, a.segments, a.rows, a.packed_rows, a.feat);
+        hipLaunchKernelGGL((quantize_segments_kernel<BITS, VEC, G, 0>), dim3(blocks), dim3(256), lds, a.st, x, packed,
+                           params, a.row_range, a.packed_range, a.segments, a.rows, a.packed_rows, a.feat);
 }
 
 template <int BITS, int VEC>
@@ -333,10 +463,13 @@ void launch_quantize_g(const float *x, uint8_t *packed, float *params, const Seg
 template <int BITS, int VEC>
 void launch_dequantize_g(const uint8_t *packed, const float *params, float *out, const SegArgs &a) {
     const int nvec = (a.feat + VEC - 1) / VEC;
-#define GNNAGG_DEQ(G)                                                                                              \
-    hipLaunchKernelGGL((dequantize_segments_kernel<BITS, VEC, G>), dim3(grid_for((int64_t)a.packed_rows * G, 256)), \
-                       dim3(256), 0, a.st, packed, params, out, a.row_range, a.packed_range, a.segments, a.rows,   \
-                       a.packed_rows, a.feat)
+    constexpr int gpl = groups_per_lane_group(BITS);
+    const int64_t lane_groups = ((int64_t)a.packed_rows + gpl - 1) / gpl;
+    const size_t lds = range_lds_bytes(a.segments);
+#define GNNAGG_DEQ(G)                                                                                            \
+    hipLaunchKernelGGL((dequantize_segments_kernel<BITS, VEC, G>),                                               \
+                       dim3(grid_for(lane_groups * G, 256 * kCodecIters)), dim3(256), lds, a.st, packed, params, \
+                       out, a.row_range, a.packed_range, a.segments, a.rows, a.packed_rows, a.feat)
     if (nvec <= 16) GNNAGG_DEQ(16);
     else if (nvec <= 32) GNNAGG_DEQ(32);
     else GNNAGG_DEQ(64);

@@ -204,8 +204,33 @@ class SeededHaloExchange:
         return None
 
 
+class SeededQuantizedHaloExchange:
+    """Quantised counterpart of SeededHaloExchange: the packed rows and the (zero_point, scale)
+    rows a real exchange would have delivered are seeded random bytes and seeded parameters
+    (already rounded through bf16, as they are on the wire), generated on the device."""
+
+    def __init__(self, seed: int = 0):
+        self.seed = seed
+        self._gen = None
+        self.calls: List[str] = []
+
+    def __call__(self, comm_splits, qbuf, tag: str, direction: str):
+        data = qbuf.quantized_recv_data_buf if direction == "forward" else qbuf.quantized_send_data_buf
+        params = qbuf.quantized_recv_params_buf_fp32 if direction == "forward" else qbuf.quantized_send_params_buf_fp32
+        if self._gen is None or self._gen.device != data.device:
+            self._gen = torch.Generator(device=data.device)
+        self._gen.manual_seed(self.seed * 1000003 + 7 + sum(ord(c) * (i + 1) for i, c in enumerate(tag)))
+        data.random_(0, 256, generator=self._gen)
+        params.normal_(generator=self._gen)
+        params[:, 1].abs_().add_(0.05)
+        params.copy_(params.to(torch.bfloat16))
+        self.calls.append(tag)
+        return None
+
+
 def build_partition_graph(part: PartitionData, max_feat_len: int, is_pre_delay: bool,
-                          exchange: Optional[Callable] = None, bits: int = 32, device="cuda"):
+                          exchange: Optional[Callable] = None, bits: int = 32, device="cuda",
+                          exchange_quantized: Optional[Callable] = None):
     """DistributedGraphForPre (pre/post-aggregation) or DistributedGraph (raw halo rows) of
     one synthetic partition."""
     local_edges = part.local_edges.clone()
@@ -213,7 +238,8 @@ def build_partition_graph(part: PartitionData, max_feat_len: int, is_pre_delay: 
     if is_pre_delay:
         return get_distributed_graph_for_pre_aggressive(
             local_edges, remote_edges, part.begins, part.num_local_nodes, max_feat_len, part.rank, part.world_size,
-            bits, graph_exchange=mirrored_graph_exchange(part), exchange=exchange, device=device)
+            bits, graph_exchange=mirrored_graph_exchange(part), exchange=exchange,
+            exchange_quantized=exchange_quantized, device=device)
     begin = int(part.begins[part.rank])
     local_nodes_list = torch.stack((torch.arange(begin, begin + part.num_local_nodes), ) * 2, dim=1)
 
@@ -228,4 +254,4 @@ def build_partition_graph(part: PartitionData, max_feat_len: int, is_pre_delay: 
 
     return get_distributed_graph(local_edges, remote_edges, local_nodes_list, part.begins, part.num_local_nodes,
                                  max_feat_len, part.world_size, bits, halo_id_exchange=halo_id_exchange,
-                                 exchange=exchange, device=device)
+                                 exchange=exchange, exchange_quantized=exchange_quantized, device=device)
