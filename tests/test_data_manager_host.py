@@ -328,3 +328,45 @@ def test_partition_files_round_trip(tmp_path):
     for m1, m2 in ((a.local_adj_t, b.local_adj_t), (a.adj_t_pre_post_aggr_from, b.adj_t_pre_post_aggr_from),
                    (a.adj_t_pre_post_aggr_to, b.adj_t_pre_post_aggr_to)):
         assert all(torch.equal(x, y) for x, y in zip(m1.csr(), m2.csr()))
+
+
+def test_quantised_exchange_buffers_and_splits_follow_the_reference_layout():
+    """data_manager/CommSplits.py:11-19, CommBuffer.py:27-49 and quantizer.py:47-50, :69-77, :94-95 of the
+    reference: packed rows per rank, buffer shapes and per-rank row prefixes."""
+    from gnn_benchmark_amd.data_manager import CommBuffer, CommBufferForQuantization, CommSplits
+    from gnn_benchmark_amd.quantizer import QuantizerForMixedBits, QuantizerForPureBits, Quantizer_for_all_procs
+    from oracle import quantization as oq
+
+    recv, send = [3, 0, 6, 2], [1, 5, 0, 4]
+    for bits, per in ((2, 4), (4, 2), (8, 1)):
+        cs = CommSplits(recv, send, 4, bits)
+        assert cs.recv_splits_int2 == [-(-r // per) for r in recv] == [oq.get_quantized_splits(r, bits) for r in recv]
+        assert cs.send_splits_int2 == [-(-s // per) for s in send]
+        q = Quantizer_for_all_procs(4, bits)
+        assert Quantizer_for_all_procs.ctx is q
+        assert [q.get_quantized_splits(r) for r in recv] == cs.recv_splits_int2
+        buf = CommBufferForQuantization(cs, 16, bits)
+        assert buf.quantized_send_data_buf.shape == (sum(cs.send_splits_int2), 16) and buf.quantized_send_data_buf.dtype == torch.uint8
+        assert buf.quantized_recv_data_buf.shape == (sum(cs.recv_splits_int2), 16)
+        assert buf.quantized_send_params_buf_fp32.shape == (10, 2) and buf.quantized_recv_params_buf_fp32.shape == (11, 2)
+        assert buf.quantized_send_params_buf_bf16.dtype == torch.bfloat16
+        assert buf.quantized_work_range_per_proc.tolist() == [0, 1, 6, 6, 10]
+        assert buf.dequantized_work_range_per_proc.tolist() == [0, 3, 3, 9, 11]
+        assert buf.quantized_work_range_per_proc.dtype == torch.int32
+        rows, packed = oq.segment_ranges(send, bits)
+        assert rows.tolist() == [0, 1, 6, 6, 10] and packed[-1] == sum(cs.send_splits_int2)
+        buf.resize_buffer(cs, 8, bits)
+        assert buf.quantized_send_data_buf.shape == (sum(cs.send_splits_int2), 8)
+        assert QuantizerForPureBits.get_quantized_buffer_size(10, bits, 16) == -(-10 // per) * 16
+    # fp32 / bf16 runs carry no packed splits
+    assert not hasattr(CommSplits(recv, send, 4, 32), "recv_splits_int2")
+    assert CommBuffer(CommSplits(recv, send, 4, 16), 8, 16).send_buf_fp16.dtype == torch.bfloat16
+    with pytest.raises(NotImplementedError):
+        CommSplits(recv, send, 4, 3)
+    with pytest.raises(ValueError):
+        Quantizer_for_all_procs(4, 3)
+    # tests/test_quantizer.py:29-56 of the reference
+    for n, f, bits_row, want in ((6, 4, [8, 4, 2, 8, 4, 2], [0, 4, 6, 7, 11, 13, 14]), (3, 1, [2, 2, 2], [0, 1, 2, 3]),
+                                 (3, 3, [4, 4, 2], [0, 2, 4, 5])):
+        got = QuantizerForMixedBits.get_quantized_nodes_feat_range(n, f, torch.tensor(bits_row))
+        assert got.dtype == torch.int64 and got.tolist() == want
