@@ -259,6 +259,29 @@ def test_full_size_properties_config2():
     _check_properties(g.adj, 100, 4000, seed=0)
 
 
+def test_full_size_properties_config3_dense_degree():
+    """The load-balance stress graph at full size (233 K nodes, ~115 M stored elements, mean
+    degree ~490, longest row in the tens of thousands), F=602 and 256.  Its values are
+    row-normalised (mean aggregation), which gives a closed form: every row holding elements
+    maps the all-ones operand to 1."""
+    from gnn_benchmark_amd.synthetic import dense_degree_graph
+
+    g = dense_degree_graph(num_nodes=233_000, mu=5.5, sigma=1.2, seed=0, device="cuda")
+    assert 100_000_000 < g.nnz < 130_000_000 and g.max_degree > 20_000
+    info = g.adj.get_plan().info()
+    assert info["max_row_len"] == g.max_degree
+    _check_properties(g.adj, 602, 1500, seed=3)
+    _check_properties(g.adj, 256, 1500, seed=4)
+    rowptr = g.adj.csr()[0]
+    ones = torch.ones(g.num_nodes, 8, device="cuda")
+    out = torch.empty(g.num_nodes, 8, device="cuda")
+    SPMM_forward(g.adj, ones, out, accumulate=False)
+    has = (rowptr[1:] > rowptr[:-1]).view(-1, 1).float()
+    # a chain of len terms 1/len: relative error <= len * 2^-24
+    assert float((out - has).abs().max()) <= 5e-3
+    assert float((out - has).abs().mean()) <= 1e-5
+
+
 def test_full_size_properties_config4_partition():
     """One partition at full size (7 M local nodes, ~100 M local and ~20 M boundary
     elements): the three matrices of the pre/post pipeline, F=128, and the pipeline itself
