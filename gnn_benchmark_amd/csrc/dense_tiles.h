@@ -1,0 +1,90 @@
+// Building blocks of the dense MFMA kernels: vector types, the chunk size of the LDS pipeline,
+// and the loader that copies a contiguous run of rows from global memory into an LDS tile
+// through registers.
+#pragma once
+
+#include "common.h"
+
+namespace gnnagg {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int kChunk = 16;    // rows per LDS stage
+constexpr int kLdsPad = 32;   // floats: shifts the second row of a k-pair onto the other half of the banks
+
+// One operand's share of the loader: thread t moves float4 number t + 256*j of the chunk.
+template <int NV, int LD>
+struct ChunkLoader {
+    int lds_off[NV];   // destination (floats) inside one LDS buffer, or -1 for a vector beyond the chunk
+    int src_off[NV];   // source offset (floats) from the start of the chunk, clamped to 0 when unused
+    floatx4 reg[NV];
+    int width;
+
+    __device__ void init(int tid, int w) {
+        width = w;
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            const int e = 4 * (tid + 256 * j);
+            const bool used = e < kChunk * w;
+            lds_off[j] = used ? (e / w) * LD + (e % w) : -1;
+            src_off[j] = used ? e : 0;
+        }
+    }
+    // all kChunk rows exist
+    __device__ void fetch(const float *chunk) {
+#pragma unroll
+        for (int j = 0; j < NV; ++j)
+            reg[j] = __builtin_nontemporal_load(reinterpret_cast<const floatx4 *>(chunk + src_off[j]));
+    }
+    // only `valid` floats exist; the rest of the chunk reads as zeros.  `aligned` is false when rows
+    // are not a whole number of float4 (then fetch() is never used either).
+    __device__ void fetch_tail(const float *chunk, int valid, bool aligned) {
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            floatx4 v = {0.f, 0.f, 0.f, 0.f};
+            const int e = src_off[j];
+            if (lds_off[j] >= 0) {
+                if (aligned) {
+                    if (e < valid) v = *reinterpret_cast<const floatx4 *>(chunk + e);
+                } else {
+                    if (e + 0 < valid) v.x = chunk[e + 0];
+                    if (e + 1 < valid) v.y = chunk[e + 1];
+                    if (e + 2 < valid) v.z = chunk[e + 2];
+                    if (e + 3 < valid) v.w = chunk[e + 3];
+                }
+            }
+            reg[j] = v;
+        }
+    }
+    // Steady-state store: unconditional, so that no load is tied to a branch; a vector beyond the
+    // chunk goes to the thread's own 16 bytes of `dump`.
+    __device__ void store_all(float *buf, float *dump) const {
+#pragma unroll
+        for (int j = 0; j < NV; ++j)
+            *reinterpret_cast<floatx4 *>(lds_off[j] >= 0 ? buf + lds_off[j] : dump) = reg[j];
+    }
+    __device__ void store(float *buf, bool aligned) const {
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            if (lds_off[j] < 0) continue;
+            if (aligned) {
+                *reinterpret_cast<floatx4 *>(buf + lds_off[j]) = reg[j];
+            } else {  // a float4 of the stream may straddle two rows
+                const int e = src_off[j];
+                const float v[4] = {reg[j].x, reg[j].y, reg[j].z, reg[j].w};
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    if (e + q < kChunk * width) buf[((e + q) / width) * LD + (e + q) % width] = v[q];
+            }
+        }
+    }
+};
+
+// Dynamic LDS beyond 64 KB has to be allowed per kernel and per device before the first launch.
+inline hipError_t allow_lds(const void *kernel, size_t bytes) {
+    if (bytes <= 64 * 1024) return hipSuccess;
+    return hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+}
+
+}  // namespace gnnagg
