@@ -328,7 +328,7 @@ def run_c4(args, graph, setup_s):
         o.backward(g)
     torch.cuda.synchronize()
     both_ms = (time.perf_counter() - t0) * 1e3 / steps
-    codec = run_c4_codec(graph, feat, steps, gen)
+    codec = run_c4_codec(graph, feat, steps, gen, cpu=not args.no_cpu_baseline)
     # the same autograd.Function with the boundary rows travelling as int2 (seeded packed rows)
     from gnn_benchmark_amd import synthetic
     from gnn_benchmark_amd.data_manager import CommBufferForQuantization, CommSplits
@@ -356,7 +356,43 @@ def run_c4(args, graph, setup_s):
             "aggregator_forward_backward_ms_int2_exchange": round(int2_both_ms, 3)}
 
 
-def run_c4_codec(graph, feat, steps, gen):
+def cpu_time_codec(x_host, bits, reps=2):
+    """Median seconds of the reference's compiled row-packed quantise / dequantise kernels on the
+    host cores (self_benchmark/a64fx/model/ops/src/quantization_x86.cpp:17-162; the parameters,
+    which that variant takes as inputs, come from the oracle and are not timed), or None when
+    oracle/_ref is not loadable."""
+    import torch
+
+    from oracle import quantization as oq
+    from oracle import spmm as ospmm
+
+    ref = ospmm.load_reference_op()
+    if ref is None:
+        return None
+    threads = ospmm.max_threads()
+    torch.set_num_threads(threads)
+    rows, feat = x_host.shape
+    params = oq.row_params(x_host, bits)
+    x = torch.from_numpy(x_host)
+    lo, scale = torch.from_numpy(params[:, 0].copy()), torch.from_numpy(params[:, 1].copy())
+    packed = torch.zeros((-(-rows // (8 // bits)), feat), dtype=torch.uint8)
+    back = torch.empty_like(x)
+    out = {}
+    for name, run in (("quantize", lambda: ref.quantize_tensor(x, packed, lo, scale, bits)),
+                      ("dequantize", lambda: ref.dequantize_tensor(packed, back, lo, scale, bits))):
+        run()
+        times = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            run()
+            times.append(time.perf_counter() - t0)
+        times.sort()
+        out[name] = times[len(times) // 2]
+    out["threads"] = threads
+    return out
+
+
+def run_c4_codec(graph, feat, steps, gen, cpu=False):
     """int2 codec of the partition's boundary buffers (one segment per peer rank): quantise the
     send buffer, dequantise into the receive buffer.  Bytes: fp32 rows + packed rows + 8 B of
     parameters per row, each moved once."""
@@ -397,6 +433,13 @@ def run_c4_codec(graph, feat, steps, gen):
             out.append({"op": name, "bits": bits, "rows": int(rows), "packed_rows": int(packed_rows), "feat": feat,
                         "ms": round(ms, 4), "bytes": nbytes, "gbs": round(nbytes / ms / 1e6, 1),
                         "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)})
+        if cpu and bits == 2:
+            host = cpu_time_codec(send_buf.cpu().numpy(), bits)
+            if host is not None:
+                out[-2]["cpu_ms"] = round(host["quantize"] * 1e3, 1)
+                out[-1]["cpu_ms"] = round(host["dequantize"] * 1e3, 1)
+                out[-2]["cpu"] = out[-1]["cpu"] = (f"reference x86 kernel on the send buffer's {send_buf.size(0)} rows, "
+                                                   f"{host['threads']} threads")
         del q
     return out
 
