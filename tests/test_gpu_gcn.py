@@ -103,7 +103,7 @@ def test_train_step_matches_cpu_autograd(gemm, tol):
     cpu_loss = F.nll_loss(F.log_softmax(h, dim=1)[train_idx.cpu()], labels.cpu()[train_idx.cpu()])
     cpu_loss.backward()
 
-    assert abs(float(loss) - float(cpu_loss)) <= tol * max(1.0, abs(float(cpu_loss)))
+    assert abs(float(loss.detach()) - float(cpu_loss.detach())) <= tol * max(1.0, abs(float(cpu_loss)))
     for (name, p_gpu), p_cpu in zip(model.named_parameters(), cpu_model.parameters()):
         scale = float(p_cpu.grad.abs().max()) + 1e-12
         assert float((p_gpu.grad.cpu() - p_cpu.grad).abs().max()) <= 10 * tol * scale, name

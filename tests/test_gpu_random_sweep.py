@@ -1,0 +1,85 @@
+"""Seeded random sweep over shapes the hand-picked cases do not name: every SpMM path
+(plan, plan-less, transposed) and the row-packed codec, bit for bit against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from gnn_benchmark_amd import SPMM_backward, SPMM_forward
+from gnn_benchmark_amd import computation_ops as ops
+from gnn_benchmark_amd.sparse_tensor import SparseTensor
+from oracle import quantization as oq
+from oracle import spmm as ospmm
+
+pytestmark = pytest.mark.gpu
+
+WIDTHS = [1, 2, 3, 4, 5, 8, 12, 16, 31, 32, 33, 48, 64, 66, 100, 127, 128, 129, 172, 200, 256, 257, 300, 512, 513, 602,
+          700, 1024, 1100]
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _degrees(rng, rows):
+    kind = int(rng.integers(0, 4))
+    if kind == 0:
+        deg = rng.poisson(rng.uniform(0.2, 12), rows)
+    elif kind == 1:
+        deg = (rng.pareto(1.2, rows) * 3).astype(np.int64)
+    elif kind == 2:  # one very long row (block-per-row kernel above 8192)
+        deg = rng.poisson(2, rows)
+        deg[rng.integers(0, rows)] = int(rng.choice([300, 2000, 9000, 20000]))
+    else:            # mostly empty
+        deg = np.zeros(rows, np.int64)
+        deg[rng.integers(0, rows, max(1, rows // 10))] = rng.integers(1, 50)
+    return np.minimum(deg, 30000).astype(np.int64)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_shapes_match_oracle_bit_for_bit(seed):
+    rng = np.random.default_rng(9000 + seed)
+    for case in range(25):
+        rows = int(rng.choice([1, 2, 7, 63, 64, 65, 300, 1000, 5000]))
+        cols = int(rng.choice([1, 3, 64, 500, 4000]))
+        feat = int(rng.choice(WIDTHS))
+        deg = _degrees(rng, rows)
+        rowptr = np.concatenate(([0], np.cumsum(deg))).astype(np.int64)
+        nnz = int(rowptr[-1])
+        col = rng.integers(0, cols, nnz).astype(np.int64)
+        val = rng.standard_normal(nnz).astype(np.float32)
+        x = rng.standard_normal((cols, feat)).astype(np.float32)
+        out0 = rng.standard_normal((rows, feat)).astype(np.float32)
+        g = rng.standard_normal((rows, feat)).astype(np.float32)
+        dx0 = rng.standard_normal((cols, feat)).astype(np.float32)
+        acc = bool(rng.integers(0, 2))
+        what = dict(seed=seed, case=case, rows=rows, cols=cols, feat=feat, nnz=nnz, longest=int(deg.max()), acc=acc)
+
+        want = ospmm.spmm(rowptr, col, val, x, out0.copy() if acc else np.zeros_like(out0))
+        src = SparseTensor(rowptr=dev(rowptr), col=dev(col), value=dev(val), sparse_sizes=(rows, cols), is_sorted=True)
+        got = dev(out0)
+        SPMM_forward(src, dev(x), got, accumulate=acc)
+        assert np.array_equal(got.cpu().numpy(), want), ("plan", what)
+        got = dev(out0 if acc else np.zeros_like(out0))
+        ops.spmm(dev(rowptr), dev(col), dev(val), dev(x), got, rows, None, None)
+        assert np.array_equal(got.cpu().numpy(), want), ("plan-less", what)
+        want_t = ospmm.spmm_transposed(rowptr, col, val, g, dx0.copy() if acc else np.zeros_like(dx0), cols)
+        got = dev(dx0)
+        SPMM_backward(src, dev(g), got, accumulate=acc)
+        assert np.array_equal(got.cpu().numpy(), want_t), ("transposed", what)
+
+        bits = int(rng.choice([2, 4, 8]))
+        nseg = int(rng.integers(1, 9))
+        splits = rng.multinomial(rows, np.ones(nseg) / nseg).tolist()
+        xq = (rng.standard_normal((rows, feat)) * rng.uniform(1e-3, 1e3, (rows, 1))).astype(np.float32)
+        want_packed, want_params = oq.quantize_segments(xq, splits, bits)
+        work_range = torch.tensor(np.concatenate(([0], np.cumsum(splits))), dtype=torch.int32)
+        packed = torch.zeros(want_packed.shape, dtype=torch.uint8, device="cuda")
+        params = torch.zeros((rows, 2), device="cuda")
+        ops.quantize_tensor_for_all_procs(dev(xq), packed, params, work_range, nseg, bits)
+        assert np.array_equal(packed.cpu().numpy(), want_packed), ("packed bytes", what, bits, splits)
+        assert np.array_equal(params.cpu().numpy(), want_params), ("parameters", what, bits, splits)
+        wire = oq.params_over_the_wire(want_params)
+        back = torch.zeros((rows, feat), device="cuda")
+        ops.dequantize_tensor_for_all_procs(packed, back, dev(wire), work_range, nseg, bits)
+        want_back = oq.dequantize_segments(want_packed, wire, splits, bits)
+        assert np.array_equal(back.cpu().numpy().view(np.uint32), want_back.view(np.uint32)), ("dequantised", what, bits)
