@@ -32,6 +32,10 @@ EXPORTS = (
     "gnnagg_relu_dropout_backward_f32",
     "gnnagg_wgrad_workspace_bytes",
     "gnnagg_wgrad_f32",
+    "gnnagg_packed_header_words",
+    "gnnagg_bias_relu_dropout_pack_f32",
+    "gnnagg_relu_dropout_backward_packed_f32",
+    "gnnagg_plan_spmm_packed_f32",
     "gnnagg_quantize_segments_f32",
     "gnnagg_dequantize_segments_f32",
     "gnnagg_quantize_mixed_f32",
@@ -100,6 +104,14 @@ def lib() -> ctypes.CDLL:
     L.gnnagg_wgrad_workspace_bytes.argtypes = [i64, i64, i64]
     L.gnnagg_wgrad_f32.restype = i32
     L.gnnagg_wgrad_f32.argtypes = [vp, vp, vp, vp, i64, i64, i64, vp]
+    L.gnnagg_packed_header_words.restype = i32
+    L.gnnagg_packed_header_words.argtypes = [i64]
+    L.gnnagg_bias_relu_dropout_pack_f32.restype = i32
+    L.gnnagg_bias_relu_dropout_pack_f32.argtypes = [vp, vp, vp, vp, ctypes.c_float, vp, vp, i64, i64, vp]
+    L.gnnagg_relu_dropout_backward_packed_f32.restype = i32
+    L.gnnagg_relu_dropout_backward_packed_f32.argtypes = [vp, vp, vp, ctypes.c_float, vp, vp, i64, i64, vp]
+    L.gnnagg_plan_spmm_packed_f32.restype = i32
+    L.gnnagg_plan_spmm_packed_f32.argtypes = [vp, vp, vp, vp, vp, i64, i32, vp]
     L.gnnagg_quantize_segments_f32.restype = i32
     L.gnnagg_quantize_segments_f32.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp]
     L.gnnagg_dequantize_segments_f32.restype = i32

@@ -39,7 +39,7 @@ What differs from the reference, on purpose:
 """
 import torch
 
-from . import _lib, computation_ops
+from . import _lib, computation_ops, packed
 from .spmm_kernel import SPMM_backward, SPMM_forward
 
 
@@ -106,95 +106,143 @@ def _dequantize_received(graph, num_bits: int, direction: str) -> None:
         computation_ops.dequantize_tensor_for_all_procs(data, incoming, params, work_range, world, num_bits)
 
 
+class _DenseFeatures:
+    """The local features as the forward pipeline reads them: two products and a row gather."""
+
+    def __init__(self, feat: torch.Tensor):
+        self.feat = feat.contiguous()
+        self.width, self.device = feat.size(-1), feat.device
+
+    def product(self, adj, out, accumulate):
+        SPMM_forward(adj, self.feat, out, accumulate=accumulate)
+
+    def gather(self, index, out):
+        _gather_rows(self.feat, index, out)
+
+
+class _PackedFeatures:
+    """The same for features kept packed (non-zero values at the front of each row + header)."""
+
+    def __init__(self, values: torch.Tensor, header: torch.Tensor):
+        self.values, self.header = values, header
+        self.width, self.device = values.size(-1), values.device
+
+    def product(self, adj, out, accumulate):
+        packed.spmm(adj, self.values, self.header, out, accumulate=accumulate)
+
+    def gather(self, index, out):
+        raise NotImplementedError("raw boundary rows of packed features: use pre-aggregation (is_pre_delay=True)")
+
+
 class Aggregator(torch.autograd.Function):
     @staticmethod
     def forward(ctx, graph, local_nodes_feat, layer, num_bits: int, is_pre_delay: bool, is_training: bool):
-        _check_bits(num_bits)
-        ctx.graph = graph
-        ctx.num_bits = num_bits
-        ctx.is_pre_delay = is_pre_delay
-        ctx.layer = layer
-
-        feat_len = local_nodes_feat.size(-1)
-        local_nodes_feat = local_nodes_feat.contiguous()
-        graph.comm_buf.resize_buffer(graph.comm_splits, feat_len, num_bits)
-        exchange = getattr(graph, "exchange", None)
-        quantized = exchange is not None and _quantized(graph, num_bits)
-        if quantized:
-            graph.comm_buf_for_quantization.resize_buffer(graph.comm_splits, feat_len, num_bits)
-        quantized = quantized and is_training  # communicator.py:64-65: fp32 rows outside training
-        comm_handle = None
-        send_buf = graph.comm_buf.send_buf
-
-        if exchange is not None:
-            if is_pre_delay:  # pre-aggregation: send_buf = A_to @ X
-                SPMM_forward(graph.adj_t_pre_post_aggr_to, local_nodes_feat, send_buf, accumulate=False)
-            else:  # raw boundary rows
-                _gather_rows(local_nodes_feat, graph.idx_nodes_send_to_others, send_buf)
-            if quantized:
-                comm_handle = _quantize_and_exchange(graph, num_bits, f"forward{layer}", "forward")
-            else:
-                comm_handle = exchange(graph.comm_splits, graph.comm_buf, f"forward{layer}", "forward")
-
-        out = torch.empty([graph.local_adj_t.sparse_size(0), feat_len], dtype=torch.float32,
-                          device=local_nodes_feat.device)
-        SPMM_forward(graph.local_adj_t, local_nodes_feat, out, accumulate=False)
-
-        if comm_handle is not None:
-            comm_handle.wait()
-        if quantized:
-            _dequantize_received(graph, num_bits, "forward")
-
-        remote_nodes_feat = graph.comm_buf.recv_buf
-        if exchange is not None and remote_nodes_feat.size(0) != 0:
-            if is_pre_delay:  # post-aggregation
-                SPMM_forward(graph.adj_t_pre_post_aggr_from, remote_nodes_feat, out)
-            else:
-                SPMM_forward(graph.remote_adj_t, remote_nodes_feat, out)
-        return out
+        return _forward(ctx, graph, _DenseFeatures(local_nodes_feat), layer, num_bits, is_pre_delay, is_training)
 
     @staticmethod
     def backward(ctx, local_out_grad):
-        graph = ctx.graph
-        num_bits = ctx.num_bits
-        is_pre_delay = ctx.is_pre_delay
-        layer = f"backward{ctx.layer}"
+        return (None, _backward(ctx, local_out_grad), None, None, None, None)
 
-        local_out_grad = local_out_grad.contiguous()
-        feat_len = local_out_grad.size(-1)
-        graph.comm_buf.resize_buffer(graph.comm_splits, feat_len, num_bits)
-        exchange = getattr(graph, "exchange", None)
-        quantized = exchange is not None and _quantized(graph, num_bits)
+
+class AggregatorPacked(torch.autograd.Function):
+    """``Aggregator`` for features given packed (``packed.empty`` / the packing epilogue): the
+    forward products read only the non-zero values; the backward is the dense one, and its
+    result is the gradient with respect to the dense features the packed pair stands for."""
+
+    @staticmethod
+    def forward(ctx, graph, values, header, layer, num_bits: int, is_pre_delay: bool, is_training: bool):
+        return _forward(ctx, graph, _PackedFeatures(values, header), layer, num_bits, is_pre_delay, is_training)
+
+    @staticmethod
+    def backward(ctx, local_out_grad):
+        return (None, _backward(ctx, local_out_grad), None, None, None, None, None)
+
+
+def _forward(ctx, graph, feats, layer, num_bits: int, is_pre_delay: bool, is_training: bool):
+    _check_bits(num_bits)
+    ctx.graph = graph
+    ctx.num_bits = num_bits
+    ctx.is_pre_delay = is_pre_delay
+    ctx.layer = layer
+
+    feat_len = feats.width
+    graph.comm_buf.resize_buffer(graph.comm_splits, feat_len, num_bits)
+    exchange = getattr(graph, "exchange", None)
+    quantized = exchange is not None and _quantized(graph, num_bits)
+    if quantized:
+        graph.comm_buf_for_quantization.resize_buffer(graph.comm_splits, feat_len, num_bits)
+    quantized = quantized and is_training  # communicator.py:64-65: fp32 rows outside training
+    comm_handle = None
+    send_buf = graph.comm_buf.send_buf
+
+    if exchange is not None:
+        if is_pre_delay:  # pre-aggregation: send_buf = A_to @ X
+            feats.product(graph.adj_t_pre_post_aggr_to, send_buf, False)
+        else:  # raw boundary rows
+            feats.gather(graph.idx_nodes_send_to_others, send_buf)
         if quantized:
-            graph.comm_buf_for_quantization.resize_buffer(graph.comm_splits, feat_len, num_bits)
+            comm_handle = _quantize_and_exchange(graph, num_bits, f"forward{layer}", "forward")
+        else:
+            comm_handle = exchange(graph.comm_splits, graph.comm_buf, f"forward{layer}", "forward")
 
-        # the receive buffer carries the outgoing halo gradients on the way back
-        remote_nodes_grad_buf = graph.comm_buf.recv_buf
-        if remote_nodes_grad_buf.size(0) != 0:
-            if is_pre_delay:
-                SPMM_backward(graph.adj_t_pre_post_aggr_from, local_out_grad, remote_nodes_grad_buf, accumulate=False)
-            else:
-                SPMM_backward(graph.remote_adj_t, local_out_grad, remote_nodes_grad_buf, accumulate=False)
+    out = torch.empty([graph.local_adj_t.sparse_size(0), feat_len], dtype=torch.float32, device=feats.device)
+    feats.product(graph.local_adj_t, out, False)
 
-        comm_handle = None
-        if quantized:
-            comm_handle = _quantize_and_exchange(graph, num_bits, layer, "backward")
-        elif exchange is not None:
-            comm_handle = exchange(graph.comm_splits, graph.comm_buf, layer, "backward")
+    if comm_handle is not None:
+        comm_handle.wait()
+    if quantized:
+        _dequantize_received(graph, num_bits, "forward")
 
-        local_nodes_grad = torch.empty([graph.local_adj_t.sparse_size(-1), feat_len], dtype=torch.float32,
-                                       device=local_out_grad.device)
-        SPMM_backward(graph.local_adj_t, local_out_grad, local_nodes_grad, accumulate=False)
+    remote_nodes_feat = graph.comm_buf.recv_buf
+    if exchange is not None and remote_nodes_feat.size(0) != 0:
+        if is_pre_delay:  # post-aggregation
+            SPMM_forward(graph.adj_t_pre_post_aggr_from, remote_nodes_feat, out)
+        else:
+            SPMM_forward(graph.remote_adj_t, remote_nodes_feat, out)
+    return out
 
-        if comm_handle is not None:
-            comm_handle.wait()
-        if quantized:
-            _dequantize_received(graph, num_bits, "backward")
 
-        local_nodes_grad_buf = graph.comm_buf.send_buf
-        if exchange is not None and local_nodes_grad_buf.size(0) != 0:
-            if is_pre_delay:
-                SPMM_backward(graph.adj_t_pre_post_aggr_to, local_nodes_grad_buf, local_nodes_grad)
-            else:
-                SPMM_forward(graph.send_scatter_adj_t(), local_nodes_grad_buf, local_nodes_grad)
-        return None, local_nodes_grad, None, None, None, None
+def _backward(ctx, local_out_grad):
+    graph = ctx.graph
+    num_bits = ctx.num_bits
+    is_pre_delay = ctx.is_pre_delay
+    layer = f"backward{ctx.layer}"
+
+    local_out_grad = local_out_grad.contiguous()
+    feat_len = local_out_grad.size(-1)
+    graph.comm_buf.resize_buffer(graph.comm_splits, feat_len, num_bits)
+    exchange = getattr(graph, "exchange", None)
+    quantized = exchange is not None and _quantized(graph, num_bits)
+    if quantized:
+        graph.comm_buf_for_quantization.resize_buffer(graph.comm_splits, feat_len, num_bits)
+
+    # the receive buffer carries the outgoing halo gradients on the way back
+    remote_nodes_grad_buf = graph.comm_buf.recv_buf
+    if remote_nodes_grad_buf.size(0) != 0:
+        if is_pre_delay:
+            SPMM_backward(graph.adj_t_pre_post_aggr_from, local_out_grad, remote_nodes_grad_buf, accumulate=False)
+        else:
+            SPMM_backward(graph.remote_adj_t, local_out_grad, remote_nodes_grad_buf, accumulate=False)
+
+    comm_handle = None
+    if quantized:
+        comm_handle = _quantize_and_exchange(graph, num_bits, layer, "backward")
+    elif exchange is not None:
+        comm_handle = exchange(graph.comm_splits, graph.comm_buf, layer, "backward")
+
+    local_nodes_grad = torch.empty([graph.local_adj_t.sparse_size(-1), feat_len], dtype=torch.float32,
+                                   device=local_out_grad.device)
+    SPMM_backward(graph.local_adj_t, local_out_grad, local_nodes_grad, accumulate=False)
+
+    if comm_handle is not None:
+        comm_handle.wait()
+    if quantized:
+        _dequantize_received(graph, num_bits, "backward")
+
+    local_nodes_grad_buf = graph.comm_buf.send_buf
+    if exchange is not None and local_nodes_grad_buf.size(0) != 0:
+        if is_pre_delay:
+            SPMM_backward(graph.adj_t_pre_post_aggr_to, local_nodes_grad_buf, local_nodes_grad)
+        else:
+            SPMM_forward(graph.send_scatter_adj_t(), local_nodes_grad_buf, local_nodes_grad)
+    return local_nodes_grad

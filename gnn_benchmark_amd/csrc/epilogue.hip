@@ -88,12 +88,15 @@ __global__ __launch_bounds__(256) void relu_dropout_backward_kernel(const float 
 // gradient BEFORE the row division (that is d/d bias) is reduced over the threads of the
 // same column vector in a fixed order and written to bias_partial[b, :].  Needs
 // feat4 <= 256 and 256 % feat4 == 0.
+// PACKED: the forward output is not there as a dense tensor; which units were active comes from
+// the bitmap words of each row's header (hdr_words 32-bit words per row, bitmaps at the even ones).
+template <bool PACKED>
 __global__ __launch_bounds__(256) void relu_dropout_backward_rows_kernel(const f4 *__restrict__ g,
-                                                                         const f4 *__restrict__ y,
+                                                                         const void *__restrict__ y_or_hdr,
                                                                          const float *__restrict__ row_div, float scale,
                                                                          f4 *__restrict__ gz,
                                                                          f4 *__restrict__ bias_partial, int64_t rows,
-                                                                         int feat4, int rows_per_block) {
+                                                                         int feat4, int rows_per_block, int hdr_words) {
     __shared__ f4 sums[256];
     const int t = (int)threadIdx.x;
     const int c = t % feat4;
@@ -105,13 +108,27 @@ __global__ __launch_bounds__(256) void relu_dropout_backward_rows_kernel(const f
     for (int64_t r = r_begin + t / feat4; r < r_end; r += lanes) {
         const int64_t i = r * feat4 + c;
         const f4 gv = __builtin_nontemporal_load(g + i);
-        const f4 yv = __builtin_nontemporal_load(y + i);
+        bool on[4];
+        if (PACKED) {
+            const uint32_t w = static_cast<const uint32_t *>(y_or_hdr)[r * hdr_words + 2 * (c >> 3)];
+            const uint32_t nib = (w >> (4 * (c & 7))) & 15u;
+            on[0] = nib & 1u;
+            on[1] = nib & 2u;
+            on[2] = nib & 4u;
+            on[3] = nib & 8u;
+        } else {
+            const f4 yv = __builtin_nontemporal_load(static_cast<const f4 *>(y_or_hdr) + i);
+            on[0] = yv.x > 0.0f;
+            on[1] = yv.y > 0.0f;
+            on[2] = yv.z > 0.0f;
+            on[3] = yv.w > 0.0f;
+        }
         const float d = row_div ? row_div[r] : 1.0f;
         f4 pre;
-        pre.x = yv.x > 0.0f ? gv.x * scale : 0.0f;
-        pre.y = yv.y > 0.0f ? gv.y * scale : 0.0f;
-        pre.z = yv.z > 0.0f ? gv.z * scale : 0.0f;
-        pre.w = yv.w > 0.0f ? gv.w * scale : 0.0f;
+        pre.x = on[0] ? gv.x * scale : 0.0f;
+        pre.y = on[1] ? gv.y * scale : 0.0f;
+        pre.z = on[2] ? gv.z * scale : 0.0f;
+        pre.w = on[3] ? gv.w * scale : 0.0f;
         acc += pre;
         f4 out;
         out.x = pre.x / d;
@@ -126,6 +143,67 @@ __global__ __launch_bounds__(256) void relu_dropout_backward_rows_kernel(const f
         f4 total = sums[t];
         for (int k = 1; k < lanes; ++k) total += sums[t + k * feat4];
         bias_partial[(int64_t)blockIdx.x * feat4 + t] = total;
+    }
+}
+
+// ---- packed activations -----------------------------------------------------------------
+// The output of a ReLU + dropout layer is mostly zeros (about three in four in training).  A
+// row can be stored with its non-zero values moved to the front (order kept; the tail of the
+// row is left as it is) plus a small header: for every 32 features a pair of 32-bit words, the
+// bitmap of those features and the number of non-zeros in front of them.  The row stride stays
+// F, so no offsets are needed; a consumer that gathers such a row touches only the header
+// (64 bytes at F = 256) and the non-zero values.  F = 4 * G with G lanes per row in {8, 16, 32, 64}.
+constexpr int packed_header_words(int feat) { return 2 * (feat / 32); }
+
+template <int G>
+__global__ __launch_bounds__(256) void bias_relu_dropout_pack_kernel(const f4 *__restrict__ z,
+                                                                     const f4 *__restrict__ bias,
+                                                                     const u8x4 *__restrict__ keep,
+                                                                     const float *__restrict__ row_div, float scale,
+                                                                     float *__restrict__ yp, uint32_t *__restrict__ hdr,
+                                                                     int64_t rows) {
+    constexpr int F = 4 * G;
+    constexpr int HW = packed_header_words(F);
+    const int64_t row = ((int64_t)blockIdx.x * 256 + threadIdx.x) / G;
+    if (row >= rows) return;               // whole rows (lane groups) leave together
+    const int l = (int)threadIdx.x & (G - 1);
+    const int64_t i = row * G + l;
+    const f4 v = __builtin_nontemporal_load(z + i);
+    const f4 b = bias[l];
+    const float d = row_div ? row_div[row] : 1.0f;
+    u8x4 k = {1, 1, 1, 1};
+    if (keep) k = __builtin_nontemporal_load(keep + i);
+    float y[4];
+    y[0] = relu_keep(v.x, d, b.x, k.x, scale);
+    y[1] = relu_keep(v.y, d, b.y, k.y, scale);
+    y[2] = relu_keep(v.z, d, b.z, k.z, scale);
+    y[3] = relu_keep(v.w, d, b.w, k.w, scale);
+    uint32_t nib = 0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) nib |= (y[e] > 0.0f ? 1u : 0u) << e;
+    const int cnt = __popc(nib);
+    int incl = cnt;                        // inclusive scan of the counts over the row's lanes
+#pragma unroll
+    for (int s = 1; s < G; s <<= 1) {
+        const int t = __shfl_up(incl, s, G);
+        if (l >= s) incl += t;
+    }
+    const int excl = incl - cnt;
+    float *dst = yp + (size_t)row * F + excl;
+    int at = 0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+        if (nib & (1u << e)) dst[at++] = y[e];
+
+    uint32_t word = nib << (4 * (l & 7));  // eight lanes make one bitmap word
+    word |= __shfl_xor(word, 1, G);
+    word |= __shfl_xor(word, 2, G);
+    word |= __shfl_xor(word, 4, G);
+    if ((l & 7) == 0) {                    // this lane's exclusive count = non-zeros in front of its word
+        uint2 pair;
+        pair.x = word;
+        pair.y = (uint32_t)excl;
+        *reinterpret_cast<uint2 *>(hdr + row * HW + 2 * (l >> 3)) = pair;
     }
 }
 
@@ -188,10 +266,10 @@ extern "C" int gnnagg_relu_dropout_backward_f32(const float *grad_y, const float
         GNNAGG_REQUIRE(aligned16(grad_y, y, grad_z) && (reinterpret_cast<uintptr_t>(bias_partial) & 15) == 0,
                        "bias partial sums need 16-byte aligned operands");
         const int64_t rpb = (rows + blocks - 1) / blocks;
-        hipLaunchKernelGGL(relu_dropout_backward_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, st,
-                           reinterpret_cast<const f4 *>(grad_y), reinterpret_cast<const f4 *>(y), row_div, scale,
+        hipLaunchKernelGGL(relu_dropout_backward_rows_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, st,
+                           reinterpret_cast<const f4 *>(grad_y), static_cast<const void *>(y), row_div, scale,
                            reinterpret_cast<f4 *>(grad_z), reinterpret_cast<f4 *>(bias_partial), rows, (int)(feat / 4),
-                           (int)rpb);
+                           (int)rpb, 0);
         GNNAGG_HIP(hipGetLastError());
         return GNNAGG_OK;
     }
@@ -203,6 +281,62 @@ extern "C" int gnnagg_relu_dropout_backward_f32(const float *grad_y, const float
         hipLaunchKernelGGL(relu_dropout_backward_kernel, dim3(stream_grid(count)), dim3(256), 0, st, grad_y, y, row_div,
                            scale, grad_z, count, (int)feat);
     }
+    GNNAGG_HIP(hipGetLastError());
+    return GNNAGG_OK;
+}
+
+extern "C" int gnnagg_packed_header_words(int64_t feat) {
+    if (feat != 32 && feat != 64 && feat != 128 && feat != 256) return 0;
+    return packed_header_words((int)feat);
+}
+
+extern "C" int gnnagg_bias_relu_dropout_pack_f32(const float *z, const float *bias, const uint8_t *keep,
+                                                 const float *row_div, float scale, float *y_packed, uint32_t *header,
+                                                 int64_t rows, int64_t feat, void *stream) {
+    GNNAGG_REQUIRE(rows >= 0, "negative size");
+    if (gnnagg_packed_header_words(feat) == 0)
+        return fail(GNNAGG_ERR_UNSUPPORTED, "packed activations exist for widths 32, 64, 128, 256 (got %lld)",
+                    (long long)feat);
+    if (rows == 0) return GNNAGG_OK;
+    GNNAGG_REQUIRE(z && bias && y_packed && header, "null z/bias/y_packed/header");
+    GNNAGG_REQUIRE(aligned16(z, bias, bias) && (reinterpret_cast<uintptr_t>(keep) & 3) == 0 &&
+                       (reinterpret_cast<uintptr_t>(y_packed) & 3) == 0,
+                   "packed epilogue needs 16-byte aligned z / bias and a 4-byte aligned mask");
+    GNNAGG_REQUIRE(rows < (int64_t(1) << 31), "too many rows");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int g = (int)(feat / 4);
+    const unsigned blocks = grid_for(rows * g, 256);
+#define GNNAGG_PACK(G)                                                                                          \
+    if (g == G)                                                                                                 \
+        hipLaunchKernelGGL(bias_relu_dropout_pack_kernel<G>, dim3(blocks), dim3(256), 0, st,                    \
+                           reinterpret_cast<const f4 *>(z), reinterpret_cast<const f4 *>(bias),                 \
+                           reinterpret_cast<const u8x4 *>(keep), row_div, scale, y_packed, header, rows)
+    GNNAGG_PACK(8);
+    GNNAGG_PACK(16);
+    GNNAGG_PACK(32);
+    GNNAGG_PACK(64);
+#undef GNNAGG_PACK
+    GNNAGG_HIP(hipGetLastError());
+    return GNNAGG_OK;
+}
+
+extern "C" int gnnagg_relu_dropout_backward_packed_f32(const float *grad_y, const uint32_t *header, const float *row_div,
+                                                       float scale, float *grad_z, float *bias_partial, int64_t rows,
+                                                       int64_t feat, void *stream) {
+    GNNAGG_REQUIRE(rows >= 0, "negative size");
+    const int hw = gnnagg_packed_header_words(feat);
+    if (hw == 0)
+        return fail(GNNAGG_ERR_UNSUPPORTED, "packed activations exist for widths 32, 64, 128, 256 (got %lld)",
+                    (long long)feat);
+    if (rows == 0) return GNNAGG_OK;
+    GNNAGG_REQUIRE(grad_y && header && grad_z && bias_partial, "null grad_y/header/grad_z/bias_partial");
+    GNNAGG_REQUIRE(aligned16(grad_y, grad_z, bias_partial), "packed backward needs 16-byte aligned operands");
+    const int blocks = gnnagg_relu_dropout_backward_blocks(rows, feat);
+    const int64_t rpb = (rows + blocks - 1) / blocks;
+    hipLaunchKernelGGL(relu_dropout_backward_rows_kernel<true>, dim3((unsigned)blocks), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), reinterpret_cast<const f4 *>(grad_y),
+                       static_cast<const void *>(header), row_div, scale, reinterpret_cast<f4 *>(grad_z),
+                       reinterpret_cast<f4 *>(bias_partial), rows, (int)(feat / 4), (int)rpb, hw);
     GNNAGG_HIP(hipGetLastError());
     return GNNAGG_OK;
 }

@@ -4,6 +4,7 @@
 
 #include <algorithm>
 #include <new>
+#include <type_traits>
 #include <vector>
 
 #include "common.h"
@@ -62,6 +63,31 @@ hipError_t launch_tasks(const SpmmArgs &a, int rows_per_group, hipStream_t strea
     hipLaunchKernelGGL((spmm_tasks_kernel<VEC, LPR, NCH, IdxT, MODE>), dim3((unsigned)nblocks), dim3(256), 0,
                        stream, args);
     return hipGetLastError();
+}
+
+// Packed source rows (16-byte lanes, one load per lane): widths 32 / 64 -> 16 lanes, 128 -> 32, 256 -> 64.
+hipError_t launch_packed(const SpmmArgs &a, int rows_per_group, hipStream_t stream) {
+    auto go = [&](auto lpr_tag) -> hipError_t {
+        constexpr int LPR = decltype(lpr_tag)::value;
+        constexpr int GPB = 256 / LPR;
+        SpmmArgs args = a;
+        if (rows_per_group > kMaxRowsPerGroup) rows_per_group = kMaxRowsPerGroup;
+        if (rows_per_group < 1) rows_per_group = 1;
+        args.tasks_per_block = GPB * rows_per_group;
+        if (args.head_tasks > args.ntasks) args.head_tasks = args.ntasks;
+        const int64_t head_blocks = (args.head_tasks + GPB - 1) / GPB;
+        const int64_t nblocks =
+            head_blocks + (args.ntasks - args.head_tasks + args.tasks_per_block - 1) / args.tasks_per_block;
+        if (nblocks == 0) return hipSuccess;
+        if (nblocks > 0x7fffffffll) return hipErrorInvalidValue;
+        args.head_blocks = (int)head_blocks;
+        hipLaunchKernelGGL((spmm_tasks_kernel<4, LPR, 1, int32_t, kRowsPlanned, kSrcPacked>), dim3((unsigned)nblocks),
+                           dim3(256), 0, stream, args);
+        return hipGetLastError();
+    };
+    if (a.feat > 128) return go(std::integral_constant<int, 64>{});
+    if (a.feat > 64) return go(std::integral_constant<int, 32>{});
+    return go(std::integral_constant<int, 16>{});
 }
 
 template <int VEC, typename IdxT, int MODE>
@@ -476,6 +502,36 @@ extern "C" int gnnagg_plan_spmm_f32(gnnagg_plan *plan, const float *value, const
     }
     if (plan->nhuge > 0) GNNAGG_HIP(hipStreamWaitEvent(st, plan->join, 0));
     if (prof) GNNAGG_HIP(hipEventRecord(plan->ev[3], st));
+    return GNNAGG_OK;
+}
+
+extern "C" int gnnagg_plan_spmm_packed_f32(gnnagg_plan *plan, const float *value, const float *y_packed,
+                                           const uint32_t *header, float *out, int64_t feat, int accumulate,
+                                           void *stream) {
+    GNNAGG_REQUIRE(plan, "null plan");
+    const int hw = gnnagg_packed_header_words(feat);
+    if (hw == 0)
+        return fail(GNNAGG_ERR_UNSUPPORTED, "packed source rows exist for widths 32, 64, 128, 256 (got %lld)",
+                    (long long)feat);
+    if (plan->rows == 0) return GNNAGG_OK;
+    GNNAGG_REQUIRE(out, "null out");
+    GNNAGG_REQUIRE(plan->nnz == 0 || (value && y_packed && header), "null value/y_packed/header");
+    GNNAGG_REQUIRE((reinterpret_cast<uintptr_t>(out) & 15) == 0 && (reinterpret_cast<uintptr_t>(y_packed) & 3) == 0,
+                   "packed SpMM needs a 16-byte aligned output");
+    SpmmArgs a{};
+    a.task = plan->task;  // every row runs in the lane-group kernel, the very longest included
+    a.col = plan->col32;
+    a.val = value;
+    a.x = y_packed;
+    a.hdr = header;
+    a.hdr_words = hw;
+    a.dst = out;
+    a.feat = (int)feat;
+    a.f_base = 0;
+    a.accumulate = accumulate;
+    a.ntasks = plan->rows - (accumulate ? plan->nempty : 0);
+    a.head_tasks = plan->nlong;
+    GNNAGG_HIP(launch_packed(a, plan->rows_per_group, static_cast<hipStream_t>(stream)));
     return GNNAGG_OK;
 }
 

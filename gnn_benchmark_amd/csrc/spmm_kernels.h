@@ -125,24 +125,86 @@ __device__ __forceinline__ int64_t uniform_i64(int64_t v) {
     return ((int64_t)hi << 32) | (uint32_t)lo;
 }
 
+enum SourceKind : int {
+    kSrcDense = 0,   // x[col, :] is a dense fp32 row
+    kSrcPacked = 1   // x[col, :] holds the row's non-zero values at its front, hdr[col, :] says which
+};
+
+typedef float f32x4_unaligned __attribute__((ext_vector_type(4), aligned(4)));
+
+// One lane's four features (f .. f+3, f a multiple of 4) of a packed row: `h` is the row's
+// header -- for every 32 features a (bitmap, non-zeros in front) pair of words -- fetched with
+// one 8-byte load; `position` then says where in the row the lane's first non-zero value sits.
+struct PackedLane {
+    uint32_t word, before;
+    __device__ __forceinline__ void request(const uint32_t *__restrict__ h, int f) {
+        const uint2 pair = *reinterpret_cast<const uint2 *>(h + 2 * (f >> 5));
+        word = pair.x;
+        before = pair.y;
+    }
+    __device__ __forceinline__ uint32_t nibble(int f) const { return (word >> (f & 31)) & 15u; }
+    __device__ __forceinline__ int position(int f) const {
+        return (int)before + __popc(word & ((1u << (f & 31)) - 1u));
+    }
+};
+
+__device__ __forceinline__ FVec<4> expand_packed(uint32_t nib, const f32x4_unaligned v) {
+    // value e sits at rank popc(nib & ((1 << e) - 1)) among the up to four loaded ones
+    FVec<4> r;
+    const float a0 = v.x, a1 = v.y, a2 = v.z, a3 = v.w;
+    r.d.x = (nib & 1u) ? a0 : 0.0f;
+    const float s1 = (nib & 1u) ? a1 : a0;
+    r.d.y = (nib & 2u) ? s1 : 0.0f;
+    const int r2 = __popc(nib & 3u);
+    const float s2 = r2 == 0 ? a0 : (r2 == 1 ? a1 : a2);
+    r.d.z = (nib & 4u) ? s2 : 0.0f;
+    const int r3 = __popc(nib & 7u);
+    const float s3 = r3 == 0 ? a0 : (r3 == 1 ? a1 : (r3 == 2 ? a2 : a3));
+    r.d.w = (nib & 8u) ? s3 : 0.0f;
+    return r;
+}
+
 // UU gathers issued back to back, then their FMAs in CSR order: elements j .. j+UU-1 of
-// the chunk held in (c_l, v_l) across the group's lanes.
-template <int UU, int VEC, int LPR, int NCH, typename IdxT>
+// the chunk held in (c_l, v_l) across the group's lanes.  For a packed source the zero
+// values are not fetched; fma(v, 0, acc) == acc, so the chain is the same (up to the sign
+// of a zero result).
+template <int UU, int VEC, int LPR, int NCH, int SRC, typename IdxT>
 __device__ __forceinline__ void gather_fma(FVec<VEC> (&acc)[NCH], IdxT c_l, float v_l, int j,
-                                           const float *__restrict__ x, int F, const int (&foff)[NCH]) {
+                                           const float *__restrict__ x, int F, const int (&foff)[NCH],
+                                           const uint32_t *__restrict__ hdr, int hdr_words) {
     const float *xr[UU];
     float vv[UU];
+    int64_t cc[UU];
 #pragma unroll
     for (int u = 0; u < UU; ++u) {
-        const int64_t c = group_bcast_idx<LPR>(c_l, j + u);
+        cc[u] = group_bcast_idx<LPR>(c_l, j + u);
         vv[u] = __int_as_float(group_bcast<LPR>(__float_as_int(v_l), j + u));
-        xr[u] = x + (size_t)c * (size_t)F;
+        xr[u] = x + (size_t)cc[u] * (size_t)F;
     }
     FVec<VEC> xv[UU][NCH];
+    if constexpr (SRC == kSrcPacked) {
+        static_assert(SRC == kSrcDense || (VEC == 4 && NCH == 1), "packed rows: 16-byte lanes, one load per lane");
+        const int f = foff[0];
+        PackedLane pl[UU];
 #pragma unroll
-    for (int u = 0; u < UU; ++u) {
+        for (int u = 0; u < UU; ++u) pl[u].request(hdr + (size_t)cc[u] * (size_t)hdr_words, f);
+        f32x4_unaligned raw[UU];
+        uint32_t nib[UU];
 #pragma unroll
-        for (int k = 0; k < NCH; ++k) xv[u][k] = FVec<VEC>::load(xr[u] + foff[k]);
+        for (int u = 0; u < UU; ++u) {
+            nib[u] = pl[u].nibble(f);
+            // a lane with nothing to fetch reads the front of the row: a valid, hot address
+            const float *src = xr[u] + (nib[u] ? pl[u].position(f) : 0);
+            raw[u] = *reinterpret_cast<const f32x4_unaligned *>(src);
+        }
+#pragma unroll
+        for (int u = 0; u < UU; ++u) xv[u][0] = expand_packed(nib[u], raw[u]);
+    } else {
+#pragma unroll
+        for (int u = 0; u < UU; ++u) {
+#pragma unroll
+            for (int k = 0; k < NCH; ++k) xv[u][k] = FVec<VEC>::load(xr[u] + foff[k]);
+        }
     }
 #pragma unroll
     for (int u = 0; u < UU; ++u) {
@@ -168,7 +230,9 @@ struct SpmmArgs {
     const RowTask *task;      // [ntasks]                       (kRowsPlanned)
     const void *col;          // IdxT [nnz]
     const float *val;         // [nnz]
-    const float *x;           // dense operand [K, F]
+    const float *x;           // dense operand [K, F] (packed source: non-zero values at the front of each row)
+    const uint32_t *hdr;      // packed source only: [K, hdr_words] row headers
+    int hdr_words;
     float *dst;               // out [rows, F]
     int64_t ntasks;
     int feat;                 // F (row stride of x and dst, in floats)
@@ -191,7 +255,7 @@ struct UnrollFor {
 
 constexpr int kMaxRowsPerGroup = 16;  // a group's task descriptors live one per lane
 
-template <int VEC, int LPR, int NCH, typename IdxT, int MODE>
+template <int VEC, int LPR, int NCH, typename IdxT, int MODE, int SRC = kSrcDense>
 __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
     constexpr int GPB = 256 / LPR;  // groups per 256-thread block
     constexpr int U = UnrollFor<VEC, NCH>::value;
@@ -307,15 +371,15 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
         // full blocks of U gathers, then a halving cascade for what is left, so that a
         // chunk of cnt elements costs at most cnt/U + log2(U) dependent round trips
         int j = 0;
-        for (; j + U <= cnt; j += U) gather_fma<U, VEC, LPR, NCH>(acc, c_l, v_l, j, x, F, foff);
+        for (; j + U <= cnt; j += U) gather_fma<U, VEC, LPR, NCH, SRC>(acc, c_l, v_l, j, x, F, foff, a.hdr, a.hdr_words);
         if constexpr (U > 4) {
-            if (j + 4 <= cnt) { gather_fma<4, VEC, LPR, NCH>(acc, c_l, v_l, j, x, F, foff); j += 4; }
+            if (j + 4 <= cnt) { gather_fma<4, VEC, LPR, NCH, SRC>(acc, c_l, v_l, j, x, F, foff, a.hdr, a.hdr_words); j += 4; }
         }
         if constexpr (U > 2) {
-            if (j + 2 <= cnt) { gather_fma<2, VEC, LPR, NCH>(acc, c_l, v_l, j, x, F, foff); j += 2; }
+            if (j + 2 <= cnt) { gather_fma<2, VEC, LPR, NCH, SRC>(acc, c_l, v_l, j, x, F, foff, a.hdr, a.hdr_words); j += 2; }
         }
         if constexpr (U > 1) {
-            if (j + 1 <= cnt) { gather_fma<1, VEC, LPR, NCH>(acc, c_l, v_l, j, x, F, foff); j += 1; }
+            if (j + 1 <= cnt) { gather_fma<1, VEC, LPR, NCH, SRC>(acc, c_l, v_l, j, x, F, foff, a.hdr, a.hdr_words); j += 1; }
         }
 
         if (row_done) {

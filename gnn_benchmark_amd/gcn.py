@@ -17,8 +17,8 @@ from typing import List, Optional, Sequence
 import torch
 import torch.nn.functional as F
 
-from . import _lib
-from .aggregator import Aggregator
+from . import _lib, packed
+from .aggregator import Aggregator, AggregatorPacked
 
 
 class _Bf16InputLinear(torch.autograd.Function):
@@ -130,6 +130,44 @@ class _BiasReluDropout(torch.autograd.Function):
         return grad_z, grad_bias, None, None, None
 
 
+class _BiasReluDropoutPacked(torch.autograd.Function):
+    """The same epilogue writing its result packed (``packed.py``): returns ``(values,
+    header)``.  The gradient that comes back for ``values`` is the one with respect to the
+    dense activations the pair stands for (``AggregatorPacked`` returns exactly that); which
+    units were active is read from the header's bitmap."""
+
+    @staticmethod
+    def forward(ctx, z, bias, keep, scale, row_div):
+        if not z.is_cuda or z.dtype != torch.float32 or not z.is_contiguous() or z.dim() != 2:
+            raise RuntimeError("Input mismatch: z must be a contiguous float32 [rows, feat] GPU (HIP) tensor")
+        values, header = packed.empty(z.size(0), z.size(1), z.device)
+        with torch.cuda.device(z.device):
+            _lib.check(_lib.lib().gnnagg_bias_relu_dropout_pack_f32(
+                _lib.ptr(z), _lib.ptr(bias.contiguous()), _lib.ptr(keep), _lib.ptr(row_div), float(scale),
+                _lib.ptr(values), _lib.ptr(header), z.size(0), z.size(1), _lib.current_stream(z.device)))
+        ctx.mark_non_differentiable(header)
+        ctx.save_for_backward(header)
+        ctx.scale = float(scale)
+        ctx.row_div = row_div
+        return values, header
+
+    @staticmethod
+    def backward(ctx, grad_y, _grad_header):
+        (header,) = ctx.saved_tensors
+        grad_y = grad_y.contiguous()
+        rows, feat = grad_y.shape
+        grad_z = torch.empty_like(grad_y)
+        L = _lib.lib()
+        blocks = int(L.gnnagg_relu_dropout_backward_blocks(rows, feat))
+        partial = torch.empty(blocks, feat, dtype=torch.float32, device=grad_y.device)
+        with torch.cuda.device(grad_y.device):
+            _lib.check(L.gnnagg_relu_dropout_backward_packed_f32(
+                _lib.ptr(grad_y), _lib.ptr(header), _lib.ptr(ctx.row_div), ctx.scale, _lib.ptr(grad_z),
+                _lib.ptr(partial), rows, feat, _lib.current_stream(grad_y.device)))
+        grad_bias = partial.sum(dim=0) if ctx.needs_input_grad[1] else None
+        return grad_z, grad_bias, None, None, None
+
+
 class GCNLayer(torch.nn.Module):
     def __init__(self, in_channels: int, out_channels: int, gemm: str = "fp32"):
         super().__init__()
@@ -140,9 +178,13 @@ class GCNLayer(torch.nn.Module):
         self.bias = torch.nn.Parameter(torch.zeros(out_channels))
         torch.nn.init.xavier_uniform_(self.weight, gain=torch.nn.init.calculate_gain("relu"))
 
-    def transform(self, graph, x: torch.Tensor, layer: int, is_pre_delay: bool) -> torch.Tensor:
-        """(A x) W: neither the degree normalisation nor the bias yet."""
-        agg = Aggregator.apply(graph, x, layer, 32, is_pre_delay, self.training)
+    def transform(self, graph, x, layer: int, is_pre_delay: bool) -> torch.Tensor:
+        """(A x) W: neither the degree normalisation nor the bias yet.  ``x`` is a dense tensor
+        or a packed ``(values, header)`` pair."""
+        if isinstance(x, tuple):
+            agg = AggregatorPacked.apply(graph, x[0], x[1], layer, 32, is_pre_delay, self.training)
+        else:
+            agg = Aggregator.apply(graph, x, layer, 32, is_pre_delay, self.training)
         if self.gemm == "bf16":
             return _Bf16InputLinear.apply(agg, self.weight)
         return _Fp32Linear.apply(agg, self.weight)
@@ -153,10 +195,13 @@ class GCNLayer(torch.nn.Module):
 
 
 class GCN(torch.nn.Module):
-    def __init__(self, dims: Sequence[int], gemm: str = "fp32", dropout: float = 0.5):
+    def __init__(self, dims: Sequence[int], gemm: str = "fp32", dropout: float = 0.5, packed_activations: bool = False):
         super().__init__()
         self.layers = torch.nn.ModuleList([GCNLayer(dims[i], dims[i + 1], gemm) for i in range(len(dims) - 1)])
         self.dropout = dropout
+        # keep hidden activations packed (non-zero values + bitmap) where their width allows and
+        # pre-aggregation is used: the next layer's aggregation then skips the zeros
+        self.packed_activations = packed_activations
 
     def forward(self, graph, x: torch.Tensor, is_pre_delay: bool,
                 masks: Optional[List[torch.Tensor]] = None) -> torch.Tensor:
@@ -168,12 +213,16 @@ class GCN(torch.nn.Module):
                 h = layer(graph, h, l, is_pre_delay)
                 break
             z = layer.transform(graph, h, l, is_pre_delay)
+            single_rank = getattr(graph, "exchange", None) is None
+            pack = (self.packed_activations and (is_pre_delay or single_rank)
+                    and packed.header_words(z.size(1)) > 0)
+            epilogue = _BiasReluDropoutPacked if pack else _BiasReluDropout
             if self.training and self.dropout > 0.0:
                 if masks is None:
                     raise ValueError("training needs the seeded dropout masks")
-                h = _BiasReluDropout.apply(z, layer.bias, masks[l], 1.0 / (1.0 - self.dropout), graph.in_degrees)
+                h = epilogue.apply(z, layer.bias, masks[l], 1.0 / (1.0 - self.dropout), graph.in_degrees)
             else:
-                h = _BiasReluDropout.apply(z, layer.bias, None, 1.0, graph.in_degrees)
+                h = epilogue.apply(z, layer.bias, None, 1.0, graph.in_degrees)
         return F.log_softmax(h, dim=1)
 
 

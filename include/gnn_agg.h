@@ -178,6 +178,35 @@ int gnnagg_wgrad_f32(const float *x, const float *g, float *w_grad, void *worksp
                      int64_t fo, void *stream);
 
 /* ---------------------------------------------------------------------------------
+ * Packed activations: the output of a ReLU + dropout layer with every row's non-zero values
+ * moved to the front of the row (order kept, row stride still feat, the tail unspecified)
+ * plus a header per row: for every 32 features a pair of 32-bit words, the bitmap of those
+ * features (bit set = non-zero) and the number of non-zeros in front of them;
+ * gnnagg_packed_header_words = 2 * feat / 32 words in all (0 = width not supported;
+ * supported: 32, 64, 128, 256).  A gather of
+ * such a row touches the header and the non-zero values only -- about a quarter of the row
+ * in training.  Skipping the zeros leaves every row's FMA chain as it is (fma(v, 0, acc) ==
+ * acc), so results equal the dense ones up to the sign of a zero.
+ *   gnnagg_bias_relu_dropout_pack_f32: gnnagg_bias_relu_dropout_f32 writing the packed form
+ *     (y_packed fp32 [rows, feat] -- allocate 4 floats more than rows * feat: the consumer's
+ *     16-byte loads may run up to 3 floats past a row -- and header uint32 [rows, words]).
+ *   gnnagg_relu_dropout_backward_packed_f32: gnnagg_relu_dropout_backward_f32 with the
+ *     header's bitmap in place of the forward output; bias_partial is required.
+ *   gnnagg_plan_spmm_packed_f32: gnnagg_plan_spmm_f32 whose dense operand is given packed.
+ * Part of this build's GCN layer stack (no counterpart in the reference, which keeps
+ * activations dense).  No allocation, no host synchronisation.
+ * ------------------------------------------------------------------------------- */
+int gnnagg_packed_header_words(int64_t feat);
+int gnnagg_bias_relu_dropout_pack_f32(const float *z, const float *bias, const uint8_t *keep, const float *row_div,
+                                      float scale, float *y_packed, uint32_t *header, int64_t rows, int64_t feat,
+                                      void *stream);
+int gnnagg_relu_dropout_backward_packed_f32(const float *grad_y, const uint32_t *header, const float *row_div,
+                                            float scale, float *grad_z, float *bias_partial, int64_t rows, int64_t feat,
+                                            void *stream);
+int gnnagg_plan_spmm_packed_f32(gnnagg_plan *plan, const float *value, const float *y_packed, const uint32_t *header,
+                                float *out, int64_t feat, int accumulate, void *stream);
+
+/* ---------------------------------------------------------------------------------
  * Codec of the boundary buffers: fp32 rows <-> int2 / int4 / int8 (bits = 2, 4, 8).
  *
  * Row-packed layout, one segment per destination rank.  Replaces

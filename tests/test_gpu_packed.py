@@ -1,0 +1,140 @@
+"""Packed activations (non-zero values at the front of each row + bitmap header): the packing
+epilogue, the SpMM that gathers packed rows and the bitmap-driven backward against their dense
+counterparts -- equal bit for bit (a zero result may differ in sign, which == ignores)."""
+import copy
+
+import numpy as np
+import pytest
+import torch
+
+from gnn_benchmark_amd import SPMM_forward, gcn, packed, synthetic
+from gnn_benchmark_amd.sparse_tensor import SparseTensor
+from tests.gpu_util import skewed_csr
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _epilogue_inputs(rows, feat, seed, with_mask=True, with_div=True):
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    z = torch.randn(rows, feat, device="cuda", generator=gen)
+    bias = torch.randn(feat, device="cuda", generator=gen) * 0.3
+    keep = (torch.rand(rows, feat, device="cuda", generator=gen) >= 0.5) if with_mask else None
+    div = torch.randint(1, 9, (rows, 1), device="cuda", generator=gen).float() if with_div else None
+    return z, bias, keep, div
+
+
+@pytest.mark.parametrize("feat", [32, 64, 128, 256])
+@pytest.mark.parametrize("rows", [1, 5, 64, 1003])
+@pytest.mark.parametrize("with_mask", [True, False])
+def test_packing_epilogue_equals_dense_epilogue(rows, feat, with_mask):
+    z, bias, keep, div = _epilogue_inputs(rows, feat, rows * 7 + feat, with_mask)
+    scale = 2.0 if with_mask else 1.0
+    dense = gcn._BiasReluDropout.apply(z.clone(), bias, keep, scale, div)
+    values, header = gcn._BiasReluDropoutPacked.apply(z, bias, keep, scale, div)
+    assert header.shape == (rows, packed.header_words(feat)) and header.dtype == torch.int32
+    assert torch.equal(packed.unpack(values, header), dense)
+    # header layout: per 32 features a pair (bitmap: bit set = non-zero, number of non-zeros in front)
+    words = feat // 32
+    on = (dense > 0).cpu().numpy()
+    bitmap = np.ascontiguousarray(header[:, 0::2].cpu().numpy()).view(np.uint32)
+    want_bits = np.packbits(on.reshape(rows, words, 32), axis=2, bitorder="little").view(np.uint32).reshape(rows, words)
+    assert np.array_equal(bitmap, want_bits)
+    before = np.concatenate((np.zeros((rows, 1), np.int64), np.cumsum(on.reshape(rows, words, 32).sum(axis=2), axis=1)[:, :-1]), axis=1)
+    assert np.array_equal(header[:, 1::2].cpu().numpy(), before)
+    # the values sit at the front of their row in feature order
+    d = dense.cpu().numpy()
+    v = values.cpu().numpy()
+    for r in range(min(rows, 40)):
+        nz = d[r][on[r]]
+        assert np.array_equal(v[r, :nz.size], nz)
+
+
+@pytest.mark.parametrize("feat", [32, 64, 128, 256])
+@pytest.mark.parametrize("accumulate", [True, False])
+def test_packed_spmm_equals_dense_spmm(feat, accumulate, low_block_row_threshold):
+    rowptr, col, val = skewed_csr(900, 450, seed=300 + feat)          # rows of 5000 / 1300 / 700, empty rows
+    src = SparseTensor(rowptr=dev(rowptr), col=dev(col), value=dev(val), sparse_sizes=(900, 450), is_sorted=True)
+    z, bias, keep, div = _epilogue_inputs(450, feat, 11 + feat)
+    dense = gcn._BiasReluDropout.apply(z.clone(), bias, keep, 2.0, div)
+    values, header = gcn._BiasReluDropoutPacked.apply(z, bias, keep, 2.0, div)
+    assert 0.6 < float((dense == 0).float().mean()) < 0.9
+    out0 = torch.randn(900, feat, device="cuda", generator=torch.Generator(device="cuda").manual_seed(5))
+    want = out0.clone()
+    SPMM_forward(src, dense, want, accumulate=accumulate)
+    got = out0.clone()
+    packed.spmm(src, values, header, got, accumulate=accumulate)
+    assert torch.equal(got, want)
+    # an all-zero operand and a fully dense one
+    for fill in (0.0, 1.5):
+        zz = torch.full((450, feat), fill, device="cuda")
+        d2 = gcn._BiasReluDropout.apply(zz.clone(), torch.zeros(feat, device="cuda"), None, 1.0, None)
+        v2, h2 = gcn._BiasReluDropoutPacked.apply(zz, torch.zeros(feat, device="cuda"), None, 1.0, None)
+        want, got = out0.clone(), out0.clone()
+        SPMM_forward(src, d2, want, accumulate=accumulate)
+        packed.spmm(src, v2, h2, got, accumulate=accumulate)
+        assert torch.equal(got, want)
+
+
+@pytest.fixture
+def low_block_row_threshold(monkeypatch):
+    # rows above 1000 elements would go to the block-per-row kernel in the dense path; the packed path
+    # keeps them in the lane-group kernel, and both must agree
+    monkeypatch.setenv("GNNAGG_HUGE_THRESH", "1000")
+
+
+@pytest.mark.parametrize("feat", [32, 64, 128, 256])
+def test_bitmap_backward_equals_dense_backward(feat):
+    rows = 1003
+    z, bias, keep, div = _epilogue_inputs(rows, feat, 99 + feat)
+    g = torch.randn(rows, feat, device="cuda", generator=torch.Generator(device="cuda").manual_seed(3))
+    z1, b1 = z.clone().requires_grad_(), bias.clone().requires_grad_()
+    gcn._BiasReluDropout.apply(z1 * 1.0, b1, keep, 2.0, div).backward(g)
+    z2, b2 = z.clone().requires_grad_(), bias.clone().requires_grad_()
+    values, _header = gcn._BiasReluDropoutPacked.apply(z2, b2, keep, 2.0, div)
+    values.backward(g)
+    assert torch.equal(z1.grad, z2.grad)
+    assert torch.equal(b1.grad, b2.grad)
+
+
+def test_train_step_with_packed_activations_equals_dense():
+    part = synthetic.partition_edges(num_local_nodes=3000, world_size=4, rank=1, local_mean_out_degree=5.0, zipf_s=1.8,
+                                     max_degree=300, num_halo_nodes=1200, num_remote_edges=6000, seed=21, device="cuda")
+    dims = [24, 64, 128, 7]
+    gen = torch.Generator(device="cuda").manual_seed(2)
+    x = torch.randn(3000, dims[0], device="cuda", generator=gen)
+    labels = torch.randint(0, dims[-1], (3000,), device="cuda", generator=gen)
+    train_idx = torch.randperm(3000, device="cuda", generator=gen)[:600]
+    masks = gcn.make_dropout_masks(3000, dims, 0.5, seed=8, device="cuda")
+    torch.manual_seed(0)
+    dense_model = gcn.GCN(dims, gemm="fp32", dropout=0.5).cuda()
+    packed_model = copy.deepcopy(dense_model)
+    packed_model.packed_activations = True
+    results = []
+    for model in (dense_model, packed_model):
+        graph = synthetic.build_partition_graph(part, max(dims), True, exchange=synthetic.SeededHaloExchange(3), device="cuda")
+        opt = torch.optim.Adam(model.parameters(), lr=0.01)
+        losses = [gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks) for _ in range(3)]
+        results.append((torch.stack(losses), [p.detach().clone() for p in model.parameters()]))
+    assert torch.equal(results[0][0], results[1][0])
+    for a, b in zip(results[0][1], results[1][1]):
+        assert torch.equal(a, b)
+
+
+def test_error_behaviour():
+    assert packed.header_words(256) == 16 and packed.header_words(128) == 8 and packed.header_words(100) == 0
+    with pytest.raises(RuntimeError, match="widths"):
+        packed.empty(4, 100, "cuda")
+    values, header = packed.empty(8, 64, "cuda")
+    src = SparseTensor(rowptr=torch.arange(9, device="cuda"), col=torch.arange(8, device="cuda"),
+                       value=torch.ones(8, device="cuda"), sparse_sizes=(8, 8), is_sorted=True)
+    out = torch.zeros(8, 64, device="cuda")
+    with pytest.raises(RuntimeError, match="slack"):
+        packed.spmm(src, torch.zeros(8, 64, device="cuda"), header, out)
+    with pytest.raises(RuntimeError, match="header"):
+        packed.spmm(src, values, header[:, :1].contiguous(), out)
+    with pytest.raises(RuntimeError, match="GPU"):
+        packed.spmm(src, values.cpu(), header.cpu(), out)
