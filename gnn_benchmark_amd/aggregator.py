@@ -36,6 +36,10 @@ What differs from the reference, on purpose:
   because an FMA chain started from a stored 0 equals one started from a register 0.
 * The backward ``index_add_`` (:197-199) runs as a deterministic SpMM with the
   selection matrix of ``idx_nodes_send_to_others``.
+
+``AggregatorPacked`` is the same pipeline for local features handed over packed
+(``packed.py``: non-zero values at the front of each row plus a bitmap header); only the
+two forward products that read the features differ.
 """
 import torch
 

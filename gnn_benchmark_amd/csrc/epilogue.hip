@@ -2,7 +2,9 @@
 // y = relu(z / row_div + bias) * (keep ? scale : 0) and its gradient.  HBM-bound streaming
 // kernels (one read and one write of the activation instead of five passes).  The
 // per-row divisor carries the mean-aggregation normalisation (1/in-degree), moved behind
-// the dense product: D^-1 (A X) W == D^-1 ((A X) W).
+// the dense product: D^-1 (A X) W == D^-1 ((A X) W).  A second forward variant writes its
+// output packed (non-zero values at the front of each row + bitmap header) for the next
+// layer's aggregation to gather, and the backward can take that bitmap in place of the output.
 #include "common.h"
 
 namespace gnnagg {
