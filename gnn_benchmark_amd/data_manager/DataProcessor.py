@@ -15,7 +15,7 @@ a caller-supplied callable instead; no process group is needed.
 Sorting.  The reference uses ``torch.argsort`` (tie order unspecified); a stable sort
 is used here, which reproduces every known-answer vector of the reference's tests.
 """
-from typing import Callable, List, Optional, Sequence
+from typing import Callable, List, Optional
 
 import torch
 

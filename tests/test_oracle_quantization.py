@@ -4,7 +4,6 @@ kernels, the live compiled kernels where oracle/_ref is built, and brute force."
 import os
 
 import numpy as np
-import pytest
 
 from oracle import quantization as oq
 
