@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 import torch
 
-from gnn_benchmark_amd import SPMM_backward, SPMM_forward
+from gnn_benchmark_amd import SPMM_backward, SPMM_forward, gcn, packed
 from gnn_benchmark_amd import computation_ops as ops
 from gnn_benchmark_amd.sparse_tensor import SparseTensor
 from oracle import quantization as oq
@@ -83,3 +83,37 @@ def test_random_shapes_match_oracle_bit_for_bit(seed):
         ops.dequantize_tensor_for_all_procs(packed, back, dev(wire), work_range, nseg, bits)
         want_back = oq.dequantize_segments(want_packed, wire, splits, bits)
         assert np.array_equal(back.cpu().numpy().view(np.uint32), want_back.view(np.uint32)), ("dequantised", what, bits)
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_packed_operands_match_the_dense_product(seed):
+    """Packed activations of random sparsity (all-zero and full rows included) through random
+    matrices: the packed-source product equals the dense one bit for bit."""
+    rng = np.random.default_rng(12000 + seed)
+    for case in range(20):
+        rows = int(rng.choice([1, 5, 64, 300, 2000]))
+        cols = int(rng.choice([1, 3, 64, 500, 3000]))
+        feat = int(rng.choice([32, 64, 128, 256]))
+        deg = _degrees(rng, rows)
+        rowptr = np.concatenate(([0], np.cumsum(deg))).astype(np.int64)
+        nnz = int(rowptr[-1])
+        col = rng.integers(0, cols, nnz).astype(np.int64)
+        val = rng.standard_normal(nnz).astype(np.float32)
+        z = rng.standard_normal((cols, feat)).astype(np.float32)
+        keep_p = float(rng.choice([0.0, 0.1, 0.5, 0.9, 1.0]))
+        keep = (rng.random((cols, feat)) < keep_p)
+        if cols > 2:
+            z[0] = -1.0          # a row of zeros after the ReLU
+            z[1] = 2.0           # a full row where kept
+            keep[1] = True
+        src = SparseTensor(rowptr=dev(rowptr), col=dev(col), value=dev(val), sparse_sizes=(rows, cols), is_sorted=True)
+        bias = torch.zeros(feat, device="cuda")
+        dense = gcn._BiasReluDropout.apply(dev(z), bias, dev(keep), 1.5, None)
+        values, header = gcn._BiasReluDropoutPacked.apply(dev(z), bias, dev(keep), 1.5, None)
+        assert torch.equal(packed.unpack(values, header), dense)
+        acc = bool(rng.integers(0, 2))
+        out0 = dev(rng.standard_normal((rows, feat)).astype(np.float32))
+        want, got = out0.clone(), out0.clone()
+        SPMM_forward(src, dense, want, accumulate=acc)
+        packed.spmm(src, values, header, got, accumulate=acc)
+        assert torch.equal(got, want), dict(seed=seed, case=case, rows=rows, cols=cols, feat=feat, keep=keep_p, acc=acc)
