@@ -36,3 +36,11 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     cpu = d["cpu_baseline"]
     assert cpu["kind"] in ("reference", "port") and cpu["cores"] >= 1 and cpu["value"] > 0 and cpu["unit"] == "GFLOP/s"
     assert isinstance(cpu["sample"], str)
+
+
+@pytest.mark.gpu
+def test_smoke_entry_point_runs_and_checks_itself():
+    sys.path.insert(0, ROOT)
+    import __graft_entry__ as entry
+
+    entry.smoke()  # raises on any mismatch with the oracle
