@@ -44,7 +44,7 @@ two forward products that read the features differ.
 import torch
 
 from . import _lib, computation_ops, packed
-from .spmm_kernel import SPMM_backward, SPMM_forward
+from .spmm_kernel import SPMM_backward, SPMM_backward_quantized, SPMM_forward, SPMM_forward_quantized
 
 
 def _gather_rows(src: torch.Tensor, index: torch.Tensor, out: torch.Tensor) -> None:
@@ -94,6 +94,13 @@ def _quantize_and_exchange(graph, num_bits: int, tag: str, direction: str):
     if outgoing.size(0) != 0:
         computation_ops.quantize_tensor_for_all_procs(outgoing, data, params, work_range, world, num_bits)
     return graph.exchange_quantized(graph.comm_splits, qbuf, tag, direction)
+
+
+def _fused_dequantize(graph, feat_len: int) -> bool:
+    """``graph.fuse_dequantize = True`` asks for the received rows to be aggregated straight from
+    the packed bytes (same values, no fp32 pass over the buffer; the fp32 buffer is then NOT
+    filled, unlike aggregator.py:85-88).  Needs a width that is a multiple of 4."""
+    return bool(getattr(graph, "fuse_dequantize", False)) and feat_len % 4 == 0
 
 
 def _dequantize_received(graph, num_bits: int, direction: str) -> None:
@@ -194,15 +201,19 @@ def _forward(ctx, graph, feats, layer, num_bits: int, is_pre_delay: bool, is_tra
 
     if comm_handle is not None:
         comm_handle.wait()
-    if quantized:
+    fused = quantized and _fused_dequantize(graph, feat_len)
+    if quantized and not fused:
         _dequantize_received(graph, num_bits, "forward")
 
     remote_nodes_feat = graph.comm_buf.recv_buf
     if exchange is not None and remote_nodes_feat.size(0) != 0:
-        if is_pre_delay:  # post-aggregation
-            SPMM_forward(graph.adj_t_pre_post_aggr_from, remote_nodes_feat, out)
+        adj = graph.adj_t_pre_post_aggr_from if is_pre_delay else graph.remote_adj_t  # post-aggregation / raw halo
+        if fused:
+            qbuf = graph.comm_buf_for_quantization
+            SPMM_forward_quantized(adj, qbuf.quantized_recv_data_buf, qbuf.quantized_recv_params_buf_fp32,
+                                   qbuf.recv_row_code, out, num_bits)
         else:
-            SPMM_forward(graph.remote_adj_t, remote_nodes_feat, out)
+            SPMM_forward(adj, remote_nodes_feat, out)
     return out
 
 
@@ -240,13 +251,23 @@ def _backward(ctx, local_out_grad):
 
     if comm_handle is not None:
         comm_handle.wait()
-    if quantized:
+    fused = quantized and _fused_dequantize(graph, feat_len)
+    if quantized and not fused:
         _dequantize_received(graph, num_bits, "backward")
 
     local_nodes_grad_buf = graph.comm_buf.send_buf
     if exchange is not None and local_nodes_grad_buf.size(0) != 0:
+        qbuf = graph.comm_buf_for_quantization
         if is_pre_delay:
-            SPMM_backward(graph.adj_t_pre_post_aggr_to, local_nodes_grad_buf, local_nodes_grad)
+            if fused:
+                SPMM_backward_quantized(graph.adj_t_pre_post_aggr_to, qbuf.quantized_send_data_buf,
+                                        qbuf.quantized_send_params_buf_fp32, qbuf.send_row_code, local_nodes_grad,
+                                        num_bits)
+            else:
+                SPMM_backward(graph.adj_t_pre_post_aggr_to, local_nodes_grad_buf, local_nodes_grad)
+        elif fused:
+            SPMM_forward_quantized(graph.send_scatter_adj_t(), qbuf.quantized_send_data_buf,
+                                   qbuf.quantized_send_params_buf_fp32, qbuf.send_row_code, local_nodes_grad, num_bits)
         else:
             SPMM_forward(graph.send_scatter_adj_t(), local_nodes_grad_buf, local_nodes_grad)
     return local_nodes_grad

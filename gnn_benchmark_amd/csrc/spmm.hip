@@ -46,7 +46,7 @@ Shape pick_shape(int vec, int64_t feat_left) {
     return Shape{vec, kShapes[kNumShapes - 1][0], kShapes[kNumShapes - 1][1]};
 }
 
-template <int VEC, int LPR, int NCH, typename IdxT, int MODE>
+template <int VEC, int LPR, int NCH, typename IdxT, int MODE, int SRC = kSrcDense>
 hipError_t launch_tasks(const SpmmArgs &a, int rows_per_group, hipStream_t stream) {
     constexpr int GPB = 256 / LPR;
     SpmmArgs args = a;
@@ -60,7 +60,7 @@ hipError_t launch_tasks(const SpmmArgs &a, int rows_per_group, hipStream_t strea
     if (nblocks == 0) return hipSuccess;
     args.head_blocks = (int)head_blocks;
     if (nblocks > 0x7fffffffll) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((spmm_tasks_kernel<VEC, LPR, NCH, IdxT, MODE>), dim3((unsigned)nblocks), dim3(256), 0,
+    hipLaunchKernelGGL((spmm_tasks_kernel<VEC, LPR, NCH, IdxT, MODE, SRC>), dim3((unsigned)nblocks), dim3(256), 0,
                        stream, args);
     return hipGetLastError();
 }
@@ -90,10 +90,10 @@ hipError_t launch_packed(const SpmmArgs &a, int rows_per_group, hipStream_t stre
     return go(std::integral_constant<int, 16>{});
 }
 
-template <int VEC, typename IdxT, int MODE>
+template <int VEC, typename IdxT, int MODE, int SRC = kSrcDense>
 hipError_t dispatch_shape(const Shape &s, const SpmmArgs &a, int rpg, hipStream_t st) {
 #define GNNAGG_CASE(L, N) \
-    if (s.lpr == L && s.nch == N) return launch_tasks<VEC, L, N, IdxT, MODE>(a, rpg, st)
+    if (s.lpr == L && s.nch == N) return launch_tasks<VEC, L, N, IdxT, MODE, SRC>(a, rpg, st)
     GNNAGG_CASE(16, 1);
     GNNAGG_CASE(32, 1);
     GNNAGG_CASE(64, 1);
@@ -532,6 +532,45 @@ extern "C" int gnnagg_plan_spmm_packed_f32(gnnagg_plan *plan, const float *value
     a.ntasks = plan->rows - (accumulate ? plan->nempty : 0);
     a.head_tasks = plan->nlong;
     GNNAGG_HIP(launch_packed(a, plan->rows_per_group, static_cast<hipStream_t>(stream)));
+    return GNNAGG_OK;
+}
+
+extern "C" int gnnagg_plan_spmm_quantized_f32(gnnagg_plan *plan, const float *value, const uint8_t *packed,
+                                              const float *params, const int32_t *row_code, float *out, int64_t feat,
+                                              int bits, int accumulate, void *stream) {
+    GNNAGG_REQUIRE(plan, "null plan");
+    GNNAGG_REQUIRE(bits == 2 || bits == 4 || bits == 8, "bits must be 2, 4 or 8 (got %d)", bits);
+    GNNAGG_REQUIRE(feat >= 0, "negative feature width");
+    if (plan->rows == 0 || feat == 0) return GNNAGG_OK;
+    if (int rc = check_feat(feat)) return rc;
+    if (feat % 4 != 0)
+        return fail(GNNAGG_ERR_UNSUPPORTED, "quantised source rows need a width that is a multiple of 4 (got %lld)",
+                    (long long)feat);
+    GNNAGG_REQUIRE(out, "null out");
+    GNNAGG_REQUIRE(plan->nnz == 0 || (value && packed && params && row_code), "null value/packed/params/row_code");
+    GNNAGG_REQUIRE((reinterpret_cast<uintptr_t>(out) & 15) == 0 && (reinterpret_cast<uintptr_t>(packed) & 3) == 0 &&
+                       (reinterpret_cast<uintptr_t>(params) & 7) == 0,
+                   "quantised SpMM needs a 16-byte aligned output, 4-byte aligned bytes and 8-byte aligned parameters");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    for (int64_t f_base = 0; f_base < feat;) {
+        const Shape s = pick_shape(4, feat - f_base);
+        SpmmArgs a{};
+        a.task = plan->task;  // every row runs in the lane-group kernel, the very longest included
+        a.col = plan->col32;
+        a.val = value;
+        a.qdata = packed;
+        a.qparams = params;
+        a.qcode = row_code;
+        a.qbits = bits;
+        a.dst = out;
+        a.feat = (int)feat;
+        a.f_base = (int)f_base;
+        a.accumulate = accumulate;
+        a.ntasks = plan->rows - (accumulate ? plan->nempty : 0);
+        a.head_tasks = plan->nlong;
+        GNNAGG_HIP((dispatch_shape<4, int32_t, kRowsPlanned, kSrcQuant>(s, a, plan->rows_per_group, st)));
+        f_base += s.width();
+    }
     return GNNAGG_OK;
 }
 

@@ -125,9 +125,47 @@ __device__ __forceinline__ int64_t uniform_i64(int64_t v) {
     return ((int64_t)hi << 32) | (uint32_t)lo;
 }
 
+enum TaskMode : int {
+    kRowsNatural = 0,  // task t is row t, described by rowptr        (plan-less entry point)
+    kRowsPlanned = 1   // task t is described by task[t] of a plan    (degree-ordered)
+};
+
+// One row of a plan's schedule: 16 bytes, fetched with a single load.
+struct __attribute__((aligned(16))) RowTask {
+    int64_t start;  // first stored element
+    int32_t len;    // stored elements
+    int32_t row;    // output row
+};
+
+struct SpmmArgs {
+    const int64_t *rowptr;    // [rows+1]                       (kRowsNatural)
+    const RowTask *task;      // [ntasks]                       (kRowsPlanned)
+    const void *col;          // IdxT [nnz]
+    const float *val;         // [nnz]
+    const float *x;           // dense operand [K, F] (packed source: non-zero values at the front of each row)
+    const uint32_t *hdr;      // packed source only: [K, hdr_words] row headers
+    int hdr_words;
+    // quantised source only (row-packed codec of the boundary buffers): byte rows [packed_rows, F] in
+    // which 8/qbits rows share a byte per column, (zero_point, scale) per row, and per row the code
+    // packed_row * 8 + (position inside its byte group)
+    const uint8_t *qdata;
+    const float *qparams;     // [K, 2]
+    const int32_t *qcode;     // [K]
+    int qbits;
+    float *dst;               // out [rows, F]
+    int64_t ntasks;
+    int feat;                 // F (row stride of x and dst, in floats)
+    int f_base;               // first feature handled by this launch
+    int accumulate;           // start every row from dst (1) or from 0 (0)
+    int tasks_per_block;      // tasks handled by one block past the head region
+    int64_t head_tasks;       // the first head_tasks tasks (the longest rows) get one lane group each
+    int head_blocks;          // = ceil(head_tasks / groups per block)
+};
+
 enum SourceKind : int {
     kSrcDense = 0,   // x[col, :] is a dense fp32 row
-    kSrcPacked = 1   // x[col, :] holds the row's non-zero values at its front, hdr[col, :] says which
+    kSrcPacked = 1,  // x[col, :] holds the row's non-zero values at its front, hdr[col, :] says which
+    kSrcQuant = 2    // row col is held quantised: qdata / qparams / qcode (boundary-buffer codec layout)
 };
 
 typedef float f32x4_unaligned __attribute__((ext_vector_type(4), aligned(4)));
@@ -169,9 +207,10 @@ __device__ __forceinline__ FVec<4> expand_packed(uint32_t nib, const f32x4_unali
 // values are not fetched; fma(v, 0, acc) == acc, so the chain is the same (up to the sign
 // of a zero result).
 template <int UU, int VEC, int LPR, int NCH, int SRC, typename IdxT>
-__device__ __forceinline__ void gather_fma(FVec<VEC> (&acc)[NCH], IdxT c_l, float v_l, int j,
-                                           const float *__restrict__ x, int F, const int (&foff)[NCH],
-                                           const uint32_t *__restrict__ hdr, int hdr_words) {
+__device__ __forceinline__ void gather_fma(FVec<VEC> (&acc)[NCH], IdxT c_l, float v_l, int j, const SpmmArgs &a,
+                                           const int (&foff)[NCH]) {
+    const float *__restrict__ x = a.x;
+    const int F = a.feat;
     const float *xr[UU];
     float vv[UU];
     int64_t cc[UU];
@@ -187,7 +226,7 @@ __device__ __forceinline__ void gather_fma(FVec<VEC> (&acc)[NCH], IdxT c_l, floa
         const int f = foff[0];
         PackedLane pl[UU];
 #pragma unroll
-        for (int u = 0; u < UU; ++u) pl[u].request(hdr + (size_t)cc[u] * (size_t)hdr_words, f);
+        for (int u = 0; u < UU; ++u) pl[u].request(a.hdr + (size_t)cc[u] * (size_t)a.hdr_words, f);
         f32x4_unaligned raw[UU];
         uint32_t nib[UU];
 #pragma unroll
@@ -199,6 +238,41 @@ __device__ __forceinline__ void gather_fma(FVec<VEC> (&acc)[NCH], IdxT c_l, floa
         }
 #pragma unroll
         for (int u = 0; u < UU; ++u) xv[u][0] = expand_packed(nib[u], raw[u]);
+    } else if constexpr (SRC == kSrcQuant) {
+        static_assert(SRC != kSrcQuant || VEC == 4, "quantised rows: four bytes per lane and load");
+        // x' = fma(q, scale, zero_point): the dequantisation of the codec, done on the gathered bytes
+        const int per_byte = 8 / a.qbits;
+        const uint32_t mask = (1u << a.qbits) - 1u;
+        uint32_t raw[UU][NCH];
+        float zp[UU], sc[UU];
+        int shift[UU];
+        int code[UU];
+#pragma unroll
+        for (int u = 0; u < UU; ++u) code[u] = a.qcode[cc[u]];
+#pragma unroll
+        for (int u = 0; u < UU; ++u) {
+            const float2 p = *reinterpret_cast<const float2 *>(a.qparams + 2 * (size_t)cc[u]);
+            zp[u] = p.x;
+            sc[u] = p.y;
+        }
+#pragma unroll
+        for (int u = 0; u < UU; ++u) {
+            const uint8_t *qrow = a.qdata + (size_t)(code[u] >> 3) * (size_t)F;
+            shift[u] = (per_byte - (code[u] & 7) - 1) * a.qbits;
+#pragma unroll
+            for (int k = 0; k < NCH; ++k) raw[u][k] = *reinterpret_cast<const uint32_t *>(qrow + foff[k]);
+        }
+#pragma unroll
+        for (int u = 0; u < UU; ++u) {
+#pragma unroll
+            for (int k = 0; k < NCH; ++k) {
+                const uint32_t w = raw[u][k] >> shift[u];
+                xv[u][k].d.x = __builtin_fmaf((float)(w & mask), sc[u], zp[u]);
+                xv[u][k].d.y = __builtin_fmaf((float)((w >> 8) & mask), sc[u], zp[u]);
+                xv[u][k].d.z = __builtin_fmaf((float)((w >> 16) & mask), sc[u], zp[u]);
+                xv[u][k].d.w = __builtin_fmaf((float)((w >> 24) & mask), sc[u], zp[u]);
+            }
+        }
     } else {
 #pragma unroll
         for (int u = 0; u < UU; ++u) {
@@ -212,36 +286,6 @@ __device__ __forceinline__ void gather_fma(FVec<VEC> (&acc)[NCH], IdxT c_l, floa
         for (int k = 0; k < NCH; ++k) acc[k].fma(vv[u], xv[u][k]);
     }
 }
-
-enum TaskMode : int {
-    kRowsNatural = 0,  // task t is row t, described by rowptr        (plan-less entry point)
-    kRowsPlanned = 1   // task t is described by task[t] of a plan    (degree-ordered)
-};
-
-// One row of a plan's schedule: 16 bytes, fetched with a single load.
-struct __attribute__((aligned(16))) RowTask {
-    int64_t start;  // first stored element
-    int32_t len;    // stored elements
-    int32_t row;    // output row
-};
-
-struct SpmmArgs {
-    const int64_t *rowptr;    // [rows+1]                       (kRowsNatural)
-    const RowTask *task;      // [ntasks]                       (kRowsPlanned)
-    const void *col;          // IdxT [nnz]
-    const float *val;         // [nnz]
-    const float *x;           // dense operand [K, F] (packed source: non-zero values at the front of each row)
-    const uint32_t *hdr;      // packed source only: [K, hdr_words] row headers
-    int hdr_words;
-    float *dst;               // out [rows, F]
-    int64_t ntasks;
-    int feat;                 // F (row stride of x and dst, in floats)
-    int f_base;               // first feature handled by this launch
-    int accumulate;           // start every row from dst (1) or from 0 (0)
-    int tasks_per_block;      // tasks handled by one block past the head region
-    int64_t head_tasks;       // the first head_tasks tasks (the longest rows) get one lane group each
-    int head_blocks;          // = ceil(head_tasks / groups per block)
-};
 
 // Gathers kept in flight per lane group, sized so that a wave stays near 64-90 VGPRs:
 // measured on MI355X, deeper unrolls (fewer waves per SIMD) bring nothing -- the
@@ -371,15 +415,15 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
         // full blocks of U gathers, then a halving cascade for what is left, so that a
         // chunk of cnt elements costs at most cnt/U + log2(U) dependent round trips
         int j = 0;
-        for (; j + U <= cnt; j += U) gather_fma<U, VEC, LPR, NCH, SRC>(acc, c_l, v_l, j, x, F, foff, a.hdr, a.hdr_words);
+        for (; j + U <= cnt; j += U) gather_fma<U, VEC, LPR, NCH, SRC>(acc, c_l, v_l, j, a, foff);
         if constexpr (U > 4) {
-            if (j + 4 <= cnt) { gather_fma<4, VEC, LPR, NCH, SRC>(acc, c_l, v_l, j, x, F, foff, a.hdr, a.hdr_words); j += 4; }
+            if (j + 4 <= cnt) { gather_fma<4, VEC, LPR, NCH, SRC>(acc, c_l, v_l, j, a, foff); j += 4; }
         }
         if constexpr (U > 2) {
-            if (j + 2 <= cnt) { gather_fma<2, VEC, LPR, NCH, SRC>(acc, c_l, v_l, j, x, F, foff, a.hdr, a.hdr_words); j += 2; }
+            if (j + 2 <= cnt) { gather_fma<2, VEC, LPR, NCH, SRC>(acc, c_l, v_l, j, a, foff); j += 2; }
         }
         if constexpr (U > 1) {
-            if (j + 1 <= cnt) { gather_fma<1, VEC, LPR, NCH, SRC>(acc, c_l, v_l, j, x, F, foff, a.hdr, a.hdr_words); j += 1; }
+            if (j + 1 <= cnt) { gather_fma<1, VEC, LPR, NCH, SRC>(acc, c_l, v_l, j, a, foff); j += 1; }
         }
 
         if (row_done) {

@@ -29,6 +29,21 @@ class CommBuffer(object):
             self.recv_buf_fp16.resize_(recv_shape)
 
 
+def _row_codes(splits, bits: int, device) -> torch.Tensor:
+    """For every row of a boundary buffer: (packed row) * 8 + (position inside its byte group), with
+    every rank's segment packed on its own -- what a consumer needs to read row i out of the packed
+    bytes without unpacking the buffer."""
+    per = 8 // bits
+    codes, packed_begin = [], 0
+    for rows in splits:
+        local = torch.arange(int(rows), dtype=torch.int64)
+        codes.append((packed_begin + local // per) * 8 + local % per)
+        packed_begin += -(-int(rows) // per)
+    out = torch.cat(codes) if codes else torch.zeros(0, dtype=torch.int64)
+    out = out.to(torch.int32)
+    return out.to(device) if device is not None else out
+
+
 def _prefix(splits, device) -> torch.Tensor:
     out = torch.zeros(len(splits) + 1, dtype=torch.int32)
     out[1:] = torch.tensor(splits, dtype=torch.int32).cumsum(0)
@@ -55,6 +70,10 @@ class CommBufferForQuantization(object):
         self.quantized_recv_params_buf_bf16 = torch.zeros((recv_rows, 2), dtype=torch.bfloat16, device=device)
         self.quantized_work_range_per_proc = _prefix(comm_splits.send_splits, device)
         self.dequantized_work_range_per_proc = _prefix(comm_splits.recv_splits, device)
+        # not in the reference: where each fp32 row sits in the packed bytes, for aggregating
+        # straight from them (spmm_kernel.SPMM_forward_quantized)
+        self.send_row_code = _row_codes(comm_splits.send_splits, bits, device)
+        self.recv_row_code = _row_codes(comm_splits.recv_splits, bits, device)
 
     def resize_buffer(self, comm_splits: CommSplits, feat_len: int, bits: int) -> None:
         if bits == self.bits:

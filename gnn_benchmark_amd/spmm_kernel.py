@@ -11,6 +11,7 @@ cached here is the degree-binned plan (``SparseTensor.get_plan``).
 """
 import torch
 
+from . import _lib
 from .sparse_tensor import SparseTensor
 
 
@@ -36,4 +37,48 @@ def SPMM_backward(src: SparseTensor, other: torch.Tensor, out: torch.Tensor, acc
     if value_T is None:
         raise RuntimeError("Input mismatch: the sparse matrix has no values")
     src.get_plan_for_transpose().spmm(_as_f32(value_T, other), other, out, accumulate)
+    return out, None
+
+
+def _spmm_quantized(plan, value, packed, params, row_code, out, bits, accumulate, operand_rows):
+    if not all(t.is_cuda for t in (value, packed, params, row_code, out)):
+        raise RuntimeError("quantised SpMM operands must be GPU (HIP) tensors; there is no CPU path")
+    feat = out.size(1) if out.dim() == 2 else -1
+    if (packed.dtype != torch.uint8 or not packed.is_contiguous() or packed.dim() != 2 or packed.size(1) != feat
+            or params.dtype != torch.float32 or not params.is_contiguous() or tuple(params.shape) != (operand_rows, 2)
+            or row_code.dtype != torch.int32 or not row_code.is_contiguous() or row_code.numel() != operand_rows
+            or out.dtype != torch.float32 or not out.is_contiguous() or value.dtype != torch.float32):
+        raise RuntimeError("Input mismatch: quantised SpMM needs uint8 [packed rows, F] bytes, float32 [rows, 2] "
+                           "parameters, int32 [rows] row codes and a contiguous float32 [*, F] output")
+    with torch.cuda.device(out.device):
+        _lib.check(_lib.lib().gnnagg_plan_spmm_quantized_f32(
+            plan._handle, _lib.ptr(value.contiguous()), _lib.ptr(packed), _lib.ptr(params), _lib.ptr(row_code),
+            _lib.ptr(out), feat, int(bits), 1 if accumulate else 0, _lib.current_stream(out.device)))
+
+
+def SPMM_forward_quantized(src: SparseTensor, packed: torch.Tensor, params: torch.Tensor, row_code: torch.Tensor,
+                           out: torch.Tensor, bits: int, accumulate: bool = True) -> None:
+    """``out += src @ dequantize(packed, params)`` without materialising the dequantised rows:
+    ``SPMM_forward`` whose dense operand is a boundary buffer still in its exchange format
+    (``CommBufferForQuantization``: packed bytes, per-row parameters, ``*_row_code``).  Equal,
+    bit for bit, to dequantising first."""
+    _, _, value = src.csr()
+    if value is None:
+        raise RuntimeError("Input mismatch: the sparse matrix has no values")
+    if out.size(0) < src.sparse_size(0):
+        raise RuntimeError("Input mismatch: out has fewer rows than the sparse matrix")
+    _spmm_quantized(src.get_plan(), value, packed, params, row_code, out, bits, accumulate, src.sparse_size(1))
+    return None
+
+
+def SPMM_backward_quantized(src: SparseTensor, packed: torch.Tensor, params: torch.Tensor, row_code: torch.Tensor,
+                            out: torch.Tensor, bits: int, accumulate: bool = True):
+    """``out += src.T @ dequantize(packed, params)``: the transposed counterpart."""
+    value_T = src.storage.value_T()
+    if value_T is None:
+        raise RuntimeError("Input mismatch: the sparse matrix has no values")
+    if out.size(0) < src.sparse_size(1):
+        raise RuntimeError("Input mismatch: out has fewer rows than the sparse matrix has columns")
+    _spmm_quantized(src.get_plan_for_transpose(), value_T, packed, params, row_code, out, bits, accumulate,
+                    src.sparse_size(0))
     return out, None

@@ -241,6 +241,17 @@ int gnnagg_quantize_segments_f32(const float *x, uint8_t *packed, float *params,
 int gnnagg_dequantize_segments_f32(const uint8_t *packed, const float *params, float *out, const int32_t *row_range,
                                    const int32_t *packed_range, int64_t segments, int64_t rows, int64_t packed_rows,
                                    int64_t feat, int bits, void *stream);
+/* Post-aggregation straight from the packed bytes: gnnagg_plan_spmm_f32 whose dense operand
+ * row c is given quantised -- packed / params as written by gnnagg_quantize_segments_f32 (or
+ * received from a peer), row_code int32 [rows of the operand] = packed_row * 8 + position of
+ * the row inside its byte group.  Each gathered value is fma(q, scale, zero_point), exactly
+ * what gnnagg_dequantize_segments_f32 would have stored, so the result equals dequantise
+ * followed by gnnagg_plan_spmm_f32 bit for bit, without the fp32 buffer ever being written
+ * or read (the reference dequantises into recv_buf and then aggregates,
+ * model/layers/aggregator.py:83-104).  feat % 4 == 0. */
+int gnnagg_plan_spmm_quantized_f32(gnnagg_plan *plan, const float *value, const uint8_t *packed, const float *params,
+                                   const int32_t *row_code, float *out, int64_t feat, int bits, int accumulate,
+                                   void *stream);
 int gnnagg_quantize_mixed_f32(const float *x, uint8_t *data, const int64_t *feat_range, float *params, int64_t rows,
                               int64_t feat, int32_t *bad_width, void *stream);
 int gnnagg_dequantize_mixed_f32(const uint8_t *data, const int64_t *feat_range, const float *params, float *out,

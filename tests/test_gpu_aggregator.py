@@ -319,6 +319,24 @@ def test_quantised_exchange_world_matches_oracle(seed, sizes, bits):
             assert np.abs(out.detach().cpu().numpy() - want[sl[r]]).max() < 0.5
             assert np.abs(xr.grad.cpu().numpy() - want_t[sl[r]]).max() < 0.5
 
+    # the same run aggregating straight from the packed bytes: same outputs, bit for bit
+    for r in range(W):
+        gr, o = graphs[r], oracle_ranks[r]
+        gr.fuse_dequantize = True
+        gr.exchange_quantized = PlayedQuantizedExchange((dev(fwd_data[r]), dev(fwd_params[r])),
+                                                        (dev(bwd_data[r]), dev(bwd_params[r])))
+        gr.comm_buf.recv_buf.fill_(float("nan"))  # must not be read
+        gr.comm_buf.send_buf.fill_(float("nan"))
+        xr = dev(x[sl[r]]).requires_grad_()
+        out = Aggregator.apply(gr, xr, 1, bits, True, True)
+        o_out = oagg.forward_out(o["local"], o["a_from"], np.ascontiguousarray(x[sl[r]]), recv[r])
+        assert np.array_equal(out.detach().cpu().numpy(), o_out)
+        gr.comm_buf.send_buf.fill_(float("nan"))
+        out.backward(dev(g[sl[r]]))
+        o_dx = oagg.backward_out(o["local"], o["a_to"], np.ascontiguousarray(g[sl[r]]), incoming[r])
+        assert np.array_equal(xr.grad.cpu().numpy(), o_dx)
+        gr.fuse_dequantize = False
+
     # outside training the forward exchange carries fp32 rows (communicator.py:64-65)
     gr = graphs[0]
     exact = host_exchange(o_send, send_splits, recv_splits)

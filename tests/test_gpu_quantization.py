@@ -194,3 +194,76 @@ def test_full_size_round_trip_properties():
     xs = x[sel].cpu().numpy()
     want = oq.row_params(xs, bits)
     assert np.array_equal(params[sel].cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("bits", [2, 4, 8])
+@pytest.mark.parametrize("feat", [4, 48, 100, 128, 256, 600, 2052])
+def test_aggregation_straight_from_packed_bytes_equals_dequantise_then_aggregate(bits, feat):
+    """SPMM_forward_quantized / SPMM_backward_quantized against the two-step path, bit for bit, on a
+    ragged matrix with long and empty rows and a boundary buffer cut into per-rank segments."""
+    from gnn_benchmark_amd import SPMM_backward, SPMM_forward
+    from gnn_benchmark_amd import computation_ops as ops
+    from gnn_benchmark_amd.data_manager import CommBufferForQuantization, CommSplits
+    from gnn_benchmark_amd.sparse_tensor import SparseTensor
+    from gnn_benchmark_amd.spmm_kernel import SPMM_backward_quantized, SPMM_forward_quantized
+    from tests.gpu_util import skewed_csr
+
+    rng = np.random.default_rng(100 * bits + feat)
+    rows_a, halo = 700, 450
+    rowptr, col, val = skewed_csr(rows_a, halo, seed=feat + bits)
+    adj = SparseTensor(rowptr=dev(rowptr), col=dev(col), value=dev(val), sparse_sizes=(rows_a, halo), is_sorted=True)
+    splits = [120, 0, 77, 253]                       # halo rows per peer rank
+    cs = CommSplits(splits, [5, 5, 5, 5], 4, bits)
+    qbuf = CommBufferForQuantization(cs, feat, bits, device="cuda")
+    recv = dev(_rows(rng, halo, feat))
+    ops.quantize_tensor_for_all_procs(recv, qbuf.quantized_recv_data_buf, qbuf.quantized_recv_params_buf_fp32,
+                                      qbuf.dequantized_work_range_per_proc, 4, bits)
+    deq = torch.empty_like(recv)
+    ops.dequantize_tensor_for_all_procs(qbuf.quantized_recv_data_buf, deq, qbuf.quantized_recv_params_buf_fp32,
+                                        qbuf.dequantized_work_range_per_proc, 4, bits)
+    out0 = dev(rng.standard_normal((rows_a, feat)).astype(np.float32))
+    want, got = out0.clone(), out0.clone()
+    SPMM_forward(adj, deq, want)
+    SPMM_forward_quantized(adj, qbuf.quantized_recv_data_buf, qbuf.quantized_recv_params_buf_fp32, qbuf.recv_row_code,
+                           got, bits)
+    assert torch.equal(got, want)
+    want2, got2 = torch.empty_like(out0), torch.empty_like(out0)
+    SPMM_forward(adj, deq, want2, accumulate=False)
+    SPMM_forward_quantized(adj, qbuf.quantized_recv_data_buf, qbuf.quantized_recv_params_buf_fp32, qbuf.recv_row_code,
+                           got2, bits, accumulate=False)
+    assert torch.equal(got2, want2)
+    # transposed: the operand has one row per ROW of the matrix
+    adj_t = SparseTensor(rowptr=dev(rowptr), col=dev(col), value=dev(val), sparse_sizes=(rows_a, halo), is_sorted=True)
+    cs_t = CommSplits([1, 1, 1, 1], [300, 0, 399, 1], 4, bits)
+    qt = CommBufferForQuantization(cs_t, feat, bits, device="cuda")
+    send = dev(_rows(rng, rows_a, feat))
+    ops.quantize_tensor_for_all_procs(send, qt.quantized_send_data_buf, qt.quantized_send_params_buf_fp32,
+                                      qt.quantized_work_range_per_proc, 4, bits)
+    deq_t = torch.empty_like(send)
+    ops.dequantize_tensor_for_all_procs(qt.quantized_send_data_buf, deq_t, qt.quantized_send_params_buf_fp32,
+                                        qt.quantized_work_range_per_proc, 4, bits)
+    dx0 = dev(rng.standard_normal((halo, feat)).astype(np.float32))
+    want3, got3 = dx0.clone(), dx0.clone()
+    SPMM_backward(adj_t, deq_t, want3)
+    SPMM_backward_quantized(adj_t, qt.quantized_send_data_buf, qt.quantized_send_params_buf_fp32, qt.send_row_code, got3,
+                            bits)
+    assert torch.equal(got3, want3)
+
+
+def test_quantised_aggregation_error_behaviour():
+    from gnn_benchmark_amd.data_manager import CommBufferForQuantization, CommSplits
+    from gnn_benchmark_amd.sparse_tensor import SparseTensor
+    from gnn_benchmark_amd.spmm_kernel import SPMM_forward_quantized
+
+    adj = SparseTensor(rowptr=torch.arange(9, device="cuda"), col=torch.arange(8, device="cuda"),
+                       value=torch.ones(8, device="cuda"), sparse_sizes=(8, 8), is_sorted=True)
+    q = CommBufferForQuantization(CommSplits([8], [8], 1, 2), 6, 2, device="cuda")
+    out = torch.zeros(8, 6, device="cuda")
+    with pytest.raises(RuntimeError, match="multiple of 4"):
+        SPMM_forward_quantized(adj, q.quantized_recv_data_buf, q.quantized_recv_params_buf_fp32, q.recv_row_code, out, 2)
+    q = CommBufferForQuantization(CommSplits([8], [8], 1, 2), 8, 2, device="cuda")
+    out = torch.zeros(8, 8, device="cuda")
+    with pytest.raises(RuntimeError, match="bits"):
+        SPMM_forward_quantized(adj, q.quantized_recv_data_buf, q.quantized_recv_params_buf_fp32, q.recv_row_code, out, 3)
+    with pytest.raises(RuntimeError, match="Input mismatch"):
+        SPMM_forward_quantized(adj, q.quantized_recv_data_buf, q.quantized_recv_params_buf_fp32[:4], q.recv_row_code, out, 2)
