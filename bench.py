@@ -502,6 +502,81 @@ def run_c5(args, graph):
         out[f"train_step_ms_{tag}"] = round((time.perf_counter() - t0) * 1e3 / steps, 2)
         out[f"loss_{tag}"] = [round(v, 5) for v in losses + [float(loss)]]
         del model, opt
+    del masks
+    torch.cuda.empty_cache()
+    out["sage"] = run_c5_sage(args, graph, x, labels, train_idx, dims, steps)
+    return out
+
+
+def run_c5_sage(args, graph, x, labels, train_idx, dims, steps):
+    """The reference's own model on the same partition (DistSAGE: lin_neigh + lin_self per layer,
+    dropout -> LayerNorm -> ReLU between layers), three ways: this build's layer stack (one
+    stacked dense product per layer on [aggregated | x] kept side by side, fused elementwise
+    chain), the same with the degree normalisation folded into the matrix values, and -- as the
+    yardstick -- plain torch ops around the same Aggregator, the way the reference writes them."""
+    import torch
+    import torch.nn.functional as F
+
+    from gnn_benchmark_amd import Aggregator, sage
+
+    dev = x.device
+    n = x.size(0)
+    hidden = dims[1]
+    masks = sage.make_dropout_masks(n, hidden, len(dims) - 1, 0.5, args.seed + 8, dev)
+    out = {"layers": "DistSAGE %d->%d->%d->%d, LayerNorm, dropout 0.5" % tuple(dims), "steps": steps}
+
+    def timed(step):
+        losses = [float(step()) for _ in range(2)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            loss = step()
+        torch.cuda.synchronize()
+        return round((time.perf_counter() - t0) * 1e3 / steps, 2), [round(v, 5) for v in losses + [float(loss)]]
+
+    staged = sage.stage_input(x)
+    for tag, g in (("", graph), ("_folded_degrees", None)):
+        if g is None:
+            g = sage.fold_in_degrees(graph)
+        torch.manual_seed(args.seed)
+        model = sage.DistSAGE(dims[0], hidden, dims[-1], num_layers=len(dims) - 1, dropout=0.5, is_pre_delay=True).to(dev)
+        opt = torch.optim.Adam(model.parameters(), lr=0.01)
+        ms, losses = timed(lambda: sage.train_step(model, opt, g, staged, labels, train_idx, masks))
+        out["train_step_ms" + tag], out["loss" + tag] = ms, losses
+        del model, opt, g
+        torch.cuda.empty_cache()
+
+    class TorchOpsSage(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            widths = list(zip(dims[:-1], dims[1:]))
+            self.lin_neigh = torch.nn.ModuleList([torch.nn.Linear(a, b, bias=False) for a, b in widths])
+            self.lin_self = torch.nn.ModuleList([torch.nn.Linear(a, b, bias=False) for a, b in widths])
+            self.bias = torch.nn.ParameterList([torch.nn.Parameter(torch.zeros(b)) for _, b in widths])
+            self.norms = torch.nn.ModuleList([torch.nn.LayerNorm(b) for _, b in widths[:-1]])
+
+        def forward(self, h):
+            last = len(self.lin_neigh) - 1
+            for i in range(last + 1):
+                agg = Aggregator.apply(graph, h, i, 32, True, True)
+                agg = agg / graph.in_degrees
+                z = self.lin_neigh[i](agg) + self.lin_self[i](h) + self.bias[i]
+                if i == last:
+                    return F.log_softmax(z, dim=1)
+                h = F.relu(self.norms[i](z * masks[i] * 2.0))
+
+    torch.manual_seed(args.seed)
+    model = TorchOpsSage().to(dev)
+    opt = torch.optim.Adam(model.parameters(), lr=0.01)
+
+    def torch_step():
+        opt.zero_grad(set_to_none=True)
+        loss = F.nll_loss(model(x)[train_idx], labels[train_idx])
+        loss.backward()
+        opt.step()
+        return loss.detach()
+
+    out["train_step_ms_torch_ops_around_aggregator"], out["loss_torch_ops_around_aggregator"] = timed(torch_step)
     return out
 
 

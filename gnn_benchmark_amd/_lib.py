@@ -21,6 +21,7 @@ EXPORTS = (
     "gnnagg_plan_create",
     "gnnagg_plan_destroy",
     "gnnagg_plan_spmm_f32",
+    "gnnagg_plan_spmm_strided_f32",
     "gnnagg_plan_info",
     "gnnagg_plan_profile",
     "gnnagg_plan_profile_read",
@@ -32,6 +33,10 @@ EXPORTS = (
     "gnnagg_relu_dropout_backward_f32",
     "gnnagg_wgrad_workspace_bytes",
     "gnnagg_wgrad_f32",
+    "gnnagg_wgrad_strided_f32",
+    "gnnagg_dropout_layernorm_relu_blocks",
+    "gnnagg_dropout_layernorm_relu_f32",
+    "gnnagg_dropout_layernorm_relu_backward_f32",
     "gnnagg_packed_header_words",
     "gnnagg_bias_relu_dropout_pack_f32",
     "gnnagg_relu_dropout_backward_packed_f32",
@@ -83,6 +88,8 @@ def lib() -> ctypes.CDLL:
     L.gnnagg_plan_destroy.argtypes = [vp]
     L.gnnagg_plan_spmm_f32.restype = i32
     L.gnnagg_plan_spmm_f32.argtypes = [vp, vp, vp, vp, i64, i32, vp]
+    L.gnnagg_plan_spmm_strided_f32.restype = i32
+    L.gnnagg_plan_spmm_strided_f32.argtypes = [vp, vp, vp, i64, vp, i64, i64, i32, vp]
     L.gnnagg_plan_info.restype = i32
     L.gnnagg_plan_info.argtypes = [vp, ctypes.POINTER(i64)]
     L.gnnagg_plan_profile.restype = i32
@@ -105,6 +112,14 @@ def lib() -> ctypes.CDLL:
     L.gnnagg_wgrad_workspace_bytes.argtypes = [i64, i64, i64]
     L.gnnagg_wgrad_f32.restype = i32
     L.gnnagg_wgrad_f32.argtypes = [vp, vp, vp, vp, i64, i64, i64, vp]
+    L.gnnagg_wgrad_strided_f32.restype = i32
+    L.gnnagg_wgrad_strided_f32.argtypes = [vp, i64, vp, i64, vp, vp, i64, i64, i64, vp]
+    L.gnnagg_dropout_layernorm_relu_blocks.restype = i32
+    L.gnnagg_dropout_layernorm_relu_blocks.argtypes = [i64, i64]
+    L.gnnagg_dropout_layernorm_relu_f32.restype = i32
+    L.gnnagg_dropout_layernorm_relu_f32.argtypes = [vp, vp, ctypes.c_float, vp, vp, ctypes.c_float, vp, i64, i64, i64, vp]
+    L.gnnagg_dropout_layernorm_relu_backward_f32.restype = i32
+    L.gnnagg_dropout_layernorm_relu_backward_f32.argtypes = [vp, i64, vp, vp, ctypes.c_float, vp, vp, ctypes.c_float, vp, vp, i64, i64, vp]
     L.gnnagg_packed_header_words.restype = i32
     L.gnnagg_packed_header_words.argtypes = [i64]
     L.gnnagg_bias_relu_dropout_pack_f32.restype = i32

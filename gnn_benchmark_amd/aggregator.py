@@ -44,6 +44,7 @@ two forward products that read the features differ.
 import torch
 
 from . import _lib, computation_ops, packed
+from .sparse_tensor import _rows_are_dense
 from .spmm_kernel import SPMM_backward, SPMM_backward_quantized, SPMM_forward, SPMM_forward_quantized
 
 
@@ -121,7 +122,8 @@ class _DenseFeatures:
     """The local features as the forward pipeline reads them: two products and a row gather."""
 
     def __init__(self, feat: torch.Tensor):
-        self.feat = feat.contiguous()
+        # a column block of a wider row-major tensor is read where it lies
+        self.feat = feat if _rows_are_dense(feat) else feat.contiguous()
         self.width, self.device = feat.size(-1), feat.device
 
     def product(self, adj, out, accumulate):
@@ -169,7 +171,16 @@ class AggregatorPacked(torch.autograd.Function):
         return (None, _backward(ctx, local_out_grad), None, None, None, None, None)
 
 
-def _forward(ctx, graph, feats, layer, num_bits: int, is_pre_delay: bool, is_training: bool):
+def _check_result(out: torch.Tensor, rows: int, feat_len: int, device) -> None:
+    if (out.dtype != torch.float32 or out.device != device or tuple(out.shape) != (rows, feat_len)
+            or not _rows_are_dense(out)):
+        raise RuntimeError("Input mismatch: the result must be a float32 [%d, %d] tensor on %s with contiguous rows"
+                           % (rows, feat_len, device))
+
+
+def _forward(ctx, graph, feats, layer, num_bits: int, is_pre_delay: bool, is_training: bool, out=None):
+    """``out``: where to write the result (every row is overwritten) -- e.g. a column block of a
+    wider tensor; a fresh tensor when None."""
     _check_bits(num_bits)
     ctx.graph = graph
     ctx.num_bits = num_bits
@@ -196,12 +207,15 @@ def _forward(ctx, graph, feats, layer, num_bits: int, is_pre_delay: bool, is_tra
         else:
             comm_handle = exchange(graph.comm_splits, graph.comm_buf, f"forward{layer}", "forward")
 
-    out = torch.empty([graph.local_adj_t.sparse_size(0), feat_len], dtype=torch.float32, device=feats.device)
+    if out is None:
+        out = torch.empty([graph.local_adj_t.sparse_size(0), feat_len], dtype=torch.float32, device=feats.device)
+    else:
+        _check_result(out, graph.local_adj_t.sparse_size(0), feat_len, feats.device)
     feats.product(graph.local_adj_t, out, False)
 
     if comm_handle is not None:
         comm_handle.wait()
-    fused = quantized and _fused_dequantize(graph, feat_len)
+    fused = quantized and _fused_dequantize(graph, feat_len) and out.is_contiguous()
     if quantized and not fused:
         _dequantize_received(graph, num_bits, "forward")
 
@@ -217,13 +231,16 @@ def _forward(ctx, graph, feats, layer, num_bits: int, is_pre_delay: bool, is_tra
     return out
 
 
-def _backward(ctx, local_out_grad):
+def _backward(ctx, local_out_grad, out=None, accumulate: bool = False):
+    """``out`` / ``accumulate``: write the gradient into ``out`` (a column block of a wider tensor
+    is fine), on top of what it holds when ``accumulate``; a fresh tensor when ``out`` is None."""
     graph = ctx.graph
     num_bits = ctx.num_bits
     is_pre_delay = ctx.is_pre_delay
     layer = f"backward{ctx.layer}"
 
-    local_out_grad = local_out_grad.contiguous()
+    if not _rows_are_dense(local_out_grad):
+        local_out_grad = local_out_grad.contiguous()
     feat_len = local_out_grad.size(-1)
     graph.comm_buf.resize_buffer(graph.comm_splits, feat_len, num_bits)
     exchange = getattr(graph, "exchange", None)
@@ -245,13 +262,18 @@ def _backward(ctx, local_out_grad):
     elif exchange is not None:
         comm_handle = exchange(graph.comm_splits, graph.comm_buf, layer, "backward")
 
-    local_nodes_grad = torch.empty([graph.local_adj_t.sparse_size(-1), feat_len], dtype=torch.float32,
-                                   device=local_out_grad.device)
-    SPMM_backward(graph.local_adj_t, local_out_grad, local_nodes_grad, accumulate=False)
+    if out is None:
+        local_nodes_grad = torch.empty([graph.local_adj_t.sparse_size(-1), feat_len], dtype=torch.float32,
+                                       device=local_out_grad.device)
+        accumulate = False
+    else:
+        _check_result(out, graph.local_adj_t.sparse_size(-1), feat_len, local_out_grad.device)
+        local_nodes_grad = out
+    SPMM_backward(graph.local_adj_t, local_out_grad, local_nodes_grad, accumulate=accumulate)
 
     if comm_handle is not None:
         comm_handle.wait()
-    fused = quantized and _fused_dequantize(graph, feat_len)
+    fused = quantized and _fused_dequantize(graph, feat_len) and local_nodes_grad.is_contiguous()
     if quantized and not fused:
         _dequantize_received(graph, num_bits, "backward")
 

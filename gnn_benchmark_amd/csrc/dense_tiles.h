@@ -13,22 +13,29 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 constexpr int kChunk = 16;    // rows per LDS stage
 constexpr int kLdsPad = 32;   // floats: shifts the second row of a k-pair onto the other half of the banks
 
-// One operand's share of the loader: thread t moves float4 number t + 256*j of the chunk.
+// One operand's share of the loader: thread t moves float4 number t + 256*j of the chunk's
+// kChunk * width values.  The rows may sit `stride` floats apart in global memory (a column
+// block of a wider row-major array).
 template <int NV, int LD>
 struct ChunkLoader {
     int lds_off[NV];   // destination (floats) inside one LDS buffer, or -1 for a vector beyond the chunk
-    int src_off[NV];   // source offset (floats) from the start of the chunk, clamped to 0 when unused
+    int elem[NV];      // number of the vector's first value inside the chunk, 0 when unused
+    int src_off[NV];   // where that value sits (floats from the start of the chunk's first row), 0 when unused
     floatx4 reg[NV];
-    int width;
+    int width, stride;
 
-    __device__ void init(int tid, int w) {
+    __device__ int offset_of(int e) const { return (e / width) * stride + e % width; }
+
+    __device__ void init(int tid, int w, int ld) {
         width = w;
+        stride = ld;
 #pragma unroll
         for (int j = 0; j < NV; ++j) {
             const int e = 4 * (tid + 256 * j);
             const bool used = e < kChunk * w;
             lds_off[j] = used ? (e / w) * LD + (e % w) : -1;
-            src_off[j] = used ? e : 0;
+            elem[j] = used ? e : 0;
+            src_off[j] = used ? offset_of(e) : 0;
         }
     }
     // all kChunk rows exist
@@ -37,21 +44,21 @@ struct ChunkLoader {
         for (int j = 0; j < NV; ++j)
             reg[j] = __builtin_nontemporal_load(reinterpret_cast<const floatx4 *>(chunk + src_off[j]));
     }
-    // only `valid` floats exist; the rest of the chunk reads as zeros.  `aligned` is false when rows
-    // are not a whole number of float4 (then fetch() is never used either).
+    // only the first `valid` values of the chunk exist; the rest reads as zeros.  `aligned` is false
+    // when rows are not a whole number of float4 (then fetch() is never used either).
     __device__ void fetch_tail(const float *chunk, int valid, bool aligned) {
 #pragma unroll
         for (int j = 0; j < NV; ++j) {
             floatx4 v = {0.f, 0.f, 0.f, 0.f};
-            const int e = src_off[j];
+            const int e = elem[j];
             if (lds_off[j] >= 0) {
                 if (aligned) {
-                    if (e < valid) v = *reinterpret_cast<const floatx4 *>(chunk + e);
+                    if (e < valid) v = *reinterpret_cast<const floatx4 *>(chunk + src_off[j]);
                 } else {
-                    if (e + 0 < valid) v.x = chunk[e + 0];
-                    if (e + 1 < valid) v.y = chunk[e + 1];
-                    if (e + 2 < valid) v.z = chunk[e + 2];
-                    if (e + 3 < valid) v.w = chunk[e + 3];
+                    if (e + 0 < valid) v.x = chunk[offset_of(e + 0)];
+                    if (e + 1 < valid) v.y = chunk[offset_of(e + 1)];
+                    if (e + 2 < valid) v.z = chunk[offset_of(e + 2)];
+                    if (e + 3 < valid) v.w = chunk[offset_of(e + 3)];
                 }
             }
             reg[j] = v;
@@ -71,7 +78,7 @@ struct ChunkLoader {
             if (aligned) {
                 *reinterpret_cast<floatx4 *>(buf + lds_off[j]) = reg[j];
             } else {  // a float4 of the stream may straddle two rows
-                const int e = src_off[j];
+                const int e = elem[j];
                 const float v[4] = {reg[j].x, reg[j].y, reg[j].z, reg[j].w};
 #pragma unroll
                 for (int q = 0; q < 4; ++q)

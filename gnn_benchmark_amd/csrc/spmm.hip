@@ -31,12 +31,16 @@ struct Shape {
 constexpr int kShapes[][2] = {{16, 1}, {32, 1}, {64, 1}, {64, 2}, {64, 3}, {64, 4}, {64, 5}, {64, 6}, {64, 8}};
 constexpr int kNumShapes = sizeof(kShapes) / sizeof(kShapes[0]);
 
-int pick_vec(int64_t feat, const void *x, const void *dst) {
-    const uintptr_t bits = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dst);
+// widest vector access that every row of x and dst allows: base addresses and row strides
+// (in floats; rows back to back when the stride is the width) must be multiples of it
+int pick_vec(int64_t feat, const void *x, const void *dst, int64_t ldx, int64_t ldd) {
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dst) |
+                           (uintptr_t)(ldx * 4) | (uintptr_t)(ldd * 4);
     if (feat % 4 == 0 && bits % 16 == 0) return 4;
     if (feat % 2 == 0 && bits % 8 == 0) return 2;
     return 1;
 }
+int pick_vec(int64_t feat, const void *x, const void *dst) { return pick_vec(feat, x, dst, feat, feat); }
 
 Shape pick_shape(int vec, int64_t feat_left) {
     for (int i = 0; i < kNumShapes; ++i) {
@@ -436,17 +440,23 @@ extern "C" int gnnagg_plan_info(const gnnagg_plan *plan, int64_t *info) {
     return GNNAGG_OK;
 }
 
-extern "C" int gnnagg_plan_spmm_f32(gnnagg_plan *plan, const float *value, const float *mat, float *out, int64_t feat,
-                                    int accumulate, void *stream) {
+namespace gnnagg {
+namespace {
+
+int plan_spmm(gnnagg_plan *plan, const float *value, const float *mat, int64_t ldx, float *out, int64_t ldd,
+              int64_t feat, int accumulate, void *stream) {
     GNNAGG_REQUIRE(plan, "null plan");
     GNNAGG_REQUIRE(feat >= 0, "negative feature width");
     if (plan->rows == 0 || feat == 0) return GNNAGG_OK;
     GNNAGG_REQUIRE(out, "null out");
     GNNAGG_REQUIRE(plan->nnz == 0 || (value && mat), "null value/mat");
     if (int rc = check_feat(feat)) return rc;
+    GNNAGG_REQUIRE(ldx >= feat && ldd >= feat && ldx < (int64_t(1) << 31) && ldd < (int64_t(1) << 31),
+                   "row strides %lld / %lld must be at least the width %lld and below 2^31", (long long)ldx,
+                   (long long)ldd, (long long)feat);
     hipStream_t st = static_cast<hipStream_t>(stream);
 
-    const int vec = pick_vec(feat, mat, out);
+    const int vec = pick_vec(feat, mat, out, ldx, ldd);
     // accumulate: empty rows keep their value, so they are not visited at all
     const int64_t nshort = plan->rows - plan->nlong - (accumulate ? plan->nempty : 0);
     const bool prof = plan->profile;
@@ -466,6 +476,8 @@ extern "C" int gnnagg_plan_spmm_f32(gnnagg_plan *plan, const float *value, const
         la.x = mat;
         la.dst = out;
         la.feat = (int)feat;
+        la.ldx = (int)ldx;
+        la.ldd = (int)ldd;
         la.accumulate = accumulate;
         if (vec == 4) GNNAGG_HIP(launch_long_rows<4>(la, plan->nhuge, plan->side));
         else if (vec == 2) GNNAGG_HIP(launch_long_rows<2>(la, plan->nhuge, plan->side));
@@ -481,6 +493,8 @@ extern "C" int gnnagg_plan_spmm_f32(gnnagg_plan *plan, const float *value, const
         a.x = mat;
         a.dst = out;
         a.feat = (int)feat;
+        a.ldx = (int)ldx;
+        a.ldd = (int)ldd;
         a.f_base = (int)f_base;
         a.accumulate = accumulate;
         // one launch over the rows, longest first; the rows above the long-row threshold
@@ -503,6 +517,20 @@ extern "C" int gnnagg_plan_spmm_f32(gnnagg_plan *plan, const float *value, const
     if (plan->nhuge > 0) GNNAGG_HIP(hipStreamWaitEvent(st, plan->join, 0));
     if (prof) GNNAGG_HIP(hipEventRecord(plan->ev[3], st));
     return GNNAGG_OK;
+}
+
+}  // namespace
+}  // namespace gnnagg
+
+extern "C" int gnnagg_plan_spmm_f32(gnnagg_plan *plan, const float *value, const float *mat, float *out, int64_t feat,
+                                    int accumulate, void *stream) {
+    return plan_spmm(plan, value, mat, feat, out, feat, feat, accumulate, stream);
+}
+
+extern "C" int gnnagg_plan_spmm_strided_f32(gnnagg_plan *plan, const float *value, const float *mat,
+                                            int64_t mat_stride, float *out, int64_t out_stride, int64_t feat,
+                                            int accumulate, void *stream) {
+    return plan_spmm(plan, value, mat, mat_stride, out, out_stride, feat, accumulate, stream);
 }
 
 extern "C" int gnnagg_plan_spmm_packed_f32(gnnagg_plan *plan, const float *value, const float *y_packed,

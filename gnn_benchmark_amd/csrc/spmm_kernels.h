@@ -154,7 +154,8 @@ struct SpmmArgs {
     int qbits;
     float *dst;               // out [rows, F]
     int64_t ntasks;
-    int feat;                 // F (row stride of x and dst, in floats)
+    int feat;                 // F
+    int ldx, ldd;             // row strides of x and dst in floats; 0 stands for F (rows back to back)
     int f_base;               // first feature handled by this launch
     int accumulate;           // start every row from dst (1) or from 0 (0)
     int tasks_per_block;      // tasks handled by one block past the head region
@@ -211,6 +212,7 @@ __device__ __forceinline__ void gather_fma(FVec<VEC> (&acc)[NCH], IdxT c_l, floa
                                            const int (&foff)[NCH]) {
     const float *__restrict__ x = a.x;
     const int F = a.feat;
+    const int ldx = a.ldx ? a.ldx : F;
     const float *xr[UU];
     float vv[UU];
     int64_t cc[UU];
@@ -218,7 +220,7 @@ __device__ __forceinline__ void gather_fma(FVec<VEC> (&acc)[NCH], IdxT c_l, floa
     for (int u = 0; u < UU; ++u) {
         cc[u] = group_bcast_idx<LPR>(c_l, j + u);
         vv[u] = __int_as_float(group_bcast<LPR>(__float_as_int(v_l), j + u));
-        xr[u] = x + (size_t)cc[u] * (size_t)F;
+        xr[u] = x + (size_t)cc[u] * (size_t)ldx;
     }
     FVec<VEC> xv[UU][NCH];
     if constexpr (SRC == kSrcPacked) {
@@ -312,7 +314,6 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
 
     const IdxT *__restrict__ col = static_cast<const IdxT *>(a.col);
     const float *__restrict__ val = a.val;
-    const float *__restrict__ x = a.x;
     const int F = a.feat;
 
     // Lanes past the end of the feature row keep a valid address (the first feature of
@@ -378,7 +379,8 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
         v_l = __builtin_nontemporal_load(val + base + lig);
     }
     const bool from_dst = a.accumulate != 0;
-    float *dst = a.dst + (size_t)row * (size_t)F;
+    const int ldd = a.ldd ? a.ldd : F;
+    float *dst = a.dst + (size_t)row * (size_t)ldd;
     V acc[NCH];
 #pragma unroll
     for (int k = 0; k < NCH; ++k) {
@@ -432,7 +434,7 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
                 if (fok[k]) acc[k].store_stream(dst + foff[k]);
             }
             if (!more) break;
-            dst = a.dst + (size_t)nrow * (size_t)F;
+            dst = a.dst + (size_t)nrow * (size_t)ldd;
 #pragma unroll
             for (int k = 0; k < NCH; ++k) {
                 acc[k] = V::zero();
@@ -472,6 +474,7 @@ struct LongArgs {
     const float *x;
     float *dst;
     int feat;        // F
+    int ldx, ldd;    // row strides of x and dst in floats; 0 stands for F
     int chunk;       // dense rows per chunk: chunk * min(F, 256) <= kLongTileFloats, chunk * (tile / VEC) <= 2048
     int accumulate;
 };
@@ -489,6 +492,7 @@ __global__ __launch_bounds__(256) void spmm_long_rows_kernel(const LongArgs a) {
     const int t = (int)threadIdx.x;
     const RowTask d = a.task[blockIdx.x];
     const int F = a.feat;
+    const int ldx = a.ldx ? a.ldx : F;
     const int f0 = (int)blockIdx.y * kLongFeatTile;
     const int fw = F - f0 < kLongFeatTile ? F - f0 : kLongFeatTile;  // width of this tile (multiple of VEC)
     const int vpr = fw / VEC;                                        // vectors per gathered row
@@ -520,14 +524,14 @@ __global__ __launch_bounds__(256) void spmm_long_rows_kernel(const LongArgs a) {
 #pragma unroll
         for (int s = 0; s < kLongLoads; ++s) {
             if (sj[s] < cnt) {
-                const V v = V::load(x + (size_t)s_col[0][sj[s]] * (size_t)F + sv[s]);
+                const V v = V::load(x + (size_t)s_col[0][sj[s]] * (size_t)ldx + sv[s]);
                 v.store(&tile[0][sj[s] * fw + sv[s]]);
             }
         }
     }
     __syncthreads();
 
-    float *dst = a.dst + (size_t)d.row * (size_t)F + f0;
+    float *dst = a.dst + (size_t)d.row * (size_t)(a.ldd ? a.ldd : F) + f0;
     float acc = 0.0f;
     const bool own = t < fw;
     if (own && a.accumulate) acc = __builtin_nontemporal_load(dst + t);
@@ -539,7 +543,7 @@ __global__ __launch_bounds__(256) void spmm_long_rows_kernel(const LongArgs a) {
         V g[kLongLoads];
 #pragma unroll
         for (int s = 0; s < kLongLoads; ++s) {
-            if (sj[s] < ncnt) g[s] = V::load(x + (size_t)s_col[(k + 1) % 3][sj[s]] * (size_t)F + sv[s]);
+            if (sj[s] < ncnt) g[s] = V::load(x + (size_t)s_col[(k + 1) % 3][sj[s]] * (size_t)ldx + sv[s]);
         }
         int ci = 0;
         float vi = 0.0f;

@@ -32,7 +32,8 @@ template <int WM, int WN>
 __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__restrict__ x,
                                                                const float *__restrict__ g,
                                                                float *__restrict__ partial, int64_t rows, int fi,
-                                                               int fo, int64_t rows_per_block, int aligned) {
+                                                               int fo, int ldx, int ldg, int64_t rows_per_block,
+                                                               int aligned) {
     using S = WgradShape<WM, WN>;
     extern __shared__ __align__(16) float smem[];
     float *xs = smem;                              // [2][kChunk][kLdx]
@@ -65,8 +66,8 @@ __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__re
 
     ChunkLoader<S::kVecX, S::kLdx> lx;
     ChunkLoader<S::kVecG, S::kLdg> lg;
-    lx.init(tid, fi);
-    lg.init(tid, fo);
+    lx.init(tid, fi, ldx);
+    lg.init(tid, fo, ldg);
 
     // Columns past fi / fo of an LDS row are never written: whatever they hold only reaches
     // accumulator entries that are never stored.
@@ -98,9 +99,9 @@ __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__re
     // steady state: whole chunks, no masks; the next chunk's global loads are in flight behind
     // this chunk's MFMAs and land in the other LDS buffer
     if (full > 0) {
-        const float *xc = x + (size_t)r_begin * (size_t)fi;
-        const float *gc = g + (size_t)r_begin * (size_t)fo;
-        const size_t xstep = (size_t)kChunk * (size_t)fi, gstep = (size_t)kChunk * (size_t)fo;
+        const float *xc = x + (size_t)r_begin * (size_t)ldx;
+        const float *gc = g + (size_t)r_begin * (size_t)ldg;
+        const size_t xstep = (size_t)kChunk * (size_t)ldx, gstep = (size_t)kChunk * (size_t)ldg;
         lx.fetch(xc);
         lg.fetch(gc);
         lx.store_all(xs, dump);
@@ -123,8 +124,8 @@ __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__re
     // what is left: the slice's last, partial chunk, or every chunk when 16-byte copies are not possible
     for (int64_t r = r_begin + full * kChunk; r < r_end; r += kChunk) {
         const int left = (int)(r_end - r < kChunk ? r_end - r : kChunk);
-        lx.fetch_tail(x + (size_t)r * (size_t)fi, left * fi, aligned != 0);
-        lg.fetch_tail(g + (size_t)r * (size_t)fo, left * fo, aligned != 0);
+        lx.fetch_tail(x + (size_t)r * (size_t)ldx, left * fi, aligned != 0);
+        lg.fetch_tail(g + (size_t)r * (size_t)ldg, left * fo, aligned != 0);
         lx.store(xs, aligned != 0);
         lg.store(gs, aligned != 0);
         __syncthreads();
@@ -174,7 +175,16 @@ extern "C" int64_t gnnagg_wgrad_workspace_bytes(int64_t rows, int64_t fi, int64_
 
 extern "C" int gnnagg_wgrad_f32(const float *x, const float *g, float *w_grad, void *workspace, int64_t rows, int64_t fi,
                                 int64_t fo, void *stream) {
+    return gnnagg_wgrad_strided_f32(x, fi, g, fo, w_grad, workspace, rows, fi, fo, stream);
+}
+
+extern "C" int gnnagg_wgrad_strided_f32(const float *x, int64_t x_stride, const float *g, int64_t g_stride,
+                                        float *w_grad, void *workspace, int64_t rows, int64_t fi, int64_t fo,
+                                        void *stream) {
     GNNAGG_REQUIRE(rows >= 0 && fi > 0 && fo > 0, "bad size");
+    GNNAGG_REQUIRE(x_stride >= fi && g_stride >= fo && x_stride < (int64_t(1) << 27) && g_stride < (int64_t(1) << 27),
+                   "row strides %lld / %lld must be at least the widths %lld / %lld and below 2^27",
+                   (long long)x_stride, (long long)g_stride, (long long)fi, (long long)fo);
     if (fi > 256 || fo > 256)
         return fail(GNNAGG_ERR_UNSUPPORTED, "weight-gradient kernel handles Fi, Fo <= 256 (got %lld, %lld)", (long long)fi,
                     (long long)fo);
@@ -191,8 +201,8 @@ extern "C" int gnnagg_wgrad_f32(const float *x, const float *g, float *w_grad, v
     const int blocks = wgrad_blocks(rows);
     // whole chunks per block, so that only a slice's last chunk is partial
     const int64_t rpb = ((rows + blocks - 1) / blocks + kChunk - 1) / kChunk * kChunk;
-    const int aligned = (fi % 4 == 0 && fo % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
-                         (reinterpret_cast<uintptr_t>(g) & 15) == 0)
+    const int aligned = (fi % 4 == 0 && fo % 4 == 0 && x_stride % 4 == 0 && g_stride % 4 == 0 &&
+                         (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(g) & 15) == 0)
                             ? 1
                             : 0;
     float *partial = static_cast<float *>(workspace);
@@ -203,7 +213,7 @@ extern "C" int gnnagg_wgrad_f32(const float *x, const float *g, float *w_grad, v
         constexpr size_t smem = (size_t)WgradShape<M, N>::kSmemFloats * sizeof(float);                       \
         GNNAGG_HIP(allow_lds(reinterpret_cast<const void *>(&wgrad_partial_kernel<M, N>), smem));           \
         hipLaunchKernelGGL((wgrad_partial_kernel<M, N>), dim3((unsigned)blocks), dim3(256), smem, st, x, g,  \
-                           partial, rows, (int)fi, (int)fo, rpb, aligned);                                   \
+                           partial, rows, (int)fi, (int)fo, (int)x_stride, (int)g_stride, rpb, aligned);     \
     } else
     GNNAGG_WGRAD(1, 1) GNNAGG_WGRAD(1, 2) GNNAGG_WGRAD(1, 3) GNNAGG_WGRAD(1, 4) GNNAGG_WGRAD(2, 1) GNNAGG_WGRAD(2, 2)
     GNNAGG_WGRAD(2, 3) GNNAGG_WGRAD(2, 4) GNNAGG_WGRAD(3, 1) GNNAGG_WGRAD(3, 2) GNNAGG_WGRAD(3, 3) GNNAGG_WGRAD(3, 4)

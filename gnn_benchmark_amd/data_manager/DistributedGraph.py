@@ -34,6 +34,7 @@ class DistributedGraph:
     comm_buf_for_quantization: Any = None      # CommBufferForQuantization for bits 2 / 4 / 8
     exchange: Optional[Callable] = None
     exchange_quantized: Optional[Callable] = None
+    in_degrees_folded: bool = False            # the matrices' rows already carry 1 / in_degrees
     _scatter: Optional[SparseTensor] = field(default=None, repr=False)
 
     def send_scatter_adj_t(self) -> SparseTensor:
@@ -63,3 +64,4 @@ class DistributedGraphForPre:
     comm_buf_for_quantization: Any = None
     exchange: Optional[Callable] = None
     exchange_quantized: Optional[Callable] = None
+    in_degrees_folded: bool = False

@@ -19,6 +19,7 @@ import torch.nn.functional as F
 
 from . import _lib, packed
 from .aggregator import Aggregator, AggregatorPacked
+from .sparse_tensor import _row_stride, _rows_are_dense
 
 
 class _Bf16InputLinear(torch.autograd.Function):
@@ -46,8 +47,12 @@ class _Bf16InputLinear(torch.autograd.Function):
 
 def weight_gradient(x: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
     """x^T @ g for tall-skinny fp32 operands through the library's MFMA kernel; falls back to
-    the BLAS library for shapes that kernel does not take (more than 256 columns)."""
-    x, g = x.contiguous(), g.contiguous()
+    the BLAS library for shapes that kernel does not take (more than 256 columns).  Column
+    blocks of wider row-major tensors are read where they lie."""
+    if not _rows_are_dense(x):
+        x = x.contiguous()
+    if not _rows_are_dense(g):
+        g = g.contiguous()
     rows, fi, fo = x.size(0), x.size(1), g.size(1)
     L = _lib.lib()
     nbytes = int(L.gnnagg_wgrad_workspace_bytes(rows, fi, fo)) if x.is_cuda and x.dtype == torch.float32 else 0
@@ -56,8 +61,8 @@ def weight_gradient(x: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
     out = torch.empty(fi, fo, dtype=torch.float32, device=x.device)
     workspace = torch.empty(nbytes // 4, dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
-        _lib.check(L.gnnagg_wgrad_f32(_lib.ptr(x), _lib.ptr(g), _lib.ptr(out), _lib.ptr(workspace), rows, fi, fo,
-                                      _lib.current_stream(x.device)))
+        _lib.check(L.gnnagg_wgrad_strided_f32(_lib.ptr(x), _row_stride(x), _lib.ptr(g), _row_stride(g), _lib.ptr(out),
+                                              _lib.ptr(workspace), rows, fi, fo, _lib.current_stream(x.device)))
     return out
 
 

@@ -52,20 +52,29 @@ class SpmmPlan:
         return float(buf[0]), float(buf[1])
 
     def spmm(self, value: torch.Tensor, mat: torch.Tensor, out: torch.Tensor, accumulate: bool = True) -> torch.Tensor:
+        """``out (+)= A @ mat``.  ``mat`` and ``out`` may be column blocks of wider row-major
+        tensors (unit stride along the features, any row stride): they are used in place."""
         if not (value.is_cuda and mat.is_cuda and out.is_cuda):
             raise RuntimeError("value, mat and out must be GPU (HIP) tensors; there is no CPU path")
         if value.dtype != torch.float32 or mat.dtype != torch.float32 or out.dtype != torch.float32:
             raise RuntimeError("Input mismatch: value/mat/out must be float32")
-        if mat.dim() != 2 or out.dim() != 2 or not out.is_contiguous():
-            raise RuntimeError("Input mismatch: mat/out must be 2-D and out contiguous")
+        if mat.dim() != 2 or out.dim() != 2 or not _rows_are_dense(out):
+            raise RuntimeError("Input mismatch: mat/out must be 2-D and the rows of out contiguous")
         if value.numel() != self.nnz or mat.size(0) < self.cols or out.size(0) < self.rows or out.size(1) != mat.size(1):
             raise RuntimeError("Input mismatch: operand shapes do not match the planned matrix")
-        mat = mat.contiguous()
+        if not _rows_are_dense(mat):
+            mat = mat.contiguous()
         value = value.contiguous()
+        feat = mat.size(1)
         with torch.cuda.device(self.device):
-            _lib.check(_lib.lib().gnnagg_plan_spmm_f32(self._handle, _lib.ptr(value), _lib.ptr(mat), _lib.ptr(out),
-                                                       mat.size(1), 1 if accumulate else 0,
-                                                       _lib.current_stream(self.device)))
+            if mat.is_contiguous() and out.is_contiguous():
+                _lib.check(_lib.lib().gnnagg_plan_spmm_f32(self._handle, _lib.ptr(value), _lib.ptr(mat), _lib.ptr(out),
+                                                           feat, 1 if accumulate else 0,
+                                                           _lib.current_stream(self.device)))
+            else:
+                _lib.check(_lib.lib().gnnagg_plan_spmm_strided_f32(
+                    self._handle, _lib.ptr(value), _lib.ptr(mat), _row_stride(mat), _lib.ptr(out), _row_stride(out),
+                    feat, 1 if accumulate else 0, _lib.current_stream(self.device)))
         return out
 
     def __del__(self):
@@ -75,6 +84,15 @@ class SpmmPlan:
                 _lib.lib().gnnagg_plan_destroy(h)
             except Exception:  # interpreter shutdown
                 pass
+
+
+def _rows_are_dense(t: torch.Tensor) -> bool:
+    """2-D, unit stride along each row, rows not overlapping (a column block of a row-major tensor)."""
+    return t.dim() == 2 and (t.size(1) <= 1 or t.stride(1) == 1) and (t.size(0) <= 1 or t.stride(0) >= t.size(1))
+
+
+def _row_stride(t: torch.Tensor) -> int:
+    return t.stride(0) if t.size(0) > 1 else t.size(1)
 
 
 def _coo_to_csr_host(row, col, value, rows):

@@ -92,6 +92,15 @@ int gnnagg_plan_destroy(gnnagg_plan *plan);
 int gnnagg_plan_spmm_f32(gnnagg_plan *plan, const float *value, const float *mat, float *out, int64_t feat,
                          int accumulate, void *stream);
 
+/* The same product for operands that are column blocks of wider row-major arrays: row r of
+ * mat starts at mat + r * mat_stride, row r of out at out + r * out_stride (strides in
+ * floats, each at least feat).  This is what lets a layer keep [A x | x] side by side in one
+ * [rows, 2 * feat] array and run lin_neigh and lin_self (model/layers/sageconv.py:87-88) as
+ * ONE dense product, without copying either half: the aggregation reads the right half and
+ * writes the left one.  Results equal gnnagg_plan_spmm_f32 on contiguous copies bit for bit. */
+int gnnagg_plan_spmm_strided_f32(gnnagg_plan *plan, const float *value, const float *mat, int64_t mat_stride,
+                                 float *out, int64_t out_stride, int64_t feat, int accumulate, void *stream);
+
 /* Host-side description of a plan, info[0..7] (host pointer):
  * rows, cols, nnz, rows handled by the block-per-row kernel (longer than the next
  * entry), that length threshold, rows with no stored element, largest row length, rows
@@ -176,6 +185,34 @@ int gnnagg_relu_dropout_backward_f32(const float *grad_y, const float *y, const 
 int64_t gnnagg_wgrad_workspace_bytes(int64_t rows, int64_t fi, int64_t fo);
 int gnnagg_wgrad_f32(const float *x, const float *g, float *w_grad, void *workspace, int64_t rows, int64_t fi,
                      int64_t fo, void *stream);
+/* The same with x and / or g being column blocks of wider row-major arrays (row strides in
+ * floats): the two halves of a SAGE layer's [A x | x] operand are read where they lie. */
+int gnnagg_wgrad_strided_f32(const float *x, int64_t x_stride, const float *g, int64_t g_stride, float *w_grad,
+                             void *workspace, int64_t rows, int64_t fi, int64_t fo, void *stream);
+
+/* ---------------------------------------------------------------------------------
+ * The elementwise chain between two SAGE layers (model/DistSAGE.py:49-53: F.dropout, LayerNorm
+ * over the features, F.relu) as one pass each way:
+ *   y = relu(layer_norm(z * keep * scale; gamma, beta, eps))
+ * z fp32 [rows, feat] contiguous (the layer output), keep uint8 [rows, feat] (NULL: nothing
+ * dropped), gamma / beta fp32 [feat].  y is written with row stride y_stride floats: the next
+ * layer keeps its input in the right half of a [rows, 2 * feat] array whose left half receives
+ * the aggregation (gnnagg_plan_spmm_strided_f32).  The backward takes the gradient with its own
+ * row stride, the SAME z / keep / scale / gamma / beta / eps (the row moments are taken again,
+ * nothing else is kept from the forward), writes grad_z fp32 [rows, feat] and, when `partial`
+ * is given, per-block sums for the LayerNorm parameters: partial fp32 [blocks, 2, feat]
+ * (blocks = gnnagg_dropout_layernorm_relu_blocks(rows, feat)); summing partial[:, 0, :] over the
+ * blocks gives d/d gamma, partial[:, 1, :] d/d beta.  feat % 4 == 0, feat <= 1024
+ * (GNNAGG_ERR_UNSUPPORTED otherwise; _blocks returns 0).  Allocates nothing, no host sync.
+ * ------------------------------------------------------------------------------- */
+int gnnagg_dropout_layernorm_relu_blocks(int64_t rows, int64_t feat);
+int gnnagg_dropout_layernorm_relu_f32(const float *z, const uint8_t *keep, float scale, const float *gamma,
+                                      const float *beta, float eps, float *y, int64_t y_stride, int64_t rows,
+                                      int64_t feat, void *stream);
+int gnnagg_dropout_layernorm_relu_backward_f32(const float *grad_y, int64_t grad_stride, const float *z,
+                                               const uint8_t *keep, float scale, const float *gamma,
+                                               const float *beta, float eps, float *grad_z, float *partial,
+                                               int64_t rows, int64_t feat, void *stream);
 
 /* ---------------------------------------------------------------------------------
  * Packed activations: the output of a ReLU + dropout layer with every row's non-zero values

@@ -103,7 +103,7 @@ def test_train_step_matches_cpu_autograd(gemm, tol):
     cpu_loss = F.nll_loss(F.log_softmax(h, dim=1)[train_idx.cpu()], labels.cpu()[train_idx.cpu()])
     cpu_loss.backward()
 
-    assert abs(float(loss.detach()) - float(cpu_loss.detach())) <= tol * max(1.0, abs(float(cpu_loss)))
+    assert abs(float(loss.detach()) - float(cpu_loss.detach())) <= tol * max(1.0, abs(float(cpu_loss.detach())))
     for (name, p_gpu), p_cpu in zip(model.named_parameters(), cpu_model.parameters()):
         scale = float(p_cpu.grad.abs().max()) + 1e-12
         assert float((p_gpu.grad.cpu() - p_cpu.grad).abs().max()) <= 10 * tol * scale, name
@@ -112,7 +112,7 @@ def test_train_step_matches_cpu_autograd(gemm, tol):
     before = [p.detach().clone() for p in model.parameters()]
     losses = [float(gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks)) for _ in range(5)]
     assert all(np.isfinite(losses)) and losses[-1] < losses[0]
-    assert abs(losses[0] - float(cpu_loss)) <= tol * max(1.0, abs(float(cpu_loss)))
+    assert abs(losses[0] - float(cpu_loss.detach())) <= tol * max(1.0, abs(float(cpu_loss.detach())))
     for b, p in zip(before, model.parameters()):
         assert float((p.detach() - b).abs().max()) <= 5 * 0.01 * 1.01
 

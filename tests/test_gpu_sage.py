@@ -1,0 +1,298 @@
+"""The layer and model that call the aggregation path (DistSAGEConvGrad, DistSAGE) and the
+pieces they are made of: SpMM on column blocks of wider arrays, the weight gradient on such
+blocks, and the fused dropout -> LayerNorm -> ReLU pass.
+
+* Strided operands must give the SAME BITS as contiguous copies (same kernels, same chains).
+* The fused LayerNorm pass is checked against torch's own ops on the CPU in fp64-free fp32:
+  tolerance 2e-5 absolute on outputs of unit scale (moments are summed in another order).
+* Layer and model are checked against an independent CPU autograd run written with torch
+  modules the way the reference writes them (two Linears, F.dropout with the same mask,
+  nn.LayerNorm, relu; model/layers/sageconv.py:65-93, model/DistSAGE.py:43-69), aggregation by
+  torch.sparse on the CPU: tolerance 1e-4 relative (dense products sum in another order).
+"""
+import copy
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from gnn_benchmark_amd import gcn, sage, synthetic
+from gnn_benchmark_amd.data_manager import CommBuffer, CommSplits, DistributedGraphForPre
+from gnn_benchmark_amd.sparse_tensor import SparseTensor
+from gnn_benchmark_amd.spmm_kernel import SPMM_backward, SPMM_forward
+from gpu_util import dev, skewed_csr
+
+pytestmark = pytest.mark.gpu
+
+
+# ------------------------------------------------------------------ strided operands
+@pytest.mark.parametrize("feat", [4, 32, 100, 128, 256, 602, 7, 30])
+@pytest.mark.parametrize("with_block_rows", [False, True])
+def test_spmm_on_column_blocks_equals_contiguous(feat, with_block_rows, monkeypatch):
+    if with_block_rows:
+        monkeypatch.setenv("GNNAGG_HUGE_THRESH", "2048")
+    rowptr, col, val = skewed_csr(900, 900, seed=feat, heavy_rows=(5000, 2500, 300))
+    src = SparseTensor(rowptr=dev(rowptr), col=dev(col), value=dev(val), sparse_sizes=(900, 900))
+    assert (src.get_plan().info()["huge_rows"] > 0) == with_block_rows
+    gen = torch.Generator(device="cuda").manual_seed(feat)
+    wide_in = torch.randn(900, 2 * feat + 8, device="cuda", generator=gen)
+    wide_out = torch.randn(900, 3 * feat, device="cuda", generator=gen)
+    x_view, out_view = wide_in[:, feat + 8:], wide_out[:, feat:2 * feat]
+    before = wide_out.clone()
+
+    for accumulate in (True, False):
+        for op in (SPMM_forward, SPMM_backward):
+            wide_out.copy_(before)
+            want = out_view.clone().contiguous()
+            op(src, x_view.contiguous(), want, accumulate=accumulate)
+            op(src, x_view, out_view, accumulate=accumulate)
+            assert torch.equal(out_view, want), (op.__name__, accumulate)
+            # nothing outside the block was touched
+            assert torch.equal(wide_out[:, :feat], before[:, :feat])
+            assert torch.equal(wide_out[:, 2 * feat:], before[:, 2 * feat:])
+    # the same tensor may hold source and result: right half in, left half out
+    both = torch.randn(900, 2 * feat, device="cuda", generator=gen)
+    want = torch.empty(900, feat, device="cuda")
+    SPMM_forward(src, both[:, feat:].contiguous(), want, accumulate=False)
+    SPMM_forward(src, both[:, feat:], both[:, :feat], accumulate=False)
+    assert torch.equal(both[:, :feat], want)
+
+
+def test_strided_spmm_rejects_rows_that_overlap_or_are_not_dense():
+    rowptr, col, val = skewed_csr(50, 50, seed=1, heavy_rows=(20,))
+    src = SparseTensor(rowptr=dev(rowptr), col=dev(col), value=dev(val), sparse_sizes=(50, 50))
+    x = torch.randn(50, 8, device="cuda")
+    with pytest.raises(RuntimeError, match="rows of out contiguous"):
+        SPMM_forward(src, x, torch.zeros(8, 50, device="cuda").t())
+    with pytest.raises(RuntimeError, match="rows of out contiguous"):
+        SPMM_forward(src, x, torch.zeros(1, 8, device="cuda").expand(50, 8))
+    # a source that is not row-dense is copied, not rejected
+    out, want = torch.zeros(50, 8, device="cuda"), torch.zeros(50, 8, device="cuda")
+    SPMM_forward(src, x.t().contiguous().t(), out)
+    SPMM_forward(src, x, want)
+    assert torch.equal(out, want)
+
+
+@pytest.mark.parametrize("rows,fi,fo", [(70_001, 256, 256), (5_000, 128, 172), (999, 40, 47), (130, 33, 250)])
+def test_weight_gradient_on_column_blocks_equals_contiguous(rows, fi, fo):
+    gen = torch.Generator(device="cuda").manual_seed(rows)
+    wide = torch.randn(rows, 2 * fi, device="cuda", generator=gen)
+    wide_g = torch.randn(rows, fo + 12, device="cuda", generator=gen)
+    g = wide_g[:, 12:]
+    for x in (wide[:, :fi], wide[:, fi:]):
+        assert torch.equal(gcn.weight_gradient(x, g), gcn.weight_gradient(x.contiguous(), g.contiguous()))
+
+
+# ------------------------------------------------------------------ dropout -> LayerNorm -> ReLU
+@pytest.mark.parametrize("rows,feat", [(4099, 256), (1000, 128), (333, 64), (77, 100), (50, 512), (9, 1000), (1, 4),
+                                       (600, 24)])
+@pytest.mark.parametrize("with_mask", [True, False])
+def test_fused_dropout_layernorm_relu_matches_torch(rows, feat, with_mask):
+    gen = torch.Generator(device="cuda").manual_seed(rows + feat)
+    z = torch.randn(rows, feat, device="cuda", generator=gen) * 3.0 + 0.5
+    keep = (torch.rand(rows, feat, device="cuda", generator=gen) >= 0.5) if with_mask else None
+    scale = 2.0 if with_mask else 1.0
+    gamma = torch.rand(feat, device="cuda", generator=gen) + 0.5
+    beta = torch.randn(feat, device="cuda", generator=gen) * 0.3
+    grad_cat = torch.randn(rows, 2 * feat, device="cuda", generator=gen)
+
+    z_ref = z.cpu().clone().requires_grad_()
+    g_ref, b_ref = gamma.cpu().clone().requires_grad_(), beta.cpu().clone().requires_grad_()
+    d = z_ref * keep.cpu() * scale if with_mask else z_ref
+    y_ref = torch.relu(F.layer_norm(d, (feat,), g_ref, b_ref, 1e-5))
+    y_ref.backward(grad_cat[:, feat:].cpu())
+
+    z_in = z.clone().requires_grad_()
+    g_in, b_in = gamma.clone().requires_grad_(), beta.clone().requires_grad_()
+    cat = sage.dropout_layernorm_relu(z_in, keep, scale, g_in, b_in, 1e-5)
+    assert cat.shape == (rows, 2 * feat)
+    cat.backward(grad_cat)
+    assert torch.allclose(cat[:, feat:].detach().cpu(), y_ref.detach(), rtol=1e-5, atol=2e-5)
+    # the gradient passes through 1/sigma: scale the tolerance by the largest entry
+    gz_scale = float(z_ref.grad.abs().max()) + 1e-6
+    assert float((z_in.grad.cpu() - z_ref.grad).abs().max()) <= 1e-4 * gz_scale
+    for got, want in ((g_in.grad, g_ref.grad), (b_in.grad, b_ref.grad)):
+        assert float((got.cpu() - want).abs().max()) <= 1e-4 * (float(want.abs().max()) + 1.0)
+    # same input, same bits
+    again = sage.dropout_layernorm_relu(z, keep, scale, gamma, beta, 1e-5)
+    assert torch.equal(again[:, feat:], cat[:, feat:].detach())
+
+
+def test_fused_layernorm_rejects_what_it_cannot_take():
+    z = torch.randn(8, 6, device="cuda")
+    with pytest.raises(RuntimeError, match="multiples of 4"):
+        sage.dropout_layernorm_relu(z, None, 1.0, torch.ones(6, device="cuda"), torch.zeros(6, device="cuda"), 1e-5)
+    with pytest.raises(RuntimeError, match="Input mismatch"):
+        sage.dropout_layernorm_relu(torch.randn(8, 8), None, 1.0, torch.ones(8), torch.zeros(8), 1e-5)
+
+
+# ------------------------------------------------------------------ layer and model
+class ReplayExchange:
+    """Delivers seeded rows like SeededHaloExchange and keeps a host copy per tag."""
+
+    def __init__(self, seed):
+        self.inner = synthetic.SeededHaloExchange(seed)
+        self.rows = {}
+
+    def __call__(self, comm_splits, comm_buf, tag, direction):
+        self.inner(comm_splits, comm_buf, tag, direction)
+        buf = comm_buf.recv_buf if direction == "forward" else comm_buf.send_buf
+        self.rows[tag] = buf.detach().cpu().clone()
+        return None
+
+
+def _torch_sparse(m):
+    rowptr, col, val = [t.cpu() for t in m.csr()]
+    return torch.sparse_csr_tensor(rowptr, col, val, size=m.sparse_sizes())
+
+
+class CpuAggregate(torch.autograd.Function):
+    """out = A_local x + A_in recv ; grad = A_local^T g + A_out^T incoming (CPU, torch.sparse)."""
+
+    @staticmethod
+    def forward(ctx, x, a_local, a_in, a_out_t, recv, incoming):
+        ctx.mats = (a_local, a_out_t, incoming)
+        return torch.sparse.mm(a_local, x) + torch.sparse.mm(a_in, recv)
+
+    @staticmethod
+    def backward(ctx, g):
+        a_local, a_out_t, incoming = ctx.mats
+        gx = torch.sparse.mm(a_local.t().to_sparse_csr(), g) + torch.sparse.mm(a_out_t, incoming)
+        return gx, None, None, None, None, None
+
+
+class CpuSageLayer(torch.nn.Module):
+    """The reference's layer, written with torch modules (sageconv.py:40-44, :65-93)."""
+
+    def __init__(self, conv: sage.DistSAGEConvGrad):
+        super().__init__()
+        self.lin_neigh = torch.nn.Linear(conv.in_channels, conv.out_channels, bias=False)
+        self.lin_self = torch.nn.Linear(conv.in_channels, conv.out_channels, bias=False)
+        with torch.no_grad():
+            self.lin_neigh.weight.copy_(conv.lin_neigh.weight.cpu())
+            self.lin_self.weight.copy_(conv.lin_self.weight.cpu())
+        self.bias = torch.nn.Parameter(conv.bias.detach().cpu().clone())
+
+    def forward(self, agg, x, deg):
+        out = agg / deg
+        out = self.lin_neigh(out)
+        out = out + self.lin_self(x)
+        return out + self.bias
+
+    def stacked_grad(self):
+        return torch.cat([self.lin_neigh.weight.grad.t(), self.lin_self.weight.grad.t()], dim=0)
+
+
+def _cpu_mats(graph, is_pre_delay):
+    a_local = _torch_sparse(graph.local_adj_t)
+    if is_pre_delay:
+        a_in = _torch_sparse(graph.adj_t_pre_post_aggr_from)
+        a_out_t = _torch_sparse(graph.adj_t_pre_post_aggr_to).t().to_sparse_csr()
+    else:
+        a_in = _torch_sparse(graph.remote_adj_t)
+        a_out_t = _torch_sparse(graph.send_scatter_adj_t())
+    return a_local, a_in, a_out_t
+
+
+@pytest.mark.parametrize("is_pre_delay", [True, False])
+@pytest.mark.parametrize("fold", [False, True])
+def test_sage_model_matches_cpu_autograd(is_pre_delay, fold):
+    dev_ = "cuda:0"
+    n, f_in, hidden, classes, layers = 5000, 32, 64, 12, 3
+    part = synthetic.partition_edges(n, 4, 2, 6, 1.8, 800, 1500, 9000, seed=11, device=dev_)
+    ex = ReplayExchange(5)
+    graph = synthetic.build_partition_graph(part, max(f_in, hidden), is_pre_delay, exchange=ex, device=dev_)
+    run_graph = sage.fold_in_degrees(graph) if fold else graph
+    torch.manual_seed(0)
+    model = sage.DistSAGE(f_in, hidden, classes, num_layers=layers, dropout=0.5, is_pre_delay=is_pre_delay).to(dev_)
+    with torch.no_grad():  # LayerNorm parameters away from (1, 0) so that their gradients matter
+        for norm in model.norms:
+            norm.weight.uniform_(0.5, 1.5)
+            norm.bias.uniform_(-0.3, 0.3)
+    gen = torch.Generator(device=dev_).manual_seed(1)
+    x = torch.randn(n, f_in, device=dev_, generator=gen)
+    labels = torch.randint(0, classes, (n,), device=dev_, generator=gen)
+    train_idx = torch.randperm(n, device=dev_, generator=gen)[: n // 10]
+    masks = sage.make_dropout_masks(n, hidden, layers, 0.5, 7, dev_)
+
+    model.train()
+    staged = sage.stage_input(x)
+    out = model(run_graph, staged, masks)
+    loss = F.nll_loss(out[train_idx], labels[train_idx])
+    loss.backward()
+
+    # the same model on the CPU, the reference's way
+    a_local, a_in, a_out_t = _cpu_mats(graph, is_pre_delay)
+    deg = graph.in_degrees.cpu()
+    cpu_layers = [CpuSageLayer(conv) for conv in model.convs]
+    cpu_norms = [copy.deepcopy(norm).cpu() for norm in model.norms]
+    h = x.cpu()
+    for i, layer in enumerate(cpu_layers):
+        width = h.size(1)
+        incoming = ex.rows.get(f"backward{i}", torch.zeros(a_out_t.shape[1], width))
+        agg = CpuAggregate.apply(h, a_local, a_in, a_out_t, ex.rows[f"forward{i}"], incoming)
+        z = layer(agg, h, deg)
+        if i == layers - 1:
+            h = z
+            break
+        h = torch.relu(cpu_norms[i](z * masks[i].cpu() * 2.0))
+    cpu_loss = F.nll_loss(F.log_softmax(h, dim=1)[train_idx.cpu()], labels.cpu()[train_idx.cpu()])
+    cpu_loss.backward()
+
+    tol = 1e-4
+    assert abs(float(loss.detach()) - float(cpu_loss.detach())) <= tol * max(1.0, abs(float(cpu_loss.detach())))
+    for i, (conv, ref) in enumerate(zip(model.convs, cpu_layers)):
+        for name, got, want in ((f"weight{i}", conv.weight.grad.cpu(), ref.stacked_grad()),
+                                (f"bias{i}", conv.bias.grad.cpu(), ref.bias.grad)):
+            scale = float(want.abs().max()) + 1e-12
+            assert float((got - want).abs().max()) <= 10 * tol * scale, name
+    for i, (norm, ref) in enumerate(zip(model.norms, cpu_norms)):
+        for name, got, want in ((f"gamma{i}", norm.weight.grad.cpu(), ref.weight.grad),
+                                (f"beta{i}", norm.bias.grad.cpu(), ref.bias.grad)):
+            scale = float(want.abs().max()) + 1e-12
+            assert float((got - want).abs().max()) <= 10 * tol * scale, name
+
+    # a few updates: the loss goes down, and handing over unstaged features gives the same loss
+    opt = torch.optim.Adam(model.parameters(), lr=0.01)
+    first = float(sage.train_step(model, opt, run_graph, x, labels, train_idx, masks))
+    assert abs(first - float(cpu_loss.detach())) <= tol * max(1.0, abs(float(cpu_loss.detach())))
+    losses = [float(sage.train_step(model, opt, run_graph, staged, labels, train_idx, masks)) for _ in range(5)]
+    assert all(np.isfinite(losses)) and losses[-1] < first
+
+
+def test_sage_layer_single_rank_and_eval_mode():
+    """No exchange (single-rank world), no dropout outside training, bias-free layer."""
+    dev_ = "cuda:0"
+    n, f_in, f_out = 3000, 16, 20
+    rowptr, col, val = skewed_csr(n, n, seed=2, heavy_rows=(400,))
+    adj = SparseTensor(rowptr=dev(rowptr), col=dev(col), value=dev(val), sparse_sizes=(n, n))
+    in_degrees = torch.from_numpy(np.maximum(np.diff(rowptr), 1).astype(np.float32)).view(-1, 1).cuda()
+    splits = CommSplits([0], [0], 1, 32)
+    graph = DistributedGraphForPre(adj, None, None, [0], [0], in_degrees, splits,
+                                   CommBuffer(splits, f_in, 32, device=dev_))
+    torch.manual_seed(1)
+    conv = sage.DistSAGEConvGrad(f_in, f_out, 32, True, bias=False).to(dev_)
+    assert conv.bias is None and conv.lin_neigh.weight.shape == (f_out, f_in)
+    x = torch.randn(n, f_in, device=dev_)
+    staged = sage.stage_input(x).requires_grad_()
+    out = conv(graph, staged, 0)
+    out.square().sum().backward()
+
+    a = _torch_sparse(adj)
+    xc = x.cpu().clone().requires_grad_()
+    wn = conv.lin_neigh.weight.detach().cpu().clone().requires_grad_()
+    ws = conv.lin_self.weight.detach().cpu().clone().requires_grad_()
+    want = (torch.sparse.mm(a, xc) / graph.in_degrees.cpu()) @ wn.t() + xc @ ws.t()
+    want.square().sum().backward()
+    assert torch.allclose(out.detach().cpu(), want.detach(), rtol=1e-4, atol=1e-4)
+    scale = float(xc.grad.abs().max())
+    assert float((staged.grad[:, f_in:].cpu() - xc.grad).abs().max()) <= 1e-4 * scale
+    got_w = conv.weight.grad.cpu()
+    want_w = torch.cat([wn.grad.t(), ws.grad.t()], dim=0)
+    assert float((got_w - want_w).abs().max()) <= 1e-4 * float(want_w.abs().max())
+
+    with pytest.raises(RuntimeError, match="Input mismatch"):
+        conv(graph, torch.randn(n, f_in + 1, device=dev_), 0)
+    with pytest.raises(RuntimeError, match="staged"):
+        conv(graph, x.clone().requires_grad_(), 0)
