@@ -17,8 +17,8 @@ host) timed on this machine's cores on the same matrices.
 
 ``extra`` carries the other workloads, run after the timed headline: c2 at F=128/256,
 c3 (dense-degree mean aggregation, F=602/256), c4 (one partition of a 16-way split:
-pre-aggregation, local SpMM, post-aggregation, F=128) and c5 (3-layer GCN train step on
-the c4 partition).  ``--only headline`` skips them.
+pre-aggregation, local SpMM, post-aggregation, F=128) and c5 (3-layer GCN train step and the
+reference's 3-layer SAGE model on the c4 partition).  ``--only headline`` skips them.
 """
 import argparse
 import json
@@ -502,13 +502,10 @@ def run_c5(args, graph):
         out[f"train_step_ms_{tag}"] = round((time.perf_counter() - t0) * 1e3 / steps, 2)
         out[f"loss_{tag}"] = [round(v, 5) for v in losses + [float(loss)]]
         del model, opt
-    del masks
-    torch.cuda.empty_cache()
-    out["sage"] = run_c5_sage(args, graph, x, labels, train_idx, dims, steps)
     return out
 
 
-def run_c5_sage(args, graph, x, labels, train_idx, dims, steps):
+def run_c5_sage(args, graph):
     """The reference's own model on the same partition (DistSAGE: lin_neigh + lin_self per layer,
     dropout -> LayerNorm -> ReLU between layers), three ways: this build's layer stack (one
     stacked dense product per layer on [aggregated | x] kept side by side, fused elementwise
@@ -519,8 +516,14 @@ def run_c5_sage(args, graph, x, labels, train_idx, dims, steps):
 
     from gnn_benchmark_amd import Aggregator, sage
 
-    dev = x.device
-    n = x.size(0)
+    dev = "cuda:0"
+    n = graph.local_adj_t.sparse_size(0)
+    dims = [128, 256, 256, 172]
+    gen = torch.Generator(device=dev).manual_seed(args.seed + 6)
+    x = torch.randn(n, dims[0], device=dev, generator=gen)
+    labels = torch.randint(0, dims[-1], (n,), device=dev, generator=gen)
+    train_idx = torch.randperm(n, device=dev, generator=gen)[: n // 10]
+    steps = max(3, args.steps // 4)
     hidden = dims[1]
     masks = sage.make_dropout_masks(n, hidden, len(dims) - 1, 0.5, args.seed + 8, dev)
     out = {"layers": "DistSAGE %d->%d->%d->%d, LayerNorm, dropout 0.5" % tuple(dims), "steps": steps}
@@ -591,7 +594,8 @@ def main():
     ap.add_argument("--c4-nodes", type=int, default=7_000_000)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--only", default="", help="'headline' = headline workload only; or a comma list of the extra "
-                                                "workloads to add: c2 (F=128/256), c3, c4, c5.  Default: all of them")
+                                                "workloads to add: c2 (F=128/256), c3, c4, c5 (GCN and SAGE train "
+                                                "steps; c5sage: the SAGE one alone).  Default: c2,c3,c4,c5")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy 3 times (a kernel of known traffic for scaling "
@@ -619,12 +623,15 @@ def main():
     if "c3" in args.extras:
         extra["c3"] = run_c3(args)
         torch.cuda.empty_cache()
-    if "c4" in args.extras or "c5" in args.extras:
+    if any(k in args.extras for k in ("c4", "c5", "c5sage")):
         _part, graph, setup_s = build_c4(args)
         if "c4" in args.extras:
             extra["c4"] = run_c4(args, graph, setup_s)
         if "c5" in args.extras:
             extra["c5"] = run_c5(args, graph)
+            torch.cuda.empty_cache()
+        if "c5" in args.extras or "c5sage" in args.extras:
+            extra["c5_sage"] = run_c5_sage(args, graph)
     line["extra"] = extra
     print(json.dumps(line), flush=True)
 
