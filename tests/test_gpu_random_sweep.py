@@ -1,5 +1,7 @@
 """Seeded random sweep over shapes the hand-picked cases do not name: every SpMM path
-(plan, plan-less, transposed) and the row-packed codec, bit for bit against the oracle."""
+(plan, plan-less, transposed) and the row-packed codec, bit for bit against the oracle; packed
+and strided operands bit for bit against the dense / contiguous product; the fused LayerNorm
+pass against torch's fp64 ops (5e-5 absolute on outputs, 2e-4 relative on gradients)."""
 import numpy as np
 import pytest
 import torch
@@ -117,3 +119,81 @@ def test_random_packed_operands_match_the_dense_product(seed):
         SPMM_forward(src, dense, want, accumulate=acc)
         packed.spmm(src, values, header, got, accumulate=acc)
         assert torch.equal(got, want), dict(seed=seed, case=case, rows=rows, cols=cols, feat=feat, keep=keep_p, acc=acc)
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_column_blocks_match_contiguous_operands(seed):
+    """SpMM (both directions) and the weight gradient on column blocks of wider arrays at random
+    offsets and strides: the same bits as on contiguous copies, nothing outside the block written."""
+    rng = np.random.default_rng(15000 + seed)
+    for case in range(20):
+        rows = int(rng.choice([1, 7, 64, 300, 3000]))
+        cols = int(rng.choice([1, 3, 64, 500, 3000]))
+        feat = int(rng.choice(WIDTHS))
+        deg = _degrees(rng, rows)
+        rowptr = np.concatenate(([0], np.cumsum(deg))).astype(np.int64)
+        nnz = int(rowptr[-1])
+        col = rng.integers(0, cols, nnz).astype(np.int64)
+        val = rng.standard_normal(nnz).astype(np.float32)
+        src = SparseTensor(rowptr=dev(rowptr), col=dev(col), value=dev(val), sparse_sizes=(rows, cols), is_sorted=True)
+        lead_x, tail_x, lead_o, tail_o = (int(v) for v in rng.integers(0, 9, 4))
+        wide_x = dev(rng.standard_normal((max(rows, cols), lead_x + feat + tail_x)).astype(np.float32))
+        wide_o = dev(rng.standard_normal((max(rows, cols), lead_o + feat + tail_o)).astype(np.float32))
+        acc = bool(rng.integers(0, 2))
+        what = dict(seed=seed, case=case, rows=rows, cols=cols, feat=feat, longest=int(deg.max()), acc=acc,
+                    offsets=(lead_x, tail_x, lead_o, tail_o))
+        for op, n_in, n_out in ((SPMM_forward, cols, rows), (SPMM_backward, rows, cols)):
+            x_view = wide_x[:n_in, lead_x:lead_x + feat]
+            before = wide_o.clone()
+            o_view = wide_o[:n_out, lead_o:lead_o + feat]
+            want = o_view.contiguous()
+            op(src, x_view.contiguous(), want, accumulate=acc)
+            op(src, x_view, o_view, accumulate=acc)
+            assert torch.equal(o_view, want), (op.__name__, what)
+            untouched = torch.ones_like(wide_o, dtype=torch.bool)
+            untouched[:n_out, lead_o:lead_o + feat] = False
+            assert torch.equal(wide_o[untouched], before[untouched]), (op.__name__, what)
+        fo = int(rng.choice([1, 5, 47, 64, 172, 256]))
+        if feat <= 256:
+            g = dev(rng.standard_normal((rows, fo + 3)).astype(np.float32))[:, 3:]
+            x_view = wide_x[:rows, lead_x:lead_x + feat]
+            assert torch.equal(gcn.weight_gradient(x_view, g),
+                               gcn.weight_gradient(x_view.contiguous(), g.contiguous())), ("weight gradient", what, fo)
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_random_fused_layernorm_passes_match_torch(seed):
+    from gnn_benchmark_amd import sage
+
+    rng = np.random.default_rng(17000 + seed)
+    for case in range(15):
+        rows = int(rng.choice([1, 3, 64, 257, 4000]))
+        feat = 4 * int(rng.integers(1, 257))
+        z = dev((rng.standard_normal((rows, feat)) * rng.uniform(0.1, 10) + rng.uniform(-2, 2)).astype(np.float32))
+        with_mask = bool(rng.integers(0, 2))
+        p = float(rng.choice([0.1, 0.5, 0.8]))
+        keep = dev(rng.random((rows, feat)) >= p) if with_mask else None
+        scale = 1.0 / (1.0 - p) if with_mask else 1.0
+        gamma = dev(rng.uniform(0.5, 1.5, feat).astype(np.float32))
+        beta = dev(rng.uniform(-0.5, 0.5, feat).astype(np.float32))
+        grad = dev(rng.standard_normal((rows, 2 * feat)).astype(np.float32))
+        what = dict(seed=seed, case=case, rows=rows, feat=feat, mask=with_mask, p=p)
+
+        z_ref = z.double().cpu().requires_grad_()
+        g_ref, b_ref = gamma.double().cpu().requires_grad_(), beta.double().cpu().requires_grad_()
+        d = z_ref * keep.cpu() * scale if with_mask else z_ref
+        y_ref = torch.relu(torch.nn.functional.layer_norm(d, (feat,), g_ref, b_ref, 1e-5))
+        y_ref.backward(grad[:, feat:].double().cpu())
+
+        z_in, g_in, b_in = z.clone().requires_grad_(), gamma.clone().requires_grad_(), beta.clone().requires_grad_()
+        cat = sage.dropout_layernorm_relu(z_in, keep, scale, g_in, b_in, 1e-5)
+        cat.backward(grad)
+        got = cat[:, feat:].detach().double().cpu()
+        # a unit sits on the ReLU's edge when |n| is within rounding of 0: compare where fp64 is clear of it
+        clear = (y_ref.detach() > 1e-4) | (torch.nn.functional.layer_norm(d, (feat,), g_ref, b_ref, 1e-5).detach() < -1e-4)
+        assert float((got - y_ref.detach()).abs().max()) <= 5e-5, what
+        gz_err = ((z_in.grad.double().cpu() - z_ref.grad).abs() * clear.all(dim=1, keepdim=True)).max()
+        assert float(gz_err) <= 2e-4 * (float(z_ref.grad.abs().max()) + 1e-9), what
+        if bool(clear.all()):
+            for got_p, want_p in ((g_in.grad, g_ref.grad), (b_in.grad, b_ref.grad)):
+                assert float((got_p.double().cpu() - want_p).abs().max()) <= 2e-4 * (float(want_p.abs().max()) + 1.0), what
