@@ -392,3 +392,34 @@ def test_plan_spmm_can_be_captured_in_a_hip_graph(monkeypatch, with_block_rows):
         graph.replay()
         torch.cuda.synchronize()
         assert np.array_equal(out.cpu().numpy(), _oracle(rowptr, col, val, xh))
+
+
+def test_more_than_2_to_31_stored_elements():
+    """Element offsets beyond 32 bits: 1 050 000 rows of 2 100 elements = 2.205e9 stored elements
+    (2^31 = 2.147e9), so the last rows' column / value reads lie past a 32-bit offset (the reference
+    truncates such offsets, model/ops/src/spmm.cpp:38-39).  Unit values and small integer features
+    make every row sum exact in fp32 whatever the order, so the result must EQUAL the integer sums
+    taken with torch -- through the plan (32-bit column copy) and through the plan-less entry."""
+    rows, cols, per_row, feat = 1_050_000, 1_000_003, 2_100, 2
+    nnz = rows * per_row
+    assert nnz > 2 ** 31
+    col = (torch.arange(nnz, device="cuda", dtype=torch.int64) * 7919) % cols
+    rowptr = torch.arange(rows + 1, device="cuda", dtype=torch.int64) * per_row
+    val = torch.ones(nnz, device="cuda")
+    x = (torch.arange(cols, device="cuda") % 5).float().view(-1, 1) + torch.tensor([0.0, 1.0], device="cuda")
+    sums = (col % 5).view(rows, per_row).sum(dim=1)                       # int64, exact
+    want = torch.stack((sums, sums + per_row), dim=1).float()             # < 2^24: exact in fp32
+    assert int(want.max()) < 2 ** 24
+
+    src = SparseTensor(rowptr=rowptr, col=col, value=val, sparse_sizes=(rows, cols), is_sorted=True)
+    out = torch.full((rows, feat), 7.0, device="cuda")
+    SPMM_forward(src, x, out, accumulate=False)
+    assert torch.equal(out, want)
+    SPMM_forward(src, x, out, accumulate=True)
+    assert torch.equal(out, 2 * want)
+    del src
+    out.zero_()
+    computation_ops.spmm(rowptr, col, val, x, out, rows, None, None)
+    assert torch.equal(out, want)
+    tail = out[-3:].clone()  # the rows whose elements start beyond 2^31
+    assert rowptr[-4] > 2 ** 31 and torch.equal(tail, want[-3:])
