@@ -423,3 +423,27 @@ def test_more_than_2_to_31_stored_elements():
     assert torch.equal(out, want)
     tail = out[-3:].clone()  # the rows whose elements start beyond 2^31
     assert rowptr[-4] > 2 ** 31 and torch.equal(tail, want[-3:])
+
+
+def test_dense_operands_beyond_2_to_31_floats():
+    """Row addresses past 2^31 floats (the reference computes them in `int`,
+    model/ops/src/spmm.cpp:38-39, :98-99): a 9 M x 9 M matrix with one stored element per row
+    (a scaled permutation), F = 256, so that both the gathered and the written rows reach
+    2.3e9 floats.  One element per row makes the result a single rounded product, hence EQUAL
+    to torch's elementwise product of the permuted operand."""
+    n, feat = 9_000_000, 256
+    assert n * feat > 2 ** 31
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    perm = torch.randperm(n, device="cuda", generator=gen)
+    perm[-1], perm[0] = n - 1, int(perm[-1])          # the last row gathers the last row
+    val = torch.rand(n, device="cuda", generator=gen) + 0.5
+    x = torch.randn(n, feat, device="cuda", generator=gen)
+    rowptr = torch.arange(n + 1, device="cuda", dtype=torch.int64)
+    src = SparseTensor(rowptr=rowptr, col=perm, value=val, sparse_sizes=(n, n), is_sorted=True)
+    out = torch.empty(n, feat, device="cuda")
+    SPMM_forward(src, x, out, accumulate=False)
+    # compare in slices to keep the temporaries small
+    for lo in range(0, n, 1_500_000):
+        hi = min(n, lo + 1_500_000)
+        assert torch.equal(out[lo:hi], val[lo:hi, None] * x[perm[lo:hi]]), lo
+    assert torch.equal(out[-1], val[-1] * x[-1])
