@@ -165,19 +165,20 @@ def test_error_behaviour():
     ops.dequantize_tensor(packed[:0], x[:0], params[:0], 2)
 
 
-def test_full_size_round_trip_properties():
-    """3 M boundary rows x 128 (config 4's receive buffer): idempotence of the codec -- what was
-    dequantised quantises back to the same bytes -- and the half-step error bound."""
+@pytest.mark.parametrize("rows,feat,bits", [(3_000_003, 128, 2), (9_000_001, 256, 4)])
+def test_full_size_round_trip_properties(rows, feat, bits):
+    """3 M boundary rows x 128 (config 4's receive buffer), and 9 M x 256 (element offsets past
+    2^31): idempotence of the codec -- what was dequantised quantises back to the same bytes --
+    and the half-step error bound."""
     from gnn_benchmark_amd import computation_ops as ops
 
-    rows, feat, bits = 3_000_003, 128, 2
     gen = torch.Generator(device="cuda").manual_seed(1)
     x = torch.randn(rows, feat, device="cuda", generator=gen)
     splits = [rows // 15] * 15
     splits[-1] += rows - sum(splits)
     splits.insert(3, 0)
     work_range = torch.tensor(np.concatenate(([0], np.cumsum(splits))), dtype=torch.int32)
-    packed_rows = sum(-(-s // 4) for s in splits)
+    packed_rows = sum(-(-s // (8 // bits)) for s in splits)
     packed = torch.zeros((packed_rows, feat), dtype=torch.uint8, device="cuda")
     params = torch.zeros((rows, 2), device="cuda")
     ops.quantize_tensor_for_all_procs(x, packed, params, work_range, 16, bits)

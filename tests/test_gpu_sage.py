@@ -333,3 +333,19 @@ def test_sage_layer_aggregates_like_the_aggregator(num_bits, is_pre_delay):
     scale = float(x_leaf.grad.abs().max())
     # the layer adds the transposed aggregation onto the direct part, autograd the other way round
     assert float((staged.grad[:, f_in:] - x_leaf.grad).abs().max()) <= 2e-6 * scale
+
+
+def test_fused_layernorm_pass_beyond_2_to_31_elements():
+    """9 M x 256 activations (2.3e9 elements): element offsets need 64 bits.  Checked in slices
+    against torch's own ops on the device (fp32; the moments are summed in another order)."""
+    rows, feat = 9_000_000, 256
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    z = torch.randn(rows, feat, device="cuda", generator=gen)
+    keep = torch.rand(rows, feat, device="cuda", generator=gen) >= 0.5
+    gamma = torch.rand(feat, device="cuda", generator=gen) + 0.5
+    beta = torch.randn(feat, device="cuda", generator=gen) * 0.2
+    cat = sage._DropoutLayerNormRelu.apply(z, keep, 2.0, gamma, beta, 1e-5)
+    for lo in (0, 4_000_000, rows - 1_000_000):
+        sl = slice(lo, lo + 1_000_000)
+        want = torch.relu(F.layer_norm(z[sl] * keep[sl] * 2.0, (feat,), gamma, beta, 1e-5))
+        assert torch.allclose(cat[sl, feat:], want, rtol=1e-5, atol=2e-5), lo
