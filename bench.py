@@ -470,6 +470,76 @@ def run_c4_codec(graph, feat, steps, gen, cpu=False):
     return out
 
 
+def run_c4_raw_halo(args, part):
+    """The same partition with raw boundary rows (``is_pre_delay=False``): rows gathered into the
+    send buffer instead of pre-aggregated, halo rows aggregated through ``remote_adj_t``, and the
+    backward's ``index_add_`` as a product with the selection matrix."""
+    import torch
+
+    from gnn_benchmark_amd import Aggregator, synthetic
+    from gnn_benchmark_amd.aggregator import _gather_rows
+
+    dev = "cuda:0"
+    feat = 128
+    steps = max(5, args.steps // 2)
+    t0 = time.perf_counter()
+    graph = synthetic.build_partition_graph(part, 256, False, exchange=synthetic.SeededHaloExchange(args.seed + 4),
+                                            device=dev)
+    torch.cuda.synchronize()
+    setup_s = time.perf_counter() - t0
+    n = graph.local_adj_t.sparse_size(0)
+    gen = torch.Generator(device=dev).manual_seed(args.seed + 5)
+    x = torch.randn(n, feat, device=dev, generator=gen)
+    g = torch.randn(n, feat, device=dev, generator=gen)
+    graph.comm_buf.resize_buffer(graph.comm_splits, feat, 32)
+    send_buf, recv_buf = graph.comm_buf.send_buf, graph.comm_buf.recv_buf
+    recv_buf.normal_(generator=gen)
+    out = torch.zeros(n, feat, device=dev)
+    idx = graph.idx_nodes_send_to_others
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for i in range(steps + 2):
+        if i == 2:
+            e0.record()
+        _gather_rows(x, idx, send_buf)
+    e1.record()
+    e1.synchronize()
+    gather_ms = e0.elapsed_time(e1) / steps
+    gather_bytes = idx.numel() * (8.0 + 2 * 4.0 * feat)
+    ops = [{"op": "gather boundary rows X[idx] -> send_buf", "rows": int(idx.numel()), "feat": feat,
+            "ms": round(gather_ms, 4), "gbs_model": round(gather_bytes / (gather_ms * 1e-3) / 1e9, 1),
+            "frac_of_hbm_peak": round(gather_bytes / (gather_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}]
+    for name, m, src_x, dst in (("halo aggregation A_remote@recv_buf -> out", graph.remote_adj_t, recv_buf, out),
+                                ("scatter of received gradients (index_add_ as a product) -> dX",
+                                 graph.send_scatter_adj_t(), send_buf, out)):
+        rows, cols = m.sparse_sizes()
+        _, ms = time_plan(m.get_plan(), m.csr()[2], src_x, dst, steps, 2, accumulate=True)
+        ops.append(op_report(name, m.nnz(), rows, cols, feat, ms, m.get_plan().info()["empty_rows"]))
+    m = graph.remote_adj_t
+    back = torch.zeros(m.sparse_size(1), feat, device=dev)
+    _, ms = time_plan(m.get_plan_for_transpose(), m.storage.value_T(), out, back, steps, 2, accumulate=True)
+    ops.append(op_report("halo aggregation transposed (gradient direction)", m.nnz(), m.sparse_size(1), m.sparse_size(0),
+                         feat, ms, m.get_plan_for_transpose().info()["empty_rows"]))
+    del back
+    xr = x.clone().requires_grad_()
+    for _ in range(2):
+        Aggregator.apply(graph, xr, 0, 32, False, True).backward(g)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        o = Aggregator.apply(graph, xr, 0, 32, False, True)
+    torch.cuda.synchronize()
+    fwd_ms = (time.perf_counter() - t0) * 1e3 / steps
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        o = Aggregator.apply(graph, xr, 0, 32, False, True)
+        o.backward(g)
+    torch.cuda.synchronize()
+    both_ms = (time.perf_counter() - t0) * 1e3 / steps
+    return {"workload": "the c4 partition with raw boundary rows (is_pre_delay=False)", "feat": feat,
+            "send_rows": int(idx.numel()), "halo_rows": int(graph.remote_adj_t.sparse_size(1)), "setup_s": round(setup_s, 2),
+            "ops": ops, "aggregator_forward_ms": round(fwd_ms, 3), "aggregator_forward_backward_ms": round(both_ms, 3)}
+
+
 def run_c5(args, graph):
     import torch
 
@@ -627,6 +697,9 @@ def main():
         _part, graph, setup_s = build_c4(args)
         if "c4" in args.extras:
             extra["c4"] = run_c4(args, graph, setup_s)
+            torch.cuda.empty_cache()
+            extra["c4_raw_halo"] = run_c4_raw_halo(args, _part)
+            torch.cuda.empty_cache()
         if "c5" in args.extras:
             extra["c5"] = run_c5(args, graph)
             torch.cuda.empty_cache()

@@ -75,19 +75,56 @@ __global__ __launch_bounds__(256) void pack_transposed_keys_kernel(const int64_t
     idx[e] = (uint32_t)e;
 }
 
-template <int VEC>
+// out[i, :] = src[index[i], :].  A group of G lanes (G * VEC floats cover a row, or one pass of it)
+// owns four rows at a time: their indices, then their vectors, are requested back to back before
+// anything is stored.  Source rows come through normal loads (a boundary row usually goes to
+// several peers, so it is asked for again soon); the result is written once, with streaming stores.
+template <int VEC, int G>
 __global__ __launch_bounds__(256) void gather_rows_kernel(const float *__restrict__ src,
                                                           const int64_t *__restrict__ index,
                                                           float *__restrict__ out, int64_t n_index, int feat_vec) {
     typedef float vec_t __attribute__((ext_vector_type(VEC)));
-    // one wavefront per output row, lanes along the feature dimension
-    const int64_t i = (int64_t)blockIdx.x * 4 + ((int)threadIdx.x >> 6);
-    if (i >= n_index) return;
-    const int lane = (int)threadIdx.x & 63;
-    const size_t r = (size_t)index[i];
-    const vec_t *s = reinterpret_cast<const vec_t *>(src) + r * (size_t)feat_vec;
-    vec_t *d = reinterpret_cast<vec_t *>(out) + (size_t)i * (size_t)feat_vec;
-    for (int f = lane; f < feat_vec; f += 64) d[f] = s[f];
+    constexpr int kGroups = 256 / G;
+    constexpr int kRows = 4;
+    const int l = (int)threadIdx.x % G;
+    const int group = (int)threadIdx.x / G;
+    const int64_t step = (int64_t)gridDim.x * kGroups * kRows;
+    for (int64_t base = ((int64_t)blockIdx.x * kGroups + group) * kRows; base < n_index; base += step) {
+        const vec_t *s[kRows];
+        vec_t *d[kRows];
+        bool ok[kRows];
+#pragma unroll
+        for (int u = 0; u < kRows; ++u) {
+            ok[u] = base + u < n_index;
+            const size_t r = ok[u] ? (size_t)__builtin_nontemporal_load(index + base + u) : 0;
+            s[u] = reinterpret_cast<const vec_t *>(src) + r * (size_t)feat_vec;
+            d[u] = reinterpret_cast<vec_t *>(out) + (size_t)(base + u) * (size_t)feat_vec;
+        }
+        for (int f = l; f < feat_vec; f += G) {
+            vec_t v[kRows];
+#pragma unroll
+            for (int u = 0; u < kRows; ++u)
+                if (ok[u]) v[u] = s[u][f];
+#pragma unroll
+            for (int u = 0; u < kRows; ++u)
+                if (ok[u]) __builtin_nontemporal_store(v[u], d[u] + f);
+        }
+    }
+}
+
+template <int VEC>
+hipError_t launch_gather_rows(const float *src, const int64_t *index, float *out, int64_t n_index, int feat_vec,
+                              hipStream_t st) {
+    int g = 8;
+    while (g < 64 && g < feat_vec) g *= 2;
+    const int64_t rows_per_block = (256 / g) * 4;
+    const int64_t need = (n_index + rows_per_block - 1) / rows_per_block;
+    const unsigned grid = (unsigned)(need < 256 * 32 ? need : 256 * 32);
+    if (g == 8) hipLaunchKernelGGL((gather_rows_kernel<VEC, 8>), dim3(grid), dim3(256), 0, st, src, index, out, n_index, feat_vec);
+    else if (g == 16) hipLaunchKernelGGL((gather_rows_kernel<VEC, 16>), dim3(grid), dim3(256), 0, st, src, index, out, n_index, feat_vec);
+    else if (g == 32) hipLaunchKernelGGL((gather_rows_kernel<VEC, 32>), dim3(grid), dim3(256), 0, st, src, index, out, n_index, feat_vec);
+    else hipLaunchKernelGGL((gather_rows_kernel<VEC, 64>), dim3(grid), dim3(256), 0, st, src, index, out, n_index, feat_vec);
+    return hipGetLastError();
 }
 
 int sort_keys(uint64_t *key_in, uint64_t *key_out, uint32_t *idx_in, uint32_t *idx_out, int64_t n, int bits,
@@ -215,13 +252,12 @@ extern "C" int gnnagg_gather_rows_f32(const float *src, const int64_t *index, fl
     if (feat > (1 << 20)) return fail(GNNAGG_ERR_UNSUPPORTED, "feature width %lld above 2^20", (long long)feat);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const uintptr_t bits = reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(out);
-    const unsigned grid = grid_for(n_index, 4);
     if (feat % 4 == 0 && bits % 16 == 0)
-        hipLaunchKernelGGL(gather_rows_kernel<4>, dim3(grid), dim3(256), 0, st, src, index, out, n_index, (int)(feat / 4));
+        GNNAGG_HIP(launch_gather_rows<4>(src, index, out, n_index, (int)(feat / 4), st));
     else if (feat % 2 == 0 && bits % 8 == 0)
-        hipLaunchKernelGGL(gather_rows_kernel<2>, dim3(grid), dim3(256), 0, st, src, index, out, n_index, (int)(feat / 2));
+        GNNAGG_HIP(launch_gather_rows<2>(src, index, out, n_index, (int)(feat / 2), st));
     else
-        hipLaunchKernelGGL(gather_rows_kernel<1>, dim3(grid), dim3(256), 0, st, src, index, out, n_index, (int)feat);
+        GNNAGG_HIP(launch_gather_rows<1>(src, index, out, n_index, (int)feat, st));
     GNNAGG_HIP(hipGetLastError());
     return GNNAGG_OK;
 }

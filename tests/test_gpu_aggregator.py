@@ -360,3 +360,24 @@ def test_quantised_run_needs_its_buffers_and_hook():
         Aggregator.apply(graphs2[0], x, 0, 2, True, True)
     with pytest.raises(NotImplementedError):
         Aggregator.apply(graphs2[0], x, 0, 3, True, True)
+
+
+@pytest.mark.parametrize("feat", [1, 2, 3, 4, 6, 20, 32, 100, 128, 130, 256, 260, 602, 1028])
+@pytest.mark.parametrize("count", [0, 1, 3, 64, 1000, 4099])
+def test_row_gather_equals_index_select(feat, count):
+    """``torch.index_select(feat, 0, idx, out=send_buf)`` (model/layers/aggregator.py:51): byte
+    copies, so the result must be identical; repeated and unsorted indices, unaligned operands."""
+    from gnn_benchmark_amd.aggregator import _gather_rows
+
+    gen = torch.Generator(device="cuda").manual_seed(feat * 7 + count)
+    src = torch.randn(777, feat, device="cuda", generator=gen)
+    index = torch.randint(0, 777, (count,), device="cuda", generator=gen)
+    out = torch.full((count, feat), -1.0, device="cuda")
+    _gather_rows(src, index, out)
+    assert torch.equal(out, src[index])
+    # operands that start 4 bytes into an allocation (scalar path)
+    flat = torch.randn(777 * feat + 1, device="cuda", generator=gen)
+    src2 = flat[1:].view(777, feat)
+    out2 = torch.empty(count * feat + 1, device="cuda")[1:].view(count, feat)
+    _gather_rows(src2, index, out2)
+    assert torch.equal(out2, src2[index])
