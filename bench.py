@@ -579,8 +579,9 @@ def run_c5_sage(args, graph):
     """The reference's own model on the same partition (DistSAGE: lin_neigh + lin_self per layer,
     dropout -> LayerNorm -> ReLU between layers), three ways: this build's layer stack (one
     stacked dense product per layer on [aggregated | x] kept side by side, fused elementwise
-    chain), the same with the degree normalisation folded into the matrix values, and -- as the
-    yardstick -- plain torch ops around the same Aggregator, the way the reference writes them."""
+    chain), the same with the degree normalisation folded into the matrix values, that with the
+    narrowing last layer applying lin_neigh before it aggregates, and -- as the yardstick -- plain
+    torch ops around the same Aggregator, the way the reference writes them."""
     import torch
     import torch.nn.functional as F
 
@@ -608,16 +609,22 @@ def run_c5_sage(args, graph):
         return round((time.perf_counter() - t0) * 1e3 / steps, 2), [round(v, 5) for v in losses + [float(loss)]]
 
     staged = sage.stage_input(x)
-    for tag, g in (("", graph), ("_folded_degrees", None)):
-        if g is None:
-            g = sage.fold_in_degrees(graph)
+    folded = None
+    for tag, fold, linear_first in (("", False, False), ("_folded_degrees", True, False),
+                                    ("_folded_degrees_linear_first_when_narrowing", True, True)):
+        if fold and folded is None:
+            folded = sage.fold_in_degrees(graph)
+        g = folded if fold else graph
         torch.manual_seed(args.seed)
-        model = sage.DistSAGE(dims[0], hidden, dims[-1], num_layers=len(dims) - 1, dropout=0.5, is_pre_delay=True).to(dev)
+        model = sage.DistSAGE(dims[0], hidden, dims[-1], num_layers=len(dims) - 1, dropout=0.5, is_pre_delay=True,
+                              linear_first_when_narrowing=linear_first).to(dev)
         opt = torch.optim.Adam(model.parameters(), lr=0.01)
         ms, losses = timed(lambda: sage.train_step(model, opt, g, staged, labels, train_idx, masks))
         out["train_step_ms" + tag], out["loss" + tag] = ms, losses
         del model, opt, g
         torch.cuda.empty_cache()
+    del folded
+    torch.cuda.empty_cache()
 
     class TorchOpsSage(torch.nn.Module):
         def __init__(self):

@@ -178,9 +178,10 @@ def _check_result(out: torch.Tensor, rows: int, feat_len: int, device) -> None:
                            % (rows, feat_len, device))
 
 
-def _forward(ctx, graph, feats, layer, num_bits: int, is_pre_delay: bool, is_training: bool, out=None):
-    """``out``: where to write the result (every row is overwritten) -- e.g. a column block of a
-    wider tensor; a fresh tensor when None."""
+def _forward(ctx, graph, feats, layer, num_bits: int, is_pre_delay: bool, is_training: bool, out=None,
+             accumulate: bool = False):
+    """``out``: where to write the result -- e.g. a column block of a wider tensor; a fresh tensor
+    when None.  Every row is overwritten unless ``accumulate``, which adds onto what ``out`` holds."""
     _check_bits(num_bits)
     ctx.graph = graph
     ctx.num_bits = num_bits
@@ -209,9 +210,10 @@ def _forward(ctx, graph, feats, layer, num_bits: int, is_pre_delay: bool, is_tra
 
     if out is None:
         out = torch.empty([graph.local_adj_t.sparse_size(0), feat_len], dtype=torch.float32, device=feats.device)
+        accumulate = False
     else:
         _check_result(out, graph.local_adj_t.sparse_size(0), feat_len, feats.device)
-    feats.product(graph.local_adj_t, out, False)
+    feats.product(graph.local_adj_t, out, accumulate)
 
     if comm_handle is not None:
         comm_handle.wait()

@@ -160,6 +160,57 @@ class _SageConv(torch.autograd.Function):
         return None, grad_cat, grad_w, grad_b, None, None, None, None, None
 
 
+class _SageConvLinearFirst(torch.autograd.Function):
+    """The same layer with the products taken first: ``A (x W_n) / deg + x W_s + bias``.  Equal to
+    aggregate-first up to rounding ((A x) W = A (x W)); the aggregation, its backward and the
+    boundary exchange then run at the OUTPUT width, which pays when the layer narrows (the switch
+    the reference sketches and leaves commented out, sageconv.py:67-71, :84)."""
+
+    @staticmethod
+    def forward(ctx, graph, feats_in, weight, bias, layer, num_bits, is_pre_delay, is_training, normalize):
+        fi = weight.size(0) // 2
+        ctx.staged = feats_in.size(1) == 2 * fi      # [N, 2 fi] with the features in the right half
+        x = feats_in[:, fi:] if ctx.staged else feats_in
+        folded = getattr(graph, "in_degrees_folded", False)
+        ctx.divide = bool(normalize) and not folded
+        left = torch.mm(x, weight[:fi])                                   # x W_n
+        out = torch.mm(x, weight[fi:]) if bias is None else torch.addmm(bias, x, weight[fi:])
+        feats = aggregator._DenseFeatures(left)
+        if ctx.divide:
+            agg = aggregator._forward(ctx, graph, feats, layer, num_bits, is_pre_delay, is_training)
+            out.addcdiv_(agg, graph.in_degrees)
+        else:  # degrees folded into the matrices (or no normalisation): add straight onto x W_s + b
+            aggregator._forward(ctx, graph, feats, layer, num_bits, is_pre_delay, is_training, out=out,
+                                accumulate=True)
+        ctx.save_for_backward(feats_in, weight)
+        ctx.has_bias = bias is not None
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        feats_in, weight = ctx.saved_tensors
+        fi = weight.size(0) // 2
+        x = feats_in[:, fi:] if ctx.staged else feats_in
+        g = g.contiguous()
+        grad_left = aggregator._backward(ctx, g / ctx.graph.in_degrees if ctx.divide else g)   # d/d (x W_n)
+        grad_x = grad_w = grad_b = None
+        if ctx.needs_input_grad[2]:
+            grad_w = torch.cat([weight_gradient(x, grad_left), weight_gradient(x, g)], dim=0)
+        if ctx.has_bias and ctx.needs_input_grad[3]:
+            grad_b = g.sum(dim=0)
+        if ctx.needs_input_grad[1]:
+            if ctx.staged:
+                # the gradient goes where the features were: the right half of an [N, 2 fi] array
+                # (its left half was scratch on the way forward and is left unwritten here)
+                grad_x = torch.empty(x.size(0), 2 * fi, dtype=torch.float32, device=x.device)
+                target = grad_x[:, fi:]
+                torch.mm(g, weight[fi:].t(), out=target)
+                target.addmm_(grad_left, weight[:fi].t())
+            else:
+                grad_x = torch.addmm(torch.mm(g, weight[fi:].t()), grad_left, weight[:fi].t())
+        return None, grad_x, grad_w, grad_b, None, None, None, None, None
+
+
 class _LinearView:
     """What the reference's ``lin_neigh`` / ``lin_self`` expose: ``weight`` as ``[out, in]`` -- here
     a view of the layer's stacked weight."""
@@ -177,8 +228,11 @@ class DistSAGEConvGrad(torch.nn.Module):
     ``[:in]`` are ``lin_neigh.weight.T``, rows ``[in:]`` are ``lin_self.weight.T``) and ``bias``."""
 
     def __init__(self, in_channels: int, out_channels: int, num_bits: int, is_pre_delay: bool,
-                 add_self_loops: bool = False, normalize: bool = True, bias: bool = True):
+                 add_self_loops: bool = False, normalize: bool = True, bias: bool = True, linear_first: bool = False):
         super().__init__()
+        # linear_first: apply lin_neigh before aggregating (same result up to rounding; the
+        # aggregation and the exchange then run at out_channels)
+        self.linear_first = linear_first
         self.in_channels = in_channels
         self.out_channels = out_channels
         self.add_self_loops = add_self_loops
@@ -221,6 +275,14 @@ class DistSAGEConvGrad(torch.nn.Module):
         already staged ``[N, 2 * in_channels]`` array (``stage_input`` / the fused LayerNorm
         pass) whose left half this call overwrites."""
         width = local_nodes_feat.size(-1)
+        if self.linear_first:
+            if width not in (self.in_channels, 2 * self.in_channels):
+                raise RuntimeError("Input mismatch: expected %d features (or %d staged), got %d"
+                                   % (self.in_channels, 2 * self.in_channels, width))
+            if not local_nodes_feat.is_cuda or local_nodes_feat.dtype != torch.float32:
+                raise RuntimeError("Input mismatch: the features must be a float32 GPU (HIP) tensor")
+            return _SageConvLinearFirst.apply(graph, local_nodes_feat, self.weight, self.bias, layer, self.num_bits,
+                                              self.is_pre_delay, self.training, self.normalize)
         if width == self.in_channels:
             if local_nodes_feat.requires_grad:
                 raise RuntimeError("features that need a gradient must be handed over staged (stage_input)")
@@ -241,7 +303,7 @@ class DistSAGE(torch.nn.Module):
     """DistSAGE.py:13-69: ``num_layers`` SAGE layers, LayerNorm after all but the last."""
 
     def __init__(self, in_channels, hidden_channels, out_channels, num_layers=3, dropout=0.5, num_bits=32,
-                 is_pre_delay=False):
+                 is_pre_delay=False, linear_first_when_narrowing=False):
         super().__init__()
         self.convs = torch.nn.ModuleList()
         self.norms = torch.nn.ModuleList()
@@ -251,6 +313,9 @@ class DistSAGE(torch.nn.Module):
             self.convs.append(DistSAGEConvGrad(hidden_channels, hidden_channels, num_bits, is_pre_delay))
             self.norms.append(torch.nn.LayerNorm(hidden_channels))
         self.convs.append(DistSAGEConvGrad(hidden_channels, out_channels, num_bits, is_pre_delay))
+        if linear_first_when_narrowing:  # a layer with fewer outputs than inputs aggregates its outputs
+            for conv in self.convs:
+                conv.linear_first = conv.out_channels < conv.in_channels
         self.dropout = dropout
 
     def reset_parameters(self):
