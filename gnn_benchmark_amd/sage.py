@@ -134,6 +134,11 @@ class _SageConv(torch.autograd.Function):
         ctx.divide = bool(normalize) and not getattr(graph, "in_degrees_folded", False)
         if ctx.divide:
             agg.div_(graph.in_degrees)  # sageconv.py:80-82
+        else:
+            # the library wrote the left half behind autograd's back: an (empty) in-place op bumps the
+            # array's version, so that an earlier call that kept this same array for its backward
+            # fails loudly there instead of reading rows that are no longer its own
+            cat[:0].zero_()
         out = torch.mm(cat, weight) if bias is None else torch.addmm(bias, cat, weight)
         ctx.save_for_backward(cat, weight)
         ctx.has_bias = bias is not None

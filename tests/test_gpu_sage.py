@@ -361,3 +361,22 @@ def test_fused_layernorm_pass_beyond_2_to_31_elements():
         sl = slice(lo, lo + 1_000_000)
         want = torch.relu(F.layer_norm(z[sl] * keep[sl] * 2.0, (feat,), gamma, beta, 1e-5))
         assert torch.allclose(cat[sl, feat:], want, rtol=1e-5, atol=2e-5), lo
+
+
+def test_reusing_a_staged_array_before_its_backward_is_detected():
+    """A layer keeps its staged array for the weight gradient; a second forward through the same
+    array overwrites the aggregated half, and the first backward must refuse to run on it."""
+    n, f_in, f_out = 500, 8, 8
+    rowptr, col, val = skewed_csr(n, n, seed=4, heavy_rows=(50,))
+    adj = SparseTensor(rowptr=dev(rowptr), col=dev(col), value=dev(val), sparse_sizes=(n, n))
+    splits = CommSplits([0], [0], 1, 32)
+    for folded in (False, True):
+        graph = DistributedGraphForPre(adj, None, None, [0], [0], torch.ones(n, 1, device="cuda"), splits,
+                                       CommBuffer(splits, f_in, 32, device="cuda"))
+        graph.in_degrees_folded = folded
+        conv = sage.DistSAGEConvGrad(f_in, f_out, 32, True).cuda()
+        staged = sage.stage_input(torch.randn(n, f_in, device="cuda"))
+        first = conv(graph, staged, 0)
+        conv(graph, staged, 0)
+        with pytest.raises(RuntimeError, match="modified by an inplace operation"):
+            first.sum().backward()
