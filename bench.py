@@ -373,11 +373,42 @@ def run_c4(args, graph, setup_s):
                   "ms": round(e0.elapsed_time(e1) / steps, 4)})
     graph.fuse_dequantize = False
     graph.comm_splits, graph.comm_buf_for_quantization, graph.exchange_quantized = fp32_splits, None, None
+    # ... and as bf16 (num_bits=16): the two conversion passes per direction around a seeded stand-in
+    from gnn_benchmark_amd.aggregator import _convert
+    from gnn_benchmark_amd.data_manager import CommBuffer
+
+    fp32_buf = graph.comm_buf
+    graph.comm_buf = CommBuffer(fp32_splits, feat, 16, device=dev)
+    graph.exchange_bf16 = synthetic.SeededBf16HaloExchange(args.seed + 7)
+    for _ in range(2):
+        Aggregator.apply(graph, xr, 0, 16, True, True).backward(g)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        o = Aggregator.apply(graph, xr, 0, 16, True, True)
+        o.backward(g)
+    torch.cuda.synchronize()
+    bf16_both_ms = (time.perf_counter() - t0) * 1e3 / steps
+    for name, src, dst in (("send_buf -> bf16", graph.comm_buf.send_buf, graph.comm_buf.send_buf_fp16),
+                           ("bf16 -> recv_buf", graph.comm_buf.recv_buf_fp16, graph.comm_buf.recv_buf)):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for i in range(steps + 2):
+            if i == 2:
+                e0.record()
+            _convert(src, dst)
+        e1.record()
+        e1.synchronize()
+        ms = e0.elapsed_time(e1) / steps
+        codec.append({"op": name, "bits": 16, "rows": int(src.size(0)), "feat": feat, "ms": round(ms, 4),
+                      "gbs": round(src.numel() * 6.0 / (ms * 1e-3) / 1e9, 1),
+                      "frac_of_hbm_peak": round(src.numel() * 6.0 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)})
+    graph.comm_buf, graph.exchange_bf16 = fp32_buf, None
     return {"partition": f"rank 3 of 16, {n} local nodes", "feat": feat, "setup_s": round(setup_s, 2), "codec": codec,
             "local_nnz": graph.local_adj_t.nnz(), "halo_rows": int(recv_buf.size(0)), "send_rows": int(send_buf.size(0)),
             "from_nnz": graph.adj_t_pre_post_aggr_from.nnz(), "to_nnz": graph.adj_t_pre_post_aggr_to.nnz(),
             "ops": ops, "aggregator_forward_ms": round(fwd_ms, 3),
             "aggregator_forward_backward_ms": round(both_ms, 3),
+            "aggregator_forward_backward_ms_bf16_exchange": round(bf16_both_ms, 3),
             "aggregator_forward_backward_ms_int2_exchange": round(int2_both_ms, 3),
             "aggregator_forward_backward_ms_int2_exchange_fused_dequantize": round(int2_fused_ms, 3)}
 

@@ -46,6 +46,8 @@ EXPORTS = (
     "gnnagg_plan_spmm_quantized_f32",
     "gnnagg_quantize_mixed_f32",
     "gnnagg_dequantize_mixed_f32",
+    "gnnagg_f32_to_bf16",
+    "gnnagg_bf16_to_f32",
 )
 
 _lib = None
@@ -112,6 +114,10 @@ def lib() -> ctypes.CDLL:
     L.gnnagg_wgrad_workspace_bytes.argtypes = [i64, i64, i64]
     L.gnnagg_wgrad_f32.restype = i32
     L.gnnagg_wgrad_f32.argtypes = [vp, vp, vp, vp, i64, i64, i64, vp]
+    L.gnnagg_f32_to_bf16.restype = i32
+    L.gnnagg_f32_to_bf16.argtypes = [vp, vp, i64, vp]
+    L.gnnagg_bf16_to_f32.restype = i32
+    L.gnnagg_bf16_to_f32.argtypes = [vp, vp, i64, vp]
     L.gnnagg_wgrad_strided_f32.restype = i32
     L.gnnagg_wgrad_strided_f32.argtypes = [vp, i64, vp, i64, vp, vp, i64, i64, i64, vp]
     L.gnnagg_dropout_layernorm_relu_blocks.restype = i32

@@ -29,6 +29,11 @@ What differs from the reference, on purpose:
   roles of the send and receive buffers swapped (:266-276).  The received rows are
   dequantised after the wait, where the reference does it (aggregator.py:83-88,
   :180-187).  Outside training the forward exchange stays fp32 (communicator.py:64-65).
+* With ``num_bits`` 16 (communicator.py:65-66, :111-137) the outgoing rows are rounded to bf16 into
+  ``comm_buf.send_buf_fp16`` (backward: ``recv_buf_fp16``) and ``graph.exchange_bf16``, same call
+  shape as ``graph.exchange``, must leave the peers' bf16 rows in ``comm_buf.recv_buf_fp16``
+  (backward: ``send_buf_fp16``); they are widened to fp32 after the wait.  Outside training the
+  forward exchange stays fp32.
 * No process group or timers are touched; the quantiser is built from the buffers' width,
   not looked up as a singleton.
 * ``torch.zeros`` + accumulate (aggregator.py:67-70, :167-170) and ``zero_()`` +
@@ -78,6 +83,32 @@ def _quantized(graph, num_bits: int) -> bool:
     if getattr(graph, "exchange_quantized", None) is None:
         raise RuntimeError("graph.exchange_quantized is required for a %d-bit boundary exchange" % num_bits)
     return True
+
+
+def _bf16_wire(graph) -> bool:
+    """communicator.py:65-66, :111-137: with ``num_bits == 16`` the rows travel as bf16 through the
+    staging copies of ``CommBuffer``; the exchange of those copies is ``graph.exchange_bf16``."""
+    cb = graph.comm_buf
+    if getattr(cb, "send_buf_fp16", None) is None or getattr(cb, "recv_buf_fp16", None) is None:
+        raise RuntimeError("Input mismatch: the graph holds no bf16 staging buffers (build it with bits=16)")
+    if getattr(graph, "exchange_bf16", None) is None:
+        raise RuntimeError("graph.exchange_bf16 is required for a 16-bit boundary exchange")
+    return True
+
+
+def _convert(src: torch.Tensor, dst: torch.Tensor) -> None:
+    """fp32 -> bf16 (round to nearest even) or bf16 -> fp32: the two ``copy_`` calls around the
+    16-bit exchange (communicator.py:128, :137)."""
+    if src.numel() != dst.numel() or not src.is_contiguous() or not dst.is_contiguous() or not src.is_cuda:
+        raise RuntimeError("Input mismatch: bf16 staging needs contiguous GPU (HIP) buffers of equal size")
+    L = _lib.lib()
+    with torch.cuda.device(src.device):
+        if src.dtype == torch.float32 and dst.dtype == torch.bfloat16:
+            _lib.check(L.gnnagg_f32_to_bf16(_lib.ptr(src), _lib.ptr(dst), src.numel(), _lib.current_stream(src.device)))
+        elif src.dtype == torch.bfloat16 and dst.dtype == torch.float32:
+            _lib.check(L.gnnagg_bf16_to_f32(_lib.ptr(src), _lib.ptr(dst), src.numel(), _lib.current_stream(src.device)))
+        else:
+            raise RuntimeError("Input mismatch: bf16 staging converts float32 <-> bfloat16 only")
 
 
 def _quantize_and_exchange(graph, num_bits: int, tag: str, direction: str):
@@ -195,6 +226,7 @@ def _forward(ctx, graph, feats, layer, num_bits: int, is_pre_delay: bool, is_tra
     if quantized:
         graph.comm_buf_for_quantization.resize_buffer(graph.comm_splits, feat_len, num_bits)
     quantized = quantized and is_training  # communicator.py:64-65: fp32 rows outside training
+    half = exchange is not None and num_bits == 16 and is_training and _bf16_wire(graph)
     comm_handle = None
     send_buf = graph.comm_buf.send_buf
 
@@ -205,6 +237,9 @@ def _forward(ctx, graph, feats, layer, num_bits: int, is_pre_delay: bool, is_tra
             feats.gather(graph.idx_nodes_send_to_others, send_buf)
         if quantized:
             comm_handle = _quantize_and_exchange(graph, num_bits, f"forward{layer}", "forward")
+        elif half:
+            _convert(send_buf, graph.comm_buf.send_buf_fp16)
+            comm_handle = graph.exchange_bf16(graph.comm_splits, graph.comm_buf, f"forward{layer}", "forward")
         else:
             comm_handle = exchange(graph.comm_splits, graph.comm_buf, f"forward{layer}", "forward")
 
@@ -220,6 +255,8 @@ def _forward(ctx, graph, feats, layer, num_bits: int, is_pre_delay: bool, is_tra
     fused = quantized and _fused_dequantize(graph, feat_len) and out.is_contiguous()
     if quantized and not fused:
         _dequantize_received(graph, num_bits, "forward")
+    if half:
+        _convert(graph.comm_buf.recv_buf_fp16, graph.comm_buf.recv_buf)
 
     remote_nodes_feat = graph.comm_buf.recv_buf
     if exchange is not None and remote_nodes_feat.size(0) != 0:
@@ -258,9 +295,13 @@ def _backward(ctx, local_out_grad, out=None, accumulate: bool = False):
         else:
             SPMM_backward(graph.remote_adj_t, local_out_grad, remote_nodes_grad_buf, accumulate=False)
 
+    half = exchange is not None and num_bits == 16 and _bf16_wire(graph)
     comm_handle = None
     if quantized:
         comm_handle = _quantize_and_exchange(graph, num_bits, layer, "backward")
+    elif half:  # the buffers swap roles on the way back (communicator.py:121-126)
+        _convert(remote_nodes_grad_buf, graph.comm_buf.recv_buf_fp16)
+        comm_handle = graph.exchange_bf16(graph.comm_splits, graph.comm_buf, layer, "backward")
     elif exchange is not None:
         comm_handle = exchange(graph.comm_splits, graph.comm_buf, layer, "backward")
 
@@ -278,6 +319,8 @@ def _backward(ctx, local_out_grad, out=None, accumulate: bool = False):
     fused = quantized and _fused_dequantize(graph, feat_len) and local_nodes_grad.is_contiguous()
     if quantized and not fused:
         _dequantize_received(graph, num_bits, "backward")
+    if half:
+        _convert(graph.comm_buf.send_buf_fp16, graph.comm_buf.send_buf)
 
     local_nodes_grad_buf = graph.comm_buf.send_buf
     if exchange is not None and local_nodes_grad_buf.size(0) != 0:

@@ -489,6 +489,57 @@ int check_segments(const void *a, const void *b, const void *c, const int32_t *r
     return GNNAGG_OK;
 }
 
+
+// ---- bf16 rows on the wire (communicator.py:111-137: send_buf_fp16.copy_(send_buf), the exchange,
+// recv_buf.copy_(recv_buf_fp16)): round to nearest even, NaN -> 0x7FC0, as the tensor copy does.
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef unsigned short u16x4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ unsigned short bf16_bits(float x) {
+    const uint32_t u = __float_as_uint(x);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)0x7fc0;
+    return (unsigned short)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+
+__global__ __launch_bounds__(256) void f32_to_bf16_kernel(const float *__restrict__ x, unsigned short *__restrict__ y,
+                                                          int64_t count, int vec) {
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    const int64_t tid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t n4 = vec ? count / 4 : 0;
+    for (int64_t i = tid; i < n4; i += stride) {
+        const f32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t *>(x) + i);
+        u16x4_t r;
+        r.x = bf16_bits(v.x);
+        r.y = bf16_bits(v.y);
+        r.z = bf16_bits(v.z);
+        r.w = bf16_bits(v.w);
+        __builtin_nontemporal_store(r, reinterpret_cast<u16x4_t *>(y) + i);
+    }
+    for (int64_t i = n4 * 4 + tid; i < count; i += stride) y[i] = bf16_bits(x[i]);
+}
+
+__global__ __launch_bounds__(256) void bf16_to_f32_kernel(const unsigned short *__restrict__ x, float *__restrict__ y,
+                                                          int64_t count, int vec) {
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    const int64_t tid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t n4 = vec ? count / 4 : 0;
+    for (int64_t i = tid; i < n4; i += stride) {
+        const u16x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u16x4_t *>(x) + i);
+        f32x4_t r;
+        r.x = __uint_as_float((uint32_t)v.x << 16);
+        r.y = __uint_as_float((uint32_t)v.y << 16);
+        r.z = __uint_as_float((uint32_t)v.z << 16);
+        r.w = __uint_as_float((uint32_t)v.w << 16);
+        __builtin_nontemporal_store(r, reinterpret_cast<f32x4_t *>(y) + i);
+    }
+    for (int64_t i = n4 * 4 + tid; i < count; i += stride) y[i] = __uint_as_float((uint32_t)x[i] << 16);
+}
+
+unsigned stream_blocks(int64_t items) {
+    const int64_t blocks = (items + 255) / 256;
+    return (unsigned)(blocks < 256 * 64 ? (blocks > 0 ? blocks : 1) : 256 * 64);
+}
+
 }  // namespace
 }  // namespace gnnagg
 
@@ -553,6 +604,28 @@ extern "C" int gnnagg_dequantize_mixed_f32(const uint8_t *data, const int64_t *f
     GNNAGG_REQUIRE(data && feat_range && params && out && bad_width, "null pointer");
     hipLaunchKernelGGL(dequantize_mixed_kernel, dim3(grid_for(rows * 64, 256)), dim3(256), 0,
                        static_cast<hipStream_t>(stream), data, feat_range, params, out, (int)rows, (int)feat, bad_width);
+    GNNAGG_HIP(hipGetLastError());
+    return GNNAGG_OK;
+}
+
+extern "C" int gnnagg_f32_to_bf16(const float *x, uint16_t *y, int64_t count, void *stream) {
+    GNNAGG_REQUIRE(count >= 0, "negative size");
+    if (count == 0) return GNNAGG_OK;
+    GNNAGG_REQUIRE(x && y, "null x / y");
+    const int vec = (reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 8 == 0) ? 1 : 0;
+    hipLaunchKernelGGL(f32_to_bf16_kernel, dim3(stream_blocks(vec ? count / 4 + 3 : count)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), x, y, count, vec);
+    GNNAGG_HIP(hipGetLastError());
+    return GNNAGG_OK;
+}
+
+extern "C" int gnnagg_bf16_to_f32(const uint16_t *x, float *y, int64_t count, void *stream) {
+    GNNAGG_REQUIRE(count >= 0, "negative size");
+    if (count == 0) return GNNAGG_OK;
+    GNNAGG_REQUIRE(x && y, "null x / y");
+    const int vec = (reinterpret_cast<uintptr_t>(x) % 8 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0) ? 1 : 0;
+    hipLaunchKernelGGL(bf16_to_f32_kernel, dim3(stream_blocks(vec ? count / 4 + 3 : count)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), x, y, count, vec);
     GNNAGG_HIP(hipGetLastError());
     return GNNAGG_OK;
 }

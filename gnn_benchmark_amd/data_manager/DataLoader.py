@@ -57,7 +57,8 @@ def _quantization_buffers(comm_splits, max_feat_len, bits, device):
 def get_distributed_graph(local_edges_list, remote_edges_list, local_nodes_list, nodes_range_on_each_subgraph,
                           num_local_nodes: int, max_feat_len: int, world_size: int, bits: int, *,
                           halo_id_exchange: Optional[Callable] = None, exchange: Optional[Callable] = None,
-                          exchange_quantized: Optional[Callable] = None, device=None) -> DistributedGraph:
+                          exchange_quantized: Optional[Callable] = None, exchange_bf16: Optional[Callable] = None,
+                          device=None) -> DistributedGraph:
     local_edges_list = _to_device(local_edges_list, device)
     remote_edges_list = _to_device(remote_edges_list, device)
     in_degrees = DataProcessor.get_in_degrees(local_edges_list, remote_edges_list, num_local_nodes)
@@ -78,7 +79,7 @@ def get_distributed_graph(local_edges_list, remote_edges_list, local_nodes_list,
                             num_local_nodes_required_by_other.tolist(), remote_nodes_num_from_each_subgraph.tolist(),
                             in_degrees, comm_splits, comm_buf,
                             _quantization_buffers(comm_splits, max_feat_len, bits, local_adj_t.device),
-                            exchange=exchange, exchange_quantized=exchange_quantized)
+                            exchange=exchange, exchange_quantized=exchange_quantized, exchange_bf16=exchange_bf16)
 
 
 def get_distributed_graph_for_pre_aggressive(local_edges_list, remote_edges_list, nodes_range_on_each_subgraph,
@@ -86,6 +87,7 @@ def get_distributed_graph_for_pre_aggressive(local_edges_list, remote_edges_list
                                              graph_exchange: Optional[Callable] = None,
                                              exchange: Optional[Callable] = None,
                                              exchange_quantized: Optional[Callable] = None,
+                                             exchange_bf16: Optional[Callable] = None,
                                              device=None) -> DistributedGraphForPre:
     local_edges_list = _to_device(local_edges_list, device)
     remote_edges_list = _to_device(remote_edges_list, device)
@@ -105,4 +107,4 @@ def get_distributed_graph_for_pre_aggressive(local_edges_list, remote_edges_list
     return DistributedGraphForPre(local_adj_t, adj_t_pre_post_aggr_from, adj_t_pre_post_aggr_to, from_splits,
                                   to_splits, in_degrees, comm_splits, comm_buf,
                                   _quantization_buffers(comm_splits, max_feat_len, bits, local_adj_t.device),
-                                  exchange=exchange, exchange_quantized=exchange_quantized)
+                                  exchange=exchange, exchange_quantized=exchange_quantized, exchange_bf16=exchange_bf16)

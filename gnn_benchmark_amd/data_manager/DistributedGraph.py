@@ -8,7 +8,8 @@ all-to-all (model/layers/aggregator.py:54-61, :156-163) -- ``None`` means a sing
 world: the aggregator then skips pre-/post-aggregation exactly like the reference does for
 ``world_size == 1`` (aggregator.py:47, :100) -- and ``exchange_quantized``, its counterpart
 for the packed bytes and per-row parameters of a quantised exchange
-(communicator.py:231-325).
+(communicator.py:231-325), and ``exchange_bf16`` for the bf16 staging copies of a 16-bit one
+(communicator.py:111-137).
 """
 from dataclasses import dataclass, field
 from typing import Any, Callable, List, Optional
@@ -34,6 +35,7 @@ class DistributedGraph:
     comm_buf_for_quantization: Any = None      # CommBufferForQuantization for bits 2 / 4 / 8
     exchange: Optional[Callable] = None
     exchange_quantized: Optional[Callable] = None
+    exchange_bf16: Optional[Callable] = None
     in_degrees_folded: bool = False            # the matrices' rows already carry 1 / in_degrees
     _scatter: Optional[SparseTensor] = field(default=None, repr=False)
 
@@ -64,4 +66,5 @@ class DistributedGraphForPre:
     comm_buf_for_quantization: Any = None
     exchange: Optional[Callable] = None
     exchange_quantized: Optional[Callable] = None
+    exchange_bf16: Optional[Callable] = None
     in_degrees_folded: bool = False

@@ -228,9 +228,27 @@ class SeededQuantizedHaloExchange:
         return None
 
 
+class SeededBf16HaloExchange:
+    """bf16 counterpart of SeededHaloExchange: fills the bf16 staging copy the aggregator widens."""
+
+    def __init__(self, seed: int = 0):
+        self.seed = seed
+        self._gen = None
+        self.calls: List[str] = []
+
+    def __call__(self, comm_splits, comm_buf, tag: str, direction: str):
+        target = comm_buf.recv_buf_fp16 if direction == "forward" else comm_buf.send_buf_fp16
+        if self._gen is None or self._gen.device != target.device:
+            self._gen = torch.Generator(device=target.device)
+        self._gen.manual_seed(self.seed * 1000003 + 11 + sum(ord(c) * (i + 1) for i, c in enumerate(tag)))
+        target.normal_(generator=self._gen)
+        self.calls.append(tag)
+        return None
+
+
 def build_partition_graph(part: PartitionData, max_feat_len: int, is_pre_delay: bool,
                           exchange: Optional[Callable] = None, bits: int = 32, device="cuda",
-                          exchange_quantized: Optional[Callable] = None):
+                          exchange_quantized: Optional[Callable] = None, exchange_bf16: Optional[Callable] = None):
     """DistributedGraphForPre (pre/post-aggregation) or DistributedGraph (raw halo rows) of
     one synthetic partition."""
     local_edges = part.local_edges.clone()
@@ -239,7 +257,7 @@ def build_partition_graph(part: PartitionData, max_feat_len: int, is_pre_delay: 
         return get_distributed_graph_for_pre_aggressive(
             local_edges, remote_edges, part.begins, part.num_local_nodes, max_feat_len, part.rank, part.world_size,
             bits, graph_exchange=mirrored_graph_exchange(part), exchange=exchange,
-            exchange_quantized=exchange_quantized, device=device)
+            exchange_quantized=exchange_quantized, exchange_bf16=exchange_bf16, device=device)
     begin = int(part.begins[part.rank])
     local_nodes_list = torch.stack((torch.arange(begin, begin + part.num_local_nodes), ) * 2, dim=1)
 
@@ -254,4 +272,5 @@ def build_partition_graph(part: PartitionData, max_feat_len: int, is_pre_delay: 
 
     return get_distributed_graph(local_edges, remote_edges, local_nodes_list, part.begins, part.num_local_nodes,
                                  max_feat_len, part.world_size, bits, halo_id_exchange=halo_id_exchange,
-                                 exchange=exchange, exchange_quantized=exchange_quantized, device=device)
+                                 exchange=exchange, exchange_quantized=exchange_quantized, exchange_bf16=exchange_bf16,
+                                 device=device)

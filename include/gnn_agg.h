@@ -294,6 +294,13 @@ int gnnagg_quantize_mixed_f32(const float *x, uint8_t *data, const int64_t *feat
 int gnnagg_dequantize_mixed_f32(const uint8_t *data, const int64_t *feat_range, const float *params, float *out,
                                 int64_t rows, int64_t feat, int32_t *bad_width, void *stream);
 
+/* bf16 rows on the wire: what `send_buf_fp16.copy_(send_buf)` and `recv_buf.copy_(recv_buf_fp16)` do
+ * around the 16-bit exchange (communicator.py:111-137).  fp32 -> bf16 rounds to nearest even (NaN ->
+ * 0x7FC0), bf16 -> fp32 is exact.  x, y: `count` contiguous values.  6 bytes moved per value;
+ * allocate nothing, no host sync. */
+int gnnagg_f32_to_bf16(const float *x, uint16_t *y, int64_t count, void *stream);
+int gnnagg_bf16_to_f32(const uint16_t *x, float *y, int64_t count, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -381,3 +381,102 @@ def test_row_gather_equals_index_select(feat, count):
     out2 = torch.empty(count * feat + 1, device="cuda")[1:].view(count, feat)
     _gather_rows(src2, index, out2)
     assert torch.equal(out2, src2[index])
+
+
+class PlayedBf16Exchange:
+    """The 16-bit exchange of one simulated rank: checks what the aggregator staged for sending and
+    delivers the peers' bf16 rows into the staging copy the aggregator widens afterwards."""
+
+    def __init__(self, forward_rows, backward_rows):
+        self.forward_rows, self.backward_rows = forward_rows, backward_rows  # fp32 values exactly representable in bf16
+        self.sent = {}
+
+    def __call__(self, comm_splits, comm_buf, tag, direction):
+        if direction == "forward":
+            self.sent[direction] = comm_buf.send_buf_fp16.clone()
+            comm_buf.recv_buf_fp16.copy_(self.forward_rows)   # exact: the values are bf16 already
+        else:
+            self.sent[direction] = comm_buf.recv_buf_fp16.clone()
+            comm_buf.send_buf_fp16.copy_(self.backward_rows)
+        return None
+
+
+@pytest.mark.parametrize("seed,sizes", [(0, (300, 450, 250)), (1, (600, 1, 400, 330))])
+def test_bf16_exchange_world_matches_oracle(seed, sizes):
+    """Boundary rows travelling as bf16 (num_bits=16, communicator.py:111-137): what every rank
+    stages for sending equals the oracle's rows rounded to bf16 bit for bit, and output and gradient
+    equal the oracle pipeline fed with the rounded rows."""
+    from oracle import quantization as oq
+
+    w = World(seed, sizes, mean_deg=8.0)
+    W, F = w.world, 40
+    graphs = _build_pre_graphs(w, F, bits=16)
+    oracle_ranks = build_pre_world(w)
+    rng = np.random.default_rng(seed + 200)
+    x = (rng.standard_normal((w.n, F)) * rng.uniform(1e-3, 1e3, (w.n, 1))).astype(np.float32)
+    g = rng.standard_normal((w.n, F)).astype(np.float32)
+    sl = [slice(int(w.begins[r]), int(w.begins[r + 1])) for r in range(W)]
+    send_splits = [gr.comm_splits.send_splits for gr in graphs]
+    recv_splits = [gr.comm_splits.recv_splits for gr in graphs]
+    o_send = [oq.to_bf16_and_back(oagg.forward_send(oracle_ranks[r]["a_to"], np.ascontiguousarray(x[sl[r]])))
+              for r in range(W)]
+    o_back = [oq.to_bf16_and_back(oagg.backward_recv(oracle_ranks[r]["a_from"], np.ascontiguousarray(g[sl[r]])))
+              for r in range(W)]
+    recv = host_exchange(o_send, send_splits, recv_splits)
+    incoming = host_exchange(o_back, recv_splits, send_splits)
+    for r in range(W):
+        gr, o = graphs[r], oracle_ranks[r]
+        gr.exchange = lambda *a: (_ for _ in ()).throw(AssertionError("fp32 exchange used in a 16-bit run"))
+        gr.exchange_bf16 = PlayedBf16Exchange(dev(recv[r]), dev(incoming[r]))
+        xr = dev(x[sl[r]]).requires_grad_()
+        out = Aggregator.apply(gr, xr, 2, 16, True, True)
+        assert np.array_equal(gr.exchange_bf16.sent["forward"].float().cpu().numpy().view(np.uint32),
+                              o_send[r].view(np.uint32))
+        assert np.array_equal(gr.comm_buf.recv_buf.cpu().numpy(), recv[r])
+        o_out = oagg.forward_out(o["local"], o["a_from"], np.ascontiguousarray(x[sl[r]]), recv[r])
+        assert np.array_equal(out.detach().cpu().numpy(), o_out)
+        out.backward(dev(g[sl[r]]))
+        assert np.array_equal(gr.exchange_bf16.sent["backward"].float().cpu().numpy().view(np.uint32),
+                              o_back[r].view(np.uint32))
+        o_dx = oagg.backward_out(o["local"], o["a_to"], np.ascontiguousarray(g[sl[r]]), incoming[r])
+        assert np.array_equal(xr.grad.cpu().numpy(), o_dx)
+    # outside training the forward exchange carries fp32 rows (communicator.py:63-64)
+    gr = graphs[0]
+    exact = host_exchange([oagg.forward_send(oracle_ranks[r]["a_to"], np.ascontiguousarray(x[sl[r]])) for r in range(W)],
+                          send_splits, recv_splits)
+    gr.exchange = PlayedExchange(dev(exact[0]), None)
+    gr.exchange_bf16 = lambda *a: (_ for _ in ()).throw(AssertionError("bf16 exchange used outside training"))
+    out = Aggregator.apply(gr, dev(x[sl[0]]), 2, 16, True, False)
+    assert np.array_equal(out.cpu().numpy(), oagg.forward_out(oracle_ranks[0]["local"], oracle_ranks[0]["a_from"],
+                                                              np.ascontiguousarray(x[sl[0]]), exact[0]))
+    # a 16-bit run needs its staging copies and its hook
+    plain = _build_pre_graphs(w, F)
+    plain[0].exchange = PlayedExchange(None, None)
+    with pytest.raises(RuntimeError, match="bf16 staging buffers"):
+        Aggregator.apply(plain[0], dev(x[sl[0]]), 0, 16, True, True)
+    graphs[1].exchange_bf16 = None
+    with pytest.raises(RuntimeError, match="exchange_bf16"):
+        Aggregator.apply(graphs[1], dev(x[sl[1]]), 0, 16, True, True)
+
+
+@pytest.mark.parametrize("count", [0, 1, 3, 4, 1000, 1_000_003])
+def test_bf16_conversion_equals_the_tensor_copy(count):
+    """fp32 -> bf16 -> fp32 through the library against torch's own conversion, bit for bit:
+    ties, both zeros, infinities, NaN, denormals, unaligned starts."""
+    from gnn_benchmark_amd.aggregator import _convert
+
+    gen = torch.Generator(device="cuda").manual_seed(count)
+    base = torch.randn(count + 1, device="cuda", generator=gen) * 100.0
+    special = torch.tensor([0.0, -0.0, float("inf"), -float("inf"), float("nan"), 1.0 + 2.0 ** -8, 1.0 + 3 * 2.0 ** -8,
+                            1e-40, -1e-40, 3.3895314e38], device="cuda")
+    k = min(count, special.numel())
+    base[1:1 + k] = special[:k]
+    for offset in (0, 1):
+        src = base[offset:offset + count]
+        half = torch.empty(count + 1, dtype=torch.bfloat16, device="cuda")[offset:offset + count]
+        _convert(src, half)
+        want = src.to(torch.bfloat16)
+        assert torch.equal(half.view(torch.int16), want.view(torch.int16))
+        back = torch.empty(count + 1, device="cuda")[offset:offset + count]
+        _convert(half, back)
+        assert torch.equal(back.view(torch.int32), want.float().view(torch.int32))
