@@ -138,7 +138,7 @@ def to_bf16_and_back(x: np.ndarray) -> np.ndarray:
     u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
     rounded = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16
     nan = (u & 0x7FFFFFFF) > 0x7F800000
-    rounded = np.where(nan, 0x7FC00000, rounded)  # the tensor copy turns every NaN into this one
+    rounded = np.where(nan, 0x7FC00000, rounded)  # c10::BFloat16's scalar conversion; NaN payloads are not pinned
     return (rounded & 0xFFFFFFFF).astype(np.uint32).view(np.float32).reshape(np.shape(x))
 
 

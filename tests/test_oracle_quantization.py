@@ -142,7 +142,8 @@ def test_bf16_round_trip_matches_torch():
 
     rng = np.random.default_rng(5)
     x = np.concatenate([(rng.standard_normal(5000) * 10.0 ** rng.integers(-20, 20, 5000)).astype(np.float32),
-                        np.array([0.0, -0.0, 1.00390625, 1.01171875, np.inf, -np.inf, 3.3895314e38, np.nan, -np.nan, 1e-40],
-                                 dtype=np.float32)])
+                        np.array([0.0, -0.0, 1.00390625, 1.01171875, np.inf, -np.inf, 3.3895314e38, 1e-40], dtype=np.float32)])
     want = torch.from_numpy(x).to(torch.bfloat16).to(torch.float32).numpy()
     assert np.array_equal(oq.to_bf16_and_back(x).view(np.uint32), want.view(np.uint32))
+    # NaN stays NaN; which NaN differs between torch's own scalar and vector code, so only that much is pinned
+    assert np.isnan(oq.to_bf16_and_back(np.array([np.nan, -np.nan], dtype=np.float32))).all()
