@@ -116,7 +116,13 @@ class _DropoutLayerNormRelu(torch.autograd.Function):
 
 
 def dropout_layernorm_relu(z, keep, scale, gamma, beta, eps) -> torch.Tensor:
-    """Staged input ``[N, 2F]`` of the next layer (right half = the activations)."""
+    """Staged input ``[N, 2F]`` of the next layer (right half = the activations).  Widths the fused
+    pass does not take (not a multiple of 4, or above 1024) go through the same torch ops on the GPU."""
+    rows, feat = z.shape
+    if z.is_cuda and rows > 0 and int(_lib.lib().gnnagg_dropout_layernorm_relu_blocks(rows, feat)) == 0:
+        d = z if keep is None else z * keep * scale
+        y = torch.relu(F.layer_norm(d, (feat,), gamma, beta, eps))
+        return torch.cat([torch.zeros_like(y), y], dim=1)
     return _DropoutLayerNormRelu.apply(z, keep, scale, gamma, beta, eps)
 
 

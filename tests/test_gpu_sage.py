@@ -121,10 +121,16 @@ def test_fused_dropout_layernorm_relu_matches_torch(rows, feat, with_mask):
 
 def test_fused_layernorm_rejects_what_it_cannot_take():
     z = torch.randn(8, 6, device="cuda")
+    gamma, beta = torch.rand(6, device="cuda") + 0.5, torch.randn(6, device="cuda")
     with pytest.raises(RuntimeError, match="multiples of 4"):
-        sage.dropout_layernorm_relu(z, None, 1.0, torch.ones(6, device="cuda"), torch.zeros(6, device="cuda"), 1e-5)
+        sage._DropoutLayerNormRelu.apply(z, None, 1.0, gamma, beta, 1e-5)
     with pytest.raises(RuntimeError, match="Input mismatch"):
         sage.dropout_layernorm_relu(torch.randn(8, 8), None, 1.0, torch.ones(8), torch.zeros(8), 1e-5)
+    # the public entry sends such a width through torch's ops on the device, same staged layout
+    keep = torch.rand(8, 6, device="cuda") >= 0.5
+    cat = sage.dropout_layernorm_relu(z, keep, 2.0, gamma, beta, 1e-5)
+    assert cat.shape == (8, 12)
+    assert torch.equal(cat[:, 6:], torch.relu(F.layer_norm(z * keep * 2.0, (6,), gamma, beta, 1e-5)))
 
 
 # ------------------------------------------------------------------ layer and model
