@@ -271,7 +271,8 @@ def build_c4(args):
                                      local_mean_out_degree=6.8, zipf_s=1.8, max_degree=15000,
                                      num_halo_nodes=int(args.c4_nodes * 3 / 7),
                                      num_remote_edges=int(args.c4_nodes * 20 / 7), seed=args.seed + 4, device=dev)
-    exchange = synthetic.SeededHaloExchange(args.seed + 4)
+    # stand-in rows on the scale of real ones: features O(0.1), gradients of a mean loss O(1e-7)
+    exchange = synthetic.SeededHaloExchange(args.seed + 4, std=0.1, backward_std=1e-7)
     graph = synthetic.build_partition_graph(part, 256, True, exchange=exchange, device=dev)
     for m in (graph.local_adj_t, graph.adj_t_pre_post_aggr_from, graph.adj_t_pre_post_aggr_to):
         m.get_plan()
@@ -588,10 +589,13 @@ def run_c5(args, graph):
     out = {"dims": dims, "nodes": n, "labelled": int(train_idx.numel()), "dropout": 0.5, "optimizer": "Adam(lr=0.01)",
            "steps": steps}
     # the two GEMM variants with dense hidden activations, then the same with the hidden activations
-    # kept packed (non-zero values + bitmap), which the next layer's aggregation gathers instead
-    for gemm, packed_activations in (("fp32", False), ("bf16", False), ("fp32", True), ("bf16", True)):
+    # kept packed (non-zero values + bitmap), which the next layer's aggregation gathers instead,
+    # then with the narrowing last layer multiplying before it aggregates (A (x W) instead of (A x) W)
+    for gemm, packed_activations, linear_first in (("fp32", False, False), ("bf16", False, False), ("fp32", True, False),
+                                                   ("bf16", True, False), ("fp32", True, True), ("bf16", True, True)):
         torch.manual_seed(args.seed)
-        model = gcn.GCN(dims, gemm=gemm, packed_activations=packed_activations).to(dev)
+        model = gcn.GCN(dims, gemm=gemm, packed_activations=packed_activations,
+                        linear_first_when_narrowing=linear_first).to(dev)
         opt = torch.optim.Adam(model.parameters(), lr=0.01)
         losses = [float(gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks)) for _ in range(2)]
         torch.cuda.synchronize()
@@ -599,7 +603,8 @@ def run_c5(args, graph):
         for _ in range(steps):
             loss = gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks)
         torch.cuda.synchronize()
-        tag = f"{gemm}_gemm" + ("_packed_activations" if packed_activations else "")
+        tag = (f"{gemm}_gemm" + ("_packed_activations" if packed_activations else "")
+               + ("_linear_first_when_narrowing" if linear_first else ""))
         out[f"train_step_ms_{tag}"] = round((time.perf_counter() - t0) * 1e3 / steps, 2)
         out[f"loss_{tag}"] = [round(v, 5) for v in losses + [float(loss)]]
         del model, opt

@@ -179,20 +179,27 @@ class GCNLayer(torch.nn.Module):
         if gemm not in ("fp32", "bf16"):
             raise ValueError("gemm must be 'fp32' or 'bf16'")
         self.gemm = gemm
+        self.linear_first = False
         self.weight = torch.nn.Parameter(torch.empty(in_channels, out_channels))
         self.bias = torch.nn.Parameter(torch.zeros(out_channels))
         torch.nn.init.xavier_uniform_(self.weight, gain=torch.nn.init.calculate_gain("relu"))
 
+    def _product(self, t: torch.Tensor) -> torch.Tensor:
+        if self.gemm == "bf16":
+            return _Bf16InputLinear.apply(t, self.weight)
+        return _Fp32Linear.apply(t, self.weight)
+
     def transform(self, graph, x, layer: int, is_pre_delay: bool) -> torch.Tensor:
         """(A x) W: neither the degree normalisation nor the bias yet.  ``x`` is a dense tensor
-        or a packed ``(values, header)`` pair."""
+        or a packed ``(values, header)`` pair.  With ``linear_first`` (and dense ``x``) the
+        product comes first, A (x W): the same up to rounding, and the aggregation, its backward
+        and the boundary rows then have the output width."""
         if isinstance(x, tuple):
             agg = AggregatorPacked.apply(graph, x[0], x[1], layer, 32, is_pre_delay, self.training)
-        else:
-            agg = Aggregator.apply(graph, x, layer, 32, is_pre_delay, self.training)
-        if self.gemm == "bf16":
-            return _Bf16InputLinear.apply(agg, self.weight)
-        return _Fp32Linear.apply(agg, self.weight)
+            return self._product(agg)
+        if self.linear_first:
+            return Aggregator.apply(graph, self._product(x), layer, 32, is_pre_delay, self.training)
+        return self._product(Aggregator.apply(graph, x, layer, 32, is_pre_delay, self.training))
 
     def forward(self, graph, x: torch.Tensor, layer: int, is_pre_delay: bool) -> torch.Tensor:
         """((A x) W) / deg + bias."""
@@ -200,9 +207,13 @@ class GCNLayer(torch.nn.Module):
 
 
 class GCN(torch.nn.Module):
-    def __init__(self, dims: Sequence[int], gemm: str = "fp32", dropout: float = 0.5, packed_activations: bool = False):
+    def __init__(self, dims: Sequence[int], gemm: str = "fp32", dropout: float = 0.5, packed_activations: bool = False,
+                 linear_first_when_narrowing: bool = False):
         super().__init__()
         self.layers = torch.nn.ModuleList([GCNLayer(dims[i], dims[i + 1], gemm) for i in range(len(dims) - 1)])
+        if linear_first_when_narrowing:  # a layer with fewer outputs than inputs aggregates its outputs
+            for i, layer in enumerate(self.layers):
+                layer.linear_first = dims[i + 1] < dims[i]
         self.dropout = dropout
         # keep hidden activations packed (non-zero values + bitmap) where their width allows and
         # pre-aggregation is used: the next layer's aggregation then skips the zeros
@@ -219,8 +230,9 @@ class GCN(torch.nn.Module):
                 break
             z = layer.transform(graph, h, l, is_pre_delay)
             single_rank = getattr(graph, "exchange", None) is None
+            # a next layer that multiplies first reads its input densely: nothing to gain from packing
             pack = (self.packed_activations and (is_pre_delay or single_rank)
-                    and packed.header_words(z.size(1)) > 0)
+                    and packed.header_words(z.size(1)) > 0 and not self.layers[l + 1].linear_first)
             epilogue = _BiasReluDropoutPacked if pack else _BiasReluDropout
             if self.training and self.dropout > 0.0:
                 if masks is None:

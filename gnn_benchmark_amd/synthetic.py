@@ -186,10 +186,13 @@ class SeededHaloExchange:
     """Stand-in for the per-layer boundary all-to-all: on "forward" the receive buffer is
     filled with seeded N(0,1) rows generated on the device, on "backward" the send
     buffer is (those are the rows a real exchange would have delivered).  The fill is
-    enqueued on the current stream; ``wait()`` is a no-op."""
+    enqueued on the current stream; ``wait()`` is a no-op.  ``std`` / ``backward_std`` scale the
+    rows (feature rows and gradient rows live on very different scales in a real run)."""
 
-    def __init__(self, seed: int = 0):
+    def __init__(self, seed: int = 0, std: float = 1.0, backward_std: Optional[float] = None):
         self.seed = seed
+        self.std = std
+        self.backward_std = std if backward_std is None else backward_std
         self._gen = None
         self.calls: List[str] = []
 
@@ -199,7 +202,7 @@ class SeededHaloExchange:
             self._gen = torch.Generator(device=buf.device)
         # one reproducible stream of numbers per (layer tag)
         self._gen.manual_seed(self.seed * 1000003 + sum(ord(c) * (i + 1) for i, c in enumerate(tag)))
-        buf.normal_(generator=self._gen)
+        buf.normal_(0.0, self.std if direction == "forward" else self.backward_std, generator=self._gen)
         self.calls.append(tag)
         return None
 
