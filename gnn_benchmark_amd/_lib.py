@@ -139,7 +139,7 @@ def lib() -> ctypes.CDLL:
     L.gnnagg_dequantize_segments_f32.restype = i32
     L.gnnagg_dequantize_segments_f32.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp]
     L.gnnagg_plan_spmm_quantized_f32.restype = i32
-    L.gnnagg_plan_spmm_quantized_f32.argtypes = [vp, vp, vp, vp, vp, vp, i64, i32, i32, vp]
+    L.gnnagg_plan_spmm_quantized_f32.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i32, i32, vp]
     L.gnnagg_quantize_mixed_f32.restype = i32
     L.gnnagg_quantize_mixed_f32.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp]
     L.gnnagg_dequantize_mixed_f32.restype = i32

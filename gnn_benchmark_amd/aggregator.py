@@ -252,7 +252,7 @@ def _forward(ctx, graph, feats, layer, num_bits: int, is_pre_delay: bool, is_tra
 
     if comm_handle is not None:
         comm_handle.wait()
-    fused = quantized and _fused_dequantize(graph, feat_len) and out.is_contiguous()
+    fused = quantized and _fused_dequantize(graph, feat_len) and out.stride(0) % 4 == 0
     if quantized and not fused:
         _dequantize_received(graph, num_bits, "forward")
     if half:
@@ -316,7 +316,7 @@ def _backward(ctx, local_out_grad, out=None, accumulate: bool = False):
 
     if comm_handle is not None:
         comm_handle.wait()
-    fused = quantized and _fused_dequantize(graph, feat_len) and local_nodes_grad.is_contiguous()
+    fused = quantized and _fused_dequantize(graph, feat_len) and local_nodes_grad.stride(0) % 4 == 0
     if quantized and not fused:
         _dequantize_received(graph, num_bits, "backward")
     if half:

@@ -564,8 +564,8 @@ extern "C" int gnnagg_plan_spmm_packed_f32(gnnagg_plan *plan, const float *value
 }
 
 extern "C" int gnnagg_plan_spmm_quantized_f32(gnnagg_plan *plan, const float *value, const uint8_t *packed,
-                                              const float *params, const int32_t *row_code, float *out, int64_t feat,
-                                              int bits, int accumulate, void *stream) {
+                                              const float *params, const int32_t *row_code, float *out,
+                                              int64_t out_stride, int64_t feat, int bits, int accumulate, void *stream) {
     GNNAGG_REQUIRE(plan, "null plan");
     GNNAGG_REQUIRE(bits == 2 || bits == 4 || bits == 8, "bits must be 2, 4 or 8 (got %d)", bits);
     GNNAGG_REQUIRE(feat >= 0, "negative feature width");
@@ -576,6 +576,9 @@ extern "C" int gnnagg_plan_spmm_quantized_f32(gnnagg_plan *plan, const float *va
                     (long long)feat);
     GNNAGG_REQUIRE(out, "null out");
     GNNAGG_REQUIRE(plan->nnz == 0 || (value && packed && params && row_code), "null value/packed/params/row_code");
+    GNNAGG_REQUIRE(out_stride >= feat && out_stride % 4 == 0 && out_stride < (int64_t(1) << 31),
+                   "output row stride %lld must be a multiple of 4, at least the width and below 2^31",
+                   (long long)out_stride);
     GNNAGG_REQUIRE((reinterpret_cast<uintptr_t>(out) & 15) == 0 && (reinterpret_cast<uintptr_t>(packed) & 3) == 0 &&
                        (reinterpret_cast<uintptr_t>(params) & 7) == 0,
                    "quantised SpMM needs a 16-byte aligned output, 4-byte aligned bytes and 8-byte aligned parameters");
@@ -591,6 +594,7 @@ extern "C" int gnnagg_plan_spmm_quantized_f32(gnnagg_plan *plan, const float *va
         a.qcode = row_code;
         a.qbits = bits;
         a.dst = out;
+        a.ldd = (int)out_stride;
         a.feat = (int)feat;
         a.f_base = (int)f_base;
         a.accumulate = accumulate;

@@ -12,7 +12,7 @@ cached here is the degree-binned plan (``SparseTensor.get_plan``).
 import torch
 
 from . import _lib
-from .sparse_tensor import SparseTensor
+from .sparse_tensor import SparseTensor, _row_stride, _rows_are_dense
 
 
 def _as_f32(value: torch.Tensor, other: torch.Tensor) -> torch.Tensor:
@@ -47,13 +47,13 @@ def _spmm_quantized(plan, value, packed, params, row_code, out, bits, accumulate
     if (packed.dtype != torch.uint8 or not packed.is_contiguous() or packed.dim() != 2 or packed.size(1) != feat
             or params.dtype != torch.float32 or not params.is_contiguous() or tuple(params.shape) != (operand_rows, 2)
             or row_code.dtype != torch.int32 or not row_code.is_contiguous() or row_code.numel() != operand_rows
-            or out.dtype != torch.float32 or not out.is_contiguous() or value.dtype != torch.float32):
+            or out.dtype != torch.float32 or not _rows_are_dense(out) or value.dtype != torch.float32):
         raise RuntimeError("Input mismatch: quantised SpMM needs uint8 [packed rows, F] bytes, float32 [rows, 2] "
-                           "parameters, int32 [rows] row codes and a contiguous float32 [*, F] output")
+                           "parameters, int32 [rows] row codes and a float32 [*, F] output with contiguous rows")
     with torch.cuda.device(out.device):
         _lib.check(_lib.lib().gnnagg_plan_spmm_quantized_f32(
             plan._handle, _lib.ptr(value.contiguous()), _lib.ptr(packed), _lib.ptr(params), _lib.ptr(row_code),
-            _lib.ptr(out), feat, int(bits), 1 if accumulate else 0, _lib.current_stream(out.device)))
+            _lib.ptr(out), _row_stride(out), feat, int(bits), 1 if accumulate else 0, _lib.current_stream(out.device)))
 
 
 def SPMM_forward_quantized(src: SparseTensor, packed: torch.Tensor, params: torch.Tensor, row_code: torch.Tensor,

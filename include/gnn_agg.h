@@ -285,10 +285,11 @@ int gnnagg_dequantize_segments_f32(const uint8_t *packed, const float *params, f
  * what gnnagg_dequantize_segments_f32 would have stored, so the result equals dequantise
  * followed by gnnagg_plan_spmm_f32 bit for bit, without the fp32 buffer ever being written
  * or read (the reference dequantises into recv_buf and then aggregates,
- * model/layers/aggregator.py:83-104).  feat % 4 == 0. */
+ * model/layers/aggregator.py:83-104).  feat % 4 == 0; row r of out starts at out + r * out_stride
+ * floats (out_stride % 4 == 0; feat for rows back to back). */
 int gnnagg_plan_spmm_quantized_f32(gnnagg_plan *plan, const float *value, const uint8_t *packed, const float *params,
-                                   const int32_t *row_code, float *out, int64_t feat, int bits, int accumulate,
-                                   void *stream);
+                                   const int32_t *row_code, float *out, int64_t out_stride, int64_t feat, int bits,
+                                   int accumulate, void *stream);
 int gnnagg_quantize_mixed_f32(const float *x, uint8_t *data, const int64_t *feat_range, float *params, int64_t rows,
                               int64_t feat, int32_t *bad_width, void *stream);
 int gnnagg_dequantize_mixed_f32(const uint8_t *data, const int64_t *feat_range, const float *params, float *out,

@@ -316,9 +316,9 @@ def test_sage_layer_single_rank_and_eval_mode():
         conv(graph, x.clone().requires_grad_(), 0)
 
 
-@pytest.mark.parametrize("num_bits", [32, 2])
+@pytest.mark.parametrize("num_bits,fuse", [(32, False), (2, False), (2, True)])
 @pytest.mark.parametrize("is_pre_delay", [True, False])
-def test_sage_layer_aggregates_like_the_aggregator(num_bits, is_pre_delay):
+def test_sage_layer_aggregates_like_the_aggregator(num_bits, fuse, is_pre_delay):
     """The layer runs the aggregation pipeline on halves of wider arrays; what lands in the left
     half must be bit for bit what ``Aggregator.apply`` returns for the same features (fp32 and
     int2 boundary rows), and the input gradient must match autograd through ``Aggregator``."""
@@ -328,6 +328,7 @@ def test_sage_layer_aggregates_like_the_aggregator(num_bits, is_pre_delay):
     graph = synthetic.build_partition_graph(part, f_in, is_pre_delay, exchange=synthetic.SeededHaloExchange(3),
                                             bits=num_bits, device=dev_,
                                             exchange_quantized=synthetic.SeededQuantizedHaloExchange(4))
+    graph.fuse_dequantize = fuse   # received rows aggregated straight from the packed bytes, into the strided half
     torch.manual_seed(2)
     conv = sage.DistSAGEConvGrad(f_in, f_out, num_bits, is_pre_delay).to(dev_)
     conv.train()
