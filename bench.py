@@ -34,9 +34,9 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak
 
 # HBM-side traffic of ONE forward launch of the headline workload (default arguments),
 # from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE:
-# FETCH_SIZE 27 768 073 KiB x 2.0 (the counter reads 0.5 KiB per KiB on a 1 GiB device copy)
-# + WRITE_SIZE 987 863 KiB x 1.0.  Keyed by (workload, nodes, mean out-degree, F, seed).
-MEASURED_TRAFFIC_BYTES = {("c2", 2_450_000, 25.0, 100, 0): (27_768_073 * 2.0 + 987_863) * 1024.0}
+# FETCH_SIZE 27 768 268 KiB x 2.0 (the counter reads 0.5 KiB per KiB on a 1 GiB device copy)
+# + WRITE_SIZE 987 837 KiB x 1.0.  Keyed by (workload, nodes, mean out-degree, F, seed).
+MEASURED_TRAFFIC_BYTES = {("c2", 2_450_000, 25.0, 100, 0): (27_768_268 * 2.0 + 987_837) * 1024.0}
 
 
 def b_alg(nnz: int, rows: int, feat: int) -> float:
