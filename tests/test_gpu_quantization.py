@@ -268,3 +268,55 @@ def test_quantised_aggregation_error_behaviour():
         SPMM_forward_quantized(adj, q.quantized_recv_data_buf, q.quantized_recv_params_buf_fp32, q.recv_row_code, out, 3)
     with pytest.raises(RuntimeError, match="Input mismatch"):
         SPMM_forward_quantized(adj, q.quantized_recv_data_buf, q.quantized_recv_params_buf_fp32[:4], q.recv_row_code, out, 2)
+
+
+@pytest.mark.parametrize("bits", [2, 4, 8])
+def test_reference_recipe_all_procs_against_per_segment_loop_and_torch(bits):
+    """The reference's own check (tests/test_quantization_ops.py:128-151, :217-235): 256 rows x 233
+    features cut into 256 random segments (most of them a row or two, many empty);
+    quantize_tensor_for_all_procs must give the bytes of quantize_tensor run segment by segment,
+    and the same values back.  For 8 and 4 bits it also compares with torch.quantize_per_channel
+    (:23-35, :156-158), which rounds x * (1/scale) + zero_point instead of (x - min) / scale: equal
+    but for ties and last-bit cases, so that comparison allows one step on a fraction of the values."""
+    from gnn_benchmark_amd import computation_ops as ops
+
+    num_nodes, feat_len, num_procs = 256, 233, 256
+    gen = torch.Generator().manual_seed(bits)
+    data = torch.randn((num_nodes, feat_len), generator=gen)
+    work_range = torch.randint(0, num_nodes, (num_procs + 1,), generator=gen, dtype=torch.int32).sort()[0]
+    work_range[0], work_range[-1] = 0, num_nodes
+    per = 8 // bits
+    sizes = [int(work_range[i + 1] - work_range[i]) for i in range(num_procs)]
+    packed_rows = sum(-(-s // per) for s in sizes)
+    x = data.cuda()
+
+    packed = torch.zeros((packed_rows, feat_len), dtype=torch.uint8, device="cuda")
+    params = torch.zeros((num_nodes, 2), device="cuda")
+    ops.quantize_tensor_for_all_procs(x, packed, params, work_range, num_procs, bits)
+
+    pieces, piece_params = [], []
+    for i, s in enumerate(sizes):
+        if s == 0:
+            continue
+        seg = x[int(work_range[i]):int(work_range[i + 1])].contiguous()
+        out = torch.zeros((-(-s // per), feat_len), dtype=torch.uint8, device="cuda")
+        prm = torch.zeros((s, 2), device="cuda")
+        ops.quantize_tensor(seg, out, prm, bits)
+        pieces.append(out)
+        piece_params.append(prm)
+    assert torch.equal(packed, torch.cat(pieces))
+    assert torch.equal(params, torch.cat(piece_params))
+
+    back = torch.zeros((num_nodes, feat_len), device="cuda")
+    ops.dequantize_tensor_for_all_procs(packed, back, params, work_range, num_procs, bits)
+    scale = params[:, 1:2]
+    assert bool(((back - x).abs() <= scale * 0.5 * (1 + 1e-5) + 1e-6).all())
+
+    if bits in (8, 4):
+        s_cpu = ((data.max(dim=1)[0] - data.min(dim=1)[0] + 10e-20) / (2 ** bits - 1))
+        zp_cpu = data.min(dim=1)[0] / s_cpu * (-1)
+        ref = torch.dequantize(torch.quantize_per_channel(data, s_cpu, zp_cpu, 0,
+                                                          torch.quint8 if bits == 8 else torch.quint4x2))
+        diff = (back.cpu() - ref).abs()
+        assert bool((diff <= s_cpu.view(-1, 1) * (1 + 1e-4) + 1e-6).all())
+        assert float((diff > 1e-6 + 1e-5 * ref.abs()).float().mean()) < 0.02
