@@ -113,29 +113,52 @@ hipError_t dispatch_shape(const Shape &s, const SpmmArgs &a, int rpg, hipStream_
 
 // The block-per-row kernel needs more than the default 64 KB of LDS per block; the limit
 // is a per-device attribute of each instantiation (set when a plan with such rows is made).
+template <int VEC, int NL>
+hipError_t allow_long_rows_lds() {
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(spmm_long_rows_kernel<VEC, NL>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLongSmemBytes);
+}
+
+template <int VEC>
+hipError_t allow_long_rows_lds_for_vec() {
+    hipError_t e = allow_long_rows_lds<VEC, 1>();
+    if (e == hipSuccess) e = allow_long_rows_lds<VEC, 2>();
+    if (e == hipSuccess) e = allow_long_rows_lds<VEC, 4>();
+    if (e == hipSuccess) e = allow_long_rows_lds<VEC, 8>();
+    return e;
+}
+
+// the block-per-row kernel uses more than 64 KB of dynamic LDS: every instance has to be told
 hipError_t enable_long_rows_lds() {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(spmm_long_rows_kernel<4>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLongSmemBytes);
-    if (e == hipSuccess)
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(spmm_long_rows_kernel<2>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLongSmemBytes);
-    if (e == hipSuccess)
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(spmm_long_rows_kernel<1>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLongSmemBytes);
+    hipError_t e = allow_long_rows_lds_for_vec<4>();
+    if (e == hipSuccess) e = allow_long_rows_lds_for_vec<2>();
+    if (e == hipSuccess) e = allow_long_rows_lds_for_vec<1>();
     return e;
 }
 
 template <int VEC>
 hipError_t launch_long_rows(const LongArgs &a, int64_t nrows, hipStream_t st) {
     LongArgs args = a;
-    const int tile = a.feat < kLongFeatTile ? a.feat : kLongFeatTile;
+    // What bounds a row is the rate at which ONE compute unit can fetch its dense rows, so with few
+    // such rows each is cut along the features into more blocks (each feature's chain is its own),
+    // down to 16 features = one 64-byte piece per stored element; a narrower tile also means a longer
+    // chunk (more stored elements per memory round trip).
+    int tile = kLongFeatTile;
+    while (tile > kLongMinFeatTile && nrows * ((a.feat + tile / 2 - 1) / (tile / 2)) <= 512) tile /= 2;
+    if (tile > a.feat) tile = a.feat;
+    args.tile = tile;
     const int vpr = tile / VEC;
     int chunk = kLongMaxChunk;
     if (chunk * vpr > 256 * kLongLoads) chunk = 256 * kLongLoads / vpr;
     if (chunk * tile > kLongTileFloats) chunk = kLongTileFloats / tile;
     args.chunk = chunk;
-    const unsigned tiles = (unsigned)((a.feat + kLongFeatTile - 1) / kLongFeatTile);
-    hipLaunchKernelGGL((spmm_long_rows_kernel<VEC>), dim3((unsigned)nrows, tiles), dim3(256), kLongSmemBytes, st, args);
+    const unsigned tiles = (unsigned)((a.feat + tile - 1) / tile);
+    const int slots = chunk * vpr;  // vectors of a whole chunk; 256 threads fetch them in NL rounds
+    const dim3 grid((unsigned)nrows, tiles);
+    if (slots <= 256) hipLaunchKernelGGL((spmm_long_rows_kernel<VEC, 1>), grid, dim3(256), kLongSmemBytes, st, args);
+    else if (slots <= 512) hipLaunchKernelGGL((spmm_long_rows_kernel<VEC, 2>), grid, dim3(256), kLongSmemBytes, st, args);
+    else if (slots <= 1024) hipLaunchKernelGGL((spmm_long_rows_kernel<VEC, 4>), grid, dim3(256), kLongSmemBytes, st, args);
+    else hipLaunchKernelGGL((spmm_long_rows_kernel<VEC, 8>), grid, dim3(256), kLongSmemBytes, st, args);
     return hipGetLastError();
 }
 
@@ -333,8 +356,9 @@ extern "C" int gnnagg_plan_create(const int64_t *rowptr, const int64_t *col, int
     p->long_thresh = env_int("GNNAGG_LONG_THRESH", 256, 1, 1 << 30);
     // A row is handed to the block-per-row kernel only when its chain, fed by one lane
     // group (a few elements per microsecond), would outlast the whole launch: that
-    // length grows with the matrix, about nnz / 4096 (measured on MI355X), floor 8192.
-    int64_t huge_default = std::max<int64_t>(8192, nnz / 4096);
+    // length grows with the matrix, about nnz / 4096 (measured on MI355X), floor 4096 (below it the
+    // block-per-row kernel, about 50 stored elements per microsecond and row, no longer pays).
+    int64_t huge_default = std::max<int64_t>(4096, nnz / 4096);
     if (huge_default > (1 << 30)) huge_default = 1 << 30;
     p->huge_thresh = env_int("GNNAGG_HUGE_THRESH", (int)huge_default, p->long_thresh, 1 << 30);
     p->rows_per_group = env_int("GNNAGG_ROWS_PER_GROUP", 4, 1, kMaxRowsPerGroup);

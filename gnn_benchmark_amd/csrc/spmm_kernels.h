@@ -452,20 +452,27 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
 
 
 // ---------------------------------------------------------------------------------------
-// Very long rows.  One 256-thread block per (row, feature tile of <= 256 floats).  The
+// Very long rows.  One 256-thread block per (row, feature tile of 16 .. 256 floats).  The
 // row's chain must stay sequential (bit-identical results), so what is parallelised is the
-// FETCH: all four waves gather a chunk of up to 64 dense rows into LDS at once (up to
-// 8 vector loads in flight per thread, 32 KB per block), while the threads that own a
-// feature each run the FMA chain over the previous chunk out of LDS, in CSR order.
-// Chunks are double-buffered; the (col, val) pairs run two chunks ahead.
+// FETCH: all four waves gather a chunk of dense rows at once (up to 8 vector loads per thread
+// and chunk), while the threads that own a feature each run the FMA chain over an earlier
+// chunk out of LDS, in CSR order.  A row advances by one chunk per memory round trip, so the
+// chunk is made as long as a 32 KB tile buffer allows -- 32 rows of 256 floats, 512 rows of
+// 16 -- and with few such rows the host cuts them into narrow feature tiles (every feature's
+// chain is its own), which also spreads one row's fetch over several compute units.
+// kLongDepth chunks are in flight in registers; the (col, val) pairs come in super-chunks of
+// kLongDepth chunks, two super-chunks ahead.
 // ---------------------------------------------------------------------------------------
 constexpr int kLongTileFloats = 8192;  // floats per LDS tile buffer (32 KB), two buffers
-constexpr int kLongMaxChunk = 64;      // dense rows gathered per chunk
-constexpr int kLongLoads = 8;          // vector loads in flight per thread
-constexpr int kLongFeatTile = 256;     // features per block
-// dynamic LDS: two tile buffers, then three (col, val) chunk buffers
+constexpr int kLongMaxChunk = 512;     // most dense rows gathered per chunk
+constexpr int kLongLoads = 8;          // most vector loads per thread and chunk
+constexpr int kLongDepth = 2;          // chunks in flight
+constexpr int kLongFeatTile = 256;     // most features per block
+constexpr int kLongMinFeatTile = 16;   // fewest: one 64-byte piece of every gathered row
+constexpr int kLongPairs = kLongDepth * kLongMaxChunk / 256;  // (col, val) pairs per thread and super-chunk
+// dynamic LDS: two tile buffers, then three (col, val) super-chunk buffers
 constexpr size_t kLongSmemBytes =
-    2 * kLongTileFloats * sizeof(float) + 3 * kLongMaxChunk * (sizeof(int) + sizeof(float));
+    2 * kLongTileFloats * sizeof(float) + 3 * kLongDepth * kLongMaxChunk * (sizeof(int) + sizeof(float));
 
 struct LongArgs {
     const RowTask *task;  // rows handled: task[0 .. gridDim.x)
@@ -475,100 +482,155 @@ struct LongArgs {
     float *dst;
     int feat;        // F
     int ldx, ldd;    // row strides of x and dst in floats; 0 stands for F
+    int tile;        // features per block (a multiple of VEC, <= kLongFeatTile)
     int chunk;       // dense rows per chunk: chunk * min(F, 256) <= kLongTileFloats, chunk * (tile / VEC) <= 2048
     int accumulate;
 };
 
-template <int VEC>
+// The chain over one whole chunk of CC stored elements for the feature a thread owns: the CC values of
+// its column are requested from LDS back to back (independent reads, fully pipelined) and the CC matrix
+// values come in with ONE read per lane and are handed to the whole wave lane by lane (v_readlane, so the
+// multiplier of every FMA is a scalar); what remains sequential is the FMA chain itself.
+template <int CC>
+__device__ __forceinline__ float chain_whole_chunk(const float *tb, const float *vb, int fw, float acc) {
+    static_assert(CC <= 64, "one matrix value per lane");
+    float xs[CC];
+#pragma unroll
+    for (int j = 0; j < CC; ++j) xs[j] = tb[j * fw];
+    const int lane = (int)__lane_id();
+    const int vl = __float_as_int(vb[lane < CC ? lane : 0]);
+#pragma unroll
+    for (int j = 0; j < CC; ++j) acc = __builtin_fmaf(__int_as_float(__builtin_amdgcn_readlane(vl, j)), xs[j], acc);
+    return acc;
+}
+
+// NL: vector loads per thread and chunk, the smallest of 1, 2, 4, 8 with NL * 256 >= chunk * (tile / VEC).
+template <int VEC, int NL>
 __global__ __launch_bounds__(256) void spmm_long_rows_kernel(const LongArgs a) {
     typedef FVec<VEC> V;
+    constexpr int D = kLongDepth;
+    constexpr int kSuper = D * kLongMaxChunk;  // index pairs per super-chunk buffer
     extern __shared__ __attribute__((aligned(16))) unsigned char long_smem[];
     float(*tile)[kLongTileFloats] = reinterpret_cast<float(*)[kLongTileFloats]>(long_smem);
-    int(*s_col)[kLongMaxChunk] =
-        reinterpret_cast<int(*)[kLongMaxChunk]>(long_smem + 2 * kLongTileFloats * sizeof(float));
-    float(*s_val)[kLongMaxChunk] = reinterpret_cast<float(*)[kLongMaxChunk]>(
-        long_smem + 2 * kLongTileFloats * sizeof(float) + 3 * kLongMaxChunk * sizeof(int));
+    int(*s_col)[kSuper] = reinterpret_cast<int(*)[kSuper]>(long_smem + 2 * kLongTileFloats * sizeof(float));
+    float(*s_val)[kSuper] = reinterpret_cast<float(*)[kSuper]>(long_smem + 2 * kLongTileFloats * sizeof(float) +
+                                                               3 * kSuper * sizeof(int));
 
     const int t = (int)threadIdx.x;
     const RowTask d = a.task[blockIdx.x];
     const int F = a.feat;
     const int ldx = a.ldx ? a.ldx : F;
-    const int f0 = (int)blockIdx.y * kLongFeatTile;
-    const int fw = F - f0 < kLongFeatTile ? F - f0 : kLongFeatTile;  // width of this tile (multiple of VEC)
+    const int f0 = (int)blockIdx.y * a.tile;
+    const int fw = F - f0 < a.tile ? F - f0 : a.tile;                // width of this tile (multiple of VEC)
     const int vpr = fw / VEC;                                        // vectors per gathered row
     const int C = a.chunk;
+    const int SC = D * C;                                            // stored elements per super-chunk
     const int nchunks = (d.len + C - 1) / C;
     const float *__restrict__ x = a.x + f0;
     const int32_t *__restrict__ col = a.col + d.start;
     const float *__restrict__ val = a.val + d.start;
 
-    // fixed (dense row in chunk, vector in row) slots of this thread
-    int sj[kLongLoads], sv[kLongLoads];
+    // fixed (dense row in chunk, vector in row) slots of this thread; slot e lands at float e * VEC of a
+    // tile buffer (= row e / vpr, vector e % vpr), always inside the buffer
+    int sj[NL], sv[NL];
 #pragma unroll
-    for (int s = 0; s < kLongLoads; ++s) {
+    for (int s = 0; s < NL; ++s) {
         const int e = t + s * 256;
         sj[s] = e / vpr;
         sv[s] = (e - sj[s] * vpr) * VEC;
     }
 
     auto chunk_len = [&](int k) { const int left = d.len - k * C; return left < C ? left : C; };
-
-    // prologue: indices of chunks 0 and 1, dense rows of chunk 0
-    if (t < C) {
-        if (t < chunk_len(0)) { s_col[0][t] = __builtin_nontemporal_load(col + t); s_val[0][t] = __builtin_nontemporal_load(val + t); }
-        if (nchunks > 1 && t < chunk_len(1)) { s_col[1][t] = __builtin_nontemporal_load(col + C + t); s_val[1][t] = __builtin_nontemporal_load(val + C + t); }
-    }
-    __syncthreads();
-    {
-        const int cnt = chunk_len(0);
+    // chunk k sits in super-chunk k / D (buffer (k / D) % 3) at offset (k % D) * C.  Every slot loads and
+    // lands, whatever the chunk holds (a slot past the chunk's last row repeats that row and lands where
+    // nobody reads): loads under a branch would make every later wait a wait for ALL loads in flight.
+    auto request = [&](int k, V(&g)[NL]) {
+        const int last = chunk_len(k) - 1;
+        const int *cb = &s_col[(k / D) % 3][(k % D) * C];
 #pragma unroll
-        for (int s = 0; s < kLongLoads; ++s) {
-            if (sj[s] < cnt) {
-                const V v = V::load(x + (size_t)s_col[0][sj[s]] * (size_t)ldx + sv[s]);
-                v.store(&tile[0][sj[s] * fw + sv[s]]);
-            }
+        for (int s = 0; s < NL; ++s) {
+            const int j = sj[s] < last ? sj[s] : last;
+            g[s] = V::load(x + (size_t)cb[j] * (size_t)ldx + sv[s]);
+        }
+    };
+    auto land = [&](int k, const V(&g)[NL]) {
+#pragma unroll
+        for (int s = 0; s < NL; ++s) g[s].store(&tile[k & 1][(t + s * 256) * VEC]);
+    };
+
+    // prologue: index pairs of super-chunks 0 and 1, dense rows of chunks 0 .. D-1, chunk 0 landed
+#pragma unroll
+    for (int p = 0; p < kLongPairs; ++p) {
+        const int e = t + p * 256;
+        if (e < SC && e < d.len) {
+            s_col[0][e] = __builtin_nontemporal_load(col + e);
+            s_val[0][e] = __builtin_nontemporal_load(val + e);
+        }
+        if (e < SC && SC + e < d.len) {
+            s_col[1][e] = __builtin_nontemporal_load(col + SC + e);
+            s_val[1][e] = __builtin_nontemporal_load(val + SC + e);
         }
     }
+    __syncthreads();
+    V g[D][NL];
+#pragma unroll
+    for (int u = 0; u < D; ++u) request(u < nchunks ? u : nchunks - 1, g[u]);
+    land(0, g[0]);
     __syncthreads();
 
     float *dst = a.dst + (size_t)d.row * (size_t)(a.ldd ? a.ldd : F) + f0;
     float acc = 0.0f;
     const bool own = t < fw;
+    const bool wave_owns = (t & ~63) < fw;  // the same for the 64 lanes of a wave
     if (own && a.accumulate) acc = __builtin_nontemporal_load(dst + t);
 
-    for (int k = 0; k < nchunks; ++k) {
-        const int cnt = chunk_len(k);
-        const int ncnt = k + 1 < nchunks ? chunk_len(k + 1) : 0;
-        // (1) request the dense rows of chunk k+1 and the indices of chunk k+2
-        V g[kLongLoads];
+    for (int kb = 0; kb < nchunks; kb += D) {
+        // index pairs of the super-chunk after the next one: requested now, stored at the end
+        const int super = kb / D;
+        const int64_t base2 = (int64_t)(super + 2) * SC;
+        int ci[kLongPairs];
+        float vi[kLongPairs];
 #pragma unroll
-        for (int s = 0; s < kLongLoads; ++s) {
-            if (sj[s] < ncnt) g[s] = V::load(x + (size_t)s_col[(k + 1) % 3][sj[s]] * (size_t)ldx + sv[s]);
+        for (int p = 0; p < kLongPairs; ++p) {
+            // past the super-chunk or the row: the row's last pair once more, stored where nobody reads
+            int64_t e2 = base2 + t + p * 256;
+            if (e2 > d.len - 1) e2 = d.len - 1;
+            ci[p] = __builtin_nontemporal_load(col + e2);
+            vi[p] = __builtin_nontemporal_load(val + e2);
         }
-        int ci = 0;
-        float vi = 0.0f;
-        const bool idx2 = k + 2 < nchunks && t < chunk_len(k + 2);
-        if (idx2) {
-            ci = __builtin_nontemporal_load(col + (size_t)(k + 2) * C + t);
-            vi = __builtin_nontemporal_load(val + (size_t)(k + 2) * C + t);
-        }
-        // (2) the chain over chunk k, in CSR order, out of LDS
-        if (own) {
-            const float *tb = &tile[k & 1][t];
-            const float *vb = s_val[k % 3];
+#pragma unroll
+        for (int u = 0; u < D; ++u) {
+            const int k = kb + u;
+            if (k >= nchunks) break;  // the same for every thread of the block
+            // (1) chunk k left its registers for LDS in the step before: request chunk k + D into them
+            //     (past the row's end: the last chunk once more, never landed where it is read)
+            request(k + D < nchunks ? k + D : nchunks - 1, g[u]);
+            // (2) the chain over chunk k, in CSR order, out of LDS (whole waves take part: a lane past the
+            //     tile's width computes a value nobody stores)
+            if (wave_owns) {
+                const int cnt = chunk_len(k);
+                const float *tb = &tile[k & 1][t];
+                const float *vb = &s_val[super % 3][u * C];
+                int j = 0;
+                for (; j + 64 <= cnt; j += 64) acc = chain_whole_chunk<64>(tb + j * fw, vb + j, fw, acc);
+                if (j + 32 <= cnt) {
+                    acc = chain_whole_chunk<32>(tb + j * fw, vb + j, fw, acc);
+                    j += 32;
+                }
 #pragma unroll 8
-            for (int j = 0; j < cnt; ++j) acc = __builtin_fmaf(vb[j], tb[j * fw], acc);
-        }
-        // (3) land what was requested in (1)
+                for (; j < cnt; ++j) acc = __builtin_fmaf(vb[j], tb[j * fw], acc);
+            }
+            // (3) land chunk k + 1 (requested D - 1 steps ago) in the other tile buffer
+            land(k + 1, g[(u + 1) % D]);
+            if (u == D - 1) {
 #pragma unroll
-        for (int s = 0; s < kLongLoads; ++s) {
-            if (sj[s] < ncnt) g[s].store(&tile[(k + 1) & 1][sj[s] * fw + sv[s]]);
+                for (int p = 0; p < kLongPairs; ++p) {
+                    s_col[(super + 2) % 3][t + p * 256] = ci[p];
+                    s_val[(super + 2) % 3][t + p * 256] = vi[p];
+                }
+            }
+            __syncthreads();
         }
-        if (idx2) {
-            s_col[(k + 2) % 3][t] = ci;
-            s_val[(k + 2) % 3][t] = vi;
-        }
-        __syncthreads();
     }
     if (own) __builtin_nontemporal_store(acc, dst + t);
 }

@@ -20,7 +20,7 @@ pytestmark = pytest.mark.gpu
 def low_block_row_threshold(monkeypatch):
     """Plans read this when they are created: rows longer than 2048 elements then go to
     the block-per-row kernel, which by default only takes rows that would outlast the
-    whole launch (about nnz / 4096 elements, at least 8192)."""
+    whole launch (about nnz / 4096 elements, at least 4096)."""
     monkeypatch.setenv("GNNAGG_HUGE_THRESH", "2048")
 
 EMPTY_I32 = torch.empty(0, dtype=torch.int32)
@@ -80,7 +80,7 @@ def test_plan_path_with_long_rows_and_empty_rows(feat, accumulate, low_block_row
     info = plan.info()
     deg = np.diff(rowptr)
     assert info["huge_rows"] == int((deg > info["huge_thresh"]).sum()) == 1
-    assert info["max_row_len"] == 5000 and info["empty_rows"] == int((deg == 0).sum()) > 100
+    assert info["max_row_len"] == 4000 and info["empty_rows"] == int((deg == 0).sum()) > 100
     out = dev(out0)
     plan.spmm(dev(val), dev(x), out, accumulate=accumulate)
     want = _oracle(rowptr, col, val, x, out0 if accumulate else None)
@@ -113,9 +113,9 @@ def test_block_per_row_kernel_chunk_edges(feat, low_block_row_threshold):
 
 
 def test_default_threshold_keeps_moderate_rows_in_the_lane_group_kernel():
-    rowptr, col, val = skewed_csr(900, 450, seed=3)  # longest row 5000 < 8192
+    rowptr, col, val = skewed_csr(900, 450, seed=3)  # longest row 4000 < 4096
     plan = SpmmPlan(dev(rowptr), dev(col), 900, 450)
-    assert plan.info()["huge_rows"] == 0 and plan.info()["huge_thresh"] == 8192
+    assert plan.info()["huge_rows"] == 0 and plan.info()["huge_thresh"] == 4096
     x = np.random.default_rng(3).standard_normal((450, 128)).astype(np.float32)
     out = torch.zeros(900, 128, device="cuda")
     plan.spmm(dev(val), dev(x), out)
@@ -447,3 +447,26 @@ def test_dense_operands_beyond_2_to_31_floats():
         hi = min(n, lo + 1_500_000)
         assert torch.equal(out[lo:hi], val[lo:hi, None] * x[perm[lo:hi]]), lo
     assert torch.equal(out[-1], val[-1] * x[-1])
+
+
+@pytest.mark.parametrize("long_rows,feat", [(320, 256), (320, 100), (320, 8), (40, 256), (40, 602), (40, 130), (3, 1030)])
+def test_many_rows_in_the_block_per_row_kernel(long_rows, feat, low_block_row_threshold):
+    """The block-per-row kernel cuts its rows into feature tiles, narrower the fewer rows there are
+    (16 .. 256 features, chunks of 512 .. 32 dense rows): many, some and few long rows at widths that
+    are, and are not, multiples of the tile and of the vector width, against the oracle bit for bit."""
+    rng = np.random.default_rng(long_rows * 1000 + feat)
+    rows, cols = long_rows + 500, 700
+    deg = rng.poisson(3, rows)
+    deg[rng.choice(rows, long_rows, replace=False)] = rng.integers(2049, 2400, long_rows)
+    rowptr = np.concatenate(([0], np.cumsum(deg))).astype(np.int64)
+    col = rng.integers(0, cols, int(rowptr[-1])).astype(np.int64)
+    val = rng.standard_normal(int(rowptr[-1])).astype(np.float32)
+    x = rng.standard_normal((cols, feat)).astype(np.float32)
+    out0 = rng.standard_normal((rows, feat)).astype(np.float32)
+    plan = SpmmPlan(dev(rowptr), dev(col), rows, cols)
+    assert plan.info()["huge_rows"] == long_rows
+    for accumulate in (True, False):
+        out = dev(out0)
+        plan.spmm(dev(val), dev(x), out, accumulate=accumulate)
+        want = _oracle(rowptr, col, val, x, out0 if accumulate else None)
+        assert np.array_equal(out.cpu().numpy(), want), accumulate
