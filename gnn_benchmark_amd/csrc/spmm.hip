@@ -128,11 +128,22 @@ hipError_t allow_long_rows_lds_for_vec() {
     return e;
 }
 
+template <int FW>
+hipError_t allow_long_rows_lds_fixed_width() {
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(spmm_long_rows_kernel<4, 8, FW>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLongSmemBytes);
+}
+
 // the block-per-row kernel uses more than 64 KB of dynamic LDS: every instance has to be told
 hipError_t enable_long_rows_lds() {
     hipError_t e = allow_long_rows_lds_for_vec<4>();
     if (e == hipSuccess) e = allow_long_rows_lds_for_vec<2>();
     if (e == hipSuccess) e = allow_long_rows_lds_for_vec<1>();
+    if (e == hipSuccess) e = allow_long_rows_lds_fixed_width<16>();
+    if (e == hipSuccess) e = allow_long_rows_lds_fixed_width<32>();
+    if (e == hipSuccess) e = allow_long_rows_lds_fixed_width<64>();
+    if (e == hipSuccess) e = allow_long_rows_lds_fixed_width<128>();
+    if (e == hipSuccess) e = allow_long_rows_lds_fixed_width<256>();
     return e;
 }
 
@@ -155,6 +166,19 @@ hipError_t launch_long_rows(const LongArgs &a, int64_t nrows, hipStream_t st) {
     const unsigned tiles = (unsigned)((a.feat + tile - 1) / tile);
     const int slots = chunk * vpr;  // vectors of a whole chunk; 256 threads fetch them in NL rounds
     const dim3 grid((unsigned)nrows, tiles);
+    if (VEC == 4 && slots > 1024 && a.feat % tile == 0 && tile >= 16 && (tile & (tile - 1)) == 0) {
+        // every tile has the same power-of-two width: the instance that knows it at compile time
+#define GNNAGG_LONG_FIXED(W)                                                                                     \
+    if (tile == W)                                                                                               \
+        hipLaunchKernelGGL((spmm_long_rows_kernel<4, 8, W>), grid, dim3(256), kLongSmemBytes, st, args)
+        GNNAGG_LONG_FIXED(16);
+        GNNAGG_LONG_FIXED(32);
+        GNNAGG_LONG_FIXED(64);
+        GNNAGG_LONG_FIXED(128);
+        GNNAGG_LONG_FIXED(256);
+#undef GNNAGG_LONG_FIXED
+        return hipGetLastError();
+    }
     if (slots <= 256) hipLaunchKernelGGL((spmm_long_rows_kernel<VEC, 1>), grid, dim3(256), kLongSmemBytes, st, args);
     else if (slots <= 512) hipLaunchKernelGGL((spmm_long_rows_kernel<VEC, 2>), grid, dim3(256), kLongSmemBytes, st, args);
     else if (slots <= 1024) hipLaunchKernelGGL((spmm_long_rows_kernel<VEC, 4>), grid, dim3(256), kLongSmemBytes, st, args);
@@ -356,9 +380,9 @@ extern "C" int gnnagg_plan_create(const int64_t *rowptr, const int64_t *col, int
     p->long_thresh = env_int("GNNAGG_LONG_THRESH", 256, 1, 1 << 30);
     // A row is handed to the block-per-row kernel only when its chain, fed by one lane
     // group (a few elements per microsecond), would outlast the whole launch: that
-    // length grows with the matrix, about nnz / 4096 (measured on MI355X), floor 4096 (below it the
-    // block-per-row kernel, about 50 stored elements per microsecond and row, no longer pays).
-    int64_t huge_default = std::max<int64_t>(4096, nnz / 4096);
+    // length grows with the matrix, about nnz / 4096 (measured on MI355X), floor 2048 (below it the
+    // block-per-row kernel, 50 .. 85 stored elements per microsecond and row, no longer pays).
+    int64_t huge_default = std::max<int64_t>(2048, nnz / 4096);
     if (huge_default > (1 << 30)) huge_default = 1 << 30;
     p->huge_thresh = env_int("GNNAGG_HUGE_THRESH", (int)huge_default, p->long_thresh, 1 << 30);
     p->rows_per_group = env_int("GNNAGG_ROWS_PER_GROUP", 4, 1, kMaxRowsPerGroup);

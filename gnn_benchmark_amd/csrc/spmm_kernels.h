@@ -491,12 +491,13 @@ struct LongArgs {
 // its column are requested from LDS back to back (independent reads, fully pipelined) and the CC matrix
 // values come in with ONE read per lane and are handed to the whole wave lane by lane (v_readlane, so the
 // multiplier of every FMA is a scalar); what remains sequential is the FMA chain itself.
-template <int CC>
+// FW: the tile's width when the host knows it (the LDS offsets are then immediates), 0: take `fw`.
+template <int CC, int FW>
 __device__ __forceinline__ float chain_whole_chunk(const float *tb, const float *vb, int fw, float acc) {
     static_assert(CC <= 64, "one matrix value per lane");
     float xs[CC];
 #pragma unroll
-    for (int j = 0; j < CC; ++j) xs[j] = tb[j * fw];
+    for (int j = 0; j < CC; ++j) xs[j] = tb[j * (FW ? FW : fw)];
     const int lane = (int)__lane_id();
     const int vl = __float_as_int(vb[lane < CC ? lane : 0]);
 #pragma unroll
@@ -505,7 +506,8 @@ __device__ __forceinline__ float chain_whole_chunk(const float *tb, const float 
 }
 
 // NL: vector loads per thread and chunk, the smallest of 1, 2, 4, 8 with NL * 256 >= chunk * (tile / VEC).
-template <int VEC, int NL>
+// FW: the width of EVERY tile of the launch when that is one of 16 .. 256 and divides F, else 0.
+template <int VEC, int NL, int FW = 0>
 __global__ __launch_bounds__(256) void spmm_long_rows_kernel(const LongArgs a) {
     typedef FVec<VEC> V;
     constexpr int D = kLongDepth;
@@ -521,7 +523,7 @@ __global__ __launch_bounds__(256) void spmm_long_rows_kernel(const LongArgs a) {
     const int F = a.feat;
     const int ldx = a.ldx ? a.ldx : F;
     const int f0 = (int)blockIdx.y * a.tile;
-    const int fw = F - f0 < a.tile ? F - f0 : a.tile;                // width of this tile (multiple of VEC)
+    const int fw = FW ? FW : (F - f0 < a.tile ? F - f0 : a.tile);    // width of this tile (multiple of VEC)
     const int vpr = fw / VEC;                                        // vectors per gathered row
     const int C = a.chunk;
     const int SC = D * C;                                            // stored elements per super-chunk
@@ -612,9 +614,9 @@ __global__ __launch_bounds__(256) void spmm_long_rows_kernel(const LongArgs a) {
                 const float *tb = &tile[k & 1][t];
                 const float *vb = &s_val[super % 3][u * C];
                 int j = 0;
-                for (; j + 64 <= cnt; j += 64) acc = chain_whole_chunk<64>(tb + j * fw, vb + j, fw, acc);
+                for (; j + 64 <= cnt; j += 64) acc = chain_whole_chunk<64, FW>(tb + j * fw, vb + j, fw, acc);
                 if (j + 32 <= cnt) {
-                    acc = chain_whole_chunk<32>(tb + j * fw, vb + j, fw, acc);
+                    acc = chain_whole_chunk<32, FW>(tb + j * fw, vb + j, fw, acc);
                     j += 32;
                 }
 #pragma unroll 8

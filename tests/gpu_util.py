@@ -30,7 +30,7 @@ def random_csr(rows, cols, density, seed, dtype=np.float32):
     return a
 
 
-def skewed_csr(rows, cols, seed, heavy_rows=(4000, 1300, 700), mean_deg=6, empty_every=7):
+def skewed_csr(rows, cols, seed, heavy_rows=(2000, 900, 700), mean_deg=6, empty_every=7):
     """Ragged test matrix: a few very long rows, many short ones, some empty ones,
     repeated column indices allowed (as the reference's CSR build keeps them)."""
     rng = np.random.default_rng(seed)

@@ -56,7 +56,7 @@ def test_packing_epilogue_equals_dense_epilogue(rows, feat, with_mask):
 @pytest.mark.parametrize("feat", [32, 64, 128, 256])
 @pytest.mark.parametrize("accumulate", [True, False])
 def test_packed_spmm_equals_dense_spmm(feat, accumulate, low_block_row_threshold):
-    rowptr, col, val = skewed_csr(900, 450, seed=300 + feat)          # rows of 4000 / 1300 / 700, empty rows
+    rowptr, col, val = skewed_csr(900, 450, seed=300 + feat)          # rows of 2000 / 900 / 700, empty rows
     src = SparseTensor(rowptr=dev(rowptr), col=dev(col), value=dev(val), sparse_sizes=(900, 450), is_sorted=True)
     z, bias, keep, div = _epilogue_inputs(450, feat, 11 + feat)
     dense = gcn._BiasReluDropout.apply(z.clone(), bias, keep, 2.0, div)

@@ -28,7 +28,7 @@ def _degrees(rng, rows):
         deg = rng.poisson(rng.uniform(0.2, 12), rows)
     elif kind == 1:
         deg = (rng.pareto(1.2, rows) * 3).astype(np.int64)
-    elif kind == 2:  # one very long row (block-per-row kernel above 4096)
+    elif kind == 2:  # one very long row (block-per-row kernel above 2048)
         deg = rng.poisson(2, rows)
         deg[rng.integers(0, rows)] = int(rng.choice([300, 2000, 9000, 20000]))
     else:            # mostly empty

@@ -31,8 +31,8 @@ pytestmark = pytest.mark.gpu
 @pytest.mark.parametrize("with_block_rows", [False, True])
 def test_spmm_on_column_blocks_equals_contiguous(feat, with_block_rows, monkeypatch):
     if with_block_rows:
-        monkeypatch.setenv("GNNAGG_HUGE_THRESH", "2048")
-    rowptr, col, val = skewed_csr(900, 900, seed=feat, heavy_rows=(4000, 2500, 300))
+        monkeypatch.setenv("GNNAGG_HUGE_THRESH", "1024")
+    rowptr, col, val = skewed_csr(900, 900, seed=feat, heavy_rows=(2000, 1500, 300))
     src = SparseTensor(rowptr=dev(rowptr), col=dev(col), value=dev(val), sparse_sizes=(900, 900))
     assert (src.get_plan().info()["huge_rows"] > 0) == with_block_rows
     gen = torch.Generator(device="cuda").manual_seed(feat)

@@ -18,10 +18,10 @@ pytestmark = pytest.mark.gpu
 
 @pytest.fixture
 def low_block_row_threshold(monkeypatch):
-    """Plans read this when they are created: rows longer than 2048 elements then go to
+    """Plans read this when they are created: rows longer than 1024 elements then go to
     the block-per-row kernel, which by default only takes rows that would outlast the
-    whole launch (about nnz / 4096 elements, at least 4096)."""
-    monkeypatch.setenv("GNNAGG_HUGE_THRESH", "2048")
+    whole launch (about nnz / 4096 elements, at least 2048)."""
+    monkeypatch.setenv("GNNAGG_HUGE_THRESH", "1024")
 
 EMPTY_I32 = torch.empty(0, dtype=torch.int32)
 
@@ -80,7 +80,7 @@ def test_plan_path_with_long_rows_and_empty_rows(feat, accumulate, low_block_row
     info = plan.info()
     deg = np.diff(rowptr)
     assert info["huge_rows"] == int((deg > info["huge_thresh"]).sum()) == 1
-    assert info["max_row_len"] == 4000 and info["empty_rows"] == int((deg == 0).sum()) > 100
+    assert info["max_row_len"] == 2000 and info["empty_rows"] == int((deg == 0).sum()) > 100
     out = dev(out0)
     plan.spmm(dev(val), dev(x), out, accumulate=accumulate)
     want = _oracle(rowptr, col, val, x, out0 if accumulate else None)
@@ -113,9 +113,9 @@ def test_block_per_row_kernel_chunk_edges(feat, low_block_row_threshold):
 
 
 def test_default_threshold_keeps_moderate_rows_in_the_lane_group_kernel():
-    rowptr, col, val = skewed_csr(900, 450, seed=3)  # longest row 4000 < 4096
+    rowptr, col, val = skewed_csr(900, 450, seed=3)  # longest row 2000 < 2048
     plan = SpmmPlan(dev(rowptr), dev(col), 900, 450)
-    assert plan.info()["huge_rows"] == 0 and plan.info()["huge_thresh"] == 4096
+    assert plan.info()["huge_rows"] == 0 and plan.info()["huge_thresh"] == 2048
     x = np.random.default_rng(3).standard_normal((450, 128)).astype(np.float32)
     out = torch.zeros(900, 128, device="cuda")
     plan.spmm(dev(val), dev(x), out)
@@ -370,7 +370,7 @@ def test_plan_spmm_can_be_captured_in_a_hip_graph(monkeypatch, with_block_rows):
     """The plan call allocates nothing and never synchronises the host, so it can be
     recorded into a graph; every replay (with fresh operand contents) must equal eager."""
     if with_block_rows:
-        monkeypatch.setenv("GNNAGG_HUGE_THRESH", "2048")
+        monkeypatch.setenv("GNNAGG_HUGE_THRESH", "1024")
     rowptr, col, val = skewed_csr(900, 450, seed=41)
     plan = SpmmPlan(dev(rowptr), dev(col), 900, 450)
     assert (plan.info()["huge_rows"] > 0) == with_block_rows
@@ -457,7 +457,7 @@ def test_many_rows_in_the_block_per_row_kernel(long_rows, feat, low_block_row_th
     rng = np.random.default_rng(long_rows * 1000 + feat)
     rows, cols = long_rows + 500, 700
     deg = rng.poisson(3, rows)
-    deg[rng.choice(rows, long_rows, replace=False)] = rng.integers(2049, 2400, long_rows)
+    deg[rng.choice(rows, long_rows, replace=False)] = rng.integers(1025, 1400, long_rows)
     rowptr = np.concatenate(([0], np.cumsum(deg))).astype(np.int64)
     col = rng.integers(0, cols, int(rowptr[-1])).astype(np.int64)
     val = rng.standard_normal(int(rowptr[-1])).astype(np.float32)
