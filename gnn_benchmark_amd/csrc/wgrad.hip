@@ -148,13 +148,27 @@ __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__re
         }
 }
 
+// out[i] = sum over the slices of partial[slice][i], in a fixed order: eight threads share an output,
+// thread s adds the slices s, s + 8, ... and the eight sums are added in order of s.  (A block covers 32
+// outputs, so that even a 128 x 128 result is spread over 512 blocks.)
+constexpr int kReduceOutputs = 32;
 __global__ __launch_bounds__(256) void wgrad_reduce_kernel(const float *__restrict__ partial, float *__restrict__ out,
                                                            int blocks, int count) {
-    const int i = (int)blockIdx.x * 256 + (int)threadIdx.x;
-    if (i >= count) return;
-    float s = 0.0f;
-    for (int b = 0; b < blocks; ++b) s += partial[(size_t)b * count + i];
-    out[i] = s;
+    __shared__ float part[8][kReduceOutputs];
+    const int o = (int)threadIdx.x & (kReduceOutputs - 1);
+    const int s = (int)threadIdx.x / kReduceOutputs;
+    const int i = (int)blockIdx.x * kReduceOutputs + o;
+    float acc = 0.0f;
+    if (i < count)
+        for (int b = s; b < blocks; b += 8) acc += partial[(size_t)b * count + i];
+    part[s][o] = acc;
+    __syncthreads();
+    if (s == 0 && i < count) {
+        float total = part[0][o];
+#pragma unroll
+        for (int k = 1; k < 8; ++k) total += part[k][o];
+        out[i] = total;
+    }
 }
 
 int wgrad_blocks(int64_t rows) {
@@ -192,7 +206,7 @@ extern "C" int gnnagg_wgrad_strided_f32(const float *x, int64_t x_stride, const 
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (rows == 0) {  // empty sum: the reduce kernel over zero partials writes zeros
         const int count0 = (int)(fi * fo);
-        hipLaunchKernelGGL(wgrad_reduce_kernel, dim3((unsigned)((count0 + 255) / 256)), dim3(256), 0, st,
+        hipLaunchKernelGGL(wgrad_reduce_kernel, dim3((unsigned)((count0 + kReduceOutputs - 1) / kReduceOutputs)), dim3(256), 0, st,
                            static_cast<const float *>(nullptr), w_grad, 0, count0);
         GNNAGG_HIP(hipGetLastError());
         return GNNAGG_OK;
@@ -223,7 +237,7 @@ extern "C" int gnnagg_wgrad_strided_f32(const float *x, int64_t x_stride, const 
 #undef GNNAGG_WGRAD
     GNNAGG_HIP(hipGetLastError());
     const int count = (int)(fi * fo);
-    hipLaunchKernelGGL(wgrad_reduce_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, st, partial, w_grad,
+    hipLaunchKernelGGL(wgrad_reduce_kernel, dim3((unsigned)((count + kReduceOutputs - 1) / kReduceOutputs)), dim3(256), 0, st, partial, w_grad,
                        blocks, count);
     GNNAGG_HIP(hipGetLastError());
     return GNNAGG_OK;
