@@ -593,11 +593,15 @@ def run_c5(args, graph):
     # the two GEMM variants with dense hidden activations, then the same with the hidden activations
     # kept packed (non-zero values + bitmap), which the next layer's aggregation gathers instead,
     # then with the narrowing last layer multiplying before it aggregates (A (x W) instead of (A x) W)
-    for gemm, packed_activations, linear_first in (("fp32", False, False), ("bf16", False, False), ("fp32", True, False),
-                                                   ("bf16", True, False), ("fp32", True, True), ("bf16", True, True)):
+    # (fp32 layers with dense activations run as one libgnnagg kernel each way; "separate_kernels" is the
+    # same model with the BLAS product and the elementwise passes apart)
+    for gemm, packed_activations, linear_first, fused in (
+            ("fp32", False, False, True), ("fp32", False, False, False), ("bf16", False, False, True),
+            ("fp32", True, False, True), ("bf16", True, False, True), ("fp32", False, True, True),
+            ("fp32", True, True, True), ("bf16", True, True, True)):
         torch.manual_seed(args.seed)
         model = gcn.GCN(dims, gemm=gemm, packed_activations=packed_activations,
-                        linear_first_when_narrowing=linear_first).to(dev)
+                        linear_first_when_narrowing=linear_first, fused_layers=fused).to(dev)
         opt = torch.optim.Adam(model.parameters(), lr=0.01)
         losses = [float(gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks)) for _ in range(2)]
         torch.cuda.synchronize()
@@ -606,7 +610,7 @@ def run_c5(args, graph):
             loss = gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks)
         torch.cuda.synchronize()
         tag = (f"{gemm}_gemm" + ("_packed_activations" if packed_activations else "")
-               + ("_linear_first_when_narrowing" if linear_first else ""))
+               + ("_linear_first_when_narrowing" if linear_first else "") + ("" if fused else "_separate_kernels"))
         out[f"train_step_ms_{tag}"] = round((time.perf_counter() - t0) * 1e3 / steps, 2)
         out[f"loss_{tag}"] = [round(v, 5) for v in losses + [float(loss)]]
         del model, opt

@@ -34,6 +34,11 @@ EXPORTS = (
     "gnnagg_wgrad_workspace_bytes",
     "gnnagg_wgrad_f32",
     "gnnagg_wgrad_strided_f32",
+    "gnnagg_linear_shape_supported",
+    "gnnagg_pack_keep_bits",
+    "gnnagg_linear_bias_relu_dropout_f32",
+    "gnnagg_wgrad_relu_dropout_backward_workspace_bytes",
+    "gnnagg_wgrad_relu_dropout_backward_f32",
     "gnnagg_dropout_layernorm_relu_blocks",
     "gnnagg_dropout_layernorm_relu_f32",
     "gnnagg_dropout_layernorm_relu_backward_f32",
@@ -120,6 +125,18 @@ def lib() -> ctypes.CDLL:
     L.gnnagg_bf16_to_f32.argtypes = [vp, vp, i64, vp]
     L.gnnagg_wgrad_strided_f32.restype = i32
     L.gnnagg_wgrad_strided_f32.argtypes = [vp, i64, vp, i64, vp, vp, i64, i64, i64, vp]
+    L.gnnagg_linear_shape_supported.restype = i32
+    L.gnnagg_linear_shape_supported.argtypes = [i64, i64]
+    L.gnnagg_pack_keep_bits.restype = i32
+    L.gnnagg_pack_keep_bits.argtypes = [vp, vp, i64, i64, vp]
+    L.gnnagg_linear_bias_relu_dropout_f32.restype = i32
+    L.gnnagg_linear_bias_relu_dropout_f32.argtypes = [vp, i64, vp, i64, vp, vp, vp, ctypes.c_float, i32, vp, i64, i64,
+                                                      i64, i64, vp]
+    L.gnnagg_wgrad_relu_dropout_backward_workspace_bytes.restype = i64
+    L.gnnagg_wgrad_relu_dropout_backward_workspace_bytes.argtypes = [i64, i64, i64]
+    L.gnnagg_wgrad_relu_dropout_backward_f32.restype = i32
+    L.gnnagg_wgrad_relu_dropout_backward_f32.argtypes = [vp, i64, vp, i64, vp, i64, vp, ctypes.c_float, vp, vp, vp, vp,
+                                                         i64, i64, i64, vp]
     L.gnnagg_dropout_layernorm_relu_blocks.restype = i32
     L.gnnagg_dropout_layernorm_relu_blocks.argtypes = [i64, i64]
     L.gnnagg_dropout_layernorm_relu_f32.restype = i32

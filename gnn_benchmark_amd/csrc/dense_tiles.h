@@ -44,6 +44,11 @@ struct ChunkLoader {
         for (int j = 0; j < NV; ++j)
             reg[j] = __builtin_nontemporal_load(reinterpret_cast<const floatx4 *>(chunk + src_off[j]));
     }
+    // the same for an operand that every block reads again (stays in cache)
+    __device__ void fetch_cached(const float *chunk) {
+#pragma unroll
+        for (int j = 0; j < NV; ++j) reg[j] = *reinterpret_cast<const floatx4 *>(chunk + src_off[j]);
+    }
     // only the first `valid` values of the chunk exist; the rest reads as zeros.  `aligned` is false
     // when rows are not a whole number of float4 (then fetch() is never used either).
     __device__ void fetch_tail(const float *chunk, int valid, bool aligned) {

@@ -1,0 +1,326 @@
+// Dense layer product with the elementwise work behind it fused in,
+// for rows in the millions and K, N <= 256 (fp32 MFMA, v_mfma_f32_32x32x2f32; 2*rows*K*N flop
+// against the 157.3 TFLOP/s fp32 matrix peak).  The epilogue divides row r by row_div[r],
+// adds the bias, applies ReLU and the dropout keep-bits while the result is still in the
+// accumulators, so the layer needs no elementwise pass over its [rows, N] result.
+//
+//     Y[rows, N] = epilogue( A[rows, K] @ W[K, N] )
+//
+// A block of four waves (2 x 2) owns 64*WM rows and all N <= 64*WN columns at a time and
+// walks its share of the row tiles; two blocks share a CU, so that one block's epilogue
+// overlaps the other's MFMAs.  The contraction runs in chunks of 16: 64*WM x 16 values of A (a 64-byte piece of each row) and 16 x N
+// values of W are copied into LDS through registers, the next chunk in flight behind the
+// MFMAs of the current one.  A is row-major with the contraction index contiguous, while
+// the MFMA wants one contraction index per lane across 32 rows; each lane therefore reads
+// four consecutive values of its row with one 16-byte LDS read and spends them on four
+// MFMAs (lanes 0-31 hold k+0..3, lanes 32-63 k+4..7 of each group of eight: the order of
+// the contraction is permuted, the same way for both operands).
+#include "common.h"
+#include "dense_tiles.h"
+
+namespace gnnagg {
+namespace {
+
+struct LinearArgs {
+    const float *a;          // [rows, K], row stride lda
+    const float *row_div;    // [rows] or nullptr
+    const float *w;          // [K, N], row stride ldw
+    const float *bias;       // [N] or nullptr
+    const uint32_t *keep;    // [rows, ceil(N/32)] keep-bits or nullptr
+    float *y;                // [rows, N], row stride ldy
+    int64_t rows;
+    int lda, ldw, ldy, k, n;
+    float scale;             // dropout scale of the epilogue
+    int relu;
+};
+
+template <int WM, int WN>
+struct LinearShape {
+    static constexpr int kRows = 64 * WM;            // rows of A per block
+    static constexpr int kLda = kChunk + 4;          // floats between staged rows: 16-byte reads of 8 rows hit 8 bank groups
+    static constexpr int kLdb = 64 * WN + 8;         // rows four apart (the two half-waves) land on the other half of the banks
+    static constexpr int kVecA = WM;                 // float4 per thread per chunk of A
+    static constexpr int kVecB = WN * kChunk / 16;   // float4 per thread per chunk of W
+    static constexpr int kBufFloats = kRows * kLda + kChunk * kLdb;
+    static constexpr int kSmemFloats = 2 * kBufFloats + 256 * 4;
+};
+
+template <int WM, int WN>
+__global__ __launch_bounds__(256, 2) void linear_kernel(const LinearArgs p) {
+    using S = LinearShape<WM, WN>;
+    extern __shared__ __align__(16) float smem[];
+    float *dump = smem + 2 * S::kBufFloats + 4 * (int)threadIdx.x;
+
+    const int tid = (int)threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int kk = lane >> 5;
+    const int idx = lane & 31;
+    const int m0 = wm * 32 * WM, n0 = wn * 32 * WN;
+    const int64_t tiles = (p.rows + S::kRows - 1) / S::kRows;
+    int64_t tile = blockIdx.x;
+    if (tile >= tiles) return;
+
+    // acc[i][j] is the 32 x 32 tile of Y^T whose columns (lanes) are rows m0 + 32 i .. of Y and whose
+    // rows (registers) are columns n0 + 32 j .. of Y: a lane ends up with runs of four consecutive
+    // columns of one row of Y, which it stores 16 bytes at a time.
+    floatx16 acc[WM][WN];
+    auto clear = [&]() {
+#pragma unroll
+        for (int i = 0; i < WM; ++i)
+#pragma unroll
+            for (int j = 0; j < WN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    };
+    clear();
+
+    // A: thread t moves the float4 number t + 256*j of a chunk, i.e. piece t%4 of row t/4 + 64*j of the
+    // tile.  Rows past the end read the last row instead; their results are never stored.
+    const float *ap[S::kVecA];
+    int a_dst[S::kVecA];
+#pragma unroll
+    for (int j = 0; j < S::kVecA; ++j) a_dst[j] = ((tid >> 2) + 64 * j) * S::kLda + 4 * (tid & 3);
+    auto enter_tile = [&](int64_t t) {
+#pragma unroll
+        for (int j = 0; j < S::kVecA; ++j) {
+            int64_t row = t * S::kRows + (tid >> 2) + 64 * j;
+            if (row >= p.rows) row = p.rows - 1;
+            ap[j] = p.a + (size_t)row * (size_t)p.lda + 4 * (tid & 3);
+        }
+    };
+    floatx4 areg[S::kVecA];
+    auto fetch_a = [&](int k0) {
+#pragma unroll
+        for (int j = 0; j < S::kVecA; ++j) areg[j] = *reinterpret_cast<const floatx4 *>(ap[j] + k0);
+    };
+    auto store_a = [&](float *buf) {
+#pragma unroll
+        for (int j = 0; j < S::kVecA; ++j) *reinterpret_cast<floatx4 *>(buf + a_dst[j]) = areg[j];
+    };
+    ChunkLoader<S::kVecB, S::kLdb> lw;
+    lw.init(tid, p.n, p.ldw);
+
+    // Columns past n of a staged row of W are never written: whatever they hold only reaches
+    // accumulator entries that are never stored.
+    auto multiply = [&](int buf) {
+        const float *as = smem + buf * S::kBufFloats + (m0 + idx) * S::kLda + 4 * kk;
+        const float *bs = smem + buf * S::kBufFloats + S::kRows * S::kLda + 4 * kk * S::kLdb + n0 + idx;
+        floatx4 av[2][WM];
+        float bv[2][WN];
+        auto read_a = [&](int h) {
+#pragma unroll
+            for (int i = 0; i < WM; ++i)
+                av[h][i] = *reinterpret_cast<const floatx4 *>(as + 32 * i * S::kLda + 8 * h);
+        };
+        auto read_b = [&](int s) {
+#pragma unroll
+            for (int j = 0; j < WN; ++j) bv[s & 1][j] = bs[(8 * (s >> 2) + (s & 3)) * S::kLdb + 32 * j];
+        };
+        read_a(0);
+        read_b(0);
+#pragma unroll
+        for (int s = 0; s < kChunk / 2; ++s) {
+            if (s + 1 < kChunk / 2) read_b(s + 1);
+            if (s == 2) read_a(1);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < WM; ++i)
+#pragma unroll
+                for (int j = 0; j < WN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[s & 1][j], av[s >> 2][i][s & 3], acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    // 32x32 accumulator layout: register r of lane l holds D[(r % 4) + 4 * (l / 32) + 8 * (r / 4)][l % 32]
+    const int words = (p.n + 31) / 32;  // keep-bit words per row
+    float rdiv[WM];                     // this lane's row divisors: loaded when a tile starts, used when it ends
+    auto load_divisors = [&](int64_t t) {
+#pragma unroll
+        for (int i = 0; i < WM; ++i) {
+            const int64_t m = t * S::kRows + m0 + 32 * i + idx;
+            rdiv[i] = (p.row_div && m < p.rows) ? p.row_div[m] : 1.0f;
+        }
+    };
+    auto finish_tile = [&](int64_t t) {
+#pragma unroll
+        for (int i = 0; i < WM; ++i) {
+            const int64_t m = t * S::kRows + m0 + 32 * i + idx;
+            const bool live = m < p.rows;
+            const float inv = 1.0f / rdiv[i];
+            float *yrow = p.y + (size_t)(live ? m : 0) * (size_t)p.ldy;
+#pragma unroll
+            for (int j = 0; j < WN; ++j) {
+                const int nt = n0 + 32 * j;
+                uint32_t bits = 0xffffffffu;
+                if (p.keep && live && nt < p.n) bits = p.keep[(size_t)m * (size_t)words + (nt >> 5)];
+                bits >>= 4 * kk;
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int n = nt + 8 * g + 4 * kk;
+                    if (!live || n >= p.n) continue;
+                    floatx4 v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+                    v *= inv;
+                    if (p.bias) v += *reinterpret_cast<const floatx4 *>(p.bias + n);
+                    if (p.relu) {
+                        v.x = fmaxf(v.x, 0.0f);
+                        v.y = fmaxf(v.y, 0.0f);
+                        v.z = fmaxf(v.z, 0.0f);
+                        v.w = fmaxf(v.w, 0.0f);
+                    }
+                    v *= p.scale;
+                    const uint32_t b = bits >> (8 * g);
+                    v.x = (b & 1u) ? v.x : 0.0f;
+                    v.y = (b & 2u) ? v.y : 0.0f;
+                    v.z = (b & 4u) ? v.z : 0.0f;
+                    v.w = (b & 8u) ? v.w : 0.0f;
+                    *reinterpret_cast<floatx4 *>(yrow + n) = v;
+                }
+            }
+        }
+    };
+
+    // One stream of chunks over all tiles of this block: the first chunk of the next tile is in
+    // flight behind the last MFMAs of the current one, and a tile's stores drain behind the next
+    // tile's MFMAs.
+    const int chunks = p.k / kChunk;
+    const size_t wstep = (size_t)kChunk * (size_t)p.ldw;
+    enter_tile(tile);
+    load_divisors(tile);
+    fetch_a(0);
+    lw.fetch_cached(p.w);
+    store_a(smem);
+    lw.store_all(smem + S::kRows * S::kLda, dump);
+    __syncthreads();
+    int buf = 0;
+    for (;;) {
+        const float *wc = p.w;
+        for (int c = 1; c < chunks; ++c) {
+            wc += wstep;
+            lw.fetch_cached(wc);
+            fetch_a(c * kChunk);
+            __builtin_amdgcn_sched_barrier(0);  // keep the loads ahead of the MFMAs
+            multiply(buf);
+            float *next = smem + (buf ^ 1) * S::kBufFloats;
+            store_a(next);
+            lw.store_all(next + S::kRows * S::kLda, dump);
+            __syncthreads();
+            buf ^= 1;
+        }
+        const int64_t done = tile;
+        tile += gridDim.x;
+        const bool more = tile < tiles;
+        if (more) {
+            enter_tile(tile);
+            lw.fetch_cached(p.w);
+            fetch_a(0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(buf);
+        if (more) {
+            float *next = smem + (buf ^ 1) * S::kBufFloats;
+            store_a(next);
+            lw.store_all(next + S::kRows * S::kLda, dump);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        finish_tile(done);
+        __builtin_amdgcn_sched_barrier(0);
+        if (!more) break;
+        load_divisors(tile);
+        clear();
+        __syncthreads();
+        buf ^= 1;
+    }
+}
+
+template <int WM, int WN>
+int launch_linear(const LinearArgs &p, hipStream_t st) {
+    using S = LinearShape<WM, WN>;
+    constexpr size_t smem = (size_t)S::kSmemFloats * sizeof(float);
+    GNNAGG_HIP(allow_lds(reinterpret_cast<const void *>(&linear_kernel<WM, WN>), smem));
+    int dev = 0, cus = 0;
+    GNNAGG_HIP(hipGetDevice(&dev));
+    GNNAGG_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    const int64_t tiles = (p.rows + S::kRows - 1) / S::kRows;
+    const int64_t resident = 2 * (int64_t)(cus > 0 ? cus : 256);  // two blocks per CU, each walks its share of the tiles
+    const unsigned blocks = (unsigned)(tiles < resident ? tiles : resident);
+    hipLaunchKernelGGL((linear_kernel<WM, WN>), dim3(blocks), dim3(256), smem, st, p);
+    GNNAGG_HIP(hipGetLastError());
+    return GNNAGG_OK;
+}
+
+int dispatch_linear(const LinearArgs &p, hipStream_t st) {
+    switch ((p.n + 63) / 64) {
+        case 1: return launch_linear<2, 1>(p, st);
+        case 2: return launch_linear<2, 2>(p, st);
+        case 3: return launch_linear<2, 3>(p, st);
+        default: return launch_linear<2, 4>(p, st);
+    }
+}
+
+bool aligned16(const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; }
+
+int check_linear(const LinearArgs &p) {
+    if (p.rows < 0 || p.k <= 0 || p.n <= 0) return fail(GNNAGG_ERR_INVALID, "negative or empty sizes");
+    if (p.k % kChunk != 0 || p.n % 4 != 0 || p.n > 256 || p.k > (1 << 20))
+        return fail(GNNAGG_ERR_UNSUPPORTED, "fused layer product takes K %% 16 == 0, N %% 4 == 0, N <= 256 (got K=%d N=%d)",
+                    p.k, p.n);
+    if (p.lda < p.k || p.ldw < p.n || p.ldy < p.n)
+        return fail(GNNAGG_ERR_INVALID, "row strides must be at least the widths");
+    if (p.lda % 4 || p.ldw % 4 || p.ldy % 4 || !aligned16(p.a) || !aligned16(p.w) || !aligned16(p.y) ||
+        !aligned16(p.bias))
+        return fail(GNNAGG_ERR_UNSUPPORTED, "fused layer product takes 16-byte aligned operands and row strides");
+    if (p.rows > 0 && (!p.a || !p.w || !p.y)) return fail(GNNAGG_ERR_INVALID, "null operand");
+    return GNNAGG_OK;
+}
+
+// one thread per word: 32 consecutive mask bytes of a row
+__global__ __launch_bounds__(256) void pack_keep_bits_kernel(const uint8_t *__restrict__ keep, uint32_t *__restrict__ bits,
+                                                             int feat, int words, int64_t total) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int64_t row = i / words;
+    const int f0 = (int)(i - row * words) * 32;
+    const uint8_t *src = keep + (size_t)row * feat + f0;
+    uint32_t w = 0;
+#pragma unroll 8
+    for (int q = 0; q < 32; ++q)
+        if (f0 + q < feat && src[q]) w |= 1u << q;
+    bits[i] = w;
+}
+
+}  // namespace
+}  // namespace gnnagg
+
+using namespace gnnagg;
+
+extern "C" int gnnagg_linear_shape_supported(int64_t k, int64_t n) {
+    return (k > 0 && n > 0 && k % kChunk == 0 && n % 4 == 0 && n <= 256 && k <= (1 << 20)) ? 1 : 0;
+}
+
+extern "C" int gnnagg_pack_keep_bits(const void *keep, uint32_t *bits, int64_t rows, int64_t feat, void *stream) {
+    GNNAGG_REQUIRE(rows >= 0 && feat > 0 && feat < (1 << 30), "bad sizes");
+    if (rows == 0) return GNNAGG_OK;
+    GNNAGG_REQUIRE(keep && bits, "null keep/bits");
+    const int words = (int)((feat + 31) / 32);
+    const int64_t total = rows * words;
+    hipLaunchKernelGGL(pack_keep_bits_kernel, dim3(grid_for(total, 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint8_t *>(keep), bits, (int)feat, words, total);
+    GNNAGG_HIP(hipGetLastError());
+    return GNNAGG_OK;
+}
+
+extern "C" int gnnagg_linear_bias_relu_dropout_f32(const float *x, int64_t x_stride, const float *w, int64_t w_stride,
+                                                   const float *bias, const uint32_t *keep_bits, const float *row_div,
+                                                   float scale, int relu, float *y, int64_t y_stride, int64_t rows,
+                                                   int64_t k, int64_t n, void *stream) {
+    GNNAGG_REQUIRE(x_stride < (1 << 27) && w_stride < (1 << 27) && y_stride < (1 << 27) && k < (1 << 27) && n < (1 << 27),
+                   "sizes and row strides must be below 2^27");
+    LinearArgs p{x, row_div, w, bias, keep_bits, y, rows, (int)x_stride, (int)w_stride, (int)y_stride, (int)k, (int)n,
+                 scale, relu};
+    if (int rc = check_linear(p)) return rc;
+    if (rows == 0) return GNNAGG_OK;
+    return dispatch_linear(p, static_cast<hipStream_t>(stream));
+}

@@ -28,12 +28,27 @@ struct WgradShape {
     static constexpr int kSmemFloats = 2 * kChunk * (kLdx + kLdg) + 256 * 4;  // + 16 bytes per thread to dump into
 };
 
-template <int WM, int WN>
+// What the MASKED form of the kernel does to G on its way into LDS: g is the gradient with respect
+// to a layer's output y = relu(z) * keep * scale, z = (x @ w) / row_div + bias.  The kernel turns it
+// into pre = (y > 0 ? g * scale : 0) (the gradient with respect to z; y is 0 exactly where the unit
+// was inactive or dropped), adds pre up per column (the bias gradient), divides by row_div, uses
+// the result as the G operand and also writes it out for the input-gradient product.
+struct MaskArgs {
+    const float *act;       // y [rows, fo], row stride ldact; with all_on: any readable array of that shape
+    const float *row_div;   // [rows] or nullptr
+    float *gz;              // out: [rows, fo] contiguous
+    float *bias_partial;    // out: [blocks][kVecG * 256] float4, the per-thread column sums
+    int ldact;
+    float scale;
+    int all_on;             // no ReLU / dropout behind the product: every entry counts
+};
+
+template <int WM, int WN, bool MASKED>
 __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__restrict__ x,
                                                                const float *__restrict__ g,
                                                                float *__restrict__ partial, int64_t rows, int fi,
                                                                int fo, int ldx, int ldg, int64_t rows_per_block,
-                                                               int aligned) {
+                                                               int aligned, const MaskArgs mk) {
     using S = WgradShape<WM, WN>;
     extern __shared__ __align__(16) float smem[];
     float *xs = smem;                              // [2][kChunk][kLdx]
@@ -69,6 +84,52 @@ __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__re
     lx.init(tid, fi, ldx);
     lg.init(tid, fo, ldg);
 
+    // MASKED: the activations come in with the same loader shape as G; thread t's vector j always sits in
+    // the same columns (the chunk is 16 whole rows), so its column sums stay in registers.
+    ChunkLoader<MASKED ? S::kVecG : 1, S::kLdg> lc;
+    floatx4 colsum[S::kVecG];
+    float dreg[S::kVecG];
+    int grow[S::kVecG];  // row of vector j inside a chunk
+    if (MASKED) {
+        lc.init(tid, fo, mk.ldact);
+#pragma unroll
+        for (int j = 0; j < S::kVecG; ++j) {
+            colsum[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+            grow[j] = lg.elem[j] / fo;
+        }
+    }
+    // any readable float per row when there is no divisor (the value is not used then)
+    const float *divp = MASKED ? (mk.row_div ? mk.row_div : x) : nullptr;
+    const int64_t divstep = MASKED ? (mk.row_div ? 1 : ldx) : 0;
+    auto fetch_divisors = [&](int64_t r, int64_t last) {  // rows r .. r+15, clamped to `last`
+#pragma unroll
+        for (int j = 0; j < S::kVecG; ++j) {
+            int64_t row = r + grow[j];
+            if (row > last) row = last;
+            dreg[j] = divp[row * divstep];
+        }
+    };
+    // turns lg.reg (g) into the G operand, with lc.reg = y; `valid` = number of values of the chunk that exist
+    auto mask_g = [&](int64_t r, int valid) {
+#pragma unroll
+        for (int j = 0; j < S::kVecG; ++j) {
+            const bool used = lg.lds_off[j] >= 0 && lg.elem[j] < valid;
+            const floatx4 gv = lg.reg[j], yv = lc.reg[j];
+            floatx4 pre;
+            const bool all = mk.all_on != 0;
+            pre.x = (used && (all || yv.x > 0.0f)) ? gv.x * mk.scale : 0.0f;
+            pre.y = (used && (all || yv.y > 0.0f)) ? gv.y * mk.scale : 0.0f;
+            pre.z = (used && (all || yv.z > 0.0f)) ? gv.z * mk.scale : 0.0f;
+            pre.w = (used && (all || yv.w > 0.0f)) ? gv.w * mk.scale : 0.0f;
+            colsum[j] += pre;
+            const float inv = mk.row_div ? 1.0f / dreg[j] : 1.0f;
+            pre *= inv;
+            lg.reg[j] = pre;
+            if (used)
+                __builtin_nontemporal_store(pre, reinterpret_cast<floatx4 *>(mk.gz + (size_t)r * (size_t)fo + lg.elem[j]));
+        }
+    };
+
     // Columns past fi / fo of an LDS row are never written: whatever they hold only reaches
     // accumulator entries that are never stored.
     auto multiply = [&](int buf) {
@@ -102,8 +163,15 @@ __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__re
         const float *xc = x + (size_t)r_begin * (size_t)ldx;
         const float *gc = g + (size_t)r_begin * (size_t)ldg;
         const size_t xstep = (size_t)kChunk * (size_t)ldx, gstep = (size_t)kChunk * (size_t)ldg;
+        const float *cc = MASKED ? mk.act + (size_t)r_begin * (size_t)mk.ldact : nullptr;
+        const size_t cstep = MASKED ? (size_t)kChunk * (size_t)mk.ldact : 0;
         lx.fetch(xc);
         lg.fetch(gc);
+        if (MASKED) {
+            lc.fetch(cc);
+            fetch_divisors(r_begin, r_end - 1);
+            mask_g(r_begin, kChunk * fo);
+        }
         lx.store_all(xs, dump);
         lg.store_all(gs, dump);
         __syncthreads();
@@ -112,8 +180,15 @@ __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__re
             gc += gstep;
             lx.fetch(xc);
             lg.fetch(gc);
+            if (MASKED) {
+                cc += cstep;
+                lc.fetch(cc);
+                fetch_divisors(r_begin + c * kChunk, r_end - 1);
+            }
             __builtin_amdgcn_sched_barrier(0);  // keep the loads ahead of the MFMAs
             multiply((int)((c - 1) & 1));
+            __builtin_amdgcn_sched_barrier(0);
+            if (MASKED) mask_g(r_begin + c * kChunk, kChunk * fo);
             lx.store_all(xs + (c & 1) * kChunk * S::kLdx, dump);
             lg.store_all(gs + (c & 1) * kChunk * S::kLdg, dump);
             __syncthreads();
@@ -126,6 +201,11 @@ __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__re
         const int left = (int)(r_end - r < kChunk ? r_end - r : kChunk);
         lx.fetch_tail(x + (size_t)r * (size_t)ldx, left * fi, aligned != 0);
         lg.fetch_tail(g + (size_t)r * (size_t)ldg, left * fo, aligned != 0);
+        if (MASKED) {  // the host only launches this form with 16-byte copies possible
+            lc.fetch_tail(mk.act + (size_t)r * (size_t)mk.ldact, left * fo, true);
+            fetch_divisors(r, r_end - 1);
+            mask_g(r, left * fo);
+        }
         lx.store(xs, aligned != 0);
         lg.store(gs, aligned != 0);
         __syncthreads();
@@ -133,6 +213,11 @@ __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__re
         __syncthreads();
     }
 
+    if (MASKED) {
+        floatx4 *bp = reinterpret_cast<floatx4 *>(mk.bias_partial) + (size_t)blockIdx.x * (S::kVecG * 256);
+#pragma unroll
+        for (int j = 0; j < S::kVecG; ++j) bp[j * 256 + tid] = colsum[j];
+    }
     // 32x32 accumulator layout: register r of lane l holds D[(r % 4) + 4 * (l / 32) + 8 * (r / 4)][l % 32]
     float *out = partial + (size_t)blockIdx.x * (size_t)fi * (size_t)fo;
 #pragma unroll
@@ -171,6 +256,30 @@ __global__ __launch_bounds__(256) void wgrad_reduce_kernel(const float *__restri
     }
 }
 
+// bias[n] = sum over the blocks and over the 16 rows of a chunk of the per-thread column sums: the
+// values of column n sit in the vectors number (4 * (n / 4) + r * fo) / 4, r < 16, of a chunk.  A block
+// of 256 threads owns 16 columns; thread (r, c) adds up row r of column c over the blocks, and the
+// 16 row sums of a column are then added in order of r.
+__global__ __launch_bounds__(256) void wgrad_bias_reduce_kernel(const float *__restrict__ partial, float *__restrict__ bias,
+                                                                int blocks, int vec_per_block, int fo) {
+    __shared__ float part[kChunk][16];
+    const int c = (int)threadIdx.x & 15, r = (int)threadIdx.x >> 4;
+    const int n = (int)blockIdx.x * 16 + c;
+    float s = 0.0f;
+    if (n < fo) {
+        const int v = (4 * (n / 4) + r * fo) / 4;
+        for (int b = 0; b < blocks; ++b) s += partial[((size_t)b * vec_per_block + v) * 4 + (n & 3)];
+    }
+    part[r][c] = s;
+    __syncthreads();
+    if (r == 0 && n < fo) {
+        float total = part[0][c];
+#pragma unroll
+        for (int k = 1; k < kChunk; ++k) total += part[k][c];
+        bias[n] = total;
+    }
+}
+
 int wgrad_blocks(int64_t rows) {
     int64_t b = 256;  // one block of four waves per CU: each wave keeps a SIMD's MFMA unit busy
     if (b * 64 > rows) b = rows / 64 > 0 ? rows / 64 : 1;
@@ -192,9 +301,10 @@ extern "C" int gnnagg_wgrad_f32(const float *x, const float *g, float *w_grad, v
     return gnnagg_wgrad_strided_f32(x, fi, g, fo, w_grad, workspace, rows, fi, fo, stream);
 }
 
-extern "C" int gnnagg_wgrad_strided_f32(const float *x, int64_t x_stride, const float *g, int64_t g_stride,
-                                        float *w_grad, void *workspace, int64_t rows, int64_t fi, int64_t fo,
-                                        void *stream) {
+namespace {
+
+int run_wgrad(const float *x, int64_t x_stride, const float *g, int64_t g_stride, float *w_grad, void *workspace,
+              int64_t rows, int64_t fi, int64_t fo, void *stream, const MaskArgs *mask, float *bias_grad) {
     GNNAGG_REQUIRE(rows >= 0 && fi > 0 && fo > 0, "bad size");
     GNNAGG_REQUIRE(x_stride >= fi && g_stride >= fo && x_stride < (int64_t(1) << 27) && g_stride < (int64_t(1) << 27),
                    "row strides %lld / %lld must be at least the widths %lld / %lld and below 2^27",
@@ -204,10 +314,13 @@ extern "C" int gnnagg_wgrad_strided_f32(const float *x, int64_t x_stride, const 
                     (long long)fo);
     GNNAGG_REQUIRE(w_grad, "null w_grad");
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (rows == 0) {  // empty sum: the reduce kernel over zero partials writes zeros
+    if (rows == 0) {  // empty sums: the reduce kernels over zero partials write zeros
         const int count0 = (int)(fi * fo);
-        hipLaunchKernelGGL(wgrad_reduce_kernel, dim3((unsigned)((count0 + kReduceOutputs - 1) / kReduceOutputs)), dim3(256), 0, st,
-                           static_cast<const float *>(nullptr), w_grad, 0, count0);
+        hipLaunchKernelGGL(wgrad_reduce_kernel, dim3((unsigned)((count0 + kReduceOutputs - 1) / kReduceOutputs)), dim3(256),
+                           0, st, static_cast<const float *>(nullptr), w_grad, 0, count0);
+        if (mask)
+            hipLaunchKernelGGL(wgrad_bias_reduce_kernel, dim3(grid_for(fo, 16)), dim3(256), 0, st,
+                               static_cast<const float *>(nullptr), bias_grad, 0, 0, (int)fo);
         GNNAGG_HIP(hipGetLastError());
         return GNNAGG_OK;
     }
@@ -220,14 +333,28 @@ extern "C" int gnnagg_wgrad_strided_f32(const float *x, int64_t x_stride, const 
                             ? 1
                             : 0;
     float *partial = static_cast<float *>(workspace);
+    MaskArgs mk{};
+    if (mask) {
+        mk = *mask;
+        if (!aligned || mk.ldact % 4 != 0 || (reinterpret_cast<uintptr_t>(mk.act) & 15) != 0 ||
+            (reinterpret_cast<uintptr_t>(mk.gz) & 15) != 0)
+            return fail(GNNAGG_ERR_UNSUPPORTED, "the masked weight gradient takes widths and row strides that are "
+                                                "multiples of 4 floats and 16-byte aligned operands");
+        mk.bias_partial = partial + (size_t)blocks * (size_t)fi * (size_t)fo;  // behind the partial weight gradients
+    }
     // wave corner = 32*WM x 32*WN, block = 2 x 2 waves
     const int wm = (int)((fi + 63) / 64), wn = (int)((fo + 63) / 64);
-#define GNNAGG_WGRAD(M, N)                                                                                   \
-    if (wm == M && wn == N) {                                                                                \
-        constexpr size_t smem = (size_t)WgradShape<M, N>::kSmemFloats * sizeof(float);                       \
-        GNNAGG_HIP(allow_lds(reinterpret_cast<const void *>(&wgrad_partial_kernel<M, N>), smem));           \
-        hipLaunchKernelGGL((wgrad_partial_kernel<M, N>), dim3((unsigned)blocks), dim3(256), smem, st, x, g,  \
-                           partial, rows, (int)fi, (int)fo, (int)x_stride, (int)g_stride, rpb, aligned);     \
+#define GNNAGG_WGRAD_FORM(M, N, MASKED)                                                                         \
+    {                                                                                                           \
+        constexpr size_t smem = (size_t)WgradShape<M, N>::kSmemFloats * sizeof(float);                          \
+        GNNAGG_HIP(allow_lds(reinterpret_cast<const void *>(&wgrad_partial_kernel<M, N, MASKED>), smem));       \
+        hipLaunchKernelGGL((wgrad_partial_kernel<M, N, MASKED>), dim3((unsigned)blocks), dim3(256), smem, st, x, g, \
+                           partial, rows, (int)fi, (int)fo, (int)x_stride, (int)g_stride, rpb, aligned, mk);    \
+    }
+#define GNNAGG_WGRAD(M, N)                         \
+    if (wm == M && wn == N) {                      \
+        if (mask) GNNAGG_WGRAD_FORM(M, N, true)    \
+        else GNNAGG_WGRAD_FORM(M, N, false)        \
     } else
     GNNAGG_WGRAD(1, 1) GNNAGG_WGRAD(1, 2) GNNAGG_WGRAD(1, 3) GNNAGG_WGRAD(1, 4) GNNAGG_WGRAD(2, 1) GNNAGG_WGRAD(2, 2)
     GNNAGG_WGRAD(2, 3) GNNAGG_WGRAD(2, 4) GNNAGG_WGRAD(3, 1) GNNAGG_WGRAD(3, 2) GNNAGG_WGRAD(3, 3) GNNAGG_WGRAD(3, 4)
@@ -235,10 +362,41 @@ extern "C" int gnnagg_wgrad_strided_f32(const float *x, int64_t x_stride, const 
         return fail(GNNAGG_ERR_UNSUPPORTED, "no weight-gradient shape for Fi=%lld Fo=%lld", (long long)fi, (long long)fo);
     }
 #undef GNNAGG_WGRAD
+#undef GNNAGG_WGRAD_FORM
     GNNAGG_HIP(hipGetLastError());
     const int count = (int)(fi * fo);
-    hipLaunchKernelGGL(wgrad_reduce_kernel, dim3((unsigned)((count + kReduceOutputs - 1) / kReduceOutputs)), dim3(256), 0, st, partial, w_grad,
-                       blocks, count);
+    hipLaunchKernelGGL(wgrad_reduce_kernel, dim3((unsigned)((count + kReduceOutputs - 1) / kReduceOutputs)), dim3(256), 0,
+                       st, partial, w_grad, blocks, count);
+    if (mask)
+        hipLaunchKernelGGL(wgrad_bias_reduce_kernel, dim3(grid_for(fo, 16)), dim3(256), 0, st, mk.bias_partial, bias_grad,
+                           blocks, wn * 256, (int)fo);
     GNNAGG_HIP(hipGetLastError());
     return GNNAGG_OK;
+}
+
+}  // namespace
+
+extern "C" int gnnagg_wgrad_strided_f32(const float *x, int64_t x_stride, const float *g, int64_t g_stride,
+                                        float *w_grad, void *workspace, int64_t rows, int64_t fi, int64_t fo,
+                                        void *stream) {
+    return run_wgrad(x, x_stride, g, g_stride, w_grad, workspace, rows, fi, fo, stream, nullptr, nullptr);
+}
+
+extern "C" int64_t gnnagg_wgrad_relu_dropout_backward_workspace_bytes(int64_t rows, int64_t fi, int64_t fo) {
+    if (rows <= 0 || fi <= 0 || fo <= 0 || fi > 256 || fo > 256 || fi % 4 != 0 || fo % 4 != 0) return 0;
+    const int64_t wn = (fo + 63) / 64;
+    return (int64_t)wgrad_blocks(rows) * (fi * fo + wn * 1024) * (int64_t)sizeof(float);
+}
+
+extern "C" int gnnagg_wgrad_relu_dropout_backward_f32(const float *x, int64_t x_stride, const float *grad_y,
+                                                      int64_t grad_stride, const float *y, int64_t y_stride,
+                                                      const float *row_div, float scale, float *grad_z, float *w_grad,
+                                                      float *bias_grad, void *workspace, int64_t rows, int64_t fi,
+                                                      int64_t fo, void *stream) {
+    GNNAGG_REQUIRE(bias_grad, "null bias_grad");
+    GNNAGG_REQUIRE(rows == 0 || grad_z, "null grad_z");
+    GNNAGG_REQUIRE(!y || (y_stride >= fo && y_stride < (int64_t(1) << 27)), "bad row stride of y");
+    // without y the kernel reads g a second time in its place (a cache hit) and ignores the values
+    MaskArgs mk{y ? y : grad_y, row_div, grad_z, nullptr, (int)(y ? y_stride : grad_stride), scale, y ? 0 : 1};
+    return run_wgrad(x, x_stride, grad_y, grad_stride, w_grad, workspace, rows, fi, fo, stream, &mk, bias_grad);
 }

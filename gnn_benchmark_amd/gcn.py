@@ -10,7 +10,11 @@ with a precomputed seeded mask, log-softmax + NLL on the labelled nodes, Adam.  
 forward and input-gradient products run on the matrix cores through the BLAS library
 behind ``torch.mm`` (fp32, or bf16 inputs with fp32 accumulation and fp32 output); the
 weight gradient -- a reduction over millions of rows into at most 256 x 256 outputs, the
-library's weakest shape -- runs in libgnnagg's own fp32 MFMA kernel.
+library's weakest shape -- runs in libgnnagg's own fp32 MFMA kernel.  With fp32 products and
+dense activations a layer whose widths the kernels take runs fused (``_FusedLayer``): the
+product, the degree division, bias, ReLU and dropout are one libgnnagg kernel, and in the
+gradient direction the ReLU / dropout mask, the degree division, the bias gradient and the
+weight gradient are another; only the input-gradient product stays with the BLAS library.
 """
 from typing import List, Optional, Sequence
 
@@ -81,6 +85,83 @@ class _Fp32Linear(torch.autograd.Function):
         gx = torch.mm(g, w.t()) if ctx.needs_input_grad[0] else None
         gw = weight_gradient(x, g) if ctx.needs_input_grad[1] else None
         return gx, gw
+
+
+def pack_keep_mask(keep: torch.Tensor) -> torch.Tensor:
+    """Bool / uint8 keep-mask [rows, feat] -> int32 [rows, ceil(feat / 32)]: bit q of word (r, v)
+    is keep[r, 32 v + q].  The form the fused layer kernel reads (1 bit instead of 1 byte per unit)."""
+    if not keep.is_cuda or keep.dtype not in (torch.bool, torch.uint8) or keep.dim() != 2 or not keep.is_contiguous():
+        raise RuntimeError("Input mismatch: keep must be a contiguous bool/uint8 [rows, feat] GPU (HIP) tensor")
+    rows, feat = keep.shape
+    bits = torch.empty(rows, (feat + 31) // 32, dtype=torch.int32, device=keep.device)
+    with torch.cuda.device(keep.device):
+        _lib.check(_lib.lib().gnnagg_pack_keep_bits(_lib.ptr(keep), _lib.ptr(bits), rows, feat,
+                                                    _lib.current_stream(keep.device)))
+    return bits
+
+
+def fused_layer_supported(x: torch.Tensor, in_channels: int, out_channels: int) -> bool:
+    """Whether ``_FusedLayer`` takes a [rows, in_channels] operand on x's device and these widths."""
+    if not (x.is_cuda and x.dtype == torch.float32):
+        return False
+    L = _lib.lib()
+    return bool(L.gnnagg_linear_shape_supported(in_channels, out_channels)
+                and L.gnnagg_wgrad_relu_dropout_backward_workspace_bytes(max(x.size(0), 1), in_channels, out_channels) > 0)
+
+
+def _kernel_ready(x: torch.Tensor) -> torch.Tensor:
+    """x as the fused kernels read it: dense rows, 16-byte aligned rows."""
+    if x.dim() == 2 and _rows_are_dense(x) and _row_stride(x) % 4 == 0 and x.data_ptr() % 16 == 0:
+        return x
+    return x.contiguous()
+
+
+class _FusedLayer(torch.autograd.Function):
+    """y = relu((x @ w) / row_div + bias) * (keep ? scale : 0) in one kernel (``relu`` False and
+    ``keep_bits`` None: y = (x @ w) / row_div + bias, the last layer).  The gradient direction
+    is one more kernel -- mask, degree division, bias gradient and weight gradient in a single
+    pass over x, the incoming gradient and y -- plus the BLAS product for the input gradient."""
+
+    @staticmethod
+    def forward(ctx, x, w, bias, keep_bits, scale, row_div, relu):
+        rows, k, n = x.size(0), x.size(1), w.size(1)
+        if keep_bits is not None and (keep_bits.dtype != torch.int32 or keep_bits.shape != (rows, (n + 31) // 32)
+                                      or not keep_bits.is_contiguous()):
+            raise RuntimeError("Input mismatch: keep_bits must be contiguous int32 [rows, ceil(feat / 32)] "
+                               "(gcn.pack_keep_mask)")
+        if row_div is not None and (row_div.dtype != torch.float32 or row_div.numel() != rows
+                                    or not row_div.is_contiguous()):
+            raise RuntimeError("Input mismatch: row_div must be contiguous float32 with one entry per row")
+        w = w.contiguous()
+        y = torch.empty(rows, n, dtype=torch.float32, device=x.device)
+        with torch.cuda.device(x.device):
+            _lib.check(_lib.lib().gnnagg_linear_bias_relu_dropout_f32(
+                _lib.ptr(x), _row_stride(x), _lib.ptr(w), n, _lib.ptr(bias.contiguous()), _lib.ptr(keep_bits),
+                _lib.ptr(row_div), float(scale), 1 if relu else 0, _lib.ptr(y), n, rows, k, n,
+                _lib.current_stream(x.device)))
+        ctx.save_for_backward(x, w, y if relu or keep_bits is not None else None)
+        ctx.scale = float(scale)
+        ctx.row_div = row_div
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_y):
+        x, w, y = ctx.saved_tensors
+        grad_y = _kernel_ready(grad_y)
+        rows, k, n = x.size(0), x.size(1), w.size(1)
+        L = _lib.lib()
+        workspace = torch.empty(int(L.gnnagg_wgrad_relu_dropout_backward_workspace_bytes(max(rows, 1), k, n)) // 4,
+                                dtype=torch.float32, device=x.device)
+        grad_z = torch.empty(rows, n, dtype=torch.float32, device=x.device)
+        grad_w = torch.empty(k, n, dtype=torch.float32, device=x.device)
+        grad_bias = torch.empty(n, dtype=torch.float32, device=x.device)
+        with torch.cuda.device(x.device):
+            _lib.check(L.gnnagg_wgrad_relu_dropout_backward_f32(
+                _lib.ptr(x), _row_stride(x), _lib.ptr(grad_y), _row_stride(grad_y), _lib.ptr(y),
+                n if y is not None else 0, _lib.ptr(ctx.row_div), ctx.scale, _lib.ptr(grad_z), _lib.ptr(grad_w),
+                _lib.ptr(grad_bias), _lib.ptr(workspace), rows, k, n, _lib.current_stream(x.device)))
+        grad_x = torch.mm(grad_z, w.t()) if ctx.needs_input_grad[0] else None
+        return grad_x, grad_w, grad_bias, None, None, None, None
 
 
 class _BiasReluDropout(torch.autograd.Function):
@@ -180,6 +261,7 @@ class GCNLayer(torch.nn.Module):
             raise ValueError("gemm must be 'fp32' or 'bf16'")
         self.gemm = gemm
         self.linear_first = False
+        self.fuse = True  # use the fused layer kernels where they apply
         self.weight = torch.nn.Parameter(torch.empty(in_channels, out_channels))
         self.bias = torch.nn.Parameter(torch.zeros(out_channels))
         torch.nn.init.xavier_uniform_(self.weight, gain=torch.nn.init.calculate_gain("relu"))
@@ -201,16 +283,32 @@ class GCNLayer(torch.nn.Module):
             return Aggregator.apply(graph, self._product(x), layer, 32, is_pre_delay, self.training)
         return self._product(Aggregator.apply(graph, x, layer, 32, is_pre_delay, self.training))
 
+    def fused(self, graph, x, layer: int, is_pre_delay: bool, keep_bits, scale: float, relu: bool):
+        """relu(((A x) W) / deg + bias) * keep * scale through the fused kernels, or None where they do
+        not apply (bf16 products, packed input, product-first order, widths the kernels do not take)."""
+        if self.gemm != "fp32" or self.linear_first or isinstance(x, tuple) or not self.fuse:
+            return None
+        if not fused_layer_supported(x, self.weight.size(0), self.weight.size(1)):
+            return None
+        agg = _kernel_ready(Aggregator.apply(graph, x, layer, 32, is_pre_delay, self.training))
+        row_div = graph.in_degrees.reshape(-1)
+        return _FusedLayer.apply(agg, self.weight, self.bias, keep_bits, scale, row_div, relu)
+
     def forward(self, graph, x: torch.Tensor, layer: int, is_pre_delay: bool) -> torch.Tensor:
         """((A x) W) / deg + bias."""
+        out = self.fused(graph, x, layer, is_pre_delay, None, 1.0, False)
+        if out is not None:
+            return out
         return torch.addcdiv(self.bias, self.transform(graph, x, layer, is_pre_delay), graph.in_degrees)
 
 
 class GCN(torch.nn.Module):
     def __init__(self, dims: Sequence[int], gemm: str = "fp32", dropout: float = 0.5, packed_activations: bool = False,
-                 linear_first_when_narrowing: bool = False):
+                 linear_first_when_narrowing: bool = False, fused_layers: bool = True):
         super().__init__()
         self.layers = torch.nn.ModuleList([GCNLayer(dims[i], dims[i + 1], gemm) for i in range(len(dims) - 1)])
+        for layer in self.layers:  # one-kernel layers where they apply (fp32 products, dense activations)
+            layer.fuse = fused_layers
         if linear_first_when_narrowing:  # a layer with fewer outputs than inputs aggregates its outputs
             for i, layer in enumerate(self.layers):
                 layer.linear_first = dims[i + 1] < dims[i]
@@ -218,29 +316,55 @@ class GCN(torch.nn.Module):
         # keep hidden activations packed (non-zero values + bitmap) where their width allows and
         # pre-aggregation is used: the next layer's aggregation then skips the zeros
         self.packed_activations = packed_activations
+        self._mask_cache = {}
 
-    def forward(self, graph, x: torch.Tensor, is_pre_delay: bool,
-                masks: Optional[List[torch.Tensor]] = None) -> torch.Tensor:
-        """``masks[l]``: bool keep-mask [N, dims[l+1]] of the dropout after layer l (training only)."""
+    def _packed_mask(self, mask: torch.Tensor) -> torch.Tensor:
+        """Bit-packed form of a bool mask, remembered while the same tensor (unchanged) comes back --
+        the seeded masks of a benchmark or test are reused step after step."""
+        key = (mask.data_ptr(), tuple(mask.shape), mask._version)
+        hit = self._mask_cache.get(key)
+        if hit is None:
+            if len(self._mask_cache) >= 2 * len(self.layers):
+                self._mask_cache.clear()
+            hit = self._mask_cache[key] = (mask, pack_keep_mask(mask))  # holding the mask keeps its address its own
+        return hit[1]
+
+    def forward(self, graph, x: torch.Tensor, is_pre_delay: bool, masks: Optional[List[torch.Tensor]] = None,
+                log_probs: bool = True) -> torch.Tensor:
+        """``masks[l]``: keep-mask of the dropout after layer l (training only): bool [N, dims[l+1]], or
+        its bit-packed form (``pack_keep_mask``) for a layer that runs fused.  ``log_probs=False``
+        returns the last layer's output before the log-softmax."""
         h = x
         last = len(self.layers) - 1
         for l, layer in enumerate(self.layers):
             if l == last:
                 h = layer(graph, h, l, is_pre_delay)
                 break
-            z = layer.transform(graph, h, l, is_pre_delay)
+            width = layer.weight.size(1)
             single_rank = getattr(graph, "exchange", None) is None
             # a next layer that multiplies first reads its input densely: nothing to gain from packing
             pack = (self.packed_activations and (is_pre_delay or single_rank)
-                    and packed.header_words(z.size(1)) > 0 and not self.layers[l + 1].linear_first)
+                    and packed.header_words(width) > 0 and not self.layers[l + 1].linear_first)
+            dropping = self.training and self.dropout > 0.0
+            if dropping and masks is None:
+                raise ValueError("training needs the seeded dropout masks")
+            mask = masks[l] if dropping else None
+            scale = 1.0 / (1.0 - self.dropout) if dropping else 1.0
+            if not pack:
+                bits = mask
+                if mask is not None and mask.dtype != torch.int32:
+                    bits = self._packed_mask(mask)
+                fused = layer.fused(graph, h, l, is_pre_delay, bits, scale, True)
+                if fused is not None:
+                    h = fused
+                    continue
+            if mask is not None and mask.dtype == torch.int32:
+                raise RuntimeError("a bit-packed dropout mask only serves the fused layer kernels; this layer needs "
+                                   "the bool mask")
+            z = layer.transform(graph, h, l, is_pre_delay)
             epilogue = _BiasReluDropoutPacked if pack else _BiasReluDropout
-            if self.training and self.dropout > 0.0:
-                if masks is None:
-                    raise ValueError("training needs the seeded dropout masks")
-                h = epilogue.apply(z, layer.bias, masks[l], 1.0 / (1.0 - self.dropout), graph.in_degrees)
-            else:
-                h = epilogue.apply(z, layer.bias, None, 1.0, graph.in_degrees)
-        return F.log_softmax(h, dim=1)
+            h = epilogue.apply(z, layer.bias, mask, scale, graph.in_degrees)
+        return F.log_softmax(h, dim=1) if log_probs else h
 
 
 def make_dropout_masks(num_nodes: int, dims: Sequence[int], p: float, seed: int, device) -> List[torch.Tensor]:
@@ -249,11 +373,12 @@ def make_dropout_masks(num_nodes: int, dims: Sequence[int], p: float, seed: int,
 
 
 def train_step(model: GCN, optimizer, graph, x, labels, train_idx, is_pre_delay: bool, masks) -> torch.Tensor:
-    """forward, NLL loss on the labelled nodes, backward, optimizer update."""
+    """forward, NLL loss on the labelled nodes, backward, optimizer update.  The log-softmax is
+    row-wise, so only the labelled rows are normalised."""
     model.train()
     optimizer.zero_grad(set_to_none=True)
-    out = model(graph, x, is_pre_delay, masks)
-    loss = F.nll_loss(out[train_idx], labels[train_idx])
+    out = model(graph, x, is_pre_delay, masks, log_probs=False)
+    loss = F.nll_loss(F.log_softmax(out[train_idx], dim=1), labels[train_idx])
     loss.backward()
     optimizer.step()
     return loss.detach()

@@ -335,9 +335,12 @@ class DistSAGE(torch.nn.Module):
         for norm in self.norms:
             norm.reset_parameters()
 
-    def forward(self, graph, nodes_feats: torch.Tensor, masks: Optional[List[torch.Tensor]] = None) -> torch.Tensor:
+    def forward(self, graph, nodes_feats: torch.Tensor, masks: Optional[List[torch.Tensor]] = None,
+                log_probs: bool = True) -> torch.Tensor:
         """``nodes_feats``: ``[N, in_channels]`` or staged (``stage_input``).  ``masks[i]``: keep
-        mask ``[N, hidden]`` of the dropout after layer i (training; drawn here when None)."""
+        mask ``[N, hidden]`` of the dropout after layer i (training; drawn here when None).
+        ``log_probs=False`` returns the last layer's output before the log-softmax of
+        model/DistSAGE.py:69 (a caller that scores a subset of the nodes applies it to those rows)."""
         for i, conv in enumerate(self.convs[:-1]):
             z = conv(graph, nodes_feats, i)
             keep, scale = None, 1.0
@@ -347,7 +350,7 @@ class DistSAGE(torch.nn.Module):
             norm = self.norms[i]
             nodes_feats = dropout_layernorm_relu(z, keep, scale, norm.weight, norm.bias, norm.eps)
         out = self.convs[-1](graph, nodes_feats, len(self.convs) - 1)
-        return F.log_softmax(out, dim=1)
+        return F.log_softmax(out, dim=1) if log_probs else out
 
 
 def make_dropout_masks(num_nodes: int, hidden_channels: int, num_layers: int, p: float, seed: int,
@@ -357,11 +360,13 @@ def make_dropout_masks(num_nodes: int, hidden_channels: int, num_layers: int, p:
 
 
 def train_step(model: DistSAGE, optimizer, graph, nodes_feats, labels, train_idx, masks=None) -> torch.Tensor:
-    """One epoch of train.py:82-98: forward, NLL loss on the training nodes, backward, update."""
+    """One epoch of train.py:82-98: forward, NLL loss on the training nodes, backward, update.
+    The log-softmax is row-wise, so it is applied to the training rows only: the same loss and
+    gradients as train.py:87-89 without normalising the rows that are not scored."""
     model.train()
     optimizer.zero_grad(set_to_none=True)
-    out = model(graph, nodes_feats, masks)
-    loss = F.nll_loss(out[train_idx], labels[train_idx])
+    out = model(graph, nodes_feats, masks, log_probs=False)
+    loss = F.nll_loss(F.log_softmax(out[train_idx], dim=1), labels[train_idx])
     loss.backward()
     optimizer.step()
     return loss.detach()

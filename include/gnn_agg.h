@@ -191,6 +191,44 @@ int gnnagg_wgrad_strided_f32(const float *x, int64_t x_stride, const float *g, i
                              void *workspace, int64_t rows, int64_t fi, int64_t fo, void *stream);
 
 /* ---------------------------------------------------------------------------------
+ * Dense layer product with the elementwise work behind it fused in (fp32 MFMA, hand-written):
+ *   y = relu((x @ w) / row_div + bias) * (keep ? scale : 0)
+ * x fp32 [rows, k] (row stride x_stride floats), w fp32 [k, n] row-major (row stride
+ * w_stride), y fp32 [rows, n] (row stride y_stride); bias fp32 [n] or NULL; row_div fp32
+ * [rows] or NULL; relu 0/1; keep_bits NULL (nothing dropped; pass scale = 1) or uint32
+ * [rows, ceil(n / 32)] as written by gnnagg_pack_keep_bits from a uint8 [rows, n] mask: bit q
+ * of word (r, v) is keep[r, 32 * v + q].  Shapes: k % 16 == 0, n % 4 == 0, n <= 256, 16-byte
+ * aligned operands and row strides (GNNAGG_ERR_UNSUPPORTED otherwise;
+ * gnnagg_linear_shape_supported tells beforehand).  The contraction is summed in a fixed
+ * order: deterministic.
+ *
+ * Its counterpart in the gradient direction rides on the weight-gradient kernel below: with
+ * g the gradient with respect to y,
+ *   pre       = (y > 0 ? g * scale : 0)          bias_grad[f] = sum over rows of pre[:, f]
+ *   grad_z    = pre / row_div                     (written out, [rows, fo] contiguous: the
+ *                                                  operand of the input-gradient product)
+ *   w_grad    = x^T @ grad_z
+ * in one pass over x, g and y.  y = NULL: no ReLU / dropout behind the product (pre = g *
+ * scale).  Needs fi, fo <= 256 and multiples of 4, 16-byte aligned
+ * operands and row strides; workspace of gnnagg_wgrad_relu_dropout_backward_workspace_bytes
+ * (0 = unsupported shape) bytes, nothing is allocated.  Deterministic.
+ * The reference leaves these products to torch's Linear and runs dropout / ReLU as separate
+ * ops (model/layers/sageconv.py:87-91, model/DistSAGE.py:49-53); the fused forms belong to
+ * this build's GCN layer stack.
+ * ------------------------------------------------------------------------------- */
+int gnnagg_linear_shape_supported(int64_t k, int64_t n);
+int gnnagg_pack_keep_bits(const void *keep, uint32_t *bits, int64_t rows, int64_t feat, void *stream);
+int gnnagg_linear_bias_relu_dropout_f32(const float *x, int64_t x_stride, const float *w, int64_t w_stride,
+                                        const float *bias, const uint32_t *keep_bits, const float *row_div,
+                                        float scale, int relu, float *y, int64_t y_stride, int64_t rows, int64_t k,
+                                        int64_t n, void *stream);
+int64_t gnnagg_wgrad_relu_dropout_backward_workspace_bytes(int64_t rows, int64_t fi, int64_t fo);
+int gnnagg_wgrad_relu_dropout_backward_f32(const float *x, int64_t x_stride, const float *grad_y, int64_t grad_stride,
+                                           const float *y, int64_t y_stride, const float *row_div, float scale,
+                                           float *grad_z, float *w_grad, float *bias_grad, void *workspace,
+                                           int64_t rows, int64_t fi, int64_t fo, void *stream);
+
+/* ---------------------------------------------------------------------------------
  * The elementwise chain between two SAGE layers (model/DistSAGE.py:49-53: F.dropout, LayerNorm
  * over the features, F.relu) as one pass each way:
  *   y = relu(layer_norm(z * keep * scale; gamma, beta, eps))
