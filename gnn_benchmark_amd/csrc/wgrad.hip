@@ -36,7 +36,7 @@ struct WgradShape {
 struct MaskArgs {
     const float *act;       // y [rows, fo], row stride ldact; with all_on: any readable array of that shape
     const float *row_div;   // [rows] or nullptr
-    float *gz;              // out: [rows, fo] contiguous
+    float *gz;              // out: [rows, fo] contiguous, or nullptr (not wanted)
     float *bias_partial;    // out: [blocks][kVecG * 256] float4, the per-thread column sums
     int ldact;
     float scale;
@@ -125,7 +125,7 @@ __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__re
             const float inv = mk.row_div ? 1.0f / dreg[j] : 1.0f;
             pre *= inv;
             lg.reg[j] = pre;
-            if (used)
+            if (used && mk.gz)
                 __builtin_nontemporal_store(pre, reinterpret_cast<floatx4 *>(mk.gz + (size_t)r * (size_t)fo + lg.elem[j]));
         }
     };
@@ -394,7 +394,6 @@ extern "C" int gnnagg_wgrad_relu_dropout_backward_f32(const float *x, int64_t x_
                                                       float *bias_grad, void *workspace, int64_t rows, int64_t fi,
                                                       int64_t fo, void *stream) {
     GNNAGG_REQUIRE(bias_grad, "null bias_grad");
-    GNNAGG_REQUIRE(rows == 0 || grad_z, "null grad_z");
     GNNAGG_REQUIRE(!y || (y_stride >= fo && y_stride < (int64_t(1) << 27)), "bad row stride of y");
     // without y the kernel reads g a second time in its place (a cache hit) and ignores the values
     MaskArgs mk{y ? y : grad_y, row_div, grad_z, nullptr, (int)(y ? y_stride : grad_stride), scale, y ? 0 : 1};

@@ -70,6 +70,26 @@ def weight_gradient(x: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def weight_and_bias_gradient(x: torch.Tensor, g: torch.Tensor):
+    """(x^T @ g, g.sum(0)): the column sums come out of the weight-gradient kernel's pass over g.
+    Falls back to separate torch ops for shapes the kernel does not take."""
+    x, g = _kernel_ready(x), _kernel_ready(g)
+    rows, fi, fo = x.size(0), x.size(1), g.size(1)
+    L = _lib.lib()
+    ok = x.is_cuda and x.dtype == torch.float32 and g.dtype == torch.float32
+    nbytes = int(L.gnnagg_wgrad_relu_dropout_backward_workspace_bytes(rows, fi, fo)) if ok else 0
+    if nbytes == 0:
+        return weight_gradient(x, g), g.sum(dim=0)
+    grad_w = torch.empty(fi, fo, dtype=torch.float32, device=x.device)
+    grad_b = torch.empty(fo, dtype=torch.float32, device=x.device)
+    workspace = torch.empty(nbytes // 4, dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        _lib.check(L.gnnagg_wgrad_relu_dropout_backward_f32(
+            _lib.ptr(x), _row_stride(x), _lib.ptr(g), _row_stride(g), None, 0, None, 1.0, None, _lib.ptr(grad_w),
+            _lib.ptr(grad_b), _lib.ptr(workspace), rows, fi, fo, _lib.current_stream(x.device)))
+    return grad_w, grad_b
+
+
 class _Fp32Linear(torch.autograd.Function):
     """y = x @ w in fp32; the weight gradient (a reduction over millions of rows) runs in
     the hand-written MFMA kernel, the two other products in the BLAS library."""

@@ -28,7 +28,7 @@ import torch
 import torch.nn.functional as F
 
 from . import _lib, aggregator
-from .gcn import weight_gradient
+from .gcn import weight_and_bias_gradient, weight_gradient
 from .sparse_tensor import SparseTensor, _row_stride
 
 
@@ -156,10 +156,16 @@ class _SageConv(torch.autograd.Function):
         fi = cat.size(1) // 2
         g = g.contiguous()
         grad_cat = grad_w = grad_b = None
+        want_b = ctx.has_bias and ctx.needs_input_grad[3]
         if ctx.needs_input_grad[2]:
-            # each half's rows of the stacked weight: x_half^T @ g, reading the half where it lies
-            grad_w = torch.cat([weight_gradient(cat[:, :fi], g), weight_gradient(cat[:, fi:], g)], dim=0)
-        if ctx.has_bias and ctx.needs_input_grad[3]:
+            # each half's rows of the stacked weight: x_half^T @ g, reading the half where it lies; the
+            # bias gradient (column sums of g) comes out of the first of the two passes over g
+            if want_b:
+                top, grad_b = weight_and_bias_gradient(cat[:, :fi], g)
+            else:
+                top = weight_gradient(cat[:, :fi], g)
+            grad_w = torch.cat([top, weight_gradient(cat[:, fi:], g)], dim=0)
+        elif want_b:
             grad_b = g.sum(dim=0)
         if ctx.needs_input_grad[1]:
             grad_cat = torch.mm(g, weight.t())  # [N, 2 fi]: d/d aggregated | d/d x (direct part)
@@ -205,9 +211,14 @@ class _SageConvLinearFirst(torch.autograd.Function):
         g = g.contiguous()
         grad_left = aggregator._backward(ctx, g / ctx.graph.in_degrees if ctx.divide else g)   # d/d (x W_n)
         grad_x = grad_w = grad_b = None
+        want_b = ctx.has_bias and ctx.needs_input_grad[3]
         if ctx.needs_input_grad[2]:
-            grad_w = torch.cat([weight_gradient(x, grad_left), weight_gradient(x, g)], dim=0)
-        if ctx.has_bias and ctx.needs_input_grad[3]:
+            if want_b:
+                bottom, grad_b = weight_and_bias_gradient(x, g)
+            else:
+                bottom = weight_gradient(x, g)
+            grad_w = torch.cat([weight_gradient(x, grad_left), bottom], dim=0)
+        elif want_b:
             grad_b = g.sum(dim=0)
         if ctx.needs_input_grad[1]:
             if ctx.staged:

@@ -209,7 +209,8 @@ int gnnagg_wgrad_strided_f32(const float *x, int64_t x_stride, const float *g, i
  *                                                  operand of the input-gradient product)
  *   w_grad    = x^T @ grad_z
  * in one pass over x, g and y.  y = NULL: no ReLU / dropout behind the product (pre = g *
- * scale).  Needs fi, fo <= 256 and multiples of 4, 16-byte aligned
+ * scale); grad_z = NULL: not written (a caller that only wants w_grad and bias_grad, e.g.
+ * the SAGE layer's `+ bias`, model/layers/sageconv.py:91).  Needs fi, fo <= 256 and multiples of 4, 16-byte aligned
  * operands and row strides; workspace of gnnagg_wgrad_relu_dropout_backward_workspace_bytes
  * (0 = unsupported shape) bytes, nothing is allocated.  Deterministic.
  * The reference leaves these products to torch's Linear and runs dropout / ReLU as separate

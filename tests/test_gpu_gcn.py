@@ -255,3 +255,23 @@ def test_fused_layer_rejects_unsupported_shapes():
     rc = L.gnnagg_linear_bias_relu_dropout_f32(_lib.ptr(x), 20, _lib.ptr(w), 32, None, None, None, 1.0, 0, _lib.ptr(y), 32,
                                                64, 20, 32, _lib.current_stream(x.device))
     assert rc == _lib.ERR_UNSUPPORTED
+
+
+@pytest.mark.parametrize("rows,fi,fo", [(70_001, 256, 172), (999, 40, 48), (128, 64, 64), (1, 4, 4), (5000, 128, 256)])
+def test_weight_and_bias_gradient_in_one_pass(rows, fi, fo):
+    """x^T @ g and the column sums of g from one pass over g; x may be a column block of a wider array."""
+    gen = torch.Generator(device="cuda").manual_seed(rows + fi + fo)
+    wide = torch.randn(rows, 2 * fi, device="cuda", generator=gen)
+    g = torch.randn(rows, fo, device="cuda", generator=gen)
+    for x in (wide[:, :fi], wide[:, fi:]):
+        gw, gb = gcn.weight_and_bias_gradient(x, g)
+        assert torch.equal(gw, gcn.weight_gradient(x, g))  # the same MFMA chain
+        want = g.double().sum(0)
+        bound = 4e-7 * g.double().abs().sum(0) + 1e-6
+        assert bool(((gb.double() - want).abs() <= bound).all())
+        assert torch.equal(gb, gcn.weight_and_bias_gradient(x, g)[1])
+    # a shape the kernel does not take falls back to torch ops
+    x = torch.randn(64, 6, device="cuda", generator=gen)
+    g6 = torch.randn(64, 6, device="cuda", generator=gen)
+    gw, gb = gcn.weight_and_bias_gradient(x, g6)
+    assert torch.allclose(gw, x.t() @ g6, rtol=1e-5, atol=1e-5) and torch.allclose(gb, g6.sum(0), rtol=1e-5, atol=1e-5)
