@@ -152,6 +152,9 @@ class _FusedLayer(torch.autograd.Function):
         if row_div is not None and (row_div.dtype != torch.float32 or row_div.numel() != rows
                                     or not row_div.is_contiguous()):
             raise RuntimeError("Input mismatch: row_div must be contiguous float32 with one entry per row")
+        if keep_bits is not None and not relu:
+            # the gradient reads which units count off the output (y > 0), which needs the ReLU in front
+            raise RuntimeError("Input mismatch: the fused layer applies dropout behind a ReLU only")
         w = w.contiguous()
         y = torch.empty(rows, n, dtype=torch.float32, device=x.device)
         with torch.cuda.device(x.device):
@@ -159,7 +162,7 @@ class _FusedLayer(torch.autograd.Function):
                 _lib.ptr(x), _row_stride(x), _lib.ptr(w), n, _lib.ptr(bias.contiguous()), _lib.ptr(keep_bits),
                 _lib.ptr(row_div), float(scale), 1 if relu else 0, _lib.ptr(y), n, rows, k, n,
                 _lib.current_stream(x.device)))
-        ctx.save_for_backward(x, w, y if relu or keep_bits is not None else None)
+        ctx.save_for_backward(x, w, y if relu else None)
         ctx.scale = float(scale)
         ctx.row_div = row_div
         return y

@@ -3,7 +3,7 @@ record them into a HIP graph (here through torch.cuda.CUDAGraph, whose capture s
 picks up as the current stream) and replay it.  One graph holds the plan SpMM with a very long row
 (block-per-row kernel on the plan's side stream, forked and joined with events), the transposed
 product, the strided product, the row gather, the codec, the bf16 conversions, both fused
-epilogues and the weight gradient; it is replayed several times, with eager work and host
+epilogues, the weight gradient, and the one-kernel dense layer with its one-pass gradient; it is replayed several times, with eager work and host
 synchronisation in between, and every replay must reproduce the eager results bit for bit."""
 import numpy as np
 import pytest
@@ -32,6 +32,9 @@ def test_entry_points_replay_from_a_hip_graph(monkeypatch):
     beta = torch.randn(feat, device="cuda", generator=gen)
     bias = torch.randn(feat, device="cuda", generator=gen)
     index = torch.randint(0, n, (777,), device="cuda", generator=gen)
+    weight = torch.randn(feat, feat, device="cuda", generator=gen) / 8
+    keep_bits = gcn.pack_keep_mask(keep)
+    div = torch.randint(1, 9, (n,), device="cuda", generator=gen).float()
     work_range = torch.tensor([0, 1000, 1000, n], dtype=torch.int32)
     packed_rows = sum(-(-s // (8 // bits)) for s in (1000, 0, n - 1000))
 
@@ -46,6 +49,9 @@ def test_entry_points_replay_from_a_hip_graph(monkeypatch):
         cat = sage._DropoutLayerNormRelu.apply(wide[:, :feat].contiguous(), keep, 2.0, gamma, beta, 1e-5)
         act = gcn._BiasReluDropout.apply(out * 1.0, bias, keep, 2.0, None)
         w = gcn.weight_gradient(x, cat[:, feat:])
+        x_in, w_in, b_in = (t.detach().clone().requires_grad_() for t in (x, weight, bias))
+        layer = gcn._FusedLayer.apply(x_in, w_in, b_in, keep_bits, 2.0, div, True)
+        layer.backward(dx)
         rows = torch.empty(index.numel(), feat, device="cuda")
         _gather_rows(act, index, rows)
         packed = torch.empty((packed_rows, feat), dtype=torch.uint8, device="cuda")
@@ -58,7 +64,8 @@ def test_entry_points_replay_from_a_hip_graph(monkeypatch):
         wire = torch.empty(n, feat, device="cuda")
         _convert(half, wire)
         # (the left half of `cat` is scratch for a following layer and is never written here)
-        return [out, dx, wide, cat[:, feat:], act, w, rows, packed, params, back, wire]
+        return [out, dx, wide, cat[:, feat:], act, w, rows, packed, params, back, wire, layer.detach(), x_in.grad,
+                w_in.grad, b_in.grad]
 
     eager = [t.clone() for t in work()]
     torch.cuda.synchronize()

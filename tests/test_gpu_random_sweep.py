@@ -197,3 +197,51 @@ def test_random_fused_layernorm_passes_match_torch(seed):
         if bool(clear.all()):
             for got_p, want_p in ((g_in.grad, g_ref.grad), (b_in.grad, b_ref.grad)):
                 assert float((got_p.double().cpu() - want_p).abs().max()) <= 2e-4 * (float(want_p.abs().max()) + 1.0), what
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_random_fused_layer_kernels_match_fp64(seed):
+    """The one-kernel dense layer (product, degree division, bias, ReLU, dropout bits) and its one-pass
+    gradient (mask, division, bias and weight gradients) over random row counts, widths, row strides and
+    option sets, against fp64 torch ops on the units the kernel found active."""
+    rng = np.random.default_rng(23000 + seed)
+    for case in range(14):
+        rows = int(rng.choice([1, 5, 127, 128, 129, 1000, 4097, 20011]))
+        k = 16 * int(rng.integers(1, 17))
+        n = 4 * int(rng.integers(1, 65))
+        pad = 4 * int(rng.integers(0, 3))
+        wide = dev(rng.standard_normal((rows, k + 2 * pad)).astype(np.float32))
+        x = wide[:, pad:pad + k]
+        w = dev((rng.standard_normal((k, n)) / np.sqrt(k)).astype(np.float32))
+        bias = dev(rng.standard_normal(n).astype(np.float32))
+        with_div, with_mask, relu = (bool(v) for v in rng.integers(0, 2, 3))
+        relu = relu or with_mask  # dropout comes behind a ReLU (the gradient reads the mask off the output)
+        p = float(rng.choice([0.2, 0.5]))
+        div = dev(rng.integers(1, 30, rows).astype(np.float32)) if with_div else None
+        keep = dev(rng.random((rows, n)) >= p) if with_mask else None
+        scale = 1.0 / (1.0 - p) if with_mask else 1.0
+        g = dev(rng.standard_normal((rows, n)).astype(np.float32))
+        what = dict(seed=seed, case=case, rows=rows, k=k, n=n, pad=pad, div=with_div, mask=with_mask, relu=relu)
+        assert gcn.fused_layer_supported(x, k, n), what
+
+        x_in, w_in, b_in = x.detach().clone().requires_grad_(), w.clone().requires_grad_(), bias.clone().requires_grad_()
+        view = wide.clone()[:, pad:pad + k].requires_grad_() if pad else x_in
+        y = gcn._FusedLayer.apply(gcn._kernel_ready(view), w_in, b_in, gcn.pack_keep_mask(keep) if with_mask else None,
+                                  scale, div, relu)
+        y.backward(g)
+        z = x.double() @ w.double()
+        if with_div:
+            z = z / div.double().view(-1, 1)
+        z = z + bias.double()
+        ref = torch.relu(z) if relu else z
+        if with_mask:
+            ref = ref * keep * scale
+        row_scale = (x.double().abs() @ w.double().abs() + bias.double().abs()).clamp(min=1.0) * scale
+        assert bool(((y.double() - ref).abs() <= 1e-5 * row_scale).all()), what
+        active = (y.detach() > 0).double() if relu else torch.ones_like(z)
+        pre = g.double() * active * scale
+        gz = pre / div.double().view(-1, 1) if with_div else pre
+        for got, want, name in ((view.grad, gz @ w.double().t(), "x"), (w_in.grad, x.double().t() @ gz, "w"),
+                                (b_in.grad, pre.sum(0), "bias")):
+            size = float(want.abs().max()) + 1e-12
+            assert float((got.double() - want).abs().max()) <= 2e-5 * size, (name, what)
