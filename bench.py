@@ -593,12 +593,12 @@ def run_c5(args, graph):
     # the two GEMM variants with dense hidden activations, then the same with the hidden activations
     # kept packed (non-zero values + bitmap), which the next layer's aggregation gathers instead,
     # then with the narrowing last layer multiplying before it aggregates (A (x W) instead of (A x) W)
-    # (fp32 layers with dense activations run as one libgnnagg kernel each way; "separate_kernels" is the
+    # (layers with dense activations run as one libgnnagg kernel each way; "separate_kernels" is the
     # same model with the BLAS product and the elementwise passes apart)
     for gemm, packed_activations, linear_first, fused in (
             ("fp32", False, False, True), ("fp32", False, False, False), ("bf16", False, False, True),
             ("fp32", True, False, True), ("bf16", True, False, True), ("fp32", False, True, True),
-            ("fp32", True, True, True), ("bf16", True, True, True)):
+            ("bf16", False, True, True), ("fp32", True, True, True), ("bf16", True, True, True)):
         torch.manual_seed(args.seed)
         model = gcn.GCN(dims, gemm=gemm, packed_activations=packed_activations,
                         linear_first_when_narrowing=linear_first, fused_layers=fused).to(dev)

@@ -37,6 +37,7 @@ EXPORTS = (
     "gnnagg_linear_shape_supported",
     "gnnagg_pack_keep_bits",
     "gnnagg_linear_bias_relu_dropout_f32",
+    "gnnagg_linear_bias_relu_dropout_bf16_f32",
     "gnnagg_wgrad_relu_dropout_backward_workspace_bytes",
     "gnnagg_wgrad_relu_dropout_backward_f32",
     "gnnagg_dropout_layernorm_relu_blocks",
@@ -132,6 +133,8 @@ def lib() -> ctypes.CDLL:
     L.gnnagg_linear_bias_relu_dropout_f32.restype = i32
     L.gnnagg_linear_bias_relu_dropout_f32.argtypes = [vp, i64, vp, i64, vp, vp, vp, ctypes.c_float, i32, vp, i64, i64,
                                                       i64, i64, vp]
+    L.gnnagg_linear_bias_relu_dropout_bf16_f32.restype = i32
+    L.gnnagg_linear_bias_relu_dropout_bf16_f32.argtypes = L.gnnagg_linear_bias_relu_dropout_f32.argtypes
     L.gnnagg_wgrad_relu_dropout_backward_workspace_bytes.restype = i64
     L.gnnagg_wgrad_relu_dropout_backward_workspace_bytes.argtypes = [i64, i64, i64]
     L.gnnagg_wgrad_relu_dropout_backward_f32.restype = i32

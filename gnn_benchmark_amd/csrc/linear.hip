@@ -15,6 +15,13 @@
 // four consecutive values of its row with one 16-byte LDS read and spends them on four
 // MFMAs (lanes 0-31 hold k+0..3, lanes 32-63 k+4..7 of each group of eight: the order of
 // the contraction is permuted, the same way for both operands).
+//
+// The BF16 form rounds both operands to bf16 (round to nearest even, in hardware) on their way into
+// LDS and multiplies with v_mfma_f32_32x32x8_bf16 (fp32 accumulation): a lane's four consecutive
+// values of a row are then one 8-byte operand.  W is staged transposed for that ([column][k]): a
+// thread loads a 4 x 4 block of it and writes four 8-byte column pieces.  The matrix work shrinks
+// to a fraction of the time the operands take to stream in, so this form is HBM-bound
+// (4 * rows * (K + N) bytes).
 #include "common.h"
 #include "dense_tiles.h"
 
@@ -43,13 +50,33 @@ struct LinearShape {
     static constexpr int kVecB = WN * kChunk / 16;   // float4 per thread per chunk of W
     static constexpr int kBufFloats = kRows * kLda + kChunk * kLdb;
     static constexpr int kSmemFloats = 2 * kBufFloats + 256 * 4;
+    // BF16 form: rows of A and columns of W staged as kChunk bf16 + 8 bytes of padding each
+    static constexpr int kLdh = 2 * kChunk + 8;      // bytes between staged rows / columns
+    static constexpr int kBufBytesH = (kRows + 64 * WN) * kLdh;
+    static constexpr int kSmemBytesH = 2 * kBufBytesH;
 };
 
-template <int WM, int WN>
+typedef short shortx4 __attribute__((ext_vector_type(4)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+// four fp32 values -> four bf16 (round to nearest even) in 8 bytes
+__device__ inline shortx4 to_bf16x4(float a, float b, float c, float d) {
+    union {
+        bf16x2 h[2];
+        shortx4 s;
+    } u;
+    u.h[0] = __builtin_convertvector(floatx2{a, b}, bf16x2);
+    u.h[1] = __builtin_convertvector(floatx2{c, d}, bf16x2);
+    return u.s;
+}
+
+template <int WM, int WN, bool BF16>
 __global__ __launch_bounds__(256, 2) void linear_kernel(const LinearArgs p) {
     using S = LinearShape<WM, WN>;
     extern __shared__ __align__(16) float smem[];
-    float *dump = smem + 2 * S::kBufFloats + 4 * (int)threadIdx.x;
+    float *dump = smem + 2 * S::kBufFloats + 4 * (int)threadIdx.x;  // (fp32 form only)
+    char *smem_h = reinterpret_cast<char *>(smem);                  // (BF16 form)
 
     const int tid = (int)threadIdx.x;
     const int lane = tid & 63;
@@ -81,7 +108,9 @@ __global__ __launch_bounds__(256, 2) void linear_kernel(const LinearArgs p) {
     const float *ap[S::kVecA];
     int a_dst[S::kVecA];
 #pragma unroll
-    for (int j = 0; j < S::kVecA; ++j) a_dst[j] = ((tid >> 2) + 64 * j) * S::kLda + 4 * (tid & 3);
+    for (int j = 0; j < S::kVecA; ++j)
+        a_dst[j] = BF16 ? ((tid >> 2) + 64 * j) * S::kLdh + 8 * (tid & 3)      // bytes
+                        : ((tid >> 2) + 64 * j) * S::kLda + 4 * (tid & 3);     // floats
     auto enter_tile = [&](int64_t t) {
 #pragma unroll
         for (int j = 0; j < S::kVecA; ++j) {
@@ -95,16 +124,72 @@ __global__ __launch_bounds__(256, 2) void linear_kernel(const LinearArgs p) {
 #pragma unroll
         for (int j = 0; j < S::kVecA; ++j) areg[j] = *reinterpret_cast<const floatx4 *>(ap[j] + k0);
     };
-    auto store_a = [&](float *buf) {
+    auto store_a = [&](int buf) {
 #pragma unroll
-        for (int j = 0; j < S::kVecA; ++j) *reinterpret_cast<floatx4 *>(buf + a_dst[j]) = areg[j];
+        for (int j = 0; j < S::kVecA; ++j) {
+            if (BF16)
+                *reinterpret_cast<shortx4 *>(smem_h + buf * S::kBufBytesH + a_dst[j]) =
+                    to_bf16x4(areg[j].x, areg[j].y, areg[j].z, areg[j].w);
+            else
+                *reinterpret_cast<floatx4 *>(smem + buf * S::kBufFloats + a_dst[j]) = areg[j];
+        }
     };
     ChunkLoader<S::kVecB, S::kLdb> lw;
-    lw.init(tid, p.n, p.ldw);
+    if (!BF16) lw.init(tid, p.n, p.ldw);
+    // BF16: thread u owns the 4 x 4 block (k-quad u / (n/4), column-quad u % (n/4)) of a chunk of W; threads
+    // past the 4 * (n/4) blocks repeat earlier ones (same values to the same place)
+    floatx4 wreg[4];
+    int w_src = 0, w_dst = 0;
+    if (BF16) {
+        const int nq = p.n / 4;
+        const int u = tid % (4 * nq);
+        w_src = 4 * (u / nq) * p.ldw + 4 * (u % nq);
+        w_dst = S::kRows * S::kLdh + 4 * (u % nq) * S::kLdh + 8 * (u / nq);
+    }
+    auto fetch_w = [&](const float *wc) {
+        if (BF16) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) wreg[c] = *reinterpret_cast<const floatx4 *>(wc + w_src + c * p.ldw);
+        } else {
+            lw.fetch_cached(wc);
+        }
+    };
+    auto store_w = [&](int buf) {
+        if (BF16) {
+            char *dst = smem_h + buf * S::kBufBytesH + w_dst;
+#pragma unroll
+            for (int c = 0; c < 4; ++c)  // column 4 q + c of the block: its four consecutive k
+                *reinterpret_cast<shortx4 *>(dst + c * S::kLdh) = to_bf16x4(wreg[0][c], wreg[1][c], wreg[2][c], wreg[3][c]);
+        } else {
+            lw.store_all(smem + buf * S::kBufFloats + S::kRows * S::kLda, dump);
+        }
+    };
 
     // Columns past n of a staged row of W are never written: whatever they hold only reaches
     // accumulator entries that are never stored.
     auto multiply = [&](int buf) {
+        if (BF16) {
+            const char *ah = smem_h + buf * S::kBufBytesH + (m0 + idx) * S::kLdh + 8 * kk;
+            const char *wh = smem_h + buf * S::kBufBytesH + S::kRows * S::kLdh + (n0 + idx) * S::kLdh + 8 * kk;
+            shortx4 ha[2][WM], hb[2][WN];
+            auto read = [&](int s) {
+#pragma unroll
+                for (int i = 0; i < WM; ++i) ha[s][i] = *reinterpret_cast<const shortx4 *>(ah + 32 * i * S::kLdh + 16 * s);
+#pragma unroll
+                for (int j = 0; j < WN; ++j) hb[s][j] = *reinterpret_cast<const shortx4 *>(wh + 32 * j * S::kLdh + 16 * s);
+            };
+            read(0);
+            read(1);
+#pragma unroll
+            for (int s = 0; s < kChunk / 8; ++s) {
+#pragma unroll
+                for (int i = 0; i < WM; ++i)
+#pragma unroll
+                    for (int j = 0; j < WN; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(hb[s][j], ha[s][i], acc[i][j], 0, 0, 0);
+            }
+            return;
+        }
         const float *as = smem + buf * S::kBufFloats + (m0 + idx) * S::kLda + 4 * kk;
         const float *bs = smem + buf * S::kBufFloats + S::kRows * S::kLda + 4 * kk * S::kLdb + n0 + idx;
         floatx4 av[2][WM];
@@ -190,22 +275,21 @@ __global__ __launch_bounds__(256, 2) void linear_kernel(const LinearArgs p) {
     enter_tile(tile);
     load_divisors(tile);
     fetch_a(0);
-    lw.fetch_cached(p.w);
-    store_a(smem);
-    lw.store_all(smem + S::kRows * S::kLda, dump);
+    fetch_w(p.w);
+    store_a(0);
+    store_w(0);
     __syncthreads();
     int buf = 0;
     for (;;) {
         const float *wc = p.w;
         for (int c = 1; c < chunks; ++c) {
             wc += wstep;
-            lw.fetch_cached(wc);
+            fetch_w(wc);
             fetch_a(c * kChunk);
             __builtin_amdgcn_sched_barrier(0);  // keep the loads ahead of the MFMAs
             multiply(buf);
-            float *next = smem + (buf ^ 1) * S::kBufFloats;
-            store_a(next);
-            lw.store_all(next + S::kRows * S::kLda, dump);
+            store_a(buf ^ 1);
+            store_w(buf ^ 1);
             __syncthreads();
             buf ^= 1;
         }
@@ -214,15 +298,14 @@ __global__ __launch_bounds__(256, 2) void linear_kernel(const LinearArgs p) {
         const bool more = tile < tiles;
         if (more) {
             enter_tile(tile);
-            lw.fetch_cached(p.w);
+            fetch_w(p.w);
             fetch_a(0);
         }
         __builtin_amdgcn_sched_barrier(0);
         multiply(buf);
         if (more) {
-            float *next = smem + (buf ^ 1) * S::kBufFloats;
-            store_a(next);
-            lw.store_all(next + S::kRows * S::kLda, dump);
+            store_a(buf ^ 1);
+            store_w(buf ^ 1);
         }
         __builtin_amdgcn_sched_barrier(0);
         finish_tile(done);
@@ -235,28 +318,29 @@ __global__ __launch_bounds__(256, 2) void linear_kernel(const LinearArgs p) {
     }
 }
 
-template <int WM, int WN>
+template <int WM, int WN, bool BF16>
 int launch_linear(const LinearArgs &p, hipStream_t st) {
     using S = LinearShape<WM, WN>;
-    constexpr size_t smem = (size_t)S::kSmemFloats * sizeof(float);
-    GNNAGG_HIP(allow_lds(reinterpret_cast<const void *>(&linear_kernel<WM, WN>), smem));
+    constexpr size_t smem = BF16 ? (size_t)S::kSmemBytesH : (size_t)S::kSmemFloats * sizeof(float);
+    GNNAGG_HIP(allow_lds(reinterpret_cast<const void *>(&linear_kernel<WM, WN, BF16>), smem));
     int dev = 0, cus = 0;
     GNNAGG_HIP(hipGetDevice(&dev));
     GNNAGG_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
     const int64_t tiles = (p.rows + S::kRows - 1) / S::kRows;
     const int64_t resident = 2 * (int64_t)(cus > 0 ? cus : 256);  // two blocks per CU, each walks its share of the tiles
     const unsigned blocks = (unsigned)(tiles < resident ? tiles : resident);
-    hipLaunchKernelGGL((linear_kernel<WM, WN>), dim3(blocks), dim3(256), smem, st, p);
+    hipLaunchKernelGGL((linear_kernel<WM, WN, BF16>), dim3(blocks), dim3(256), smem, st, p);
     GNNAGG_HIP(hipGetLastError());
     return GNNAGG_OK;
 }
 
+template <bool BF16>
 int dispatch_linear(const LinearArgs &p, hipStream_t st) {
     switch ((p.n + 63) / 64) {
-        case 1: return launch_linear<2, 1>(p, st);
-        case 2: return launch_linear<2, 2>(p, st);
-        case 3: return launch_linear<2, 3>(p, st);
-        default: return launch_linear<2, 4>(p, st);
+        case 1: return launch_linear<2, 1, BF16>(p, st);
+        case 2: return launch_linear<2, 2, BF16>(p, st);
+        case 3: return launch_linear<2, 3, BF16>(p, st);
+        default: return launch_linear<2, 4, BF16>(p, st);
     }
 }
 
@@ -312,15 +396,34 @@ extern "C" int gnnagg_pack_keep_bits(const void *keep, uint32_t *bits, int64_t r
     return GNNAGG_OK;
 }
 
-extern "C" int gnnagg_linear_bias_relu_dropout_f32(const float *x, int64_t x_stride, const float *w, int64_t w_stride,
-                                                   const float *bias, const uint32_t *keep_bits, const float *row_div,
-                                                   float scale, int relu, float *y, int64_t y_stride, int64_t rows,
-                                                   int64_t k, int64_t n, void *stream) {
+namespace {
+int run_linear(bool bf16, const float *x, int64_t x_stride, const float *w, int64_t w_stride, const float *bias,
+               const uint32_t *keep_bits, const float *row_div, float scale, int relu, float *y, int64_t y_stride,
+               int64_t rows, int64_t k, int64_t n, void *stream) {
     GNNAGG_REQUIRE(x_stride < (1 << 27) && w_stride < (1 << 27) && y_stride < (1 << 27) && k < (1 << 27) && n < (1 << 27),
                    "sizes and row strides must be below 2^27");
     LinearArgs p{x, row_div, w, bias, keep_bits, y, rows, (int)x_stride, (int)w_stride, (int)y_stride, (int)k, (int)n,
                  scale, relu};
     if (int rc = check_linear(p)) return rc;
     if (rows == 0) return GNNAGG_OK;
-    return dispatch_linear(p, static_cast<hipStream_t>(stream));
+    return bf16 ? dispatch_linear<true>(p, static_cast<hipStream_t>(stream))
+                : dispatch_linear<false>(p, static_cast<hipStream_t>(stream));
+}
+}  // namespace
+
+extern "C" int gnnagg_linear_bias_relu_dropout_f32(const float *x, int64_t x_stride, const float *w, int64_t w_stride,
+                                                   const float *bias, const uint32_t *keep_bits, const float *row_div,
+                                                   float scale, int relu, float *y, int64_t y_stride, int64_t rows,
+                                                   int64_t k, int64_t n, void *stream) {
+    return run_linear(false, x, x_stride, w, w_stride, bias, keep_bits, row_div, scale, relu, y, y_stride, rows, k, n,
+                      stream);
+}
+
+extern "C" int gnnagg_linear_bias_relu_dropout_bf16_f32(const float *x, int64_t x_stride, const float *w,
+                                                        int64_t w_stride, const float *bias, const uint32_t *keep_bits,
+                                                        const float *row_div, float scale, int relu, float *y,
+                                                        int64_t y_stride, int64_t rows, int64_t k, int64_t n,
+                                                        void *stream) {
+    return run_linear(true, x, x_stride, w, w_stride, bias, keep_bits, row_div, scale, relu, y, y_stride, rows, k, n,
+                      stream);
 }

@@ -10,11 +10,12 @@ with a precomputed seeded mask, log-softmax + NLL on the labelled nodes, Adam.  
 forward and input-gradient products run on the matrix cores through the BLAS library
 behind ``torch.mm`` (fp32, or bf16 inputs with fp32 accumulation and fp32 output); the
 weight gradient -- a reduction over millions of rows into at most 256 x 256 outputs, the
-library's weakest shape -- runs in libgnnagg's own fp32 MFMA kernel.  With fp32 products and
-dense activations a layer whose widths the kernels take runs fused (``_FusedLayer``): the
-product, the degree division, bias, ReLU and dropout are one libgnnagg kernel, and in the
-gradient direction the ReLU / dropout mask, the degree division, the bias gradient and the
-weight gradient are another; only the input-gradient product stays with the BLAS library.
+library's weakest shape -- runs in libgnnagg's own fp32 MFMA kernel.  With dense
+activations a layer whose widths the kernels take runs fused (``_FusedLayer``): the
+product (fp32, or bf16 inputs), the degree division, bias, ReLU and dropout are one libgnnagg
+kernel, and in the gradient direction the ReLU / dropout mask, the degree division, the bias
+gradient and the weight gradient are another; the fp32 input-gradient product stays with the
+BLAS library, the bf16-input one is the same libgnnagg product kernel.
 """
 from typing import List, Optional, Sequence
 
@@ -136,14 +137,29 @@ def _kernel_ready(x: torch.Tensor) -> torch.Tensor:
     return x.contiguous()
 
 
+def _fused_product(x, w, bias, keep_bits, row_div, scale, relu, bf16):
+    """The one-kernel layer product of libgnnagg on kernel-ready operands."""
+    rows, k, n = x.size(0), x.size(1), w.size(1)
+    y = torch.empty(rows, n, dtype=torch.float32, device=x.device)
+    L = _lib.lib()
+    entry = L.gnnagg_linear_bias_relu_dropout_bf16_f32 if bf16 else L.gnnagg_linear_bias_relu_dropout_f32
+    with torch.cuda.device(x.device):
+        _lib.check(entry(_lib.ptr(x), _row_stride(x), _lib.ptr(w), n, _lib.ptr(bias), _lib.ptr(keep_bits),
+                         _lib.ptr(row_div), float(scale), 1 if relu else 0, _lib.ptr(y), n, rows, k, n,
+                         _lib.current_stream(x.device)))
+    return y
+
+
 class _FusedLayer(torch.autograd.Function):
     """y = relu((x @ w) / row_div + bias) * (keep ? scale : 0) in one kernel (``relu`` False and
     ``keep_bits`` None: y = (x @ w) / row_div + bias, the last layer).  The gradient direction
     is one more kernel -- mask, degree division, bias gradient and weight gradient in a single
-    pass over x, the incoming gradient and y -- plus the BLAS product for the input gradient."""
+    pass over x, the incoming gradient and y -- plus the product for the input gradient.  With
+    ``bf16`` the forward and input-gradient products round their operands to bf16 (fp32
+    accumulation); the weight gradient reads the fp32 operands as they are."""
 
     @staticmethod
-    def forward(ctx, x, w, bias, keep_bits, scale, row_div, relu):
+    def forward(ctx, x, w, bias, keep_bits, scale, row_div, relu, bf16=False):
         rows, k, n = x.size(0), x.size(1), w.size(1)
         if keep_bits is not None and (keep_bits.dtype != torch.int32 or keep_bits.shape != (rows, (n + 31) // 32)
                                       or not keep_bits.is_contiguous()):
@@ -156,15 +172,11 @@ class _FusedLayer(torch.autograd.Function):
             # the gradient reads which units count off the output (y > 0), which needs the ReLU in front
             raise RuntimeError("Input mismatch: the fused layer applies dropout behind a ReLU only")
         w = w.contiguous()
-        y = torch.empty(rows, n, dtype=torch.float32, device=x.device)
-        with torch.cuda.device(x.device):
-            _lib.check(_lib.lib().gnnagg_linear_bias_relu_dropout_f32(
-                _lib.ptr(x), _row_stride(x), _lib.ptr(w), n, _lib.ptr(bias.contiguous()), _lib.ptr(keep_bits),
-                _lib.ptr(row_div), float(scale), 1 if relu else 0, _lib.ptr(y), n, rows, k, n,
-                _lib.current_stream(x.device)))
+        y = _fused_product(x, w, bias.contiguous(), keep_bits, row_div, scale, relu, bf16)
         ctx.save_for_backward(x, w, y if relu else None)
         ctx.scale = float(scale)
         ctx.row_div = row_div
+        ctx.bf16 = bool(bf16)
         return y
 
     @staticmethod
@@ -175,7 +187,8 @@ class _FusedLayer(torch.autograd.Function):
         L = _lib.lib()
         workspace = torch.empty(int(L.gnnagg_wgrad_relu_dropout_backward_workspace_bytes(max(rows, 1), k, n)) // 4,
                                 dtype=torch.float32, device=x.device)
-        grad_z = torch.empty(rows, n, dtype=torch.float32, device=x.device)
+        want_x = ctx.needs_input_grad[0]
+        grad_z = torch.empty(rows, n, dtype=torch.float32, device=x.device) if want_x else None
         grad_w = torch.empty(k, n, dtype=torch.float32, device=x.device)
         grad_bias = torch.empty(n, dtype=torch.float32, device=x.device)
         with torch.cuda.device(x.device):
@@ -183,8 +196,15 @@ class _FusedLayer(torch.autograd.Function):
                 _lib.ptr(x), _row_stride(x), _lib.ptr(grad_y), _row_stride(grad_y), _lib.ptr(y),
                 n if y is not None else 0, _lib.ptr(ctx.row_div), ctx.scale, _lib.ptr(grad_z), _lib.ptr(grad_w),
                 _lib.ptr(grad_bias), _lib.ptr(workspace), rows, k, n, _lib.current_stream(x.device)))
-        grad_x = torch.mm(grad_z, w.t()) if ctx.needs_input_grad[0] else None
-        return grad_x, grad_w, grad_bias, None, None, None, None
+        grad_x = None
+        if want_x:
+            if not ctx.bf16:
+                grad_x = torch.mm(grad_z, w.t())
+            elif L.gnnagg_linear_shape_supported(n, k):
+                grad_x = _fused_product(grad_z, w.t().contiguous(), None, None, None, 1.0, False, True)
+            else:
+                grad_x = _Bf16InputLinear._mm(grad_z, w.t())
+        return grad_x, grad_w, grad_bias, None, None, None, None, None
 
 
 class _BiasReluDropout(torch.autograd.Function):
@@ -308,14 +328,14 @@ class GCNLayer(torch.nn.Module):
 
     def fused(self, graph, x, layer: int, is_pre_delay: bool, keep_bits, scale: float, relu: bool):
         """relu(((A x) W) / deg + bias) * keep * scale through the fused kernels, or None where they do
-        not apply (bf16 products, packed input, product-first order, widths the kernels do not take)."""
-        if self.gemm != "fp32" or self.linear_first or isinstance(x, tuple) or not self.fuse:
+        not apply (packed input, product-first order, widths the kernels do not take)."""
+        if self.linear_first or isinstance(x, tuple) or not self.fuse:
             return None
         if not fused_layer_supported(x, self.weight.size(0), self.weight.size(1)):
             return None
         agg = _kernel_ready(Aggregator.apply(graph, x, layer, 32, is_pre_delay, self.training))
         row_div = graph.in_degrees.reshape(-1)
-        return _FusedLayer.apply(agg, self.weight, self.bias, keep_bits, scale, row_div, relu)
+        return _FusedLayer.apply(agg, self.weight, self.bias, keep_bits, scale, row_div, relu, self.gemm == "bf16")
 
     def forward(self, graph, x: torch.Tensor, layer: int, is_pre_delay: bool) -> torch.Tensor:
         """((A x) W) / deg + bias."""

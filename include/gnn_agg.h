@@ -223,6 +223,12 @@ int gnnagg_linear_bias_relu_dropout_f32(const float *x, int64_t x_stride, const 
                                         const float *bias, const uint32_t *keep_bits, const float *row_div,
                                         float scale, int relu, float *y, int64_t y_stride, int64_t rows, int64_t k,
                                         int64_t n, void *stream);
+/* The same with both operands of the product rounded to bf16 (round to nearest even) on their way
+ * into the matrix units and fp32 accumulation: config 5's bf16-input variant.  HBM-bound. */
+int gnnagg_linear_bias_relu_dropout_bf16_f32(const float *x, int64_t x_stride, const float *w, int64_t w_stride,
+                                             const float *bias, const uint32_t *keep_bits, const float *row_div,
+                                             float scale, int relu, float *y, int64_t y_stride, int64_t rows,
+                                             int64_t k, int64_t n, void *stream);
 int64_t gnnagg_wgrad_relu_dropout_backward_workspace_bytes(int64_t rows, int64_t fi, int64_t fo);
 int gnnagg_wgrad_relu_dropout_backward_f32(const float *x, int64_t x_stride, const float *grad_y, int64_t grad_stride,
                                            const float *y, int64_t y_stride, const float *row_div, float scale,

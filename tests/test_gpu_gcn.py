@@ -66,7 +66,8 @@ class CpuBf16Linear(torch.autograd.Function):
         return _bf16_mm(g, w.t()), _bf16_mm(x.t(), g)
 
 
-@pytest.mark.parametrize("gemm,tol,fuse", [("fp32", 1e-4, True), ("fp32", 1e-4, False), ("bf16", 2e-2, True)])
+@pytest.mark.parametrize("gemm,tol,fuse", [("fp32", 1e-4, True), ("fp32", 1e-4, False), ("bf16", 2e-2, True),
+                                           ("bf16", 2e-2, False)])
 @pytest.mark.parametrize("linear_first", [False, True])
 def test_train_step_matches_cpu_autograd(gemm, tol, fuse, linear_first):
     dev = "cuda:0"
@@ -77,7 +78,7 @@ def test_train_step_matches_cpu_autograd(gemm, tol, fuse, linear_first):
     torch.manual_seed(0)
     model = gcn.GCN(dims, gemm=gemm, linear_first_when_narrowing=linear_first).to(dev)
     assert [layer.linear_first for layer in model.layers] == [False, False, linear_first]  # 32 -> 64 -> 64 -> 12
-    for layer in model.layers:  # fp32 layers that aggregate first run through the fused kernels unless told not to
+    for layer in model.layers:  # layers that aggregate first run through the fused kernels unless told not to
         layer.fuse = fuse
     cpu_model = copy.deepcopy(model).cpu()
     opt = torch.optim.Adam(model.parameters(), lr=0.01)
@@ -275,3 +276,29 @@ def test_weight_and_bias_gradient_in_one_pass(rows, fi, fo):
     g6 = torch.randn(64, 6, device="cuda", generator=gen)
     gw, gb = gcn.weight_and_bias_gradient(x, g6)
     assert torch.allclose(gw, x.t() @ g6, rtol=1e-5, atol=1e-5) and torch.allclose(gb, g6.sum(0), rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("rows,k,n", [(1000, 64, 32), (777, 128, 172), (4099, 256, 256), (130, 16, 4), (20_001, 128, 256)])
+def test_fused_layer_with_bf16_inputs(rows, k, n):
+    """The bf16-input form: operands rounded to bf16 (round to nearest even, as torch's .bfloat16()), exact
+    products, fp32 accumulation -- within 1e-5 of the fp64 product of the rounded operands; the input
+    gradient is the same kind of product of the masked gradient with w^T."""
+    gen = torch.Generator(device="cuda").manual_seed(rows + k + n)
+    x = torch.randn(rows, k, device="cuda", generator=gen)
+    w = torch.randn(k, n, device="cuda", generator=gen) / k ** 0.5
+    bias = torch.randn(n, device="cuda", generator=gen)
+    div = torch.randint(1, 9, (rows,), device="cuda", generator=gen).float()
+    keep = torch.rand(rows, n, device="cuda", generator=gen) >= 0.5
+    g = torch.randn(rows, n, device="cuda", generator=gen)
+    x_in, w_in, b_in = (t.detach().clone().requires_grad_() for t in (x, w, bias))
+    y = gcn._FusedLayer.apply(x_in, w_in, b_in, gcn.pack_keep_mask(keep), 2.0, div, True, True)
+    y.backward(g)
+    xb, wb = x.bfloat16().double(), w.bfloat16().double()
+    ref = torch.relu((xb @ wb) / div.double().view(-1, 1) + bias.double()) * keep * 2.0
+    row_scale = (xb.abs() @ wb.abs() + bias.double().abs()).clamp(min=1.0) * 2.0
+    assert bool(((y.double() - ref).abs() <= 1e-5 * row_scale).all())
+    gz = g.double() * (y.detach() > 0) * 2.0 / div.double().view(-1, 1)
+    want_x = gz.float().bfloat16().double() @ wb.t()          # the kernel rounds the fp32 masked gradient
+    assert float((x_in.grad.double() - want_x).abs().max()) <= 1e-4 * (float(want_x.abs().max()) + 1e-12)
+    want_w = x.double().t() @ gz                               # the weight gradient stays in fp32
+    assert float((w_in.grad.double() - want_w).abs().max()) <= 1e-5 * (float(want_w.abs().max()) + 1e-12)
