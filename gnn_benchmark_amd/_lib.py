@@ -40,6 +40,7 @@ EXPORTS = (
     "gnnagg_linear_bias_relu_dropout_bf16_f32",
     "gnnagg_wgrad_relu_dropout_backward_workspace_bytes",
     "gnnagg_wgrad_relu_dropout_backward_f32",
+    "gnnagg_wgrad_relu_dropout_backward_bf16_f32",
     "gnnagg_dropout_layernorm_relu_blocks",
     "gnnagg_dropout_layernorm_relu_f32",
     "gnnagg_dropout_layernorm_relu_backward_f32",
@@ -140,6 +141,8 @@ def lib() -> ctypes.CDLL:
     L.gnnagg_wgrad_relu_dropout_backward_f32.restype = i32
     L.gnnagg_wgrad_relu_dropout_backward_f32.argtypes = [vp, i64, vp, i64, vp, i64, vp, ctypes.c_float, vp, vp, vp, vp,
                                                          i64, i64, i64, vp]
+    L.gnnagg_wgrad_relu_dropout_backward_bf16_f32.restype = i32
+    L.gnnagg_wgrad_relu_dropout_backward_bf16_f32.argtypes = L.gnnagg_wgrad_relu_dropout_backward_f32.argtypes
     L.gnnagg_dropout_layernorm_relu_blocks.restype = i32
     L.gnnagg_dropout_layernorm_relu_blocks.argtypes = [i64, i64]
     L.gnnagg_dropout_layernorm_relu_f32.restype = i32

@@ -10,6 +10,21 @@ namespace gnnagg {
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
+typedef short shortx4 __attribute__((ext_vector_type(4)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+// four fp32 values -> four bf16 (round to nearest even, the hardware's packed conversion) in 8 bytes
+__device__ inline shortx4 to_bf16x4(float a, float b, float c, float d) {
+    union {
+        bf16x2 h[2];
+        shortx4 s;
+    } u;
+    u.h[0] = __builtin_convertvector(floatx2{a, b}, bf16x2);
+    u.h[1] = __builtin_convertvector(floatx2{c, d}, bf16x2);
+    return u.s;
+}
+
 constexpr int kChunk = 16;    // rows per LDS stage
 constexpr int kLdsPad = 32;   // floats: shifts the second row of a k-pair onto the other half of the banks
 

@@ -56,21 +56,6 @@ struct LinearShape {
     static constexpr int kSmemBytesH = 2 * kBufBytesH;
 };
 
-typedef short shortx4 __attribute__((ext_vector_type(4)));
-typedef float floatx2 __attribute__((ext_vector_type(2)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-
-// four fp32 values -> four bf16 (round to nearest even) in 8 bytes
-__device__ inline shortx4 to_bf16x4(float a, float b, float c, float d) {
-    union {
-        bf16x2 h[2];
-        shortx4 s;
-    } u;
-    u.h[0] = __builtin_convertvector(floatx2{a, b}, bf16x2);
-    u.h[1] = __builtin_convertvector(floatx2{c, d}, bf16x2);
-    return u.s;
-}
-
 template <int WM, int WN, bool BF16>
 __global__ __launch_bounds__(256, 2) void linear_kernel(const LinearArgs p) {
     using S = LinearShape<WM, WN>;

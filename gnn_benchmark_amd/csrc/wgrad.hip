@@ -280,6 +280,175 @@ __global__ __launch_bounds__(256) void wgrad_bias_reduce_kernel(const float *__r
     }
 }
 
+// ---- bf16-input form ---------------------------------------------------------------------------
+// The same product with both operands rounded to bf16 (round to nearest even) on their way into
+// LDS and v_mfma_f32_32x32x8_bf16 (fp32 accumulation).  The matrix work is then a fraction of the
+// time the operands take to stream in: this form is HBM-bound.  The MFMA wants, per lane, four
+// consecutive ROWS of one column (the contraction runs over rows), so a chunk is staged
+// transposed: a thread loads a 4 x 4 block (four rows, four columns: one float4 per row) and
+// writes four 8-byte column pieces, [column][16 rows as bf16 + 8 bytes of padding].  Rows past
+// the slice read the slice's last row and count as zeros, so there is no separate tail path.
+constexpr int kLdh = 2 * kChunk + 8;  // bytes between staged columns
+
+template <int WM, int WN, bool MASKED>
+__global__ __launch_bounds__(256, 1) void wgrad_bf16_partial_kernel(const float *__restrict__ x,
+                                                                    const float *__restrict__ g,
+                                                                    float *__restrict__ partial, int64_t rows, int fi,
+                                                                    int fo, int ldx, int ldg, int64_t rows_per_block,
+                                                                    const MaskArgs mk) {
+    extern __shared__ __align__(16) float smem[];
+    char *lds = reinterpret_cast<char *>(smem);
+    constexpr int kBufBytes = (64 * WM + 64 * WN) * kLdh;
+    constexpr int kGOff = 64 * WM * kLdh;
+
+    const int tid = (int)threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int kk = lane >> 5;
+    const int idx = lane & 31;
+    const int m0 = wm * 32 * WM, n0 = wn * 32 * WN;
+
+    floatx16 acc[WM][WN];
+#pragma unroll
+    for (int a = 0; a < WM; ++a)
+#pragma unroll
+        for (int b = 0; b < WN; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
+
+    const int64_t r_begin = (int64_t)blockIdx.x * rows_per_block;
+    int64_t r_end = r_begin + rows_per_block;
+    if (r_end > rows) r_end = rows;
+    const int64_t chunks = r_begin < r_end ? (r_end - r_begin + kChunk - 1) / kChunk : 0;
+
+    // thread u owns the block (row-quad u / (width/4), column-quad u % (width/4)) of each operand's chunk;
+    // threads past the 4 * (width/4) blocks repeat earlier ones (same values to the same place)
+    const int xq = fi / 4, gq = fo / 4;
+    const int ux = tid % (4 * xq), ug = tid % (4 * gq);
+    const int x_rq = ux / xq, x_cq = ux % xq, g_rq = ug / gq, g_cq = ug % gq;
+    const bool g_first = tid < 4 * gq;  // the one thread that accounts for its block of G
+    const int x_dst = 4 * x_cq * kLdh + 8 * x_rq;
+    const int g_dst = kGOff + 4 * g_cq * kLdh + 8 * g_rq;
+
+    floatx4 xr[4], gr[4], yr[4];
+    float dr[4];
+    floatx4 colsum = {0.f, 0.f, 0.f, 0.f};
+    const float *divp = MASKED ? (mk.row_div ? mk.row_div : x) : nullptr;  // any readable float per row without a divisor
+    const int64_t divstep = MASKED ? (mk.row_div ? 1 : ldx) : 0;
+    auto fetch = [&](int64_t r0) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            int64_t rx = r0 + 4 * x_rq + c, rg = r0 + 4 * g_rq + c;
+            if (rx >= r_end) rx = r_end - 1;
+            if (rg >= r_end) rg = r_end - 1;
+            xr[c] = __builtin_nontemporal_load(reinterpret_cast<const floatx4 *>(x + (size_t)rx * (size_t)ldx + 4 * x_cq));
+            gr[c] = __builtin_nontemporal_load(reinterpret_cast<const floatx4 *>(g + (size_t)rg * (size_t)ldg + 4 * g_cq));
+            if (MASKED) {
+                yr[c] = __builtin_nontemporal_load(
+                    reinterpret_cast<const floatx4 *>(mk.act + (size_t)rg * (size_t)mk.ldact + 4 * g_cq));
+                dr[c] = divp[rg * divstep];
+            }
+        }
+    };
+    auto stage = [&](int64_t r0, int buf) {
+        char *dst = lds + buf * kBufBytes;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const bool live_x = r0 + 4 * x_rq + c < r_end, live_g = r0 + 4 * g_rq + c < r_end;
+            if (!live_x) xr[c] = floatx4{0.f, 0.f, 0.f, 0.f};
+            if (MASKED) {
+                const bool all = mk.all_on != 0;
+                floatx4 pre;
+                pre.x = (live_g && (all || yr[c].x > 0.0f)) ? gr[c].x * mk.scale : 0.0f;
+                pre.y = (live_g && (all || yr[c].y > 0.0f)) ? gr[c].y * mk.scale : 0.0f;
+                pre.z = (live_g && (all || yr[c].z > 0.0f)) ? gr[c].z * mk.scale : 0.0f;
+                pre.w = (live_g && (all || yr[c].w > 0.0f)) ? gr[c].w * mk.scale : 0.0f;
+                if (g_first) colsum += pre;
+                const float inv = mk.row_div ? 1.0f / dr[c] : 1.0f;
+                pre *= inv;
+                gr[c] = pre;
+                if (live_g && g_first && mk.gz)
+                    __builtin_nontemporal_store(
+                        pre, reinterpret_cast<floatx4 *>(mk.gz + (size_t)(r0 + 4 * g_rq + c) * (size_t)fo + 4 * g_cq));
+            } else if (!live_g) {
+                gr[c] = floatx4{0.f, 0.f, 0.f, 0.f};
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {  // column 4 q + c of the block: its four consecutive rows
+            *reinterpret_cast<shortx4 *>(dst + x_dst + c * kLdh) = to_bf16x4(xr[0][c], xr[1][c], xr[2][c], xr[3][c]);
+            *reinterpret_cast<shortx4 *>(dst + g_dst + c * kLdh) = to_bf16x4(gr[0][c], gr[1][c], gr[2][c], gr[3][c]);
+        }
+    };
+    // Columns past fi / fo are never written: whatever they hold only reaches accumulator entries
+    // that are never stored.
+    auto multiply = [&](int buf) {
+        const char *xa = lds + buf * kBufBytes + (m0 + idx) * kLdh + 8 * kk;
+        const char *gb = lds + buf * kBufBytes + kGOff + (n0 + idx) * kLdh + 8 * kk;
+        shortx4 a[2][WM], b[2][WN];
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+#pragma unroll
+            for (int i = 0; i < WM; ++i) a[s][i] = *reinterpret_cast<const shortx4 *>(xa + 32 * i * kLdh + 16 * s);
+#pragma unroll
+            for (int j = 0; j < WN; ++j) b[s][j] = *reinterpret_cast<const shortx4 *>(gb + 32 * j * kLdh + 16 * s);
+        }
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+            for (int i = 0; i < WM; ++i)
+#pragma unroll
+                for (int j = 0; j < WN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(a[s][i], b[s][j], acc[i][j], 0, 0, 0);
+    };
+
+    if (chunks > 0) {
+        fetch(r_begin);
+        stage(r_begin, 0);
+        __syncthreads();
+        for (int64_t c = 1; c < chunks; ++c) {
+            const int64_t r0 = r_begin + c * kChunk;
+            fetch(r0);
+            __builtin_amdgcn_sched_barrier(0);  // keep the loads ahead of the MFMAs
+            multiply((int)((c - 1) & 1));
+            __builtin_amdgcn_sched_barrier(0);
+            stage(r0, (int)(c & 1));
+            __syncthreads();
+        }
+        multiply((int)((chunks - 1) & 1));
+    }
+
+    if (MASKED) reinterpret_cast<floatx4 *>(mk.bias_partial)[(size_t)blockIdx.x * 256 + tid] = g_first ? colsum : floatx4{0.f, 0.f, 0.f, 0.f};
+    // 32x32 accumulator layout: register r of lane l holds D[(r % 4) + 4 * (l / 32) + 8 * (r / 4)][l % 32]
+    float *out = partial + (size_t)blockIdx.x * (size_t)fi * (size_t)fo;
+#pragma unroll
+    for (int a = 0; a < WM; ++a)
+#pragma unroll
+        for (int b = 0; b < WN; ++b) {
+            const int n = n0 + b * 32 + idx;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = m0 + a * 32 + (r & 3) + 4 * kk + 8 * (r >> 2);
+                if (m < fi && n < fo) out[(size_t)m * fo + n] = acc[a][b][r];
+            }
+        }
+}
+
+// bias[n] for the bf16 form: thread u = rq * (fo/4) + cq of a block holds the sums of columns 4 cq .. 4 cq + 3 over
+// the rows 4 rq .. 4 rq + 3 of every chunk.  One thread per column, blocks then row-quads in order.
+__global__ __launch_bounds__(256) void wgrad_bias_reduce_quads_kernel(const float *__restrict__ partial,
+                                                                      float *__restrict__ bias, int blocks, int fo) {
+    const int n = (int)blockIdx.x * 256 + (int)threadIdx.x;
+    if (n >= fo) return;
+    const int gq = fo / 4;
+    float s[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int b = 0; b < blocks; ++b)
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq) s[rq] += partial[((size_t)b * 256 + rq * gq + n / 4) * 4 + (n & 3)];
+    bias[n] = (s[0] + s[1]) + (s[2] + s[3]);
+}
+
 int wgrad_blocks(int64_t rows) {
     int64_t b = 256;  // one block of four waves per CU: each wave keeps a SIMD's MFMA unit busy
     if (b * 64 > rows) b = rows / 64 > 0 ? rows / 64 : 1;
@@ -304,7 +473,8 @@ extern "C" int gnnagg_wgrad_f32(const float *x, const float *g, float *w_grad, v
 namespace {
 
 int run_wgrad(const float *x, int64_t x_stride, const float *g, int64_t g_stride, float *w_grad, void *workspace,
-              int64_t rows, int64_t fi, int64_t fo, void *stream, const MaskArgs *mask, float *bias_grad) {
+              int64_t rows, int64_t fi, int64_t fo, void *stream, const MaskArgs *mask, float *bias_grad,
+              bool bf16 = false) {
     GNNAGG_REQUIRE(rows >= 0 && fi > 0 && fo > 0, "bad size");
     GNNAGG_REQUIRE(x_stride >= fi && g_stride >= fo && x_stride < (int64_t(1) << 27) && g_stride < (int64_t(1) << 27),
                    "row strides %lld / %lld must be at least the widths %lld / %lld and below 2^27",
@@ -351,10 +521,17 @@ int run_wgrad(const float *x, int64_t x_stride, const float *g, int64_t g_stride
         hipLaunchKernelGGL((wgrad_partial_kernel<M, N, MASKED>), dim3((unsigned)blocks), dim3(256), smem, st, x, g, \
                            partial, rows, (int)fi, (int)fo, (int)x_stride, (int)g_stride, rpb, aligned, mk);    \
     }
-#define GNNAGG_WGRAD(M, N)                         \
-    if (wm == M && wn == N) {                      \
-        if (mask) GNNAGG_WGRAD_FORM(M, N, true)    \
-        else GNNAGG_WGRAD_FORM(M, N, false)        \
+#define GNNAGG_WGRAD_BF16(M, N)                                                                                  \
+    {                                                                                                           \
+        constexpr size_t smem = (size_t)2 * (64 * M + 64 * N) * kLdh;                                            \
+        hipLaunchKernelGGL((wgrad_bf16_partial_kernel<M, N, true>), dim3((unsigned)blocks), dim3(256), smem, st, x, \
+                           g, partial, rows, (int)fi, (int)fo, (int)x_stride, (int)g_stride, rpb, mk);           \
+    }
+#define GNNAGG_WGRAD(M, N)                          \
+    if (wm == M && wn == N) {                       \
+        if (bf16) GNNAGG_WGRAD_BF16(M, N)           \
+        else if (mask) GNNAGG_WGRAD_FORM(M, N, true) \
+        else GNNAGG_WGRAD_FORM(M, N, false)         \
     } else
     GNNAGG_WGRAD(1, 1) GNNAGG_WGRAD(1, 2) GNNAGG_WGRAD(1, 3) GNNAGG_WGRAD(1, 4) GNNAGG_WGRAD(2, 1) GNNAGG_WGRAD(2, 2)
     GNNAGG_WGRAD(2, 3) GNNAGG_WGRAD(2, 4) GNNAGG_WGRAD(3, 1) GNNAGG_WGRAD(3, 2) GNNAGG_WGRAD(3, 3) GNNAGG_WGRAD(3, 4)
@@ -363,11 +540,15 @@ int run_wgrad(const float *x, int64_t x_stride, const float *g, int64_t g_stride
     }
 #undef GNNAGG_WGRAD
 #undef GNNAGG_WGRAD_FORM
+#undef GNNAGG_WGRAD_BF16
     GNNAGG_HIP(hipGetLastError());
     const int count = (int)(fi * fo);
     hipLaunchKernelGGL(wgrad_reduce_kernel, dim3((unsigned)((count + kReduceOutputs - 1) / kReduceOutputs)), dim3(256), 0,
                        st, partial, w_grad, blocks, count);
-    if (mask)
+    if (mask && bf16)
+        hipLaunchKernelGGL(wgrad_bias_reduce_quads_kernel, dim3(grid_for(fo, 256)), dim3(256), 0, st, mk.bias_partial,
+                           bias_grad, blocks, (int)fo);
+    else if (mask)
         hipLaunchKernelGGL(wgrad_bias_reduce_kernel, dim3(grid_for(fo, 16)), dim3(256), 0, st, mk.bias_partial, bias_grad,
                            blocks, wn * 256, (int)fo);
     GNNAGG_HIP(hipGetLastError());
@@ -398,4 +579,15 @@ extern "C" int gnnagg_wgrad_relu_dropout_backward_f32(const float *x, int64_t x_
     // without y the kernel reads g a second time in its place (a cache hit) and ignores the values
     MaskArgs mk{y ? y : grad_y, row_div, grad_z, nullptr, (int)(y ? y_stride : grad_stride), scale, y ? 0 : 1};
     return run_wgrad(x, x_stride, grad_y, grad_stride, w_grad, workspace, rows, fi, fo, stream, &mk, bias_grad);
+}
+
+extern "C" int gnnagg_wgrad_relu_dropout_backward_bf16_f32(const float *x, int64_t x_stride, const float *grad_y,
+                                                           int64_t grad_stride, const float *y, int64_t y_stride,
+                                                           const float *row_div, float scale, float *grad_z,
+                                                           float *w_grad, float *bias_grad, void *workspace, int64_t rows,
+                                                           int64_t fi, int64_t fo, void *stream) {
+    GNNAGG_REQUIRE(bias_grad, "null bias_grad");
+    GNNAGG_REQUIRE(!y || (y_stride >= fo && y_stride < (int64_t(1) << 27)), "bad row stride of y");
+    MaskArgs mk{y ? y : grad_y, row_div, grad_z, nullptr, (int)(y ? y_stride : grad_stride), scale, y ? 0 : 1};
+    return run_wgrad(x, x_stride, grad_y, grad_stride, w_grad, workspace, rows, fi, fo, stream, &mk, bias_grad, true);
 }

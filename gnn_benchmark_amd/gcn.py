@@ -155,8 +155,8 @@ class _FusedLayer(torch.autograd.Function):
     ``keep_bits`` None: y = (x @ w) / row_div + bias, the last layer).  The gradient direction
     is one more kernel -- mask, degree division, bias gradient and weight gradient in a single
     pass over x, the incoming gradient and y -- plus the product for the input gradient.  With
-    ``bf16`` the forward and input-gradient products round their operands to bf16 (fp32
-    accumulation); the weight gradient reads the fp32 operands as they are."""
+    ``bf16`` all three products round their operands to bf16 on the way into the matrix units
+    (fp32 accumulation); mask, division and bias gradient stay in fp32."""
 
     @staticmethod
     def forward(ctx, x, w, bias, keep_bits, scale, row_div, relu, bf16=False):
@@ -191,11 +191,12 @@ class _FusedLayer(torch.autograd.Function):
         grad_z = torch.empty(rows, n, dtype=torch.float32, device=x.device) if want_x else None
         grad_w = torch.empty(k, n, dtype=torch.float32, device=x.device)
         grad_bias = torch.empty(n, dtype=torch.float32, device=x.device)
+        entry = L.gnnagg_wgrad_relu_dropout_backward_bf16_f32 if ctx.bf16 else L.gnnagg_wgrad_relu_dropout_backward_f32
         with torch.cuda.device(x.device):
-            _lib.check(L.gnnagg_wgrad_relu_dropout_backward_f32(
-                _lib.ptr(x), _row_stride(x), _lib.ptr(grad_y), _row_stride(grad_y), _lib.ptr(y),
-                n if y is not None else 0, _lib.ptr(ctx.row_div), ctx.scale, _lib.ptr(grad_z), _lib.ptr(grad_w),
-                _lib.ptr(grad_bias), _lib.ptr(workspace), rows, k, n, _lib.current_stream(x.device)))
+            _lib.check(entry(_lib.ptr(x), _row_stride(x), _lib.ptr(grad_y), _row_stride(grad_y), _lib.ptr(y),
+                             n if y is not None else 0, _lib.ptr(ctx.row_div), ctx.scale, _lib.ptr(grad_z),
+                             _lib.ptr(grad_w), _lib.ptr(grad_bias), _lib.ptr(workspace), rows, k, n,
+                             _lib.current_stream(x.device)))
         grad_x = None
         if want_x:
             if not ctx.bf16:

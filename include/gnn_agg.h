@@ -230,10 +230,17 @@ int gnnagg_linear_bias_relu_dropout_bf16_f32(const float *x, int64_t x_stride, c
                                              float scale, int relu, float *y, int64_t y_stride, int64_t rows,
                                              int64_t k, int64_t n, void *stream);
 int64_t gnnagg_wgrad_relu_dropout_backward_workspace_bytes(int64_t rows, int64_t fi, int64_t fo);
+/* (the _bf16_ form below takes the same arguments and workspace; it rounds x and grad_z to bf16 for the
+ * product x^T @ grad_z -- fp32 accumulation -- while grad_z and bias_grad are computed and written in fp32) */
 int gnnagg_wgrad_relu_dropout_backward_f32(const float *x, int64_t x_stride, const float *grad_y, int64_t grad_stride,
                                            const float *y, int64_t y_stride, const float *row_div, float scale,
                                            float *grad_z, float *w_grad, float *bias_grad, void *workspace,
                                            int64_t rows, int64_t fi, int64_t fo, void *stream);
+int gnnagg_wgrad_relu_dropout_backward_bf16_f32(const float *x, int64_t x_stride, const float *grad_y,
+                                                int64_t grad_stride, const float *y, int64_t y_stride,
+                                                const float *row_div, float scale, float *grad_z, float *w_grad,
+                                                float *bias_grad, void *workspace, int64_t rows, int64_t fi, int64_t fo,
+                                                void *stream);
 
 /* ---------------------------------------------------------------------------------
  * The elementwise chain between two SAGE layers (model/DistSAGE.py:49-53: F.dropout, LayerNorm

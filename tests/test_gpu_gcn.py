@@ -300,5 +300,7 @@ def test_fused_layer_with_bf16_inputs(rows, k, n):
     gz = g.double() * (y.detach() > 0) * 2.0 / div.double().view(-1, 1)
     want_x = gz.float().bfloat16().double() @ wb.t()          # the kernel rounds the fp32 masked gradient
     assert float((x_in.grad.double() - want_x).abs().max()) <= 1e-4 * (float(want_x.abs().max()) + 1e-12)
-    want_w = x.double().t() @ gz                               # the weight gradient stays in fp32
-    assert float((w_in.grad.double() - want_w).abs().max()) <= 1e-5 * (float(want_w.abs().max()) + 1e-12)
+    want_w = xb.t() @ gz.float().bfloat16().double()          # ... and so does the weight gradient
+    assert float((w_in.grad.double() - want_w).abs().max()) <= 1e-4 * (float(want_w.abs().max()) + 1e-12)
+    want_b = (g.double() * (y.detach() > 0) * 2.0).sum(0)      # the bias gradient is summed in fp32
+    assert float((b_in.grad.double() - want_b).abs().max()) <= 1e-5 * (float(want_b.abs().max()) + 1e-12)
