@@ -206,12 +206,20 @@ __global__ __launch_bounds__(256, 2) void linear_kernel(const LinearArgs p) {
 
     // 32x32 accumulator layout: register r of lane l holds D[(r % 4) + 4 * (l / 32) + 8 * (r / 4)][l % 32]
     const int words = (p.n + 31) / 32;  // keep-bit words per row
-    float rdiv[WM];                     // this lane's row divisors: loaded when a tile starts, used when it ends
+    // this lane's row divisors and keep-bit words: loaded when a tile starts, used when it ends
+    float rdiv[WM];
+    uint32_t kbits[WM][WN];
     auto load_divisors = [&](int64_t t) {
 #pragma unroll
         for (int i = 0; i < WM; ++i) {
             const int64_t m = t * S::kRows + m0 + 32 * i + idx;
-            rdiv[i] = (p.row_div && m < p.rows) ? p.row_div[m] : 1.0f;
+            const bool live = m < p.rows;
+            rdiv[i] = (p.row_div && live) ? p.row_div[m] : 1.0f;
+#pragma unroll
+            for (int j = 0; j < WN; ++j) {
+                const int nt = n0 + 32 * j;
+                kbits[i][j] = (p.keep && live && nt < p.n) ? p.keep[(size_t)m * (size_t)words + (nt >> 5)] : 0xffffffffu;
+            }
         }
     };
     auto finish_tile = [&](int64_t t) {
@@ -224,9 +232,7 @@ __global__ __launch_bounds__(256, 2) void linear_kernel(const LinearArgs p) {
 #pragma unroll
             for (int j = 0; j < WN; ++j) {
                 const int nt = n0 + 32 * j;
-                uint32_t bits = 0xffffffffu;
-                if (p.keep && live && nt < p.n) bits = p.keep[(size_t)m * (size_t)words + (nt >> 5)];
-                bits >>= 4 * kk;
+                const uint32_t bits = kbits[i][j] >> (4 * kk);
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
                     const int n = nt + 8 * g + 4 * kk;
