@@ -110,7 +110,8 @@ def test_train_step_with_packed_activations_equals_dense():
     train_idx = torch.randperm(3000, device="cuda", generator=gen)[:600]
     masks = gcn.make_dropout_masks(3000, dims, 0.5, seed=8, device="cuda")
     torch.manual_seed(0)
-    dense_model = gcn.GCN(dims, gemm="fp32", dropout=0.5).cuda()
+    # (like with like: both models on the separate product / epilogue kernels, whose roundings the packed form shares)
+    dense_model = gcn.GCN(dims, gemm="fp32", dropout=0.5, fused_layers=False).cuda()
     packed_model = copy.deepcopy(dense_model)
     packed_model.packed_activations = True
     results = []
