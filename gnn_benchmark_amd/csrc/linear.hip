@@ -1,27 +1,30 @@
 // Dense layer product with the elementwise work behind it fused in,
+//
+//     Y[rows, N] = epilogue( A[rows, K] @ W[K, N] ),
+//
 // for rows in the millions and K, N <= 256 (fp32 MFMA, v_mfma_f32_32x32x2f32; 2*rows*K*N flop
 // against the 157.3 TFLOP/s fp32 matrix peak).  The epilogue divides row r by row_div[r],
 // adds the bias, applies ReLU and the dropout keep-bits while the result is still in the
 // accumulators, so the layer needs no elementwise pass over its [rows, N] result.
 //
-//     Y[rows, N] = epilogue( A[rows, K] @ W[K, N] )
-//
 // A block of four waves (2 x 2) owns 64*WM rows and all N <= 64*WN columns at a time and
 // walks its share of the row tiles; two blocks share a CU, so that one block's epilogue
-// overlaps the other's MFMAs.  The contraction runs in chunks of 16: 64*WM x 16 values of A (a 64-byte piece of each row) and 16 x N
-// values of W are copied into LDS through registers, the next chunk in flight behind the
-// MFMAs of the current one.  A is row-major with the contraction index contiguous, while
-// the MFMA wants one contraction index per lane across 32 rows; each lane therefore reads
-// four consecutive values of its row with one 16-byte LDS read and spends them on four
-// MFMAs (lanes 0-31 hold k+0..3, lanes 32-63 k+4..7 of each group of eight: the order of
-// the contraction is permuted, the same way for both operands).
+// overlaps the other's MFMAs.  The contraction runs in chunks of 16: 64*WM x 16 values of A
+// (a 64-byte piece of each row) and 16 x N values of W are copied into LDS through registers,
+// the next chunk -- of this tile or the next -- in flight behind the MFMAs of the current one.
+// A is row-major with the contraction index contiguous, while the MFMA wants one contraction
+// index per lane across 32 rows; each lane therefore reads four consecutive values of its row
+// with one 16-byte LDS read and spends them on four MFMAs (lanes 0-31 hold k+0..3, lanes 32-63
+// k+4..7 of each group of eight: the order of the contraction is permuted, the same way for
+// both operands).  W is the MFMA's A operand, so the accumulators hold tiles of Y^T and a lane
+// owns runs of four consecutive columns of one row of Y: 16-byte stores.
 //
-// The BF16 form rounds both operands to bf16 (round to nearest even, in hardware) on their way into
-// LDS and multiplies with v_mfma_f32_32x32x8_bf16 (fp32 accumulation): a lane's four consecutive
-// values of a row are then one 8-byte operand.  W is staged transposed for that ([column][k]): a
-// thread loads a 4 x 4 block of it and writes four 8-byte column pieces.  The matrix work shrinks
-// to a fraction of the time the operands take to stream in, so this form is HBM-bound
-// (4 * rows * (K + N) bytes).
+// The BF16 form rounds both operands to bf16 (round to nearest even, in hardware) on their way
+// into LDS and multiplies with v_mfma_f32_32x32x8_bf16 (fp32 accumulation): a lane's four
+// consecutive values of a row are then one 8-byte operand.  W is staged transposed for that
+// ([column][k]): a thread loads a 4 x 4 block of it and writes four 8-byte column pieces.  The
+// matrix work shrinks to a fraction of the time the operands take to stream in, so this form
+// is HBM-bound (4 * rows * (K + N) bytes).
 #include "common.h"
 #include "dense_tiles.h"
 
