@@ -34,7 +34,7 @@ struct WgradShape {
 // was inactive or dropped), adds pre up per column (the bias gradient), divides by row_div, uses
 // the result as the G operand and also writes it out for the input-gradient product.
 struct MaskArgs {
-    const float *act;       // y [rows, fo], row stride ldact; with all_on: any readable array of that shape
+    const float *act;       // y [rows, fo], row stride ldact; with all_on: any readable row of fo floats, ldact = 0
     const float *row_div;   // [rows] or nullptr
     float *gz;              // out: [rows, fo] contiguous, or nullptr (not wanted)
     float *bias_partial;    // out: [blocks][kVecG * 256] float4, the per-thread column sums
@@ -43,12 +43,16 @@ struct MaskArgs {
     int all_on;             // no ReLU / dropout behind the product: every entry counts
 };
 
-template <int WM, int WN, bool MASKED>
+// MODE 0: plain product.  MODE 1: the masked form above.  MODE 2: only the column sums of g * scale ride along (no
+// mask, no division, nothing written out): the bias gradient of a layer without ReLU / dropout behind its product.
+template <int WM, int WN, int MODE>
 __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__restrict__ x,
                                                                const float *__restrict__ g,
                                                                float *__restrict__ partial, int64_t rows, int fi,
                                                                int fo, int ldx, int ldg, int64_t rows_per_block,
                                                                int aligned, const MaskArgs mk) {
+    constexpr bool MASKED = MODE != 0;   // something rides along with G
+    constexpr bool FULL = MODE == 1;     // ... the whole mask pass
     using S = WgradShape<WM, WN>;
     extern __shared__ __align__(16) float smem[];
     float *xs = smem;                              // [2][kChunk][kLdx]
@@ -91,7 +95,7 @@ __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__re
     float dreg[S::kVecG];
     int grow[S::kVecG];  // row of vector j inside a chunk
     if (MASKED) {
-        lc.init(tid, fo, mk.ldact);
+        if (FULL) lc.init(tid, fo, mk.ldact);
 #pragma unroll
         for (int j = 0; j < S::kVecG; ++j) {
             colsum[j] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -99,8 +103,8 @@ __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__re
         }
     }
     // any readable float per row when there is no divisor (the value is not used then)
-    const float *divp = MASKED ? (mk.row_div ? mk.row_div : x) : nullptr;
-    const int64_t divstep = MASKED ? (mk.row_div ? 1 : ldx) : 0;
+    const float *divp = FULL ? (mk.row_div ? mk.row_div : x) : nullptr;
+    const int64_t divstep = FULL ? (mk.row_div ? 1 : ldx) : 0;
     auto fetch_divisors = [&](int64_t r, int64_t last) {  // rows r .. r+15, clamped to `last`
 #pragma unroll
         for (int j = 0; j < S::kVecG; ++j) {
@@ -109,30 +113,38 @@ __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__re
             dreg[j] = divp[row * divstep];
         }
     };
-    // turns lg.reg (g) into the G operand, with lc.reg = y; `valid` = number of values of the chunk that exist
+    // turns vector j of lg.reg (g) into the G operand, with lc.reg = y; `valid` = number of values of the chunk that exist
+    auto mask_piece = [&](int64_t r, int valid, int j) __attribute__((always_inline)) {
+        const bool used = lg.lds_off[j] >= 0 && lg.elem[j] < valid;
+        const floatx4 gv = lg.reg[j];
+        floatx4 pre;
+        if (!FULL) {  // column sums only: G itself stays the operand
+            pre = used ? gv * mk.scale : floatx4{0.f, 0.f, 0.f, 0.f};
+            colsum[j] += pre;
+            return;
+        }
+        const floatx4 yv = lc.reg[j];
+        const bool all = mk.all_on != 0;
+        pre.x = (used && (all || yv.x > 0.0f)) ? gv.x * mk.scale : 0.0f;
+        pre.y = (used && (all || yv.y > 0.0f)) ? gv.y * mk.scale : 0.0f;
+        pre.z = (used && (all || yv.z > 0.0f)) ? gv.z * mk.scale : 0.0f;
+        pre.w = (used && (all || yv.w > 0.0f)) ? gv.w * mk.scale : 0.0f;
+        colsum[j] += pre;
+        const float inv = mk.row_div ? 1.0f / dreg[j] : 1.0f;
+        pre *= inv;
+        lg.reg[j] = pre;
+        if (used && mk.gz)
+            __builtin_nontemporal_store(pre, reinterpret_cast<floatx4 *>(mk.gz + (size_t)r * (size_t)fo + lg.elem[j]));
+    };
     auto mask_g = [&](int64_t r, int valid) {
 #pragma unroll
-        for (int j = 0; j < S::kVecG; ++j) {
-            const bool used = lg.lds_off[j] >= 0 && lg.elem[j] < valid;
-            const floatx4 gv = lg.reg[j], yv = lc.reg[j];
-            floatx4 pre;
-            const bool all = mk.all_on != 0;
-            pre.x = (used && (all || yv.x > 0.0f)) ? gv.x * mk.scale : 0.0f;
-            pre.y = (used && (all || yv.y > 0.0f)) ? gv.y * mk.scale : 0.0f;
-            pre.z = (used && (all || yv.z > 0.0f)) ? gv.z * mk.scale : 0.0f;
-            pre.w = (used && (all || yv.w > 0.0f)) ? gv.w * mk.scale : 0.0f;
-            colsum[j] += pre;
-            const float inv = mk.row_div ? 1.0f / dreg[j] : 1.0f;
-            pre *= inv;
-            lg.reg[j] = pre;
-            if (used && mk.gz)
-                __builtin_nontemporal_store(pre, reinterpret_cast<floatx4 *>(mk.gz + (size_t)r * (size_t)fo + lg.elem[j]));
-        }
+        for (int j = 0; j < S::kVecG; ++j) mask_piece(r, valid, j);
     };
 
     // Columns past fi / fo of an LDS row are never written: whatever they hold only reaches
     // accumulator entries that are never stored.
-    auto multiply = [&](int buf) {
+    // `between(s)` runs behind the MFMAs of k-pair s: work that does not depend on them executes in their shadow
+    auto multiply_and = [&](int buf, auto between) __attribute__((always_inline)) {
         const float *xa = xs + buf * kChunk * S::kLdx + kk * S::kLdx + m0 + idx;
         const float *gb = gs + buf * kChunk * S::kLdg + kk * S::kLdg + n0 + idx;
         // operands of k-pair s+1 are read from LDS while the MFMAs of k-pair s run
@@ -153,9 +165,11 @@ __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__re
 #pragma unroll
                 for (int j = 0; j < WN; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s & 1][i], b[s & 1][j], acc[i][j], 0, 0, 0);
+            between(s);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
+    auto multiply = [&](int buf) { multiply_and(buf, [](int) {}); };
 
     // steady state: whole chunks, no masks; the next chunk's global loads are in flight behind
     // this chunk's MFMAs and land in the other LDS buffer
@@ -168,8 +182,10 @@ __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__re
         lx.fetch(xc);
         lg.fetch(gc);
         if (MASKED) {
-            lc.fetch(cc);
-            fetch_divisors(r_begin, r_end - 1);
+            if (FULL) {
+                lc.fetch(cc);
+                fetch_divisors(r_begin, r_end - 1);
+            }
             mask_g(r_begin, kChunk * fo);
         }
         lx.store_all(xs, dump);
@@ -182,13 +198,23 @@ __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__re
             lg.fetch(gc);
             if (MASKED) {
                 cc += cstep;
-                lc.fetch(cc);
-                fetch_divisors(r_begin + c * kChunk, r_end - 1);
+                if (FULL) {
+                    lc.fetch(cc);
+                    fetch_divisors(r_begin + c * kChunk, r_end - 1);
+                }
             }
             __builtin_amdgcn_sched_barrier(0);  // keep the loads ahead of the MFMAs
-            multiply((int)((c - 1) & 1));
+            if (MASKED) {
+                // the chunk's MFMAs cover the flight of the loads; the mask work on what they brought runs in
+                // the shadow of the last k-pair's MFMAs
+                const int64_t r = r_begin + c * kChunk;
+                multiply_and((int)((c - 1) & 1), [&](int s) __attribute__((always_inline)) {
+                    if (s == kChunk / 2 - 1) mask_g(r, kChunk * fo);
+                });
+            } else {
+                multiply((int)((c - 1) & 1));
+            }
             __builtin_amdgcn_sched_barrier(0);
-            if (MASKED) mask_g(r_begin + c * kChunk, kChunk * fo);
             lx.store_all(xs + (c & 1) * kChunk * S::kLdx, dump);
             lg.store_all(gs + (c & 1) * kChunk * S::kLdg, dump);
             __syncthreads();
@@ -202,8 +228,10 @@ __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__re
         lx.fetch_tail(x + (size_t)r * (size_t)ldx, left * fi, aligned != 0);
         lg.fetch_tail(g + (size_t)r * (size_t)ldg, left * fo, aligned != 0);
         if (MASKED) {  // the host only launches this form with 16-byte copies possible
-            lc.fetch_tail(mk.act + (size_t)r * (size_t)mk.ldact, left * fo, true);
-            fetch_divisors(r, r_end - 1);
+            if (FULL) {
+                lc.fetch_tail(mk.act + (size_t)r * (size_t)mk.ldact, left * fo, true);
+                fetch_divisors(r, r_end - 1);
+            }
             mask_g(r, left * fo);
         }
         lx.store(xs, aligned != 0);
@@ -514,6 +542,7 @@ int run_wgrad(const float *x, int64_t x_stride, const float *g, int64_t g_stride
     }
     // wave corner = 32*WM x 32*WN, block = 2 x 2 waves
     const int wm = (int)((fi + 63) / 64), wn = (int)((fo + 63) / 64);
+    const bool sums_only = mask && mk.all_on && !mk.row_div && !mk.gz;
 #define GNNAGG_WGRAD_FORM(M, N, MASKED)                                                                         \
     {                                                                                                           \
         constexpr size_t smem = (size_t)WgradShape<M, N>::kSmemFloats * sizeof(float);                          \
@@ -530,8 +559,9 @@ int run_wgrad(const float *x, int64_t x_stride, const float *g, int64_t g_stride
 #define GNNAGG_WGRAD(M, N)                          \
     if (wm == M && wn == N) {                       \
         if (bf16) GNNAGG_WGRAD_BF16(M, N)           \
-        else if (mask) GNNAGG_WGRAD_FORM(M, N, true) \
-        else GNNAGG_WGRAD_FORM(M, N, false)         \
+        else if (mask && sums_only) GNNAGG_WGRAD_FORM(M, N, 2) \
+        else if (mask) GNNAGG_WGRAD_FORM(M, N, 1)   \
+        else GNNAGG_WGRAD_FORM(M, N, 0)             \
     } else
     GNNAGG_WGRAD(1, 1) GNNAGG_WGRAD(1, 2) GNNAGG_WGRAD(1, 3) GNNAGG_WGRAD(1, 4) GNNAGG_WGRAD(2, 1) GNNAGG_WGRAD(2, 2)
     GNNAGG_WGRAD(2, 3) GNNAGG_WGRAD(2, 4) GNNAGG_WGRAD(3, 1) GNNAGG_WGRAD(3, 2) GNNAGG_WGRAD(3, 3) GNNAGG_WGRAD(3, 4)
@@ -576,8 +606,9 @@ extern "C" int gnnagg_wgrad_relu_dropout_backward_f32(const float *x, int64_t x_
                                                       int64_t fo, void *stream) {
     GNNAGG_REQUIRE(bias_grad, "null bias_grad");
     GNNAGG_REQUIRE(!y || (y_stride >= fo && y_stride < (int64_t(1) << 27)), "bad row stride of y");
-    // without y the kernel reads g a second time in its place (a cache hit) and ignores the values
-    MaskArgs mk{y ? y : grad_y, row_div, grad_z, nullptr, (int)(y ? y_stride : grad_stride), scale, y ? 0 : 1};
+    // without y the kernel reads the first row of g over and over in its place (row stride 0: a cache hit) and
+    // ignores the values
+    MaskArgs mk{y ? y : grad_y, row_div, grad_z, nullptr, (int)(y ? y_stride : 0), scale, y ? 0 : 1};
     return run_wgrad(x, x_stride, grad_y, grad_stride, w_grad, workspace, rows, fi, fo, stream, &mk, bias_grad);
 }
 
@@ -588,6 +619,6 @@ extern "C" int gnnagg_wgrad_relu_dropout_backward_bf16_f32(const float *x, int64
                                                            int64_t fi, int64_t fo, void *stream) {
     GNNAGG_REQUIRE(bias_grad, "null bias_grad");
     GNNAGG_REQUIRE(!y || (y_stride >= fo && y_stride < (int64_t(1) << 27)), "bad row stride of y");
-    MaskArgs mk{y ? y : grad_y, row_div, grad_z, nullptr, (int)(y ? y_stride : grad_stride), scale, y ? 0 : 1};
+    MaskArgs mk{y ? y : grad_y, row_div, grad_z, nullptr, (int)(y ? y_stride : 0), scale, y ? 0 : 1};
     return run_wgrad(x, x_stride, grad_y, grad_stride, w_grad, workspace, rows, fi, fo, stream, &mk, bias_grad, true);
 }
