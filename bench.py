@@ -593,27 +593,41 @@ def run_c5(args, graph):
     # the two GEMM variants with dense hidden activations, then the same with the hidden activations
     # kept packed (non-zero values + bitmap), which the next layer's aggregation gathers instead,
     # then with the narrowing last layer multiplying before it aggregates (A (x W) instead of (A x) W)
+    folded = None
     # (layers with dense activations run as one libgnnagg kernel each way; "separate_kernels" is the
     # same model with the BLAS product and the elementwise passes apart)
     for gemm, packed_activations, linear_first, fused in (
             ("fp32", False, False, True), ("fp32", False, False, False), ("bf16", False, False, True),
             ("fp32", True, False, True), ("bf16", True, False, True), ("fp32", False, True, True),
-            ("bf16", False, True, True), ("fp32", True, True, True), ("bf16", True, True, True)):
+            ("bf16", False, True, True), ("fp32", True, True, True), ("bf16", True, True, True),
+            ("fp32", True, True, "folded"), ("bf16", True, True, "folded")):
+        g = graph
+        if fused == "folded":  # the degree division carried by the matrix values instead of the layers' epilogues
+            if folded is None:
+                from gnn_benchmark_amd import sage
+                folded = sage.fold_in_degrees(graph)
+                for m in (folded.local_adj_t, folded.adj_t_pre_post_aggr_from):
+                    m.get_plan()
+                    m.get_plan_for_transpose()
+            g, fused = folded, True
+        folded_tag = "_folded_degrees" if g is not graph else ""
         torch.manual_seed(args.seed)
         model = gcn.GCN(dims, gemm=gemm, packed_activations=packed_activations,
                         linear_first_when_narrowing=linear_first, fused_layers=fused).to(dev)
         opt = torch.optim.Adam(model.parameters(), lr=0.01)
-        losses = [float(gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks)) for _ in range(2)]
+        losses = [float(gcn.train_step(model, opt, g, x, labels, train_idx, True, masks)) for _ in range(2)]
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(steps):
-            loss = gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks)
+            loss = gcn.train_step(model, opt, g, x, labels, train_idx, True, masks)
         torch.cuda.synchronize()
         tag = (f"{gemm}_gemm" + ("_packed_activations" if packed_activations else "")
-               + ("_linear_first_when_narrowing" if linear_first else "") + ("" if fused else "_separate_kernels"))
+               + ("_linear_first_when_narrowing" if linear_first else "") + ("" if fused else "_separate_kernels")
+               + folded_tag)
         out[f"train_step_ms_{tag}"] = round((time.perf_counter() - t0) * 1e3 / steps, 2)
         out[f"loss_{tag}"] = [round(v, 5) for v in losses + [float(loss)]]
         del model, opt
+    del folded
     return out
 
 

@@ -38,9 +38,11 @@ EXPORTS = (
     "gnnagg_pack_keep_bits",
     "gnnagg_linear_bias_relu_dropout_f32",
     "gnnagg_linear_bias_relu_dropout_bf16_f32",
+    "gnnagg_linear_bias_relu_dropout_pack_f32",
     "gnnagg_wgrad_relu_dropout_backward_workspace_bytes",
     "gnnagg_wgrad_relu_dropout_backward_f32",
     "gnnagg_wgrad_relu_dropout_backward_bf16_f32",
+    "gnnagg_wgrad_relu_dropout_backward_from_header_f32",
     "gnnagg_dropout_layernorm_relu_blocks",
     "gnnagg_dropout_layernorm_relu_f32",
     "gnnagg_dropout_layernorm_relu_backward_f32",
@@ -136,6 +138,9 @@ def lib() -> ctypes.CDLL:
                                                       i64, i64, vp]
     L.gnnagg_linear_bias_relu_dropout_bf16_f32.restype = i32
     L.gnnagg_linear_bias_relu_dropout_bf16_f32.argtypes = L.gnnagg_linear_bias_relu_dropout_f32.argtypes
+    L.gnnagg_linear_bias_relu_dropout_pack_f32.restype = i32
+    L.gnnagg_linear_bias_relu_dropout_pack_f32.argtypes = [vp, i64, vp, i64, vp, vp, vp, ctypes.c_float, vp, vp, i64, i64,
+                                                           i64, i32, vp]
     L.gnnagg_wgrad_relu_dropout_backward_workspace_bytes.restype = i64
     L.gnnagg_wgrad_relu_dropout_backward_workspace_bytes.argtypes = [i64, i64, i64]
     L.gnnagg_wgrad_relu_dropout_backward_f32.restype = i32
@@ -143,6 +148,9 @@ def lib() -> ctypes.CDLL:
                                                          i64, i64, i64, vp]
     L.gnnagg_wgrad_relu_dropout_backward_bf16_f32.restype = i32
     L.gnnagg_wgrad_relu_dropout_backward_bf16_f32.argtypes = L.gnnagg_wgrad_relu_dropout_backward_f32.argtypes
+    L.gnnagg_wgrad_relu_dropout_backward_from_header_f32.restype = i32
+    L.gnnagg_wgrad_relu_dropout_backward_from_header_f32.argtypes = [vp, i64, vp, i64, vp, vp, ctypes.c_float, vp, vp, vp,
+                                                                     vp, i64, i64, i64, i32, vp]
     L.gnnagg_dropout_layernorm_relu_blocks.restype = i32
     L.gnnagg_dropout_layernorm_relu_blocks.argtypes = [i64, i64]
     L.gnnagg_dropout_layernorm_relu_f32.restype = i32

@@ -38,6 +38,8 @@ struct LinearArgs {
     const float *bias;       // [N] or nullptr
     const uint32_t *keep;    // [rows, ceil(N/32)] keep-bits or nullptr
     float *y;                // [rows, N], row stride ldy
+    uint32_t *header;        // PACK: [rows, 2 * (N / 32)] (bitmap, non-zeros in front) pairs; y then holds each row's
+                             // non-zero values at its front
     int64_t rows;
     int lda, ldw, ldy, k, n;
     float scale;             // dropout scale of the epilogue
@@ -59,12 +61,14 @@ struct LinearShape {
     static constexpr int kSmemBytesH = 2 * kBufBytesH;
 };
 
-template <int WM, int WN, bool BF16>
+template <int WM, int WN, bool BF16, bool PACK>
 __global__ __launch_bounds__(256, 2) void linear_kernel(const LinearArgs p) {
     using S = LinearShape<WM, WN>;
     extern __shared__ __align__(16) float smem[];
     float *dump = smem + 2 * S::kBufFloats + 4 * (int)threadIdx.x;  // (fp32 form only)
     char *smem_h = reinterpret_cast<char *>(smem);                  // (BF16 form)
+    // PACK: non-zeros of each tile row in the block's left column half, behind the staging buffers
+    int *row_count = reinterpret_cast<int *>(smem_h + (BF16 ? (size_t)S::kSmemBytesH : (size_t)S::kSmemFloats * sizeof(float)));
 
     const int tid = (int)threadIdx.x;
     const int lane = tid & 63;
@@ -225,7 +229,7 @@ __global__ __launch_bounds__(256, 2) void linear_kernel(const LinearArgs p) {
             }
         }
     };
-    auto finish_tile = [&](int64_t t) {
+    auto finish_tile_dense = [&](int64_t t) {
 #pragma unroll
         for (int i = 0; i < WM; ++i) {
             const int64_t m = t * S::kRows + m0 + 32 * i + idx;
@@ -259,6 +263,74 @@ __global__ __launch_bounds__(256, 2) void linear_kernel(const LinearArgs p) {
                 }
             }
         }
+    };
+
+    // PACK: the same values, but every row keeps only its non-zeros, moved to its front in column order, and a
+    // header says where they belong: per 32 columns the bitmap of the non-zeros and the number of non-zeros in
+    // front of them.  Four lanes share a row (two per wave: columns 8g + 4kk + c of each 32-column tile; the block's
+    // two column halves in two waves), so ranks come from the tile bitmaps (exchanged between the two lanes), a
+    // running count over the wave's tiles, and the left half's total handed to the right half through LDS.
+    auto finish_tile_packed = [&](int64_t t) {
+        uint32_t word[WM][WN];
+#pragma unroll
+        for (int i = 0; i < WM; ++i) {
+            const int64_t m = t * S::kRows + m0 + 32 * i + idx;
+            const bool live = m < p.rows;
+            const float inv = 1.0f / rdiv[i];
+            int total = 0;
+#pragma unroll
+            for (int j = 0; j < WN; ++j) {
+                const int nt = n0 + 32 * j;
+                const uint32_t bits = kbits[i][j] >> (4 * kk);
+                uint32_t mine = 0;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int local = 8 * (r >> 2) + (r & 3);  // + 4 kk: this value's column inside the tile
+                    float v = acc[i][j][r] * inv;
+                    if (p.bias && nt < p.n) v += p.bias[nt + local + 4 * kk];
+                    v = fmaxf(v, 0.0f) * p.scale;
+                    if (!((bits >> local) & 1u) || !live || nt >= p.n) v = 0.0f;
+                    acc[i][j][r] = v;
+                    mine |= (v > 0.0f ? 1u : 0u) << local;
+                }
+                mine <<= 4 * kk;
+                word[i][j] = mine | (uint32_t)__shfl_xor((int)mine, 32);
+                total += __popc(word[i][j]);
+            }
+            if (wn == 0 && kk == 0) row_count[m0 + 32 * i + idx] = total;
+        }
+        __syncthreads();
+        const int hw = 2 * (p.n / 32);
+#pragma unroll
+        for (int i = 0; i < WM; ++i) {
+            const int64_t m = t * S::kRows + m0 + 32 * i + idx;
+            if (m >= p.rows) continue;
+            int front = wn == 1 ? row_count[m0 + 32 * i + idx] : 0;
+            float *yrow = p.y + (size_t)m * (size_t)p.ldy;
+            uint32_t *hrow = p.header + (size_t)m * (size_t)hw;
+#pragma unroll
+            for (int j = 0; j < WN; ++j) {
+                const int nt = n0 + 32 * j;
+                if (nt >= p.n) continue;
+                const uint32_t w = word[i][j];
+                if (kk == 0) {
+                    hrow[2 * (nt >> 5)] = w;
+                    hrow[2 * (nt >> 5) + 1] = (uint32_t)front;
+                }
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int local = 8 * (r >> 2) + (r & 3) + 4 * kk;
+                    if ((w >> local) & 1u) yrow[front + __popc(w & ((1u << local) - 1u))] = acc[i][j][r];
+                }
+                front += __popc(w);
+            }
+        }
+    };
+    auto finish_tile = [&](int64_t t) {
+        if (PACK)
+            finish_tile_packed(t);
+        else
+            finish_tile_dense(t);
     };
 
     // One stream of chunks over all tiles of this block: the first chunk of the next tile is in
@@ -312,29 +384,37 @@ __global__ __launch_bounds__(256, 2) void linear_kernel(const LinearArgs p) {
     }
 }
 
-template <int WM, int WN, bool BF16>
+template <int WM, int WN, bool BF16, bool PACK>
 int launch_linear(const LinearArgs &p, hipStream_t st) {
     using S = LinearShape<WM, WN>;
-    constexpr size_t smem = BF16 ? (size_t)S::kSmemBytesH : (size_t)S::kSmemFloats * sizeof(float);
-    GNNAGG_HIP(allow_lds(reinterpret_cast<const void *>(&linear_kernel<WM, WN, BF16>), smem));
+    constexpr size_t smem = (BF16 ? (size_t)S::kSmemBytesH : (size_t)S::kSmemFloats * sizeof(float)) +
+                            (PACK ? S::kRows * sizeof(int) : 0);
+    GNNAGG_HIP(allow_lds(reinterpret_cast<const void *>(&linear_kernel<WM, WN, BF16, PACK>), smem));
     int dev = 0, cus = 0;
     GNNAGG_HIP(hipGetDevice(&dev));
     GNNAGG_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
     const int64_t tiles = (p.rows + S::kRows - 1) / S::kRows;
     const int64_t resident = 2 * (int64_t)(cus > 0 ? cus : 256);  // two blocks per CU, each walks its share of the tiles
     const unsigned blocks = (unsigned)(tiles < resident ? tiles : resident);
-    hipLaunchKernelGGL((linear_kernel<WM, WN, BF16>), dim3(blocks), dim3(256), smem, st, p);
+    hipLaunchKernelGGL((linear_kernel<WM, WN, BF16, PACK>), dim3(blocks), dim3(256), smem, st, p);
     GNNAGG_HIP(hipGetLastError());
     return GNNAGG_OK;
 }
 
 template <bool BF16>
 int dispatch_linear(const LinearArgs &p, hipStream_t st) {
+    if (p.header) {  // packed output: widths 32, 64, 128, 256
+        switch ((p.n + 63) / 64) {
+            case 1: return launch_linear<2, 1, BF16, true>(p, st);
+            case 2: return launch_linear<2, 2, BF16, true>(p, st);
+            default: return launch_linear<2, 4, BF16, true>(p, st);
+        }
+    }
     switch ((p.n + 63) / 64) {
-        case 1: return launch_linear<2, 1, BF16>(p, st);
-        case 2: return launch_linear<2, 2, BF16>(p, st);
-        case 3: return launch_linear<2, 3, BF16>(p, st);
-        default: return launch_linear<2, 4, BF16>(p, st);
+        case 1: return launch_linear<2, 1, BF16, false>(p, st);
+        case 2: return launch_linear<2, 2, BF16, false>(p, st);
+        case 3: return launch_linear<2, 3, BF16, false>(p, st);
+        default: return launch_linear<2, 4, BF16, false>(p, st);
     }
 }
 
@@ -393,12 +473,16 @@ extern "C" int gnnagg_pack_keep_bits(const void *keep, uint32_t *bits, int64_t r
 namespace {
 int run_linear(bool bf16, const float *x, int64_t x_stride, const float *w, int64_t w_stride, const float *bias,
                const uint32_t *keep_bits, const float *row_div, float scale, int relu, float *y, int64_t y_stride,
-               int64_t rows, int64_t k, int64_t n, void *stream) {
+               uint32_t *header, int64_t rows, int64_t k, int64_t n, void *stream) {
     GNNAGG_REQUIRE(x_stride < (1 << 27) && w_stride < (1 << 27) && y_stride < (1 << 27) && k < (1 << 27) && n < (1 << 27),
                    "sizes and row strides must be below 2^27");
-    LinearArgs p{x, row_div, w, bias, keep_bits, y, rows, (int)x_stride, (int)w_stride, (int)y_stride, (int)k, (int)n,
-                 scale, relu};
+    LinearArgs p{x, row_div, w, bias, keep_bits, y, header, rows, (int)x_stride, (int)w_stride, (int)y_stride, (int)k,
+                 (int)n, scale, relu};
     if (int rc = check_linear(p)) return rc;
+    if (header && !(n == 32 || n == 64 || n == 128 || n == 256))
+        return fail(GNNAGG_ERR_UNSUPPORTED, "packed activations exist for widths 32, 64, 128, 256 (got %lld)", (long long)n);
+    if (header && (!relu || y_stride != n))
+        return fail(GNNAGG_ERR_INVALID, "packed output follows a ReLU and has row stride n");
     if (rows == 0) return GNNAGG_OK;
     return bf16 ? dispatch_linear<true>(p, static_cast<hipStream_t>(stream))
                 : dispatch_linear<false>(p, static_cast<hipStream_t>(stream));
@@ -409,8 +493,8 @@ extern "C" int gnnagg_linear_bias_relu_dropout_f32(const float *x, int64_t x_str
                                                    const float *bias, const uint32_t *keep_bits, const float *row_div,
                                                    float scale, int relu, float *y, int64_t y_stride, int64_t rows,
                                                    int64_t k, int64_t n, void *stream) {
-    return run_linear(false, x, x_stride, w, w_stride, bias, keep_bits, row_div, scale, relu, y, y_stride, rows, k, n,
-                      stream);
+    return run_linear(false, x, x_stride, w, w_stride, bias, keep_bits, row_div, scale, relu, y, y_stride, nullptr, rows,
+                      k, n, stream);
 }
 
 extern "C" int gnnagg_linear_bias_relu_dropout_bf16_f32(const float *x, int64_t x_stride, const float *w,
@@ -418,6 +502,16 @@ extern "C" int gnnagg_linear_bias_relu_dropout_bf16_f32(const float *x, int64_t 
                                                         const float *row_div, float scale, int relu, float *y,
                                                         int64_t y_stride, int64_t rows, int64_t k, int64_t n,
                                                         void *stream) {
-    return run_linear(true, x, x_stride, w, w_stride, bias, keep_bits, row_div, scale, relu, y, y_stride, rows, k, n,
-                      stream);
+    return run_linear(true, x, x_stride, w, w_stride, bias, keep_bits, row_div, scale, relu, y, y_stride, nullptr, rows,
+                      k, n, stream);
+}
+
+extern "C" int gnnagg_linear_bias_relu_dropout_pack_f32(const float *x, int64_t x_stride, const float *w, int64_t w_stride,
+                                                        const float *bias, const uint32_t *keep_bits,
+                                                        const float *row_div, float scale, float *y_packed,
+                                                        uint32_t *header, int64_t rows, int64_t k, int64_t n,
+                                                        int bf16_inputs, void *stream) {
+    GNNAGG_REQUIRE(header || rows == 0, "null header");
+    return run_linear(bf16_inputs != 0, x, x_stride, w, w_stride, bias, keep_bits, row_div, scale, 1, y_packed, n, header,
+                      rows, k, n, stream);
 }

@@ -41,10 +41,15 @@ struct MaskArgs {
     int ldact;
     float scale;
     int all_on;             // no ReLU / dropout behind the product: every entry counts
+    // alternative to act: one bit per unit (set = the unit was active); the word of columns 32 v .. 32 v + 31 of row
+    // r is bits[r * bits_stride + v * bits_step] (the header of packed activations: stride 2 * (fo / 32), step 2)
+    const uint32_t *bits;
+    int bits_stride, bits_step;
 };
 
 // MODE 0: plain product.  MODE 1: the masked form above.  MODE 2: only the column sums of g * scale ride along (no
 // mask, no division, nothing written out): the bias gradient of a layer without ReLU / dropout behind its product.
+// MODE 3: MODE 1 with the activity read from a bitmap (4 bytes per 32 units) instead of the activations themselves.
 template <int WM, int WN, int MODE>
 __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__restrict__ x,
                                                                const float *__restrict__ g,
@@ -52,7 +57,8 @@ __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__re
                                                                int fo, int ldx, int ldg, int64_t rows_per_block,
                                                                int aligned, const MaskArgs mk) {
     constexpr bool MASKED = MODE != 0;   // something rides along with G
-    constexpr bool FULL = MODE == 1;     // ... the whole mask pass
+    constexpr bool FULL = MODE == 1 || MODE == 3;  // ... the whole mask pass
+    constexpr bool BITS = MODE == 3;               // ... with the activity from a bitmap
     using S = WgradShape<WM, WN>;
     extern __shared__ __align__(16) float smem[];
     float *xs = smem;                              // [2][kChunk][kLdx]
@@ -94,12 +100,17 @@ __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__re
     floatx4 colsum[S::kVecG];
     float dreg[S::kVecG];
     int grow[S::kVecG];  // row of vector j inside a chunk
+    int bit_word[S::kVecG], bit_shift[S::kVecG];  // BITS: where the vector's four activity bits sit in its row's words
+    uint32_t breg[S::kVecG];
     if (MASKED) {
-        if (FULL) lc.init(tid, fo, mk.ldact);
+        if (FULL && !BITS) lc.init(tid, fo, mk.ldact);
 #pragma unroll
         for (int j = 0; j < S::kVecG; ++j) {
             colsum[j] = floatx4{0.f, 0.f, 0.f, 0.f};
             grow[j] = lg.elem[j] / fo;
+            const int col = lg.elem[j] % fo;
+            bit_word[j] = (col >> 5) * mk.bits_step;
+            bit_shift[j] = col & 31;
         }
     }
     // any readable float per row when there is no divisor (the value is not used then)
@@ -111,6 +122,7 @@ __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__re
             int64_t row = r + grow[j];
             if (row > last) row = last;
             dreg[j] = divp[row * divstep];
+            if (BITS) breg[j] = mk.bits[(size_t)row * (size_t)mk.bits_stride + bit_word[j]];
         }
     };
     // turns vector j of lg.reg (g) into the G operand, with lc.reg = y; `valid` = number of values of the chunk that exist
@@ -123,12 +135,20 @@ __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__re
             colsum[j] += pre;
             return;
         }
-        const floatx4 yv = lc.reg[j];
-        const bool all = mk.all_on != 0;
-        pre.x = (used && (all || yv.x > 0.0f)) ? gv.x * mk.scale : 0.0f;
-        pre.y = (used && (all || yv.y > 0.0f)) ? gv.y * mk.scale : 0.0f;
-        pre.z = (used && (all || yv.z > 0.0f)) ? gv.z * mk.scale : 0.0f;
-        pre.w = (used && (all || yv.w > 0.0f)) ? gv.w * mk.scale : 0.0f;
+        if (BITS) {
+            const uint32_t nib = breg[j] >> bit_shift[j];
+            pre.x = (used && (nib & 1u)) ? gv.x * mk.scale : 0.0f;
+            pre.y = (used && (nib & 2u)) ? gv.y * mk.scale : 0.0f;
+            pre.z = (used && (nib & 4u)) ? gv.z * mk.scale : 0.0f;
+            pre.w = (used && (nib & 8u)) ? gv.w * mk.scale : 0.0f;
+        } else {
+            const floatx4 yv = lc.reg[j];
+            const bool all = mk.all_on != 0;
+            pre.x = (used && (all || yv.x > 0.0f)) ? gv.x * mk.scale : 0.0f;
+            pre.y = (used && (all || yv.y > 0.0f)) ? gv.y * mk.scale : 0.0f;
+            pre.z = (used && (all || yv.z > 0.0f)) ? gv.z * mk.scale : 0.0f;
+            pre.w = (used && (all || yv.w > 0.0f)) ? gv.w * mk.scale : 0.0f;
+        }
         colsum[j] += pre;
         const float inv = mk.row_div ? 1.0f / dreg[j] : 1.0f;
         pre *= inv;
@@ -183,7 +203,7 @@ __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__re
         lg.fetch(gc);
         if (MASKED) {
             if (FULL) {
-                lc.fetch(cc);
+                if (!BITS) lc.fetch(cc);
                 fetch_divisors(r_begin, r_end - 1);
             }
             mask_g(r_begin, kChunk * fo);
@@ -199,7 +219,7 @@ __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__re
             if (MASKED) {
                 cc += cstep;
                 if (FULL) {
-                    lc.fetch(cc);
+                    if (!BITS) lc.fetch(cc);
                     fetch_divisors(r_begin + c * kChunk, r_end - 1);
                 }
             }
@@ -229,7 +249,7 @@ __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__re
         lg.fetch_tail(g + (size_t)r * (size_t)ldg, left * fo, aligned != 0);
         if (MASKED) {  // the host only launches this form with 16-byte copies possible
             if (FULL) {
-                lc.fetch_tail(mk.act + (size_t)r * (size_t)mk.ldact, left * fo, true);
+                if (!BITS) lc.fetch_tail(mk.act + (size_t)r * (size_t)mk.ldact, left * fo, true);
                 fetch_divisors(r, r_end - 1);
             }
             mask_g(r, left * fo);
@@ -318,7 +338,7 @@ __global__ __launch_bounds__(256) void wgrad_bias_reduce_kernel(const float *__r
 // the slice read the slice's last row and count as zeros, so there is no separate tail path.
 constexpr int kLdh = 2 * kChunk + 8;  // bytes between staged columns
 
-template <int WM, int WN, bool MASKED>
+template <int WM, int WN, bool MASKED, bool BITS>
 __global__ __launch_bounds__(256, 1) void wgrad_bf16_partial_kernel(const float *__restrict__ x,
                                                                     const float *__restrict__ g,
                                                                     float *__restrict__ partial, int64_t rows, int fi,
@@ -361,6 +381,8 @@ __global__ __launch_bounds__(256, 1) void wgrad_bf16_partial_kernel(const float 
 
     floatx4 xr[4], gr[4], yr[4];
     float dr[4];
+    uint32_t br[4];  // BITS: the word that holds the activity bits of the block's four columns, per row
+    const int b_word = ((4 * g_cq) >> 5) * mk.bits_step, b_shift = (4 * g_cq) & 31;
     floatx4 colsum = {0.f, 0.f, 0.f, 0.f};
     const float *divp = MASKED ? (mk.row_div ? mk.row_div : x) : nullptr;  // any readable float per row without a divisor
     const int64_t divstep = MASKED ? (mk.row_div ? 1 : ldx) : 0;
@@ -373,8 +395,11 @@ __global__ __launch_bounds__(256, 1) void wgrad_bf16_partial_kernel(const float 
             xr[c] = __builtin_nontemporal_load(reinterpret_cast<const floatx4 *>(x + (size_t)rx * (size_t)ldx + 4 * x_cq));
             gr[c] = __builtin_nontemporal_load(reinterpret_cast<const floatx4 *>(g + (size_t)rg * (size_t)ldg + 4 * g_cq));
             if (MASKED) {
-                yr[c] = __builtin_nontemporal_load(
-                    reinterpret_cast<const floatx4 *>(mk.act + (size_t)rg * (size_t)mk.ldact + 4 * g_cq));
+                if (BITS)
+                    br[c] = mk.bits[(size_t)rg * (size_t)mk.bits_stride + b_word];
+                else
+                    yr[c] = __builtin_nontemporal_load(
+                        reinterpret_cast<const floatx4 *>(mk.act + (size_t)rg * (size_t)mk.ldact + 4 * g_cq));
                 dr[c] = divp[rg * divstep];
             }
         }
@@ -387,11 +412,19 @@ __global__ __launch_bounds__(256, 1) void wgrad_bf16_partial_kernel(const float 
             if (!live_x) xr[c] = floatx4{0.f, 0.f, 0.f, 0.f};
             if (MASKED) {
                 const bool all = mk.all_on != 0;
+                bool on[4];
+                if (BITS) {
+                    const uint32_t nib = br[c] >> b_shift;
+                    on[0] = nib & 1u, on[1] = nib & 2u, on[2] = nib & 4u, on[3] = nib & 8u;
+                } else {
+                    on[0] = all || yr[c].x > 0.0f, on[1] = all || yr[c].y > 0.0f;
+                    on[2] = all || yr[c].z > 0.0f, on[3] = all || yr[c].w > 0.0f;
+                }
                 floatx4 pre;
-                pre.x = (live_g && (all || yr[c].x > 0.0f)) ? gr[c].x * mk.scale : 0.0f;
-                pre.y = (live_g && (all || yr[c].y > 0.0f)) ? gr[c].y * mk.scale : 0.0f;
-                pre.z = (live_g && (all || yr[c].z > 0.0f)) ? gr[c].z * mk.scale : 0.0f;
-                pre.w = (live_g && (all || yr[c].w > 0.0f)) ? gr[c].w * mk.scale : 0.0f;
+                pre.x = (live_g && on[0]) ? gr[c].x * mk.scale : 0.0f;
+                pre.y = (live_g && on[1]) ? gr[c].y * mk.scale : 0.0f;
+                pre.z = (live_g && on[2]) ? gr[c].z * mk.scale : 0.0f;
+                pre.w = (live_g && on[3]) ? gr[c].w * mk.scale : 0.0f;
                 if (g_first) colsum += pre;
                 const float inv = mk.row_div ? 1.0f / dr[c] : 1.0f;
                 pre *= inv;
@@ -534,7 +567,7 @@ int run_wgrad(const float *x, int64_t x_stride, const float *g, int64_t g_stride
     MaskArgs mk{};
     if (mask) {
         mk = *mask;
-        if (!aligned || mk.ldact % 4 != 0 || (reinterpret_cast<uintptr_t>(mk.act) & 15) != 0 ||
+        if (!aligned || (!mk.bits && (mk.ldact % 4 != 0 || (reinterpret_cast<uintptr_t>(mk.act) & 15) != 0)) ||
             (reinterpret_cast<uintptr_t>(mk.gz) & 15) != 0)
             return fail(GNNAGG_ERR_UNSUPPORTED, "the masked weight gradient takes widths and row strides that are "
                                                 "multiples of 4 floats and 16-byte aligned operands");
@@ -542,7 +575,7 @@ int run_wgrad(const float *x, int64_t x_stride, const float *g, int64_t g_stride
     }
     // wave corner = 32*WM x 32*WN, block = 2 x 2 waves
     const int wm = (int)((fi + 63) / 64), wn = (int)((fo + 63) / 64);
-    const bool sums_only = mask && mk.all_on && !mk.row_div && !mk.gz;
+    const bool sums_only = mask && mk.all_on && !mk.row_div && !mk.gz && !mk.bits;
 #define GNNAGG_WGRAD_FORM(M, N, MASKED)                                                                         \
     {                                                                                                           \
         constexpr size_t smem = (size_t)WgradShape<M, N>::kSmemFloats * sizeof(float);                          \
@@ -553,13 +586,18 @@ int run_wgrad(const float *x, int64_t x_stride, const float *g, int64_t g_stride
 #define GNNAGG_WGRAD_BF16(M, N)                                                                                  \
     {                                                                                                           \
         constexpr size_t smem = (size_t)2 * (64 * M + 64 * N) * kLdh;                                            \
-        hipLaunchKernelGGL((wgrad_bf16_partial_kernel<M, N, true>), dim3((unsigned)blocks), dim3(256), smem, st, x, \
-                           g, partial, rows, (int)fi, (int)fo, (int)x_stride, (int)g_stride, rpb, mk);           \
+        if (mk.bits)                                                                                            \
+            hipLaunchKernelGGL((wgrad_bf16_partial_kernel<M, N, true, true>), dim3((unsigned)blocks), dim3(256), smem, st, \
+                               x, g, partial, rows, (int)fi, (int)fo, (int)x_stride, (int)g_stride, rpb, mk);   \
+        else                                                                                                    \
+            hipLaunchKernelGGL((wgrad_bf16_partial_kernel<M, N, true, false>), dim3((unsigned)blocks), dim3(256), smem, st, \
+                               x, g, partial, rows, (int)fi, (int)fo, (int)x_stride, (int)g_stride, rpb, mk);   \
     }
 #define GNNAGG_WGRAD(M, N)                          \
     if (wm == M && wn == N) {                       \
         if (bf16) GNNAGG_WGRAD_BF16(M, N)           \
         else if (mask && sums_only) GNNAGG_WGRAD_FORM(M, N, 2) \
+        else if (mask && mk.bits) GNNAGG_WGRAD_FORM(M, N, 3) \
         else if (mask) GNNAGG_WGRAD_FORM(M, N, 1)   \
         else GNNAGG_WGRAD_FORM(M, N, 0)             \
     } else
@@ -608,7 +646,7 @@ extern "C" int gnnagg_wgrad_relu_dropout_backward_f32(const float *x, int64_t x_
     GNNAGG_REQUIRE(!y || (y_stride >= fo && y_stride < (int64_t(1) << 27)), "bad row stride of y");
     // without y the kernel reads the first row of g over and over in its place (row stride 0: a cache hit) and
     // ignores the values
-    MaskArgs mk{y ? y : grad_y, row_div, grad_z, nullptr, (int)(y ? y_stride : 0), scale, y ? 0 : 1};
+    MaskArgs mk{y ? y : grad_y, row_div, grad_z, nullptr, (int)(y ? y_stride : 0), scale, y ? 0 : 1, nullptr, 0, 0};
     return run_wgrad(x, x_stride, grad_y, grad_stride, w_grad, workspace, rows, fi, fo, stream, &mk, bias_grad);
 }
 
@@ -619,6 +657,21 @@ extern "C" int gnnagg_wgrad_relu_dropout_backward_bf16_f32(const float *x, int64
                                                            int64_t fi, int64_t fo, void *stream) {
     GNNAGG_REQUIRE(bias_grad, "null bias_grad");
     GNNAGG_REQUIRE(!y || (y_stride >= fo && y_stride < (int64_t(1) << 27)), "bad row stride of y");
-    MaskArgs mk{y ? y : grad_y, row_div, grad_z, nullptr, (int)(y ? y_stride : 0), scale, y ? 0 : 1};
+    MaskArgs mk{y ? y : grad_y, row_div, grad_z, nullptr, (int)(y ? y_stride : 0), scale, y ? 0 : 1, nullptr, 0, 0};
     return run_wgrad(x, x_stride, grad_y, grad_stride, w_grad, workspace, rows, fi, fo, stream, &mk, bias_grad, true);
+}
+
+extern "C" int gnnagg_wgrad_relu_dropout_backward_from_header_f32(const float *x, int64_t x_stride, const float *grad_y,
+                                                                  int64_t grad_stride, const uint32_t *header,
+                                                                  const float *row_div, float scale, float *grad_z,
+                                                                  float *w_grad, float *bias_grad, void *workspace,
+                                                                  int64_t rows, int64_t fi, int64_t fo, int bf16_inputs,
+                                                                  void *stream) {
+    GNNAGG_REQUIRE(bias_grad, "null bias_grad");
+    GNNAGG_REQUIRE(header || rows == 0, "null header");
+    if (!(fo == 32 || fo == 64 || fo == 128 || fo == 256))
+        return fail(GNNAGG_ERR_UNSUPPORTED, "packed activations exist for widths 32, 64, 128, 256 (got %lld)", (long long)fo);
+    MaskArgs mk{nullptr, row_div, grad_z, nullptr, 0, scale, 0, header, (int)(2 * (fo / 32)), 2};
+    return run_wgrad(x, x_stride, grad_y, grad_stride, w_grad, workspace, rows, fi, fo, stream, &mk, bias_grad,
+                     bf16_inputs != 0);
 }

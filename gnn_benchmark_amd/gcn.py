@@ -121,6 +121,12 @@ def pack_keep_mask(keep: torch.Tensor) -> torch.Tensor:
     return bits
 
 
+def _row_divisors(graph):
+    """The in-degrees a layer divides its aggregation by, or None when the graph's matrices already carry that
+    division in their values (``sage.fold_in_degrees``)."""
+    return None if getattr(graph, "in_degrees_folded", False) else graph.in_degrees
+
+
 def fused_layer_supported(x: torch.Tensor, in_channels: int, out_channels: int) -> bool:
     """Whether ``_FusedLayer`` takes a [rows, in_channels] operand on x's device and these widths."""
     if not (x.is_cuda and x.dtype == torch.float32):
@@ -182,30 +188,78 @@ class _FusedLayer(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_y):
         x, w, y = ctx.saved_tensors
-        grad_y = _kernel_ready(grad_y)
-        rows, k, n = x.size(0), x.size(1), w.size(1)
-        L = _lib.lib()
-        workspace = torch.empty(int(L.gnnagg_wgrad_relu_dropout_backward_workspace_bytes(max(rows, 1), k, n)) // 4,
-                                dtype=torch.float32, device=x.device)
-        want_x = ctx.needs_input_grad[0]
-        grad_z = torch.empty(rows, n, dtype=torch.float32, device=x.device) if want_x else None
-        grad_w = torch.empty(k, n, dtype=torch.float32, device=x.device)
-        grad_bias = torch.empty(n, dtype=torch.float32, device=x.device)
-        entry = L.gnnagg_wgrad_relu_dropout_backward_bf16_f32 if ctx.bf16 else L.gnnagg_wgrad_relu_dropout_backward_f32
-        with torch.cuda.device(x.device):
+        grads = _fused_backward(x, w, grad_y, y, None, ctx.row_div, ctx.scale, ctx.bf16, ctx.needs_input_grad[0])
+        return grads + (None, None, None, None, None)
+
+
+def _fused_backward(x, w, grad_y, y, header, row_div, scale, bf16, want_x):
+    """(grad_x, grad_w, grad_bias) of the fused layer: one pass of the weight-gradient kernel (mask from ``y`` or from
+    the packed output's ``header``, degree division, bias gradient, weight gradient) plus the input-gradient product."""
+    grad_y = _kernel_ready(grad_y)
+    rows, k, n = x.size(0), x.size(1), w.size(1)
+    L = _lib.lib()
+    workspace = torch.empty(int(L.gnnagg_wgrad_relu_dropout_backward_workspace_bytes(max(rows, 1), k, n)) // 4,
+                            dtype=torch.float32, device=x.device)
+    grad_z = torch.empty(rows, n, dtype=torch.float32, device=x.device) if want_x else None
+    grad_w = torch.empty(k, n, dtype=torch.float32, device=x.device)
+    grad_bias = torch.empty(n, dtype=torch.float32, device=x.device)
+    stream = _lib.current_stream(x.device)
+    with torch.cuda.device(x.device):
+        if header is not None:
+            _lib.check(L.gnnagg_wgrad_relu_dropout_backward_from_header_f32(
+                _lib.ptr(x), _row_stride(x), _lib.ptr(grad_y), _row_stride(grad_y), _lib.ptr(header), _lib.ptr(row_div),
+                scale, _lib.ptr(grad_z), _lib.ptr(grad_w), _lib.ptr(grad_bias), _lib.ptr(workspace), rows, k, n,
+                1 if bf16 else 0, stream))
+        else:
+            entry = L.gnnagg_wgrad_relu_dropout_backward_bf16_f32 if bf16 else L.gnnagg_wgrad_relu_dropout_backward_f32
             _lib.check(entry(_lib.ptr(x), _row_stride(x), _lib.ptr(grad_y), _row_stride(grad_y), _lib.ptr(y),
-                             n if y is not None else 0, _lib.ptr(ctx.row_div), ctx.scale, _lib.ptr(grad_z),
-                             _lib.ptr(grad_w), _lib.ptr(grad_bias), _lib.ptr(workspace), rows, k, n,
-                             _lib.current_stream(x.device)))
-        grad_x = None
-        if want_x:
-            if not ctx.bf16:
-                grad_x = torch.mm(grad_z, w.t())
-            elif L.gnnagg_linear_shape_supported(n, k):
-                grad_x = _fused_product(grad_z, w.t().contiguous(), None, None, None, 1.0, False, True)
-            else:
-                grad_x = _Bf16InputLinear._mm(grad_z, w.t())
-        return grad_x, grad_w, grad_bias, None, None, None, None, None
+                             n if y is not None else 0, _lib.ptr(row_div), scale, _lib.ptr(grad_z), _lib.ptr(grad_w),
+                             _lib.ptr(grad_bias), _lib.ptr(workspace), rows, k, n, stream))
+    grad_x = None
+    if want_x:
+        if not bf16:
+            grad_x = torch.mm(grad_z, w.t())
+        elif L.gnnagg_linear_shape_supported(n, k):
+            grad_x = _fused_product(grad_z, w.t().contiguous(), None, None, None, 1.0, False, True)
+        else:
+            grad_x = _Bf16InputLinear._mm(grad_z, w.t())
+    return grad_x, grad_w, grad_bias
+
+
+class _FusedLayerPacked(torch.autograd.Function):
+    """``_FusedLayer`` writing its result packed (``packed.py``): returns ``(values, header)``.  The gradient that comes
+    back for ``values`` is the one with respect to the dense activations the pair stands for (``AggregatorPacked``
+    returns exactly that); which units were active is read from the header's bitmaps."""
+
+    @staticmethod
+    def forward(ctx, x, w, bias, keep_bits, scale, row_div, bf16):
+        rows, k, n = x.size(0), x.size(1), w.size(1)
+        if keep_bits is not None and (keep_bits.dtype != torch.int32 or keep_bits.shape != (rows, (n + 31) // 32)
+                                      or not keep_bits.is_contiguous()):
+            raise RuntimeError("Input mismatch: keep_bits must be contiguous int32 [rows, ceil(feat / 32)] "
+                               "(gcn.pack_keep_mask)")
+        if row_div is not None and (row_div.dtype != torch.float32 or row_div.numel() != rows
+                                    or not row_div.is_contiguous()):
+            raise RuntimeError("Input mismatch: row_div must be contiguous float32 with one entry per row")
+        w = w.contiguous()
+        values, header = packed.empty(rows, n, x.device)
+        with torch.cuda.device(x.device):
+            _lib.check(_lib.lib().gnnagg_linear_bias_relu_dropout_pack_f32(
+                _lib.ptr(x), _row_stride(x), _lib.ptr(w), n, _lib.ptr(bias.contiguous()), _lib.ptr(keep_bits),
+                _lib.ptr(row_div), float(scale), _lib.ptr(values), _lib.ptr(header), rows, k, n, 1 if bf16 else 0,
+                _lib.current_stream(x.device)))
+        ctx.mark_non_differentiable(header)
+        ctx.save_for_backward(x, w, header)
+        ctx.scale = float(scale)
+        ctx.row_div = row_div
+        ctx.bf16 = bool(bf16)
+        return values, header
+
+    @staticmethod
+    def backward(ctx, grad_y, _grad_header):
+        x, w, header = ctx.saved_tensors
+        grads = _fused_backward(x, w, grad_y, None, header, ctx.row_div, ctx.scale, ctx.bf16, ctx.needs_input_grad[0])
+        return grads + (None, None, None, None)
 
 
 class _BiasReluDropout(torch.autograd.Function):
@@ -327,23 +381,35 @@ class GCNLayer(torch.nn.Module):
             return Aggregator.apply(graph, self._product(x), layer, 32, is_pre_delay, self.training)
         return self._product(Aggregator.apply(graph, x, layer, 32, is_pre_delay, self.training))
 
-    def fused(self, graph, x, layer: int, is_pre_delay: bool, keep_bits, scale: float, relu: bool):
-        """relu(((A x) W) / deg + bias) * keep * scale through the fused kernels, or None where they do
-        not apply (packed input, product-first order, widths the kernels do not take)."""
-        if self.linear_first or isinstance(x, tuple) or not self.fuse:
+    def fused(self, graph, x, layer: int, is_pre_delay: bool, keep_bits, scale: float, relu: bool,
+              pack_out: bool = False):
+        """relu(((A x) W) / deg + bias) * keep * scale through the fused kernels -- dense, or as a packed
+        ``(values, header)`` pair with ``pack_out`` -- or None where they do not apply (product-first order, widths
+        the kernels do not take).  ``x`` is a dense tensor or a packed pair."""
+        if self.linear_first or not self.fuse:
             return None
-        if not fused_layer_supported(x, self.weight.size(0), self.weight.size(1)):
+        probe = x[0] if isinstance(x, tuple) else x
+        if not fused_layer_supported(probe, self.weight.size(0), self.weight.size(1)):
             return None
-        agg = _kernel_ready(Aggregator.apply(graph, x, layer, 32, is_pre_delay, self.training))
-        row_div = graph.in_degrees.reshape(-1)
-        return _FusedLayer.apply(agg, self.weight, self.bias, keep_bits, scale, row_div, relu, self.gemm == "bf16")
+        if isinstance(x, tuple):
+            agg = AggregatorPacked.apply(graph, x[0], x[1], layer, 32, is_pre_delay, self.training)
+        else:
+            agg = Aggregator.apply(graph, x, layer, 32, is_pre_delay, self.training)
+        agg = _kernel_ready(agg)
+        row_div = _row_divisors(graph)
+        row_div = None if row_div is None else row_div.reshape(-1)
+        bf16 = self.gemm == "bf16"
+        if pack_out:
+            return _FusedLayerPacked.apply(agg, self.weight, self.bias, keep_bits, scale, row_div, bf16)
+        return _FusedLayer.apply(agg, self.weight, self.bias, keep_bits, scale, row_div, relu, bf16)
 
     def forward(self, graph, x: torch.Tensor, layer: int, is_pre_delay: bool) -> torch.Tensor:
         """((A x) W) / deg + bias."""
         out = self.fused(graph, x, layer, is_pre_delay, None, 1.0, False)
         if out is not None:
             return out
-        return torch.addcdiv(self.bias, self.transform(graph, x, layer, is_pre_delay), graph.in_degrees)
+        z, row_div = self.transform(graph, x, layer, is_pre_delay), _row_divisors(graph)
+        return z + self.bias if row_div is None else torch.addcdiv(self.bias, z, row_div)
 
 
 class GCN(torch.nn.Module):
@@ -394,20 +460,19 @@ class GCN(torch.nn.Module):
                 raise ValueError("training needs the seeded dropout masks")
             mask = masks[l] if dropping else None
             scale = 1.0 / (1.0 - self.dropout) if dropping else 1.0
-            if not pack:
-                bits = mask
-                if mask is not None and mask.dtype != torch.int32:
-                    bits = self._packed_mask(mask)
-                fused = layer.fused(graph, h, l, is_pre_delay, bits, scale, True)
-                if fused is not None:
-                    h = fused
-                    continue
+            bits = mask
+            if mask is not None and mask.dtype != torch.int32 and layer.fuse and not layer.linear_first:
+                bits = self._packed_mask(mask)
+            fused = layer.fused(graph, h, l, is_pre_delay, bits, scale, True, pack_out=pack)
+            if fused is not None:
+                h = fused
+                continue
             if mask is not None and mask.dtype == torch.int32:
                 raise RuntimeError("a bit-packed dropout mask only serves the fused layer kernels; this layer needs "
                                    "the bool mask")
             z = layer.transform(graph, h, l, is_pre_delay)
             epilogue = _BiasReluDropoutPacked if pack else _BiasReluDropout
-            h = epilogue.apply(z, layer.bias, mask, scale, graph.in_degrees)
+            h = epilogue.apply(z, layer.bias, mask, scale, _row_divisors(graph))
         return F.log_softmax(h, dim=1) if log_probs else h
 
 

@@ -229,6 +229,14 @@ int gnnagg_linear_bias_relu_dropout_bf16_f32(const float *x, int64_t x_stride, c
                                              const float *bias, const uint32_t *keep_bits, const float *row_div,
                                              float scale, int relu, float *y, int64_t y_stride, int64_t rows,
                                              int64_t k, int64_t n, void *stream);
+/* The same layer writing its result packed (the format of gnnagg_bias_relu_dropout_pack_f32 below: every row's
+ * non-zero values at its front, plus the header of (bitmap, non-zeros in front) pairs): n in {32, 64, 128, 256},
+ * ReLU always on, y_packed [rows, n] contiguous with 4 floats of slack behind it, header uint32 [rows, 2 * (n / 32)];
+ * bf16_inputs 0/1 picks the product's form. */
+int gnnagg_linear_bias_relu_dropout_pack_f32(const float *x, int64_t x_stride, const float *w, int64_t w_stride,
+                                             const float *bias, const uint32_t *keep_bits, const float *row_div,
+                                             float scale, float *y_packed, uint32_t *header, int64_t rows, int64_t k,
+                                             int64_t n, int bf16_inputs, void *stream);
 int64_t gnnagg_wgrad_relu_dropout_backward_workspace_bytes(int64_t rows, int64_t fi, int64_t fo);
 /* (the _bf16_ form below takes the same arguments and workspace; it rounds x and grad_z to bf16 for the
  * product x^T @ grad_z -- fp32 accumulation -- while grad_z and bias_grad are computed and written in fp32) */
@@ -236,6 +244,13 @@ int gnnagg_wgrad_relu_dropout_backward_f32(const float *x, int64_t x_stride, con
                                            const float *y, int64_t y_stride, const float *row_div, float scale,
                                            float *grad_z, float *w_grad, float *bias_grad, void *workspace,
                                            int64_t rows, int64_t fi, int64_t fo, void *stream);
+/* The same when the layer's output was written packed: which units were active is read from the bitmaps of its
+ * header (fo in {32, 64, 128, 256}) instead of from y; bf16_inputs 0/1 picks the product's form. */
+int gnnagg_wgrad_relu_dropout_backward_from_header_f32(const float *x, int64_t x_stride, const float *grad_y,
+                                                       int64_t grad_stride, const uint32_t *header, const float *row_div,
+                                                       float scale, float *grad_z, float *w_grad, float *bias_grad,
+                                                       void *workspace, int64_t rows, int64_t fi, int64_t fo,
+                                                       int bf16_inputs, void *stream);
 int gnnagg_wgrad_relu_dropout_backward_bf16_f32(const float *x, int64_t x_stride, const float *grad_y,
                                                 int64_t grad_stride, const float *y, int64_t y_stride,
                                                 const float *row_div, float scale, float *grad_z, float *w_grad,

@@ -100,18 +100,21 @@ def test_bitmap_backward_equals_dense_backward(feat):
     assert torch.equal(b1.grad, b2.grad)
 
 
-def test_train_step_with_packed_activations_equals_dense():
+@pytest.mark.parametrize("fused,gemm,dims", [(False, "fp32", [24, 64, 128, 7]), (True, "fp32", [32, 64, 128, 8]),
+                                             (True, "bf16", [32, 64, 256, 8])])
+def test_train_step_with_packed_activations_equals_dense(fused, gemm, dims):
+    """Packed hidden activations change nothing but the sign of a zero: losses and updated weights are bit for bit
+    those of the dense model -- with the separate product / epilogue kernels on both sides, and with the one-kernel
+    layers on both sides (whose packed form reads the activity from the header's bitmaps in the gradient direction)."""
     part = synthetic.partition_edges(num_local_nodes=3000, world_size=4, rank=1, local_mean_out_degree=5.0, zipf_s=1.8,
                                      max_degree=300, num_halo_nodes=1200, num_remote_edges=6000, seed=21, device="cuda")
-    dims = [24, 64, 128, 7]
     gen = torch.Generator(device="cuda").manual_seed(2)
     x = torch.randn(3000, dims[0], device="cuda", generator=gen)
     labels = torch.randint(0, dims[-1], (3000,), device="cuda", generator=gen)
     train_idx = torch.randperm(3000, device="cuda", generator=gen)[:600]
     masks = gcn.make_dropout_masks(3000, dims, 0.5, seed=8, device="cuda")
     torch.manual_seed(0)
-    # (like with like: both models on the separate product / epilogue kernels, whose roundings the packed form shares)
-    dense_model = gcn.GCN(dims, gemm="fp32", dropout=0.5, fused_layers=False).cuda()
+    dense_model = gcn.GCN(dims, gemm=gemm, dropout=0.5, fused_layers=fused).cuda()
     packed_model = copy.deepcopy(dense_model)
     packed_model.packed_activations = True
     results = []
