@@ -245,8 +245,12 @@ __global__ __launch_bounds__(256, 2) void linear_kernel(const LinearArgs p) {
                     const int n = nt + 8 * g + 4 * kk;
                     if (!live || n >= p.n) continue;
                     floatx4 v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
-                    v *= inv;
-                    if (p.bias) v += *reinterpret_cast<const floatx4 *>(p.bias + n);
+                    // (acc * inv + bias as one fused multiply-add per value, here and in the packed form)
+                    const floatx4 b4 = p.bias ? *reinterpret_cast<const floatx4 *>(p.bias + n) : floatx4{0.f, 0.f, 0.f, 0.f};
+                    v.x = __builtin_fmaf(v.x, inv, b4.x);
+                    v.y = __builtin_fmaf(v.y, inv, b4.y);
+                    v.z = __builtin_fmaf(v.z, inv, b4.z);
+                    v.w = __builtin_fmaf(v.w, inv, b4.w);
                     if (p.relu) {
                         v.x = fmaxf(v.x, 0.0f);
                         v.y = fmaxf(v.y, 0.0f);
@@ -283,11 +287,15 @@ __global__ __launch_bounds__(256, 2) void linear_kernel(const LinearArgs p) {
                 const int nt = n0 + 32 * j;
                 const uint32_t bits = kbits[i][j] >> (4 * kk);
                 uint32_t mine = 0;
+                floatx4 b4[4];
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+                    b4[g] = (p.bias && nt < p.n) ? *reinterpret_cast<const floatx4 *>(p.bias + nt + 8 * g + 4 * kk)
+                                                 : floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int local = 8 * (r >> 2) + (r & 3);  // + 4 kk: this value's column inside the tile
-                    float v = acc[i][j][r] * inv;
-                    if (p.bias && nt < p.n) v += p.bias[nt + local + 4 * kk];
+                    float v = __builtin_fmaf(acc[i][j][r], inv, b4[r >> 2][r & 3]);
                     v = fmaxf(v, 0.0f) * p.scale;
                     if (!((bits >> local) & 1u) || !live || nt >= p.n) v = 0.0f;
                     acc[i][j][r] = v;
