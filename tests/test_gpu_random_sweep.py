@@ -208,7 +208,7 @@ def test_random_fused_layer_kernels_match_fp64(seed):
     for case in range(14):
         rows = int(rng.choice([1, 5, 127, 128, 129, 1000, 4097, 20011]))
         k = 16 * int(rng.integers(1, 17))
-        n = 4 * int(rng.integers(1, 65))
+        n = int(rng.choice([32, 64, 128, 256])) if rng.random() < 0.4 else 4 * int(rng.integers(1, 65))
         pad = 4 * int(rng.integers(0, 3))
         wide = dev(rng.standard_normal((rows, k + 2 * pad)).astype(np.float32))
         x = wide[:, pad:pad + k]
@@ -245,3 +245,13 @@ def test_random_fused_layer_kernels_match_fp64(seed):
                                 (b_in.grad, pre.sum(0), "bias")):
             size = float(want.abs().max()) + 1e-12
             assert float((got.double() - want).abs().max()) <= 2e-5 * size, (name, what)
+        if relu and n in (32, 64, 128, 256):
+            # the same layer writing its output packed: the same values bit for bit, and -- its gradient pass reading
+            # the activity from the header's bitmaps -- the same gradients bit for bit
+            x2, w2, b2 = x.detach().clone().requires_grad_(), w.clone().requires_grad_(), bias.clone().requires_grad_()
+            values, header = gcn._FusedLayerPacked.apply(gcn._kernel_ready(x2), w2, b2,
+                                                         gcn.pack_keep_mask(keep) if with_mask else None, scale, div, False)
+            assert torch.equal(packed.unpack(values, header), y.detach()), what
+            values.backward(g)
+            for got, want, name in ((x2.grad, view.grad, "x"), (w2.grad, w_in.grad, "w"), (b2.grad, b_in.grad, "bias")):
+                assert torch.equal(got, want), (name, what)
