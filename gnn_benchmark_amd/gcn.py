@@ -481,13 +481,19 @@ def make_dropout_masks(num_nodes: int, dims: Sequence[int], p: float, seed: int,
     return [torch.rand(num_nodes, dims[l + 1], device=device, generator=gen) >= p for l in range(len(dims) - 2)]
 
 
+def _mean_nll(log_probs: torch.Tensor, target: torch.Tensor) -> torch.Tensor:
+    """F.nll_loss(log_probs, target) (mean over the rows, every target a class index) as a gather and a mean: the
+    library's reduction kernel for it runs in a single block and takes 1.6 ms on 700 000 rows."""
+    return -log_probs.gather(1, target.unsqueeze(1)).mean()
+
+
 def train_step(model: GCN, optimizer, graph, x, labels, train_idx, is_pre_delay: bool, masks) -> torch.Tensor:
     """forward, NLL loss on the labelled nodes, backward, optimizer update.  The log-softmax is
     row-wise, so only the labelled rows are normalised."""
     model.train()
     optimizer.zero_grad(set_to_none=True)
     out = model(graph, x, is_pre_delay, masks, log_probs=False)
-    loss = F.nll_loss(F.log_softmax(out[train_idx], dim=1), labels[train_idx])
+    loss = _mean_nll(F.log_softmax(out[train_idx], dim=1), labels[train_idx])
     loss.backward()
     optimizer.step()
     return loss.detach()

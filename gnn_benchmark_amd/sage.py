@@ -28,7 +28,7 @@ import torch
 import torch.nn.functional as F
 
 from . import _lib, aggregator
-from .gcn import weight_and_bias_gradient, weight_gradient
+from .gcn import _mean_nll, weight_and_bias_gradient, weight_gradient
 from .sparse_tensor import SparseTensor, _row_stride
 
 
@@ -377,7 +377,7 @@ def train_step(model: DistSAGE, optimizer, graph, nodes_feats, labels, train_idx
     model.train()
     optimizer.zero_grad(set_to_none=True)
     out = model(graph, nodes_feats, masks, log_probs=False)
-    loss = F.nll_loss(F.log_softmax(out[train_idx], dim=1), labels[train_idx])
+    loss = _mean_nll(F.log_softmax(out[train_idx], dim=1), labels[train_idx])
     loss.backward()
     optimizer.step()
     return loss.detach()
