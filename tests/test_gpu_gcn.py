@@ -256,6 +256,23 @@ def test_fused_layer_rejects_unsupported_shapes():
     rc = L.gnnagg_linear_bias_relu_dropout_f32(_lib.ptr(x), 20, _lib.ptr(w), 32, None, None, None, 1.0, 0, _lib.ptr(y), 32,
                                                64, 20, 32, _lib.current_stream(x.device))
     assert rc == _lib.ERR_UNSUPPORTED
+    # packed output and the header-driven gradient pass exist for widths 32, 64, 128, 256 only
+    x16, w100 = torch.randn(64, 16, device="cuda"), torch.randn(16, 100, device="cuda")
+    vals, hdr = torch.empty(64 * 100 + 4, device="cuda"), torch.zeros(64, 8, dtype=torch.int32, device="cuda")
+    rc = L.gnnagg_linear_bias_relu_dropout_pack_f32(_lib.ptr(x16), 16, _lib.ptr(w100), 100, None, None, None, 1.0,
+                                                    _lib.ptr(vals), _lib.ptr(hdr), 64, 16, 100, 0,
+                                                    _lib.current_stream(x.device))
+    assert rc == _lib.ERR_UNSUPPORTED
+    g100 = torch.randn(64, 100, device="cuda")
+    ws = torch.empty(int(L.gnnagg_wgrad_relu_dropout_backward_workspace_bytes(64, 16, 100)) // 4, device="cuda")
+    gw, gb = torch.empty(16, 100, device="cuda"), torch.empty(100, device="cuda")
+    rc = L.gnnagg_wgrad_relu_dropout_backward_from_header_f32(_lib.ptr(x16), 16, _lib.ptr(g100), 100, _lib.ptr(hdr), None,
+                                                              1.0, None, _lib.ptr(gw), _lib.ptr(gb), _lib.ptr(ws), 64, 16,
+                                                              100, 0, _lib.current_stream(x.device))
+    assert rc == _lib.ERR_UNSUPPORTED
+    with pytest.raises(RuntimeError, match="behind a ReLU"):
+        gcn._FusedLayer.apply(x16, torch.randn(16, 32, device="cuda"), torch.zeros(32, device="cuda"),
+                              torch.zeros(64, 1, dtype=torch.int32, device="cuda"), 2.0, None, False)
 
 
 @pytest.mark.parametrize("rows,fi,fo", [(70_001, 256, 172), (999, 40, 48), (128, 64, 64), (1, 4, 4), (5000, 128, 256)])
