@@ -115,7 +115,7 @@ __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__re
     }
     // any readable float per row when there is no divisor (the value is not used then)
     const float *divp = FULL ? (mk.row_div ? mk.row_div : x) : nullptr;
-    const int64_t divstep = FULL ? (mk.row_div ? 1 : ldx) : 0;
+    const int divstep = (FULL && mk.row_div) ? 1 : 0;
     auto fetch_divisors = [&](int64_t r, int64_t last) {  // rows r .. r+15, clamped to `last`
 #pragma unroll
         for (int j = 0; j < S::kVecG; ++j) {
@@ -123,6 +123,27 @@ __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__re
             if (row > last) row = last;
             dreg[j] = divp[row * divstep];
             if (BITS) breg[j] = mk.bits[(size_t)row * (size_t)mk.bits_stride + bit_word[j]];
+        }
+    };
+    // The same for the whole chunks of the steady state: no clamp, and 32-bit offsets from the slice's first row that
+    // advance by one chunk per call (no 64-bit index arithmetic ahead of the MFMAs).
+    const float *div_base = FULL ? divp + (size_t)r_begin * (size_t)divstep : nullptr;
+    const uint32_t *bits_base = BITS ? mk.bits + (size_t)r_begin * (size_t)mk.bits_stride : nullptr;
+    int div_off[S::kVecG], bits_off[S::kVecG];
+#pragma unroll
+    for (int j = 0; j < S::kVecG; ++j) {
+        div_off[j] = MASKED ? grow[j] * divstep : 0;
+        bits_off[j] = BITS ? grow[j] * mk.bits_stride + bit_word[j] : 0;
+    }
+    auto fetch_divisors_next = [&]() {
+#pragma unroll
+        for (int j = 0; j < S::kVecG; ++j) {
+            dreg[j] = div_base[div_off[j]];
+            div_off[j] += kChunk * divstep;
+            if (BITS) {
+                breg[j] = bits_base[bits_off[j]];
+                bits_off[j] += kChunk * mk.bits_stride;
+            }
         }
     };
     // turns vector j of lg.reg (g) into the G operand, with lc.reg = y; `valid` = number of values of the chunk that exist
@@ -204,7 +225,7 @@ __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__re
         if (MASKED) {
             if (FULL) {
                 if (!BITS) lc.fetch(cc);
-                fetch_divisors(r_begin, r_end - 1);
+                fetch_divisors_next();
             }
             mask_g(r_begin, kChunk * fo);
         }
@@ -220,7 +241,7 @@ __global__ __launch_bounds__(256, 1) void wgrad_partial_kernel(const float *__re
                 cc += cstep;
                 if (FULL) {
                     if (!BITS) lc.fetch(cc);
-                    fetch_divisors(r_begin + c * kChunk, r_end - 1);
+                    fetch_divisors_next();
                 }
             }
             __builtin_amdgcn_sched_barrier(0);  // keep the loads ahead of the MFMAs
