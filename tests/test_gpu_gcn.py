@@ -349,3 +349,17 @@ def test_degrees_folded_into_the_matrices_change_rounding_only(fused):
         grads.append([out.detach().clone()] + [p.grad.detach().clone() for p in model.parameters()])
     for a, b in zip(*grads):
         assert torch.allclose(a, b, rtol=1e-4, atol=1e-6 + 1e-4 * float(a.abs().max()))
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+def test_fused_layer_with_no_rows(bf16):
+    """An empty partition: empty outputs, zero weight and bias gradients, nothing launched out of bounds."""
+    x = torch.empty(0, 32, device="cuda", requires_grad=True)
+    w = torch.randn(32, 64, device="cuda", requires_grad=True)
+    b = torch.randn(64, device="cuda", requires_grad=True)
+    y = gcn._FusedLayer.apply(x, w, b, None, 1.0, None, True, bf16)
+    assert y.shape == (0, 64)
+    y.backward(torch.empty(0, 64, device="cuda"))
+    assert x.grad.shape == (0, 32) and not w.grad.any() and not b.grad.any()
+    values, header = gcn._FusedLayerPacked.apply(x, w, b, None, 1.0, None, bf16)
+    assert values.shape == (0, 64) and header.shape == (0, 4)
