@@ -46,10 +46,12 @@ What differs from the reference, on purpose:
 (``packed.py``: non-zero values at the front of each row plus a bitmap header); only the
 two forward products that read the features differ.
 """
+import copy
+
 import torch
 
 from . import _lib, computation_ops, packed
-from .sparse_tensor import _rows_are_dense
+from .sparse_tensor import SparseTensor, _rows_are_dense
 from .spmm_kernel import SPMM_backward, SPMM_backward_quantized, SPMM_forward, SPMM_forward_quantized
 
 
@@ -270,6 +272,95 @@ def _forward(ctx, graph, feats, layer, num_bits: int, is_pre_delay: bool, is_tra
     return out
 
 
+class _BackwardSupport:
+    """The transposed matrices of one layer's gradient direction with only the entries that meet a given set of
+    gradient rows (``restricted_transpose``)."""
+
+    def __init__(self, local_T, remote_T):
+        self.local_T, self.remote_T = local_T, remote_T
+
+
+def restricted_transpose(m: SparseTensor, row_mask: torch.Tensor) -> SparseTensor:
+    """``m^T`` as a CSR of its own, keeping only the entries of ``m`` whose row is set in ``row_mask``: for a dense
+    operand ``g`` whose other rows are zero, ``restricted @ g == m^T @ g`` -- every term left out is a product with
+    zero, and the terms kept stay in their order, so each output row is the same FMA chain (up to the sign of a zero)."""
+    s = m.storage
+    colptr, row_t, value_t = s.colptr(), s.row_T(), s.value_T()
+    keep = row_mask[row_t]
+    kept_before = torch.zeros(row_t.numel() + 1, dtype=torch.int64, device=row_t.device)
+    torch.cumsum(keep, dim=0, out=kept_before[1:])
+    value = None if value_t is None else value_t[keep]
+    return SparseTensor(rowptr=kept_before[colptr], col=row_t[keep], value=value,
+                        sparse_sizes=(m.sparse_size(1), m.sparse_size(0)), is_sorted=True)
+
+
+def backward_support(graph, rows: torch.Tensor, is_pre_delay: bool) -> _BackwardSupport:
+    """What ``_backward`` needs to skip the zero rows of a gradient that is non-zero only in ``rows`` (local node
+    ids): the restricted transposes of the local matrix and of the matrix that produces the outgoing halo gradients.
+    Built once per (graph, row set) and kept on the graph."""
+    cache = graph.__dict__.setdefault("_backward_support_cache", {})
+    # (a shallow copy of a graph with other matrices -- degrees folded into the values -- shares this dictionary)
+    key = (rows.data_ptr(), rows.numel(), rows._version, bool(is_pre_delay), id(graph.local_adj_t))
+    hit = cache.get(key)
+    if hit is None:
+        n = graph.local_adj_t.sparse_size(0)
+        mask = torch.zeros(n, dtype=torch.bool, device=rows.device)
+        mask[rows] = True
+        remote = graph.adj_t_pre_post_aggr_from if is_pre_delay else graph.remote_adj_t
+        built = _BackwardSupport(restricted_transpose(graph.local_adj_t, mask),
+                                 restricted_transpose(remote, mask) if remote is not None else None)
+        for t in (built.local_T, built.remote_T):
+            if t is not None:
+                t.get_plan()
+        if len(cache) >= 4:
+            cache.clear()
+        hit = cache[key] = (rows, built, graph.local_adj_t)  # holding the tensors keeps their addresses their own
+    return hit[1]
+
+
+def select_rows(m: SparseTensor, rows: torch.Tensor) -> SparseTensor:
+    """``m[rows, :]`` as a CSR of its own (row i of the result is row ``rows[i]`` of ``m``, entries in their order)."""
+    rowptr, col, value = m.csr()
+    start = rowptr[rows]
+    counts = rowptr[rows + 1] - start
+    new_rowptr = torch.zeros(rows.numel() + 1, dtype=torch.int64, device=rowptr.device)
+    torch.cumsum(counts, dim=0, out=new_rowptr[1:])
+    total = int(new_rowptr[-1])
+    index = (torch.arange(total, dtype=torch.int64, device=rowptr.device)
+             + torch.repeat_interleave(start - new_rowptr[:-1], counts, output_size=total))
+    return SparseTensor(rowptr=new_rowptr, col=col[index], value=None if value is None else value[index],
+                        sparse_sizes=(rows.numel(), m.sparse_size(1)), is_sorted=True)
+
+
+def restrict_output_rows(graph, rows: torch.Tensor, is_pre_delay: bool):
+    """A view of ``graph`` whose aggregation produces only the output rows ``rows`` (local node ids, in that order):
+    the local matrix and the matrix that adds the received rows keep just those rows, the in-degrees likewise; what
+    is sent to other ranks is untouched.  ``Aggregator`` on it returns ``Aggregator(graph, ...)[rows]`` -- each kept
+    row is the same FMA chain -- at the cost of those rows only, forward and backward.  For the last layer of a model
+    whose loss scores a subset of the nodes.  Built once per (graph, row set) and kept on the graph."""
+    cache = graph.__dict__.setdefault("_restricted_rows_cache", {})
+    # (a shallow copy of a graph with other matrices -- degrees folded into the values -- shares this dictionary)
+    key = (rows.data_ptr(), rows.numel(), rows._version, bool(is_pre_delay), id(graph.local_adj_t))
+    hit = cache.get(key)
+    if hit is None:
+        g = copy.copy(graph)
+        g.__dict__.pop("_restricted_rows_cache", None)
+        g.local_adj_t = select_rows(graph.local_adj_t, rows)
+        name = "adj_t_pre_post_aggr_from" if is_pre_delay else "remote_adj_t"
+        remote = getattr(graph, name, None)
+        if remote is not None:
+            setattr(g, name, select_rows(remote, rows))
+        g.in_degrees = graph.in_degrees[rows].contiguous()
+        for m in (g.local_adj_t, getattr(g, name, None)):
+            if m is not None:
+                m.get_plan()
+                m.get_plan_for_transpose()
+        if len(cache) >= 4:
+            cache.clear()
+        hit = cache[key] = (rows, g, graph.local_adj_t)  # holding the tensors keeps their addresses their own
+    return hit[1]
+
+
 def _backward(ctx, local_out_grad, out=None, accumulate: bool = False):
     """``out`` / ``accumulate``: write the gradient into ``out`` (a column block of a wider tensor
     is fine), on top of what it holds when ``accumulate``; a fresh tensor when ``out`` is None."""
@@ -288,9 +379,14 @@ def _backward(ctx, local_out_grad, out=None, accumulate: bool = False):
         graph.comm_buf_for_quantization.resize_buffer(graph.comm_splits, feat_len, num_bits)
 
     # the receive buffer carries the outgoing halo gradients on the way back
+    # a caller that knows the gradient to be zero outside a set of rows (a loss that scores only the training nodes,
+    # for the last layer) declares it in graph.backward_row_support[layer]: the products below then skip those rows
+    support = (getattr(graph, "backward_row_support", None) or {}).get(ctx.layer)
     remote_nodes_grad_buf = graph.comm_buf.recv_buf
     if remote_nodes_grad_buf.size(0) != 0:
-        if is_pre_delay:
+        if support is not None:
+            SPMM_forward(support.remote_T, local_out_grad, remote_nodes_grad_buf, accumulate=False)
+        elif is_pre_delay:
             SPMM_backward(graph.adj_t_pre_post_aggr_from, local_out_grad, remote_nodes_grad_buf, accumulate=False)
         else:
             SPMM_backward(graph.remote_adj_t, local_out_grad, remote_nodes_grad_buf, accumulate=False)
@@ -312,7 +408,10 @@ def _backward(ctx, local_out_grad, out=None, accumulate: bool = False):
     else:
         _check_result(out, graph.local_adj_t.sparse_size(-1), feat_len, local_out_grad.device)
         local_nodes_grad = out
-    SPMM_backward(graph.local_adj_t, local_out_grad, local_nodes_grad, accumulate=accumulate)
+    if support is not None:
+        SPMM_forward(support.local_T, local_out_grad, local_nodes_grad, accumulate=accumulate)
+    else:
+        SPMM_backward(graph.local_adj_t, local_out_grad, local_nodes_grad, accumulate=accumulate)
 
     if comm_handle is not None:
         comm_handle.wait()

@@ -28,7 +28,7 @@ import torch
 import torch.nn.functional as F
 
 from . import _lib, aggregator
-from .gcn import _mean_nll, weight_and_bias_gradient, weight_gradient
+from .gcn import _mean_nll, scored_rows, weight_and_bias_gradient, weight_gradient
 from .sparse_tensor import SparseTensor, _row_stride
 
 
@@ -177,6 +177,57 @@ class _SageConv(torch.autograd.Function):
         return None, grad_cat, grad_w, grad_b, None, None, None, None, None
 
 
+class _SageConvRows(torch.autograd.Function):
+    """The same layer for the local nodes ``rows`` only: ``[A[rows] x / deg[rows] | x[rows]] @ W + bias`` through a
+    row-restricted view of the graph (``aggregator.restrict_output_rows``).  What a loss over those nodes needs of the
+    last layer, at a fraction of its aggregation and products, forward and backward; each row is the same FMA chain."""
+
+    @staticmethod
+    def forward(ctx, graph_rows, cat, weight, bias, layer, num_bits, is_pre_delay, is_training, normalize, rows):
+        fi = cat.size(1) // 2
+        x = cat[:, fi:]
+        agg = aggregator._forward(ctx, graph_rows, aggregator._DenseFeatures(x), layer, num_bits, is_pre_delay,
+                                  is_training)
+        ctx.divide = bool(normalize) and not getattr(graph_rows, "in_degrees_folded", False)
+        if ctx.divide:
+            agg.div_(graph_rows.in_degrees)
+        small = torch.cat([agg, x.index_select(0, rows)], dim=1)  # [len(rows), 2 fi]
+        out = torch.mm(small, weight) if bias is None else torch.addmm(bias, small, weight)
+        ctx.save_for_backward(small, weight, rows)
+        ctx.has_bias = bias is not None
+        ctx.nodes = cat.size(0)
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        small, weight, rows = ctx.saved_tensors
+        fi = small.size(1) // 2
+        g = g.contiguous()
+        grad_cat = grad_w = grad_b = None
+        want_b = ctx.has_bias and ctx.needs_input_grad[3]
+        if ctx.needs_input_grad[2]:
+            if want_b:
+                top, grad_b = weight_and_bias_gradient(small[:, :fi], g)
+            else:
+                top = weight_gradient(small[:, :fi], g)
+            grad_w = torch.cat([top, weight_gradient(small[:, fi:], g)], dim=0)
+        elif want_b:
+            grad_b = g.sum(dim=0)
+        if ctx.needs_input_grad[1]:
+            grad_small = torch.mm(g, weight.t())  # [len(rows), 2 fi]: d/d aggregated | d/d x[rows] (direct part)
+            grad_agg = grad_small[:, :fi]
+            if ctx.divide:
+                grad_agg.div_(ctx.graph.in_degrees)
+            # the gradient goes where the features were: the right half of an [N, 2 fi] array (its left half was
+            # scratch on the way forward and is left unwritten here): A[rows]^T (d/d aggregated), then the direct
+            # part added onto the rows it belongs to (every row once: deterministic)
+            grad_cat = torch.empty(ctx.nodes, 2 * fi, dtype=torch.float32, device=g.device)
+            target = grad_cat[:, fi:]
+            aggregator._backward(ctx, grad_agg, out=target, accumulate=False)
+            target.index_add_(0, rows, grad_small[:, fi:])
+        return None, grad_cat, grad_w, grad_b, None, None, None, None, None, None
+
+
 class _SageConvLinearFirst(torch.autograd.Function):
     """The same layer with the products taken first: ``A (x W_n) / deg + x W_s + bias``.  Equal to
     aggregate-first up to rounding ((A x) W = A (x W)); the aggregation, its backward and the
@@ -292,11 +343,15 @@ class DistSAGEConvGrad(torch.nn.Module):
             self.weight[:self.in_channels] = lin_neigh_weight.t()
             self.weight[self.in_channels:] = lin_self_weight.t()
 
-    def forward(self, graph, local_nodes_feat: torch.Tensor, layer: int) -> torch.Tensor:
+    def forward(self, graph, local_nodes_feat: torch.Tensor, layer: int,
+                rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         """``local_nodes_feat``: ``[N, in_channels]`` features (staged here, one copy) or an
         already staged ``[N, 2 * in_channels]`` array (``stage_input`` / the fused LayerNorm
-        pass) whose left half this call overwrites."""
+        pass) whose left half this call overwrites.  ``rows`` (local node ids): the output for
+        those nodes only, ``[len(rows), out_channels]`` (aggregate-first order only)."""
         width = local_nodes_feat.size(-1)
+        if self.linear_first and rows is not None:
+            raise RuntimeError("a layer that multiplies first has no row-restricted form")
         if self.linear_first:
             if width not in (self.in_channels, 2 * self.in_channels):
                 raise RuntimeError("Input mismatch: expected %d features (or %d staged), got %d"
@@ -316,6 +371,10 @@ class DistSAGEConvGrad(torch.nn.Module):
                                % (self.in_channels, 2 * self.in_channels, width))
         if not cat.is_cuda or cat.dtype != torch.float32 or not cat.is_contiguous():
             raise RuntimeError("Input mismatch: the staged input must be a contiguous float32 GPU (HIP) tensor")
+        if rows is not None:
+            graph_rows = aggregator.restrict_output_rows(graph, rows, self.is_pre_delay)
+            return _SageConvRows.apply(graph_rows, cat, self.weight, self.bias, layer, self.num_bits, self.is_pre_delay,
+                                       self.training, self.normalize, rows)
         return _SageConv.apply(graph, cat, self.weight, self.bias, layer, self.num_bits, self.is_pre_delay,
                                self.training, self.normalize)
 
@@ -347,11 +406,13 @@ class DistSAGE(torch.nn.Module):
             norm.reset_parameters()
 
     def forward(self, graph, nodes_feats: torch.Tensor, masks: Optional[List[torch.Tensor]] = None,
-                log_probs: bool = True) -> torch.Tensor:
+                log_probs: bool = True, last_rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         """``nodes_feats``: ``[N, in_channels]`` or staged (``stage_input``).  ``masks[i]``: keep
         mask ``[N, hidden]`` of the dropout after layer i (training; drawn here when None).
         ``log_probs=False`` returns the last layer's output before the log-softmax of
-        model/DistSAGE.py:69 (a caller that scores a subset of the nodes applies it to those rows)."""
+        model/DistSAGE.py:69 (a caller that scores a subset of the nodes applies it to those rows).
+        ``last_rows`` (local node ids): evaluate the last layer for those nodes only and return
+        ``[len(last_rows), out_channels]``."""
         for i, conv in enumerate(self.convs[:-1]):
             z = conv(graph, nodes_feats, i)
             keep, scale = None, 1.0
@@ -360,7 +421,7 @@ class DistSAGE(torch.nn.Module):
                 scale = 1.0 / (1.0 - self.dropout)
             norm = self.norms[i]
             nodes_feats = dropout_layernorm_relu(z, keep, scale, norm.weight, norm.bias, norm.eps)
-        out = self.convs[-1](graph, nodes_feats, len(self.convs) - 1)
+        out = self.convs[-1](graph, nodes_feats, len(self.convs) - 1, last_rows)
         return F.log_softmax(out, dim=1) if log_probs else out
 
 
@@ -372,12 +433,20 @@ def make_dropout_masks(num_nodes: int, hidden_channels: int, num_layers: int, p:
 
 def train_step(model: DistSAGE, optimizer, graph, nodes_feats, labels, train_idx, masks=None) -> torch.Tensor:
     """One epoch of train.py:82-98: forward, NLL loss on the training nodes, backward, update.
-    The log-softmax is row-wise, so it is applied to the training rows only: the same loss and
-    gradients as train.py:87-89 without normalising the rows that are not scored."""
+    The loss reads only the training rows of the last layer, so only those are evaluated (or, for a
+    last layer that multiplies first, the zero rows of its gradient are skipped): the same loss and
+    gradients as train.py:87-89, to the rounding of the last layer's dense products."""
     model.train()
     optimizer.zero_grad(set_to_none=True)
-    out = model(graph, nodes_feats, masks, log_probs=False)
-    loss = _mean_nll(F.log_softmax(out[train_idx], dim=1), labels[train_idx])
-    loss.backward()
+    last = model.convs[-1]
+    if last.linear_first:  # no row-restricted form: every node through the last layer, zero gradient rows skipped
+        out = model(graph, nodes_feats, masks, log_probs=False)
+        loss = _mean_nll(F.log_softmax(out[train_idx], dim=1), labels[train_idx])
+        with scored_rows(graph, len(model.convs) - 1, train_idx, last.is_pre_delay):
+            loss.backward()
+    else:
+        out = model(graph, nodes_feats, masks, log_probs=False, last_rows=train_idx)
+        loss = _mean_nll(F.log_softmax(out, dim=1), labels[train_idx])
+        loss.backward()
     optimizer.step()
     return loss.detach()

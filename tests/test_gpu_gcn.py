@@ -363,3 +363,63 @@ def test_fused_layer_with_no_rows(bf16):
     assert x.grad.shape == (0, 32) and not w.grad.any() and not b.grad.any()
     values, header = gcn._FusedLayerPacked.apply(x, w, b, None, 1.0, None, bf16)
     assert values.shape == (0, 64) and header.shape == (0, 4)
+
+
+def _full_step(forward, opt, labels, train_idx):
+    """The train step the long way round: every node through the last layer, the loss on the training rows."""
+    opt.zero_grad(set_to_none=True)
+    out = forward()
+    loss = F.nll_loss(out[train_idx], labels[train_idx])
+    loss.backward()
+    opt.step()
+    return loss.detach()
+
+
+@pytest.mark.parametrize("model_kind", ["gcn", "gcn_separate_kernels", "gcn_linear_first", "gcn_packed", "gcn_bf16", "sage",
+                                        "sage_linear_first"])
+def test_scoring_only_the_training_rows_changes_nothing(model_kind):
+    """A loss over the training rows needs only those rows of the last layer.  The train steps evaluate the last layer
+    for the training rows only (``restrict_output_rows``: every row kept is the same FMA chain); where the last layer
+    has no such form (a SAGE layer that multiplies first) they declare the zero rows of its gradient for the backward
+    pass instead (``scored_rows``: every term skipped is a product with zero).  The gradients are those of the step
+    that evaluates every node -- to the rounding of the last layer's dense products, which now sum the training rows
+    only; bit for bit in the ``scored_rows`` case, where the same kernels run on the same rows."""
+    from gnn_benchmark_amd import sage
+
+    dev = "cuda:0"
+    n, dims = 6000, [32, 64, 64, 12]
+    part = synthetic.partition_edges(n, 4, 2, 6, 1.8, 800, 1500, 9000, seed=3, device=dev)
+    gen = torch.Generator(device=dev).manual_seed(1)
+    x = torch.randn(n, dims[0], device=dev, generator=gen)
+    labels = torch.randint(0, dims[-1], (n,), device=dev, generator=gen)
+    train_idx = torch.randperm(n, device=dev, generator=gen)[: n // 10]
+    results = []
+    for short_cut in (True, False):
+        graph = synthetic.build_partition_graph(part, max(dims), True, exchange=synthetic.SeededHaloExchange(5), device=dev)
+        torch.manual_seed(0)
+        if model_kind.startswith("sage"):
+            model = sage.DistSAGE(dims[0], dims[1], dims[-1], num_layers=3, dropout=0.5, is_pre_delay=True,
+                                  linear_first_when_narrowing=(model_kind == "sage_linear_first")).to(dev)
+            masks = sage.make_dropout_masks(n, dims[1], 3, 0.5, 8, dev)
+            feats = sage.stage_input(x)
+            quick = lambda: sage.train_step(model, opt, graph, feats, labels, train_idx, masks)
+            full = lambda: _full_step(lambda: model(graph, feats, masks), opt, labels, train_idx)
+        else:
+            model = gcn.GCN(dims, gemm="bf16" if model_kind == "gcn_bf16" else "fp32",
+                            linear_first_when_narrowing=(model_kind == "gcn_linear_first"),
+                            packed_activations=(model_kind == "gcn_packed"),
+                            fused_layers=(model_kind != "gcn_separate_kernels")).to(dev)
+            masks = gcn.make_dropout_masks(n, dims, 0.5, 7, dev)
+            quick = lambda: gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks)
+            full = lambda: _full_step(lambda: model(graph, x, True, masks), opt, labels, train_idx)
+        model.train()
+        opt = torch.optim.Adam(model.parameters(), lr=0.01)
+        losses = [float((quick if short_cut else full)())]
+        results.append((losses, [p.grad.detach().clone() for p in model.parameters()]))
+        assert getattr(graph, "backward_row_support", None) is None  # declared for the backward pass only
+    assert np.allclose(results[0][0], results[1][0], rtol=1e-6)
+    for a, b in zip(results[0][1], results[1][1]):
+        if model_kind == "sage_linear_first":
+            assert torch.equal(a, b)
+        else:
+            assert float((a - b).abs().max()) <= 1e-5 * float(b.abs().max()) + 1e-12
