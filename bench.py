@@ -600,8 +600,15 @@ def run_c5(args, graph):
             ("fp32", False, False, True), ("fp32", False, False, False), ("bf16", False, False, True),
             ("fp32", True, False, True), ("bf16", True, False, True), ("fp32", False, True, True),
             ("bf16", False, True, True), ("fp32", True, True, True), ("bf16", True, True, True),
-            ("fp32", True, True, "folded"), ("bf16", True, True, "folded")):
+            ("fp32", True, True, "folded"), ("bf16", True, True, "folded"),
+            ("fp32", False, False, "all_nodes"), ("bf16", False, False, "all_nodes"), ("fp32", True, False, "all_nodes"),
+            ("bf16", True, False, "all_nodes")):
         g = graph
+        # the train step evaluates the last layer for the labelled rows only (the loss reads no others: same loss and
+        # gradients); "all_nodes" sends every node through the last layer, as the reference's epoch does
+        restrict = fused != "all_nodes"
+        if not restrict:
+            fused = True
         if fused == "folded":  # the degree division carried by the matrix values instead of the layers' epilogues
             if folded is None:
                 from gnn_benchmark_amd import sage
@@ -615,15 +622,15 @@ def run_c5(args, graph):
         model = gcn.GCN(dims, gemm=gemm, packed_activations=packed_activations,
                         linear_first_when_narrowing=linear_first, fused_layers=fused).to(dev)
         opt = torch.optim.Adam(model.parameters(), lr=0.01)
-        losses = [float(gcn.train_step(model, opt, g, x, labels, train_idx, True, masks)) for _ in range(2)]
+        losses = [float(gcn.train_step(model, opt, g, x, labels, train_idx, True, masks, restrict)) for _ in range(2)]
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(steps):
-            loss = gcn.train_step(model, opt, g, x, labels, train_idx, True, masks)
+            loss = gcn.train_step(model, opt, g, x, labels, train_idx, True, masks, restrict)
         torch.cuda.synchronize()
         tag = (f"{gemm}_gemm" + ("_packed_activations" if packed_activations else "")
                + ("_linear_first_when_narrowing" if linear_first else "") + ("" if fused else "_separate_kernels")
-               + folded_tag)
+               + folded_tag + ("" if restrict else "_all_nodes_through_last_layer"))
         out[f"train_step_ms_{tag}"] = round((time.perf_counter() - t0) * 1e3 / steps, 2)
         out[f"loss_{tag}"] = [round(v, 5) for v in losses + [float(loss)]]
         del model, opt
@@ -666,8 +673,10 @@ def run_c5_sage(args, graph):
 
     staged = sage.stage_input(x)
     folded = None
-    for tag, fold, linear_first in (("", False, False), ("_folded_degrees", True, False),
-                                    ("_folded_degrees_linear_first_when_narrowing", True, True)):
+    for tag, fold, linear_first, restrict in (
+            ("", False, False, True), ("_folded_degrees", True, False, True),
+            ("_folded_degrees_linear_first_when_narrowing", True, True, True),
+            ("_folded_degrees_all_nodes_through_last_layer", True, False, False)):
         if fold and folded is None:
             folded = sage.fold_in_degrees(graph)
         g = folded if fold else graph
@@ -675,7 +684,7 @@ def run_c5_sage(args, graph):
         model = sage.DistSAGE(dims[0], hidden, dims[-1], num_layers=len(dims) - 1, dropout=0.5, is_pre_delay=True,
                               linear_first_when_narrowing=linear_first).to(dev)
         opt = torch.optim.Adam(model.parameters(), lr=0.01)
-        ms, losses = timed(lambda: sage.train_step(model, opt, g, staged, labels, train_idx, masks))
+        ms, losses = timed(lambda: sage.train_step(model, opt, g, staged, labels, train_idx, masks, restrict))
         out["train_step_ms" + tag], out["loss" + tag] = ms, losses
         del model, opt, g
         torch.cuda.empty_cache()

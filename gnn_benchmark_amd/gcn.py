@@ -510,12 +510,17 @@ def _mean_nll(log_probs: torch.Tensor, target: torch.Tensor) -> torch.Tensor:
     return -log_probs.gather(1, target.unsqueeze(1)).mean()
 
 
-def train_step(model: GCN, optimizer, graph, x, labels, train_idx, is_pre_delay: bool, masks) -> torch.Tensor:
+def train_step(model: GCN, optimizer, graph, x, labels, train_idx, is_pre_delay: bool, masks,
+               restrict_last_layer: bool = True) -> torch.Tensor:
     """forward, NLL loss on the labelled nodes, backward, optimizer update.  Only the labelled rows of the last layer
-    are evaluated (the loss reads no others): the same loss, gradients and update as evaluating every node."""
+    are evaluated (the loss reads no others): the same loss, gradients and update as evaluating every node, which
+    ``restrict_last_layer=False`` does."""
     model.train()
     optimizer.zero_grad(set_to_none=True)
-    out = model(graph, x, is_pre_delay, masks, log_probs=False, last_rows=train_idx)
+    if restrict_last_layer:
+        out = model(graph, x, is_pre_delay, masks, log_probs=False, last_rows=train_idx)
+    else:  # every node through the last layer, as the reference's epoch does; the loss reads the labelled rows
+        out = model(graph, x, is_pre_delay, masks, log_probs=False)[train_idx]
     loss = _mean_nll(F.log_softmax(out, dim=1), labels[train_idx])
     loss.backward()
     optimizer.step()

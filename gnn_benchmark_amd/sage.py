@@ -431,7 +431,8 @@ def make_dropout_masks(num_nodes: int, hidden_channels: int, num_layers: int, p:
     return [torch.rand(num_nodes, hidden_channels, device=device, generator=gen) >= p for _ in range(num_layers - 1)]
 
 
-def train_step(model: DistSAGE, optimizer, graph, nodes_feats, labels, train_idx, masks=None) -> torch.Tensor:
+def train_step(model: DistSAGE, optimizer, graph, nodes_feats, labels, train_idx, masks=None,
+               restrict_last_layer: bool = True) -> torch.Tensor:
     """One epoch of train.py:82-98: forward, NLL loss on the training nodes, backward, update.
     The loss reads only the training rows of the last layer, so only those are evaluated (or, for a
     last layer that multiplies first, the zero rows of its gradient are skipped): the same loss and
@@ -439,7 +440,11 @@ def train_step(model: DistSAGE, optimizer, graph, nodes_feats, labels, train_idx
     model.train()
     optimizer.zero_grad(set_to_none=True)
     last = model.convs[-1]
-    if last.linear_first:  # no row-restricted form: every node through the last layer, zero gradient rows skipped
+    if not restrict_last_layer:  # every node through the last layer, exactly as train.py:87-90
+        out = model(graph, nodes_feats, masks, log_probs=False)
+        loss = _mean_nll(F.log_softmax(out[train_idx], dim=1), labels[train_idx])
+        loss.backward()
+    elif last.linear_first:  # no row-restricted form: every node through the last layer, zero gradient rows skipped
         out = model(graph, nodes_feats, masks, log_probs=False)
         loss = _mean_nll(F.log_softmax(out[train_idx], dim=1), labels[train_idx])
         with scored_rows(graph, len(model.convs) - 1, train_idx, last.is_pre_delay):

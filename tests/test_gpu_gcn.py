@@ -423,3 +423,41 @@ def test_scoring_only_the_training_rows_changes_nothing(model_kind):
             assert torch.equal(a, b)
         else:
             assert float((a - b).abs().max()) <= 1e-5 * float(b.abs().max()) + 1e-12
+
+
+@pytest.mark.parametrize("model_kind", ["gcn", "sage"])
+def test_train_step_can_send_every_node_through_the_last_layer(model_kind):
+    """``restrict_last_layer=False`` is the reference's epoch (train.py:87-90): every node through every layer, the
+    loss on the labelled rows.  The gradients of the weights are those of the step spelled out with torch's own
+    ``nll_loss`` (the log-softmax of a row does not depend on which other rows are evaluated beside it)."""
+    from gnn_benchmark_amd import sage
+
+    dev = "cuda:0"
+    n, dims = 5000, [32, 64, 64, 12]
+    part = synthetic.partition_edges(n, 4, 2, 6, 1.8, 700, 1200, 8000, seed=4, device=dev)
+    gen = torch.Generator(device=dev).manual_seed(2)
+    x = torch.randn(n, dims[0], device=dev, generator=gen)
+    labels = torch.randint(0, dims[-1], (n,), device=dev, generator=gen)
+    train_idx = torch.randperm(n, device=dev, generator=gen)[: n // 8]
+    results = []
+    for own_step in (True, False):
+        graph = synthetic.build_partition_graph(part, max(dims), True, exchange=synthetic.SeededHaloExchange(6), device=dev)
+        torch.manual_seed(0)
+        if model_kind == "sage":
+            model = sage.DistSAGE(dims[0], dims[1], dims[-1], num_layers=3, dropout=0.5, is_pre_delay=True).to(dev)
+            masks = sage.make_dropout_masks(n, dims[1], 3, 0.5, 8, dev)
+            feats = sage.stage_input(x)
+            step = lambda: sage.train_step(model, opt, graph, feats, labels, train_idx, masks, restrict_last_layer=False)
+            full = lambda: _full_step(lambda: model(graph, feats, masks), opt, labels, train_idx)
+        else:
+            model = gcn.GCN(dims).to(dev)
+            masks = gcn.make_dropout_masks(n, dims, 0.5, 7, dev)
+            step = lambda: gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks, restrict_last_layer=False)
+            full = lambda: _full_step(lambda: model(graph, x, True, masks), opt, labels, train_idx)
+        model.train()
+        opt = torch.optim.Adam(model.parameters(), lr=0.01)
+        loss = float((step if own_step else full)())
+        results.append((loss, [p.grad.detach().clone() for p in model.parameters()]))
+    assert np.isclose(results[0][0], results[1][0], rtol=1e-6)
+    for a, b in zip(results[0][1], results[1][1]):
+        assert float((a - b).abs().max()) <= 1e-5 * float(b.abs().max()) + 1e-12
