@@ -46,7 +46,6 @@ What differs from the reference, on purpose:
 (``packed.py``: non-zero values at the front of each row plus a bitmap header); only the
 two forward products that read the features differ.
 """
-import copy
 
 import torch
 
@@ -332,6 +331,21 @@ def select_rows(m: SparseTensor, rows: torch.Tensor) -> SparseTensor:
                         sparse_sizes=(rows.numel(), m.sparse_size(1)), is_sorted=True)
 
 
+class _RowRestrictedGraph:
+    """``graph`` with a few attributes replaced; everything else (buffers, splits, exchange hooks, the matrices that
+    feed the send buffer) is read from ``graph`` at the time of use, so what is attached to it later is seen here."""
+
+    def __init__(self, graph, replaced: dict):
+        self.__dict__["_graph"] = graph
+        self.__dict__.update(replaced)
+
+    def __getattr__(self, name):  # only reached for names this object does not hold itself
+        graph = self.__dict__.get("_graph")
+        if graph is None or name.startswith("__"):
+            raise AttributeError(name)
+        return getattr(graph, name)
+
+
 def restrict_output_rows(graph, rows: torch.Tensor, is_pre_delay: bool):
     """A view of ``graph`` whose aggregation produces only the output rows ``rows`` (local node ids, in that order):
     the local matrix and the matrix that adds the received rows keep just those rows, the in-degrees likewise; what
@@ -343,15 +357,14 @@ def restrict_output_rows(graph, rows: torch.Tensor, is_pre_delay: bool):
     key = (rows.data_ptr(), rows.numel(), rows._version, bool(is_pre_delay), id(graph.local_adj_t))
     hit = cache.get(key)
     if hit is None:
-        g = copy.copy(graph)
-        g.__dict__.pop("_restricted_rows_cache", None)
-        g.local_adj_t = select_rows(graph.local_adj_t, rows)
         name = "adj_t_pre_post_aggr_from" if is_pre_delay else "remote_adj_t"
         remote = getattr(graph, name, None)
-        if remote is not None:
-            setattr(g, name, select_rows(remote, rows))
-        g.in_degrees = graph.in_degrees[rows].contiguous()
-        for m in (g.local_adj_t, getattr(g, name, None)):
+        g = _RowRestrictedGraph(graph, {
+            "local_adj_t": select_rows(graph.local_adj_t, rows),
+            name: None if remote is None else select_rows(remote, rows),
+            "in_degrees": graph.in_degrees[rows].contiguous(),
+            "backward_row_support": None})
+        for m in (g.local_adj_t, getattr(g, name)):
             if m is not None:
                 m.get_plan()
                 m.get_plan_for_transpose()
