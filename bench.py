@@ -601,6 +601,7 @@ def run_c5(args, graph):
             ("fp32", True, False, True), ("bf16", True, False, True), ("fp32", False, True, True),
             ("bf16", False, True, True), ("fp32", True, True, True), ("bf16", True, True, True),
             ("fp32", True, True, "folded"), ("bf16", True, True, "folded"),
+            ("bf16x3", False, False, True), ("bf16x3", True, False, True),
             ("fp32", False, False, "all_nodes"), ("bf16", False, False, "all_nodes"), ("fp32", True, False, "all_nodes"),
             ("bf16", True, False, "all_nodes")):
         g = graph

@@ -38,6 +38,7 @@ EXPORTS = (
     "gnnagg_pack_keep_bits",
     "gnnagg_linear_bias_relu_dropout_f32",
     "gnnagg_linear_bias_relu_dropout_bf16_f32",
+    "gnnagg_linear_bias_relu_dropout_bf16x3_f32",
     "gnnagg_linear_bias_relu_dropout_pack_f32",
     "gnnagg_wgrad_relu_dropout_backward_workspace_bytes",
     "gnnagg_wgrad_relu_dropout_backward_f32",
@@ -138,6 +139,8 @@ def lib() -> ctypes.CDLL:
                                                       i64, i64, vp]
     L.gnnagg_linear_bias_relu_dropout_bf16_f32.restype = i32
     L.gnnagg_linear_bias_relu_dropout_bf16_f32.argtypes = L.gnnagg_linear_bias_relu_dropout_f32.argtypes
+    L.gnnagg_linear_bias_relu_dropout_bf16x3_f32.restype = i32
+    L.gnnagg_linear_bias_relu_dropout_bf16x3_f32.argtypes = L.gnnagg_linear_bias_relu_dropout_f32.argtypes
     L.gnnagg_linear_bias_relu_dropout_pack_f32.restype = i32
     L.gnnagg_linear_bias_relu_dropout_pack_f32.argtypes = [vp, i64, vp, i64, vp, vp, vp, ctypes.c_float, vp, vp, i64, i64,
                                                            i64, i32, vp]

@@ -14,6 +14,28 @@ typedef short shortx4 __attribute__((ext_vector_type(4)));
 typedef float floatx2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+// Four fp32 values as three times four bf16: hi = bf16(v), mid = bf16(v - hi), lo = bf16(v - hi - mid).  Both
+// differences are exact in fp32, so hi + mid + lo is v to 2^-25 of its size (three 8-bit pieces of a 24-bit mantissa).
+__device__ inline void split_bf16x3(float a, float b, float c, float d, shortx4 (&out)[3]) {
+    union {
+        bf16x2 h[2];
+        shortx4 s;
+    } u[3];
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+        const floatx2 v = q == 0 ? floatx2{a, b} : floatx2{c, d};
+        u[0].h[q] = __builtin_convertvector(v, bf16x2);
+        const floatx2 r = v - __builtin_convertvector(u[0].h[q], floatx2);
+        u[1].h[q] = __builtin_convertvector(r, bf16x2);
+        u[2].h[q] = __builtin_convertvector(r - __builtin_convertvector(u[1].h[q], floatx2), bf16x2);
+    }
+    out[0] = u[0].s;
+    out[1] = u[1].s;
+    out[2] = u[2].s;
+}
+
 // four fp32 values -> four bf16 (round to nearest even, the hardware's packed conversion) in 8 bytes
 __device__ inline shortx4 to_bf16x4(float a, float b, float c, float d) {
     union {

@@ -46,6 +46,13 @@ struct LinearArgs {
     int relu;
 };
 
+// SPLIT form, LDS records: a row of A / a column of W is 32 bytes per plane, its 16 k in the order 0-3, 8-11 | 4-7,
+// 12-15 (the 16 bytes a lane of either half-wave feeds to one MFMA sit together); rows / columns whose bit 3 is set
+// hold the two halves swapped, and the columns of W are permuted inside each group of 32 (both so that the 16-byte
+// reads of neighbouring lanes and the 8-byte writes of the staging threads spread over the banks).
+__device__ inline int split_offset(int kq, int row) { return (16 * (kq & 1) + 8 * (kq >> 1)) ^ (16 * ((row >> 3) & 1)); }
+__device__ inline int split_column(int col) { return (col & ~7) | ((col & 7) ^ ((col >> 3) & 3)); }
+
 template <int WM, int WN>
 struct LinearShape {
     static constexpr int kRows = 64 * WM;            // rows of A per block
@@ -59,16 +66,29 @@ struct LinearShape {
     static constexpr int kLdh = 2 * kChunk + 8;      // bytes between staged rows / columns
     static constexpr int kBufBytesH = (kRows + 64 * WN) * kLdh;
     static constexpr int kSmemBytesH = 2 * kBufBytesH;
+    // SPLIT form: three bf16 planes (hi, mid, lo) of the rows of A and of the columns of W, 16 k = 32 bytes a record
+    static constexpr int kPlaneA = kRows * 32;
+    static constexpr int kPlaneW = 64 * WN * 32;
+    static constexpr int kBufBytesS = 3 * (kPlaneA + kPlaneW);
+    static constexpr int kSmemBytesS = 2 * kBufBytesS;
 };
 
-template <int WM, int WN, bool BF16, bool PACK>
+// SPLIT (BF16 == false): every fp32 operand value is cut into three bf16 pieces on its way into LDS and a product
+// runs as six bf16 MFMAs (hi*hi, hi*mid, mid*hi, mid*mid, hi*lo, lo*hi; the pieces left out are below 2^-24 of
+// |a||w|, the size of an fp32 rounding) accumulated in fp32 -- 192 MFMA cycles per 32 x 32 x 16 block of products
+// instead of the fp32 MFMA's 512.
+template <int WM, int WN, bool BF16, bool PACK, bool SPLIT = false>
 __global__ __launch_bounds__(256, 2) void linear_kernel(const LinearArgs p) {
+    static_assert(!(BF16 && SPLIT), "the split form stages fp32");
+    static_assert(!SPLIT || kChunk == 16, "one 32x32x16 MFMA group per chunk");
     using S = LinearShape<WM, WN>;
     extern __shared__ __align__(16) float smem[];
     float *dump = smem + 2 * S::kBufFloats + 4 * (int)threadIdx.x;  // (fp32 form only)
     char *smem_h = reinterpret_cast<char *>(smem);                  // (BF16 form)
     // PACK: non-zeros of each tile row in the block's left column half, behind the staging buffers
-    int *row_count = reinterpret_cast<int *>(smem_h + (BF16 ? (size_t)S::kSmemBytesH : (size_t)S::kSmemFloats * sizeof(float)));
+    int *row_count = reinterpret_cast<int *>(smem_h + (BF16    ? (size_t)S::kSmemBytesH
+                                                       : SPLIT ? (size_t)S::kSmemBytesS
+                                                               : (size_t)S::kSmemFloats * sizeof(float)));
 
     const int tid = (int)threadIdx.x;
     const int lane = tid & 63;
@@ -101,8 +121,9 @@ __global__ __launch_bounds__(256, 2) void linear_kernel(const LinearArgs p) {
     int a_dst[S::kVecA];
 #pragma unroll
     for (int j = 0; j < S::kVecA; ++j)
-        a_dst[j] = BF16 ? ((tid >> 2) + 64 * j) * S::kLdh + 8 * (tid & 3)      // bytes
-                        : ((tid >> 2) + 64 * j) * S::kLda + 4 * (tid & 3);     // floats
+        a_dst[j] = BF16    ? ((tid >> 2) + 64 * j) * S::kLdh + 8 * (tid & 3)                          // bytes
+                   : SPLIT ? ((tid >> 2) + 64 * j) * 32 + split_offset(tid & 3, tid >> 2)             // bytes
+                           : ((tid >> 2) + 64 * j) * S::kLda + 4 * (tid & 3);                         // floats
     auto enter_tile = [&](int64_t t) {
 #pragma unroll
         for (int j = 0; j < S::kVecA; ++j) {
@@ -119,27 +140,42 @@ __global__ __launch_bounds__(256, 2) void linear_kernel(const LinearArgs p) {
     auto store_a = [&](int buf) {
 #pragma unroll
         for (int j = 0; j < S::kVecA; ++j) {
-            if (BF16)
+            if (BF16) {
                 *reinterpret_cast<shortx4 *>(smem_h + buf * S::kBufBytesH + a_dst[j]) =
                     to_bf16x4(areg[j].x, areg[j].y, areg[j].z, areg[j].w);
-            else
+            } else if (SPLIT) {
+                shortx4 piece[3];
+                split_bf16x3(areg[j].x, areg[j].y, areg[j].z, areg[j].w, piece);
+#pragma unroll
+                for (int q = 0; q < 3; ++q)
+                    *reinterpret_cast<shortx4 *>(smem_h + buf * S::kBufBytesS + q * S::kPlaneA + a_dst[j]) = piece[q];
+            } else
                 *reinterpret_cast<floatx4 *>(smem + buf * S::kBufFloats + a_dst[j]) = areg[j];
         }
     };
     ChunkLoader<S::kVecB, S::kLdb> lw;
-    if (!BF16) lw.init(tid, p.n, p.ldw);
+    if (!BF16 && !SPLIT) lw.init(tid, p.n, p.ldw);
     // BF16: thread u owns the 4 x 4 block (k-quad u / (n/4), column-quad u % (n/4)) of a chunk of W; threads
     // past the 4 * (n/4) blocks repeat earlier ones (same values to the same place)
     floatx4 wreg[4];
     int w_src = 0, w_dst = 0;
+    int w_dst_split[4] = {0, 0, 0, 0};
     if (BF16) {
         const int nq = p.n / 4;
         const int u = tid % (4 * nq);
         w_src = 4 * (u / nq) * p.ldw + 4 * (u % nq);
         w_dst = S::kRows * S::kLdh + 4 * (u % nq) * S::kLdh + 8 * (u / nq);
     }
+    if (SPLIT) {  // k-quads fastest: four neighbouring threads fill one column's record
+        const int u = tid % p.n;
+        const int kq = u & 3, cq = u >> 2;
+        w_src = 4 * kq * p.ldw + 4 * cq;
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+            w_dst_split[c] = 3 * S::kPlaneA + split_column(4 * cq + c) * 32 + split_offset(kq, 4 * cq + c);
+    }
     auto fetch_w = [&](const float *wc) {
-        if (BF16) {
+        if (BF16 || SPLIT) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) wreg[c] = *reinterpret_cast<const floatx4 *>(wc + w_src + c * p.ldw);
         } else {
@@ -152,6 +188,16 @@ __global__ __launch_bounds__(256, 2) void linear_kernel(const LinearArgs p) {
 #pragma unroll
             for (int c = 0; c < 4; ++c)  // column 4 q + c of the block: its four consecutive k
                 *reinterpret_cast<shortx4 *>(dst + c * S::kLdh) = to_bf16x4(wreg[0][c], wreg[1][c], wreg[2][c], wreg[3][c]);
+        } else if (SPLIT) {
+            char *dst = smem_h + buf * S::kBufBytesS;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                shortx4 piece[3];
+                split_bf16x3(wreg[0][c], wreg[1][c], wreg[2][c], wreg[3][c], piece);
+#pragma unroll
+                for (int q = 0; q < 3; ++q)
+                    *reinterpret_cast<shortx4 *>(dst + q * S::kPlaneW + w_dst_split[c]) = piece[q];
+            }
         } else {
             lw.store_all(smem + buf * S::kBufFloats + S::kRows * S::kLda, dump);
         }
@@ -179,6 +225,34 @@ __global__ __launch_bounds__(256, 2) void linear_kernel(const LinearArgs p) {
 #pragma unroll
                     for (int j = 0; j < WN; ++j)
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(hb[s][j], ha[s][i], acc[i][j], 0, 0, 0);
+            }
+            return;
+        }
+        if (SPLIT) {
+            const int half = 16 * (kk ^ ((idx >> 3) & 1));
+            const char *ab = smem_h + buf * S::kBufBytesS + (m0 + idx) * 32 + half;
+            const char *wb = smem_h + buf * S::kBufBytesS + 3 * S::kPlaneA + (n0 + split_column(idx)) * 32 + half;
+            bf16x8 a3[WM][3];
+#pragma unroll
+            for (int i = 0; i < WM; ++i)
+#pragma unroll
+                for (int q = 0; q < 3; ++q)
+                    a3[i][q] = *reinterpret_cast<const bf16x8 *>(ab + q * S::kPlaneA + 32 * i * 32);
+#pragma unroll
+            for (int j = 0; j < WN; ++j) {
+                bf16x8 b3[3];
+#pragma unroll
+                for (int q = 0; q < 3; ++q) b3[q] = *reinterpret_cast<const bf16x8 *>(wb + q * S::kPlaneW + 32 * j * 32);
+#pragma unroll
+                for (int i = 0; i < WM; ++i) {  // smallest pieces first
+                    floatx16 c = acc[i][j];
+                    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b3[2], a3[i][0], c, 0, 0, 0);
+                    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b3[0], a3[i][2], c, 0, 0, 0);
+                    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b3[1], a3[i][1], c, 0, 0, 0);
+                    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b3[1], a3[i][0], c, 0, 0, 0);
+                    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b3[0], a3[i][1], c, 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b3[0], a3[i][0], c, 0, 0, 0);
+                }
             }
             return;
         }
@@ -392,37 +466,39 @@ __global__ __launch_bounds__(256, 2) void linear_kernel(const LinearArgs p) {
     }
 }
 
-template <int WM, int WN, bool BF16, bool PACK>
+template <int WM, int WN, bool BF16, bool PACK, bool SPLIT>
 int launch_linear(const LinearArgs &p, hipStream_t st) {
     using S = LinearShape<WM, WN>;
-    constexpr size_t smem = (BF16 ? (size_t)S::kSmemBytesH : (size_t)S::kSmemFloats * sizeof(float)) +
+    constexpr size_t smem = (BF16    ? (size_t)S::kSmemBytesH
+                             : SPLIT ? (size_t)S::kSmemBytesS
+                                     : (size_t)S::kSmemFloats * sizeof(float)) +
                             (PACK ? S::kRows * sizeof(int) : 0);
-    GNNAGG_HIP(allow_lds(reinterpret_cast<const void *>(&linear_kernel<WM, WN, BF16, PACK>), smem));
+    GNNAGG_HIP(allow_lds(reinterpret_cast<const void *>(&linear_kernel<WM, WN, BF16, PACK, SPLIT>), smem));
     int dev = 0, cus = 0;
     GNNAGG_HIP(hipGetDevice(&dev));
     GNNAGG_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
     const int64_t tiles = (p.rows + S::kRows - 1) / S::kRows;
     const int64_t resident = 2 * (int64_t)(cus > 0 ? cus : 256);  // two blocks per CU, each walks its share of the tiles
     const unsigned blocks = (unsigned)(tiles < resident ? tiles : resident);
-    hipLaunchKernelGGL((linear_kernel<WM, WN, BF16, PACK>), dim3(blocks), dim3(256), smem, st, p);
+    hipLaunchKernelGGL((linear_kernel<WM, WN, BF16, PACK, SPLIT>), dim3(blocks), dim3(256), smem, st, p);
     GNNAGG_HIP(hipGetLastError());
     return GNNAGG_OK;
 }
 
-template <bool BF16>
+template <bool BF16, bool SPLIT>
 int dispatch_linear(const LinearArgs &p, hipStream_t st) {
     if (p.header) {  // packed output: widths 32, 64, 128, 256
         switch ((p.n + 63) / 64) {
-            case 1: return launch_linear<2, 1, BF16, true>(p, st);
-            case 2: return launch_linear<2, 2, BF16, true>(p, st);
-            default: return launch_linear<2, 4, BF16, true>(p, st);
+            case 1: return launch_linear<2, 1, BF16, true, SPLIT>(p, st);
+            case 2: return launch_linear<2, 2, BF16, true, SPLIT>(p, st);
+            default: return launch_linear<2, 4, BF16, true, SPLIT>(p, st);
         }
     }
     switch ((p.n + 63) / 64) {
-        case 1: return launch_linear<2, 1, BF16, false>(p, st);
-        case 2: return launch_linear<2, 2, BF16, false>(p, st);
-        case 3: return launch_linear<2, 3, BF16, false>(p, st);
-        default: return launch_linear<2, 4, BF16, false>(p, st);
+        case 1: return launch_linear<2, 1, BF16, false, SPLIT>(p, st);
+        case 2: return launch_linear<2, 2, BF16, false, SPLIT>(p, st);
+        case 3: return launch_linear<2, 3, BF16, false, SPLIT>(p, st);
+        default: return launch_linear<2, 4, BF16, false, SPLIT>(p, st);
     }
 }
 
@@ -479,7 +555,8 @@ extern "C" int gnnagg_pack_keep_bits(const void *keep, uint32_t *bits, int64_t r
 }
 
 namespace {
-int run_linear(bool bf16, const float *x, int64_t x_stride, const float *w, int64_t w_stride, const float *bias,
+// form: 0 fp32 MFMA, 1 operands rounded to bf16, 2 every fp32 operand as three bf16 pieces (six bf16 MFMAs per product)
+int run_linear(int form, const float *x, int64_t x_stride, const float *w, int64_t w_stride, const float *bias,
                const uint32_t *keep_bits, const float *row_div, float scale, int relu, float *y, int64_t y_stride,
                uint32_t *header, int64_t rows, int64_t k, int64_t n, void *stream) {
     GNNAGG_REQUIRE(x_stride < (1 << 27) && w_stride < (1 << 27) && y_stride < (1 << 27) && k < (1 << 27) && n < (1 << 27),
@@ -492,8 +569,13 @@ int run_linear(bool bf16, const float *x, int64_t x_stride, const float *w, int6
     if (header && (!relu || y_stride != n))
         return fail(GNNAGG_ERR_INVALID, "packed output follows a ReLU and has row stride n");
     if (rows == 0) return GNNAGG_OK;
-    return bf16 ? dispatch_linear<true>(p, static_cast<hipStream_t>(stream))
-                : dispatch_linear<false>(p, static_cast<hipStream_t>(stream));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (form) {
+        case 0: return dispatch_linear<false, false>(p, st);
+        case 1: return dispatch_linear<true, false>(p, st);
+        case 2: return dispatch_linear<false, true>(p, st);
+        default: return fail(GNNAGG_ERR_INVALID, "product form is 0 (fp32), 1 (bf16 inputs) or 2 (bf16 x 3 pieces), got %d", form);
+    }
 }
 }  // namespace
 
@@ -501,7 +583,16 @@ extern "C" int gnnagg_linear_bias_relu_dropout_f32(const float *x, int64_t x_str
                                                    const float *bias, const uint32_t *keep_bits, const float *row_div,
                                                    float scale, int relu, float *y, int64_t y_stride, int64_t rows,
                                                    int64_t k, int64_t n, void *stream) {
-    return run_linear(false, x, x_stride, w, w_stride, bias, keep_bits, row_div, scale, relu, y, y_stride, nullptr, rows,
+    return run_linear(0, x, x_stride, w, w_stride, bias, keep_bits, row_div, scale, relu, y, y_stride, nullptr, rows,
+                      k, n, stream);
+}
+
+extern "C" int gnnagg_linear_bias_relu_dropout_bf16x3_f32(const float *x, int64_t x_stride, const float *w,
+                                                          int64_t w_stride, const float *bias, const uint32_t *keep_bits,
+                                                          const float *row_div, float scale, int relu, float *y,
+                                                          int64_t y_stride, int64_t rows, int64_t k, int64_t n,
+                                                          void *stream) {
+    return run_linear(2, x, x_stride, w, w_stride, bias, keep_bits, row_div, scale, relu, y, y_stride, nullptr, rows,
                       k, n, stream);
 }
 
@@ -510,7 +601,7 @@ extern "C" int gnnagg_linear_bias_relu_dropout_bf16_f32(const float *x, int64_t 
                                                         const float *row_div, float scale, int relu, float *y,
                                                         int64_t y_stride, int64_t rows, int64_t k, int64_t n,
                                                         void *stream) {
-    return run_linear(true, x, x_stride, w, w_stride, bias, keep_bits, row_div, scale, relu, y, y_stride, nullptr, rows,
+    return run_linear(1, x, x_stride, w, w_stride, bias, keep_bits, row_div, scale, relu, y, y_stride, nullptr, rows,
                       k, n, stream);
 }
 
@@ -520,6 +611,6 @@ extern "C" int gnnagg_linear_bias_relu_dropout_pack_f32(const float *x, int64_t 
                                                         uint32_t *header, int64_t rows, int64_t k, int64_t n,
                                                         int bf16_inputs, void *stream) {
     GNNAGG_REQUIRE(header || rows == 0, "null header");
-    return run_linear(bf16_inputs != 0, x, x_stride, w, w_stride, bias, keep_bits, row_div, scale, 1, y_packed, n, header,
+    return run_linear(bf16_inputs, x, x_stride, w, w_stride, bias, keep_bits, row_div, scale, 1, y_packed, n, header,
                       rows, k, n, stream);
 }

@@ -15,7 +15,10 @@ activations a layer whose widths the kernels take runs fused (``_FusedLayer``): 
 product (fp32, or bf16 inputs), the degree division, bias, ReLU and dropout are one libgnnagg
 kernel, and in the gradient direction the ReLU / dropout mask, the degree division, the bias
 gradient and the weight gradient are another; the fp32 input-gradient product stays with the
-BLAS library, the bf16-input one is the same libgnnagg product kernel.
+BLAS library, the bf16-input one is the same libgnnagg product kernel.  ``gemm="bf16x3"`` keeps
+fp32 accuracy but feeds the matrix units every fp32 operand as three bf16 pieces (six bf16 MFMAs
+a product, a fraction of the fp32 MFMA's cycles): the layer product and the input-gradient
+product run that way, the weight gradient stays the fp32 kernel.
 """
 import contextlib
 from typing import List, Optional, Sequence
@@ -110,6 +113,31 @@ class _Fp32Linear(torch.autograd.Function):
         return gx, gw
 
 
+def _product_bf16x3(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """a @ b with every fp32 operand fed to the matrix units as three bf16 pieces (fp32 accuracy); the BLAS library's
+    fp32 product for shapes the kernel does not take."""
+    if a.is_cuda and a.dtype == torch.float32 and _lib.lib().gnnagg_linear_shape_supported(a.size(1), b.size(1)):
+        return _fused_product(_kernel_ready(a), b.contiguous(), None, None, None, 1.0, False, BF16X3)
+    return torch.mm(a, b)
+
+
+class _Bf16x3Linear(torch.autograd.Function):
+    """y = x @ w, the product and the input-gradient product in the bf16 x 3 form of libgnnagg's product kernel; the
+    weight gradient in the fp32 MFMA kernel."""
+
+    @staticmethod
+    def forward(ctx, x, w):
+        ctx.save_for_backward(x, w)
+        return _product_bf16x3(x, w)
+
+    @staticmethod
+    def backward(ctx, g):
+        x, w = ctx.saved_tensors
+        gx = _product_bf16x3(g, w.t()) if ctx.needs_input_grad[0] else None
+        gw = weight_gradient(x, g) if ctx.needs_input_grad[1] else None
+        return gx, gw
+
+
 def pack_keep_mask(keep: torch.Tensor) -> torch.Tensor:
     """Bool / uint8 keep-mask [rows, feat] -> int32 [rows, ceil(feat / 32)]: bit q of word (r, v)
     is keep[r, 32 v + q].  The form the fused layer kernel reads (1 bit instead of 1 byte per unit)."""
@@ -145,12 +173,19 @@ def _kernel_ready(x: torch.Tensor) -> torch.Tensor:
     return x.contiguous()
 
 
-def _fused_product(x, w, bias, keep_bits, row_div, scale, relu, bf16):
+# how the matrix units see the fp32 operands of a product (the result is accumulated and returned in fp32):
+FP32, BF16, BF16X3 = 0, 1, 2  # as they are / rounded to bf16 / as three bf16 pieces each (six bf16 MFMAs a product:
+#                               fp32 accuracy at a fraction of the fp32 MFMA's cycles)
+_FORMS = {"fp32": FP32, "bf16": BF16, "bf16x3": BF16X3}
+
+
+def _fused_product(x, w, bias, keep_bits, row_div, scale, relu, form):
     """The one-kernel layer product of libgnnagg on kernel-ready operands."""
     rows, k, n = x.size(0), x.size(1), w.size(1)
     y = torch.empty(rows, n, dtype=torch.float32, device=x.device)
     L = _lib.lib()
-    entry = L.gnnagg_linear_bias_relu_dropout_bf16_f32 if bf16 else L.gnnagg_linear_bias_relu_dropout_f32
+    entry = (L.gnnagg_linear_bias_relu_dropout_f32, L.gnnagg_linear_bias_relu_dropout_bf16_f32,
+             L.gnnagg_linear_bias_relu_dropout_bf16x3_f32)[int(form)]
     with torch.cuda.device(x.device):
         _lib.check(entry(_lib.ptr(x), _row_stride(x), _lib.ptr(w), n, _lib.ptr(bias), _lib.ptr(keep_bits),
                          _lib.ptr(row_div), float(scale), 1 if relu else 0, _lib.ptr(y), n, rows, k, n,
@@ -163,11 +198,13 @@ class _FusedLayer(torch.autograd.Function):
     ``keep_bits`` None: y = (x @ w) / row_div + bias, the last layer).  The gradient direction
     is one more kernel -- mask, degree division, bias gradient and weight gradient in a single
     pass over x, the incoming gradient and y -- plus the product for the input gradient.  With
-    ``bf16`` all three products round their operands to bf16 on the way into the matrix units
-    (fp32 accumulation); mask, division and bias gradient stay in fp32."""
+    ``form`` ``BF16`` all three products round their operands to bf16 on the way into the matrix units
+    (fp32 accumulation); with ``BF16X3`` the layer product and the input-gradient product feed every operand
+    as three bf16 pieces (fp32 accuracy; the weight gradient is the fp32 kernel); mask, division and bias
+    gradient stay in fp32."""
 
     @staticmethod
-    def forward(ctx, x, w, bias, keep_bits, scale, row_div, relu, bf16=False):
+    def forward(ctx, x, w, bias, keep_bits, scale, row_div, relu, form=FP32):
         rows, k, n = x.size(0), x.size(1), w.size(1)
         if keep_bits is not None and (keep_bits.dtype != torch.int32 or keep_bits.shape != (rows, (n + 31) // 32)
                                       or not keep_bits.is_contiguous()):
@@ -180,21 +217,21 @@ class _FusedLayer(torch.autograd.Function):
             # the gradient reads which units count off the output (y > 0), which needs the ReLU in front
             raise RuntimeError("Input mismatch: the fused layer applies dropout behind a ReLU only")
         w = w.contiguous()
-        y = _fused_product(x, w, bias.contiguous(), keep_bits, row_div, scale, relu, bf16)
+        y = _fused_product(x, w, bias.contiguous(), keep_bits, row_div, scale, relu, form)
         ctx.save_for_backward(x, w, y if relu else None)
         ctx.scale = float(scale)
         ctx.row_div = row_div
-        ctx.bf16 = bool(bf16)
+        ctx.form = int(form)
         return y
 
     @staticmethod
     def backward(ctx, grad_y):
         x, w, y = ctx.saved_tensors
-        grads = _fused_backward(x, w, grad_y, y, None, ctx.row_div, ctx.scale, ctx.bf16, ctx.needs_input_grad[0])
+        grads = _fused_backward(x, w, grad_y, y, None, ctx.row_div, ctx.scale, ctx.form, ctx.needs_input_grad[0])
         return grads + (None, None, None, None, None)
 
 
-def _fused_backward(x, w, grad_y, y, header, row_div, scale, bf16, want_x):
+def _fused_backward(x, w, grad_y, y, header, row_div, scale, form, want_x):
     """(grad_x, grad_w, grad_bias) of the fused layer: one pass of the weight-gradient kernel (mask from ``y`` or from
     the packed output's ``header``, degree division, bias gradient, weight gradient) plus the input-gradient product."""
     grad_y = _kernel_ready(grad_y)
@@ -206,6 +243,7 @@ def _fused_backward(x, w, grad_y, y, header, row_div, scale, bf16, want_x):
     grad_w = torch.empty(k, n, dtype=torch.float32, device=x.device)
     grad_bias = torch.empty(n, dtype=torch.float32, device=x.device)
     stream = _lib.current_stream(x.device)
+    bf16 = form == BF16
     with torch.cuda.device(x.device):
         if header is not None:
             _lib.check(L.gnnagg_wgrad_relu_dropout_backward_from_header_f32(
@@ -219,12 +257,12 @@ def _fused_backward(x, w, grad_y, y, header, row_div, scale, bf16, want_x):
                              _lib.ptr(grad_bias), _lib.ptr(workspace), rows, k, n, stream))
     grad_x = None
     if want_x:
-        if not bf16:
-            grad_x = torch.mm(grad_z, w.t())
-        elif L.gnnagg_linear_shape_supported(n, k):
-            grad_x = _fused_product(grad_z, w.t().contiguous(), None, None, None, 1.0, False, True)
-        else:
+        if form != FP32 and L.gnnagg_linear_shape_supported(n, k):
+            grad_x = _fused_product(grad_z, w.t().contiguous(), None, None, None, 1.0, False, form)
+        elif bf16:
             grad_x = _Bf16InputLinear._mm(grad_z, w.t())
+        else:
+            grad_x = torch.mm(grad_z, w.t())
     return grad_x, grad_w, grad_bias
 
 
@@ -234,7 +272,7 @@ class _FusedLayerPacked(torch.autograd.Function):
     returns exactly that); which units were active is read from the header's bitmaps."""
 
     @staticmethod
-    def forward(ctx, x, w, bias, keep_bits, scale, row_div, bf16):
+    def forward(ctx, x, w, bias, keep_bits, scale, row_div, form):
         rows, k, n = x.size(0), x.size(1), w.size(1)
         if keep_bits is not None and (keep_bits.dtype != torch.int32 or keep_bits.shape != (rows, (n + 31) // 32)
                                       or not keep_bits.is_contiguous()):
@@ -248,19 +286,19 @@ class _FusedLayerPacked(torch.autograd.Function):
         with torch.cuda.device(x.device):
             _lib.check(_lib.lib().gnnagg_linear_bias_relu_dropout_pack_f32(
                 _lib.ptr(x), _row_stride(x), _lib.ptr(w), n, _lib.ptr(bias.contiguous()), _lib.ptr(keep_bits),
-                _lib.ptr(row_div), float(scale), _lib.ptr(values), _lib.ptr(header), rows, k, n, 1 if bf16 else 0,
+                _lib.ptr(row_div), float(scale), _lib.ptr(values), _lib.ptr(header), rows, k, n, int(form),
                 _lib.current_stream(x.device)))
         ctx.mark_non_differentiable(header)
         ctx.save_for_backward(x, w, header)
         ctx.scale = float(scale)
         ctx.row_div = row_div
-        ctx.bf16 = bool(bf16)
+        ctx.form = int(form)
         return values, header
 
     @staticmethod
     def backward(ctx, grad_y, _grad_header):
         x, w, header = ctx.saved_tensors
-        grads = _fused_backward(x, w, grad_y, None, header, ctx.row_div, ctx.scale, ctx.bf16, ctx.needs_input_grad[0])
+        grads = _fused_backward(x, w, grad_y, None, header, ctx.row_div, ctx.scale, ctx.form, ctx.needs_input_grad[0])
         return grads + (None, None, None, None)
 
 
@@ -357,8 +395,8 @@ class _BiasReluDropoutPacked(torch.autograd.Function):
 class GCNLayer(torch.nn.Module):
     def __init__(self, in_channels: int, out_channels: int, gemm: str = "fp32"):
         super().__init__()
-        if gemm not in ("fp32", "bf16"):
-            raise ValueError("gemm must be 'fp32' or 'bf16'")
+        if gemm not in _FORMS:
+            raise ValueError("gemm must be 'fp32', 'bf16' or 'bf16x3'")
         self.gemm = gemm
         self.linear_first = False
         self.fuse = True  # use the fused layer kernels where they apply
@@ -369,6 +407,8 @@ class GCNLayer(torch.nn.Module):
     def _product(self, t: torch.Tensor) -> torch.Tensor:
         if self.gemm == "bf16":
             return _Bf16InputLinear.apply(t, self.weight)
+        if self.gemm == "bf16x3":
+            return _Bf16x3Linear.apply(t, self.weight)
         return _Fp32Linear.apply(t, self.weight)
 
     def transform(self, graph, x, layer: int, is_pre_delay: bool) -> torch.Tensor:
@@ -400,10 +440,10 @@ class GCNLayer(torch.nn.Module):
         agg = _kernel_ready(agg)
         row_div = _row_divisors(graph)
         row_div = None if row_div is None else row_div.reshape(-1)
-        bf16 = self.gemm == "bf16"
+        form = _FORMS[self.gemm]
         if pack_out:
-            return _FusedLayerPacked.apply(agg, self.weight, self.bias, keep_bits, scale, row_div, bf16)
-        return _FusedLayer.apply(agg, self.weight, self.bias, keep_bits, scale, row_div, relu, bf16)
+            return _FusedLayerPacked.apply(agg, self.weight, self.bias, keep_bits, scale, row_div, form)
+        return _FusedLayer.apply(agg, self.weight, self.bias, keep_bits, scale, row_div, relu, form)
 
     def forward(self, graph, x: torch.Tensor, layer: int, is_pre_delay: bool) -> torch.Tensor:
         """((A x) W) / deg + bias."""

@@ -229,10 +229,19 @@ int gnnagg_linear_bias_relu_dropout_bf16_f32(const float *x, int64_t x_stride, c
                                              const float *bias, const uint32_t *keep_bits, const float *row_div,
                                              float scale, int relu, float *y, int64_t y_stride, int64_t rows,
                                              int64_t k, int64_t n, void *stream);
+/* The same in fp32 accuracy on the bf16 matrix units: every fp32 operand value is cut into three bf16 pieces
+ * (hi = bf16(v), mid = bf16(v - hi), lo = bf16(v - hi - mid): both differences are exact) on its way into LDS, and
+ * a product is the sum of six bf16 MFMAs (hi*hi, hi*mid, mid*hi, mid*mid, hi*lo, lo*hi) accumulated in fp32; what
+ * is left out is below 2^-24 |x||w| per term, an fp32 rounding.  192 MFMA cycles per 32 x 32 x 16 block of
+ * products instead of the fp32 MFMA's 512. */
+int gnnagg_linear_bias_relu_dropout_bf16x3_f32(const float *x, int64_t x_stride, const float *w, int64_t w_stride,
+                                               const float *bias, const uint32_t *keep_bits, const float *row_div,
+                                               float scale, int relu, float *y, int64_t y_stride, int64_t rows,
+                                               int64_t k, int64_t n, void *stream);
 /* The same layer writing its result packed (the format of gnnagg_bias_relu_dropout_pack_f32 below: every row's
  * non-zero values at its front, plus the header of (bitmap, non-zeros in front) pairs): n in {32, 64, 128, 256},
  * ReLU always on, y_packed [rows, n] contiguous with 4 floats of slack behind it, header uint32 [rows, 2 * (n / 32)];
- * bf16_inputs 0/1 picks the product's form. */
+ * bf16_inputs picks the product's form: 0 fp32 MFMA, 1 operands rounded to bf16, 2 three bf16 pieces per operand. */
 int gnnagg_linear_bias_relu_dropout_pack_f32(const float *x, int64_t x_stride, const float *w, int64_t w_stride,
                                              const float *bias, const uint32_t *keep_bits, const float *row_div,
                                              float scale, float *y_packed, uint32_t *header, int64_t rows, int64_t k,

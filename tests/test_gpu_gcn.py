@@ -67,7 +67,7 @@ class CpuBf16Linear(torch.autograd.Function):
 
 
 @pytest.mark.parametrize("gemm,tol,fuse", [("fp32", 1e-4, True), ("fp32", 1e-4, False), ("bf16", 2e-2, True),
-                                           ("bf16", 2e-2, False)])
+                                           ("bf16", 2e-2, False), ("bf16x3", 1e-4, True), ("bf16x3", 1e-4, False)])
 @pytest.mark.parametrize("linear_first", [False, True])
 def test_train_step_matches_cpu_autograd(gemm, tol, fuse, linear_first):
     dev = "cuda:0"
@@ -323,6 +323,32 @@ def test_fused_layer_with_bf16_inputs(rows, k, n):
     assert float((b_in.grad.double() - want_b).abs().max()) <= 1e-5 * (float(want_b.abs().max()) + 1e-12)
 
 
+@pytest.mark.parametrize("rows,k,n", [(1000, 64, 32), (777, 128, 172), (4099, 256, 256), (130, 16, 4), (2000, 1024, 128),
+                                      (20_001, 128, 256)])
+def test_product_in_three_bf16_pieces_is_as_exact_as_the_fp32_product(rows, k, n):
+    """The bf16 x 3 form cuts every fp32 operand into hi + mid + lo bf16 pieces (the cuts are exact) and sums six
+    bf16 MFMAs per product; what it leaves out is below 2^-24 |x||w| per term.  Rows spread over e^+-9 in size:
+    per element the error stays within 1e-6 of sum |x||w| -- the bound the fp32 MFMA product meets, and three
+    orders of magnitude under the bf16-input form's."""
+    gen = torch.Generator(device="cuda").manual_seed(rows + k + n)
+    x = torch.randn(rows, k, device="cuda", generator=gen) * torch.exp(3 * torch.randn(rows, 1, device="cuda", generator=gen))
+    w = torch.randn(k, n, device="cuda", generator=gen) / k ** 0.5
+    ref = x.double() @ w.double()
+    size = x.double().abs() @ w.double().abs()
+    errors = {}
+    for name, form in (("fp32", gcn.FP32), ("bf16", gcn.BF16), ("bf16x3", gcn.BF16X3)):
+        y = gcn._fused_product(x, w, None, None, None, 1.0, False, form)
+        errors[name] = float(((y.double() - ref).abs() / size).max())
+    assert errors["bf16x3"] <= 1e-6 and errors["fp32"] <= 1e-6, errors
+    assert errors["bf16"] > 1e-4, errors  # (what rounding the operands to one bf16 piece costs)
+    # an operand that one bf16 piece holds exactly goes through unchanged: integers below 256 times a power of two
+    xi = torch.randint(-255, 256, (rows, k), device="cuda", generator=gen).float()
+    wi = torch.randint(-255, 256, (k, n), device="cuda", generator=gen).float() / 64
+    exact = xi.double() @ wi.double()  # every partial sum is an integer / 64 below 2^24: exact in fp32 too
+    if k <= 128:
+        assert torch.equal(gcn._fused_product(xi, wi, None, None, None, 1.0, False, gcn.BF16X3).double(), exact)
+
+
 @pytest.mark.parametrize("fused", [True, False])
 def test_degrees_folded_into_the_matrices_change_rounding_only(fused):
     """With the in-degree division carried by the matrix values (sage.fold_in_degrees) the layers skip their own
@@ -351,7 +377,7 @@ def test_degrees_folded_into_the_matrices_change_rounding_only(fused):
         assert torch.allclose(a, b, rtol=1e-4, atol=1e-6 + 1e-4 * float(a.abs().max()))
 
 
-@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("bf16", [gcn.FP32, gcn.BF16, gcn.BF16X3])
 def test_fused_layer_with_no_rows(bf16):
     """An empty partition: empty outputs, zero weight and bias gradients, nothing launched out of bounds."""
     x = torch.empty(0, 32, device="cuda", requires_grad=True)

@@ -199,11 +199,13 @@ def test_random_fused_layernorm_passes_match_torch(seed):
                 assert float((got_p.double().cpu() - want_p).abs().max()) <= 2e-4 * (float(want_p.abs().max()) + 1.0), what
 
 
+@pytest.mark.parametrize("form", [gcn.FP32, gcn.BF16X3])
 @pytest.mark.parametrize("seed", range(3))
-def test_random_fused_layer_kernels_match_fp64(seed):
+def test_random_fused_layer_kernels_match_fp64(seed, form):
     """The one-kernel dense layer (product, degree division, bias, ReLU, dropout bits) and its one-pass
     gradient (mask, division, bias and weight gradients) over random row counts, widths, row strides and
-    option sets, against fp64 torch ops on the units the kernel found active."""
+    option sets, against fp64 torch ops on the units the kernel found active.  The bf16 x 3 form of the
+    products (every fp32 operand as three bf16 pieces) is held to the same fp32 tolerances."""
     rng = np.random.default_rng(23000 + seed)
     for case in range(14):
         rows = int(rng.choice([1, 5, 127, 128, 129, 1000, 4097, 20011]))
@@ -221,13 +223,13 @@ def test_random_fused_layer_kernels_match_fp64(seed):
         keep = dev(rng.random((rows, n)) >= p) if with_mask else None
         scale = 1.0 / (1.0 - p) if with_mask else 1.0
         g = dev(rng.standard_normal((rows, n)).astype(np.float32))
-        what = dict(seed=seed, case=case, rows=rows, k=k, n=n, pad=pad, div=with_div, mask=with_mask, relu=relu)
+        what = dict(seed=seed, form=form, case=case, rows=rows, k=k, n=n, pad=pad, div=with_div, mask=with_mask, relu=relu)
         assert gcn.fused_layer_supported(x, k, n), what
 
         x_in, w_in, b_in = x.detach().clone().requires_grad_(), w.clone().requires_grad_(), bias.clone().requires_grad_()
         view = wide.clone()[:, pad:pad + k].requires_grad_() if pad else x_in
         y = gcn._FusedLayer.apply(gcn._kernel_ready(view), w_in, b_in, gcn.pack_keep_mask(keep) if with_mask else None,
-                                  scale, div, relu)
+                                  scale, div, relu, form)
         y.backward(g)
         z = x.double() @ w.double()
         if with_div:
@@ -250,7 +252,7 @@ def test_random_fused_layer_kernels_match_fp64(seed):
             # the activity from the header's bitmaps -- the same gradients bit for bit
             x2, w2, b2 = x.detach().clone().requires_grad_(), w.clone().requires_grad_(), bias.clone().requires_grad_()
             values, header = gcn._FusedLayerPacked.apply(gcn._kernel_ready(x2), w2, b2,
-                                                         gcn.pack_keep_mask(keep) if with_mask else None, scale, div, False)
+                                                         gcn.pack_keep_mask(keep) if with_mask else None, scale, div, form)
             assert torch.equal(packed.unpack(values, header), y.detach()), what
             values.backward(g)
             for got, want, name in ((x2.grad, view.grad, "x"), (w2.grad, w_in.grad, "w"), (b2.grad, b_in.grad, "bias")):
