@@ -43,6 +43,7 @@ EXPORTS = (
     "gnnagg_wgrad_relu_dropout_backward_workspace_bytes",
     "gnnagg_wgrad_relu_dropout_backward_f32",
     "gnnagg_wgrad_relu_dropout_backward_bf16_f32",
+    "gnnagg_wgrad_relu_dropout_backward_bf16x3_f32",
     "gnnagg_wgrad_relu_dropout_backward_from_header_f32",
     "gnnagg_dropout_layernorm_relu_blocks",
     "gnnagg_dropout_layernorm_relu_f32",
@@ -151,6 +152,8 @@ def lib() -> ctypes.CDLL:
                                                          i64, i64, i64, vp]
     L.gnnagg_wgrad_relu_dropout_backward_bf16_f32.restype = i32
     L.gnnagg_wgrad_relu_dropout_backward_bf16_f32.argtypes = L.gnnagg_wgrad_relu_dropout_backward_f32.argtypes
+    L.gnnagg_wgrad_relu_dropout_backward_bf16x3_f32.restype = i32
+    L.gnnagg_wgrad_relu_dropout_backward_bf16x3_f32.argtypes = L.gnnagg_wgrad_relu_dropout_backward_f32.argtypes
     L.gnnagg_wgrad_relu_dropout_backward_from_header_f32.restype = i32
     L.gnnagg_wgrad_relu_dropout_backward_from_header_f32.argtypes = [vp, i64, vp, i64, vp, vp, ctypes.c_float, vp, vp, vp,
                                                                      vp, i64, i64, i64, i32, vp]

@@ -359,7 +359,10 @@ __global__ __launch_bounds__(256) void wgrad_bias_reduce_kernel(const float *__r
 // the slice read the slice's last row and count as zeros, so there is no separate tail path.
 constexpr int kLdh = 2 * kChunk + 8;  // bytes between staged columns
 
-template <int WM, int WN, bool MASKED, bool BITS>
+// SPLIT: fp32 accuracy on the same units -- every operand value is cut into three bf16 pieces (hi, mid, lo: three
+// planes of the staging layout) and a product is the sum of six v_mfma_f32_32x32x16_bf16 (hi*hi, hi*mid, mid*hi,
+// mid*mid, hi*lo, lo*hi; what is left out is below 2^-24 |x||g| per term).
+template <int WM, int WN, bool MASKED, bool BITS, bool SPLIT = false>
 __global__ __launch_bounds__(256, 1) void wgrad_bf16_partial_kernel(const float *__restrict__ x,
                                                                     const float *__restrict__ g,
                                                                     float *__restrict__ partial, int64_t rows, int fi,
@@ -367,7 +370,8 @@ __global__ __launch_bounds__(256, 1) void wgrad_bf16_partial_kernel(const float 
                                                                     const MaskArgs mk) {
     extern __shared__ __align__(16) float smem[];
     char *lds = reinterpret_cast<char *>(smem);
-    constexpr int kBufBytes = (64 * WM + 64 * WN) * kLdh;
+    constexpr int kPlaneBytes = (64 * WM + 64 * WN) * kLdh;
+    constexpr int kBufBytes = (SPLIT ? 3 : 1) * kPlaneBytes;
     constexpr int kGOff = 64 * WM * kLdh;
 
     const int tid = (int)threadIdx.x;
@@ -459,8 +463,19 @@ __global__ __launch_bounds__(256, 1) void wgrad_bf16_partial_kernel(const float 
         }
 #pragma unroll
         for (int c = 0; c < 4; ++c) {  // column 4 q + c of the block: its four consecutive rows
-            *reinterpret_cast<shortx4 *>(dst + x_dst + c * kLdh) = to_bf16x4(xr[0][c], xr[1][c], xr[2][c], xr[3][c]);
-            *reinterpret_cast<shortx4 *>(dst + g_dst + c * kLdh) = to_bf16x4(gr[0][c], gr[1][c], gr[2][c], gr[3][c]);
+            if (SPLIT) {
+                shortx4 px[3], pg[3];
+                split_bf16x3(xr[0][c], xr[1][c], xr[2][c], xr[3][c], px);
+                split_bf16x3(gr[0][c], gr[1][c], gr[2][c], gr[3][c], pg);
+#pragma unroll
+                for (int q = 0; q < 3; ++q) {
+                    *reinterpret_cast<shortx4 *>(dst + q * kPlaneBytes + x_dst + c * kLdh) = px[q];
+                    *reinterpret_cast<shortx4 *>(dst + q * kPlaneBytes + g_dst + c * kLdh) = pg[q];
+                }
+            } else {
+                *reinterpret_cast<shortx4 *>(dst + x_dst + c * kLdh) = to_bf16x4(xr[0][c], xr[1][c], xr[2][c], xr[3][c]);
+                *reinterpret_cast<shortx4 *>(dst + g_dst + c * kLdh) = to_bf16x4(gr[0][c], gr[1][c], gr[2][c], gr[3][c]);
+            }
         }
     };
     // Columns past fi / fo are never written: whatever they hold only reaches accumulator entries
@@ -468,6 +483,41 @@ __global__ __launch_bounds__(256, 1) void wgrad_bf16_partial_kernel(const float 
     auto multiply = [&](int buf) {
         const char *xa = lds + buf * kBufBytes + (m0 + idx) * kLdh + 8 * kk;
         const char *gb = lds + buf * kBufBytes + kGOff + (n0 + idx) * kLdh + 8 * kk;
+        if (SPLIT) {
+            // a lane feeds rows 4 kk .. 4 kk + 3 and 8 + 4 kk .. of its column to one 32x32x16 MFMA (both operands
+            // in the same order, so the sum over the chunk's 16 rows is the same)
+            auto piece8 = [](const char *at) {
+                union {
+                    shortx4 h[2];
+                    bf16x8 v;
+                } u;
+                u.h[0] = *reinterpret_cast<const shortx4 *>(at);
+                u.h[1] = *reinterpret_cast<const shortx4 *>(at + 16);
+                return u.v;
+            };
+            bf16x8 a3[WM][3];
+#pragma unroll
+            for (int i = 0; i < WM; ++i)
+#pragma unroll
+                for (int q = 0; q < 3; ++q) a3[i][q] = piece8(xa + q * kPlaneBytes + 32 * i * kLdh);
+#pragma unroll
+            for (int j = 0; j < WN; ++j) {
+                bf16x8 b3[3];
+#pragma unroll
+                for (int q = 0; q < 3; ++q) b3[q] = piece8(gb + q * kPlaneBytes + 32 * j * kLdh);
+#pragma unroll
+                for (int i = 0; i < WM; ++i) {  // smallest pieces first
+                    floatx16 c = acc[i][j];
+                    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a3[i][2], b3[0], c, 0, 0, 0);
+                    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a3[i][0], b3[2], c, 0, 0, 0);
+                    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a3[i][1], b3[1], c, 0, 0, 0);
+                    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a3[i][1], b3[0], c, 0, 0, 0);
+                    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a3[i][0], b3[1], c, 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a3[i][0], b3[0], c, 0, 0, 0);
+                }
+            }
+            return;
+        }
         shortx4 a[2][WM], b[2][WN];
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
@@ -556,7 +606,10 @@ namespace {
 
 int run_wgrad(const float *x, int64_t x_stride, const float *g, int64_t g_stride, float *w_grad, void *workspace,
               int64_t rows, int64_t fi, int64_t fo, void *stream, const MaskArgs *mask, float *bias_grad,
-              bool bf16 = false) {
+              int form = 0) {  // 0 fp32 MFMA, 1 operands rounded to bf16, 2 three bf16 pieces per operand (both masked only)
+    GNNAGG_REQUIRE(form >= 0 && form <= 2, "product form is 0 (fp32), 1 (bf16 inputs) or 2 (bf16 x 3 pieces), got %d", form);
+    GNNAGG_REQUIRE(form == 0 || mask, "the bf16 forms of the weight gradient come with the masked pass");
+    const bool bf16 = form != 0;
     GNNAGG_REQUIRE(rows >= 0 && fi > 0 && fo > 0, "bad size");
     GNNAGG_REQUIRE(x_stride >= fi && g_stride >= fo && x_stride < (int64_t(1) << 27) && g_stride < (int64_t(1) << 27),
                    "row strides %lld / %lld must be at least the widths %lld / %lld and below 2^27",
@@ -604,10 +657,21 @@ int run_wgrad(const float *x, int64_t x_stride, const float *g, int64_t g_stride
         hipLaunchKernelGGL((wgrad_partial_kernel<M, N, MASKED>), dim3((unsigned)blocks), dim3(256), smem, st, x, g, \
                            partial, rows, (int)fi, (int)fo, (int)x_stride, (int)g_stride, rpb, aligned, mk);    \
     }
+#define GNNAGG_WGRAD_SPLIT(M, N, BITS)                                                                          \
+    {                                                                                                           \
+        constexpr size_t smem = (size_t)6 * (64 * M + 64 * N) * kLdh;                                            \
+        GNNAGG_HIP(allow_lds(reinterpret_cast<const void *>(&wgrad_bf16_partial_kernel<M, N, true, BITS, true>), smem)); \
+        hipLaunchKernelGGL((wgrad_bf16_partial_kernel<M, N, true, BITS, true>), dim3((unsigned)blocks), dim3(256), smem, st, \
+                           x, g, partial, rows, (int)fi, (int)fo, (int)x_stride, (int)g_stride, rpb, mk);       \
+    }
 #define GNNAGG_WGRAD_BF16(M, N)                                                                                  \
     {                                                                                                           \
         constexpr size_t smem = (size_t)2 * (64 * M + 64 * N) * kLdh;                                            \
-        if (mk.bits)                                                                                            \
+        if (form == 2 && mk.bits)                                                                               \
+            GNNAGG_WGRAD_SPLIT(M, N, true)                                                                      \
+        else if (form == 2)                                                                                     \
+            GNNAGG_WGRAD_SPLIT(M, N, false)                                                                     \
+        else if (mk.bits)                                                                                       \
             hipLaunchKernelGGL((wgrad_bf16_partial_kernel<M, N, true, true>), dim3((unsigned)blocks), dim3(256), smem, st, \
                                x, g, partial, rows, (int)fi, (int)fo, (int)x_stride, (int)g_stride, rpb, mk);   \
         else                                                                                                    \
@@ -630,6 +694,7 @@ int run_wgrad(const float *x, int64_t x_stride, const float *g, int64_t g_stride
 #undef GNNAGG_WGRAD
 #undef GNNAGG_WGRAD_FORM
 #undef GNNAGG_WGRAD_BF16
+#undef GNNAGG_WGRAD_SPLIT
     GNNAGG_HIP(hipGetLastError());
     const int count = (int)(fi * fo);
     hipLaunchKernelGGL(wgrad_reduce_kernel, dim3((unsigned)((count + kReduceOutputs - 1) / kReduceOutputs)), dim3(256), 0,
@@ -679,7 +744,18 @@ extern "C" int gnnagg_wgrad_relu_dropout_backward_bf16_f32(const float *x, int64
     GNNAGG_REQUIRE(bias_grad, "null bias_grad");
     GNNAGG_REQUIRE(!y || (y_stride >= fo && y_stride < (int64_t(1) << 27)), "bad row stride of y");
     MaskArgs mk{y ? y : grad_y, row_div, grad_z, nullptr, (int)(y ? y_stride : 0), scale, y ? 0 : 1, nullptr, 0, 0};
-    return run_wgrad(x, x_stride, grad_y, grad_stride, w_grad, workspace, rows, fi, fo, stream, &mk, bias_grad, true);
+    return run_wgrad(x, x_stride, grad_y, grad_stride, w_grad, workspace, rows, fi, fo, stream, &mk, bias_grad, 1);
+}
+
+extern "C" int gnnagg_wgrad_relu_dropout_backward_bf16x3_f32(const float *x, int64_t x_stride, const float *grad_y,
+                                                             int64_t grad_stride, const float *y, int64_t y_stride,
+                                                             const float *row_div, float scale, float *grad_z,
+                                                             float *w_grad, float *bias_grad, void *workspace,
+                                                             int64_t rows, int64_t fi, int64_t fo, void *stream) {
+    GNNAGG_REQUIRE(bias_grad, "null bias_grad");
+    GNNAGG_REQUIRE(!y || (y_stride >= fo && y_stride < (int64_t(1) << 27)), "bad row stride of y");
+    MaskArgs mk{y ? y : grad_y, row_div, grad_z, nullptr, (int)(y ? y_stride : 0), scale, y ? 0 : 1, nullptr, 0, 0};
+    return run_wgrad(x, x_stride, grad_y, grad_stride, w_grad, workspace, rows, fi, fo, stream, &mk, bias_grad, 2);
 }
 
 extern "C" int gnnagg_wgrad_relu_dropout_backward_from_header_f32(const float *x, int64_t x_stride, const float *grad_y,
@@ -694,5 +770,5 @@ extern "C" int gnnagg_wgrad_relu_dropout_backward_from_header_f32(const float *x
         return fail(GNNAGG_ERR_UNSUPPORTED, "packed activations exist for widths 32, 64, 128, 256 (got %lld)", (long long)fo);
     MaskArgs mk{nullptr, row_div, grad_z, nullptr, 0, scale, 0, header, (int)(2 * (fo / 32)), 2};
     return run_wgrad(x, x_stride, grad_y, grad_stride, w_grad, workspace, rows, fi, fo, stream, &mk, bias_grad,
-                     bf16_inputs != 0);
+                     bf16_inputs);
 }

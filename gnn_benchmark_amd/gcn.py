@@ -17,8 +17,8 @@ kernel, and in the gradient direction the ReLU / dropout mask, the degree divisi
 gradient and the weight gradient are another; the fp32 input-gradient product stays with the
 BLAS library, the bf16-input one is the same libgnnagg product kernel.  ``gemm="bf16x3"`` keeps
 fp32 accuracy but feeds the matrix units every fp32 operand as three bf16 pieces (six bf16 MFMAs
-a product, a fraction of the fp32 MFMA's cycles): the layer product and the input-gradient
-product run that way, the weight gradient stays the fp32 kernel.
+a product, a fraction of the fp32 MFMA's cycles): all three products of a fused layer run that
+way (where a layer is not fused, the weight gradient stays the fp32 kernel).
 """
 import contextlib
 from typing import List, Optional, Sequence
@@ -199,9 +199,8 @@ class _FusedLayer(torch.autograd.Function):
     is one more kernel -- mask, degree division, bias gradient and weight gradient in a single
     pass over x, the incoming gradient and y -- plus the product for the input gradient.  With
     ``form`` ``BF16`` all three products round their operands to bf16 on the way into the matrix units
-    (fp32 accumulation); with ``BF16X3`` the layer product and the input-gradient product feed every operand
-    as three bf16 pieces (fp32 accuracy; the weight gradient is the fp32 kernel); mask, division and bias
-    gradient stay in fp32."""
+    (fp32 accumulation); with ``BF16X3`` they feed every operand as three bf16 pieces (fp32 accuracy); mask,
+    division and bias gradient stay in fp32."""
 
     @staticmethod
     def forward(ctx, x, w, bias, keep_bits, scale, row_div, relu, form=FP32):
@@ -249,9 +248,10 @@ def _fused_backward(x, w, grad_y, y, header, row_div, scale, form, want_x):
             _lib.check(L.gnnagg_wgrad_relu_dropout_backward_from_header_f32(
                 _lib.ptr(x), _row_stride(x), _lib.ptr(grad_y), _row_stride(grad_y), _lib.ptr(header), _lib.ptr(row_div),
                 scale, _lib.ptr(grad_z), _lib.ptr(grad_w), _lib.ptr(grad_bias), _lib.ptr(workspace), rows, k, n,
-                1 if bf16 else 0, stream))
+                int(form), stream))
         else:
-            entry = L.gnnagg_wgrad_relu_dropout_backward_bf16_f32 if bf16 else L.gnnagg_wgrad_relu_dropout_backward_f32
+            entry = (L.gnnagg_wgrad_relu_dropout_backward_f32, L.gnnagg_wgrad_relu_dropout_backward_bf16_f32,
+                     L.gnnagg_wgrad_relu_dropout_backward_bf16x3_f32)[int(form)]
             _lib.check(entry(_lib.ptr(x), _row_stride(x), _lib.ptr(grad_y), _row_stride(grad_y), _lib.ptr(y),
                              n if y is not None else 0, _lib.ptr(row_div), scale, _lib.ptr(grad_z), _lib.ptr(grad_w),
                              _lib.ptr(grad_bias), _lib.ptr(workspace), rows, k, n, stream))

@@ -254,7 +254,8 @@ int gnnagg_wgrad_relu_dropout_backward_f32(const float *x, int64_t x_stride, con
                                            float *grad_z, float *w_grad, float *bias_grad, void *workspace,
                                            int64_t rows, int64_t fi, int64_t fo, void *stream);
 /* The same when the layer's output was written packed: which units were active is read from the bitmaps of its
- * header (fo in {32, 64, 128, 256}) instead of from y; bf16_inputs 0/1 picks the product's form. */
+ * header (fo in {32, 64, 128, 256}) instead of from y; bf16_inputs picks the product's form (0 fp32 MFMA, 1 operands
+ * rounded to bf16, 2 three bf16 pieces per operand). */
 int gnnagg_wgrad_relu_dropout_backward_from_header_f32(const float *x, int64_t x_stride, const float *grad_y,
                                                        int64_t grad_stride, const uint32_t *header, const float *row_div,
                                                        float scale, float *grad_z, float *w_grad, float *bias_grad,
@@ -265,6 +266,13 @@ int gnnagg_wgrad_relu_dropout_backward_bf16_f32(const float *x, int64_t x_stride
                                                 const float *row_div, float scale, float *grad_z, float *w_grad,
                                                 float *bias_grad, void *workspace, int64_t rows, int64_t fi, int64_t fo,
                                                 void *stream);
+/* (the _bf16x3_ form: the product x^T @ grad_z in fp32 accuracy on the bf16 matrix units, every value of x and
+ * grad_z cut into three bf16 pieces, six bf16 MFMAs a product -- see gnnagg_linear_bias_relu_dropout_bf16x3_f32) */
+int gnnagg_wgrad_relu_dropout_backward_bf16x3_f32(const float *x, int64_t x_stride, const float *grad_y,
+                                                  int64_t grad_stride, const float *y, int64_t y_stride,
+                                                  const float *row_div, float scale, float *grad_z, float *w_grad,
+                                                  float *bias_grad, void *workspace, int64_t rows, int64_t fi,
+                                                  int64_t fo, void *stream);
 
 /* ---------------------------------------------------------------------------------
  * The elementwise chain between two SAGE layers (model/DistSAGE.py:49-53: F.dropout, LayerNorm
