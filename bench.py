@@ -674,16 +674,17 @@ def run_c5_sage(args, graph):
 
     staged = sage.stage_input(x)
     folded = None
-    for tag, fold, linear_first, restrict in (
-            ("", False, False, True), ("_folded_degrees", True, False, True),
-            ("_folded_degrees_linear_first_when_narrowing", True, True, True),
-            ("_folded_degrees_all_nodes_through_last_layer", True, False, False)):
+    for tag, fold, linear_first, restrict, gemm in (
+            ("", False, False, True, "fp32"), ("_folded_degrees", True, False, True, "fp32"),
+            ("_folded_degrees_linear_first_when_narrowing", True, True, True, "fp32"),
+            ("_folded_degrees_bf16x3_gemm", True, False, True, "bf16x3"),
+            ("_folded_degrees_all_nodes_through_last_layer", True, False, False, "fp32")):
         if fold and folded is None:
             folded = sage.fold_in_degrees(graph)
         g = folded if fold else graph
         torch.manual_seed(args.seed)
         model = sage.DistSAGE(dims[0], hidden, dims[-1], num_layers=len(dims) - 1, dropout=0.5, is_pre_delay=True,
-                              linear_first_when_narrowing=linear_first).to(dev)
+                              linear_first_when_narrowing=linear_first, gemm=gemm).to(dev)
         opt = torch.optim.Adam(model.parameters(), lr=0.01)
         ms, losses = timed(lambda: sage.train_step(model, opt, g, staged, labels, train_idx, masks, restrict))
         out["train_step_ms" + tag], out["loss" + tag] = ms, losses

@@ -76,9 +76,10 @@ def weight_gradient(x: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def weight_and_bias_gradient(x: torch.Tensor, g: torch.Tensor):
+def weight_and_bias_gradient(x: torch.Tensor, g: torch.Tensor, form: int = 0):
     """(x^T @ g, g.sum(0)): the column sums come out of the weight-gradient kernel's pass over g.
-    Falls back to separate torch ops for shapes the kernel does not take."""
+    Falls back to separate torch ops for shapes the kernel does not take.  ``form`` ``BF16X3``: the product
+    with every operand as three bf16 pieces (fp32 accuracy, fewer matrix-unit cycles)."""
     x, g = _kernel_ready(x), _kernel_ready(g)
     rows, fi, fo = x.size(0), x.size(1), g.size(1)
     L = _lib.lib()
@@ -90,7 +91,8 @@ def weight_and_bias_gradient(x: torch.Tensor, g: torch.Tensor):
     grad_b = torch.empty(fo, dtype=torch.float32, device=x.device)
     workspace = torch.empty(nbytes // 4, dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
-        _lib.check(L.gnnagg_wgrad_relu_dropout_backward_f32(
+        entry = L.gnnagg_wgrad_relu_dropout_backward_bf16x3_f32 if form == 2 else L.gnnagg_wgrad_relu_dropout_backward_f32
+        _lib.check(entry(
             _lib.ptr(x), _row_stride(x), _lib.ptr(g), _row_stride(g), None, 0, None, 1.0, None, _lib.ptr(grad_w),
             _lib.ptr(grad_b), _lib.ptr(workspace), rows, fi, fo, _lib.current_stream(x.device)))
     return grad_w, grad_b
@@ -179,18 +181,45 @@ FP32, BF16, BF16X3 = 0, 1, 2  # as they are / rounded to bf16 / as three bf16 pi
 _FORMS = {"fp32": FP32, "bf16": BF16, "bf16x3": BF16X3}
 
 
-def _fused_product(x, w, bias, keep_bits, row_div, scale, relu, form):
-    """The one-kernel layer product of libgnnagg on kernel-ready operands."""
+def _fused_product(x, w, bias, keep_bits, row_div, scale, relu, form, out=None):
+    """The one-kernel layer product of libgnnagg on kernel-ready operands (``out``: a kernel-ready [rows, n] array,
+    e.g. a column block of a wider one, to write into)."""
     rows, k, n = x.size(0), x.size(1), w.size(1)
-    y = torch.empty(rows, n, dtype=torch.float32, device=x.device)
+    y = torch.empty(rows, n, dtype=torch.float32, device=x.device) if out is None else out
     L = _lib.lib()
     entry = (L.gnnagg_linear_bias_relu_dropout_f32, L.gnnagg_linear_bias_relu_dropout_bf16_f32,
              L.gnnagg_linear_bias_relu_dropout_bf16x3_f32)[int(form)]
     with torch.cuda.device(x.device):
         _lib.check(entry(_lib.ptr(x), _row_stride(x), _lib.ptr(w), n, _lib.ptr(bias), _lib.ptr(keep_bits),
-                         _lib.ptr(row_div), float(scale), 1 if relu else 0, _lib.ptr(y), n, rows, k, n,
+                         _lib.ptr(row_div), float(scale), 1 if relu else 0, _lib.ptr(y), _row_stride(y), rows, k, n,
                          _lib.current_stream(x.device)))
     return y
+
+
+def stacked_product(cat: torch.Tensor, weight: torch.Tensor, bias, form: int) -> torch.Tensor:
+    """cat @ weight (+ bias).  ``form`` ``BF16X3``: libgnnagg's product kernel with every operand as three bf16
+    pieces where it takes the widths; the BLAS library's fp32 product otherwise."""
+    if (form == BF16X3 and cat.is_cuda and cat.dtype == torch.float32 and cat.size(0) > 0
+            and _lib.lib().gnnagg_linear_shape_supported(cat.size(1), weight.size(1))):
+        return _fused_product(_kernel_ready(cat), weight.contiguous(), None if bias is None else bias.contiguous(),
+                              None, None, 1.0, False, BF16X3)
+    return torch.mm(cat, weight) if bias is None else torch.addmm(bias, cat, weight)
+
+
+def input_gradient(g: torch.Tensor, weight: torch.Tensor, form: int) -> torch.Tensor:
+    """g @ weight^T, [rows, weight rows].  ``form`` ``BF16X3``: libgnnagg's product kernel, one call per block of at
+    most 256 output columns, each writing its columns of the result; the BLAS library's product otherwise."""
+    wide, inner = weight.size(0), weight.size(1)
+    blocks = [(c, min(c + 256, wide)) for c in range(0, wide, 256)]
+    L = _lib.lib()
+    if (form == BF16X3 and g.is_cuda and g.dtype == torch.float32 and g.size(0) > 0 and wide % 4 == 0
+            and all(L.gnnagg_linear_shape_supported(inner, hi - lo) for lo, hi in blocks)):
+        g = _kernel_ready(g)
+        out = torch.empty(g.size(0), wide, dtype=torch.float32, device=g.device)
+        for lo, hi in blocks:
+            _fused_product(g, weight[lo:hi].t().contiguous(), None, None, None, 1.0, False, BF16X3, out=out[:, lo:hi])
+        return out
+    return torch.mm(g, weight.t())
 
 
 class _FusedLayer(torch.autograd.Function):

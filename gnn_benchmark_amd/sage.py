@@ -28,7 +28,7 @@ import torch
 import torch.nn.functional as F
 
 from . import _lib, aggregator
-from .gcn import _mean_nll, scored_rows, weight_and_bias_gradient, weight_gradient
+from .gcn import _FORMS, _mean_nll, input_gradient, scored_rows, stacked_product, weight_and_bias_gradient, weight_gradient
 from .sparse_tensor import SparseTensor, _row_stride
 
 
@@ -132,7 +132,7 @@ class _SageConv(torch.autograd.Function):
     overwritten with the aggregated rows and kept for the weight gradient)."""
 
     @staticmethod
-    def forward(ctx, graph, cat, weight, bias, layer, num_bits, is_pre_delay, is_training, normalize):
+    def forward(ctx, graph, cat, weight, bias, layer, num_bits, is_pre_delay, is_training, normalize, form=0):
         fi = cat.size(1) // 2
         x, agg = cat[:, fi:], cat[:, :fi]
         aggregator._forward(ctx, graph, aggregator._DenseFeatures(x), layer, num_bits, is_pre_delay, is_training,
@@ -145,9 +145,10 @@ class _SageConv(torch.autograd.Function):
             # array's version, so that an earlier call that kept this same array for its backward
             # fails loudly there instead of reading rows that are no longer its own
             cat[:0].zero_()
-        out = torch.mm(cat, weight) if bias is None else torch.addmm(bias, cat, weight)
+        out = stacked_product(cat, weight, bias, form)
         ctx.save_for_backward(cat, weight)
         ctx.has_bias = bias is not None
+        ctx.form = form
         return out
 
     @staticmethod
@@ -160,21 +161,23 @@ class _SageConv(torch.autograd.Function):
         if ctx.needs_input_grad[2]:
             # each half's rows of the stacked weight: x_half^T @ g, reading the half where it lies; the
             # bias gradient (column sums of g) comes out of the first of the two passes over g
-            if want_b:
-                top, grad_b = weight_and_bias_gradient(cat[:, :fi], g)
+            if want_b or ctx.form:
+                top, grad_b = weight_and_bias_gradient(cat[:, :fi], g, ctx.form)
             else:
                 top = weight_gradient(cat[:, :fi], g)
-            grad_w = torch.cat([top, weight_gradient(cat[:, fi:], g)], dim=0)
+            bottom = weight_and_bias_gradient(cat[:, fi:], g, ctx.form)[0] if ctx.form else weight_gradient(cat[:, fi:], g)
+            grad_w = torch.cat([top, bottom], dim=0)
+            grad_b = grad_b if want_b else None
         elif want_b:
             grad_b = g.sum(dim=0)
         if ctx.needs_input_grad[1]:
-            grad_cat = torch.mm(g, weight.t())  # [N, 2 fi]: d/d aggregated | d/d x (direct part)
+            grad_cat = input_gradient(g, weight, ctx.form)  # [N, 2 fi]: d/d aggregated | d/d x (direct part)
             grad_agg = grad_cat[:, :fi]
             if ctx.divide:
                 grad_agg.div_(ctx.graph.in_degrees)
             # d/d x += A^T (d/d aggregated), accumulated where the direct part already lies
             aggregator._backward(ctx, grad_agg, out=grad_cat[:, fi:], accumulate=True)
-        return None, grad_cat, grad_w, grad_b, None, None, None, None, None
+        return None, grad_cat, grad_w, grad_b, None, None, None, None, None, None
 
 
 class _SageConvRows(torch.autograd.Function):
@@ -183,7 +186,7 @@ class _SageConvRows(torch.autograd.Function):
     last layer, at a fraction of its aggregation and products, forward and backward; each row is the same FMA chain."""
 
     @staticmethod
-    def forward(ctx, graph_rows, cat, weight, bias, layer, num_bits, is_pre_delay, is_training, normalize, rows):
+    def forward(ctx, graph_rows, cat, weight, bias, layer, num_bits, is_pre_delay, is_training, normalize, rows, form=0):
         fi = cat.size(1) // 2
         x = cat[:, fi:]
         agg = aggregator._forward(ctx, graph_rows, aggregator._DenseFeatures(x), layer, num_bits, is_pre_delay,
@@ -192,9 +195,10 @@ class _SageConvRows(torch.autograd.Function):
         if ctx.divide:
             agg.div_(graph_rows.in_degrees)
         small = torch.cat([agg, x.index_select(0, rows)], dim=1)  # [len(rows), 2 fi]
-        out = torch.mm(small, weight) if bias is None else torch.addmm(bias, small, weight)
+        out = stacked_product(small, weight, bias, form)
         ctx.save_for_backward(small, weight, rows)
         ctx.has_bias = bias is not None
+        ctx.form = form
         ctx.nodes = cat.size(0)
         return out
 
@@ -206,15 +210,17 @@ class _SageConvRows(torch.autograd.Function):
         grad_cat = grad_w = grad_b = None
         want_b = ctx.has_bias and ctx.needs_input_grad[3]
         if ctx.needs_input_grad[2]:
-            if want_b:
-                top, grad_b = weight_and_bias_gradient(small[:, :fi], g)
+            if want_b or ctx.form:
+                top, grad_b = weight_and_bias_gradient(small[:, :fi], g, ctx.form)
             else:
                 top = weight_gradient(small[:, :fi], g)
-            grad_w = torch.cat([top, weight_gradient(small[:, fi:], g)], dim=0)
+            bottom = weight_and_bias_gradient(small[:, fi:], g, ctx.form)[0] if ctx.form else weight_gradient(small[:, fi:], g)
+            grad_w = torch.cat([top, bottom], dim=0)
+            grad_b = grad_b if want_b else None
         elif want_b:
             grad_b = g.sum(dim=0)
         if ctx.needs_input_grad[1]:
-            grad_small = torch.mm(g, weight.t())  # [len(rows), 2 fi]: d/d aggregated | d/d x[rows] (direct part)
+            grad_small = input_gradient(g, weight, ctx.form)  # [len(rows), 2 fi]: d/d aggregated | d/d x[rows] (direct part)
             grad_agg = grad_small[:, :fi]
             if ctx.divide:
                 grad_agg.div_(ctx.graph.in_degrees)
@@ -225,7 +231,7 @@ class _SageConvRows(torch.autograd.Function):
             target = grad_cat[:, fi:]
             aggregator._backward(ctx, grad_agg, out=target, accumulate=False)
             target.index_add_(0, rows, grad_small[:, fi:])
-        return None, grad_cat, grad_w, grad_b, None, None, None, None, None, None
+        return None, grad_cat, grad_w, grad_b, None, None, None, None, None, None, None
 
 
 class _SageConvLinearFirst(torch.autograd.Function):
@@ -301,11 +307,17 @@ class DistSAGEConvGrad(torch.nn.Module):
     ``[:in]`` are ``lin_neigh.weight.T``, rows ``[in:]`` are ``lin_self.weight.T``) and ``bias``."""
 
     def __init__(self, in_channels: int, out_channels: int, num_bits: int, is_pre_delay: bool,
-                 add_self_loops: bool = False, normalize: bool = True, bias: bool = True, linear_first: bool = False):
+                 add_self_loops: bool = False, normalize: bool = True, bias: bool = True, linear_first: bool = False,
+                 gemm: str = "fp32"):
         super().__init__()
         # linear_first: apply lin_neigh before aggregating (same result up to rounding; the
         # aggregation and the exchange then run at out_channels)
         self.linear_first = linear_first
+        # gemm "bf16x3": the layer's dense products in libgnnagg's kernels with every fp32 operand as three bf16
+        # pieces (fp32 accuracy on the bf16 matrix units); "fp32": the BLAS library's products
+        if gemm not in ("fp32", "bf16x3"):
+            raise ValueError("gemm must be 'fp32' or 'bf16x3'")
+        self.gemm = gemm
         self.in_channels = in_channels
         self.out_channels = out_channels
         self.add_self_loops = add_self_loops
@@ -374,9 +386,9 @@ class DistSAGEConvGrad(torch.nn.Module):
         if rows is not None:
             graph_rows = aggregator.restrict_output_rows(graph, rows, self.is_pre_delay)
             return _SageConvRows.apply(graph_rows, cat, self.weight, self.bias, layer, self.num_bits, self.is_pre_delay,
-                                       self.training, self.normalize, rows)
+                                       self.training, self.normalize, rows, _FORMS[self.gemm])
         return _SageConv.apply(graph, cat, self.weight, self.bias, layer, self.num_bits, self.is_pre_delay,
-                               self.training, self.normalize)
+                               self.training, self.normalize, _FORMS[self.gemm])
 
 
 # ---------------------------------------------------------------------------- the model
@@ -384,16 +396,16 @@ class DistSAGE(torch.nn.Module):
     """DistSAGE.py:13-69: ``num_layers`` SAGE layers, LayerNorm after all but the last."""
 
     def __init__(self, in_channels, hidden_channels, out_channels, num_layers=3, dropout=0.5, num_bits=32,
-                 is_pre_delay=False, linear_first_when_narrowing=False):
+                 is_pre_delay=False, linear_first_when_narrowing=False, gemm="fp32"):
         super().__init__()
         self.convs = torch.nn.ModuleList()
         self.norms = torch.nn.ModuleList()
-        self.convs.append(DistSAGEConvGrad(in_channels, hidden_channels, num_bits, is_pre_delay))
+        self.convs.append(DistSAGEConvGrad(in_channels, hidden_channels, num_bits, is_pre_delay, gemm=gemm))
         self.norms.append(torch.nn.LayerNorm(hidden_channels))
         for _ in range(num_layers - 2):
-            self.convs.append(DistSAGEConvGrad(hidden_channels, hidden_channels, num_bits, is_pre_delay))
+            self.convs.append(DistSAGEConvGrad(hidden_channels, hidden_channels, num_bits, is_pre_delay, gemm=gemm))
             self.norms.append(torch.nn.LayerNorm(hidden_channels))
-        self.convs.append(DistSAGEConvGrad(hidden_channels, out_channels, num_bits, is_pre_delay))
+        self.convs.append(DistSAGEConvGrad(hidden_channels, out_channels, num_bits, is_pre_delay, gemm=gemm))
         if linear_first_when_narrowing:  # a layer with fewer outputs than inputs aggregates its outputs
             for conv in self.convs:
                 conv.linear_first = conv.out_channels < conv.in_channels

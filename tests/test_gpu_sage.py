@@ -207,7 +207,8 @@ def _cpu_mats(graph, is_pre_delay):
 @pytest.mark.parametrize("is_pre_delay", [True, False])
 @pytest.mark.parametrize("fold", [False, True])
 @pytest.mark.parametrize("linear_first", [False, True])
-def test_sage_model_matches_cpu_autograd(is_pre_delay, fold, linear_first):
+@pytest.mark.parametrize("gemm", ["fp32", "bf16x3"])
+def test_sage_model_matches_cpu_autograd(is_pre_delay, fold, linear_first, gemm):
     dev_ = "cuda:0"
     n, f_in, hidden, classes, layers = 5000, 32, 64, 12, 3
     part = synthetic.partition_edges(n, 4, 2, 6, 1.8, 800, 1500, 9000, seed=11, device=dev_)
@@ -216,7 +217,7 @@ def test_sage_model_matches_cpu_autograd(is_pre_delay, fold, linear_first):
     run_graph = sage.fold_in_degrees(graph) if fold else graph
     torch.manual_seed(0)
     model = sage.DistSAGE(f_in, hidden, classes, num_layers=layers, dropout=0.5, is_pre_delay=is_pre_delay,
-                          linear_first_when_narrowing=linear_first).to(dev_)
+                          linear_first_when_narrowing=linear_first, gemm=gemm).to(dev_)
     assert [c.linear_first for c in model.convs] == [False, False, linear_first]   # 32 -> 64 -> 64 -> 12
     with torch.no_grad():  # LayerNorm parameters away from (1, 0) so that their gradients matter
         for norm in model.norms:
@@ -277,6 +278,36 @@ def test_sage_model_matches_cpu_autograd(is_pre_delay, fold, linear_first):
     for b, p in zip(before, model.parameters()):
         moved = float((p.detach() - b).abs().max())
         assert 0.0 < moved <= 5 * 0.01 * 1.01
+
+
+@pytest.mark.parametrize("rows,fi,fo", [(3001, 256, 256), (1000, 128, 172), (517, 32, 12), (0, 64, 64)])
+def test_dense_products_of_the_layer_in_three_bf16_pieces(rows, fi, fo):
+    """The SAGE layer's three dense products in the bf16 x 3 form -- [agg | x] @ W + b, g @ W^T written as column
+    blocks of at most 256 (two blocks at fi = 256), and the two halves of the weight gradient with the bias
+    gradient -- against fp64, at the fp32 kernels' tolerances."""
+    from gnn_benchmark_amd import gcn
+
+    gen = torch.Generator(device="cuda").manual_seed(rows + fi + fo)
+    cat = torch.randn(rows, 2 * fi, device="cuda", generator=gen)
+    w = torch.randn(2 * fi, fo, device="cuda", generator=gen) / (2 * fi) ** 0.5
+    b = torch.randn(fo, device="cuda", generator=gen)
+    g = torch.randn(rows, fo, device="cuda", generator=gen)
+    out = gcn.stacked_product(cat, w, b, gcn.BF16X3)
+    ref = cat.double() @ w.double() + b.double()
+    size = cat.double().abs() @ w.double().abs() + b.double().abs()
+    assert out.shape == ref.shape and bool(((out.double() - ref).abs() <= 1e-6 * size).all())
+    grad_cat = gcn.input_gradient(g, w, gcn.BF16X3)
+    ref = g.double() @ w.double().t()
+    size = g.double().abs() @ w.double().abs().t()
+    assert grad_cat.shape == ref.shape and bool(((grad_cat.double() - ref).abs() <= 1e-6 * size).all())
+    if rows:
+        assert torch.equal(grad_cat, torch.cat([gcn.input_gradient(g, w[:fi], gcn.BF16X3),
+                                                gcn.input_gradient(g, w[fi:], gcn.BF16X3)], dim=1))
+    for half in (cat[:, :fi], cat[:, fi:]):
+        gw, gb = gcn.weight_and_bias_gradient(half, g, gcn.BF16X3)
+        ref = half.double().t() @ g.double()
+        assert float((gw.double() - ref).abs().max()) <= 2e-5 * (float(ref.abs().max()) + 1e-12)
+        assert float((gb.double() - g.double().sum(0)).abs().max()) <= 2e-5 * (float(g.double().sum(0).abs().max()) + 1e-12)
 
 
 def test_sage_layer_single_rank_and_eval_mode():
