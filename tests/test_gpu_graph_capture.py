@@ -52,6 +52,9 @@ def test_entry_points_replay_from_a_hip_graph(monkeypatch):
         x_in, w_in, b_in = (t.detach().clone().requires_grad_() for t in (x, weight, bias))
         layer = gcn._FusedLayer.apply(x_in, w_in, b_in, keep_bits, 2.0, div, True)
         layer.backward(dx)
+        x3, w3, b3 = (t.detach().clone().requires_grad_() for t in (x, weight, bias))
+        layer3 = gcn._FusedLayer.apply(x3, w3, b3, keep_bits, 2.0, div, True, gcn.BF16X3)  # the bf16 x 3 product kernels
+        layer3.backward(dx)
         rows = torch.empty(index.numel(), feat, device="cuda")
         _gather_rows(act, index, rows)
         packed = torch.empty((packed_rows, feat), dtype=torch.uint8, device="cuda")
@@ -65,7 +68,7 @@ def test_entry_points_replay_from_a_hip_graph(monkeypatch):
         _convert(half, wire)
         # (the left half of `cat` is scratch for a following layer and is never written here)
         return [out, dx, wide, cat[:, feat:], act, w, rows, packed, params, back, wire, layer.detach(), x_in.grad,
-                w_in.grad, b_in.grad]
+                w_in.grad, b_in.grad, layer3.detach(), x3.grad, w3.grad, b3.grad]
 
     eager = [t.clone() for t in work()]
     torch.cuda.synchronize()
