@@ -34,6 +34,7 @@ EXPORTS = (
     "gnnagg_wgrad_workspace_bytes",
     "gnnagg_wgrad_f32",
     "gnnagg_wgrad_strided_f32",
+    "gnnagg_wgrad_noalloc_f32",
     "gnnagg_linear_shape_supported",
     "gnnagg_pack_keep_bits",
     "gnnagg_linear_bias_relu_dropout_f32",
@@ -131,6 +132,8 @@ def lib() -> ctypes.CDLL:
     L.gnnagg_bf16_to_f32.argtypes = [vp, vp, i64, vp]
     L.gnnagg_wgrad_strided_f32.restype = i32
     L.gnnagg_wgrad_strided_f32.argtypes = [vp, i64, vp, i64, vp, vp, i64, i64, i64, vp]
+    L.gnnagg_wgrad_noalloc_f32.restype = i32
+    L.gnnagg_wgrad_noalloc_f32.argtypes = [vp, vp, vp, i64, i64, i64, vp]
     L.gnnagg_linear_shape_supported.restype = i32
     L.gnnagg_linear_shape_supported.argtypes = [i64, i64]
     L.gnnagg_pack_keep_bits.restype = i32

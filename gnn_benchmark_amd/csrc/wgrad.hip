@@ -13,6 +13,8 @@
 // and the B operand wants G[r][n] across lanes n, so no transpose is needed.  Per-slice
 // partial outputs are added up in slice order by a second kernel (deterministic, no
 // atomics).
+#include <mutex>
+
 #include "common.h"
 #include "dense_tiles.h"
 
@@ -715,6 +717,56 @@ extern "C" int gnnagg_wgrad_strided_f32(const float *x, int64_t x_stride, const 
                                         float *w_grad, void *workspace, int64_t rows, int64_t fi, int64_t fo,
                                         void *stream) {
     return run_wgrad(x, x_stride, g, g_stride, w_grad, workspace, rows, fi, fo, stream, nullptr, nullptr);
+}
+
+// ---- the entry point that allocates nothing -------------------------------------------------------------------
+// The per-slice partial results of gnnagg_wgrad_f32 normally live in a workspace the caller allocates.  Callers that
+// cannot allocate (code under HIP graph capture, serving loops) get the same kernels with the partial results in a
+// file-scope device array instead.  256 slices x 256 x 256 outputs x 4 bytes = 64 MiB per GPU the library runs on,
+// held until the process ends: every shape the kernels take (Fi, Fo <= 256) fits.
+constexpr size_t kScratchFloats = (size_t)256 * 256 * 256;
+static __device__ __align__(256) float scratch[kScratchFloats];
+
+namespace {
+
+// `scratch` above is a host-side stand-in for the symbol, not a device address; every GPU holds its own copy of
+// the array at its own address, looked up once per device with that device current.
+constexpr int kMaxDevices = 64;
+float *scratch_ptr[kMaxDevices];
+std::mutex scratch_mutex;
+
+int scratch_of_current_device(float **out) {
+    int dev = -1;
+    GNNAGG_HIP(hipGetDevice(&dev));
+    GNNAGG_REQUIRE(dev >= 0 && dev < kMaxDevices, "device ordinal %d outside 0..%d", dev, kMaxDevices - 1);
+    std::lock_guard<std::mutex> hold(scratch_mutex);
+    if (!scratch_ptr[dev]) {
+        void *p = nullptr;
+        GNNAGG_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        GNNAGG_REQUIRE(p, "no device address for the built-in scratch array on device %d", dev);
+        scratch_ptr[dev] = static_cast<float *>(p);
+    }
+    *out = scratch_ptr[dev];
+    return GNNAGG_OK;
+}
+
+}  // namespace
+
+extern "C" int gnnagg_wgrad_noalloc_f32(const float *x, const float *g, float *w_grad, int64_t rows, int64_t fi,
+                                        int64_t fo, void *stream) {
+    GNNAGG_REQUIRE(rows >= 0 && fi > 0 && fo > 0, "bad size");
+    const int64_t need = rows == 0 ? 0 : (int64_t)wgrad_blocks(rows) * fi * fo * (int64_t)sizeof(float);
+    if (fi > 256 || fo > 256 || need > (int64_t)(kScratchFloats * sizeof(float)))
+        return fail(GNNAGG_ERR_UNSUPPORTED,
+                    "Fi=%lld Fo=%lld needs more than the %lld bytes of the built-in scratch array (Fi, Fo <= 256); "
+                    "use gnnagg_wgrad_f32 with a workspace",
+                    (long long)fi, (long long)fo, (long long)(kScratchFloats * sizeof(float)));
+    float *partial = nullptr;
+    const int rc = scratch_of_current_device(&partial);
+    if (rc != GNNAGG_OK) return rc;
+    // every slice writes all Fi x Fo of its partial results before the reduction reads them: nothing in the array
+    // has to start at zero, whatever the previous call left there
+    return run_wgrad(x, fi, g, fo, w_grad, partial, rows, fi, fo, stream, nullptr, nullptr);
 }
 
 extern "C" int64_t gnnagg_wgrad_relu_dropout_backward_workspace_bytes(int64_t rows, int64_t fi, int64_t fo) {

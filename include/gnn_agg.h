@@ -190,6 +190,16 @@ int gnnagg_wgrad_f32(const float *x, const float *g, float *w_grad, void *worksp
 int gnnagg_wgrad_strided_f32(const float *x, int64_t x_stride, const float *g, int64_t g_stride, float *w_grad,
                              void *workspace, int64_t rows, int64_t fi, int64_t fo, void *stream);
 
+/* gnnagg_wgrad_f32 for callers that cannot allocate device memory (code recorded into a HIP graph, tight serving
+ * loops, harnesses that forbid hipMalloc): no workspace argument, the per-slice partial results go to a 64 MiB
+ * device array built into the library (one per GPU the library runs on, held until the process ends), which fits
+ * every shape gnnagg_wgrad_f32 takes; fi or fo above 256 return GNNAGG_ERR_UNSUPPORTED.  Same kernels, same result
+ * bit for bit.  Calls no hipMalloc / hipFree; its first call on a device looks the array's address up (make that call
+ * outside any capture).  All calls on one GPU share that GPU's array: calls that overlap on one GPU (two streams, two
+ * host threads) race -- order them.  No counterpart in the reference. */
+int gnnagg_wgrad_noalloc_f32(const float *x, const float *g, float *w_grad, int64_t rows, int64_t fi, int64_t fo,
+                             void *stream);
+
 /* ---------------------------------------------------------------------------------
  * Dense layer product with the elementwise work behind it fused in (fp32 MFMA, hand-written):
  *   y = relu((x @ w) / row_div + bias) * (keep ? scale : 0)
