@@ -511,15 +511,20 @@ class GCN(torch.nn.Module):
         return hit[1]
 
     def forward(self, graph, x: torch.Tensor, is_pre_delay: bool, masks: Optional[List[torch.Tensor]] = None,
-                log_probs: bool = True, last_rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+                log_probs: bool = True, last_rows: Optional[torch.Tensor] = None,
+                hidden: Optional[list] = None) -> torch.Tensor:
         """``masks[l]``: keep-mask of the dropout after layer l (training only): bool [N, dims[l+1]], or
         its bit-packed form (``pack_keep_mask``) for a layer that runs fused.  ``log_probs=False``
         returns the last layer's output before the log-softmax.  ``last_rows`` (local node ids): evaluate the last
         layer for those nodes only and return ``[len(last_rows), classes]`` -- the rows a loss over them needs, at a
-        fraction of the last aggregation and product, forward and backward (``aggregator.restrict_output_rows``)."""
+        fraction of the last aggregation and product, forward and backward (``aggregator.restrict_output_rows``).
+        ``hidden``: a list that receives every hidden layer's output (the tensors themselves -- a ``(values, header)``
+        pair where activations are kept packed), for callers that want to look at them."""
         h = x
         last = len(self.layers) - 1
         for l, layer in enumerate(self.layers):
+            if hidden is not None and l > 0:
+                hidden.append(h)
             if l == last:
                 g_last = graph
                 if last_rows is not None:

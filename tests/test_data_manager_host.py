@@ -1,6 +1,8 @@
 """Host logic: the vectorised index-map builders of gnn_benchmark_amd.data_manager must
 reproduce (a) the reference's known-answer vectors and (b) the loop-faithful oracle on
-seeded random partitions, bit for bit (int64 maps)."""
+seeded random partitions, bit for bit (int64 maps).  The reference's vectors run twice: on
+host tensors here, and -- marked ``gpu`` -- on device tensors, where the sorts, scans and the
+CSR builds are the device code the product runs."""
 import numpy as np
 import pytest
 import torch
@@ -17,24 +19,44 @@ def N(x):
     return np.asarray(x, dtype=np.int64)
 
 
+def same(a, b):
+    """Equal values; the per-rank prefix arrays ([world + 1] entries) stay on the host whatever the edge lists' device."""
+    return torch.equal(a.cpu(), b.cpu())
+
+
+@pytest.fixture(params=["cpu", pytest.param("cuda", marks=pytest.mark.gpu)])
+def on(request):
+    """Maker of int64 tensors on the device under test."""
+    device = request.param
+
+    def make(x):
+        return torch.tensor(x, dtype=torch.int64, device=device)
+
+    make.device = device
+    return make
+
+
 # ------------------------------------------------------------------ reference vectors
-def test_sort_remote_edges(golden):
+def test_sort_remote_edges(golden, on):
+    T = on
     for c in golden["sort_remote_edges"]:
         out = DataProcessor.sort_remote_edges_list_based_on_remote_nodes(T(c["edges"]))
         assert torch.equal(out, T(c["expected"]))
 
 
-def test_obtain_remote_nodes_list(golden):
+def test_obtain_remote_nodes_list(golden, on):
+    T = on
     for c in golden["obtain_remote_nodes_list"]:
         edges = DataProcessor.sort_remote_edges_list_based_on_remote_nodes(T(c["edges"]))
         nodes, ranges, counts = DataProcessor.obtain_remote_nodes_list(edges, c["num_local_nodes"], T(c["begins"]),
                                                                        c["world_size"])
         assert torch.equal(edges, T(c["expected_edges"]))
         assert torch.equal(nodes, T(c["expected_remote_nodes"]))
-        assert torch.equal(ranges, T(c["expected_ranges"])) and torch.equal(counts, T(c["expected_counts"]))
+        assert same(ranges, T(c["expected_ranges"])) and same(counts, T(c["expected_counts"]))
 
 
-def test_transform_edge_index_to_sparse_tensor(golden):
+def test_transform_edge_index_to_sparse_tensor(golden, on):
+    T = on
     for c in golden["transform_edge_index_to_sparse_tensor"]:
         local, remote = DataProcessor.transform_edge_index_to_sparse_tensor(
             [T(c["local_edges"][0]), T(c["local_edges"][1])], [T(c["remote_edges"][0]), T(c["remote_edges"][1])],
@@ -45,29 +67,35 @@ def test_transform_edge_index_to_sparse_tensor(golden):
             expect = torch.zeros(coo["size"])
             expect[coo["row"], coo["col"]] = torch.tensor(coo["val"])
             assert list(got.sparse_sizes()) == coo["size"]
-            assert torch.equal(got.to_dense() > 0, expect > 0)
+            assert got.device.type == on.device
+            assert torch.equal(got.to_dense().cpu() > 0, expect > 0)
             assert got.nnz() == len(edges[0]) and float(got.to_dense().sum()) == len(edges[0])
 
 
-def test_get_in_degrees(golden):
+def test_get_in_degrees(golden, on):
+    T = on
     for c in golden["get_in_degrees"]:
         got = DataProcessor.get_in_degrees([T(x) for x in c["local_edges"]], [T(x) for x in c["remote_edges"]],
                                            c["num_local_nodes"])
-        assert got.dtype == torch.float32 and torch.equal(got, torch.tensor(c["expected"]))
+        assert got.device.type == on.device
+        assert got.dtype == torch.float32 and torch.equal(got.cpu(), torch.tensor(c["expected"]))
 
 
-def test_get_degrees(golden):
+def test_get_degrees(golden, on):
+    T = on
     for c in golden["get_degrees"]:
         assert DataProcessorForPreAggresive.get_degrees(T(c["nodes"])) == {int(k): v for k, v in c["expected"].items()}
 
 
-def test_decide_pre_or_post_aggr(golden):
+def test_decide_pre_or_post_aggr(golden, on):
+    T = on
     for c in golden["decide_pre_or_post_aggr"]:
         got = DataProcessorForPreAggresive.decide_pre_or_post_aggr(T(c["src"]), T(c["dst"]), c["is_pre"], c["is_post"])
         assert got.dtype == torch.int64 and torch.equal(got, T(c["expected"])), c["source"]
 
 
-def test_collect_edges_sent_to_other_subgraphs(golden):
+def test_collect_edges_sent_to_other_subgraphs(golden, on):
+    T = on
     for c in golden["collect_edges_sent_to_other_subgraphs"]:
         sent = []
         DataProcessorForPreAggresive.collect_edges_sent_to_other_subgraphs(
@@ -77,16 +105,18 @@ def test_collect_edges_sent_to_other_subgraphs(golden):
         assert torch.equal(sent[0][n:], T(c["expected_dst_to_send"])), c["source"]
 
 
-def test_collect_edges_for_aggregation(golden):
+def test_collect_edges_for_aggregation(golden, on):
+    T = on
     for c in golden["collect_edges_for_aggregation"]:
-        lists, splits, begin = [T([]), T([])], [], torch.zeros(2, dtype=torch.int64)
+        lists, splits, begin = [T([]), T([])], [], torch.zeros(2, dtype=torch.int64, device=on.device)
         DataProcessorForPreAggresive.collect_edges_for_aggregation(
             T(c["src"]), T(c["dst"]), T(c["pre_idx"]), T(c["post_idx"]), lists, splits, begin, 0)
         assert torch.equal(lists[0], T(c["expected_src"])) and torch.equal(lists[1], T(c["expected_dst"]))
-        assert splits == c["expected_splits"] and torch.equal(begin, T(c["expected_begin_edge"]))
+        assert splits == c["expected_splits"] and same(begin, T(c["expected_begin_edge"]))
 
 
-def test_split_remote_edges_for_aggr_and_graph_exchange(golden):
+def test_split_remote_edges_for_aggr_and_graph_exchange(golden, on):
+    T = on
     for c in golden["split_remote_edges_for_aggr_and_graph_exchange"]:
         sent, aggr, begin_from, recv_splits = (
             DataProcessorForPreAggresive.split_remote_edges_for_aggr_and_graph_exchange(
@@ -95,18 +125,20 @@ def test_split_remote_edges_for_aggr_and_graph_exchange(golden):
             assert torch.equal(got, T(exp))
         assert torch.equal(aggr[0], T(c["expected_aggr_on_recv"][0]))
         assert torch.equal(aggr[1], T(c["expected_aggr_on_recv"][1]))
-        assert torch.equal(begin_from, T(c["expected_begin_edge_from"])) and recv_splits == c["expected_recv_splits"]
+        assert same(begin_from, T(c["expected_begin_edge_from"])) and recv_splits == c["expected_recv_splits"]
 
 
-def test_split_remote_edges_recv_from_graph_exchange(golden):
+def test_split_remote_edges_recv_from_graph_exchange(golden, on):
+    T = on
     for c in golden["split_remote_edges_recv_from_graph_exchange"]:
         lists, begin_to, splits = DataProcessorForPreAggresive.split_remote_edges_recv_from_graph_exchange(
             [T(x) for x in c["recv_lists"]], c["world_size"])
         assert torch.equal(lists[0], T(c["expected_lists"][0])) and torch.equal(lists[1], T(c["expected_lists"][1]))
-        assert torch.equal(begin_to, T(c["expected_begin_edge_to"])) and splits == c["expected_send_splits"]
+        assert same(begin_to, T(c["expected_begin_edge_to"])) and splits == c["expected_send_splits"]
 
 
-def test_remap_remote_nodes_id(golden):
+def test_remap_remote_nodes_id(golden, on):
+    T = on
     for c in golden["remap_remote_nodes_id"]:
         nodes = T(c["nodes"])
         assert DataProcessorForPreAggresive.remap_remote_nodes_id(nodes, T(c["begins"])) == c["expected_count"]
@@ -293,7 +325,8 @@ def test_synthetic_partition_maps_equal_oracle_on_host():
 
 
 # ------------------------------------------------------------------ input-side file contract
-def test_divide_edges_into_local_and_remote(golden):
+def test_divide_edges_into_local_and_remote(golden, on):
+    T = on
     from gnn_benchmark_amd.data_manager import divide_edges_into_local_and_remote
 
     for c in golden["divide_edges_into_local_and_remote"]:

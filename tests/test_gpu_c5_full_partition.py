@@ -1,0 +1,134 @@
+"""The full train-step workload at its stated shape: a 3-layer GCN, widths 128 -> 256 -> 256 -> 172, on one rank's
+partition of a 16-way split (7 M local nodes, ~100 M local edges, ~20 M edges into ~3 M halo rows), labels on a tenth
+of the nodes, dropout 0.5 with seeded masks, seeded halo rows in place of the exchange.
+
+No CPU run finishes this size in test time, so the check is agreement between the forms the step can take, each of
+which is pinned against CPU autograd at the same widths on a 20 000-node partition
+(``test_gpu_gcn.py::test_train_step_matches_cpu_autograd[c5_widths-...]``):
+
+* one fused kernel per layer each way (fp32 MFMA products) -- the yardstick;
+* the BLAS product and the elementwise passes apart (``fused_layers=False``);
+* the products as three bf16 pieces per operand (``gemm="bf16x3"``: fp32 accuracy);
+* hidden activations kept packed (equal to the dense form bit for bit);
+* every node through the last layer (``restrict_last_layer=False``, the reference's epoch as written) against the
+  last layer evaluated for the labelled rows only.
+
+Tolerances: loss within 1e-4 relative (as at small size).  A weight gradient here is a sum over 7 M rows whose terms
+largely cancel, added up in a different order by every form (and among 1.8 billion hidden units a few have a
+pre-activation within rounding of zero, active in one form and not in another), so single entries differ by more than at small size
+(where 1e-3 of the largest entry holds): every entry within 3e-3 of the largest one, and the whole gradient within
+1e-3 in norm (measured: 1.4e-3 and 2.7e-4 at worst, between the fp32 MFMA and the three-bf16-piece products; the two
+fp32 forms differ by 8e-4 and 2e-4 themselves)."""
+import pytest
+import torch
+
+from gnn_benchmark_amd import gcn, synthetic
+
+pytestmark = pytest.mark.gpu
+
+NODES = 7_000_000
+DIMS = [128, 256, 256, 172]
+TOL = 1e-4
+GRAD_TOL, GRAD_NORM_TOL = 3e-3, 1e-3
+
+
+@pytest.fixture(scope="module")
+def workload():
+    dev = "cuda:0"
+    print(f"building the {NODES}-node partition", flush=True)
+    part = synthetic.partition_edges(num_local_nodes=NODES, world_size=16, rank=3, local_mean_out_degree=6.8,
+                                     zipf_s=1.8, max_degree=15000, num_halo_nodes=int(NODES * 3 / 7),
+                                     num_remote_edges=int(NODES * 20 / 7), seed=4, device=dev)
+    exchange = synthetic.SeededHaloExchange(4, std=0.1, backward_std=1e-7)
+    graph = synthetic.build_partition_graph(part, max(DIMS), True, exchange=exchange, device=dev)
+    del part
+    gen = torch.Generator(device=dev).manual_seed(6)
+    x = torch.randn(NODES, DIMS[0], device=dev, generator=gen)
+    labels = torch.randint(0, DIMS[-1], (NODES,), device=dev, generator=gen)
+    train_idx = torch.randperm(NODES, device=dev, generator=gen)[: NODES // 10]
+    masks = gcn.make_dropout_masks(NODES, DIMS, 0.5, 7, dev)
+    results = {}
+
+    def step(gemm="fp32", fused=True, packed=False, restrict=True):
+        """Loss and parameter gradients of the first train step from the same initial weights (kept per form)."""
+        key = (gemm, fused, packed, restrict)
+        if key not in results:
+            print(f"train step: gemm={gemm} fused={fused} packed={packed} restrict_last_layer={restrict}", flush=True)
+            torch.manual_seed(0)
+            model = gcn.GCN(DIMS, gemm=gemm, packed_activations=packed, fused_layers=fused).to(dev)
+            opt = torch.optim.Adam(model.parameters(), lr=0.01)
+            loss = gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks, restrict)
+            grads = [p.grad.detach().clone() for p in model.parameters()]
+            updated = [p.detach().clone() for p in model.parameters()]
+            torch.cuda.synchronize()
+            results[key] = (float(loss), grads, updated)
+            del model, opt
+            torch.cuda.empty_cache()
+        return results[key]
+
+    yield graph, step
+    results.clear()
+    torch.cuda.empty_cache()
+
+
+def _assert_same_step(got, want, what):
+    loss, grads, _ = got
+    ref_loss, ref_grads, _ = want
+    assert loss == loss and abs(loss - ref_loss) <= TOL * max(1.0, abs(ref_loss)), (what, loss, ref_loss)
+    for i, (a, b) in enumerate(zip(grads, ref_grads)):
+        assert bool(torch.isfinite(a).all()), (what, i)
+        scale = float(b.abs().max()) + 1e-30
+        worst = float((a - b).abs().max()) / scale
+        whole = float((a - b).norm()) / (float(b.norm()) + 1e-30)
+        print(f"{what}: parameter {i}: worst entry {worst:.2e} of the largest, norm of the difference {whole:.2e}", flush=True)
+        assert worst <= GRAD_TOL and whole <= GRAD_NORM_TOL, (what, i, worst, whole)
+
+
+def test_partition_has_the_stated_shape(workload):
+    graph, _ = workload
+    assert graph.local_adj_t.sparse_sizes() == (NODES, NODES)
+    assert 90e6 < graph.local_adj_t.nnz() < 115e6
+    assert 2.7e6 < graph.adj_t_pre_post_aggr_from.sparse_size(1) < 3.3e6
+    assert 18e6 < graph.adj_t_pre_post_aggr_from.nnz() <= 20.5e6
+
+
+def test_loss_starts_at_the_uniform_guess(workload):
+    """Random weights, 172 classes, uniform labels: the first loss sits near log(172) and every gradient is non-zero."""
+    _, step = workload
+    loss, grads, _ = step()
+    assert 4.5 < loss < 6.5, loss
+    for g in grads:
+        assert float(g.abs().max()) > 0.0
+
+
+def test_separate_kernels_agree_with_the_fused_layers(workload):
+    _, step = workload
+    _assert_same_step(step(fused=False), step(), "fused_layers=False")
+
+
+def test_three_bf16_pieces_agree_with_the_fp32_products(workload):
+    _, step = workload
+    _assert_same_step(step(gemm="bf16x3"), step(), "bf16x3")
+
+
+def test_every_node_through_the_last_layer_agrees_with_the_labelled_rows_only(workload):
+    _, step = workload
+    _assert_same_step(step(restrict=False), step(), "restrict_last_layer=False")
+
+
+def test_packed_activations_equal_the_dense_ones(workload):
+    """Packing moves the non-zero values of a hidden row to its front; every sum keeps its terms and their order."""
+    _, step = workload
+    for restrict in (True, False):
+        loss, grads, updated = step(packed=True, restrict=restrict)
+        ref_loss, ref_grads, ref_updated = step(restrict=restrict)
+        assert loss == ref_loss
+        for a, b in zip(grads, ref_grads):
+            assert torch.equal(a, b)
+        for a, b in zip(updated, ref_updated):
+            assert torch.equal(a, b)
+
+
+def test_packed_bf16x3_agrees_with_the_fp32_products(workload):
+    _, step = workload
+    _assert_same_step(step(gemm="bf16x3", packed=True), step(), "bf16x3 packed")

@@ -251,12 +251,15 @@ def _check_properties(src, feat, n_sample, seed):
 
 
 def test_full_size_properties_config2():
-    """The headline workload at its full size: 2.45 M nodes, ~122 M stored elements, F=100."""
+    """The headline workload at its full size: 2.45 M nodes, ~122 M stored elements, F=100, 128 and 256."""
     from gnn_benchmark_amd.synthetic import power_law_graph
 
     g = power_law_graph(num_nodes=2_450_000, mean_out_degree=25.0, zipf_s=1.8, max_degree=15000, seed=0, device="cuda")
     assert 115_000_000 < g.nnz < 130_000_000 and g.max_degree > 10_000
     _check_properties(g.adj, 100, 4000, seed=0)
+    # the two other widths the workload is run at (other launch shapes: 32 lanes x 16 bytes, 64 lanes x 16 bytes)
+    _check_properties(g.adj, 128, 2000, seed=1)
+    _check_properties(g.adj, 256, 2000, seed=2)
 
 
 def test_full_size_properties_config3_dense_degree():
