@@ -15,7 +15,8 @@ with HIP events on the launch stream inside the timed region.  ``cpu_baseline`` 
 reference's own compiled operator (or the C port of it when that cannot run on the
 host) timed on this machine's cores on the same matrices.
 
-``extra`` carries the other workloads, run after the timed headline: c2 at F=128/256,
+``extra`` carries the other workloads, run after the timed headline: c1 (the single-rank 2-layer GCN
+forward + backward, with the same step on the host cores beside it), c2 at F=128/256,
 c3 (dense-degree mean aggregation, F=602/256), c4 (one partition of a 16-way split:
 pre-aggregation, local SpMM, post-aggregation, F=128) and c5 (3-layer GCN train step and the
 reference's 3-layer SAGE model on the c4 partition).  ``--only headline`` skips them.
@@ -32,15 +33,71 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak
 
-# HBM-side traffic of ONE forward launch of the headline workload (default arguments),
-# from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE:
-# FETCH_SIZE 27 768 268 KiB x 2.0 (the counter reads 0.5 KiB per KiB on a 1 GiB device copy)
-# + WRITE_SIZE 987 837 KiB x 1.0.  Keyed by (workload, nodes, mean out-degree, F, seed).
-MEASURED_TRAFFIC_BYTES = {("c2", 2_450_000, 25.0, 100, 0): (27_768_268 * 2.0 + 987_837) * 1024.0}
+# HBM-side traffic of ONE launch, measured with rocprofv3 --pmc on this file's own workloads (default sizes and
+# seed): bytes read = 32 / 64 / 128-byte read requests of the L2 to the memory side, counted by size
+# (TCC_EA0_RDREQ_32B / _64B / _128B), bytes written = WRITE_SIZE.  (workload, op, F) -> (bytes read, bytes written,
+# the summary under profiles/ that holds the counter readings and the commands).  These are constants taken from
+# those profile runs, not something a timed run can produce (the counters need the profiler): the JSON labels
+# them "profile".  Any other size or seed: no entry, and the measured fields are left out.
+MEASURED_TRAFFIC = {
+}
 
 
-def b_alg(nnz: int, rows: int, feat: int) -> float:
-    """Algorithmic bytes of one out += A @ X call (no-reuse gather model)."""
+def measured_traffic(args, workload, op, feat):
+    """(read bytes, written bytes, source) of one launch from MEASURED_TRAFFIC, or None when the run's sizes are
+    not the ones the profiles were taken at."""
+    if (args.nodes, args.mean_out_degree, args.c4_nodes, args.seed) != (2_450_000, 25.0, 7_000_000, 0):
+        return None
+    return MEASURED_TRAFFIC.get((workload, op, feat))
+
+
+def host_cpu():
+    """(model name, physical cores, logical CPUs) of the host, from /proc/cpuinfo."""
+    model, cores, logical = "unknown", set(), 0
+    try:
+        with open("/proc/cpuinfo") as f:
+            phys = core = None
+            for line in f:
+                key, _, val = line.partition(":")
+                key, val = key.strip(), val.strip()
+                if key == "processor":
+                    logical += 1
+                elif key == "model name":
+                    model = val
+                elif key == "physical id":
+                    phys = val
+                elif key == "core id":
+                    core = val
+                elif not key and phys is not None:
+                    cores.add((phys, core))
+                    phys = core = None
+            if phys is not None:
+                cores.add((phys, core))
+    except OSError:
+        pass
+    return model, (len(cores) or logical), logical
+
+
+def cpu_median_seconds(run, warmups=2, reps=5):
+    """Median wall time of `run` over `reps` calls after `warmups` untimed ones."""
+    for _ in range(warmups):
+        run()
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    return times[len(times) // 2]
+
+
+def b_alg(nnz: int, rows: int, feat: int, overwrite_rows: int = None) -> float:
+    """Algorithmic bytes of one call (no-reuse gather model).  out += A @ X over `rows` visited rows: per stored
+    element an int64 column index, an fp32 value and one F-wide fp32 row; per row its rowptr entry and the read and
+    write of its output row.  With `overwrite_rows` (out = A @ X: nothing is read from out, and every one of those
+    rows is written, the ones without stored elements as zeros) the output side is one write per row."""
+    if overwrite_rows is not None:
+        return nnz * 12.0 + (overwrite_rows + 1) * 8.0 + nnz * feat * 4.0 + overwrite_rows * feat * 4.0
     return nnz * 12.0 + (rows + 1) * 8.0 + nnz * feat * 4.0 + 2.0 * rows * feat * 4.0
 
 
@@ -63,27 +120,69 @@ def time_plan(plan, value, x, out, steps, warmup, accumulate=True):
     return sum(k_ms) / len(k_ms), sum(c_ms) / len(c_ms)
 
 
-def op_report(name, nnz, rows, cols, feat, ms, empty_rows=0):
-    """Rates of one accumulate call; rows without stored elements are neither read nor
-    written by the kernel, so they are left out of the byte model."""
+def op_report(name, nnz, rows, cols, feat, ms, empty_rows=0, accumulate=True, measured=None):
+    """Rates of one call.  `frac_model` prices the MODEL bytes (no-reuse gather: every stored element fetches a
+    whole dense row) against the 8 TB/s HBM peak; where gathered rows are re-read out of L2 or the 256 MB
+    memory-side cache the model counts bytes HBM never moved, so it can exceed 1 and is not an HBM fraction.
+    `frac_measured` prices the traffic the counters saw on the memory side of the L2 (`measured`: bytes read,
+    bytes written, profile) in the time measured here.  Accumulate calls neither read nor write rows without
+    stored elements; overwrite calls write every row."""
     rows_total, rows = rows, rows - empty_rows
-    gbs = b_alg(nnz, rows, feat) / (ms * 1e-3) / 1e9
-    return {"op": name, "rows": rows_total, "rows_visited": rows, "cols": cols, "nnz": nnz, "feat": feat,
-            "ms": round(ms, 4),
-            "gflops": round(2.0 * nnz * feat / (ms * 1e-3) / 1e9, 1), "gbs_model": round(gbs, 1),
-            "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
-            "gbs_floor": round(b_min(nnz, rows, cols, feat) / (ms * 1e-3) / 1e9, 1)}
+    model = b_alg(nnz, rows, feat) if accumulate else b_alg(nnz, rows, feat, overwrite_rows=rows_total)
+    gbs = model / (ms * 1e-3) / 1e9
+    r = {"op": name, "rows": rows_total, "rows_visited": rows if accumulate else rows_total, "cols": cols, "nnz": nnz,
+         "feat": feat, "accumulate": bool(accumulate), "ms": round(ms, 4),
+         "gflops": round(2.0 * nnz * feat / (ms * 1e-3) / 1e9, 1), "bytes_model": model, "gbs_model": round(gbs, 1),
+         "frac_model": round(gbs / HBM_PEAK_GBS, 4),
+         "gbs_floor": round(b_min(nnz, rows, cols, feat) / (ms * 1e-3) / 1e9, 1)}
+    if measured is not None:
+        rd, wr, source = measured
+        r["traffic_measured"] = {"read_bytes": rd, "written_bytes": wr, "kind": "profile", "source": source}
+        r["gbs_measured"] = round((rd + wr) / (ms * 1e-3) / 1e9, 1)
+        r["frac_measured"] = round((rd + wr) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+    return r
 
 
-def cpu_baseline_spmm(src, x_host, g_host, reps=3):
-    """Forward + transposed backward on the host cores with the reference's compiled
-    operator when oracle/_ref holds it (kind "reference"), else the C port (kind "port")."""
-    import numpy as np
+def cpu_operator(threads):
+    """``run(rowptr, col, val, x, out, row_split)`` doing one out += A @ x on the host cores: the reference's own
+    compiled operator when oracle/_ref holds it and the host has AVX-512 (kind "reference"), else the C port of it
+    (kind "port")."""
     import torch
 
     from oracle import spmm as ospmm
 
+    ref = ospmm.load_reference_op()
+    if ref is not None:
+        torch.set_num_threads(threads)
+
+        def run(rowptr, col, val, x, out, row_split):
+            t = torch.from_numpy
+            ref.spmm(t(rowptr), t(col), t(val), t(x), t(out), rowptr.shape[0] - 1, t(row_split),
+                     torch.tensor([0, x.shape[1]], dtype=torch.int32))
+
+        return run, "reference"
+
+    def run(rowptr, col, val, x, out, row_split):
+        ospmm.spmm(rowptr, col, val, x, out, row_split, threads)
+
+    return run, "port"
+
+
+def cpu_description(kind, threads):
+    model, physical, logical = host_cpu()
+    return {"kind": kind, "cores": int(threads), "threads": int(threads), "host_physical_cores": physical,
+            "host_logical_cpus": logical, "cpu_model": model,
+            "protocol": "median of 5 timed calls after 2 warm-ups, OpenMP threads = the host share given to this job"}
+
+
+def cpu_baseline_spmm(src, x_host, g_host):
+    """Forward + transposed backward of the headline workload on the host cores."""
+    import numpy as np
+
+    from oracle import spmm as ospmm
+
     threads = ospmm.max_threads()
+    run, kind = cpu_operator(threads)
     rowptr, col, val = [t.cpu().numpy() for t in src.csr()]
     colptr = src.storage.colptr().cpu().numpy()
     row_t = src.storage.row_T().cpu().numpy()
@@ -93,72 +192,55 @@ def cpu_baseline_spmm(src, x_host, g_host, reps=3):
     # the reference balances its threads on per-row work (model/ops/spmm_kernel.py:7-28); unit weights = nnz
     rs_f = ospmm.distribute_work_for_row(rowptr, np.ones(col.shape[0], np.float32), threads)
     rs_b = ospmm.distribute_work_for_row(colptr, np.ones(col.shape[0], np.float32), threads)
-    ref = ospmm.load_reference_op()
     out_f = np.zeros((rows, feat), dtype=np.float32)
     out_b = np.zeros((cols, feat), dtype=np.float32)
-    if ref is not None:
-        kind = "reference"
-        torch.set_num_threads(threads)
-        t = lambda a: torch.from_numpy(a)  # noqa: E731
-        cs = torch.tensor([0, feat], dtype=torch.int32)
-        args_f = (t(rowptr), t(col), t(val), t(x_host), t(out_f), rows, t(rs_f), cs)
-        args_b = (t(colptr), t(row_t), t(val_t), t(g_host), t(out_b), cols, t(rs_b), cs)
 
-        def run():
-            ref.spmm(*args_f)
-            ref.spmm(*args_b)
-    else:
-        kind = "port"
+    def step():
+        run(rowptr, col, val, x_host, out_f, rs_f)
+        run(colptr, row_t, val_t, g_host, out_b, rs_b)
 
-        def run():
-            ospmm.spmm(rowptr, col, val, x_host, out_f, rs_f, threads)
-            ospmm.spmm(colptr, row_t, val_t, g_host, out_b, rs_b, threads)
-
-    run()  # warm-up
-    times = []
-    for _ in range(reps):
-        t0 = time.perf_counter()
-        run()
-        times.append(time.perf_counter() - t0)
-    times.sort()
-    sec = times[len(times) // 2]
+    sec = cpu_median_seconds(step)
     flops = 2 * 2.0 * col.shape[0] * feat
-    return {"value": round(flops / sec / 1e9, 3), "unit": "GFLOP/s", "cores": int(threads), "kind": kind,
-            "sample": f"full workload: 1 forward + 1 transposed backward, F={feat}, median of {reps} after 1 warm-up",
-            "ms_per_step": round(sec * 1e3, 2)}
+    r = {"value": round(flops / sec / 1e9, 3), "unit": "GFLOP/s"}
+    r.update(cpu_description(kind, threads))
+    r["sample"] = f"the whole workload: 1 forward + 1 transposed backward per step, F={feat} (7 steps, about 2 s)"
+    r["ms_per_step"] = round(sec * 1e3, 2)
+    return r
 
 
-def cpu_time_product(rowptr, col, val, x_host, rows, reps=2):
-    """Median seconds of one out += A @ x on the host cores (reference's compiled operator if
-    loadable, else the C port), plus which of the two ran and the thread count."""
+def cpu_time_product(rowptr, col, val, x_host, rows):
+    """Median seconds of one out += A @ x on the host cores, which operator ran, and the thread count."""
     import numpy as np
-    import torch
 
     from oracle import spmm as ospmm
 
     threads = ospmm.max_threads()
-    feat = x_host.shape[1]
+    run, kind = cpu_operator(threads)
     rs = ospmm.distribute_work_for_row(rowptr, np.ones(col.shape[0], np.float32), threads)
-    out = np.zeros((rows, feat), dtype=np.float32)
-    ref = ospmm.load_reference_op()
-    if ref is not None:
-        torch.set_num_threads(threads)
-        args = (torch.from_numpy(rowptr), torch.from_numpy(col), torch.from_numpy(val), torch.from_numpy(x_host),
-                torch.from_numpy(out), rows, torch.from_numpy(rs), torch.tensor([0, feat], dtype=torch.int32))
-        run = lambda: ref.spmm(*args)  # noqa: E731
-    else:
-        run = lambda: ospmm.spmm(rowptr, col, val, x_host, out, rs, threads)  # noqa: E731
-    run()
-    times = []
-    for _ in range(reps):
-        t0 = time.perf_counter()
-        run()
-        times.append(time.perf_counter() - t0)
-    times.sort()
-    return times[len(times) // 2], ("reference" if ref is not None else "port"), threads
+    out = np.zeros((rows, x_host.shape[1]), dtype=np.float32)
+    return cpu_median_seconds(lambda: run(rowptr, col, val, x_host, out, rs)), kind, threads
 
 
-def spmm_pair(src, feat, steps, warmup, gen):
+def time_planless(src, x, out, steps, warmup=2):
+    """Mean ms of ``computation_ops.spmm`` -- the literal export of the reference's op (ops.cpp:23): rows in their
+    natural order, int64 column indices, no cached plan -- on the launch stream."""
+    import torch
+
+    from gnn_benchmark_amd import computation_ops
+
+    rowptr, col, val = src.csr()
+    empty = torch.empty(0, dtype=torch.int32, device=x.device)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for i in range(warmup + steps):
+        if i == warmup:
+            e0.record()
+        computation_ops.spmm(rowptr, col, val, x, out, src.sparse_size(0), empty, empty)
+    e1.record()
+    e1.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+
+def spmm_pair(src, feat, steps, warmup, gen, args=None, workload=None, planless=False):
     """Times `steps` (forward + transposed backward) steps; returns (report, x, g)."""
     import torch
 
@@ -190,13 +272,29 @@ def spmm_pair(src, feat, steps, warmup, gen):
     bytes_launch = b_alg(nnz, rows - info["empty_rows"], feat)  # empty rows are not visited
     _, fwd_ms = time_plan(plan_f, val, x, out, max(3, steps // 2), 1)
     _, bwd_ms = time_plan(plan_b, val_t, g, dx, max(3, steps // 2), 1)
+    m_f = measured_traffic(args, workload, "A@X", feat) if args is not None else None
+    m_b = measured_traffic(args, workload, "A^T@G", feat) if args is not None else None
     r = {"feat": feat, "steps": steps, "ms_per_step": round(ms_step, 4),
          "gflops": round(2 * 2.0 * nnz * feat / (ms_step * 1e-3) / 1e9, 2),
-         "forward": op_report("A@X", nnz, rows, cols, feat, fwd_ms, info["empty_rows"]),
-         "backward": op_report("A^T@G", nnz, cols, rows, feat, bwd_ms, plan_b.info()["empty_rows"]),
+         "forward": op_report("A@X", nnz, rows, cols, feat, fwd_ms, info["empty_rows"], measured=m_f),
+         "backward": op_report("A^T@G", nnz, cols, rows, feat, bwd_ms, plan_b.info()["empty_rows"], measured=m_b),
          "kernel_ms": round(kern_ms, 4), "kernel_ms_median": round(sorted(k_ms)[len(k_ms) // 2], 4),
          "kernel_ms_min": round(min(k_ms), 4), "kernel_bytes": bytes_launch}
+    if planless:
+        ms = time_planless(src, x, out, max(3, steps // 2))
+        r["forward_without_plan"] = op_report("A@X through computation_ops.spmm (no plan: natural row order, int64 "
+                                              "column indices)", nnz, rows, cols, feat, ms, info["empty_rows"])
+        # that kernel reads the int64 column array itself: 8 more bytes per stored element than the model counts
+        r["forward_without_plan"]["ms_with_plan"] = round(fwd_ms, 4)
     return r, x, g
+
+
+def spmm_kernel_name(feat, planned=True):
+    """The instance of the row kernel a contiguous, 16-byte aligned operand of this width runs in."""
+    vec = 4 if feat % 4 == 0 else (2 if feat % 2 == 0 else 1)
+    shapes = [(32, 1), (64, 1), (64, 2), (64, 3), (64, 4), (64, 5), (64, 6), (64, 8)]
+    lpr, nch = next(((l, n) for l, n in shapes if vec * l * n >= feat), shapes[-1])
+    return f"gnnagg::spmm_tasks_kernel<{vec},{lpr},{nch},{'int' if planned else 'long'},{1 if planned else 0},0>"
 
 
 def run_c2(args):
@@ -214,9 +312,9 @@ def run_c2(args):
     torch.cuda.synchronize()
     setup_s = time.perf_counter() - t0
     gen = torch.Generator(device=dev).manual_seed(args.seed)
-    r, x, gr = spmm_pair(src, args.feat, args.steps, args.warmup, gen)
+    r, x, gr = spmm_pair(src, args.feat, args.steps, args.warmup, gen, args, "c2", planless="c2" in args.extras)
     achieved = r["kernel_bytes"] / (r["kernel_ms"] * 1e-3) / 1e9
-    traffic = MEASURED_TRAFFIC_BYTES.get(("c2", args.nodes, args.mean_out_degree, args.feat, args.seed))
+    m = measured_traffic(args, "c2", "A@X", args.feat)
     line = {
         "metric": "spmm_fwd_bwd_gflops", "value": r["gflops"], "unit": "GFLOP/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": r["ms_per_step"], "higher_is_better": True, "scaling": "weak",
@@ -227,8 +325,11 @@ def run_c2(args):
                    "nodes": g.num_nodes, "nnz": g.nnz, "feat": args.feat, "seed": args.seed,
                    "huge_rows": info["huge_rows"], "max_row_len": info["max_row_len"], "setup_s": round(setup_s, 2)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
-                     "kernel": "gnnagg::spmm_tasks_kernel<4,32,1,int,1> (forward A@X, one launch over all rows)",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": None if m is None else m[0] + m[1],
+                     "traffic_kind": None if m is None else "constant from a rocprofv3 --pmc run of this workload "
+                                                            "(not produced by this run): " + m[2],
+                     "kernel": spmm_kernel_name(args.feat) + " (forward A@X, one launch over all rows)",
                      "kernel_ms": r["kernel_ms"], "kernel_ms_median": r["kernel_ms_median"],
                      "kernel_ms_min": r["kernel_ms_min"], "bytes_per_launch": r["kernel_bytes"]},
     }
@@ -236,9 +337,147 @@ def run_c2(args):
     if "c2" in args.extras:
         for f in (128, 256):
             if f != args.feat:
-                extra["c2"].append(spmm_pair(src, f, max(3, args.steps // 4), 2, gen)[0])
+                extra["c2"].append(spmm_pair(src, f, max(3, args.steps // 4), 2, gen, args, "c2")[0])
     line["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline_spmm(src, x.cpu().numpy(), gr.cpu().numpy())
     return line, extra
+
+
+def run_c1(args):
+    """The single-rank case: 2-layer GCN forward + backward (no halo, no exchange) on a power-law graph of 100 000
+    nodes, Zipf(2.0) out-degrees with mean 16, symmetrised with self-loops, values D^-1/2 (A+I) D^-1/2; features
+    N(0,1) F=128, hidden 128, 16 classes, uniform labels.  The same step on the host cores beside it: the
+    aggregations through the reference's compiled operator (forward through the CSR, backward through the
+    transposed CSR, as its wrappers do), the dense parts by torch on the CPU."""
+    import numpy as np
+    import torch
+    import torch.nn.functional as F
+
+    from gnn_benchmark_amd import gcn, synthetic
+    from gnn_benchmark_amd.data_manager import CommBuffer, CommSplits, DistributedGraphForPre
+
+    dev = "cuda:0"
+    n, feat, hidden, classes = 100_000, 128, 128, 16
+    g = synthetic.power_law_graph(n, 16, 2.0, 20_000, seed=args.seed + 1, device=dev)
+    splits = CommSplits([0], [0], 1, 32)
+    graph = DistributedGraphForPre(g.adj, None, None, [0], [0], torch.ones(n, 1, device=dev), splits,
+                                   CommBuffer(splits, feat, 32, device=dev), None, exchange=None)
+    gen = torch.Generator(device=dev).manual_seed(args.seed + 2)
+    x = torch.randn(n, feat, device=dev, generator=gen)
+    labels = torch.randint(0, classes, (n,), device=dev, generator=gen)
+    torch.manual_seed(args.seed + 3)
+    model = gcn.GCN([feat, hidden, classes], dropout=0.0).to(dev)
+    model.train()
+
+    def step():
+        model.zero_grad(set_to_none=True)
+        loss = F.nll_loss(model(graph, x, True, None), labels)
+        loss.backward()
+        return loss
+
+    steps = max(10, args.steps)
+    for _ in range(3):
+        loss = step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        loss = step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    plan = g.adj.get_plan()
+    out_buf = torch.zeros(n, feat, device=dev)
+    _, spmm_ms = time_plan(plan, g.adj.csr()[2], x, out_buf, steps, 2, accumulate=False)
+    r = {"workload": f"c1: single rank, 2-layer GCN forward + backward, {n} nodes / {g.nnz} nnz (longest row "
+                     f"{g.max_degree}), F={feat}, hidden {hidden}, {classes} classes",
+         "forward_backward_ms": round(ms, 3), "loss": round(float(loss.detach()), 5), "steps": steps,
+         "aggregation": op_report("A@X (overwriting)", g.nnz, n, n, feat, spmm_ms, plan.info()["empty_rows"], False)}
+    if args.no_cpu_baseline:
+        return r
+    from oracle import spmm as ospmm
+
+    threads = ospmm.max_threads()
+    run, kind = cpu_operator(threads)
+    csr = [t.cpu().numpy() for t in g.adj.csr()]
+    csc = [g.adj.storage.colptr().cpu().numpy(), g.adj.storage.row_T().cpu().numpy(),
+           g.adj.storage.value_T().cpu().numpy()]
+    ones = np.ones(csr[1].shape[0], np.float32)
+    rs_f = ospmm.distribute_work_for_row(csr[0], ones, threads)
+    rs_b = ospmm.distribute_work_for_row(csc[0], ones, threads)
+
+    class HostAggregate(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, t):
+            out = np.zeros((n, t.shape[1]), dtype=np.float32)
+            run(csr[0], csr[1], csr[2], np.ascontiguousarray(t.detach().numpy()), out, rs_f)
+            return torch.from_numpy(out)
+
+        @staticmethod
+        def backward(ctx, grad):
+            out = np.zeros((n, grad.shape[1]), dtype=np.float32)
+            run(csc[0], csc[1], csc[2], np.ascontiguousarray(grad.numpy()), out, rs_b)
+            return torch.from_numpy(out)
+
+    w = [p.detach().cpu().clone().requires_grad_() for p in model.parameters()]  # W1, b1, W2, b2
+    x_host, labels_host = x.cpu(), labels.cpu()
+
+    def host_step():
+        for p in w:
+            p.grad = None
+        h = torch.relu(HostAggregate.apply(x_host) @ w[0] + w[1])
+        z = HostAggregate.apply(h) @ w[2] + w[3]
+        host_loss = F.nll_loss(F.log_softmax(z, dim=1), labels_host)
+        host_loss.backward()
+        return host_loss
+
+    sec = cpu_median_seconds(host_step)
+    r["cpu"] = {"forward_backward_ms": round(sec * 1e3, 2), "loss": round(float(host_step().detach()), 5)}
+    r["cpu"].update(cpu_description(kind, threads))
+    return r
+
+
+def run_ceilings(args):
+    """What the memory system delivers, in this run, for plain kernels with the access mixes of the aggregation
+    path (`gnnagg_memory_probe`): streams, uniformly random 512-byte row gathers with nothing written, and the
+    same gathers mixed with the row writes / row read-modify-writes of the boundary products (7 gathers per row
+    written: the pre-aggregation's mix; 3 per row read and written: the post-aggregation's; 15: the local product's
+    on a graph without hub rows).  Sizes of the c4 partition at F=128: 7 M source rows, 20 M gathers."""
+    import torch
+
+    from gnn_benchmark_amd import _lib
+
+    dev = torch.device("cuda:0")
+    rows, feat, gathers = args.c4_nodes, 128, int(args.c4_nodes * 20 / 7)
+    gen = torch.Generator(device=dev).manual_seed(args.seed + 9)
+    src = torch.randn(rows, feat, device=dev, generator=gen)
+    dst = torch.zeros(rows, feat, device=dev)
+    index = torch.randint(0, rows, (gathers,), device=dev, generator=gen, dtype=torch.int32)
+    L = _lib.lib()
+    stream = _lib.current_stream(dev)
+
+    def timed(kind, count, per_row, nbytes, reps=10):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for i in range(reps + 2):
+            if i == 2:
+                e0.record()
+            _lib.check(L.gnnagg_memory_probe(kind, _lib.ptr(src), _lib.ptr(index), _lib.ptr(dst), count, feat, per_row,
+                                             stream))
+        e1.record()
+        e1.synchronize()
+        ms = e0.elapsed_time(e1) / reps
+        return {"ms": round(ms, 4), "bytes": nbytes, "gbs": round(nbytes / ms / 1e6, 1),
+                "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+
+    n = rows * feat
+    row_b = feat * 4.0
+    out = {"sizes": f"{rows} rows x {feat} fp32, {gathers} gathers through uniformly random int32 row numbers",
+           "stream_read": timed(0, n, 1, n * 4.0), "stream_write": timed(1, n, 1, n * 4.0),
+           "stream_copy": timed(2, n, 1, n * 8.0)}
+    for name, kind, per_row in (("gather_only", 3, 8), ("gather_7_per_row_written", 4, 7),
+                                ("gather_3_per_row_read_and_written", 5, 3),
+                                ("gather_15_per_row_read_and_written", 5, 15), ("gather_15_per_row_written", 4, 15)):
+        results = gathers // per_row
+        nbytes = results * per_row * (row_b + 4.0) + (results * row_b if kind >= 4 else 0) + (results * row_b if kind == 5 else 0)
+        out[name] = timed(kind, results, per_row, nbytes)
+    return out
 
 
 def run_c3(args):
@@ -251,7 +490,7 @@ def run_c3(args):
     gen = torch.Generator(device=dev).manual_seed(args.seed + 3)
     out = {"graph": g.description, "nodes": g.num_nodes, "nnz": g.nnz, "max_row_len": g.max_degree, "runs": []}
     for f in (602, 256):
-        r, x, _g = spmm_pair(g.adj, f, max(3, args.steps // 4), 2, gen)
+        r, x, _g = spmm_pair(g.adj, f, max(3, args.steps // 4), 2, gen, args, "c3")
         if not args.no_cpu_baseline and f == 602:
             rowptr, col, val = [t.cpu().numpy() for t in g.adj.csr()]
             sec, kind, threads = cpu_time_product(rowptr, col, val, x.cpu().numpy(), g.num_nodes)
@@ -274,7 +513,9 @@ def build_c4(args):
                                      num_halo_nodes=int(args.c4_nodes * 3 / 7),
                                      num_remote_edges=int(args.c4_nodes * 20 / 7), seed=args.seed + 4, device=dev)
     # stand-in rows on the scale of real ones: features O(0.1), gradients of a mean loss O(1e-7)
-    exchange = synthetic.SeededHaloExchange(args.seed + 4, std=0.1, backward_std=1e-7)
+    # (the seeded rows are drawn once per layer and direction and kept on the device; a step points the boundary
+    # buffers at them -- no random-number work, and no other work of the stand-in, inside a timed step)
+    exchange = synthetic.PregeneratedHaloExchange(args.seed + 4, std=0.1, backward_std=1e-7)
     graph = synthetic.build_partition_graph(part, 256, True, exchange=exchange, device=dev)
     for m in (graph.local_adj_t, graph.adj_t_pre_post_aggr_from, graph.adj_t_pre_post_aggr_to):
         m.get_plan()
@@ -299,22 +540,40 @@ def run_c4(args, graph, setup_s):
     recv_buf.normal_(generator=gen)
     out = torch.zeros(n, feat, device=dev)
     ops = []
-    for name, m, src_x, dst in (("pre-aggregation A_to@X -> send_buf", graph.adj_t_pre_post_aggr_to, x, send_buf),
-                                ("local A_local@X -> out", graph.local_adj_t, x, out),
-                                ("post-aggregation A_from@recv_buf -> out", graph.adj_t_pre_post_aggr_from, recv_buf, out)):
+    # Each product is timed the way Aggregator runs it (`as_run`): the pre-aggregation OVERWRITES the send buffer and
+    # the local product OVERWRITES the fresh output (no read of the old rows, every row written), the post-aggregation
+    # accumulates onto the output; in the gradient direction A_from^T @ G overwrites the receive buffer, A_local^T @ G
+    # overwrites the fresh gradient and A_to^T @ send_buf accumulates onto it.  The other mode of each is timed too.
+    for key, name, m, src_x, dst, fwd_overwrites, bwd_overwrites in (
+            ("pre", "pre-aggregation A_to@X -> send_buf", graph.adj_t_pre_post_aggr_to, x, send_buf, True, False),
+            ("local", "local A_local@X -> out", graph.local_adj_t, x, out, True, True),
+            ("post", "post-aggregation A_from@recv_buf -> out", graph.adj_t_pre_post_aggr_from, recv_buf, out, False, True)):
         rows, cols = m.sparse_sizes()
-        _, ms = time_plan(m.get_plan(), m.csr()[2], src_x, dst, steps, 2, accumulate=True)
-        ops.append(op_report(name, m.nnz(), rows, cols, feat, ms, m.get_plan().info()["empty_rows"]))
-        if not args.no_cpu_baseline:
-            rowptr, col, val = [t.cpu().numpy() for t in m.csr()]
-            sec, kind, threads = cpu_time_product(rowptr, col, val, src_x.cpu().numpy(), rows)
-            ops[-1]["cpu_ms"] = round(sec * 1e3, 1)
-            ops[-1]["cpu"] = f"{kind} operator, {threads} threads"
+        plan, plan_t = m.get_plan(), m.get_plan_for_transpose()
+        for accumulate in (True, False):
+            _, ms = time_plan(plan, m.csr()[2], src_x, dst, steps, 2, accumulate=accumulate)
+            ops.append(op_report(name + ("" if accumulate else " (overwriting)"), m.nnz(), rows, cols, feat, ms,
+                                 plan.info()["empty_rows"], accumulate,
+                                 measured_traffic(args, "c4", key + ("" if accumulate else "_overwrite"), feat)))
+            ops[-1]["as_run_by_aggregator"] = accumulate != fwd_overwrites
+            if accumulate and not args.no_cpu_baseline:
+                rowptr, col, val = [t.cpu().numpy() for t in m.csr()]
+                sec, kind, threads = cpu_time_product(rowptr, col, val, src_x.cpu().numpy(), rows)
+                ops[-1]["cpu_ms"] = round(sec * 1e3, 1)
+                ops[-1]["cpu"] = f"{kind} operator, {threads} threads"
         back = torch.zeros(cols, feat, device=dev)
-        _, ms = time_plan(m.get_plan_for_transpose(), m.storage.value_T(), dst, back, steps, 2, accumulate=True)
-        ops.append(op_report(name.split(" ")[0] + " transposed (gradient direction)", m.nnz(), cols, rows, feat, ms,
-                             m.get_plan_for_transpose().info()["empty_rows"]))
+        for accumulate in (True, False):
+            _, ms = time_plan(plan_t, m.storage.value_T(), dst, back, steps, 2, accumulate=accumulate)
+            ops.append(op_report(name.split(" ")[0] + " transposed (gradient direction)"
+                                 + ("" if accumulate else " (overwriting)"), m.nnz(), cols, rows, feat, ms,
+                                 plan_t.info()["empty_rows"], accumulate,
+                                 measured_traffic(args, "c4", key + "_T" + ("" if accumulate else "_overwrite"), feat)))
+            ops[-1]["as_run_by_aggregator"] = accumulate != bwd_overwrites
         del back
+    ms = time_planless(graph.local_adj_t, x, out, steps)
+    ops.append(op_report("local A_local@X through computation_ops.spmm (no plan: natural row order, int64 column "
+                         "indices)", graph.local_adj_t.nnz(), n, n, feat, ms,
+                         graph.local_adj_t.get_plan().info()["empty_rows"]))
     # the whole autograd.Function, forward and backward, synthetic halo rows generated on the device
     xr = x.clone().requires_grad_()
     for _ in range(2):
@@ -331,6 +590,7 @@ def run_c4(args, graph, setup_s):
         o.backward(g)
     torch.cuda.synchronize()
     both_ms = (time.perf_counter() - t0) * 1e3 / steps
+    graph.comm_buf.resize_buffer(graph.comm_splits, feat, 32)  # (the buffer's own tensors again, not delivered rows)
     codec = run_c4_codec(graph, feat, steps, gen, cpu=not args.no_cpu_baseline)
     # the same autograd.Function with the boundary rows travelling as int2 (seeded packed rows)
     from gnn_benchmark_amd import synthetic
@@ -517,7 +777,7 @@ def run_c4_raw_halo(args, part):
     feat = 128
     steps = max(5, args.steps // 2)
     t0 = time.perf_counter()
-    graph = synthetic.build_partition_graph(part, 256, False, exchange=synthetic.SeededHaloExchange(args.seed + 4),
+    graph = synthetic.build_partition_graph(part, 256, False, exchange=synthetic.PregeneratedHaloExchange(args.seed + 4),
                                             device=dev)
     torch.cuda.synchronize()
     setup_s = time.perf_counter() - t0
@@ -636,6 +896,25 @@ def run_c5(args, graph):
         out[f"loss_{tag}"] = [round(v, 5) for v in losses + [float(loss)]]
         del model, opt
     del folded
+    # the same default step with the stand-in exchange drawing its rows inside the step (random-number kernels in
+    # the timed region, which a real exchange would not run): how much of a step that was
+    from gnn_benchmark_amd import synthetic
+
+    kept = graph.exchange
+    graph.exchange = synthetic.SeededHaloExchange(kept.seed, std=kept.std, backward_std=kept.backward_std)
+    torch.manual_seed(args.seed)
+    model = gcn.GCN(dims).to(dev)
+    opt = torch.optim.Adam(model.parameters(), lr=0.01)
+    for _ in range(2):
+        gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks, True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks, True)
+    torch.cuda.synchronize()
+    out["train_step_ms_fp32_gemm_halo_rows_drawn_inside_the_step"] = round((time.perf_counter() - t0) * 1e3 / steps, 2)
+    graph.exchange = kept
+    del model, opt
     return out
 
 
@@ -738,14 +1017,16 @@ def main():
     ap.add_argument("--c4-nodes", type=int, default=7_000_000)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--only", default="", help="'headline' = headline workload only; or a comma list of the extra "
-                                                "workloads to add: c2 (F=128/256), c3, c4, c5 (GCN and SAGE train "
-                                                "steps; c5sage: the SAGE one alone).  Default: c2,c3,c4,c5")
+                                                "workloads to add: c1 (single-rank 2-layer GCN), c2 (F=128/256 and "
+                                                "the plan-less operator), c3, c4, c5 (GCN and SAGE train steps; "
+                                                "c5sage: the SAGE one alone).  Default: c1,c2,c3,c4,c5")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy 3 times (a kernel of known traffic for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
-    args.extras = [s for s in (args.only.split(",") if args.only else ["c2", "c3", "c4", "c5"]) if s and s != "headline"]
+    args.extras = [s for s in (args.only.split(",") if args.only else ["c1", "c2", "c3", "c4", "c5"])
+                   if s and s != "headline"]
     if args.gpus != 1:
         print("bench.py measures one GPU's share of the partitioned graph; --gpus must be 1 "
               "(no multi-GPU path exists in this build)", file=sys.stderr)
@@ -764,6 +1045,12 @@ def main():
         del a, b
     line, extra = run_c2(args)
     torch.cuda.empty_cache()
+    if "c1" in args.extras:
+        extra["c1"] = run_c1(args)
+        torch.cuda.empty_cache()
+    if "c4" in args.extras or "ceilings" in args.extras:
+        extra["memory_ceilings"] = run_ceilings(args)
+        torch.cuda.empty_cache()
     if "c3" in args.extras:
         extra["c3"] = run_c3(args)
         torch.cuda.empty_cache()

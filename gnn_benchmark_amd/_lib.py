@@ -19,6 +19,7 @@ EXPORTS = (
     "gnnagg_last_error",
     "gnnagg_spmm_csr_f32",
     "gnnagg_plan_create",
+    "gnnagg_plan_create_ex",
     "gnnagg_plan_destroy",
     "gnnagg_plan_spmm_f32",
     "gnnagg_plan_spmm_strided_f32",
@@ -60,9 +61,18 @@ EXPORTS = (
     "gnnagg_dequantize_mixed_f32",
     "gnnagg_f32_to_bf16",
     "gnnagg_bf16_to_f32",
+    "gnnagg_memory_probe",
 )
 
 _lib = None
+
+
+class PlanOptions(ctypes.Structure):
+    """``gnnagg_plan_options`` of include/gnn_agg.h (a field left 0: the library's default)."""
+    _fields_ = [("long_row_threshold", ctypes.c_int32), ("block_row_threshold", ctypes.c_int32),
+                ("rows_per_group", ctypes.c_int32), ("short_rows_per_group", ctypes.c_int32),
+                ("lanes_per_row", ctypes.c_int32), ("loads_per_lane", ctypes.c_int32),
+                ("reserved", ctypes.c_int32 * 2)]
 
 
 class GnnAggError(RuntimeError):
@@ -98,6 +108,8 @@ def lib() -> ctypes.CDLL:
     L.gnnagg_spmm_csr_f32.argtypes = [vp, vp, vp, vp, vp, i64, i64, vp]
     L.gnnagg_plan_create.restype = i32
     L.gnnagg_plan_create.argtypes = [vp, vp, i64, i64, i64, vp, ctypes.POINTER(vp)]
+    L.gnnagg_plan_create_ex.restype = i32
+    L.gnnagg_plan_create_ex.argtypes = [vp, vp, i64, i64, i64, ctypes.POINTER(PlanOptions), vp, ctypes.POINTER(vp)]
     L.gnnagg_plan_destroy.restype = i32
     L.gnnagg_plan_destroy.argtypes = [vp]
     L.gnnagg_plan_spmm_f32.restype = i32
@@ -184,6 +196,8 @@ def lib() -> ctypes.CDLL:
     L.gnnagg_quantize_mixed_f32.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp]
     L.gnnagg_dequantize_mixed_f32.restype = i32
     L.gnnagg_dequantize_mixed_f32.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp]
+    L.gnnagg_memory_probe.restype = i32
+    L.gnnagg_memory_probe.argtypes = [i32, vp, vp, vp, i64, i64, i64, vp]
     if L.gnnagg_abi_version() != ABI_VERSION:
         raise RuntimeError("libgnnagg.so was built from a different include/gnn_agg.h; rebuild it")
     _lib = L

@@ -1,0 +1,134 @@
+// Memory-system probes: plain kernels with the access mixes of the aggregation path and nothing else, so that a
+// benchmark can put the rate of a product kernel next to what the machine delivers for the same mix of row gathers,
+// row reads and row writes in the same run.  Measurement aids; nothing in the product path calls them.
+#include "common.h"
+
+namespace gnnagg {
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// every lane streams 16-byte pieces, U of them in flight
+template <int U>
+__global__ __launch_bounds__(256) void probe_stream_read_kernel(const f32x4 *__restrict__ x, size_t n4,
+                                                                float *__restrict__ sink) {
+    size_t i = (size_t)blockIdx.x * 256 * U + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * 256 * U;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (; i + 256 * (U - 1) < n4; i += stride) {
+        f32x4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(x + i + 256 * u);
+#pragma unroll
+        for (int u = 0; u < U; ++u) acc += v[u];
+    }
+    // never true for finite data: keeps the loads alive without a store in the measured stream
+    if (acc.x + acc.y + acc.z + acc.w == 1.2345678e38f) sink[0] = acc.x;
+}
+
+__global__ __launch_bounds__(256) void probe_stream_write_kernel(f32x4 *__restrict__ y, size_t n4) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * 256;
+    const f32x4 v = {1.f, 2.f, 3.f, 4.f};
+    for (; i < n4; i += stride) __builtin_nontemporal_store(v, y + i);
+}
+
+__global__ __launch_bounds__(256) void probe_stream_copy_kernel(const f32x4 *__restrict__ x, f32x4 *__restrict__ y,
+                                                                size_t n4) {
+    size_t i = (size_t)blockIdx.x * 1024 + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * 1024;
+    for (; i + 768 < n4; i += stride) {
+        f32x4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = __builtin_nontemporal_load(x + i + 256 * u);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) __builtin_nontemporal_store(v[u], y + i + 256 * u);
+    }
+}
+
+// A group of LPR lanes sums `per_row` gathered rows of LPR * 16 bytes (8 gathers in flight) into one result row:
+// mode 0 drops the result (reads only), 1 writes it, 2 adds it onto the row the destination holds (read + write).
+template <int LPR>
+__global__ __launch_bounds__(256) void probe_gather_kernel(const float *__restrict__ x, const int32_t *__restrict__ index,
+                                                           float *__restrict__ dst, int64_t results, int per_row,
+                                                           int mode, float *__restrict__ sink) {
+    constexpr int U = 8;
+    const int lig = (int)threadIdx.x & (LPR - 1);
+    const int64_t group = ((int64_t)blockIdx.x * 256 + threadIdx.x) / LPR;
+    const int64_t ngroups = (int64_t)gridDim.x * 256 / LPR;
+    constexpr int kRowFloats = LPR * 4;
+    f32x4 keep = {0.f, 0.f, 0.f, 0.f};
+    for (int64_t o = group; o < results; o += ngroups) {
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        float *row = dst + o * kRowFloats + lig * 4;
+        if (mode == 2) acc = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(row));
+        const int32_t *ip = index + o * per_row;
+        for (int j = 0; j < per_row; j += U) {
+            f32x4 v[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int jj = j + u < per_row ? j + u : per_row - 1;  // (a repeated gather: a cache hit)
+                v[u] = *reinterpret_cast<const f32x4 *>(x + (size_t)ip[jj] * kRowFloats + lig * 4);
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (j + u < per_row) acc += v[u];
+        }
+        if (mode == 0) keep += acc;
+        else __builtin_nontemporal_store(acc, reinterpret_cast<f32x4 *>(row));
+    }
+    if (mode == 0 && keep.x + keep.y + keep.z + keep.w == 1.2345678e38f) sink[0] = keep.x;
+}
+
+}  // namespace
+}  // namespace gnnagg
+
+using namespace gnnagg;
+
+extern "C" int gnnagg_memory_probe(int kind, const float *src, const int32_t *index, float *dst, int64_t count,
+                                   int64_t row_floats, int64_t per_row, void *stream) {
+    GNNAGG_REQUIRE(kind >= 0 && kind <= 5, "probe kind %d outside 0..5", kind);
+    GNNAGG_REQUIRE(count >= 0 && count < (int64_t(1) << 40), "bad count");
+    if (count == 0) return GNNAGG_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (kind <= 2) {  // streams over `count` floats
+        GNNAGG_REQUIRE(count % 4 == 0, "stream probes take a multiple of 4 floats");
+        GNNAGG_REQUIRE((kind == 1 || src) && (kind == 0 || dst), "null src/dst");
+        GNNAGG_REQUIRE(((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) == 0,
+                       "stream probes take 16-byte aligned arrays");
+        const size_t n4 = (size_t)count / 4;
+        const unsigned blocks = 32768;
+        if (kind == 0) {
+            GNNAGG_REQUIRE(dst, "the read probe needs 4 writable bytes in dst (never written for finite data)");
+            hipLaunchKernelGGL(probe_stream_read_kernel<8>, dim3(blocks), dim3(256), 0, st,
+                               reinterpret_cast<const f32x4 *>(src), n4, dst);
+        } else if (kind == 1) {
+            hipLaunchKernelGGL(probe_stream_write_kernel, dim3(blocks), dim3(256), 0, st, reinterpret_cast<f32x4 *>(dst), n4);
+        } else {
+            hipLaunchKernelGGL(probe_stream_copy_kernel, dim3(blocks), dim3(256), 0, st,
+                               reinterpret_cast<const f32x4 *>(src), reinterpret_cast<f32x4 *>(dst), n4);
+        }
+        GNNAGG_HIP(hipGetLastError());
+        return GNNAGG_OK;
+    }
+    // row gathers: `count` result rows, each the sum of `per_row` gathered rows
+    GNNAGG_REQUIRE(src && index && dst, "null src/index/dst");
+    GNNAGG_REQUIRE(per_row >= 1 && per_row < (1 << 20), "gathers per result row outside 1 .. 2^20");
+    GNNAGG_REQUIRE(((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) == 0,
+                   "gather probes take 16-byte aligned arrays");
+    const int mode = kind - 3;
+    const unsigned blocks = 65536;
+    // in mode 0 the last 4 bytes of dst stand in for the sink (never written for finite data)
+    float *sink = dst;
+    if (row_floats == 64)
+        hipLaunchKernelGGL(probe_gather_kernel<16>, dim3(blocks), dim3(256), 0, st, src, index, dst, count, (int)per_row, mode, sink);
+    else if (row_floats == 128)
+        hipLaunchKernelGGL(probe_gather_kernel<32>, dim3(blocks), dim3(256), 0, st, src, index, dst, count, (int)per_row, mode, sink);
+    else if (row_floats == 256)
+        hipLaunchKernelGGL(probe_gather_kernel<64>, dim3(blocks), dim3(256), 0, st, src, index, dst, count, (int)per_row, mode, sink);
+    else
+        return fail(GNNAGG_ERR_UNSUPPORTED, "gather probes exist for rows of 64, 128 and 256 floats (got %lld)",
+                    (long long)row_floats);
+    GNNAGG_HIP(hipGetLastError());
+    return GNNAGG_OK;
+}

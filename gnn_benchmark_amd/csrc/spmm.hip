@@ -3,6 +3,7 @@
 #include <hipcub/hipcub.hpp>
 
 #include <algorithm>
+#include <atomic>
 #include <new>
 #include <type_traits>
 #include <vector>
@@ -28,8 +29,13 @@ struct Shape {
     int width() const { return vec * lpr * nch; }
 };
 
-constexpr int kShapes[][2] = {{16, 1}, {32, 1}, {64, 1}, {64, 2}, {64, 3}, {64, 4}, {64, 5}, {64, 6}, {64, 8}};
+// (rows of up to 64 floats would fit 16 lanes, but measured on MI355X 32 lanes per row are 7-8 % faster at every
+// such width -- 16, 20, 40, 48, 64 floats -- so the narrowest shape picked is 32 x 1)
+constexpr int kShapes[][2] = {{32, 1}, {64, 1}, {64, 2}, {64, 3}, {64, 4}, {64, 5}, {64, 6}, {64, 8}};
 constexpr int kNumShapes = sizeof(kShapes) / sizeof(kShapes[0]);
+// every (lanes, loads) pair the row kernel is instantiated for; a plan's options may name one of them
+constexpr int kAllShapes[][2] = {{16, 1}, {16, 2}, {32, 1}, {16, 3}, {32, 2}, {64, 1}, {64, 2},
+                                 {64, 3}, {64, 4}, {64, 5}, {64, 6}, {64, 8}};
 
 // widest vector access that every row of x and dst allows: base addresses and row strides
 // (in floats; rows back to back when the stride is the width) must be multiples of it
@@ -42,7 +48,14 @@ int pick_vec(int64_t feat, const void *x, const void *dst, int64_t ldx, int64_t 
 }
 int pick_vec(int64_t feat, const void *x, const void *dst) { return pick_vec(feat, x, dst, feat, feat); }
 
-Shape pick_shape(int vec, int64_t feat_left) {
+bool shape_exists(int lanes, int loads) {
+    for (const auto &sh : kAllShapes)
+        if (sh[0] == lanes && sh[1] == loads) return true;
+    return false;
+}
+
+Shape pick_shape(int vec, int64_t feat_left, int lanes = 0, int loads = 0) {
+    if (lanes > 0 && loads > 0) return Shape{vec, lanes, loads};  // the plan's options name the shape
     for (int i = 0; i < kNumShapes; ++i) {
         Shape s{vec, kShapes[i][0], kShapes[i][1]};
         if (s.width() >= feat_left) return s;
@@ -50,56 +63,59 @@ Shape pick_shape(int vec, int64_t feat_left) {
     return Shape{vec, kShapes[kNumShapes - 1][0], kShapes[kNumShapes - 1][1]};
 }
 
+// How the rows of one launch are handed to blocks: `rpg` rows per lane group in the middle region, `tail_rpg` in the
+// tail region (the last `tail_tasks` tasks; 0: none).  Fills the region fields of `args`; returns the block count.
+struct Regions {
+    int rpg, tail_rpg;
+    int64_t tail_tasks;
+};
+
+int64_t lay_out_blocks(SpmmArgs &args, int gpb, Regions r) {
+    r.rpg = std::min(std::max(r.rpg, 1), kMaxRowsPerGroup);
+    r.tail_rpg = std::min(std::max(r.tail_rpg, 1), kMaxRowsPerGroup);
+    if (args.head_tasks > args.ntasks) args.head_tasks = args.ntasks;
+    int64_t tail = std::min(std::max<int64_t>(r.tail_tasks, 0), args.ntasks - args.head_tasks);
+    if (r.tail_rpg == r.rpg) tail = 0;  // one region does
+    args.tail_first = args.ntasks - tail;
+    args.tasks_per_block = gpb * r.rpg;
+    args.tail_tasks_per_block = gpb * r.tail_rpg;
+    const int64_t head_blocks = (args.head_tasks + gpb - 1) / gpb;
+    const int64_t mid_blocks = (args.tail_first - args.head_tasks + args.tasks_per_block - 1) / args.tasks_per_block;
+    const int64_t tail_blocks = (tail + args.tail_tasks_per_block - 1) / args.tail_tasks_per_block;
+    if (head_blocks + mid_blocks + tail_blocks > 0x7fffffffll) return -1;
+    args.head_blocks = (int)head_blocks;
+    args.mid_blocks = (int)mid_blocks;
+    return head_blocks + mid_blocks + tail_blocks;
+}
+
 template <int VEC, int LPR, int NCH, typename IdxT, int MODE, int SRC = kSrcDense>
-hipError_t launch_tasks(const SpmmArgs &a, int rows_per_group, hipStream_t stream) {
+hipError_t launch_tasks(const SpmmArgs &a, Regions r, hipStream_t stream) {
     constexpr int GPB = 256 / LPR;
     SpmmArgs args = a;
-    if (rows_per_group > kMaxRowsPerGroup) rows_per_group = kMaxRowsPerGroup;
-    if (rows_per_group < 1) rows_per_group = 1;
-    args.tasks_per_block = GPB * rows_per_group;
-    if (args.head_tasks > args.ntasks) args.head_tasks = args.ntasks;
-    const int64_t head_blocks = (args.head_tasks + GPB - 1) / GPB;
-    const int64_t nblocks =
-        head_blocks + (args.ntasks - args.head_tasks + args.tasks_per_block - 1) / args.tasks_per_block;
+    const int64_t nblocks = lay_out_blocks(args, GPB, r);
     if (nblocks == 0) return hipSuccess;
-    args.head_blocks = (int)head_blocks;
-    if (nblocks > 0x7fffffffll) return hipErrorInvalidValue;
+    if (nblocks < 0) return hipErrorInvalidValue;
     hipLaunchKernelGGL((spmm_tasks_kernel<VEC, LPR, NCH, IdxT, MODE, SRC>), dim3((unsigned)nblocks), dim3(256), 0,
                        stream, args);
     return hipGetLastError();
 }
 
 // Packed source rows (16-byte lanes, one load per lane): widths 32 / 64 -> 16 lanes, 128 -> 32, 256 -> 64.
-hipError_t launch_packed(const SpmmArgs &a, int rows_per_group, hipStream_t stream) {
-    auto go = [&](auto lpr_tag) -> hipError_t {
-        constexpr int LPR = decltype(lpr_tag)::value;
-        constexpr int GPB = 256 / LPR;
-        SpmmArgs args = a;
-        if (rows_per_group > kMaxRowsPerGroup) rows_per_group = kMaxRowsPerGroup;
-        if (rows_per_group < 1) rows_per_group = 1;
-        args.tasks_per_block = GPB * rows_per_group;
-        if (args.head_tasks > args.ntasks) args.head_tasks = args.ntasks;
-        const int64_t head_blocks = (args.head_tasks + GPB - 1) / GPB;
-        const int64_t nblocks =
-            head_blocks + (args.ntasks - args.head_tasks + args.tasks_per_block - 1) / args.tasks_per_block;
-        if (nblocks == 0) return hipSuccess;
-        if (nblocks > 0x7fffffffll) return hipErrorInvalidValue;
-        args.head_blocks = (int)head_blocks;
-        hipLaunchKernelGGL((spmm_tasks_kernel<4, LPR, 1, int32_t, kRowsPlanned, kSrcPacked>), dim3((unsigned)nblocks),
-                           dim3(256), 0, stream, args);
-        return hipGetLastError();
-    };
-    if (a.feat > 128) return go(std::integral_constant<int, 64>{});
-    if (a.feat > 64) return go(std::integral_constant<int, 32>{});
-    return go(std::integral_constant<int, 16>{});
+hipError_t launch_packed(const SpmmArgs &a, Regions r, hipStream_t stream) {
+    if (a.feat > 128) return launch_tasks<4, 64, 1, int32_t, kRowsPlanned, kSrcPacked>(a, r, stream);
+    if (a.feat > 64) return launch_tasks<4, 32, 1, int32_t, kRowsPlanned, kSrcPacked>(a, r, stream);
+    return launch_tasks<4, 16, 1, int32_t, kRowsPlanned, kSrcPacked>(a, r, stream);
 }
 
 template <int VEC, typename IdxT, int MODE, int SRC = kSrcDense>
-hipError_t dispatch_shape(const Shape &s, const SpmmArgs &a, int rpg, hipStream_t st) {
+hipError_t dispatch_shape(const Shape &s, const SpmmArgs &a, Regions rpg, hipStream_t st) {
 #define GNNAGG_CASE(L, N) \
     if (s.lpr == L && s.nch == N) return launch_tasks<VEC, L, N, IdxT, MODE, SRC>(a, rpg, st)
     GNNAGG_CASE(16, 1);
+    GNNAGG_CASE(16, 2);
     GNNAGG_CASE(32, 1);
+    GNNAGG_CASE(16, 3);
+    GNNAGG_CASE(32, 2);
     GNNAGG_CASE(64, 1);
     GNNAGG_CASE(64, 2);
     GNNAGG_CASE(64, 3);
@@ -187,7 +203,7 @@ hipError_t launch_long_rows(const LongArgs &a, int64_t nrows, hipStream_t st) {
 }
 
 template <typename IdxT, int MODE>
-hipError_t dispatch_tasks(const Shape &s, const SpmmArgs &a, int rpg, hipStream_t st) {
+hipError_t dispatch_tasks(const Shape &s, const SpmmArgs &a, Regions rpg, hipStream_t st) {
     if (s.vec == 4) return dispatch_shape<4, IdxT, MODE>(s, a, rpg, st);
     if (s.vec == 2) return dispatch_shape<2, IdxT, MODE>(s, a, rpg, st);
     return dispatch_shape<1, IdxT, MODE>(s, a, rpg, st);
@@ -270,14 +286,6 @@ __global__ __launch_bounds__(256) void build_tasks_kernel(const int64_t *__restr
     task[t] = d;
 }
 
-int env_int(const char *name, int dflt, int lo, int hi) {
-    const char *v = getenv(name);
-    if (!v || !*v) return dflt;
-    const long x = strtol(v, nullptr, 10);
-    if (x < lo || x > hi) return dflt;
-    return (int)x;
-}
-
 }  // namespace
 }  // namespace gnnagg
 
@@ -294,7 +302,13 @@ struct gnnagg_plan {
     int device = 0;
     int32_t *col32 = nullptr;   // [nnz]
     RowTask *task = nullptr;    // [rows] rows by degree class, longest first; ascending row id inside a class
-    int rows_per_group = 4;
+    int64_t nshort = 0;       // rows of 1 .. kShortRowLen elements (the last non-empty tasks)
+    // (measured on MI355X: 1, 2, 4, 8 or 16 rows per group move the boundary products by +-2 % and the local product by
+    // less -- the memory system, not the hand-out of rows, is what bounds them; 2 is the best all round)
+    int rows_per_group = 2;        // rows a lane group walks in the middle region
+    int short_rows_per_group = 2;  // ... and in the tail region of the shortest rows (equal: one region)
+    int lanes = 0, loads = 0;      // launch shape named by the options (0: chosen from the width)
+    std::atomic<bool> busy{false}; // a call is being enqueued (the plan's events and side stream are in use)
     hipStream_t side = nullptr;          // the block-per-row kernel runs here, next to the main launch
     hipEvent_t fork = nullptr, join = nullptr;
     bool profile = false;
@@ -337,7 +351,7 @@ extern "C" int gnnagg_spmm_csr_f32(const int64_t *rowptr, const int64_t *col, co
         a.feat = (int)feat;
         a.f_base = (int)f_base;
         a.accumulate = 1;
-        GNNAGG_HIP((dispatch_tasks<int64_t, kRowsNatural>(s, a, 4, st)));
+        GNNAGG_HIP((dispatch_tasks<int64_t, kRowsNatural>(s, a, Regions{4, 4, 0}, st)));
         f_base += s.width();
     }
     return GNNAGG_OK;
@@ -357,8 +371,25 @@ static void plan_free(gnnagg_plan *p) {
 
 extern "C" int gnnagg_plan_create(const int64_t *rowptr, const int64_t *col, int64_t rows, int64_t cols, int64_t nnz,
                                   void *stream, gnnagg_plan **plan_out) {
+    return gnnagg_plan_create_ex(rowptr, col, rows, cols, nnz, nullptr, stream, plan_out);
+}
+
+// rows of at most this many elements form the tail region (more rows per lane group)
+constexpr int kShortRowLen = 8;
+
+extern "C" int gnnagg_plan_create_ex(const int64_t *rowptr, const int64_t *col, int64_t rows, int64_t cols, int64_t nnz,
+                                     const gnnagg_plan_options *options, void *stream, gnnagg_plan **plan_out) {
     GNNAGG_REQUIRE(plan_out, "null plan_out");
     *plan_out = nullptr;
+    gnnagg_plan_options opt{};
+    if (options) opt = *options;
+    GNNAGG_REQUIRE(opt.long_row_threshold >= 0 && opt.block_row_threshold >= 0 && opt.rows_per_group >= 0 &&
+                       opt.short_rows_per_group >= 0 && opt.rows_per_group <= kMaxRowsPerGroup &&
+                       opt.short_rows_per_group <= kMaxRowsPerGroup,
+                   "plan options: thresholds must not be negative, rows per group lie in 0 .. %d", kMaxRowsPerGroup);
+    GNNAGG_REQUIRE((opt.lanes_per_row == 0 && opt.loads_per_lane == 0) || shape_exists(opt.lanes_per_row, opt.loads_per_lane),
+                   "plan options: no row kernel with %d lanes per row and %d loads per lane", opt.lanes_per_row,
+                   opt.loads_per_lane);
     GNNAGG_REQUIRE(rows >= 0 && cols >= 0 && nnz >= 0, "negative size");
     GNNAGG_REQUIRE(rowptr, "null rowptr");
     GNNAGG_REQUIRE(nnz == 0 || col, "null col with nnz > 0");
@@ -377,15 +408,18 @@ extern "C" int gnnagg_plan_create(const int64_t *rowptr, const int64_t *col, int
     p->rows = rows;
     p->cols = cols;
     p->nnz = nnz;
-    p->long_thresh = env_int("GNNAGG_LONG_THRESH", 256, 1, 1 << 30);
+    p->long_thresh = opt.long_row_threshold > 0 ? opt.long_row_threshold : 256;
     // A row is handed to the block-per-row kernel only when its chain, fed by one lane
     // group (a few elements per microsecond), would outlast the whole launch: that
     // length grows with the matrix, about nnz / 4096 (measured on MI355X), floor 2048 (below it the
     // block-per-row kernel, 50 .. 85 stored elements per microsecond and row, no longer pays).
     int64_t huge_default = std::max<int64_t>(2048, nnz / 4096);
     if (huge_default > (1 << 30)) huge_default = 1 << 30;
-    p->huge_thresh = env_int("GNNAGG_HUGE_THRESH", (int)huge_default, p->long_thresh, 1 << 30);
-    p->rows_per_group = env_int("GNNAGG_ROWS_PER_GROUP", 4, 1, kMaxRowsPerGroup);
+    p->huge_thresh = opt.block_row_threshold > 0 ? std::max(opt.block_row_threshold, p->long_thresh) : (int)huge_default;
+    if (opt.rows_per_group > 0) p->rows_per_group = opt.rows_per_group;
+    if (opt.short_rows_per_group > 0) p->short_rows_per_group = opt.short_rows_per_group;
+    p->lanes = opt.lanes_per_row;
+    p->loads = opt.loads_per_lane;
     GNNAGG_HIP(hipGetDevice(&p->device));
 
     // rowptr end points (host check; also forces the inputs to be ready)
@@ -448,6 +482,8 @@ extern "C" int gnnagg_plan_create(const int64_t *rowptr, const int64_t *col, int
     for (int c = 0; c < thresh_class; ++c) p->nlong += (int64_t)h_out.class_count[c];
     const int huge_class = degree_class(p->huge_thresh);
     for (int c = 0; c < huge_class; ++c) p->nhuge += (int64_t)h_out.class_count[c];
+    for (int c = degree_class(kShortRowLen); c < kEmptyClass; ++c) p->nshort += (int64_t)h_out.class_count[c];
+    if (p->long_thresh < kShortRowLen) p->nshort = 0;  // (such rows sit in the head region then)
     if (p->nhuge > 0) {
         GNNAGG_HIP(enable_long_rows_lds());
         GNNAGG_HIP(hipStreamCreateWithFlags(&p->side, hipStreamNonBlocking));
@@ -485,11 +521,28 @@ extern "C" int gnnagg_plan_info(const gnnagg_plan *plan, int64_t *info) {
     info[5] = plan->nempty;
     info[6] = plan->max_deg;
     info[7] = plan->rows_per_group;
+    info[8] = plan->nshort;
+    info[9] = plan->short_rows_per_group;
+    info[10] = plan->nlong;
+    info[11] = plan->long_thresh;
     return GNNAGG_OK;
 }
 
 namespace gnnagg {
 namespace {
+
+// Marks a plan as in use for the duration of one enqueueing call (host side): a second call that arrives meanwhile
+// is refused instead of re-recording the first one's events.
+struct BusyGuard {
+    gnnagg_plan *plan;
+    bool mine;
+    explicit BusyGuard(gnnagg_plan *p) : plan(p), mine(!p->busy.exchange(true, std::memory_order_acquire)) {}
+    ~BusyGuard() {
+        if (mine) plan->busy.store(false, std::memory_order_release);
+    }
+    BusyGuard(const BusyGuard &) = delete;
+    BusyGuard &operator=(const BusyGuard &) = delete;
+};
 
 int plan_spmm(gnnagg_plan *plan, const float *value, const float *mat, int64_t ldx, float *out, int64_t ldd,
               int64_t feat, int accumulate, void *stream) {
@@ -503,10 +556,20 @@ int plan_spmm(gnnagg_plan *plan, const float *value, const float *mat, int64_t l
                    "row strides %lld / %lld must be at least the width %lld and below 2^31", (long long)ldx,
                    (long long)ldd, (long long)feat);
     hipStream_t st = static_cast<hipStream_t>(stream);
+    BusyGuard in_use(plan);
+    if (!in_use.mine)
+        return fail(GNNAGG_ERR_INVALID, "this plan is in use by another call (two calls on one plan must not overlap: "
+                                        "its events and side stream belong to one call at a time)");
 
     const int vec = pick_vec(feat, mat, out, ldx, ldd);
     // accumulate: empty rows keep their value, so they are not visited at all
     const int64_t nshort = plan->rows - plan->nlong - (accumulate ? plan->nempty : 0);
+    // the tail region: the rows of at most kShortRowLen elements and, when every row is written, the empty ones
+    const Regions regions{plan->rows_per_group, plan->short_rows_per_group,
+                          plan->nshort + (accumulate ? 0 : plan->nempty)};
+    if (plan->lanes > 0 && (int64_t)vec * plan->lanes * plan->loads < feat)
+        return fail(GNNAGG_ERR_INVALID, "the plan's launch shape (%d lanes x %d loads x %d floats) does not cover %lld features",
+                    plan->lanes, plan->loads, vec, (long long)feat);
     const bool prof = plan->profile;
     if (prof) {
         plan->profile_valid = false;
@@ -533,7 +596,7 @@ int plan_spmm(gnnagg_plan *plan, const float *value, const float *mat, int64_t l
         GNNAGG_HIP(hipEventRecord(plan->join, plan->side));
     }
     for (int64_t f_base = 0; f_base < feat;) {
-        const Shape s = pick_shape(vec, feat - f_base);
+        const Shape s = pick_shape(vec, feat - f_base, plan->lanes, plan->loads);
         SpmmArgs a{};
         a.task = plan->task;
         a.col = plan->col32;
@@ -554,7 +617,7 @@ int plan_spmm(gnnagg_plan *plan, const float *value, const float *mat, int64_t l
             a.ntasks = plan->nlong + nshort - plan->nhuge;
             a.head_tasks = plan->nlong - plan->nhuge;
             if (timed) GNNAGG_HIP(hipEventRecord(plan->ev[1], st));
-            GNNAGG_HIP((dispatch_tasks<int32_t, kRowsPlanned>(s, a, plan->rows_per_group, st)));
+            GNNAGG_HIP((dispatch_tasks<int32_t, kRowsPlanned>(s, a, regions, st)));
             if (timed) {
                 GNNAGG_HIP(hipEventRecord(plan->ev[2], st));
                 plan->profile_valid = true;
@@ -607,7 +670,9 @@ extern "C" int gnnagg_plan_spmm_packed_f32(gnnagg_plan *plan, const float *value
     a.accumulate = accumulate;
     a.ntasks = plan->rows - (accumulate ? plan->nempty : 0);
     a.head_tasks = plan->nlong;
-    GNNAGG_HIP(launch_packed(a, plan->rows_per_group, static_cast<hipStream_t>(stream)));
+    const Regions regions{plan->rows_per_group, plan->short_rows_per_group,
+                          plan->nshort + (accumulate ? 0 : plan->nempty)};
+    GNNAGG_HIP(launch_packed(a, regions, static_cast<hipStream_t>(stream)));
     return GNNAGG_OK;
 }
 
@@ -631,6 +696,8 @@ extern "C" int gnnagg_plan_spmm_quantized_f32(gnnagg_plan *plan, const float *va
                        (reinterpret_cast<uintptr_t>(params) & 7) == 0,
                    "quantised SpMM needs a 16-byte aligned output, 4-byte aligned bytes and 8-byte aligned parameters");
     hipStream_t st = static_cast<hipStream_t>(stream);
+    const Regions regions{plan->rows_per_group, plan->short_rows_per_group,
+                          plan->nshort + (accumulate ? 0 : plan->nempty)};
     for (int64_t f_base = 0; f_base < feat;) {
         const Shape s = pick_shape(4, feat - f_base);
         SpmmArgs a{};
@@ -648,7 +715,7 @@ extern "C" int gnnagg_plan_spmm_quantized_f32(gnnagg_plan *plan, const float *va
         a.accumulate = accumulate;
         a.ntasks = plan->rows - (accumulate ? plan->nempty : 0);
         a.head_tasks = plan->nlong;
-        GNNAGG_HIP((dispatch_shape<4, int32_t, kRowsPlanned, kSrcQuant>(s, a, plan->rows_per_group, st)));
+        GNNAGG_HIP((dispatch_shape<4, int32_t, kRowsPlanned, kSrcQuant>(s, a, regions, st)));
         f_base += s.width();
     }
     return GNNAGG_OK;

@@ -158,9 +158,15 @@ struct SpmmArgs {
     int ldx, ldd;             // row strides of x and dst in floats; 0 stands for F (rows back to back)
     int f_base;               // first feature handled by this launch
     int accumulate;           // start every row from dst (1) or from 0 (0)
-    int tasks_per_block;      // tasks handled by one block past the head region
+    int tasks_per_block;      // tasks handled by one block of the middle region
     int64_t head_tasks;       // the first head_tasks tasks (the longest rows) get one lane group each
     int head_blocks;          // = ceil(head_tasks / groups per block)
+    // The tasks from tail_first on (the shortest rows: a plan orders its rows by length) are handed out
+    // tail_tasks_per_block to a block, more rows per lane group than in the middle region: what a group pays once
+    // per block (row descriptors, the first column chunk: two dependent round trips) is spread over more rows.
+    int64_t tail_first;       // first task of the tail region (== ntasks: none)
+    int mid_blocks;           // blocks of the middle region
+    int tail_tasks_per_block;
 };
 
 enum SourceKind : int {
@@ -207,9 +213,13 @@ __device__ __forceinline__ FVec<4> expand_packed(uint32_t nib, const f32x4_unali
 // the chunk held in (c_l, v_l) across the group's lanes.  For a packed source the zero
 // values are not fetched; fma(v, 0, acc) == acc, so the chain is the same (up to the sign
 // of a zero result).
-template <int UU, int VEC, int LPR, int NCH, int SRC, typename IdxT>
+// `valid` < UU (the tail of a row's last chunk): all UU gathers are still issued at once -- one memory round trip
+// instead of a cascade of ever shorter dependent ones; the lanes past the row's end hold column 0 with value 0, so the
+// surplus gathers read row 0 of x (a valid, hot address) -- and only the first `valid` results enter the chain (selected,
+// not multiplied by zero: row 0 of x may hold anything).
+template <int UU, int VEC, int LPR, int NCH, int SRC, typename IdxT, bool TAIL = false>
 __device__ __forceinline__ void gather_fma(FVec<VEC> (&acc)[NCH], IdxT c_l, float v_l, int j, const SpmmArgs &a,
-                                           const int (&foff)[NCH]) {
+                                           const int (&foff)[NCH], int valid = UU) {
     const float *__restrict__ x = a.x;
     const int F = a.feat;
     const int ldx = a.ldx ? a.ldx : F;
@@ -284,8 +294,15 @@ __device__ __forceinline__ void gather_fma(FVec<VEC> (&acc)[NCH], IdxT c_l, floa
     }
 #pragma unroll
     for (int u = 0; u < UU; ++u) {
+        if constexpr (TAIL) {
+            if (u < valid) {
 #pragma unroll
-        for (int k = 0; k < NCH; ++k) acc[k].fma(vv[u], xv[u][k]);
+                for (int k = 0; k < NCH; ++k) acc[k].fma(vv[u], xv[u][k]);
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < NCH; ++k) acc[k].fma(vv[u], xv[u][k]);
+        }
     }
 }
 
@@ -336,9 +353,13 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
         t0 = (int64_t)blockIdx.x * GPB;
         t1 = t0 + GPB;
         if (t1 > a.head_tasks) t1 = a.head_tasks;
-    } else {
+    } else if ((int)blockIdx.x < a.head_blocks + a.mid_blocks) {
         t0 = a.head_tasks + (int64_t)((int)blockIdx.x - a.head_blocks) * a.tasks_per_block;
         t1 = t0 + a.tasks_per_block;
+        if (t1 > a.tail_first) t1 = a.tail_first;
+    } else {
+        t0 = a.tail_first + (int64_t)((int)blockIdx.x - a.head_blocks - a.mid_blocks) * a.tail_tasks_per_block;
+        t1 = t0 + a.tail_tasks_per_block;
         if (t1 > a.ntasks) t1 = a.ntasks;
     }
     // this group's tasks: t0 + group + i * GPB, i < ntask  (ntask <= kMaxRowsPerGroup <= LPR)
@@ -414,18 +435,22 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
             nv = __builtin_nontemporal_load(val + nbase + lig);
         }
 
-        // full blocks of U gathers, then a halving cascade for what is left, so that a
-        // chunk of cnt elements costs at most cnt/U + log2(U) dependent round trips
+        // full blocks of U gathers, then ONE more round for what is left (the smallest power of two of gathers
+        // that covers it, the surplus ones masked): a chunk of cnt elements costs ceil(cnt / U) dependent round trips
         int j = 0;
         for (; j + U <= cnt; j += U) gather_fma<U, VEC, LPR, NCH, SRC>(acc, c_l, v_l, j, a, foff);
-        if constexpr (U > 4) {
-            if (j + 4 <= cnt) { gather_fma<4, VEC, LPR, NCH, SRC>(acc, c_l, v_l, j, a, foff); j += 4; }
-        }
-        if constexpr (U > 2) {
-            if (j + 2 <= cnt) { gather_fma<2, VEC, LPR, NCH, SRC>(acc, c_l, v_l, j, a, foff); j += 2; }
-        }
-        if constexpr (U > 1) {
-            if (j + 1 <= cnt) { gather_fma<1, VEC, LPR, NCH, SRC>(acc, c_l, v_l, j, a, foff); j += 1; }
+        const int rem = cnt - j;
+        if (rem > 0) {
+            if constexpr (U > 4) {
+                if (rem > 4) gather_fma<8, VEC, LPR, NCH, SRC, IdxT, true>(acc, c_l, v_l, j, a, foff, rem);
+            }
+            if constexpr (U > 2) {
+                if (rem > 2 && rem <= 4) gather_fma<4, VEC, LPR, NCH, SRC, IdxT, true>(acc, c_l, v_l, j, a, foff, rem);
+            }
+            if constexpr (U > 1) {
+                if (rem == 2) gather_fma<2, VEC, LPR, NCH, SRC, IdxT, false>(acc, c_l, v_l, j, a, foff);
+            }
+            if (rem == 1) gather_fma<1, VEC, LPR, NCH, SRC, IdxT, false>(acc, c_l, v_l, j, a, foff);
         }
 
         if (row_done) {

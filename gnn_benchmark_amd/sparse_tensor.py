@@ -20,25 +20,36 @@ import torch
 from . import _lib
 
 
+# Tuning values new plans are created with: a dict with any of the keys of ``_lib.PlanOptions`` (long_row_threshold,
+# block_row_threshold, rows_per_group, short_rows_per_group, lanes_per_row, loads_per_lane); None or a missing key
+# = the library's default.  Results never depend on them.  Tests and sweeps set this; ``SpmmPlan(options=...)``
+# overrides it for one plan.
+PLAN_OPTIONS: Optional[dict] = None
+
+
 class SpmmPlan:
     """Cached GPU schedule of one CSR matrix (the counterpart of the per-matrix CPU work
     range the reference caches, model/ops/spmm_kernel.py:48-57)."""
 
-    def __init__(self, rowptr: torch.Tensor, col: torch.Tensor, rows: int, cols: int):
+    def __init__(self, rowptr: torch.Tensor, col: torch.Tensor, rows: int, cols: int, options: Optional[dict] = None):
         if not rowptr.is_cuda:
             raise RuntimeError("SpMM plans exist only for matrices on a GPU (HIP) device")
         self.device = rowptr.device
         self.rows, self.cols, self.nnz = int(rows), int(cols), int(col.numel())
         handle = ctypes.c_void_p()
+        options = PLAN_OPTIONS if options is None else options
+        opt = _lib.PlanOptions(**options) if options else None
         with torch.cuda.device(self.device):
-            _lib.check(_lib.lib().gnnagg_plan_create(_lib.ptr(rowptr), _lib.ptr(col), self.rows, self.cols, self.nnz,
-                                                     _lib.current_stream(self.device), ctypes.byref(handle)))
+            _lib.check(_lib.lib().gnnagg_plan_create_ex(_lib.ptr(rowptr), _lib.ptr(col), self.rows, self.cols, self.nnz,
+                                                        None if opt is None else ctypes.byref(opt),
+                                                        _lib.current_stream(self.device), ctypes.byref(handle)))
         self._handle = handle
 
     def info(self) -> dict:
-        buf = (ctypes.c_int64 * 8)()
+        buf = (ctypes.c_int64 * 12)()
         _lib.check(_lib.lib().gnnagg_plan_info(self._handle, buf))
-        keys = ("rows", "cols", "nnz", "huge_rows", "huge_thresh", "empty_rows", "max_row_len", "rows_per_group")
+        keys = ("rows", "cols", "nnz", "huge_rows", "huge_thresh", "empty_rows", "max_row_len", "rows_per_group",
+                "short_rows", "short_rows_per_group", "long_rows", "long_thresh")
         return dict(zip(keys, [int(x) for x in buf]))
 
     def profile(self, enable: bool = True) -> None:

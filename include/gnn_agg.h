@@ -77,6 +77,30 @@ typedef struct gnnagg_plan gnnagg_plan;
 int gnnagg_plan_create(const int64_t *rowptr, const int64_t *col, int64_t rows, int64_t cols, int64_t nnz,
                        void *stream, gnnagg_plan **plan_out);
 
+/* The same with the schedule's tuning values given explicitly (NULL, or a field left 0: the default).
+ *   long_row_threshold   rows longer than this get a lane group of their own at the head of the launch (256)
+ *   block_row_threshold  rows longer than this run in the block-per-row kernel (max(2048, nnz / 4096))
+ *   rows_per_group       rows a lane group walks, one after the other, in the middle of the launch (2; at most 16)
+ *   short_rows_per_group the same for the rows of at most 8 elements at the end of the launch (2; at most 16)
+ *   lanes_per_row, loads_per_lane  launch shape of the row kernel instead of the one chosen from the feature
+ *                        width: lanes x loads x (4, 2 or 1 floats, by alignment) must cover the width, else the
+ *                        product calls return GNNAGG_ERR_INVALID.  Instances: 16x1, 16x2, 16x3, 32x1, 32x2, 64x1,
+ *                        64x2, 64x3, 64x4, 64x5, 64x6, 64x8.
+ * Results do not depend on any of them (every row stays one FMA chain); they only move time.  No counterpart
+ * in the reference (its cached split depends on the thread count alone, model/ops/spmm_kernel.py:48-57). */
+typedef struct gnnagg_plan_options {
+    int32_t long_row_threshold;
+    int32_t block_row_threshold;
+    int32_t rows_per_group;
+    int32_t short_rows_per_group;
+    int32_t lanes_per_row;
+    int32_t loads_per_lane;
+    int32_t reserved[2]; /* must be 0 */
+} gnnagg_plan_options;
+
+int gnnagg_plan_create_ex(const int64_t *rowptr, const int64_t *col, int64_t rows, int64_t cols, int64_t nnz,
+                          const gnnagg_plan_options *options, void *stream, gnnagg_plan **plan_out);
+
 /* Frees a plan (synchronises the device; NULL is accepted). */
 int gnnagg_plan_destroy(gnnagg_plan *plan);
 
@@ -87,8 +111,9 @@ int gnnagg_plan_destroy(gnnagg_plan *plan);
  * model/layers/aggregator.py:67-70, :167-170).  Allocates nothing and does not
  * synchronise the host.  A plan owns a few events (and, when it holds very long rows, a
  * side stream joined back into `stream` before the call returns), so two calls on the
- * SAME plan must not overlap: issue them on one stream, or order them yourself.  Calls
- * on different plans are independent. */
+ * SAME plan must not overlap: issue them on one stream, or order them yourself (a call that
+ * arrives while another thread is still inside a call on the same plan returns
+ * GNNAGG_ERR_INVALID).  Calls on different plans are independent. */
 int gnnagg_plan_spmm_f32(gnnagg_plan *plan, const float *value, const float *mat, float *out, int64_t feat,
                          int accumulate, void *stream);
 
@@ -101,10 +126,11 @@ int gnnagg_plan_spmm_f32(gnnagg_plan *plan, const float *value, const float *mat
 int gnnagg_plan_spmm_strided_f32(gnnagg_plan *plan, const float *value, const float *mat, int64_t mat_stride,
                                  float *out, int64_t out_stride, int64_t feat, int accumulate, void *stream);
 
-/* Host-side description of a plan, info[0..7] (host pointer):
+/* Host-side description of a plan, info[0..11] (host pointer):
  * rows, cols, nnz, rows handled by the block-per-row kernel (longer than the next
  * entry), that length threshold, rows with no stored element, largest row length, rows
- * handled per lane group. */
+ * handled per lane group, rows of at most 8 elements, rows per lane group for those, rows
+ * with a lane group of their own (longer than the next entry), that length threshold. */
 int gnnagg_plan_info(const gnnagg_plan *plan, int64_t *info);
 
 /* Kernel timing of a plan, for benchmarks.  After gnnagg_plan_profile(plan, 1) every
@@ -395,6 +421,24 @@ int gnnagg_dequantize_mixed_f32(const uint8_t *data, const int64_t *feat_range, 
  * allocate nothing, no host sync. */
 int gnnagg_f32_to_bf16(const float *x, uint16_t *y, int64_t count, void *stream);
 int gnnagg_bf16_to_f32(const uint16_t *x, float *y, int64_t count, void *stream);
+
+/* ---------------------------------------------------------------------------------
+ * Memory-system probes: plain kernels with the access mixes of the aggregation path and nothing else, for
+ * benchmarks that want the machine's own rate for a mix next to a product kernel's (a copy or a read stream is the
+ * usual yardstick; row gathers mixed with row writes are what the boundary products do).  Nothing in the product
+ * path calls them; no counterpart in the reference (its `#define PROFILE` timers, spmm.cpp:12, time the operator
+ * only).  Allocate nothing, no host synchronisation.
+ *   kind 0  read `count` floats of src as a stream (dst: 4 writable bytes, never written for finite data)
+ *   kind 1  write `count` floats of dst as a stream
+ *   kind 2  copy `count` floats from src to dst
+ *   kind 3  `count` result rows, each the sum of `per_row` rows of src gathered through index[count * per_row]
+ *           (int32 row numbers of src); the results are dropped: reads only
+ *   kind 4  the same, every result row written to dst[count, row_floats]
+ *   kind 5  the same, every result row added onto the row dst holds: one row read and one written per result
+ * row_floats (kinds 3-5): 64, 128 or 256; src and dst 16-byte aligned; count a multiple of 4 for kinds 0-2.
+ * ------------------------------------------------------------------------------- */
+int gnnagg_memory_probe(int kind, const float *src, const int32_t *index, float *dst, int64_t count,
+                        int64_t row_floats, int64_t per_row, void *stream);
 
 #ifdef __cplusplus
 }

@@ -9,6 +9,8 @@ import numpy as np
 import pytest
 import torch
 
+from gnn_benchmark_amd import sparse_tensor
+
 from gnn_benchmark_amd import SPMM_backward, SPMM_forward, gcn, sage
 from gnn_benchmark_amd import computation_ops as ops
 from gnn_benchmark_amd.aggregator import _convert, _gather_rows
@@ -19,7 +21,7 @@ pytestmark = pytest.mark.gpu
 
 
 def test_entry_points_replay_from_a_hip_graph(monkeypatch):
-    monkeypatch.setenv("GNNAGG_HUGE_THRESH", "2048")
+    monkeypatch.setattr(sparse_tensor, "PLAN_OPTIONS", {"block_row_threshold": 2048})
     n, feat, bits = 3000, 64, 2
     rowptr, col, val = skewed_csr(n, n, seed=3, heavy_rows=(5000, 900))
     src = SparseTensor(rowptr=dev(rowptr), col=dev(col), value=dev(val), sparse_sizes=(n, n))

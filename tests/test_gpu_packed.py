@@ -7,6 +7,8 @@ import numpy as np
 import pytest
 import torch
 
+from gnn_benchmark_amd import sparse_tensor
+
 from gnn_benchmark_amd import SPMM_forward, gcn, packed, synthetic
 from gnn_benchmark_amd.sparse_tensor import SparseTensor
 from tests.gpu_util import skewed_csr
@@ -83,7 +85,7 @@ def test_packed_spmm_equals_dense_spmm(feat, accumulate, low_block_row_threshold
 def low_block_row_threshold(monkeypatch):
     # rows above 1000 elements would go to the block-per-row kernel in the dense path; the packed path
     # keeps them in the lane-group kernel, and both must agree
-    monkeypatch.setenv("GNNAGG_HUGE_THRESH", "1000")
+    monkeypatch.setattr(sparse_tensor, "PLAN_OPTIONS", {"block_row_threshold": 1000})
 
 
 @pytest.mark.parametrize("feat", [32, 64, 128, 256])

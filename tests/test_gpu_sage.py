@@ -17,7 +17,7 @@ import pytest
 import torch
 import torch.nn.functional as F
 
-from gnn_benchmark_amd import gcn, sage, synthetic
+from gnn_benchmark_amd import gcn, sage, sparse_tensor, synthetic
 from gnn_benchmark_amd.data_manager import CommBuffer, CommSplits, DistributedGraphForPre
 from gnn_benchmark_amd.sparse_tensor import SparseTensor
 from gnn_benchmark_amd.spmm_kernel import SPMM_backward, SPMM_forward
@@ -31,7 +31,7 @@ pytestmark = pytest.mark.gpu
 @pytest.mark.parametrize("with_block_rows", [False, True])
 def test_spmm_on_column_blocks_equals_contiguous(feat, with_block_rows, monkeypatch):
     if with_block_rows:
-        monkeypatch.setenv("GNNAGG_HUGE_THRESH", "1024")
+        monkeypatch.setattr(sparse_tensor, "PLAN_OPTIONS", {"block_row_threshold": 1024})
     rowptr, col, val = skewed_csr(900, 900, seed=feat, heavy_rows=(2000, 1500, 300))
     src = SparseTensor(rowptr=dev(rowptr), col=dev(col), value=dev(val), sparse_sizes=(900, 900))
     assert (src.get_plan().info()["huge_rows"] > 0) == with_block_rows

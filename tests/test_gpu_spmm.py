@@ -7,6 +7,8 @@ import numpy as np
 import pytest
 import torch
 
+from gnn_benchmark_amd import sparse_tensor
+
 from gnn_benchmark_amd import SPMM_backward, SPMM_forward, SparseTensor, computation_ops
 from gnn_benchmark_amd.sparse_tensor import SpmmPlan
 from oracle import index_maps as om
@@ -18,10 +20,10 @@ pytestmark = pytest.mark.gpu
 
 @pytest.fixture
 def low_block_row_threshold(monkeypatch):
-    """Plans read this when they are created: rows longer than 1024 elements then go to
+    """Plans are created with these options: rows longer than 1024 elements then go to
     the block-per-row kernel, which by default only takes rows that would outlast the
     whole launch (about nnz / 4096 elements, at least 2048)."""
-    monkeypatch.setenv("GNNAGG_HUGE_THRESH", "1024")
+    monkeypatch.setattr(sparse_tensor, "PLAN_OPTIONS", {"block_row_threshold": 1024})
 
 EMPTY_I32 = torch.empty(0, dtype=torch.int32)
 
@@ -110,6 +112,79 @@ def test_block_per_row_kernel_chunk_edges(feat, low_block_row_threshold):
         plan.spmm(dev(val), dev(x), out, accumulate=accumulate)
         want = _oracle(rowptr, col, val, x, out0 if accumulate else None)
         assert np.array_equal(out.cpu().numpy(), want), (feat, accumulate)
+
+
+def _row_lengths_around_the_unroll():
+    """A matrix whose rows have every length 0 .. 40 (and a few longer ones), several rows of each: the masked last
+    round of a row (1 .. 7 surplus gathers) and the tail region of short rows are all exercised."""
+    rng = np.random.default_rng(123)
+    deg = np.concatenate([np.repeat(np.arange(0, 41), 9), [300, 77, 65, 64, 63, 33, 1000]]).astype(np.int64)
+    rng.shuffle(deg)
+    rowptr = np.concatenate(([0], np.cumsum(deg))).astype(np.int64)
+    cols = 500
+    col = rng.integers(0, cols, rowptr[-1]).astype(np.int64)
+    val = rng.standard_normal(rowptr[-1]).astype(np.float32)
+    return rowptr, col, val, deg.shape[0], cols
+
+
+@pytest.mark.parametrize("feat", [3, 16, 40, 47, 64, 100, 128, 172, 256, 602])
+@pytest.mark.parametrize("accumulate", [True, False])
+def test_every_row_length_around_the_gather_unroll(feat, accumulate):
+    """Row 0 of the dense operand is NaN / inf: the surplus gathers of a row's last round read it (lanes past the
+    row's end hold column 0) and must not leak into any row that does not reference column 0."""
+    rowptr, col, val, rows, cols = _row_lengths_around_the_unroll()
+    col = np.where(col == 0, 1, col)  # no row references column 0 ...
+    rng = np.random.default_rng(feat)
+    x = rng.standard_normal((cols, feat)).astype(np.float32)
+    x[0, ::2] = np.nan  # ... so nothing of this may show
+    x[0, 1::2] = np.inf
+    out0 = rng.standard_normal((rows, feat)).astype(np.float32)
+    plan = SpmmPlan(dev(rowptr), dev(col), rows, cols)
+    info = plan.info()
+    assert info["short_rows"] == int(((np.diff(rowptr) >= 1) & (np.diff(rowptr) <= 8)).sum())
+    out = dev(out0)
+    plan.spmm(dev(val), dev(x), out, accumulate=accumulate)
+    want = _oracle(rowptr, col, val, x, out0 if accumulate else None)
+    assert np.isfinite(want).all()
+    assert np.array_equal(out.cpu().numpy(), want)
+    direct = dev(out0 if accumulate else np.zeros_like(out0))
+    computation_ops.spmm(dev(rowptr), dev(col), dev(val), dev(x), direct, rows, EMPTY_I32, EMPTY_I32)
+    assert np.array_equal(direct.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("options", [
+    {"rows_per_group": 1, "short_rows_per_group": 16}, {"rows_per_group": 16, "short_rows_per_group": 1},
+    {"rows_per_group": 3, "short_rows_per_group": 3}, {"long_row_threshold": 4}, {"long_row_threshold": 20},
+    {"long_row_threshold": 100000, "block_row_threshold": 100000}, {"block_row_threshold": 50},
+    {"lanes_per_row": 16, "loads_per_lane": 2}, {"lanes_per_row": 16, "loads_per_lane": 3},
+    {"lanes_per_row": 32, "loads_per_lane": 2}, {"lanes_per_row": 64, "loads_per_lane": 8}])
+@pytest.mark.parametrize("feat", [12, 47, 100, 128])
+def test_plan_options_move_time_not_results(options, feat):
+    rowptr, col, val, rows, cols = _row_lengths_around_the_unroll()
+    rng = np.random.default_rng(feat)
+    x = rng.standard_normal((cols, feat)).astype(np.float32)
+    want = _oracle(rowptr, col, val, x)
+    plan = SpmmPlan(dev(rowptr), dev(col), rows, cols, options=options)
+    info = plan.info()
+    for key in ("rows_per_group", "short_rows_per_group"):
+        if key in options:
+            assert info[key] == options[key]
+    out = torch.full((rows, feat), float("nan"), device="cuda")
+    vec = 4 if feat % 4 == 0 else (2 if feat % 2 == 0 else 1)
+    if "lanes_per_row" in options and options["lanes_per_row"] * options["loads_per_lane"] * vec < feat:
+        with pytest.raises(RuntimeError, match="does not cover"):
+            plan.spmm(dev(val), dev(x), out, accumulate=False)
+        return
+    plan.spmm(dev(val), dev(x), out, accumulate=False)
+    assert np.array_equal(out.cpu().numpy(), want)
+
+
+def test_plan_options_are_checked():
+    rowptr, col, val, rows, cols = _row_lengths_around_the_unroll()
+    for bad in ({"rows_per_group": 17}, {"short_rows_per_group": -1}, {"lanes_per_row": 24, "loads_per_lane": 1},
+                {"lanes_per_row": 16}, {"long_row_threshold": -5}):
+        with pytest.raises(RuntimeError, match="plan options"):
+            SpmmPlan(dev(rowptr), dev(col), rows, cols, options=bad)
 
 
 def test_default_threshold_keeps_moderate_rows_in_the_lane_group_kernel():
@@ -373,7 +448,7 @@ def test_plan_spmm_can_be_captured_in_a_hip_graph(monkeypatch, with_block_rows):
     """The plan call allocates nothing and never synchronises the host, so it can be
     recorded into a graph; every replay (with fresh operand contents) must equal eager."""
     if with_block_rows:
-        monkeypatch.setenv("GNNAGG_HUGE_THRESH", "1024")
+        monkeypatch.setattr(sparse_tensor, "PLAN_OPTIONS", {"block_row_threshold": 1024})
     rowptr, col, val = skewed_csr(900, 450, seed=41)
     plan = SpmmPlan(dev(rowptr), dev(col), 900, 450)
     assert (plan.info()["huge_rows"] > 0) == with_block_rows
