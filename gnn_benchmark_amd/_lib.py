@@ -29,6 +29,7 @@ EXPORTS = (
     "gnnagg_csr_transpose",
     "gnnagg_coo_to_csr",
     "gnnagg_gather_rows_f32",
+    "gnnagg_check_index",
     "gnnagg_bias_relu_dropout_f32",
     "gnnagg_relu_dropout_backward_blocks",
     "gnnagg_relu_dropout_backward_f32",
@@ -127,7 +128,9 @@ def lib() -> ctypes.CDLL:
     L.gnnagg_coo_to_csr.restype = i32
     L.gnnagg_coo_to_csr.argtypes = [vp, vp, vp, i64, i64, i64, vp, vp, vp, vp]
     L.gnnagg_gather_rows_f32.restype = i32
-    L.gnnagg_gather_rows_f32.argtypes = [vp, vp, vp, i64, i64, vp]
+    L.gnnagg_gather_rows_f32.argtypes = [vp, i64, vp, vp, i64, i64, vp]
+    L.gnnagg_check_index.restype = i32
+    L.gnnagg_check_index.argtypes = [vp, i32, i64, i32, i64, vp]
     L.gnnagg_bias_relu_dropout_f32.restype = i32
     L.gnnagg_bias_relu_dropout_f32.argtypes = [vp, vp, vp, vp, ctypes.c_float, vp, i64, i64, vp]
     L.gnnagg_relu_dropout_backward_f32.restype = i32
@@ -137,13 +140,13 @@ def lib() -> ctypes.CDLL:
     L.gnnagg_wgrad_workspace_bytes.restype = i64
     L.gnnagg_wgrad_workspace_bytes.argtypes = [i64, i64, i64]
     L.gnnagg_wgrad_f32.restype = i32
-    L.gnnagg_wgrad_f32.argtypes = [vp, vp, vp, vp, i64, i64, i64, vp]
+    L.gnnagg_wgrad_f32.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, vp]
     L.gnnagg_f32_to_bf16.restype = i32
     L.gnnagg_f32_to_bf16.argtypes = [vp, vp, i64, vp]
     L.gnnagg_bf16_to_f32.restype = i32
     L.gnnagg_bf16_to_f32.argtypes = [vp, vp, i64, vp]
     L.gnnagg_wgrad_strided_f32.restype = i32
-    L.gnnagg_wgrad_strided_f32.argtypes = [vp, i64, vp, i64, vp, vp, i64, i64, i64, vp]
+    L.gnnagg_wgrad_strided_f32.argtypes = [vp, i64, vp, i64, vp, vp, i64, i64, i64, i64, vp]
     L.gnnagg_wgrad_noalloc_f32.restype = i32
     L.gnnagg_wgrad_noalloc_f32.argtypes = [vp, vp, vp, i64, i64, i64, vp]
     L.gnnagg_linear_shape_supported.restype = i32
@@ -164,14 +167,14 @@ def lib() -> ctypes.CDLL:
     L.gnnagg_wgrad_relu_dropout_backward_workspace_bytes.argtypes = [i64, i64, i64]
     L.gnnagg_wgrad_relu_dropout_backward_f32.restype = i32
     L.gnnagg_wgrad_relu_dropout_backward_f32.argtypes = [vp, i64, vp, i64, vp, i64, vp, ctypes.c_float, vp, vp, vp, vp,
-                                                         i64, i64, i64, vp]
+                                                         i64, i64, i64, i64, vp]
     L.gnnagg_wgrad_relu_dropout_backward_bf16_f32.restype = i32
     L.gnnagg_wgrad_relu_dropout_backward_bf16_f32.argtypes = L.gnnagg_wgrad_relu_dropout_backward_f32.argtypes
     L.gnnagg_wgrad_relu_dropout_backward_bf16x3_f32.restype = i32
     L.gnnagg_wgrad_relu_dropout_backward_bf16x3_f32.argtypes = L.gnnagg_wgrad_relu_dropout_backward_f32.argtypes
     L.gnnagg_wgrad_relu_dropout_backward_from_header_f32.restype = i32
     L.gnnagg_wgrad_relu_dropout_backward_from_header_f32.argtypes = [vp, i64, vp, i64, vp, vp, ctypes.c_float, vp, vp, vp,
-                                                                     vp, i64, i64, i64, i32, vp]
+                                                                     vp, i64, i64, i64, i64, i32, vp]
     L.gnnagg_dropout_layernorm_relu_blocks.restype = i32
     L.gnnagg_dropout_layernorm_relu_blocks.argtypes = [i64, i64]
     L.gnnagg_dropout_layernorm_relu_f32.restype = i32
@@ -212,6 +215,38 @@ def check(rc: int) -> None:
 def ptr(t):
     """Device address of a tensor (None -> NULL)."""
     return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+_CHECKED_INDEX = {}
+
+
+def check_index(index, bound: int, shift: int = 0, what: str = "index") -> None:
+    """Raise unless every ``index[i] >> shift`` lies in [0, bound).  The values are looked at on the device once per
+    (tensor, bound, shift) -- one stream synchronisation -- and the verdict is remembered for as long as the same
+    tensor, unchanged, comes back (an in-place change bumps ``_version``; a new tensor at a freed one's address fails
+    the identity check).  The counterpart of the bounds checks torch's indexing ops make in the reference
+    (``torch.index_select`` raises on a bad index, self_benchmark/a64fx/model/layers/aggregator.py:51)."""
+    import weakref
+
+    n = int(index.numel())
+    if n == 0:
+        return
+    key = (index.data_ptr(), index._version, n, index.dtype, str(index.device), int(bound), int(shift))
+    hit = _CHECKED_INDEX.get(key)
+    if hit is not None and hit() is index:
+        return
+    if not index.is_contiguous():
+        raise RuntimeError(f"Input mismatch: {what} must be contiguous")
+    import torch
+
+    with torch.cuda.device(index.device):
+        rc = lib().gnnagg_check_index(ptr(index), index.element_size(), n, int(shift), int(bound),
+                                      current_stream(index.device))
+    if rc != OK:
+        raise RuntimeError(f"Input mismatch: {what}: " + lib().gnnagg_last_error().decode("utf-8", "replace"))
+    if len(_CHECKED_INDEX) >= 64:
+        _CHECKED_INDEX.clear()
+    _CHECKED_INDEX[key] = weakref.ref(index)
 
 
 def current_stream(device):

@@ -63,9 +63,11 @@ def _gather_rows(src: torch.Tensor, index: torch.Tensor, out: torch.Tensor) -> N
     if out.size(0) != index.numel() or out.size(1) != src.size(1) or not out.is_contiguous():
         raise RuntimeError("Input mismatch: gather output shape")
     src = src.contiguous()
+    # torch.index_select raises on an index outside the source; here the list is looked at once (cached per tensor)
+    _lib.check_index(index, src.size(0), what="boundary row list (idx_nodes_send_to_others)")
     with torch.cuda.device(src.device):
-        _lib.check(_lib.lib().gnnagg_gather_rows_f32(_lib.ptr(src), _lib.ptr(index), _lib.ptr(out), index.numel(),
-                                                     src.size(1), _lib.current_stream(src.device)))
+        _lib.check(_lib.lib().gnnagg_gather_rows_f32(_lib.ptr(src), src.size(0), _lib.ptr(index), _lib.ptr(out),
+                                                     index.numel(), src.size(1), _lib.current_stream(src.device)))
 
 
 def _check_bits(num_bits: int) -> None:

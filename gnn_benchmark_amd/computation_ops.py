@@ -65,6 +65,9 @@ def spmm(rowptr: torch.Tensor, col: torch.Tensor, value: Optional[torch.Tensor],
     rowptr = rowptr.contiguous()
     col = col.contiguous()
     value = value.contiguous()
+    # the reference reads mat[col[e]] unchecked (spmm.cpp:38-39); a bad column here would be a GPU memory fault, so
+    # the column array is range-checked on the device the first time it is seen (remembered per tensor)
+    _lib.check_index(col, mat.size(0), what="col")
     with torch.cuda.device(dev):
         _lib.check(_lib.lib().gnnagg_spmm_csr_f32(_lib.ptr(rowptr), _lib.ptr(col), _lib.ptr(value), _lib.ptr(mat),
                                                   _lib.ptr(out), sparse_rows, mat.size(1), _lib.current_stream(dev)))
@@ -146,8 +149,18 @@ def dequantize_tensor_for_all_procs(input: torch.Tensor, output: torch.Tensor, d
             num_procs, rows, packed_rows, output.size(1), bits, _lib.current_stream(dev)))
 
 
+_ONE_SEGMENT = {}
+
+
 def _one_segment(rows: int) -> torch.Tensor:
-    return torch.tensor([0, rows], dtype=torch.int32)
+    """The [0, rows] work range of a buffer that is one segment; one tensor per height, so that the device copies
+    derived from it (``_packed_range``) are found again on the next call."""
+    hit = _ONE_SEGMENT.get(rows)
+    if hit is None:
+        if len(_ONE_SEGMENT) >= 16:
+            _ONE_SEGMENT.clear()
+        hit = _ONE_SEGMENT[rows] = torch.tensor([0, rows], dtype=torch.int32)
+    return hit
 
 
 def quantize_tensor(input: torch.Tensor, output: torch.Tensor, quantized_params: torch.Tensor, bits: int) -> None:

@@ -80,7 +80,7 @@ __global__ __launch_bounds__(256) void pack_transposed_keys_kernel(const int64_t
 // anything is stored.  Source rows come through normal loads (a boundary row usually goes to
 // several peers, so it is asked for again soon); the result is written once, with streaming stores.
 template <int VEC, int G>
-__global__ __launch_bounds__(256) void gather_rows_kernel(const float *__restrict__ src,
+__global__ __launch_bounds__(256) void gather_rows_kernel(const float *__restrict__ src, int64_t src_rows,
                                                           const int64_t *__restrict__ index,
                                                           float *__restrict__ out, int64_t n_index, int feat_vec) {
     typedef float vec_t __attribute__((ext_vector_type(VEC)));
@@ -92,12 +92,14 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const float *__restric
     for (int64_t base = ((int64_t)blockIdx.x * kGroups + group) * kRows; base < n_index; base += step) {
         const vec_t *s[kRows];
         vec_t *d[kRows];
-        bool ok[kRows];
+        bool ok[kRows], inside[kRows];
 #pragma unroll
         for (int u = 0; u < kRows; ++u) {
             ok[u] = base + u < n_index;
-            const size_t r = ok[u] ? (size_t)__builtin_nontemporal_load(index + base + u) : 0;
-            s[u] = reinterpret_cast<const vec_t *>(src) + r * (size_t)feat_vec;
+            const int64_t r = ok[u] ? __builtin_nontemporal_load(index + base + u) : 0;
+            // an index outside the source is never dereferenced: row 0 is read in its place and NaN is stored
+            inside[u] = (uint64_t)r < (uint64_t)src_rows;
+            s[u] = reinterpret_cast<const vec_t *>(src) + (inside[u] ? (size_t)r : 0) * (size_t)feat_vec;
             d[u] = reinterpret_cast<vec_t *>(out) + (size_t)(base + u) * (size_t)feat_vec;
         }
         for (int f = l; f < feat_vec; f += G) {
@@ -107,23 +109,36 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const float *__restric
                 if (ok[u]) v[u] = s[u][f];
 #pragma unroll
             for (int u = 0; u < kRows; ++u)
-                if (ok[u]) __builtin_nontemporal_store(v[u], d[u] + f);
+                if (ok[u]) __builtin_nontemporal_store(inside[u] ? v[u] : v[u] * __builtin_nanf(""), d[u] + f);
         }
     }
 }
 
+// any (index[i] >> shift) outside [0, bound): the lowest such position found by a block goes to *first_bad
+template <typename T>
+__global__ __launch_bounds__(256) void check_index_kernel(const T *__restrict__ index, int64_t count, int shift,
+                                                          int64_t bound, unsigned long long *__restrict__ first_bad) {
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    unsigned long long bad = ~0ull;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < count; i += stride) {
+        const int64_t v = (int64_t)index[i] >> shift;
+        if ((v < 0 || v >= bound) && (unsigned long long)i < bad) bad = (unsigned long long)i;
+    }
+    if (bad != ~0ull) atomicMin(first_bad, bad);
+}
+
 template <int VEC>
-hipError_t launch_gather_rows(const float *src, const int64_t *index, float *out, int64_t n_index, int feat_vec,
-                              hipStream_t st) {
+hipError_t launch_gather_rows(const float *src, int64_t src_rows, const int64_t *index, float *out, int64_t n_index,
+                              int feat_vec, hipStream_t st) {
     int g = 8;
     while (g < 64 && g < feat_vec) g *= 2;
     const int64_t rows_per_block = (256 / g) * 4;
     const int64_t need = (n_index + rows_per_block - 1) / rows_per_block;
     const unsigned grid = (unsigned)(need < 256 * 32 ? need : 256 * 32);
-    if (g == 8) hipLaunchKernelGGL((gather_rows_kernel<VEC, 8>), dim3(grid), dim3(256), 0, st, src, index, out, n_index, feat_vec);
-    else if (g == 16) hipLaunchKernelGGL((gather_rows_kernel<VEC, 16>), dim3(grid), dim3(256), 0, st, src, index, out, n_index, feat_vec);
-    else if (g == 32) hipLaunchKernelGGL((gather_rows_kernel<VEC, 32>), dim3(grid), dim3(256), 0, st, src, index, out, n_index, feat_vec);
-    else hipLaunchKernelGGL((gather_rows_kernel<VEC, 64>), dim3(grid), dim3(256), 0, st, src, index, out, n_index, feat_vec);
+    if (g == 8) hipLaunchKernelGGL((gather_rows_kernel<VEC, 8>), dim3(grid), dim3(256), 0, st, src, src_rows, index, out, n_index, feat_vec);
+    else if (g == 16) hipLaunchKernelGGL((gather_rows_kernel<VEC, 16>), dim3(grid), dim3(256), 0, st, src, src_rows, index, out, n_index, feat_vec);
+    else if (g == 32) hipLaunchKernelGGL((gather_rows_kernel<VEC, 32>), dim3(grid), dim3(256), 0, st, src, src_rows, index, out, n_index, feat_vec);
+    else hipLaunchKernelGGL((gather_rows_kernel<VEC, 64>), dim3(grid), dim3(256), 0, st, src, src_rows, index, out, n_index, feat_vec);
     return hipGetLastError();
 }
 
@@ -244,20 +259,47 @@ extern "C" int gnnagg_csr_transpose(const int64_t *rowptr, const int64_t *col, c
     return GNNAGG_OK;
 }
 
-extern "C" int gnnagg_gather_rows_f32(const float *src, const int64_t *index, float *out, int64_t n_index, int64_t feat,
-                                      void *stream) {
-    GNNAGG_REQUIRE(n_index >= 0 && feat >= 0, "negative size");
+extern "C" int gnnagg_gather_rows_f32(const float *src, int64_t src_rows, const int64_t *index, float *out,
+                                      int64_t n_index, int64_t feat, void *stream) {
+    GNNAGG_REQUIRE(n_index >= 0 && feat >= 0 && src_rows >= 0, "negative size");
     if (n_index == 0 || feat == 0) return GNNAGG_OK;
     GNNAGG_REQUIRE(src && index && out, "null src/index/out");
+    GNNAGG_REQUIRE(src_rows > 0, "rows are asked of a source without rows");
     if (feat > (1 << 20)) return fail(GNNAGG_ERR_UNSUPPORTED, "feature width %lld above 2^20", (long long)feat);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const uintptr_t bits = reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(out);
     if (feat % 4 == 0 && bits % 16 == 0)
-        GNNAGG_HIP(launch_gather_rows<4>(src, index, out, n_index, (int)(feat / 4), st));
+        GNNAGG_HIP(launch_gather_rows<4>(src, src_rows, index, out, n_index, (int)(feat / 4), st));
     else if (feat % 2 == 0 && bits % 8 == 0)
-        GNNAGG_HIP(launch_gather_rows<2>(src, index, out, n_index, (int)(feat / 2), st));
+        GNNAGG_HIP(launch_gather_rows<2>(src, src_rows, index, out, n_index, (int)(feat / 2), st));
     else
-        GNNAGG_HIP(launch_gather_rows<1>(src, index, out, n_index, (int)feat, st));
+        GNNAGG_HIP(launch_gather_rows<1>(src, src_rows, index, out, n_index, (int)feat, st));
     GNNAGG_HIP(hipGetLastError());
+    return GNNAGG_OK;
+}
+
+extern "C" int gnnagg_check_index(const void *index, int elem_bytes, int64_t count, int shift, int64_t bound,
+                                  void *stream) {
+    GNNAGG_REQUIRE(elem_bytes == 4 || elem_bytes == 8, "index elements are 4 or 8 bytes wide (got %d)", elem_bytes);
+    GNNAGG_REQUIRE(count >= 0 && bound >= 0 && shift >= 0 && shift < 8 * elem_bytes, "bad count / bound / shift");
+    if (count == 0) return GNNAGG_OK;
+    GNNAGG_REQUIRE(index, "null index");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    DevBuf<unsigned long long> first_bad;
+    GNNAGG_HIP(first_bad.alloc(1));
+    GNNAGG_HIP(hipMemsetAsync(first_bad.p, 0xff, sizeof(unsigned long long), st));
+    const unsigned grid = (unsigned)std::min<int64_t>((count + 255) / 256, 256 * 16);
+    if (elem_bytes == 8)
+        hipLaunchKernelGGL(check_index_kernel<int64_t>, dim3(grid), dim3(256), 0, st, static_cast<const int64_t *>(index),
+                           count, shift, bound, first_bad.p);
+    else
+        hipLaunchKernelGGL(check_index_kernel<int32_t>, dim3(grid), dim3(256), 0, st, static_cast<const int32_t *>(index),
+                           count, shift, bound, first_bad.p);
+    GNNAGG_HIP(hipGetLastError());
+    unsigned long long h = ~0ull;
+    GNNAGG_HIP(hipMemcpyAsync(&h, first_bad.p, sizeof(h), hipMemcpyDeviceToHost, st));
+    GNNAGG_HIP(hipStreamSynchronize(st));
+    GNNAGG_REQUIRE(h == ~0ull, "index %llu of %lld lies outside [0, %lld)%s", h, (long long)count, (long long)bound,
+                   shift ? " (after the shift)" : "");
     return GNNAGG_OK;
 }

@@ -4,6 +4,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <mutex>
 #include <new>
 #include <type_traits>
 #include <vector>
@@ -369,6 +370,31 @@ static void plan_free(gnnagg_plan *p) {
     delete p;
 }
 
+// Plans handed to gnnagg_plan_destroy wait here until the next plan is created: freeing device memory synchronises
+// the whole device (and is illegal while a stream is being captured), which a destructor run by a garbage collector
+// in the middle of a training step must not do.  Plan creation is set-up work that synchronises anyway.
+static std::mutex retired_mutex;
+static std::vector<gnnagg_plan *> retired_plans;
+
+static void free_retired_plans(int device) {
+    std::vector<gnnagg_plan *> mine;
+    {
+        std::lock_guard<std::mutex> hold(retired_mutex);
+        for (size_t i = 0; i < retired_plans.size();) {
+            if (retired_plans[i]->device == device) {
+                mine.push_back(retired_plans[i]);
+                retired_plans[i] = retired_plans.back();
+                retired_plans.pop_back();
+            } else {
+                ++i;
+            }
+        }
+    }
+    if (mine.empty()) return;
+    (void)hipDeviceSynchronize();  // whatever still reads their arrays finishes first
+    for (gnnagg_plan *p : mine) plan_free(p);
+}
+
 extern "C" int gnnagg_plan_create(const int64_t *rowptr, const int64_t *col, int64_t rows, int64_t cols, int64_t nnz,
                                   void *stream, gnnagg_plan **plan_out) {
     return gnnagg_plan_create_ex(rowptr, col, rows, cols, nnz, nullptr, stream, plan_out);
@@ -421,6 +447,7 @@ extern "C" int gnnagg_plan_create_ex(const int64_t *rowptr, const int64_t *col, 
     p->lanes = opt.lanes_per_row;
     p->loads = opt.loads_per_lane;
     GNNAGG_HIP(hipGetDevice(&p->device));
+    free_retired_plans(p->device);
 
     // rowptr end points (host check; also forces the inputs to be ready)
     int64_t ends[2] = {0, 0};
@@ -498,16 +525,8 @@ extern "C" int gnnagg_plan_create_ex(const int64_t *rowptr, const int64_t *col, 
 
 extern "C" int gnnagg_plan_destroy(gnnagg_plan *plan) {
     if (!plan) return GNNAGG_OK;
-    // wait for the work of the plan's own device, whichever device is current
-    const int device = plan->device;
-    int current = 0;
-    GNNAGG_HIP(hipGetDevice(&current));
-    if (current != device) GNNAGG_HIP(hipSetDevice(device));
-    const hipError_t sync = hipDeviceSynchronize();
-    plan_free(plan);
-    if (current != device) (void)hipSetDevice(current);
-    if (sync != hipSuccess)
-        return fail(GNNAGG_ERR_HIP, "hipDeviceSynchronize failed while destroying a plan: %s", hipGetErrorString(sync));
+    std::lock_guard<std::mutex> hold(retired_mutex);
+    retired_plans.push_back(plan);
     return GNNAGG_OK;
 }
 

@@ -599,16 +599,16 @@ extern "C" int64_t gnnagg_wgrad_workspace_bytes(int64_t rows, int64_t fi, int64_
     return (int64_t)wgrad_blocks(rows) * fi * fo * (int64_t)sizeof(float);
 }
 
-extern "C" int gnnagg_wgrad_f32(const float *x, const float *g, float *w_grad, void *workspace, int64_t rows, int64_t fi,
-                                int64_t fo, void *stream) {
-    return gnnagg_wgrad_strided_f32(x, fi, g, fo, w_grad, workspace, rows, fi, fo, stream);
+extern "C" int gnnagg_wgrad_f32(const float *x, const float *g, float *w_grad, void *workspace, int64_t workspace_bytes,
+                                int64_t rows, int64_t fi, int64_t fo, void *stream) {
+    return gnnagg_wgrad_strided_f32(x, fi, g, fo, w_grad, workspace, workspace_bytes, rows, fi, fo, stream);
 }
 
 namespace {
 
 int run_wgrad(const float *x, int64_t x_stride, const float *g, int64_t g_stride, float *w_grad, void *workspace,
-              int64_t rows, int64_t fi, int64_t fo, void *stream, const MaskArgs *mask, float *bias_grad,
-              int form = 0) {  // 0 fp32 MFMA, 1 operands rounded to bf16, 2 three bf16 pieces per operand (both masked only)
+              int64_t workspace_bytes, int64_t rows, int64_t fi, int64_t fo, void *stream, const MaskArgs *mask,
+              float *bias_grad, int form = 0) {  // 0 fp32 MFMA, 1 operands rounded to bf16, 2 three bf16 pieces per operand (both masked only)
     GNNAGG_REQUIRE(form >= 0 && form <= 2, "product form is 0 (fp32), 1 (bf16 inputs) or 2 (bf16 x 3 pieces), got %d", form);
     GNNAGG_REQUIRE(form == 0 || mask, "the bf16 forms of the weight gradient come with the masked pass");
     const bool bf16 = form != 0;
@@ -633,6 +633,16 @@ int run_wgrad(const float *x, int64_t x_stride, const float *g, int64_t g_stride
     }
     GNNAGG_REQUIRE(x && g && workspace, "null x/g/workspace");
     const int blocks = wgrad_blocks(rows);
+    {   // the kernels write one partial result per slice (and, masked, per-thread bias sums) into the workspace
+        const int64_t need = mask ? gnnagg_wgrad_relu_dropout_backward_workspace_bytes(rows, fi, fo)
+                                  : gnnagg_wgrad_workspace_bytes(rows, fi, fo);
+        if (need <= 0)
+            return fail(GNNAGG_ERR_UNSUPPORTED, "no weight-gradient kernel for rows=%lld Fi=%lld Fo=%lld%s", (long long)rows,
+                        (long long)fi, (long long)fo, mask ? " with the masked pass (widths must be multiples of 4)" : "");
+        GNNAGG_REQUIRE(workspace_bytes >= need,
+                       "workspace of %lld bytes given, %lld needed for rows=%lld Fi=%lld Fo=%lld",
+                       (long long)workspace_bytes, (long long)need, (long long)rows, (long long)fi, (long long)fo);
+    }
     // whole chunks per block, so that only a slice's last chunk is partial
     const int64_t rpb = ((rows + blocks - 1) / blocks + kChunk - 1) / kChunk * kChunk;
     const int aligned = (fi % 4 == 0 && fo % 4 == 0 && x_stride % 4 == 0 && g_stride % 4 == 0 &&
@@ -714,9 +724,9 @@ int run_wgrad(const float *x, int64_t x_stride, const float *g, int64_t g_stride
 }  // namespace
 
 extern "C" int gnnagg_wgrad_strided_f32(const float *x, int64_t x_stride, const float *g, int64_t g_stride,
-                                        float *w_grad, void *workspace, int64_t rows, int64_t fi, int64_t fo,
-                                        void *stream) {
-    return run_wgrad(x, x_stride, g, g_stride, w_grad, workspace, rows, fi, fo, stream, nullptr, nullptr);
+                                        float *w_grad, void *workspace, int64_t workspace_bytes, int64_t rows,
+                                        int64_t fi, int64_t fo, void *stream) {
+    return run_wgrad(x, x_stride, g, g_stride, w_grad, workspace, workspace_bytes, rows, fi, fo, stream, nullptr, nullptr);
 }
 
 // ---- the entry point that allocates nothing -------------------------------------------------------------------
@@ -766,7 +776,8 @@ extern "C" int gnnagg_wgrad_noalloc_f32(const float *x, const float *g, float *w
     if (rc != GNNAGG_OK) return rc;
     // every slice writes all Fi x Fo of its partial results before the reduction reads them: nothing in the array
     // has to start at zero, whatever the previous call left there
-    return run_wgrad(x, fi, g, fo, w_grad, partial, rows, fi, fo, stream, nullptr, nullptr);
+    return run_wgrad(x, fi, g, fo, w_grad, partial, (int64_t)(kScratchFloats * sizeof(float)), rows, fi, fo, stream,
+                     nullptr, nullptr);
 }
 
 extern "C" int64_t gnnagg_wgrad_relu_dropout_backward_workspace_bytes(int64_t rows, int64_t fi, int64_t fo) {
@@ -778,42 +789,42 @@ extern "C" int64_t gnnagg_wgrad_relu_dropout_backward_workspace_bytes(int64_t ro
 extern "C" int gnnagg_wgrad_relu_dropout_backward_f32(const float *x, int64_t x_stride, const float *grad_y,
                                                       int64_t grad_stride, const float *y, int64_t y_stride,
                                                       const float *row_div, float scale, float *grad_z, float *w_grad,
-                                                      float *bias_grad, void *workspace, int64_t rows, int64_t fi,
+                                                      float *bias_grad, void *workspace, int64_t workspace_bytes, int64_t rows, int64_t fi,
                                                       int64_t fo, void *stream) {
     GNNAGG_REQUIRE(bias_grad, "null bias_grad");
     GNNAGG_REQUIRE(!y || (y_stride >= fo && y_stride < (int64_t(1) << 27)), "bad row stride of y");
     // without y the kernel reads the first row of g over and over in its place (row stride 0: a cache hit) and
     // ignores the values
     MaskArgs mk{y ? y : grad_y, row_div, grad_z, nullptr, (int)(y ? y_stride : 0), scale, y ? 0 : 1, nullptr, 0, 0};
-    return run_wgrad(x, x_stride, grad_y, grad_stride, w_grad, workspace, rows, fi, fo, stream, &mk, bias_grad);
+    return run_wgrad(x, x_stride, grad_y, grad_stride, w_grad, workspace, workspace_bytes, rows, fi, fo, stream, &mk, bias_grad);
 }
 
 extern "C" int gnnagg_wgrad_relu_dropout_backward_bf16_f32(const float *x, int64_t x_stride, const float *grad_y,
                                                            int64_t grad_stride, const float *y, int64_t y_stride,
                                                            const float *row_div, float scale, float *grad_z,
-                                                           float *w_grad, float *bias_grad, void *workspace, int64_t rows,
+                                                           float *w_grad, float *bias_grad, void *workspace, int64_t workspace_bytes, int64_t rows,
                                                            int64_t fi, int64_t fo, void *stream) {
     GNNAGG_REQUIRE(bias_grad, "null bias_grad");
     GNNAGG_REQUIRE(!y || (y_stride >= fo && y_stride < (int64_t(1) << 27)), "bad row stride of y");
     MaskArgs mk{y ? y : grad_y, row_div, grad_z, nullptr, (int)(y ? y_stride : 0), scale, y ? 0 : 1, nullptr, 0, 0};
-    return run_wgrad(x, x_stride, grad_y, grad_stride, w_grad, workspace, rows, fi, fo, stream, &mk, bias_grad, 1);
+    return run_wgrad(x, x_stride, grad_y, grad_stride, w_grad, workspace, workspace_bytes, rows, fi, fo, stream, &mk, bias_grad, 1);
 }
 
 extern "C" int gnnagg_wgrad_relu_dropout_backward_bf16x3_f32(const float *x, int64_t x_stride, const float *grad_y,
                                                              int64_t grad_stride, const float *y, int64_t y_stride,
                                                              const float *row_div, float scale, float *grad_z,
-                                                             float *w_grad, float *bias_grad, void *workspace,
+                                                             float *w_grad, float *bias_grad, void *workspace, int64_t workspace_bytes,
                                                              int64_t rows, int64_t fi, int64_t fo, void *stream) {
     GNNAGG_REQUIRE(bias_grad, "null bias_grad");
     GNNAGG_REQUIRE(!y || (y_stride >= fo && y_stride < (int64_t(1) << 27)), "bad row stride of y");
     MaskArgs mk{y ? y : grad_y, row_div, grad_z, nullptr, (int)(y ? y_stride : 0), scale, y ? 0 : 1, nullptr, 0, 0};
-    return run_wgrad(x, x_stride, grad_y, grad_stride, w_grad, workspace, rows, fi, fo, stream, &mk, bias_grad, 2);
+    return run_wgrad(x, x_stride, grad_y, grad_stride, w_grad, workspace, workspace_bytes, rows, fi, fo, stream, &mk, bias_grad, 2);
 }
 
 extern "C" int gnnagg_wgrad_relu_dropout_backward_from_header_f32(const float *x, int64_t x_stride, const float *grad_y,
                                                                   int64_t grad_stride, const uint32_t *header,
                                                                   const float *row_div, float scale, float *grad_z,
-                                                                  float *w_grad, float *bias_grad, void *workspace,
+                                                                  float *w_grad, float *bias_grad, void *workspace, int64_t workspace_bytes,
                                                                   int64_t rows, int64_t fi, int64_t fo, int bf16_inputs,
                                                                   void *stream) {
     GNNAGG_REQUIRE(bias_grad, "null bias_grad");
@@ -821,6 +832,6 @@ extern "C" int gnnagg_wgrad_relu_dropout_backward_from_header_f32(const float *x
     if (!(fo == 32 || fo == 64 || fo == 128 || fo == 256))
         return fail(GNNAGG_ERR_UNSUPPORTED, "packed activations exist for widths 32, 64, 128, 256 (got %lld)", (long long)fo);
     MaskArgs mk{nullptr, row_div, grad_z, nullptr, 0, scale, 0, header, (int)(2 * (fo / 32)), 2};
-    return run_wgrad(x, x_stride, grad_y, grad_stride, w_grad, workspace, rows, fi, fo, stream, &mk, bias_grad,
+    return run_wgrad(x, x_stride, grad_y, grad_stride, w_grad, workspace, workspace_bytes, rows, fi, fo, stream, &mk, bias_grad,
                      bf16_inputs);
 }

@@ -72,7 +72,8 @@ def weight_gradient(x: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
     workspace = torch.empty(nbytes // 4, dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
         _lib.check(L.gnnagg_wgrad_strided_f32(_lib.ptr(x), _row_stride(x), _lib.ptr(g), _row_stride(g), _lib.ptr(out),
-                                              _lib.ptr(workspace), rows, fi, fo, _lib.current_stream(x.device)))
+                                              _lib.ptr(workspace), nbytes, rows, fi, fo,
+                                              _lib.current_stream(x.device)))
     return out
 
 
@@ -94,7 +95,7 @@ def weight_and_bias_gradient(x: torch.Tensor, g: torch.Tensor, form: int = 0):
         entry = L.gnnagg_wgrad_relu_dropout_backward_bf16x3_f32 if form == 2 else L.gnnagg_wgrad_relu_dropout_backward_f32
         _lib.check(entry(
             _lib.ptr(x), _row_stride(x), _lib.ptr(g), _row_stride(g), None, 0, None, 1.0, None, _lib.ptr(grad_w),
-            _lib.ptr(grad_b), _lib.ptr(workspace), rows, fi, fo, _lib.current_stream(x.device)))
+            _lib.ptr(grad_b), _lib.ptr(workspace), nbytes, rows, fi, fo, _lib.current_stream(x.device)))
     return grad_w, grad_b
 
 
@@ -265,8 +266,8 @@ def _fused_backward(x, w, grad_y, y, header, row_div, scale, form, want_x):
     grad_y = _kernel_ready(grad_y)
     rows, k, n = x.size(0), x.size(1), w.size(1)
     L = _lib.lib()
-    workspace = torch.empty(int(L.gnnagg_wgrad_relu_dropout_backward_workspace_bytes(max(rows, 1), k, n)) // 4,
-                            dtype=torch.float32, device=x.device)
+    nbytes = int(L.gnnagg_wgrad_relu_dropout_backward_workspace_bytes(max(rows, 1), k, n))
+    workspace = torch.empty(nbytes // 4, dtype=torch.float32, device=x.device)
     grad_z = torch.empty(rows, n, dtype=torch.float32, device=x.device) if want_x else None
     grad_w = torch.empty(k, n, dtype=torch.float32, device=x.device)
     grad_bias = torch.empty(n, dtype=torch.float32, device=x.device)
@@ -276,14 +277,14 @@ def _fused_backward(x, w, grad_y, y, header, row_div, scale, form, want_x):
         if header is not None:
             _lib.check(L.gnnagg_wgrad_relu_dropout_backward_from_header_f32(
                 _lib.ptr(x), _row_stride(x), _lib.ptr(grad_y), _row_stride(grad_y), _lib.ptr(header), _lib.ptr(row_div),
-                scale, _lib.ptr(grad_z), _lib.ptr(grad_w), _lib.ptr(grad_bias), _lib.ptr(workspace), rows, k, n,
+                scale, _lib.ptr(grad_z), _lib.ptr(grad_w), _lib.ptr(grad_bias), _lib.ptr(workspace), nbytes, rows, k, n,
                 int(form), stream))
         else:
             entry = (L.gnnagg_wgrad_relu_dropout_backward_f32, L.gnnagg_wgrad_relu_dropout_backward_bf16_f32,
                      L.gnnagg_wgrad_relu_dropout_backward_bf16x3_f32)[int(form)]
             _lib.check(entry(_lib.ptr(x), _row_stride(x), _lib.ptr(grad_y), _row_stride(grad_y), _lib.ptr(y),
                              n if y is not None else 0, _lib.ptr(row_div), scale, _lib.ptr(grad_z), _lib.ptr(grad_w),
-                             _lib.ptr(grad_bias), _lib.ptr(workspace), rows, k, n, stream))
+                             _lib.ptr(grad_bias), _lib.ptr(workspace), nbytes, rows, k, n, stream))
     grad_x = None
     if want_x:
         if form != FP32 and L.gnnagg_linear_shape_supported(n, k):

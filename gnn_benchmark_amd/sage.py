@@ -224,10 +224,13 @@ class _SageConvRows(torch.autograd.Function):
             grad_agg = grad_small[:, :fi]
             if ctx.divide:
                 grad_agg.div_(ctx.graph.in_degrees)
-            # the gradient goes where the features were: the right half of an [N, 2 fi] array (its left half was
-            # scratch on the way forward and is left unwritten here): A[rows]^T (d/d aggregated), then the direct
-            # part added onto the rows it belongs to (every row once: deterministic)
+            # the gradient goes where the features were: the right half of an [N, 2 fi] array: A[rows]^T (d/d
+            # aggregated), then the direct part added onto the rows it belongs to (every row once: deterministic).
+            # The left half was scratch on the way forward: nothing depends on it, so its gradient is zero -- written
+            # as such, because autograd hands this array on (to a leaf that requires grad, or into a sum with another
+            # consumer's gradient) and uninitialised memory there could be anything, NaN included.
             grad_cat = torch.empty(ctx.nodes, 2 * fi, dtype=torch.float32, device=g.device)
+            grad_cat[:, :fi].zero_()
             target = grad_cat[:, fi:]
             aggregator._backward(ctx, grad_agg, out=target, accumulate=False)
             target.index_add_(0, rows, grad_small[:, fi:])
@@ -280,8 +283,9 @@ class _SageConvLinearFirst(torch.autograd.Function):
         if ctx.needs_input_grad[1]:
             if ctx.staged:
                 # the gradient goes where the features were: the right half of an [N, 2 fi] array
-                # (its left half was scratch on the way forward and is left unwritten here)
+                # (its left half was scratch on the way forward: zero gradient, written as such)
                 grad_x = torch.empty(x.size(0), 2 * fi, dtype=torch.float32, device=x.device)
+                grad_x[:, :fi].zero_()
                 target = grad_x[:, fi:]
                 torch.mm(g, weight[fi:].t(), out=target)
                 target.addmm_(grad_left, weight[:fi].t())

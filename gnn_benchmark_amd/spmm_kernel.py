@@ -50,6 +50,8 @@ def _spmm_quantized(plan, value, packed, params, row_code, out, bits, accumulate
             or out.dtype != torch.float32 or not _rows_are_dense(out) or value.dtype != torch.float32):
         raise RuntimeError("Input mismatch: quantised SpMM needs uint8 [packed rows, F] bytes, float32 [rows, 2] "
                            "parameters, int32 [rows] row codes and a float32 [*, F] output with contiguous rows")
+    # the kernel addresses byte row (row_code >> 3) of the packed buffer: checked once per code tensor and buffer height
+    _lib.check_index(row_code, packed.size(0), shift=3, what="row codes of the packed buffer")
     with torch.cuda.device(out.device):
         _lib.check(_lib.lib().gnnagg_plan_spmm_quantized_f32(
             plan._handle, _lib.ptr(value.contiguous()), _lib.ptr(packed), _lib.ptr(params), _lib.ptr(row_code),

@@ -101,7 +101,10 @@ typedef struct gnnagg_plan_options {
 int gnnagg_plan_create_ex(const int64_t *rowptr, const int64_t *col, int64_t rows, int64_t cols, int64_t nnz,
                           const gnnagg_plan_options *options, void *stream, gnnagg_plan **plan_out);
 
-/* Frees a plan (synchronises the device; NULL is accepted). */
+/* Gives a plan back (NULL is accepted).  Makes no HIP call and never synchronises -- safe from a destructor in the
+ * middle of a training step or while a stream is being captured; work already enqueued with the plan runs to its
+ * end.  The plan's device memory is released by the next gnnagg_plan_create[_ex] on the same device (set-up work
+ * that synchronises anyway), after a device synchronisation. */
 int gnnagg_plan_destroy(gnnagg_plan *plan);
 
 /* out (+)= A @ mat through a plan.  `value` is the fp32 [nnz] array in the CSR order
@@ -172,10 +175,20 @@ int gnnagg_coo_to_csr(const int64_t *row, const int64_t *col, const float *value
 /* ---------------------------------------------------------------------------------
  * Boundary-row gather, out[i,:] = src[index[i],:].  Replaces
  * `torch.index_select(local_nodes_feat, 0, idx_nodes_send_to_others, out=send_buf)`
- * (model/layers/aggregator.py:51).  index int64 [n_index]; not range-checked.
+ * (model/layers/aggregator.py:51).  src fp32 [src_rows, feat], index int64 [n_index].  An index outside
+ * [0, src_rows) is never dereferenced: its output row is filled with NaN (torch.index_select raises for it;
+ * raising needs the index values on the host -- gnnagg_check_index below does that once per index list).
  * ------------------------------------------------------------------------------- */
-int gnnagg_gather_rows_f32(const float *src, const int64_t *index, float *out, int64_t n_index, int64_t feat,
-                           void *stream);
+int gnnagg_gather_rows_f32(const float *src, int64_t src_rows, const int64_t *index, float *out, int64_t n_index,
+                           int64_t feat, void *stream);
+
+/* Range check of an index list held on the device: GNNAGG_OK when every (index[i] >> shift) lies in [0, bound),
+ * GNNAGG_ERR_INVALID (naming the first offending position found) otherwise.  index: `count` integers of
+ * elem_bytes 4 (int32) or 8 (int64).  SYNCHRONISES the stream: meant to run once per index list (the boundary
+ * row list of a graph, the column array handed to gnnagg_spmm_csr_f32, the row codes of a packed buffer), not per
+ * call.  Replaces the bounds checks torch's indexing ops make on the host in the reference
+ * (torch.index_select / index_add_, model/layers/aggregator.py:51, :197-199). */
+int gnnagg_check_index(const void *index, int elem_bytes, int64_t count, int shift, int64_t bound, void *stream);
 
 /* ---------------------------------------------------------------------------------
  * Fused layer epilogue around the aggregation path (the full train-step workload):
@@ -205,16 +218,17 @@ int gnnagg_relu_dropout_backward_f32(const float *grad_y, const float *y, const 
  * otherwise).  Hand-written fp32 MFMA kernel plus a fixed-order reduction of per-slice
  * partial results: deterministic.  `workspace` is caller-provided device memory of
  * gnnagg_wgrad_workspace_bytes(rows, fi, fo) bytes (0 = unsupported shape); nothing is
- * allocated here.  Part of this build's GCN layer stack (the reference leaves this product
+ * allocated here.  `workspace_bytes` is the size of what the caller passes: less than that
+ * figure returns GNNAGG_ERR_INVALID before anything is launched.  Part of this build's GCN layer stack (the reference leaves this product
  * to torch's Linear backward, model/layers/sageconv.py:87-88).
  * ------------------------------------------------------------------------------- */
 int64_t gnnagg_wgrad_workspace_bytes(int64_t rows, int64_t fi, int64_t fo);
-int gnnagg_wgrad_f32(const float *x, const float *g, float *w_grad, void *workspace, int64_t rows, int64_t fi,
-                     int64_t fo, void *stream);
+int gnnagg_wgrad_f32(const float *x, const float *g, float *w_grad, void *workspace, int64_t workspace_bytes,
+                     int64_t rows, int64_t fi, int64_t fo, void *stream);
 /* The same with x and / or g being column blocks of wider row-major arrays (row strides in
  * floats): the two halves of a SAGE layer's [A x | x] operand are read where they lie. */
 int gnnagg_wgrad_strided_f32(const float *x, int64_t x_stride, const float *g, int64_t g_stride, float *w_grad,
-                             void *workspace, int64_t rows, int64_t fi, int64_t fo, void *stream);
+                             void *workspace, int64_t workspace_bytes, int64_t rows, int64_t fi, int64_t fo, void *stream);
 
 /* gnnagg_wgrad_f32 for callers that cannot allocate device memory (code recorded into a HIP graph, tight serving
  * loops, harnesses that forbid hipMalloc): no workspace argument, the per-slice partial results go to a 64 MiB
@@ -248,7 +262,8 @@ int gnnagg_wgrad_noalloc_f32(const float *x, const float *g, float *w_grad, int6
  * scale); grad_z = NULL: not written (a caller that only wants w_grad and bias_grad, e.g.
  * the SAGE layer's `+ bias`, model/layers/sageconv.py:91).  Needs fi, fo <= 256 and multiples of 4, 16-byte aligned
  * operands and row strides; workspace of gnnagg_wgrad_relu_dropout_backward_workspace_bytes
- * (0 = unsupported shape) bytes, nothing is allocated.  Deterministic.
+ * (0 = unsupported shape) bytes, its size passed as workspace_bytes (too small: GNNAGG_ERR_INVALID);
+ * nothing is allocated.  Deterministic.
  * The reference leaves these products to torch's Linear and runs dropout / ReLU as separate
  * ops (model/layers/sageconv.py:87-91, model/DistSAGE.py:49-53); the fused forms belong to
  * this build's GCN layer stack.
@@ -288,27 +303,27 @@ int64_t gnnagg_wgrad_relu_dropout_backward_workspace_bytes(int64_t rows, int64_t
 int gnnagg_wgrad_relu_dropout_backward_f32(const float *x, int64_t x_stride, const float *grad_y, int64_t grad_stride,
                                            const float *y, int64_t y_stride, const float *row_div, float scale,
                                            float *grad_z, float *w_grad, float *bias_grad, void *workspace,
-                                           int64_t rows, int64_t fi, int64_t fo, void *stream);
+                                           int64_t workspace_bytes, int64_t rows, int64_t fi, int64_t fo, void *stream);
 /* The same when the layer's output was written packed: which units were active is read from the bitmaps of its
  * header (fo in {32, 64, 128, 256}) instead of from y; bf16_inputs picks the product's form (0 fp32 MFMA, 1 operands
  * rounded to bf16, 2 three bf16 pieces per operand). */
 int gnnagg_wgrad_relu_dropout_backward_from_header_f32(const float *x, int64_t x_stride, const float *grad_y,
                                                        int64_t grad_stride, const uint32_t *header, const float *row_div,
                                                        float scale, float *grad_z, float *w_grad, float *bias_grad,
-                                                       void *workspace, int64_t rows, int64_t fi, int64_t fo,
-                                                       int bf16_inputs, void *stream);
+                                                       void *workspace, int64_t workspace_bytes, int64_t rows, int64_t fi,
+                                                       int64_t fo, int bf16_inputs, void *stream);
 int gnnagg_wgrad_relu_dropout_backward_bf16_f32(const float *x, int64_t x_stride, const float *grad_y,
                                                 int64_t grad_stride, const float *y, int64_t y_stride,
                                                 const float *row_div, float scale, float *grad_z, float *w_grad,
-                                                float *bias_grad, void *workspace, int64_t rows, int64_t fi, int64_t fo,
-                                                void *stream);
+                                                float *bias_grad, void *workspace, int64_t workspace_bytes, int64_t rows,
+                                                int64_t fi, int64_t fo, void *stream);
 /* (the _bf16x3_ form: the product x^T @ grad_z in fp32 accuracy on the bf16 matrix units, every value of x and
  * grad_z cut into three bf16 pieces, six bf16 MFMAs a product -- see gnnagg_linear_bias_relu_dropout_bf16x3_f32) */
 int gnnagg_wgrad_relu_dropout_backward_bf16x3_f32(const float *x, int64_t x_stride, const float *grad_y,
                                                   int64_t grad_stride, const float *y, int64_t y_stride,
                                                   const float *row_div, float scale, float *grad_z, float *w_grad,
-                                                  float *bias_grad, void *workspace, int64_t rows, int64_t fi,
-                                                  int64_t fo, void *stream);
+                                                  float *bias_grad, void *workspace, int64_t workspace_bytes, int64_t rows,
+                                                  int64_t fi, int64_t fo, void *stream);
 
 /* ---------------------------------------------------------------------------------
  * The elementwise chain between two SAGE layers (model/DistSAGE.py:49-53: F.dropout, LayerNorm

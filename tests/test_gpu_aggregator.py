@@ -510,3 +510,48 @@ def test_pregenerated_halo_rows_equal_the_seeded_ones():
     assert len(results[0]) == len(results[1])
     for a, b in zip(*results):
         assert torch.equal(a, b)
+
+
+def test_bad_indices_raise_instead_of_reading_out_of_bounds():
+    """torch.index_select raises on an index outside its source (the reference's gather); so do the gather, the
+    plan-less operator (column indices) and the aggregation straight from packed bytes (row codes) -- the lists are
+    looked at on the device once per tensor.  The gather kernel itself never dereferences such an index either."""
+    from gnn_benchmark_amd import _lib, computation_ops
+    from gnn_benchmark_amd.aggregator import _gather_rows
+    from gnn_benchmark_amd.spmm_kernel import SPMM_forward_quantized
+    from gnn_benchmark_amd.sparse_tensor import SparseTensor
+
+    src = torch.randn(50, 8, device="cuda")
+    out = torch.zeros(4, 8, device="cuda")
+    for bad in ([0, 50, 3, 4], [0, -1, 3, 4], [0, 1, 2, 2 ** 40]):
+        with pytest.raises(RuntimeError, match="outside"):
+            _gather_rows(src, torch.tensor(bad, device="cuda"), out)
+    good = torch.tensor([0, 49, 3, 4], device="cuda")
+    _gather_rows(src, good, out)
+    assert torch.equal(out, src[good])
+    good[1] = 50  # an in-place change is seen (the tensor's version counter moves)
+    with pytest.raises(RuntimeError, match="outside"):
+        _gather_rows(src, good, out)
+    # the C entry point on its own: the row of the bad index is NaN, its neighbours are gathered, nothing faults
+    idx = torch.tensor([7, 1 << 33, -5, 2], device="cuda")
+    _lib.check(_lib.lib().gnnagg_gather_rows_f32(_lib.ptr(src), 50, _lib.ptr(idx), _lib.ptr(out), 4, 8,
+                                                 _lib.current_stream(src.device)))
+    torch.cuda.synchronize()
+    assert torch.equal(out[0], src[7]) and torch.equal(out[3], src[2]) and bool(torch.isnan(out[1:3]).all())
+
+    rowptr = torch.tensor([0, 2, 3], device="cuda")
+    val = torch.ones(3, device="cuda")
+    res = torch.zeros(2, 8, device="cuda")
+    empty = torch.empty(0, dtype=torch.int32)
+    for bad_col in ([0, 50, 1], [0, -2, 1]):
+        with pytest.raises(RuntimeError, match="col"):
+            computation_ops.spmm(rowptr, torch.tensor(bad_col, device="cuda"), val, src, res, 2, empty, empty)
+    assert not res.any()
+
+    m = SparseTensor(rowptr=rowptr, col=torch.tensor([0, 3, 1], device="cuda"), value=val, sparse_sizes=(2, 4),
+                     is_sorted=True)
+    packed = torch.zeros(1, 8, dtype=torch.uint8, device="cuda")      # one byte row = four 2-bit rows
+    params = torch.ones(4, 2, device="cuda")
+    SPMM_forward_quantized(m, packed, params, torch.tensor([0, 1, 2, 3], dtype=torch.int32, device="cuda"), res, 2)
+    with pytest.raises(RuntimeError, match="row codes"):
+        SPMM_forward_quantized(m, packed, params, torch.tensor([0, 1, 2, 8], dtype=torch.int32, device="cuda"), res, 2)

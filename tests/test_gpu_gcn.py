@@ -283,12 +283,22 @@ def test_fused_layer_rejects_unsupported_shapes():
                                                     _lib.current_stream(x.device))
     assert rc == _lib.ERR_UNSUPPORTED
     g100 = torch.randn(64, 100, device="cuda")
-    ws = torch.empty(int(L.gnnagg_wgrad_relu_dropout_backward_workspace_bytes(64, 16, 100)) // 4, device="cuda")
+    nbytes = int(L.gnnagg_wgrad_relu_dropout_backward_workspace_bytes(64, 16, 100))
+    ws = torch.empty(nbytes // 4, device="cuda")
     gw, gb = torch.empty(16, 100, device="cuda"), torch.empty(100, device="cuda")
     rc = L.gnnagg_wgrad_relu_dropout_backward_from_header_f32(_lib.ptr(x16), 16, _lib.ptr(g100), 100, _lib.ptr(hdr), None,
-                                                              1.0, None, _lib.ptr(gw), _lib.ptr(gb), _lib.ptr(ws), 64, 16,
-                                                              100, 0, _lib.current_stream(x.device))
+                                                              1.0, None, _lib.ptr(gw), _lib.ptr(gb), _lib.ptr(ws), nbytes,
+                                                              64, 16, 100, 0, _lib.current_stream(x.device))
     assert rc == _lib.ERR_UNSUPPORTED
+    # a workspace smaller than the kernels write into is refused before anything is launched
+    xs, gs = torch.randn(5000, 64, device="cuda"), torch.randn(5000, 32, device="cuda")
+    need = int(L.gnnagg_wgrad_workspace_bytes(5000, 64, 32))
+    small = torch.empty(need // 4 - 1, device="cuda")
+    out = torch.zeros(64, 32, device="cuda")
+    rc = L.gnnagg_wgrad_f32(_lib.ptr(xs), _lib.ptr(gs), _lib.ptr(out), _lib.ptr(small), need - 4, 5000, 64, 32,
+                            _lib.current_stream(x.device))
+    assert rc == _lib.ERR_INVALID and b"workspace" in L.gnnagg_last_error()
+    assert not out.any()
     with pytest.raises(RuntimeError, match="behind a ReLU"):
         gcn._FusedLayer.apply(x16, torch.randn(16, 32, device="cuda"), torch.zeros(32, device="cuda"),
                               torch.zeros(64, 1, dtype=torch.int32, device="cuda"), 2.0, None, False)

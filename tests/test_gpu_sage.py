@@ -418,3 +418,43 @@ def test_reusing_a_staged_array_before_its_backward_is_detected():
         conv(graph, staged, 0)
         with pytest.raises(RuntimeError, match="modified by an inplace operation"):
             first.sum().backward()
+
+
+@pytest.mark.parametrize("linear_first", [False, True])
+def test_gradient_of_a_staged_leaf_is_clean_in_its_scratch_half(linear_first):
+    """Staged features that are a leaf requiring grad: the gradient autograd stores for them holds d loss / d x in the
+    right half and -- the left half being scratch that nothing reads -- finite zeros in the left half of whatever the
+    single-layer forms allocate themselves (row-restricted last layer; a layer that multiplies first), never
+    uninitialised memory."""
+    dev = "cuda:0"
+    n, fi, fo = 4000, 32, 12
+    part = synthetic.partition_edges(n, 4, 1, 5, 1.8, 400, 900, 5000, seed=6, device=dev)
+    graph = synthetic.build_partition_graph(part, fi, True, exchange=synthetic.SeededHaloExchange(2), device=dev)
+    gen = torch.Generator(device=dev).manual_seed(4)
+    x = torch.randn(n, fi, device=dev, generator=gen)
+    rows = torch.randperm(n, device=dev, generator=gen)[:500]
+    torch.manual_seed(1)
+    conv = sage.DistSAGEConvGrad(fi, fo, 32, True).to(dev)
+    conv.linear_first = linear_first
+    # poison freshly released memory so that an uninitialised result cannot pass by luck
+    junk = torch.full((n, 2 * fi), float("nan"), device=dev)
+    del junk
+    staged = sage.stage_input(x)
+    staged[:, :fi] = 0.0
+    staged.requires_grad_()
+    out = conv(graph, staged, 0) if linear_first else conv(graph, staged, 0, rows)
+    out.square().sum().backward()
+    grad = staged.grad
+    assert grad.shape == (n, 2 * fi) and bool(torch.isfinite(grad).all())
+    assert not bool(grad[:, :fi].any())
+    # the right half is the gradient another route to the same loss gives: plain features through the layer that
+    # multiplies first; every node through the aggregate-first layer, the loss reading the same rows
+    if linear_first:
+        other = x.clone().requires_grad_()
+        conv(graph, other, 0).square().sum().backward()
+        want = other.grad
+    else:
+        other = sage.stage_input(x).requires_grad_()
+        conv(graph, other, 0)[rows].square().sum().backward()
+        want = other.grad[:, fi:]
+    assert torch.allclose(grad[:, fi:], want, rtol=1e-4, atol=1e-5)

@@ -19,7 +19,7 @@ def _with_workspace(L, x, g):
     assert nbytes > 0
     ws = torch.empty(nbytes // 4, dtype=torch.float32, device=x.device)
     out = torch.empty(fi, fo, dtype=torch.float32, device=x.device)
-    _lib.check(L.gnnagg_wgrad_f32(_lib.ptr(x), _lib.ptr(g), _lib.ptr(out), _lib.ptr(ws), rows, fi, fo,
+    _lib.check(L.gnnagg_wgrad_f32(_lib.ptr(x), _lib.ptr(g), _lib.ptr(out), _lib.ptr(ws), nbytes, rows, fi, fo,
                                   _lib.current_stream(x.device)))
     return out
 
