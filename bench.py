@@ -222,12 +222,13 @@ def cpu_time_product(rowptr, col, val, x_host, rows):
 
 
 def time_planless(src, x, out, steps, warmup=2):
-    """Mean ms of ``computation_ops.spmm`` -- the literal export of the reference's op (ops.cpp:23): rows in their
-    natural order, int64 column indices, no cached plan -- on the launch stream."""
+    """Mean ms of ``computation_ops.spmm`` of the compiled extension module -- the literal export of the reference's
+    op (ops.cpp:23): rows in their natural order, int64 column indices, no cached plan -- on the launch stream."""
     import torch
 
-    from gnn_benchmark_amd import computation_ops
+    from gnn_benchmark_amd import ext
 
+    computation_ops = ext.load()  # the compiled pybind11 module, as the reference's wrapper would import it
     rowptr, col, val = src.csr()
     empty = torch.empty(0, dtype=torch.int32, device=x.device)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)

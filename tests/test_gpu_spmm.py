@@ -548,3 +548,35 @@ def test_many_rows_in_the_block_per_row_kernel(long_rows, feat, low_block_row_th
         plan.spmm(dev(val), dev(x), out, accumulate=accumulate)
         want = _oracle(rowptr, col, val, x, out0 if accumulate else None)
         assert np.array_equal(out.cpu().numpy(), want), accumulate
+
+
+def test_compiled_extension_module_on_the_committed_reference_outputs():
+    """The pybind11 module ``computation_ops`` (gnn_benchmark_amd/ext) called the way the reference's wrapper calls its
+    own (model/ops/spmm_kernel.py:62-64: eight positional arguments, split tensors included): the committed outputs of
+    the reference's compiled operator come back bit for bit, in the SAME storage as the ``out`` argument, with None
+    beside it."""
+    from gnn_benchmark_amd import ext
+    from tests.test_oracle_spmm import _golden_cases
+
+    mod = ext.load()
+    for c in _golden_cases():
+        rows, feat = c["out0"].shape
+        out = dev(c["out0"])
+        row_split = torch.zeros(9, dtype=torch.int32)                 # CPU thread ranges: accepted, ignored
+        col_split = torch.tensor([0, feat], dtype=torch.int32)
+        ret = mod.spmm(dev(c["rowptr"]), dev(c["col"]), dev(c["val"]), dev(c["x"]), out, rows, row_split, col_split)
+        assert isinstance(ret, tuple) and len(ret) == 2 and ret[1] is None
+        assert ret[0].data_ptr() == out.data_ptr() and ret[0].shape == out.shape
+        assert np.array_equal(out.cpu().numpy(), c["out"])
+    # a non-contiguous dense operand is made contiguous (spmm.cpp:350); errors surface as RuntimeError
+    c = _golden_cases()[1]
+    wide = dev(np.concatenate([c["x"], c["x"]], axis=1))
+    out = dev(c["out0"])
+    mod.spmm(dev(c["rowptr"]), dev(c["col"]), dev(c["val"]), wide[:, :c["x"].shape[1]], out, c["out0"].shape[0],
+             EMPTY_I32, EMPTY_I32)
+    assert np.array_equal(out.cpu().numpy(), c["out"])
+    with pytest.raises(RuntimeError, match="value is required"):
+        mod.spmm(dev(c["rowptr"]), dev(c["col"]), None, dev(c["x"]), out, c["out0"].shape[0], EMPTY_I32, EMPTY_I32)
+    with pytest.raises(RuntimeError, match="Input mismatch"):
+        mod.spmm(dev(c["rowptr"]), dev(c["col"]), dev(c["val"]).double(), dev(c["x"]), out, c["out0"].shape[0], EMPTY_I32,
+                 EMPTY_I32)

@@ -76,3 +76,26 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libgnnagg.so"))
     with pytest.raises(RuntimeError, match="libgnnagg.so is missing"):
         _lib.lib()
+
+
+def test_compiled_extension_module_keeps_the_reference_signature():
+    """``computation_ops.spmm`` as a compiled pybind11 module (self_benchmark/a64fx/model/ops/src/ops.cpp:23): eight
+    positional arguments, value optional in the signature, ``(out, None)`` back; CPU tensors are refused before any
+    GPU work."""
+    import torch
+
+    from gnn_benchmark_amd import ext
+
+    try:
+        mod = ext.load()
+    except RuntimeError:
+        pytest.skip("the extension module is not built yet (gnn_benchmark_amd/ext/build.sh)")
+    assert mod.__name__ == "computation_ops"
+    doc = mod.spmm.__doc__
+    assert doc.count("torch.Tensor") >= 8 and "tuple[torch.Tensor, torch.Tensor | None]" in doc.replace("Optional[torch.Tensor]", "torch.Tensor | None")
+    empty = torch.empty(0, dtype=torch.int32)
+    args = (torch.tensor([0, 1]), torch.tensor([0]), torch.ones(1), torch.ones(1, 4), torch.zeros(1, 4), 1, empty, empty)
+    with pytest.raises(RuntimeError, match="GPU"):
+        mod.spmm(*args)
+    with pytest.raises(TypeError):
+        mod.spmm(*args[:7])
