@@ -35,11 +35,27 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak
 
 # HBM-side traffic of ONE launch, measured with rocprofv3 --pmc on this file's own workloads (default sizes and
 # seed): bytes read = 32 / 64 / 128-byte read requests of the L2 to the memory side, counted by size
-# (TCC_EA0_RDREQ_32B / _64B / _128B), bytes written = WRITE_SIZE.  (workload, op, F) -> (bytes read, bytes written,
+# (TCC_EA0_RDREQ_32B / _64B / _128B; on this GPU practically all are 128-byte requests), bytes written =
+# WRITE_SIZE.  "Memory side" is what lies behind the L2: HBM and the 256 MB memory-side cache in front of it, which
+# these counters cannot tell apart.  (workload, op, F) -> (bytes read, bytes written,
 # the summary under profiles/ that holds the counter readings and the commands).  These are constants taken from
 # those profile runs, not something a timed run can produce (the counters need the profiler): the JSON labels
 # them "profile".  Any other size or seed: no entry, and the measured fields are left out.
+_P = "profiles/spmm_memory_traffic_c2_c3_c4.md"
 MEASURED_TRAFFIC = {
+    ("c2", "A@X", 100): (5.68207e+10, 1.01207e+09, _P), ("c2", "A^T@G", 100): (5.68207e+10, 1.01207e+09, _P),
+    ("c2", "A@X", 128): (5.71924e+10, 1.25440e+09, _P), ("c2", "A^T@G", 128): (5.71924e+10, 1.25440e+09, _P),
+    ("c2", "A@X", 256): (1.18675e+11, 2.50880e+09, _P), ("c2", "A^T@G", 256): (1.18675e+11, 2.50880e+09, _P),
+    # (c3: the block-per-row kernel's share, 0.8 / 0.3 GB, is included in the forward figures)
+    ("c3", "A@X", 602): (2.94247e+11, 5.82812e+08, _P), ("c3", "A^T@G", 602): (2.85891e+11, 5.91882e+08, _P),
+    ("c3", "A@X", 256): (1.18438e+11, 2.38592e+08, _P), ("c3", "A^T@G", 256): (1.12242e+11, 2.38592e+08, _P),
+    ("c4", "pre", 128): (1.22851e+10, 1.53568e+09, _P), ("c4", "pre_overwrite", 128): (1.07445e+10, 1.53568e+09, _P),
+    ("c4", "pre_T", 128): (1.43904e+10, 3.37825e+09, _P), ("c4", "pre_T_overwrite", 128): (1.10097e+10, 3.58400e+09, _P),
+    ("c4", "local", 128): (5.48747e+10, 3.58400e+09, _P), ("c4", "local_overwrite", 128): (5.12406e+10, 3.58400e+09, _P),
+    ("c4", "local_T", 128): (5.48742e+10, 3.58400e+09, _P), ("c4", "local_T_overwrite", 128): (5.12387e+10, 3.58400e+09, _P),
+    ("c4", "post", 128): (1.43898e+10, 3.37825e+09, _P), ("c4", "post_overwrite", 128): (1.10093e+10, 3.58400e+09, _P),
+    ("c4", "post_T", 128): (1.22983e+10, 1.55268e+09, _P), ("c4", "post_T_overwrite", 128): (1.07407e+10, 1.55268e+09, _P),
+    ("c4", "local_planless", 128): (5.58080e+10, 3.58400e+09, _P),
 }
 
 
@@ -574,7 +590,8 @@ def run_c4(args, graph, setup_s):
     ms = time_planless(graph.local_adj_t, x, out, steps)
     ops.append(op_report("local A_local@X through computation_ops.spmm (no plan: natural row order, int64 column "
                          "indices)", graph.local_adj_t.nnz(), n, n, feat, ms,
-                         graph.local_adj_t.get_plan().info()["empty_rows"]))
+                         graph.local_adj_t.get_plan().info()["empty_rows"],
+                         measured=measured_traffic(args, "c4", "local_planless", feat)))
     # the whole autograd.Function, forward and backward, synthetic halo rows generated on the device
     xr = x.clone().requires_grad_()
     for _ in range(2):

@@ -36,6 +36,9 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     cpu = d["cpu_baseline"]
     assert cpu["kind"] in ("reference", "port") and cpu["cores"] >= 1 and cpu["value"] > 0 and cpu["unit"] == "GFLOP/s"
     assert isinstance(cpu["sample"], str)
+    assert isinstance(cpu["cpu_model"], str) and cpu["host_physical_cores"] >= 1 and "2 warm-ups" in cpu["protocol"]
+    fwd = d["extra"]["c2"][0]["forward"]
+    assert "frac_model" in fwd and "frac_of_hbm_peak" not in fwd and "frac_measured" not in fwd  # (no profile for this size)
 
 
 @pytest.mark.gpu
