@@ -494,6 +494,28 @@ def run_ceilings(args):
         results = gathers // per_row
         nbytes = results * per_row * (row_b + 4.0) + (results * row_b if kind >= 4 else 0) + (results * row_b if kind == 5 else 0)
         out[name] = timed(kind, results, per_row, nbytes)
+
+    # matrix pipe and vector ALU of a SIMD, fed by different waves (`gnnagg_issue_probe`): alone and together
+    def issue(mfma_rounds, valu_rounds, reps=5):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for i in range(reps + 2):
+            if i == 2:
+                e0.record()
+            _lib.check(L.gnnagg_issue_probe(mfma_rounds, valu_rounds, _lib.ptr(dst), stream))
+        e1.record()
+        e1.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    rounds = 5000
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    m, v, both = issue(rounds, 0), issue(0, rounds), issue(rounds, rounds)
+    out["matrix_pipe_and_vector_alu"] = {
+        "what": f"one block of 8 waves per compute unit; waves 0-3 issue {8 * rounds} independent v_mfma_f32_32x32x16_bf16 "
+                f"each, waves 4-7 run {8 * rounds} rounds of the fp32 -> bf16-pieces cutting sequence each",
+        "mfma_alone_ms": round(m, 4), "vector_alone_ms": round(v, 4), "together_ms": round(both, 4),
+        "sum_of_the_two_ms": round(m + v, 4),
+        "mfma_alone_tflops": round(2.0 * 32 * 32 * 16 * 8 * rounds * 4 * cus / m / 1e9, 1),
+        "reading": "together = max of the two: the pipes overlap; together = their sum: they take turns"}
     return out
 
 

@@ -63,6 +63,7 @@ EXPORTS = (
     "gnnagg_f32_to_bf16",
     "gnnagg_bf16_to_f32",
     "gnnagg_memory_probe",
+    "gnnagg_issue_probe",
 )
 
 _lib = None
@@ -201,6 +202,8 @@ def lib() -> ctypes.CDLL:
     L.gnnagg_dequantize_mixed_f32.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp]
     L.gnnagg_memory_probe.restype = i32
     L.gnnagg_memory_probe.argtypes = [i32, vp, vp, vp, i64, i64, i64, vp]
+    L.gnnagg_issue_probe.restype = i32
+    L.gnnagg_issue_probe.argtypes = [i32, i32, vp, vp]
     if L.gnnagg_abi_version() != ABI_VERSION:
         raise RuntimeError("libgnnagg.so was built from a different include/gnn_agg.h; rebuild it")
     _lib = L

@@ -80,6 +80,57 @@ __global__ __launch_bounds__(256) void probe_gather_kernel(const float *__restri
     if (mode == 0 && keep.x + keep.y + keep.z + keep.w == 1.2345678e38f) sink[0] = keep.x;
 }
 
+
+// Issue probe: do the matrix pipe and the vector ALU of a SIMD work at the same time when different waves feed
+// them?  One block of eight waves per compute unit; waves 0-3 (one per SIMD) issue independent bf16 MFMAs
+// (v_mfma_f32_32x32x16_bf16, eight accumulators), waves 4-7 (one per SIMD) run the vector-ALU sequence that cuts fp32
+// values into three bf16 pieces.  Either side can be switched off; the caller times the three combinations.
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 probe_bf16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 probe_bf16x8 __attribute__((ext_vector_type(8)));
+
+__global__ __launch_bounds__(512) void probe_issue_kernel(float *__restrict__ sink, int mfma_rounds, int valu_rounds) {
+    const int wave = threadIdx.x >> 6;
+    float s = 0.f;
+    if (wave < 4) {
+        f32x16 acc[8];
+#pragma unroll
+        for (int a = 0; a < 8; ++a)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[a][r] = 0.f;
+        probe_bf16x8 x, y;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            x[e] = (__bf16)(float)((threadIdx.x + e) & 7);
+            y[e] = (__bf16)(float)(e + 1);
+        }
+        for (int i = 0; i < mfma_rounds; ++i) {
+#pragma unroll
+            for (int a = 0; a < 8; ++a) acc[a] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x, y, acc[a], 0, 0, 0);
+        }
+#pragma unroll
+        for (int a = 0; a < 8; ++a) s += acc[a][0] + acc[a][15];
+    } else {
+        f32x2 v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = f32x2{(float)(threadIdx.x + e) * 1.37f, (float)(e + 1) * 0.77f};
+        for (int i = 0; i < valu_rounds; ++i) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {  // hi = bf16(v), mid = bf16(v - hi), what is left feeds the next round
+                const probe_bf16x2 hi = __builtin_convertvector(v[e], probe_bf16x2);
+                const f32x2 r = v[e] - __builtin_convertvector(hi, f32x2);
+                const probe_bf16x2 mid = __builtin_convertvector(r, probe_bf16x2);
+                const f32x2 r2 = r - __builtin_convertvector(mid, f32x2);
+                v[e] = r2 * 65536.0f + v[e];
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s += v[e].x + v[e].y;
+    }
+    if (s == 1.2345678e38f) sink[0] = s;  // never true: keeps the work alive
+}
+
 }  // namespace
 }  // namespace gnnagg
 
@@ -129,6 +180,19 @@ extern "C" int gnnagg_memory_probe(int kind, const float *src, const int32_t *in
     else
         return fail(GNNAGG_ERR_UNSUPPORTED, "gather probes exist for rows of 64, 128 and 256 floats (got %lld)",
                     (long long)row_floats);
+    GNNAGG_HIP(hipGetLastError());
+    return GNNAGG_OK;
+}
+
+extern "C" int gnnagg_issue_probe(int mfma_rounds, int valu_rounds, float *sink, void *stream) {
+    GNNAGG_REQUIRE(mfma_rounds >= 0 && valu_rounds >= 0 && mfma_rounds <= (1 << 20) && valu_rounds <= (1 << 20),
+                   "rounds outside 0 .. 2^20");
+    GNNAGG_REQUIRE(sink, "null sink");
+    int dev = 0, cus = 0;
+    GNNAGG_HIP(hipGetDevice(&dev));
+    GNNAGG_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    hipLaunchKernelGGL(probe_issue_kernel, dim3(cus > 0 ? cus : 256), dim3(512), 0, static_cast<hipStream_t>(stream), sink,
+                       mfma_rounds, valu_rounds);
     GNNAGG_HIP(hipGetLastError());
     return GNNAGG_OK;
 }

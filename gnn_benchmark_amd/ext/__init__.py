@@ -11,6 +11,7 @@ import subprocess
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _module = None
+_DOC_PREFIX = "MI355X drop-in"   # how computation_ops.cpp documents the module
 
 
 def build(verbose: bool = False) -> str:
@@ -38,5 +39,10 @@ def load():
         spec = importlib.util.spec_from_file_location("computation_ops", path)
         module = importlib.util.module_from_spec(spec)
         spec.loader.exec_module(module)
+        # pybind11 keeps one module object per module NAME in a process: had another pybind11 module called
+        # `computation_ops` (the reference's CPU build, say) been imported first, its object would come back here
+        if not (module.__doc__ or "").startswith(_DOC_PREFIX):
+            raise RuntimeError("another compiled module named computation_ops is already loaded in this process; "
+                               f"{path} cannot be loaded beside it")
         _module = module
     return _module

@@ -455,6 +455,14 @@ int gnnagg_bf16_to_f32(const uint16_t *x, float *y, int64_t count, void *stream)
 int gnnagg_memory_probe(int kind, const float *src, const int32_t *index, float *dst, int64_t count,
                         int64_t row_floats, int64_t per_row, void *stream);
 
+/* Issue probe.  One block of eight waves per compute unit: waves 0-3 (one per SIMD) issue `mfma_rounds` x 8
+ * independent v_mfma_f32_32x32x16_bf16, waves 4-7 (one per SIMD) run `valu_rounds` x 8 rounds of the vector-ALU
+ * sequence that cuts a pair of fp32 values into bf16 pieces (about 11 instructions a round).  Timing (mfma, 0),
+ * (0, valu) and (mfma, valu) shows whether the two pipes of a SIMD overlap when different waves feed them; the
+ * bf16 x 3 dense-layer kernels are designed around the answer.  No counterpart in the reference.  sink: 4 writable
+ * bytes, never written.  Allocates nothing, no host synchronisation. */
+int gnnagg_issue_probe(int mfma_rounds, int valu_rounds, float *sink, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -142,12 +142,16 @@ def cpu_has_avx512() -> bool:
 
 
 def load_reference_op():
-    """The reference's own ``computation_ops`` built by oracle/build_ref.sh, or None."""
-    hits = glob.glob(os.path.join(_HERE, "_ref", "computation_ops*.so"))
+    """The reference's own native module built by oracle/build_ref.sh (under the module name
+    ``reference_computation_ops``, so that it cannot be mistaken for, or handed out in place of, the product's
+    ``computation_ops``: pybind11 keeps one module object per module name in a process), or None."""
+    hits = glob.glob(os.path.join(_HERE, "_ref", "reference_computation_ops*.so"))
     if not hits or not cpu_has_avx512():
         return None
     import torch  # noqa: F401  (the module links against libtorch)
-    spec = importlib.util.spec_from_file_location("computation_ops", hits[0])
+    spec = importlib.util.spec_from_file_location("reference_computation_ops", hits[0])
     mod = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(mod)
+    if not hasattr(mod, "quantize_tensor"):  # the reference binds its quantisation kernels beside spmm (ops.cpp:11-40)
+        raise RuntimeError(f"{hits[0]} did not load as the reference's module")
     return mod
