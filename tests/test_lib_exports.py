@@ -106,7 +106,8 @@ def test_compiled_extension_module_keeps_the_reference_signature():
 def test_reference_build_and_drop_in_module_stay_apart_in_one_process(reference_op):
     """pybind11 keeps one module object per module name in a process, so the checker's build of the reference's
     module carries its own name: loaded in either order, it and the product's ``computation_ops`` are two modules
-    (the reference's binds the quantisation kernels too, the drop-in refuses CPU tensors)."""
+    (the reference's binds the quantisation kernels too, the drop-in refuses CPU tensors; the tests of the oracle
+    call the reference's ``spmm`` on CPU tensors in this same process)."""
     import torch
 
     from gnn_benchmark_amd import ext
@@ -118,11 +119,7 @@ def test_reference_build_and_drop_in_module_stay_apart_in_one_process(reference_
     assert mod is not reference_op
     assert mod.__name__ == "computation_ops" and reference_op.__name__ == "reference_computation_ops"
     assert hasattr(reference_op, "quantize_tensor") and not hasattr(mod, "quantize_tensor")
-    out = torch.zeros(1, 4)
     empty = torch.empty(0, dtype=torch.int32)
-    args = (torch.tensor([0, 1]), torch.tensor([0]), torch.ones(1), torch.ones(1, 4), out, 1,
-            torch.tensor([0, 1], dtype=torch.int32), torch.tensor([0, 4], dtype=torch.int32))
-    reference_op.spmm(*args)                       # the CPU operator computes
-    assert torch.equal(out, torch.ones(1, 4))
-    with pytest.raises(RuntimeError, match="GPU"):
-        mod.spmm(*args[:6], empty, empty)          # the drop-in has no CPU path
+    with pytest.raises(RuntimeError, match="GPU"):   # the drop-in has no CPU path (the reference's module computes)
+        mod.spmm(torch.tensor([0, 1]), torch.tensor([0]), torch.ones(1), torch.ones(1, 4), torch.zeros(1, 4), 1, empty,
+                 empty)
