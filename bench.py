@@ -352,7 +352,9 @@ def run_c2(args):
     }
     extra = {"c2": [r]}
     if "c2" in args.extras:
-        for f in (128, 256):
+        # the hidden widths of c4 / c5, c5's class count (172) and two narrow widths whose rows are not whole
+        # 16-byte vectors or 64-byte multiples (class counts 40 and 47)
+        for f in (128, 256, 172, 40, 47):
             if f != args.feat:
                 extra["c2"].append(spmm_pair(src, f, max(3, args.steps // 4), 2, gen, args, "c2")[0])
     line["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline_spmm(src, x.cpu().numpy(), gr.cpu().numpy())
