@@ -25,6 +25,9 @@
 // ([column][k]): a thread loads a 4 x 4 block of it and writes four 8-byte column pieces.  The
 // matrix work shrinks to a fraction of the time the operands take to stream in, so this form
 // is HBM-bound (4 * rows * (K + N) bytes).
+#include <type_traits>
+#include <utility>
+
 #include "common.h"
 #include "dense_tiles.h"
 
@@ -466,6 +469,353 @@ __global__ __launch_bounds__(256, 2) void linear_kernel(const LinearArgs p) {
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// The bf16-input form with the waves of a block split by role, and W resident in LDS.
+//
+// In the kernel above every wave does everything, one phase after the other: it issues the global loads of the next
+// chunk, multiplies the current one, converts what the loads brought and writes it to LDS.  With bf16 operands the
+// matrix work is a fraction of the time the operands take to stream in, so what counts is how many bytes of A a compute
+// unit keeps in flight.  Here one block of twelve waves owns a compute unit:
+//   * all of W, rounded to bf16 and transposed ([chunk of 16 k][column][16 k]: 32 bytes a column, the two 16-byte halves
+//     swapped for columns whose bit 3 is set so that sixteen neighbouring lanes read 64 distinct banks), is written to
+//     LDS once when the block starts (K x 256 x 2 bytes: 128 KB at K = 256) and stays there -- per-chunk loads of W would
+//     queue behind the deep stream of A in the compute unit's in-order vector-memory path (measured: 0.3-0.6 ms of 3.4);
+//   * waves 0-7 multiply: 4 x 2 over a tile of 128 rows x 256 columns, 32 rows x 128 columns each.  They read their rows
+//     of A as fp32 from LDS (16 floats per row and chunk), round them to bf16 in registers (v_cvt_pk_bf16_f32) and feed
+//     v_mfma_f32_32x32x16_bf16; the two waves of a SIMD (w and w + 4) work half an iteration apart, one multiplying while
+//     the other reads and converts;
+//   * waves 8-11 stream A: a 64-byte piece of each of the tile's 128 rows per chunk, kStreamDepth chunks (64 KB) in
+//     flight in their registers, written to a ring of three 8 KB LDS slots two chunks ahead of the multiplying waves.
+// One barrier per chunk hands slots over.  The epilogue is the same arithmetic as above on the same accumulator layout.
+// ---------------------------------------------------------------------------------------------------------------
+constexpr int kStreamRows = 128;
+constexpr int kStreamDepth = 8;                    // chunks of A in flight in the loading waves' registers
+constexpr int kStreamSlots = 3;                    // raw A slots in LDS: chunks q, q + 1 being read, q + 2 being written
+constexpr int kStreamASlot = kStreamRows * 64;     // 8 KB: 128 rows x 16 fp32
+constexpr int kStreamWChunk = 256 * 32;            // 8 KB: 256 columns x 16 bf16
+constexpr int kStreamBias = 256 * 4;               // the bias (zeros when there is none), staged once per block
+constexpr int kStreamMaxK = 256;                   // W resident: K * 512 bytes of LDS
+inline size_t stream_smem_bytes(int k, bool pack) {
+    return (size_t)(k / kChunk) * kStreamWChunk + kStreamSlots * kStreamASlot + kStreamBias + (pack ? kStreamRows * sizeof(int) : 0);
+}
+
+// f(integral_constant<int, 0>{}), ..., f(integral_constant<int, N - 1>{}): a loop whose index is a constant expression
+template <int... Is, typename F>
+__device__ __forceinline__ void static_for_each(std::integer_sequence<int, Is...>, F &&f) {
+    (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+    static_for_each(std::make_integer_sequence<int, N>{}, f);
+}
+
+template <bool PACK>
+__global__ __launch_bounds__(768, 1) void linear_stream_bf16_kernel(const LinearArgs p) {
+    extern __shared__ __align__(16) char lds[];
+    const int nk = p.k / kChunk;
+    char *wres = lds;                                   // nk chunks of W
+    char *aring = lds + nk * kStreamWChunk;             // kStreamSlots chunks of A, fp32
+    float *bias_lds = reinterpret_cast<float *>(aring + kStreamSlots * kStreamASlot);
+    int *row_count = reinterpret_cast<int *>(bias_lds + 256);  // PACK: non-zeros of each tile row in columns 0-127
+    const int tid = (int)threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int64_t tiles = (p.rows + kStreamRows - 1) / kStreamRows;
+    if ((int64_t)blockIdx.x >= tiles) return;
+    const int my_tiles = (int)((tiles - blockIdx.x + gridDim.x - 1) / gridDim.x);
+    const int total = my_tiles * nk;  // chunks this block walks through, tile after tile
+    // the loading waves' loop is unrolled kStreamDepth times: everybody meets at `padded` + 1 barriers
+    const int padded = (total + kStreamDepth - 1) / kStreamDepth * kStreamDepth;
+    if (tid < 256) bias_lds[tid] = (p.bias && tid < p.n) ? p.bias[tid] : 0.0f;
+    // W: unit u = (chunk, half of the chunk's k, group of four columns); eight 16-byte loads, four 16-byte LDS writes
+    for (int u = tid; u < nk * 128; u += 768) {
+        const int cg = u & 63, khalf = (u >> 6) & 1, c = u >> 7;
+        // columns past n: any valid address; what they hold only reaches results that are never stored
+        const float *src = p.w + (size_t)(kChunk * c + 8 * khalf) * (size_t)p.ldw + (4 * cg < p.n ? 4 * cg : 0);
+        floatx4 wreg[8];
+#pragma unroll
+        for (int kr = 0; kr < 8; ++kr) wreg[kr] = *reinterpret_cast<const floatx4 *>(src + (size_t)kr * (size_t)p.ldw);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int col = 4 * cg + j;
+            union {
+                bf16x2 h[4];
+                floatx4 v;
+            } cv;
+#pragma unroll
+            for (int h = 0; h < 4; ++h) cv.h[h] = __builtin_convertvector(floatx2{wreg[2 * h][j], wreg[2 * h + 1][j]}, bf16x2);
+            *reinterpret_cast<floatx4 *>(wres + c * kStreamWChunk + col * 32 + 16 * (khalf ^ ((col >> 3) & 1))) = cv.v;
+        }
+    }
+    // (visible to the multiplying waves behind the first barrier below)
+
+    if (wave < 8) {
+        const int wr = wave >> 1, wc = wave & 1;
+        const int m0 = 32 * wr, n0 = 128 * wc;
+        const int kk = lane >> 5, idx = lane & 31;
+        // raw A slot: 16-byte unit (row, piece) sits at row * 4 + (piece ^ ((row >> 2) & 3)): sixteen neighbouring lanes
+        // (rows) reading the same piece hit 64 distinct banks
+        int a_off[2];
+        {
+            const int row = m0 + idx, sw = (row >> 2) & 3;
+            a_off[0] = (row * 4 + ((2 * kk) ^ sw)) * 16;
+            a_off[1] = (row * 4 + ((2 * kk + 1) ^ sw)) * 16;
+        }
+        const int b_off = (n0 + idx) * 32 + 16 * (kk ^ ((idx >> 3) & 1));
+        floatx16 acc[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[j][r] = 0.0f;
+        bf16x8 a_op, b_op[4];
+        auto read_convert = [&](int sa, int c) __attribute__((always_inline)) {
+            const char *pa = aring + sa * kStreamASlot;
+            const char *pw = wres + c * kStreamWChunk + b_off;
+            const floatx4 r0 = *reinterpret_cast<const floatx4 *>(pa + a_off[0]);
+            const floatx4 r1 = *reinterpret_cast<const floatx4 *>(pa + a_off[1]);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) b_op[j] = *reinterpret_cast<const bf16x8 *>(pw + j * 1024);
+            union {
+                bf16x2 h[4];
+                bf16x8 v;
+            } u;
+            u.h[0] = __builtin_convertvector(floatx2{r0.x, r0.y}, bf16x2);
+            u.h[1] = __builtin_convertvector(floatx2{r0.z, r0.w}, bf16x2);
+            u.h[2] = __builtin_convertvector(floatx2{r1.x, r1.y}, bf16x2);
+            u.h[3] = __builtin_convertvector(floatx2{r1.z, r1.w}, bf16x2);
+            a_op = u.v;
+        };
+        auto multiply = [&]() __attribute__((always_inline)) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b_op[j], a_op, acc[j], 0, 0, 0);
+        };
+
+        // 32x32 accumulator layout: register r of lane l holds D[(r % 4) + 4 * (l / 32) + 8 * (r / 4)][l % 32], D = a tile
+        // of Y^T: this lane owns runs of four consecutive columns of row m0 + idx
+        const int words = (p.n + 31) / 32;
+        float rdiv = 1.0f;
+        uint32_t kbits[4];
+        auto load_divisors = [&](int s) __attribute__((always_inline)) {
+            const int64_t m = ((int64_t)blockIdx.x + (int64_t)s * gridDim.x) * kStreamRows + m0 + idx;
+            const bool live = m < p.rows;
+            rdiv = (p.row_div && live) ? p.row_div[m] : 1.0f;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int nt = n0 + 32 * j;
+                kbits[j] = (p.keep && live && nt < p.n) ? p.keep[(size_t)m * (size_t)words + (nt >> 5)] : 0xffffffffu;
+            }
+        };
+        auto finish_tile = [&](int s) __attribute__((always_inline)) {
+            const int64_t m = ((int64_t)blockIdx.x + (int64_t)s * gridDim.x) * kStreamRows + m0 + idx;
+            const bool live = m < p.rows;
+            const float inv = 1.0f / rdiv;
+            if (!PACK) {
+                // branch-free but for the store itself: ReLU and keep-bits as selects
+                float *yrow = p.y + (size_t)(live ? m : 0) * (size_t)p.ldy;
+                const bool relu = p.relu != 0;
+                auto act = [&](float a, float bias) __attribute__((always_inline)) {
+                    const float z = __builtin_fmaf(a, inv, bias);  // (acc * inv + bias as one fused multiply-add, as above)
+                    return (relu ? fmaxf(z, 0.0f) : z) * p.scale;
+                };
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int nt = n0 + 32 * j;
+                    const uint32_t bits = kbits[j] >> (4 * kk);
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const int n = nt + 8 * g + 4 * kk;
+                        const floatx4 b4 = *reinterpret_cast<const floatx4 *>(bias_lds + (n & 255));
+                        const uint32_t b = bits >> (8 * g);
+                        floatx4 v;
+                        v.x = act(acc[j][4 * g], b4.x);
+                        v.y = act(acc[j][4 * g + 1], b4.y);
+                        v.z = act(acc[j][4 * g + 2], b4.z);
+                        v.w = act(acc[j][4 * g + 3], b4.w);
+                        v.x = (b & 1u) ? v.x : 0.0f;
+                        v.y = (b & 2u) ? v.y : 0.0f;
+                        v.z = (b & 4u) ? v.z : 0.0f;
+                        v.w = (b & 8u) ? v.w : 0.0f;
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) acc[j][4 * g + r] = 0.0f;
+                        if (live && n < p.n) *reinterpret_cast<floatx4 *>(yrow + n) = v;
+                    }
+                }
+                return;
+            }
+            // PACK: every row keeps only its non-zeros, moved to its front in column order, and a header says where
+            // they belong (per 32 columns the bitmap of the non-zeros and the number of non-zeros in front of them).
+            // Four lanes share a row: two per wave (columns 8g + 4kk + c of each 32-column tile) and the block's two
+            // column halves in two waves; the left half's total reaches the right half through LDS.
+            uint32_t word[4];
+            int count = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int nt = n0 + 32 * j;
+                const uint32_t bits = kbits[j] >> (4 * kk);
+                uint32_t mine = 0;
+                floatx4 b4[4];
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+                    b4[g] = *reinterpret_cast<const floatx4 *>(bias_lds + nt + 8 * g + 4 * kk);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int local = 8 * (r >> 2) + (r & 3);  // + 4 kk: this value's column inside the tile
+                    float v = __builtin_fmaf(acc[j][r], inv, b4[r >> 2][r & 3]);
+                    v = fmaxf(v, 0.0f) * p.scale;
+                    if (!((bits >> local) & 1u) || !live || nt >= p.n) v = 0.0f;
+                    acc[j][r] = v;
+                    mine |= (v > 0.0f ? 1u : 0u) << local;
+                }
+                mine <<= 4 * kk;
+                word[j] = mine | (uint32_t)__shfl_xor((int)mine, 32);
+                count += __popc(word[j]);
+            }
+            if (wc == 0 && kk == 0) row_count[m0 + idx] = count;
+            __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the count is in LDS
+            __builtin_amdgcn_s_barrier();        // (every wave of the block, the loading ones included, meets here)
+            int front = wc == 1 ? row_count[m0 + idx] : 0;
+            if (live) {
+                const int hw = 2 * (p.n / 32);
+                float *yrow = p.y + (size_t)m * (size_t)p.ldy;
+                uint32_t *hrow = p.header + (size_t)m * (size_t)hw;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int nt = n0 + 32 * j;
+                    if (nt >= p.n) continue;
+                    const uint32_t w = word[j];
+                    if (kk == 0) {
+                        hrow[2 * (nt >> 5)] = w;
+                        hrow[2 * (nt >> 5) + 1] = (uint32_t)front;
+                    }
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int local = 8 * (r >> 2) + (r & 3) + 4 * kk;
+                        if ((w >> local) & 1u) yrow[front + __popc(w & ((1u << local) - 1u))] = acc[j][r];
+                    }
+                    front += __popc(w);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[j][r] = 0.0f;
+        };
+
+        // `early` waves multiply chunk q first and then prepare chunk q + 1; the others prepare chunk q, then multiply it
+        const bool early = wave < 4;
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // this wave's share of W and of the bias is in LDS
+        __builtin_amdgcn_s_barrier();
+        int q = 0, sa = 0;  // sa = q % kStreamSlots
+        if (early) {
+            read_convert(0, 0);
+            for (int s = 0; s < my_tiles; ++s) {
+                load_divisors(s);
+                for (int c = 0; c < nk; ++c, ++q) {
+                    multiply();
+                    if (c + 1 == nk) finish_tile(s);
+                    sa = sa + 1 == kStreamSlots ? 0 : sa + 1;
+                    if (q + 1 < total) read_convert(sa, c + 1 == nk ? 0 : c + 1);
+                    __builtin_amdgcn_s_barrier();
+                }
+            }
+        } else {
+            for (int s = 0; s < my_tiles; ++s) {
+                load_divisors(s);
+                for (int c = 0; c < nk; ++c, ++q) {
+                    read_convert(sa, c);
+                    sa = sa + 1 == kStreamSlots ? 0 : sa + 1;
+                    multiply();
+                    if (c + 1 == nk) finish_tile(s);
+                    __builtin_amdgcn_s_barrier();
+                }
+            }
+        }
+        for (; q < padded; ++q) __builtin_amdgcn_s_barrier();
+    } else {
+        // ---- four waves stream A through their registers: two 16-byte pieces of every chunk per thread ----
+        const int pt = tid - 512;
+        int a_row[2], a_piece[2];
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const int u = e * 256 + pt;  // 16-byte unit of the chunk, also its place in the slot: row u / 4
+            a_row[e] = u >> 2;
+            a_piece[e] = (u & 3) ^ ((a_row[e] >> 2) & 3);
+        }
+        const int a_dst = pt * 16;
+        int a_tile = 0, a_c = 0, a_q = 0;  // the next chunk to request
+        const float *a_ptr[2];
+        auto enter_tile = [&]() __attribute__((always_inline)) {
+            const int64_t first = ((int64_t)blockIdx.x + (int64_t)a_tile * gridDim.x) * kStreamRows;
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                int64_t r = first + a_row[e];
+                if (r >= p.rows) r = p.rows - 1;  // rows past the end read the last row; their results are never stored
+                a_ptr[e] = p.a + (size_t)r * (size_t)p.lda + 4 * a_piece[e];
+            }
+        };
+        enter_tile();
+        floatx4 areg[kStreamDepth][2];
+        auto fetch = [&](auto set) __attribute__((always_inline)) {
+            constexpr int S = decltype(set)::value;
+#pragma unroll
+            for (int e = 0; e < 2; ++e) areg[S][e] = __builtin_nontemporal_load(reinterpret_cast<const floatx4 *>(a_ptr[e] + kChunk * a_c));
+            ++a_q;
+            if (a_q < total) {  // past the end: the same chunk again, never used
+                if (++a_c == nk) {
+                    a_c = 0;
+                    ++a_tile;
+                    enter_tile();
+                }
+            }
+        };
+        auto store = [&](auto set, int slot) __attribute__((always_inline)) {
+            constexpr int S = decltype(set)::value;
+            char *dst = aring + slot * kStreamASlot + a_dst;
+#pragma unroll
+            for (int e = 0; e < 2; ++e) *reinterpret_cast<floatx4 *>(dst + e * 4096) = areg[S][e];
+        };
+        // chunks 0 .. kStreamDepth-1 into registers; chunks 0 and 1 into LDS and their sets refilled
+        static_for<kStreamDepth>([&](auto set) __attribute__((always_inline)) { fetch(set); });
+        store(std::integral_constant<int, 0>{}, 0);
+        fetch(std::integral_constant<int, 0>{});
+        store(std::integral_constant<int, 1>{}, 1);
+        fetch(std::integral_constant<int, 1>{});
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's LDS writes (A, W, bias) have landed
+        __builtin_amdgcn_s_barrier();
+        // iteration q: chunk q + 2 (set (q + 2) % kStreamDepth) goes to slot (q + 2) % kStreamSlots; the set takes chunk
+        // q + 2 + kStreamDepth
+        int slot = 2, c = 0;
+        for (int q = 0; q < padded; q += kStreamDepth) {
+            static_for<kStreamDepth>([&](auto ph) __attribute__((always_inline)) {
+                constexpr int S = (decltype(ph)::value + 2) % kStreamDepth;
+                store(std::integral_constant<int, S>{}, slot);
+                fetch(std::integral_constant<int, S>{});
+                slot = slot + 1 == kStreamSlots ? 0 : slot + 1;
+                if (PACK && q + decltype(ph)::value < total && ++c == nk) {
+                    c = 0;
+                    __builtin_amdgcn_s_barrier();  // the multiplying waves' exchange of row counts
+                }
+                __builtin_amdgcn_s_waitcnt(0xc07f);
+                __builtin_amdgcn_s_barrier();
+            });
+        }
+    }
+}
+
+template <bool PACK>
+int launch_linear_stream(const LinearArgs &p, hipStream_t st) {
+    const size_t smem = stream_smem_bytes(p.k, PACK);
+    GNNAGG_HIP(allow_lds(reinterpret_cast<const void *>(&linear_stream_bf16_kernel<PACK>), smem));
+    int dev = 0, cus = 0;
+    GNNAGG_HIP(hipGetDevice(&dev));
+    GNNAGG_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    const int64_t tiles = (p.rows + kStreamRows - 1) / kStreamRows;
+    const int64_t resident = (int64_t)(cus > 0 ? cus : 256);  // one block of twelve waves per compute unit
+    const unsigned blocks = (unsigned)(tiles < resident ? tiles : resident);
+    hipLaunchKernelGGL((linear_stream_bf16_kernel<PACK>), dim3(blocks), dim3(768), smem, st, p);
+    GNNAGG_HIP(hipGetLastError());
+    return GNNAGG_OK;
+}
+
 template <int WM, int WN, bool BF16, bool PACK, bool SPLIT>
 int launch_linear(const LinearArgs &p, hipStream_t st) {
     using S = LinearShape<WM, WN>;
@@ -487,6 +837,12 @@ int launch_linear(const LinearArgs &p, hipStream_t st) {
 
 template <bool BF16, bool SPLIT>
 int dispatch_linear(const LinearArgs &p, hipStream_t st) {
+    if constexpr (BF16) {
+        // the kernel with W resident in LDS: K * 512 bytes of it, and an int chunk counter
+        const int64_t tiles = (p.rows + kStreamRows - 1) / kStreamRows;
+        if (p.k <= kStreamMaxK && tiles * (p.k / kChunk) < (int64_t(1) << 30))
+            return p.header ? launch_linear_stream<true>(p, st) : launch_linear_stream<false>(p, st);
+    }
     if (p.header) {  // packed output: widths 32, 64, 128, 256
         switch ((p.n + 63) / 64) {
             case 1: return launch_linear<2, 1, BF16, true, SPLIT>(p, st);
