@@ -516,3 +516,33 @@ def test_train_step_can_send_every_node_through_the_last_layer(model_kind):
     assert np.isclose(results[0][0], results[1][0], rtol=1e-6)
     for a, b in zip(results[0][1], results[1][1]):
         assert float((a - b).abs().max()) <= 1e-5 * float(b.abs().max()) + 1e-12
+
+
+@pytest.mark.parametrize("form", [gcn.FP32, gcn.BF16, gcn.BF16X3])
+@pytest.mark.parametrize("rows,k,n", [(70_001, 48, 64), (66_000, 256, 256), (1, 16, 32), (129, 32, 128)])
+def test_layer_kernels_walk_several_tiles_per_block(form, rows, k, n):
+    """Rows beyond one tile per resident block (256 compute units x 128-row tiles = 32 768 rows, twice that for the
+    kernels with two blocks per unit): every block walks several tiles, the chunk stream crosses tile boundaries, and
+    K = 48 leaves a chunk count that is no multiple of the loading waves' unroll.  The dense result is checked against
+    fp64 on the operands as the form sees them; the packed result must be the dense one bit for bit."""
+    gen = torch.Generator(device="cuda").manual_seed(rows + k + n)
+    x = torch.randn(rows, k, device="cuda", generator=gen)
+    w = torch.randn(k, n, device="cuda", generator=gen) / k ** 0.5
+    bias = torch.randn(n, device="cuda", generator=gen)
+    div = torch.randint(1, 9, (rows,), device="cuda", generator=gen).float()
+    keep = torch.rand(rows, n, device="cuda", generator=gen) >= 0.5
+    bits = gcn.pack_keep_mask(keep)
+    y = gcn._FusedLayer.apply(x, w, bias, bits, 2.0, div, True, form)
+    xs, ws = (x.bfloat16().double(), w.bfloat16().double()) if form == gcn.BF16 else (x.double(), w.double())
+    ref = torch.relu((xs @ ws) / div.double().view(-1, 1) + bias.double()) * keep * 2.0
+    scale = (xs.abs() @ ws.abs() + bias.double().abs()).clamp(min=1.0) * 2.0
+    assert bool(((y.double() - ref).abs() <= 1e-5 * scale).all())
+    # the last rows and the first rows of the second round of tiles, where a wrong tile walk would show
+    for r in {0, rows - 1, min(rows - 1, 32768), min(rows - 1, 65536)}:
+        assert bool(((y[r].double() - ref[r]).abs() <= 1e-5 * scale[r]).all()), r
+    values, header = gcn._FusedLayerPacked.apply(x, w, bias, bits, 2.0, div, form)
+    from gnn_benchmark_amd import packed
+    assert torch.equal(packed.unpack(values, header), y)
+    # no bias, no mask, no divisor, no ReLU: the bare product (what the input-gradient product runs)
+    bare = gcn._fused_product(x, w, None, None, None, 1.0, False, form)
+    assert bool(((bare.double() - xs @ ws).abs() <= 1e-5 * (xs.abs() @ ws.abs()).clamp(min=1.0)).all())
