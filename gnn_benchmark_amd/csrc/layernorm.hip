@@ -300,7 +300,7 @@ extern "C" int gnnagg_dropout_layernorm_relu_backward_f32(const float *grad_y, i
         return fail(GNNAGG_ERR_UNSUPPORTED, "the fused LayerNorm pass takes widths that are multiples of 4 up to 1024 "
                     "(got %lld)", (long long)feat);
     if (rows == 0) return GNNAGG_OK;
-    GNNAGG_REQUIRE(grad_y && z && gamma && beta && grad_z, "null grad_y/z/gamma/beta/grad_z");
+    GNNAGG_REQUIRE(grad_y && z && gamma && beta && grad_z && partial, "null grad_y/z/gamma/beta/grad_z/partial");
     GNNAGG_REQUIRE(grad_stride >= feat && grad_stride % 4 == 0, "gradient row stride %lld must be a multiple of 4 and "
                    "at least the width", (long long)grad_stride);
     GNNAGG_REQUIRE(aligned16(grad_y) && aligned16(z) && aligned16(gamma) && aligned16(beta) && aligned16(grad_z) &&

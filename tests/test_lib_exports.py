@@ -51,6 +51,9 @@ def test_argument_errors_without_gpu_work():
     assert L.gnnagg_memory_probe(9, None, None, None, 4, 128, 1, None) == _lib.ERR_INVALID
     assert L.gnnagg_memory_probe(0, None, None, None, 0, 128, 1, None) == _lib.OK
     assert L.gnnagg_issue_probe(-1, 0, None, None) == _lib.ERR_INVALID
+    # a null partial-sums workspace is refused on the host, not dereferenced on the device (fake non-null operands)
+    assert L.gnnagg_dropout_layernorm_relu_backward_f32(256, 128, 256, None, 1.0, 256, 256, 1e-5, 256, None, 4, 128, None) == _lib.ERR_INVALID
+    assert b"partial" in L.gnnagg_last_error()
     assert L.gnnagg_issue_probe(1, 1, None, None) == _lib.ERR_INVALID   # null sink
 
 
