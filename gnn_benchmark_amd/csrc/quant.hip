@@ -186,15 +186,15 @@ __global__ __launch_bounds__(256) void quantize_segments_kernel(const float *__r
 #pragma unroll
             for (int u = 0; u < GPL; ++u)
 #pragma unroll
-                for (int k = 0; k < EPB; ++k)
-                    if (k < sl.rg[u].count) {
-                        const float *row = x + (size_t)(sl.rg[u].first + k) * (size_t)feat;
+                for (int k = 0; k < EPB; ++k) {
+                    // a row the group does not have reads row 0 instead (never used): loads without branches
+                    const float *row = x + (size_t)(k < sl.rg[u].count ? sl.rg[u].first + k : 0) * (size_t)feat;
 #pragma unroll
-                        for (int j = 0; j < KEEP; ++j) {
-                            const int v = l + G * j;
-                            if (v < nvec) sl.held[u][k][j] = QVec<VEC>::load(row + (size_t)v * VEC);
-                        }
+                    for (int j = 0; j < KEEP; ++j) {
+                        const int v = l + G * j;
+                        if (v < nvec) sl.held[u][k][j] = QVec<VEC>::load(row + (size_t)v * VEC);
                     }
+                }
         }
     };
     auto process = [&](const Slice &sl) {
@@ -335,8 +335,8 @@ __global__ __launch_bounds__(256) void dequantize_segments_kernel(const uint8_t 
     for (int v = l; v < nvec; v += G) {
         uint32_t byte[GPL][VEC];
 #pragma unroll
-        for (int u = 0; u < GPL; ++u)
-            if (rg[u].count > 0) QVec<VEC>::load_bytes(packed + (size_t)(g0 + u) * (size_t)feat + (size_t)v * VEC, byte[u]);
+        for (int u = 0; u < GPL; ++u)  // (a group past the end reads packed row 0 instead: loads without branches)
+            QVec<VEC>::load_bytes(packed + (size_t)(rg[u].count > 0 ? g0 + u : 0) * (size_t)feat + (size_t)v * VEC, byte[u]);
 #pragma unroll
         for (int u = 0; u < GPL; ++u)
 #pragma unroll
