@@ -74,15 +74,16 @@ __device__ __forceinline__ uint32_t quantize_one(float x, float zp, float scale)
 
 // The same value without an IEEE division per element.  t = d * rcp(scale) lies within 2.4e-7 * |t|
 // of the correctly rounded quotient fl(d / scale) (v_rcp_f32 is good to 1 ulp, the product adds
-// half an ulp, fl() itself another half).  Unless t comes closer than that to a half-integer, t
-// and fl(d / scale) round to the same integer; the rare close calls (and anything huge or not
-// finite) take the exact division.
+// half an ulp, fl() itself another half).  For |t| < 512 that is less than 1.3e-4, so unless t comes
+// closer than 2e-4 to a half-integer, t and fl(d / scale) round to the same integer; the rare close
+// calls, and anything large or not finite (every comparison with a NaN is false), take the exact
+// division.  (Codes are at most 255, so a larger |t| only arises from non-finite or overflowing input.)
 __device__ __forceinline__ uint32_t quantize_one_fast(float x, float zp, float scale, float inv_scale) {
     const float d = __fsub_rn(x, zp);
     const float t = __fmul_rn(d, inv_scale);
     float k = rintf(t);
-    const float gap = 0.5f - fabsf(__fsub_rn(t, k));
-    if (!(fabsf(t) < 1.0e6f) || gap <= 4.0e-7f * fabsf(t) + 1.0e-30f) k = rintf(__fdiv_rn(d, scale));
+    const bool safe = (fabsf(__fsub_rn(t, k)) < 0.4998f) & (fabsf(t) < 512.0f);
+    if (!safe) k = rintf(__fdiv_rn(d, scale));
     return (uint32_t)(int)k;
 }
 
