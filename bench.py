@@ -46,6 +46,9 @@ MEASURED_TRAFFIC = {
     ("c2", "A@X", 100): (5.68207e+10, 1.01207e+09, _P), ("c2", "A^T@G", 100): (5.68207e+10, 1.01207e+09, _P),
     ("c2", "A@X", 128): (5.71924e+10, 1.25440e+09, _P), ("c2", "A^T@G", 128): (5.71924e+10, 1.25440e+09, _P),
     ("c2", "A@X", 256): (1.18675e+11, 2.50880e+09, _P), ("c2", "A^T@G", 256): (1.18675e+11, 2.50880e+09, _P),
+    ("c2", "A@X", 172): (9.10710e+10, 1.73200e+09, _P), ("c2", "A^T@G", 172): (9.10710e+10, 1.73200e+09, _P),
+    ("c2", "A@X", 40): (2.72050e+10, 4.00000e+08, _P), ("c2", "A^T@G", 40): (2.72050e+10, 4.00000e+08, _P),
+    ("c2", "A@X", 47): (3.31340e+10, 5.38000e+08, _P), ("c2", "A^T@G", 47): (3.31340e+10, 5.38000e+08, _P),
     # (c3: the block-per-row kernel's share, 0.8 / 0.3 GB, is included in the forward figures)
     ("c3", "A@X", 602): (2.94247e+11, 5.82812e+08, _P), ("c3", "A^T@G", 602): (2.85891e+11, 5.91882e+08, _P),
     ("c3", "A@X", 256): (1.18438e+11, 2.38592e+08, _P), ("c3", "A^T@G", 256): (1.12242e+11, 2.38592e+08, _P),
