@@ -99,6 +99,16 @@ def _bf16_wire(graph) -> bool:
     return True
 
 
+def _bf16_in_the_products(graph, feats_or_grad, feat_len: int) -> bool:
+    """Whether the products next to a 16-bit exchange read and write the bf16 staging buffers themselves (the
+    default; ``graph.fuse_bf16_staging = False`` keeps the two tensor copies of communicator.py:128,137 as separate
+    passes).  The bits are the same either way: the copy rounds the fp32 sum to nearest even, widening is exact."""
+    if getattr(graph, "fuse_bf16_staging", True) is False or feat_len % 4 != 0:
+        return False
+    t = getattr(feats_or_grad, "feat", feats_or_grad)
+    return isinstance(t, torch.Tensor) and t.dtype == torch.float32
+
+
 def _convert(src: torch.Tensor, dst: torch.Tensor) -> None:
     """fp32 -> bf16 (round to nearest even) or bf16 -> fp32: the two ``copy_`` calls around the
     16-bit exchange (communicator.py:128, :137)."""
@@ -233,15 +243,17 @@ def _forward(ctx, graph, feats, layer, num_bits: int, is_pre_delay: bool, is_tra
     comm_handle = None
     send_buf = graph.comm_buf.send_buf
 
+    half_fused = half and isinstance(feats, _DenseFeatures) and _bf16_in_the_products(graph, feats, feat_len)
     if exchange is not None:
-        if is_pre_delay:  # pre-aggregation: send_buf = A_to @ X
-            feats.product(graph.adj_t_pre_post_aggr_to, send_buf, False)
+        if is_pre_delay:  # pre-aggregation: send_buf = A_to @ X (straight into the bf16 staging rows when they travel)
+            feats.product(graph.adj_t_pre_post_aggr_to, graph.comm_buf.send_buf_fp16 if half_fused else send_buf, False)
         else:  # raw boundary rows
             feats.gather(graph.idx_nodes_send_to_others, send_buf)
         if quantized:
             comm_handle = _quantize_and_exchange(graph, num_bits, f"forward{layer}", "forward")
         elif half:
-            _convert(send_buf, graph.comm_buf.send_buf_fp16)
+            if not (half_fused and is_pre_delay):
+                _convert(send_buf, graph.comm_buf.send_buf_fp16)
             comm_handle = graph.exchange_bf16(graph.comm_splits, graph.comm_buf, f"forward{layer}", "forward")
         else:
             comm_handle = exchange(graph.comm_splits, graph.comm_buf, f"forward{layer}", "forward")
@@ -258,10 +270,12 @@ def _forward(ctx, graph, feats, layer, num_bits: int, is_pre_delay: bool, is_tra
     fused = quantized and _fused_dequantize(graph, feat_len) and out.stride(0) % 4 == 0
     if quantized and not fused:
         _dequantize_received(graph, num_bits, "forward")
-    if half:
+    half_fused = half_fused and out.stride(0) % 4 == 0
+    if half and not half_fused:
         _convert(graph.comm_buf.recv_buf_fp16, graph.comm_buf.recv_buf)
 
-    remote_nodes_feat = graph.comm_buf.recv_buf
+    # (fused: the received bf16 rows are gathered as they are; recv_buf is not written)
+    remote_nodes_feat = graph.comm_buf.recv_buf_fp16 if half_fused else graph.comm_buf.recv_buf
     if exchange is not None and remote_nodes_feat.size(0) != 0:
         adj = graph.adj_t_pre_post_aggr_from if is_pre_delay else graph.remote_adj_t  # post-aggregation / raw halo
         if fused:
@@ -397,7 +411,10 @@ def _backward(ctx, local_out_grad, out=None, accumulate: bool = False):
     # a caller that knows the gradient to be zero outside a set of rows (a loss that scores only the training nodes,
     # for the last layer) declares it in graph.backward_row_support[layer]: the products below then skip those rows
     support = (getattr(graph, "backward_row_support", None) or {}).get(ctx.layer)
-    remote_nodes_grad_buf = graph.comm_buf.recv_buf
+    half = exchange is not None and num_bits == 16 and _bf16_wire(graph)
+    half_fused = half and not quantized and _bf16_in_the_products(graph, local_out_grad, feat_len)
+    # the outgoing halo gradients: straight into the bf16 staging rows when they travel as bf16
+    remote_nodes_grad_buf = graph.comm_buf.recv_buf_fp16 if half_fused else graph.comm_buf.recv_buf
     if remote_nodes_grad_buf.size(0) != 0:
         if support is not None:
             SPMM_forward(support.remote_T, local_out_grad, remote_nodes_grad_buf, accumulate=False)
@@ -406,12 +423,12 @@ def _backward(ctx, local_out_grad, out=None, accumulate: bool = False):
         else:
             SPMM_backward(graph.remote_adj_t, local_out_grad, remote_nodes_grad_buf, accumulate=False)
 
-    half = exchange is not None and num_bits == 16 and _bf16_wire(graph)
     comm_handle = None
     if quantized:
         comm_handle = _quantize_and_exchange(graph, num_bits, layer, "backward")
     elif half:  # the buffers swap roles on the way back (communicator.py:121-126)
-        _convert(remote_nodes_grad_buf, graph.comm_buf.recv_buf_fp16)
+        if not half_fused:
+            _convert(remote_nodes_grad_buf, graph.comm_buf.recv_buf_fp16)
         comm_handle = graph.exchange_bf16(graph.comm_splits, graph.comm_buf, layer, "backward")
     elif exchange is not None:
         comm_handle = exchange(graph.comm_splits, graph.comm_buf, layer, "backward")
@@ -433,10 +450,11 @@ def _backward(ctx, local_out_grad, out=None, accumulate: bool = False):
     fused = quantized and _fused_dequantize(graph, feat_len) and local_nodes_grad.stride(0) % 4 == 0
     if quantized and not fused:
         _dequantize_received(graph, num_bits, "backward")
-    if half:
+    half_fused = half_fused and local_nodes_grad.stride(0) % 4 == 0
+    if half and not half_fused:
         _convert(graph.comm_buf.send_buf_fp16, graph.comm_buf.send_buf)
 
-    local_nodes_grad_buf = graph.comm_buf.send_buf
+    local_nodes_grad_buf = graph.comm_buf.send_buf_fp16 if half_fused else graph.comm_buf.send_buf
     if exchange is not None and local_nodes_grad_buf.size(0) != 0:
         qbuf = graph.comm_buf_for_quantization
         if is_pre_delay:

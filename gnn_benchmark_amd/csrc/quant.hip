@@ -82,7 +82,7 @@ __device__ __forceinline__ uint32_t quantize_one_fast(float x, float zp, float s
     const float d = __fsub_rn(x, zp);
     const float t = __fmul_rn(d, inv_scale);
     float k = rintf(t);
-    const bool safe = (fabsf(__fsub_rn(t, k)) < 0.4998f) & (fabsf(t) < 512.0f);
+    const bool safe = fabsf(__fsub_rn(t, k)) < 0.4998f && fabsf(t) < 512.0f;
     if (!safe) k = rintf(__fdiv_rn(d, scale));
     return (uint32_t)(int)k;
 }

@@ -740,6 +740,56 @@ extern "C" int gnnagg_plan_spmm_quantized_f32(gnnagg_plan *plan, const float *va
     return GNNAGG_OK;
 }
 
+extern "C" int gnnagg_plan_spmm_bf16_f32(gnnagg_plan *plan, const float *value, const void *mat, int mat_is_bf16,
+                                         int64_t mat_stride, void *out, int out_is_bf16, int64_t out_stride,
+                                         int64_t feat, int accumulate, void *stream) {
+    GNNAGG_REQUIRE(plan, "null plan");
+    GNNAGG_REQUIRE(feat >= 0, "negative feature width");
+    GNNAGG_REQUIRE(mat_is_bf16 || out_is_bf16, "neither operand is bf16: use gnnagg_plan_spmm_strided_f32");
+    if (plan->rows == 0 || feat == 0) return GNNAGG_OK;
+    if (int rc = check_feat(feat)) return rc;
+    if (feat % 4 != 0)
+        return fail(GNNAGG_ERR_UNSUPPORTED, "bf16 rows need a width that is a multiple of 4 (got %lld)", (long long)feat);
+    if (out_is_bf16 && accumulate)
+        return fail(GNNAGG_ERR_UNSUPPORTED, "bf16 result rows are written, not accumulated onto (accumulate must be 0)");
+    GNNAGG_REQUIRE(out, "null out");
+    GNNAGG_REQUIRE(plan->nnz == 0 || (value && mat), "null value/mat");
+    GNNAGG_REQUIRE(mat_stride >= feat && mat_stride % 4 == 0 && mat_stride < (int64_t(1) << 31) && out_stride >= feat &&
+                       out_stride % 4 == 0 && out_stride < (int64_t(1) << 31),
+                   "row strides (%lld, %lld) must be multiples of 4, at least the width and below 2^31",
+                   (long long)mat_stride, (long long)out_stride);
+    // a lane moves four values at a time: 8 bytes of a bf16 row, 16 of an fp32 row
+    GNNAGG_REQUIRE((reinterpret_cast<uintptr_t>(mat) & (mat_is_bf16 ? 7 : 15)) == 0 &&
+                       (reinterpret_cast<uintptr_t>(out) & (out_is_bf16 ? 7 : 15)) == 0,
+                   "bf16 rows must be 8-byte aligned, fp32 rows 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const Regions regions{plan->rows_per_group, plan->short_rows_per_group,
+                          plan->nshort + (accumulate ? 0 : plan->nempty)};
+    for (int64_t f_base = 0; f_base < feat;) {
+        const Shape s = pick_shape(4, feat - f_base);
+        SpmmArgs a{};
+        a.task = plan->task;  // every row runs in the lane-group kernel, the very longest included
+        a.col = plan->col32;
+        a.val = value;
+        a.x = static_cast<const float *>(mat);
+        a.ldx = (int)mat_stride;
+        a.dst = static_cast<float *>(out);
+        a.ldd = (int)out_stride;
+        a.dst_bf16 = out_is_bf16 ? 1 : 0;
+        a.feat = (int)feat;
+        a.f_base = (int)f_base;
+        a.accumulate = accumulate;
+        a.ntasks = plan->rows - (accumulate ? plan->nempty : 0);
+        a.head_tasks = plan->nlong;
+        if (mat_is_bf16)
+            GNNAGG_HIP((dispatch_shape<4, int32_t, kRowsPlanned, kSrcBf16>(s, a, regions, st)));
+        else
+            GNNAGG_HIP((dispatch_shape<4, int32_t, kRowsPlanned, kSrcDense>(s, a, regions, st)));
+        f_base += s.width();
+    }
+    return GNNAGG_OK;
+}
+
 extern "C" int gnnagg_plan_profile(gnnagg_plan *plan, int enable) {
     GNNAGG_REQUIRE(plan, "null plan");
     if (enable) {

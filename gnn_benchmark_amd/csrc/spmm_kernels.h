@@ -158,6 +158,8 @@ struct SpmmArgs {
     int ldx, ldd;             // row strides of x and dst in floats; 0 stands for F (rows back to back)
     int f_base;               // first feature handled by this launch
     int accumulate;           // start every row from dst (1) or from 0 (0)
+    int dst_bf16;             // 1: dst points at bf16 rows (ldd counts 16-bit values), rounded on the way out;
+                              // overwriting launches with 16-byte vector lanes only
     int tasks_per_block;      // tasks handled by one block of the middle region
     int64_t head_tasks;       // the first head_tasks tasks (the longest rows) get one lane group each
     int head_blocks;          // = ceil(head_tasks / groups per block)
@@ -172,8 +174,16 @@ struct SpmmArgs {
 enum SourceKind : int {
     kSrcDense = 0,   // x[col, :] is a dense fp32 row
     kSrcPacked = 1,  // x[col, :] holds the row's non-zero values at its front, hdr[col, :] says which
-    kSrcQuant = 2    // row col is held quantised: qdata / qparams / qcode (boundary-buffer codec layout)
+    kSrcQuant = 2,   // row col is held quantised: qdata / qparams / qcode (boundary-buffer codec layout)
+    kSrcBf16 = 3     // x[col, :] is a bf16 row (x points at 16-bit values, ldx counts them): widened in the gather
 };
+
+// fp32 -> bf16 as the tensor copy does it: round to nearest even, NaN -> 0x7FC0
+__device__ __forceinline__ unsigned short bf16_bits(float x) {
+    const uint32_t u = __float_as_uint(x);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)0x7fc0;
+    return (unsigned short)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
 
 typedef float f32x4_unaligned __attribute__((ext_vector_type(4), aligned(4)));
 
@@ -283,6 +293,27 @@ __device__ __forceinline__ void gather_fma(FVec<VEC> (&acc)[NCH], IdxT c_l, floa
                 xv[u][k].d.y = __builtin_fmaf((float)((w >> 8) & mask), sc[u], zp[u]);
                 xv[u][k].d.z = __builtin_fmaf((float)((w >> 16) & mask), sc[u], zp[u]);
                 xv[u][k].d.w = __builtin_fmaf((float)((w >> 24) & mask), sc[u], zp[u]);
+            }
+        }
+    } else if constexpr (SRC == kSrcBf16) {
+        static_assert(SRC != kSrcBf16 || VEC == 4, "bf16 rows: four values (8 bytes) per lane and load");
+        // a bf16 value is the upper half of the fp32 value it stands for: widening is exact
+        const unsigned short *xb = reinterpret_cast<const unsigned short *>(x);
+        uint2 raw[UU][NCH];
+#pragma unroll
+        for (int u = 0; u < UU; ++u) {
+#pragma unroll
+            for (int k = 0; k < NCH; ++k)
+                raw[u][k] = *reinterpret_cast<const uint2 *>(xb + (size_t)cc[u] * (size_t)ldx + foff[k]);
+        }
+#pragma unroll
+        for (int u = 0; u < UU; ++u) {
+#pragma unroll
+            for (int k = 0; k < NCH; ++k) {
+                xv[u][k].d.x = __uint_as_float(raw[u][k].x << 16);
+                xv[u][k].d.y = __uint_as_float(raw[u][k].x & 0xffff0000u);
+                xv[u][k].d.z = __uint_as_float(raw[u][k].y << 16);
+                xv[u][k].d.w = __uint_as_float(raw[u][k].y & 0xffff0000u);
             }
         }
     } else {
@@ -454,9 +485,30 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
         }
 
         if (row_done) {
+            if constexpr (VEC == 4) {
+                if (a.dst_bf16) {  // the result rows are bf16 (overwriting only): rounded once, here
+                    unsigned short *d16 = reinterpret_cast<unsigned short *>(a.dst) + (size_t)row * (size_t)ldd;
 #pragma unroll
-            for (int k = 0; k < NCH; ++k) {
-                if (fok[k]) acc[k].store_stream(dst + foff[k]);
+                    for (int k = 0; k < NCH; ++k) {
+                        if (fok[k]) {
+                            typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+                            u32x2 r;
+                            r.x = (uint32_t)bf16_bits(acc[k].d.x) | ((uint32_t)bf16_bits(acc[k].d.y) << 16);
+                            r.y = (uint32_t)bf16_bits(acc[k].d.z) | ((uint32_t)bf16_bits(acc[k].d.w) << 16);
+                            __builtin_nontemporal_store(r, reinterpret_cast<u32x2 *>(d16 + foff[k]));
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int k = 0; k < NCH; ++k) {
+                        if (fok[k]) acc[k].store_stream(dst + foff[k]);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int k = 0; k < NCH; ++k) {
+                    if (fok[k]) acc[k].store_stream(dst + foff[k]);
+                }
             }
             if (!more) break;
             dst = a.dst + (size_t)nrow * (size_t)ldd;

@@ -67,6 +67,8 @@ class SpmmPlan:
         tensors (unit stride along the features, any row stride): they are used in place."""
         if not (value.is_cuda and mat.is_cuda and out.is_cuda):
             raise RuntimeError("value, mat and out must be GPU (HIP) tensors; there is no CPU path")
+        if torch.bfloat16 in (mat.dtype, out.dtype):
+            return self._spmm_bf16(value, mat, out, accumulate)
         if value.dtype != torch.float32 or mat.dtype != torch.float32 or out.dtype != torch.float32:
             raise RuntimeError("Input mismatch: value/mat/out must be float32")
         if mat.dim() != 2 or out.dim() != 2 or not _rows_are_dense(out):
@@ -86,6 +88,27 @@ class SpmmPlan:
                 _lib.check(_lib.lib().gnnagg_plan_spmm_strided_f32(
                     self._handle, _lib.ptr(value), _lib.ptr(mat), _row_stride(mat), _lib.ptr(out), _row_stride(out),
                     feat, 1 if accumulate else 0, _lib.current_stream(self.device)))
+        return out
+
+    def _spmm_bf16(self, value, mat, out, accumulate):
+        """The product with bf16 rows on either side (the staging buffers of a 16-bit exchange): a bf16 ``mat`` is
+        widened in the gather, a bf16 ``out`` receives the fp32 sums rounded to nearest even -- the same bits as the
+        tensor copies around an fp32 product, without the copies."""
+        ok = (torch.float32, torch.bfloat16)
+        if value.dtype != torch.float32 or mat.dtype not in ok or out.dtype not in ok:
+            raise RuntimeError("Input mismatch: value must be float32, mat/out float32 or bfloat16")
+        if mat.dim() != 2 or out.dim() != 2 or not _rows_are_dense(out) or not _rows_are_dense(mat):
+            raise RuntimeError("Input mismatch: mat/out must be 2-D with contiguous rows")
+        if value.numel() != self.nnz or mat.size(0) < self.cols or out.size(0) < self.rows or out.size(1) != mat.size(1):
+            raise RuntimeError("Input mismatch: operand shapes do not match the planned matrix")
+        if accumulate and out.dtype == torch.bfloat16:
+            raise RuntimeError("Input mismatch: a bfloat16 result is written, not accumulated onto")
+        feat = mat.size(1)
+        with torch.cuda.device(self.device):
+            _lib.check(_lib.lib().gnnagg_plan_spmm_bf16_f32(
+                self._handle, _lib.ptr(value.contiguous()), _lib.ptr(mat), 1 if mat.dtype == torch.bfloat16 else 0,
+                _row_stride(mat), _lib.ptr(out), 1 if out.dtype == torch.bfloat16 else 0, _row_stride(out), feat,
+                1 if accumulate else 0, _lib.current_stream(self.device)))
         return out
 
     def __del__(self):

@@ -16,7 +16,10 @@ from .sparse_tensor import SparseTensor, _row_stride, _rows_are_dense
 
 
 def _as_f32(value: torch.Tensor, other: torch.Tensor) -> torch.Tensor:
-    # reference: value = value.to(other.dtype) (spmm_kernel.py:59-60)
+    # reference: value = value.to(other.dtype) (spmm_kernel.py:59-60); the values stay fp32 beside bf16 rows (the staging
+    # buffers of a 16-bit exchange, which the plan widens / rounds itself)
+    if other.dtype == torch.bfloat16:
+        return value if value.dtype == torch.float32 else value.float()
     return value if value.dtype == other.dtype else value.to(other.dtype)
 
 

@@ -425,6 +425,20 @@ int gnnagg_dequantize_segments_f32(const uint8_t *packed, const float *params, f
 int gnnagg_plan_spmm_quantized_f32(gnnagg_plan *plan, const float *value, const uint8_t *packed, const float *params,
                                    const int32_t *row_code, float *out, int64_t out_stride, int64_t feat, int bits,
                                    int accumulate, void *stream);
+
+/* The pre- and post-aggregation of a 16-bit exchange (communicator.py:111-137) without the two tensor copies around
+ * it: gnnagg_plan_spmm_strided_f32 whose dense operand rows and / or result rows are bf16.
+ *   mat_is_bf16: row c of the operand is mat + c * mat_stride 16-bit values, widened in the gather (exact), so the
+ *                result equals recv_buf.copy_(recv_buf_fp16) followed by the fp32 product, bit for bit
+ *                (model/layers/aggregator.py:98-104 behind communicator.py:137);
+ *   out_is_bf16: row r of the result is out + r * out_stride 16-bit values, each the fp32 sum rounded to nearest even
+ *                (NaN -> 0x7FC0), i.e. what send_buf_fp16.copy_(send_buf) stores behind the fp32 product
+ *                (aggregator.py:47-49, communicator.py:128); accumulate must be 0.
+ * An operand that is not bf16 is fp32 as everywhere else.  feat and both strides multiples of 4; bf16 rows 8-byte
+ * aligned, fp32 rows 16-byte aligned.  Allocates nothing, no host synchronisation. */
+int gnnagg_plan_spmm_bf16_f32(gnnagg_plan *plan, const float *value, const void *mat, int mat_is_bf16,
+                              int64_t mat_stride, void *out, int out_is_bf16, int64_t out_stride, int64_t feat,
+                              int accumulate, void *stream);
 int gnnagg_quantize_mixed_f32(const float *x, uint8_t *data, const int64_t *feat_range, float *params, int64_t rows,
                               int64_t feat, int32_t *bad_width, void *stream);
 int gnnagg_dequantize_mixed_f32(const uint8_t *data, const int64_t *feat_range, const float *params, float *out,

@@ -401,11 +401,14 @@ class PlayedBf16Exchange:
         return None
 
 
+@pytest.mark.parametrize("fused", [True, False])
 @pytest.mark.parametrize("seed,sizes", [(0, (300, 450, 250)), (1, (600, 1, 400, 330))])
-def test_bf16_exchange_world_matches_oracle(seed, sizes):
+def test_bf16_exchange_world_matches_oracle(seed, sizes, fused):
     """Boundary rows travelling as bf16 (num_bits=16, communicator.py:111-137): what every rank
     stages for sending equals the oracle's rows rounded to bf16 bit for bit, and output and gradient
-    equal the oracle pipeline fed with the rounded rows."""
+    equal the oracle pipeline fed with the rounded rows -- with the two tensor copies around the exchange as passes
+    of their own (``fuse_bf16_staging = False``) and with the products reading and writing the bf16 rows themselves
+    (the default)."""
     from oracle import quantization as oq
 
     w = World(seed, sizes, mean_deg=8.0)
@@ -428,11 +431,17 @@ def test_bf16_exchange_world_matches_oracle(seed, sizes):
         gr, o = graphs[r], oracle_ranks[r]
         gr.exchange = lambda *a: (_ for _ in ()).throw(AssertionError("fp32 exchange used in a 16-bit run"))
         gr.exchange_bf16 = PlayedBf16Exchange(dev(recv[r]), dev(incoming[r]))
+        gr.fuse_bf16_staging = fused
+        gr.comm_buf.recv_buf.fill_(float("nan"))
         xr = dev(x[sl[r]]).requires_grad_()
         out = Aggregator.apply(gr, xr, 2, 16, True, True)
         assert np.array_equal(gr.exchange_bf16.sent["forward"].float().cpu().numpy().view(np.uint32),
                               o_send[r].view(np.uint32))
-        assert np.array_equal(gr.comm_buf.recv_buf.cpu().numpy(), recv[r])
+        if fused:   # the received rows are gathered as bf16: the fp32 copy is never written
+            assert bool(torch.isnan(gr.comm_buf.recv_buf).all()) or gr.comm_buf.recv_buf.numel() == 0
+            assert np.array_equal(gr.comm_buf.recv_buf_fp16.float().cpu().numpy(), recv[r])
+        else:
+            assert np.array_equal(gr.comm_buf.recv_buf.cpu().numpy(), recv[r])
         o_out = oagg.forward_out(o["local"], o["a_from"], np.ascontiguousarray(x[sl[r]]), recv[r])
         assert np.array_equal(out.detach().cpu().numpy(), o_out)
         out.backward(dev(g[sl[r]]))

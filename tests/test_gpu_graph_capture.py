@@ -2,7 +2,7 @@
 record them into a HIP graph (here through torch.cuda.CUDAGraph, whose capture stream the library
 picks up as the current stream) and replay it.  One graph holds the plan SpMM with a very long row
 (block-per-row kernel on the plan's side stream, forked and joined with events), the transposed
-product, the strided product, the row gather, the codec, the bf16 conversions, both fused
+product, the strided product, the products with bf16 rows, the row gather, the codec, the bf16 conversions, both fused
 epilogues, the weight gradient, and the one-kernel dense layer with its one-pass gradient; it is replayed several times, with eager work and host
 synchronisation in between, and every replay must reproduce the eager results bit for bit."""
 import numpy as np
@@ -68,9 +68,13 @@ def test_entry_points_replay_from_a_hip_graph(monkeypatch):
         _convert(back, half)
         wire = torch.empty(n, feat, device="cuda")
         _convert(half, wire)
+        rounded = torch.empty(n, feat, dtype=torch.bfloat16, device="cuda")
+        SPMM_forward(src, x, rounded, accumulate=False)               # bf16 result rows (a 16-bit exchange's send side)
+        widened = torch.empty(n, feat, device="cuda")
+        SPMM_backward(src, rounded, widened, accumulate=False)        # bf16 operand rows (its receive side)
         # (the left half of `cat` is scratch for a following layer and is never written here)
         return [out, dx, wide, cat[:, feat:], act, w, rows, packed, params, back, wire, layer.detach(), x_in.grad,
-                w_in.grad, b_in.grad, layer3.detach(), x3.grad, w3.grad, b3.grad]
+                w_in.grad, b_in.grad, layer3.detach(), x3.grad, w3.grad, b3.grad, rounded, widened]
 
     eager = [t.clone() for t in work()]
     torch.cuda.synchronize()

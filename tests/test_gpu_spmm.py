@@ -580,3 +580,58 @@ def test_compiled_extension_module_on_the_committed_reference_outputs():
     with pytest.raises(RuntimeError, match="Input mismatch"):
         mod.spmm(dev(c["rowptr"]), dev(c["col"]), dev(c["val"]).double(), dev(c["x"]), out, c["out0"].shape[0], EMPTY_I32,
                  EMPTY_I32)
+
+
+@pytest.mark.parametrize("feat", [4, 40, 100, 128, 172, 256, 260, 516])
+def test_products_with_bf16_rows_equal_the_copies_around_an_fp32_product(feat):
+    """``gnnagg_plan_spmm_bf16_f32`` (the staging buffers of a 16-bit exchange, communicator.py:128,137): gathering bf16
+    rows equals widening them first, writing bf16 rows equals rounding the fp32 result afterwards -- bit for bit, rows
+    of every length class (an empty one, a hub) included, forward and transposed, rows back to back or column blocks of
+    a wider array."""
+    n = 1500
+    rowptr, col, val = skewed_csr(n, n, seed=feat, heavy_rows=(3000, 700))
+    src = SparseTensor(rowptr=dev(rowptr), col=dev(col), value=dev(val), sparse_sizes=(n, n))
+    gen = torch.Generator(device="cuda").manual_seed(feat)
+    x = torch.randn(n, feat, device="cuda", generator=gen) * 37.0
+    x[3, 0] = float("nan")
+    x[5, 1] = float("inf")
+    xb = x.bfloat16()
+    for product in (SPMM_forward, SPMM_backward):
+        want = torch.zeros(n, feat, device="cuda")
+        product(src, xb.float(), want, accumulate=False)            # widen, then the fp32 product
+        got = torch.empty(n, feat, device="cuda")
+        product(src, xb, got, accumulate=False)
+        assert torch.equal(got.view(torch.int32), want.view(torch.int32))
+        product(src, xb, got, accumulate=True)                        # accumulating onto an fp32 result
+        product(src, xb.float(), want, accumulate=True)
+        assert torch.equal(got.view(torch.int32), want.view(torch.int32))
+        full = torch.zeros(n, feat, device="cuda")
+        product(src, x, full, accumulate=False)                       # the fp32 product, then the rounding copy
+        half = torch.empty(n, feat, dtype=torch.bfloat16, device="cuda")
+        product(src, x, half, accumulate=False)
+        assert torch.equal(half.view(torch.int16), full.bfloat16().view(torch.int16))
+        both = torch.empty(n, feat, dtype=torch.bfloat16, device="cuda")
+        product(src, xb, both, accumulate=False)
+        assert torch.equal(both.view(torch.int16), want_bf16(src, xb, product).view(torch.int16))
+        wide_in = torch.zeros(n, feat + 8, dtype=torch.bfloat16, device="cuda")
+        wide_in[:, 4:4 + feat] = xb
+        wide_out = torch.full((n, feat + 12), 7.0, dtype=torch.bfloat16, device="cuda")
+        product(src, wide_in[:, 4:4 + feat], wide_out[:, 8:8 + feat], accumulate=False)
+        assert torch.equal(wide_out[:, 8:8 + feat].contiguous().view(torch.int16), both.view(torch.int16))
+        assert bool((wide_out[:, :8] == 7.0).all()) and bool((wide_out[:, 8 + feat:] == 7.0).all())
+    with pytest.raises(RuntimeError, match="accumulated"):
+        SPMM_forward(src, x, torch.empty(n, feat, dtype=torch.bfloat16, device="cuda"), accumulate=True)
+
+
+def want_bf16(src, xb, product):
+    out = torch.zeros(src.sparse_size(0), xb.size(1), device="cuda")
+    product(src, xb.float(), out, accumulate=False)
+    return out.bfloat16()
+
+
+def test_bf16_rows_need_a_width_of_whole_vectors():
+    n = 50
+    rowptr, col, val = skewed_csr(n, n, seed=1)
+    src = SparseTensor(rowptr=dev(rowptr), col=dev(col), value=dev(val), sparse_sizes=(n, n))
+    with pytest.raises(RuntimeError, match="multiple of 4"):
+        SPMM_forward(src, torch.zeros(n, 6, dtype=torch.bfloat16, device="cuda"), torch.zeros(n, 6, device="cuda"))
