@@ -687,7 +687,8 @@ def run_c4(args, graph, setup_s):
 
     fp32_buf = graph.comm_buf
     graph.comm_buf = CommBuffer(fp32_splits, feat, 16, device=dev)
-    graph.exchange_bf16 = synthetic.SeededBf16HaloExchange(args.seed + 7)
+    synthetic.PregeneratedHaloExchange.attach(graph)
+    graph.exchange_bf16 = synthetic.PregeneratedBf16HaloExchange(args.seed + 7)
     for _ in range(2):
         Aggregator.apply(graph, xr, 0, 16, True, True).backward(g)
     torch.cuda.synchronize()
@@ -709,6 +710,7 @@ def run_c4(args, graph, setup_s):
     torch.cuda.synchronize()
     bf16_unfused_ms = (time.perf_counter() - t0) * 1e3 / steps
     graph.fuse_bf16_staging = True
+    graph.comm_buf.resize_buffer(fp32_splits, feat, 16)   # the buffer's own rows again, not the delivered ones
     # the two products of the fused form: pre-aggregation writing bf16 rows, post-aggregation gathering bf16 rows
     from gnn_benchmark_amd import SPMM_forward
 
@@ -903,9 +905,44 @@ def run_c4_raw_halo(args, part):
         o.backward(g)
     torch.cuda.synchronize()
     both_ms = (time.perf_counter() - t0) * 1e3 / steps
+    # the same with bf16 rows on the wire (num_bits=16): the gather writes the bf16 staging rows itself, or the tensor
+    # copy follows it as a pass of its own (the reference's form)
+    from gnn_benchmark_amd.data_manager import CommBuffer
+
+    fp32_buf = graph.comm_buf
+    graph.comm_buf = CommBuffer(graph.comm_splits, feat, 16, device=dev)
+    synthetic.PregeneratedHaloExchange.attach(graph)
+    graph.exchange_bf16 = synthetic.PregeneratedBf16HaloExchange(args.seed + 7)
+    for i in range(steps + 2):
+        if i == 2:
+            e0.record()
+        _gather_rows(x, idx, graph.comm_buf.send_buf_fp16)
+    e1.record()
+    e1.synchronize()
+    ms = e0.elapsed_time(e1) / steps
+    gather16_bytes = idx.numel() * (8.0 + 6.0 * feat)
+    ops.append({"op": "gather boundary rows X[idx] -> bf16 send rows", "rows": int(idx.numel()), "feat": feat,
+                "ms": round(ms, 4), "gbs_model": round(gather16_bytes / (ms * 1e-3) / 1e9, 1),
+                "frac_of_hbm_peak": round(gather16_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)})
+    bf16_ms = {}
+    for fused in (True, False):
+        graph.fuse_bf16_staging = fused
+        for _ in range(2):
+            Aggregator.apply(graph, xr, 0, 16, False, True).backward(g)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            o = Aggregator.apply(graph, xr, 0, 16, False, True)
+            o.backward(g)
+        torch.cuda.synchronize()
+        bf16_ms[fused] = (time.perf_counter() - t0) * 1e3 / steps
+    graph.fuse_bf16_staging = True
+    graph.comm_buf, graph.exchange_bf16 = fp32_buf, None
     return {"workload": "the c4 partition with raw boundary rows (is_pre_delay=False)", "feat": feat,
             "send_rows": int(idx.numel()), "halo_rows": int(graph.remote_adj_t.sparse_size(1)), "setup_s": round(setup_s, 2),
-            "ops": ops, "aggregator_forward_ms": round(fwd_ms, 3), "aggregator_forward_backward_ms": round(both_ms, 3)}
+            "ops": ops, "aggregator_forward_ms": round(fwd_ms, 3), "aggregator_forward_backward_ms": round(both_ms, 3),
+            "aggregator_forward_backward_ms_bf16_exchange": round(bf16_ms[True], 3),
+            "aggregator_forward_backward_ms_bf16_exchange_separate_copies": round(bf16_ms[False], 3)}
 
 
 def run_c5(args, graph):

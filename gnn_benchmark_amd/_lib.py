@@ -29,6 +29,7 @@ EXPORTS = (
     "gnnagg_csr_transpose",
     "gnnagg_coo_to_csr",
     "gnnagg_gather_rows_f32",
+    "gnnagg_gather_rows_f32_bf16",
     "gnnagg_check_index",
     "gnnagg_bias_relu_dropout_f32",
     "gnnagg_relu_dropout_backward_blocks",
@@ -131,6 +132,8 @@ def lib() -> ctypes.CDLL:
     L.gnnagg_coo_to_csr.argtypes = [vp, vp, vp, i64, i64, i64, vp, vp, vp, vp]
     L.gnnagg_gather_rows_f32.restype = i32
     L.gnnagg_gather_rows_f32.argtypes = [vp, i64, vp, vp, i64, i64, vp]
+    L.gnnagg_gather_rows_f32_bf16.restype = i32
+    L.gnnagg_gather_rows_f32_bf16.argtypes = [vp, i64, vp, vp, i64, i64, vp]
     L.gnnagg_check_index.restype = i32
     L.gnnagg_check_index.argtypes = [vp, i32, i64, i32, i64, vp]
     L.gnnagg_bias_relu_dropout_f32.restype = i32

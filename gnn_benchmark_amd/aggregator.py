@@ -58,16 +58,19 @@ def _gather_rows(src: torch.Tensor, index: torch.Tensor, out: torch.Tensor) -> N
     # torch.index_select(local_nodes_feat, 0, idx, out=send_buf)   (aggregator.py:51)
     if not (src.is_cuda and index.is_cuda and out.is_cuda):
         raise RuntimeError("gather operands must be GPU (HIP) tensors; there is no CPU path")
-    if src.dtype != torch.float32 or out.dtype != torch.float32 or index.dtype != torch.int64:
+    if src.dtype != torch.float32 or out.dtype not in (torch.float32, torch.bfloat16) or index.dtype != torch.int64:
         raise RuntimeError("Input mismatch: gather needs float32 rows and int64 indices")
     if out.size(0) != index.numel() or out.size(1) != src.size(1) or not out.is_contiguous():
         raise RuntimeError("Input mismatch: gather output shape")
     src = src.contiguous()
     # torch.index_select raises on an index outside the source; here the list is looked at once (cached per tensor)
     _lib.check_index(index, src.size(0), what="boundary row list (idx_nodes_send_to_others)")
+    # bf16 result rows: the gather and the copy into the staging buffer of a 16-bit exchange in one pass
+    L = _lib.lib()
+    entry = L.gnnagg_gather_rows_f32_bf16 if out.dtype == torch.bfloat16 else L.gnnagg_gather_rows_f32
     with torch.cuda.device(src.device):
-        _lib.check(_lib.lib().gnnagg_gather_rows_f32(_lib.ptr(src), src.size(0), _lib.ptr(index), _lib.ptr(out),
-                                                     index.numel(), src.size(1), _lib.current_stream(src.device)))
+        _lib.check(entry(_lib.ptr(src), src.size(0), _lib.ptr(index), _lib.ptr(out), index.numel(), src.size(1),
+                         _lib.current_stream(src.device)))
 
 
 def _check_bits(num_bits: int) -> None:
@@ -247,12 +250,12 @@ def _forward(ctx, graph, feats, layer, num_bits: int, is_pre_delay: bool, is_tra
     if exchange is not None:
         if is_pre_delay:  # pre-aggregation: send_buf = A_to @ X (straight into the bf16 staging rows when they travel)
             feats.product(graph.adj_t_pre_post_aggr_to, graph.comm_buf.send_buf_fp16 if half_fused else send_buf, False)
-        else:  # raw boundary rows
-            feats.gather(graph.idx_nodes_send_to_others, send_buf)
+        else:  # raw boundary rows (as bf16 at once when they travel so)
+            feats.gather(graph.idx_nodes_send_to_others, graph.comm_buf.send_buf_fp16 if half_fused else send_buf)
         if quantized:
             comm_handle = _quantize_and_exchange(graph, num_bits, f"forward{layer}", "forward")
         elif half:
-            if not (half_fused and is_pre_delay):
+            if not half_fused:
                 _convert(send_buf, graph.comm_buf.send_buf_fp16)
             comm_handle = graph.exchange_bf16(graph.comm_splits, graph.comm_buf, f"forward{layer}", "forward")
         else:

@@ -74,4 +74,11 @@ inline int ceil_log2_u64(uint64_t x) {  // smallest b with 2^b >= x (x >= 1)
 
 inline unsigned grid_for(int64_t n, int block) { return (unsigned)((n + block - 1) / block); }
 
+// fp32 -> bf16 as the tensor copy does it: round to nearest even, NaN -> 0x7FC0
+__device__ __forceinline__ unsigned short bf16_bits(float x) {
+    const uint32_t u = __float_as_uint(x);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)0x7fc0;
+    return (unsigned short)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+
 }  // namespace gnnagg

@@ -3,6 +3,7 @@
 #include <hipcub/hipcub.hpp>
 
 #include <algorithm>
+#include <type_traits>
 
 #include "common.h"
 
@@ -79,11 +80,15 @@ __global__ __launch_bounds__(256) void pack_transposed_keys_kernel(const int64_t
 // owns four rows at a time: their indices, then their vectors, are requested back to back before
 // anything is stored.  Source rows come through normal loads (a boundary row usually goes to
 // several peers, so it is asked for again soon); the result is written once, with streaming stores.
-template <int VEC, int G>
+// OUT16 (VEC == 4 only): the rows are stored as bf16, rounded as the tensor copy rounds them.
+template <int VEC, int G, bool OUT16>
 __global__ __launch_bounds__(256) void gather_rows_kernel(const float *__restrict__ src, int64_t src_rows,
                                                           const int64_t *__restrict__ index,
-                                                          float *__restrict__ out, int64_t n_index, int feat_vec) {
+                                                          void *__restrict__ out, int64_t n_index, int feat_vec) {
+    static_assert(!OUT16 || VEC == 4, "bf16 rows are stored four values at a time");
     typedef float vec_t __attribute__((ext_vector_type(VEC)));
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    using out_t = typename std::conditional<OUT16, u32x2, vec_t>::type;
     constexpr int kGroups = 256 / G;
     constexpr int kRows = 4;
     const int l = (int)threadIdx.x % G;
@@ -91,7 +96,7 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const float *__restric
     const int64_t step = (int64_t)gridDim.x * kGroups * kRows;
     for (int64_t base = ((int64_t)blockIdx.x * kGroups + group) * kRows; base < n_index; base += step) {
         const vec_t *s[kRows];
-        vec_t *d[kRows];
+        out_t *d[kRows];
         bool ok[kRows], inside[kRows];
 #pragma unroll
         for (int u = 0; u < kRows; ++u) {
@@ -100,7 +105,7 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const float *__restric
             // an index outside the source is never dereferenced: row 0 is read in its place and NaN is stored
             inside[u] = (uint64_t)r < (uint64_t)src_rows;
             s[u] = reinterpret_cast<const vec_t *>(src) + (inside[u] ? (size_t)r : 0) * (size_t)feat_vec;
-            d[u] = reinterpret_cast<vec_t *>(out) + (size_t)(base + u) * (size_t)feat_vec;
+            d[u] = reinterpret_cast<out_t *>(out) + (size_t)(base + u) * (size_t)feat_vec;
         }
         for (int f = l; f < feat_vec; f += G) {
             vec_t v[kRows];
@@ -108,8 +113,18 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const float *__restric
             for (int u = 0; u < kRows; ++u)
                 if (ok[u]) v[u] = s[u][f];
 #pragma unroll
-            for (int u = 0; u < kRows; ++u)
-                if (ok[u]) __builtin_nontemporal_store(inside[u] ? v[u] : v[u] * __builtin_nanf(""), d[u] + f);
+            for (int u = 0; u < kRows; ++u) {
+                if (!ok[u]) continue;
+                const vec_t w = inside[u] ? v[u] : v[u] * __builtin_nanf("");
+                if constexpr (OUT16) {
+                    u32x2 r;
+                    r.x = (uint32_t)bf16_bits(w[0]) | ((uint32_t)bf16_bits(w[1]) << 16);
+                    r.y = (uint32_t)bf16_bits(w[2]) | ((uint32_t)bf16_bits(w[3]) << 16);
+                    __builtin_nontemporal_store(r, d[u] + f);
+                } else {
+                    __builtin_nontemporal_store(w, d[u] + f);
+                }
+            }
         }
     }
 }
@@ -127,18 +142,18 @@ __global__ __launch_bounds__(256) void check_index_kernel(const T *__restrict__ 
     if (bad != ~0ull) atomicMin(first_bad, bad);
 }
 
-template <int VEC>
-hipError_t launch_gather_rows(const float *src, int64_t src_rows, const int64_t *index, float *out, int64_t n_index,
+template <int VEC, bool OUT16 = false>
+hipError_t launch_gather_rows(const float *src, int64_t src_rows, const int64_t *index, void *out, int64_t n_index,
                               int feat_vec, hipStream_t st) {
     int g = 8;
     while (g < 64 && g < feat_vec) g *= 2;
     const int64_t rows_per_block = (256 / g) * 4;
     const int64_t need = (n_index + rows_per_block - 1) / rows_per_block;
     const unsigned grid = (unsigned)(need < 256 * 32 ? need : 256 * 32);
-    if (g == 8) hipLaunchKernelGGL((gather_rows_kernel<VEC, 8>), dim3(grid), dim3(256), 0, st, src, src_rows, index, out, n_index, feat_vec);
-    else if (g == 16) hipLaunchKernelGGL((gather_rows_kernel<VEC, 16>), dim3(grid), dim3(256), 0, st, src, src_rows, index, out, n_index, feat_vec);
-    else if (g == 32) hipLaunchKernelGGL((gather_rows_kernel<VEC, 32>), dim3(grid), dim3(256), 0, st, src, src_rows, index, out, n_index, feat_vec);
-    else hipLaunchKernelGGL((gather_rows_kernel<VEC, 64>), dim3(grid), dim3(256), 0, st, src, src_rows, index, out, n_index, feat_vec);
+    if (g == 8) hipLaunchKernelGGL((gather_rows_kernel<VEC, 8, OUT16>), dim3(grid), dim3(256), 0, st, src, src_rows, index, out, n_index, feat_vec);
+    else if (g == 16) hipLaunchKernelGGL((gather_rows_kernel<VEC, 16, OUT16>), dim3(grid), dim3(256), 0, st, src, src_rows, index, out, n_index, feat_vec);
+    else if (g == 32) hipLaunchKernelGGL((gather_rows_kernel<VEC, 32, OUT16>), dim3(grid), dim3(256), 0, st, src, src_rows, index, out, n_index, feat_vec);
+    else hipLaunchKernelGGL((gather_rows_kernel<VEC, 64, OUT16>), dim3(grid), dim3(256), 0, st, src, src_rows, index, out, n_index, feat_vec);
     return hipGetLastError();
 }
 
@@ -275,6 +290,22 @@ extern "C" int gnnagg_gather_rows_f32(const float *src, int64_t src_rows, const 
     else
         GNNAGG_HIP(launch_gather_rows<1>(src, src_rows, index, out, n_index, (int)feat, st));
     GNNAGG_HIP(hipGetLastError());
+    return GNNAGG_OK;
+}
+
+extern "C" int gnnagg_gather_rows_f32_bf16(const float *src, int64_t src_rows, const int64_t *index, void *out,
+                                           int64_t n_index, int64_t feat, void *stream) {
+    GNNAGG_REQUIRE(n_index >= 0 && feat >= 0 && src_rows >= 0, "negative size");
+    if (n_index == 0 || feat == 0) return GNNAGG_OK;
+    GNNAGG_REQUIRE(src && index && out, "null src/index/out");
+    GNNAGG_REQUIRE(src_rows > 0, "rows are asked of a source without rows");
+    if (feat > (1 << 20)) return fail(GNNAGG_ERR_UNSUPPORTED, "feature width %lld above 2^20", (long long)feat);
+    if (feat % 4 != 0 || reinterpret_cast<uintptr_t>(src) % 16 != 0 || reinterpret_cast<uintptr_t>(out) % 8 != 0)
+        return fail(GNNAGG_ERR_UNSUPPORTED,
+                    "bf16 result rows need a width that is a multiple of 4 (got %lld), a 16-byte aligned source and "
+                    "an 8-byte aligned result", (long long)feat);
+    GNNAGG_HIP((launch_gather_rows<4, true>(src, src_rows, index, out, n_index, (int)(feat / 4),
+                                            static_cast<hipStream_t>(stream))));
     return GNNAGG_OK;
 }
 

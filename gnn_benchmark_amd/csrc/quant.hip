@@ -496,12 +496,6 @@ int check_segments(const void *a, const void *b, const void *c, const int32_t *r
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef unsigned short u16x4_t __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ unsigned short bf16_bits(float x) {
-    const uint32_t u = __float_as_uint(x);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)0x7fc0;
-    return (unsigned short)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
-}
-
 __global__ __launch_bounds__(256) void f32_to_bf16_kernel(const float *__restrict__ x, unsigned short *__restrict__ y,
                                                           int64_t count, int vec) {
     const int64_t stride = (int64_t)gridDim.x * 256;

@@ -23,6 +23,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "common.h"
+
 namespace gnnagg {
 
 typedef float f32x2 __attribute__((ext_vector_type(2)));
@@ -177,13 +179,6 @@ enum SourceKind : int {
     kSrcQuant = 2,   // row col is held quantised: qdata / qparams / qcode (boundary-buffer codec layout)
     kSrcBf16 = 3     // x[col, :] is a bf16 row (x points at 16-bit values, ldx counts them): widened in the gather
 };
-
-// fp32 -> bf16 as the tensor copy does it: round to nearest even, NaN -> 0x7FC0
-__device__ __forceinline__ unsigned short bf16_bits(float x) {
-    const uint32_t u = __float_as_uint(x);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)0x7fc0;
-    return (unsigned short)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
-}
 
 typedef float f32x4_unaligned __attribute__((ext_vector_type(4), aligned(4)));
 

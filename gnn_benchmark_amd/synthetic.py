@@ -215,10 +215,10 @@ class _DeliveredInPlaceCommBuffer(CommBuffer):
 
     def __init__(self, inner: CommBuffer):
         self.__dict__.update(inner.__dict__)
-        self._own = (inner.send_buf, inner.recv_buf)
+        self._own = (inner.send_buf, inner.recv_buf, inner.send_buf_fp16, inner.recv_buf_fp16)
 
     def resize_buffer(self, comm_splits, feat_len: int, bits: int) -> None:
-        self.send_buf, self.recv_buf = self._own
+        self.send_buf, self.recv_buf, self.send_buf_fp16, self.recv_buf_fp16 = self._own
         super().resize_buffer(comm_splits, feat_len, bits)
 
 
@@ -295,6 +295,32 @@ class SeededBf16HaloExchange:
         self._gen.manual_seed(self.seed * 1000003 + 11 + sum(ord(c) * (i + 1) for i, c in enumerate(tag)))
         target.normal_(generator=self._gen)
         self.calls.append(tag)
+        return None
+
+
+class PregeneratedBf16HaloExchange(SeededBf16HaloExchange):
+    """bf16 counterpart of ``PregeneratedHaloExchange``: the seeded bf16 rows are drawn once per (tag, shape) and a
+    call points the receiving staging buffer at them, so nothing is enqueued inside a timed step."""
+
+    def __init__(self, seed: int = 0):
+        super().__init__(seed)
+        self._rows = {}
+
+    def __call__(self, comm_splits, comm_buf, tag: str, direction: str):
+        if not isinstance(comm_buf, _DeliveredInPlaceCommBuffer):
+            raise RuntimeError("PregeneratedBf16HaloExchange needs PregeneratedHaloExchange.attach(graph) first")
+        buf = comm_buf.recv_buf_fp16 if direction == "forward" else comm_buf.send_buf_fp16
+        key = (tag, tuple(buf.shape), str(buf.device))
+        rows = self._rows.get(key)
+        if rows is None:
+            super().__call__(comm_splits, comm_buf, tag, direction)
+            rows = self._rows[key] = buf.clone()
+        else:
+            self.calls.append(tag)
+        if direction == "forward":
+            comm_buf.recv_buf_fp16 = rows
+        else:
+            comm_buf.send_buf_fp16 = rows
         return None
 
 

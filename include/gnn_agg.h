@@ -182,6 +182,13 @@ int gnnagg_coo_to_csr(const int64_t *row, const int64_t *col, const float *value
 int gnnagg_gather_rows_f32(const float *src, int64_t src_rows, const int64_t *index, float *out, int64_t n_index,
                            int64_t feat, void *stream);
 
+/* The same gather with the result rows stored as bf16 (round to nearest even, NaN -> 0x7FC0): the gather and the
+ * `send_buf_fp16.copy_(send_buf)` of a 16-bit exchange (model/layers/aggregator.py:51 followed by
+ * communicator/communicator.py:128) in one pass, the same bits as the two apart.  out: bf16 [n_index, feat];
+ * feat a multiple of 4, src 16-byte and out 8-byte aligned (GNNAGG_ERR_UNSUPPORTED otherwise). */
+int gnnagg_gather_rows_f32_bf16(const float *src, int64_t src_rows, const int64_t *index, void *out, int64_t n_index,
+                                int64_t feat, void *stream);
+
 /* Range check of an index list held on the device: GNNAGG_OK when every (index[i] >> shift) lies in [0, bound),
  * GNNAGG_ERR_INVALID (naming the first offending position found) otherwise.  index: `count` integers of
  * elem_bytes 4 (int32) or 8 (int64).  SYNCHRONISES the stream: meant to run once per index list (the boundary

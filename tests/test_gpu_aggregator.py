@@ -123,10 +123,9 @@ def test_pre_post_world_matches_oracle_and_global_product(seed, sizes):
         assert_math_close(xr.grad, want_t[sl[r]], "gradient vs global transposed product")
 
 
-@pytest.mark.parametrize("seed,sizes", [(4, (300, 450, 250)), (5, (600, 1, 400, 330))])
-def test_raw_halo_world_matches_oracle_and_global_product(seed, sizes):
-    w = World(seed, sizes, mean_deg=8.0)
-    W, F = w.world, 40
+def _build_raw_graphs(w, F, bits=32):
+    """Every rank's graph for the raw-halo mode (``get_distributed_graph``), the halo id exchange played on the host."""
+    W, sizes = w.world, w.sizes
     parts = [w.partition(r) for r in range(W)]
     # pass 1: halo id lists of every rank (what the id exchange moves)
     halo = []
@@ -140,8 +139,16 @@ def test_raw_halo_world_matches_oracle_and_global_product(seed, sizes):
         local_nodes_list = torch.stack((torch.arange(begin, begin + int(sizes[r])),) * 2, dim=1) if sizes[r] else torch.zeros((1, 2), dtype=torch.int64)
         asked = lambda _s, r=r: [halo[i][0][int(halo[i][1][r]):int(halo[i][1][r + 1])] for i in range(W)]
         graphs.append(get_distributed_graph(torch.from_numpy(parts[r][0].copy()), torch.from_numpy(parts[r][1].copy()),
-                                            local_nodes_list, torch.from_numpy(w.begins), int(sizes[r]), F, W, 32,
+                                            local_nodes_list, torch.from_numpy(w.begins), int(sizes[r]), F, W, bits,
                                             halo_id_exchange=asked, device="cuda"))
+    return graphs
+
+
+@pytest.mark.parametrize("seed,sizes", [(4, (300, 450, 250)), (5, (600, 1, 400, 330))])
+def test_raw_halo_world_matches_oracle_and_global_product(seed, sizes):
+    w = World(seed, sizes, mean_deg=8.0)
+    W, F = w.world, 40
+    graphs = _build_raw_graphs(w, F)
     rng = np.random.default_rng(seed)
     x = rng.standard_normal((w.n, F)).astype(np.float32)
     g = rng.standard_normal((w.n, F)).astype(np.float32)
@@ -468,6 +475,81 @@ def test_bf16_exchange_world_matches_oracle(seed, sizes, fused):
         Aggregator.apply(graphs[1], dev(x[sl[1]]), 0, 16, True, True)
 
 
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("seed,sizes", [(6, (300, 450, 250)), (7, (600, 1, 400, 330))])
+def test_raw_halo_bf16_exchange_matches_oracle(seed, sizes, fused):
+    """The raw-halo mode with 16-bit rows on the wire (aggregator.py:51 then communicator.py:111-137): the staged rows
+    are the gathered boundary rows rounded to bf16, bit for bit, whether the gather writes them as bf16 itself (the
+    default) or the tensor copy follows it; output and gradient equal the oracle pipeline fed with the rounded rows."""
+    from oracle import quantization as oq
+
+    w = World(seed, sizes, mean_deg=8.0)
+    W, F = w.world, 40
+    graphs = _build_raw_graphs(w, F, bits=16)
+    rng = np.random.default_rng(seed + 300)
+    x = (rng.standard_normal((w.n, F)) * rng.uniform(1e-3, 1e3, (w.n, 1))).astype(np.float32)
+    g = rng.standard_normal((w.n, F)).astype(np.float32)
+    sl = [slice(int(w.begins[r]), int(w.begins[r + 1])) for r in range(W)]
+    csr = [(_csr_np(gr.local_adj_t) + [gr.local_adj_t.sparse_sizes()], _csr_np(gr.remote_adj_t) + [gr.remote_adj_t.sparse_sizes()])
+           for gr in graphs]
+    idx = [gr.idx_nodes_send_to_others.cpu().numpy() for gr in graphs]
+    o_send = [oq.to_bf16_and_back(oagg.forward_send_raw(idx[r], x[sl[r]])) for r in range(W)]
+    o_back = [oq.to_bf16_and_back(oagg.backward_recv(csr[r][1], np.ascontiguousarray(g[sl[r]]))) for r in range(W)]
+    send_splits = [gr.comm_splits.send_splits for gr in graphs]
+    recv_splits = [gr.comm_splits.recv_splits for gr in graphs]
+    recv = host_exchange(o_send, send_splits, recv_splits)
+    incoming = host_exchange(o_back, recv_splits, send_splits)
+    for r in range(W):
+        gr = graphs[r]
+        gr.exchange = lambda *a: (_ for _ in ()).throw(AssertionError("fp32 exchange used in a 16-bit run"))
+        gr.exchange_bf16 = PlayedBf16Exchange(dev(recv[r]), dev(incoming[r]))
+        gr.fuse_bf16_staging = fused
+        gr.comm_buf.send_buf.fill_(float("nan"))
+        xr = dev(x[sl[r]]).requires_grad_()
+        out = Aggregator.apply(gr, xr, 1, 16, False, True)
+        assert np.array_equal(gr.exchange_bf16.sent["forward"].float().cpu().numpy().view(np.uint32),
+                              o_send[r].view(np.uint32))
+        if fused and gr.comm_buf.send_buf.numel():   # the fp32 rows are never written
+            assert bool(torch.isnan(gr.comm_buf.send_buf).all())
+        o_out = oagg.forward_out(csr[r][0], csr[r][1], np.ascontiguousarray(x[sl[r]]), recv[r])
+        assert np.array_equal(out.detach().cpu().numpy(), o_out)
+        out.backward(dev(g[sl[r]]))
+        assert np.array_equal(gr.exchange_bf16.sent["backward"].float().cpu().numpy().view(np.uint32),
+                              o_back[r].view(np.uint32))
+        o_dx = oagg.backward_out_raw(csr[r][0], idx[r], np.ascontiguousarray(g[sl[r]]), incoming[r])
+        assert_close(xr.grad, o_dx, "raw halo gradient vs oracle, bf16 rows")
+
+
+@pytest.mark.parametrize("feat", [4, 8, 20, 40, 128, 132, 256, 604, 1028])
+@pytest.mark.parametrize("count", [0, 1, 3, 64, 1000, 4099])
+def test_row_gather_into_bf16_rows_equals_gather_then_copy(feat, count):
+    """``index_select`` into the fp32 buffer followed by ``send_buf_fp16.copy_(send_buf)`` (aggregator.py:51,
+    communicator.py:128) against the one-pass gather with bf16 result rows: the same bits, special values included."""
+    from gnn_benchmark_amd.aggregator import _gather_rows
+
+    gen = torch.Generator(device="cuda").manual_seed(feat * 11 + count)
+    src = torch.randn(777, feat, device="cuda", generator=gen) * 100.0
+    src[5, :4] = torch.tensor([float("nan"), float("inf"), -0.0, 1.0 + 2.0 ** -8], device="cuda")
+    src[6, :4] = torch.tensor([1.0 + 3 * 2.0 ** -8, 1e-40, 3.3895314e38, -float("inf")], device="cuda")
+    index = torch.randint(0, 777, (count,), device="cuda", generator=gen)
+    if count > 2:
+        index[:2] = torch.tensor([5, 6], device="cuda")
+    out = torch.full((count, feat), -1.0, device="cuda", dtype=torch.bfloat16)
+    _gather_rows(src, index, out)
+    want = torch.empty_like(out)
+    want.copy_(src[index])
+    assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+
+
+def test_row_gather_into_bf16_rows_needs_whole_vectors():
+    from gnn_benchmark_amd import _lib
+    from gnn_benchmark_amd.aggregator import _gather_rows
+
+    src = torch.randn(10, 6, device="cuda")
+    with pytest.raises(_lib.GnnAggError, match="multiple of 4"):
+        _gather_rows(src, torch.tensor([1, 2], device="cuda"), torch.empty(2, 6, device="cuda", dtype=torch.bfloat16))
+
+
 @pytest.mark.parametrize("count", [0, 1, 3, 4, 1000, 1_000_003])
 def test_bf16_conversion_equals_the_tensor_copy(count):
     """fp32 -> bf16 -> fp32 through the library against torch's own conversion, bit for bit:
@@ -519,6 +601,38 @@ def test_pregenerated_halo_rows_equal_the_seeded_ones():
     assert len(results[0]) == len(results[1])
     for a, b in zip(*results):
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("is_pre_delay", [True, False])
+def test_pregenerated_bf16_halo_rows_equal_the_seeded_ones(is_pre_delay):
+    """The same for the 16-bit exchange: bf16 rows kept on the device and handed over by pointing the staging buffer
+    at them give what drawing them in every call gives, with the copies fused into the products or apart."""
+    from gnn_benchmark_amd import synthetic
+
+    n = 30_000
+    part = synthetic.partition_edges(n, 8, 5, 6.0, 1.8, 1500, 11_000, 70_000, seed=13, device="cuda")
+    results = []
+    for exchange_bf16, fused in ((synthetic.SeededBf16HaloExchange(9), True), (synthetic.PregeneratedBf16HaloExchange(9), True),
+                                 (synthetic.PregeneratedBf16HaloExchange(9), False)):
+        graph = synthetic.build_partition_graph(part, 96, is_pre_delay, exchange=synthetic.PregeneratedHaloExchange(1),
+                                                bits=16, exchange_bf16=exchange_bf16, device="cuda")
+        graph.fuse_bf16_staging = fused
+        gen = torch.Generator(device="cuda").manual_seed(3)
+        seen = []
+        for call in range(3):
+            for layer, feat in ((0, 64), (1, 96)):
+                x = torch.randn(n, feat, device="cuda", generator=gen, requires_grad=True)
+                g = torch.randn(n, feat, device="cuda", generator=gen)
+                out = Aggregator.apply(graph, x, layer, 16, is_pre_delay, True)
+                out.backward(g)
+                seen += [out.detach().clone(), x.grad.clone()]
+        torch.cuda.synchronize()
+        assert exchange_bf16.calls == ["forward0", "backward0", "forward1", "backward1"] * 3
+        results.append(seen)
+    for other in results[1:]:
+        assert len(results[0]) == len(other)
+        for a, b in zip(results[0], other):
+            assert torch.equal(a, b)
 
 
 def test_bad_indices_raise_instead_of_reading_out_of_bounds():

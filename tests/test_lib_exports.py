@@ -44,6 +44,8 @@ def test_argument_errors_without_gpu_work():
     assert L.gnnagg_gather_rows_f32(None, 0, None, None, 0, 8, None) == _lib.OK
     with pytest.raises(_lib.GnnAggError):
         _lib.check(L.gnnagg_gather_rows_f32(None, 3, None, None, 5, 8, None))
+    assert L.gnnagg_gather_rows_f32_bf16(None, 0, None, None, 0, 8, None) == _lib.OK
+    assert L.gnnagg_gather_rows_f32_bf16(None, 3, None, None, 5, 8, None) == _lib.ERR_INVALID
     assert L.gnnagg_check_index(None, 8, 0, 0, 10, None) == _lib.OK
     assert L.gnnagg_check_index(None, 3, 5, 0, 10, None) == _lib.ERR_INVALID
     assert L.gnnagg_wgrad_f32(None, None, None, None, 0, 5, 8, 8, None) == _lib.ERR_INVALID   # null operands
