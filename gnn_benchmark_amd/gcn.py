@@ -208,18 +208,29 @@ def stacked_product(cat: torch.Tensor, weight: torch.Tensor, bias, form: int) ->
 
 
 def input_gradient(g: torch.Tensor, weight: torch.Tensor, form: int) -> torch.Tensor:
-    """g @ weight^T, [rows, weight rows].  ``form`` ``BF16X3``: libgnnagg's product kernel, one call per block of at
-    most 256 output columns, each writing its columns of the result; the BLAS library's product otherwise."""
+    """g @ weight^T, [rows, weight rows], through libgnnagg's product kernel: one call per block of at most 256 output
+    columns, each writing its columns of the result.  ``form`` ``BF16`` rounds the operands to bf16; ``FP32`` and
+    ``BF16X3`` both feed every operand as three bf16 pieces -- fp32 accuracy (errors at the level of the BLAS library's
+    fp32 product), and for this plain product faster than the fp32 matrix instruction and than the library
+    (7 M x 256 x 256: 5.8 ms against 8.0 and 7.0).  An inner width that is no multiple of 16 goes through a zero-padded
+    copy of ``g``.  The BLAS library's product only for what the kernel does not take."""
     wide, inner = weight.size(0), weight.size(1)
     blocks = [(c, min(c + 256, wide)) for c in range(0, wide, 256)]
     L = _lib.lib()
-    if (form == BF16X3 and g.is_cuda and g.dtype == torch.float32 and g.size(0) > 0 and wide % 4 == 0
-            and all(L.gnnagg_linear_shape_supported(inner, hi - lo) for lo, hi in blocks)):
+    padded = inner + (-inner) % 16
+    if (g.is_cuda and g.dtype == torch.float32 and g.size(0) > 0 and wide % 4 == 0
+            and all(L.gnnagg_linear_shape_supported(padded, hi - lo) for lo, hi in blocks)):
+        if padded != inner:
+            g = torch.nn.functional.pad(g, (0, padded - inner))
+            weight = torch.nn.functional.pad(weight, (0, padded - inner))
         g = _kernel_ready(g)
+        kernel_form = BF16 if form == BF16 else BF16X3
         out = torch.empty(g.size(0), wide, dtype=torch.float32, device=g.device)
         for lo, hi in blocks:
-            _fused_product(g, weight[lo:hi].t().contiguous(), None, None, None, 1.0, False, BF16X3, out=out[:, lo:hi])
+            _fused_product(g, weight[lo:hi].t().contiguous(), None, None, None, 1.0, False, kernel_form, out=out[:, lo:hi])
         return out
+    if form == BF16:
+        return _Bf16InputLinear._mm(g, weight.t())
     return torch.mm(g, weight.t())
 
 
@@ -230,7 +241,8 @@ class _FusedLayer(torch.autograd.Function):
     pass over x, the incoming gradient and y -- plus the product for the input gradient.  With
     ``form`` ``BF16`` all three products round their operands to bf16 on the way into the matrix units
     (fp32 accumulation); with ``BF16X3`` they feed every operand as three bf16 pieces (fp32 accuracy); mask,
-    division and bias gradient stay in fp32."""
+    division and bias gradient stay in fp32.  The input-gradient product is ``input_gradient``: libgnnagg's kernel in
+    every form (three bf16 pieces an operand for ``FP32`` too), no BLAS-library call."""
 
     @staticmethod
     def forward(ctx, x, w, bias, keep_bits, scale, row_div, relu, form=FP32):
@@ -272,7 +284,6 @@ def _fused_backward(x, w, grad_y, y, header, row_div, scale, form, want_x):
     grad_w = torch.empty(k, n, dtype=torch.float32, device=x.device)
     grad_bias = torch.empty(n, dtype=torch.float32, device=x.device)
     stream = _lib.current_stream(x.device)
-    bf16 = form == BF16
     with torch.cuda.device(x.device):
         if header is not None:
             _lib.check(L.gnnagg_wgrad_relu_dropout_backward_from_header_f32(
@@ -285,14 +296,7 @@ def _fused_backward(x, w, grad_y, y, header, row_div, scale, form, want_x):
             _lib.check(entry(_lib.ptr(x), _row_stride(x), _lib.ptr(grad_y), _row_stride(grad_y), _lib.ptr(y),
                              n if y is not None else 0, _lib.ptr(row_div), scale, _lib.ptr(grad_z), _lib.ptr(grad_w),
                              _lib.ptr(grad_bias), _lib.ptr(workspace), nbytes, rows, k, n, stream))
-    grad_x = None
-    if want_x:
-        if form != FP32 and L.gnnagg_linear_shape_supported(n, k):
-            grad_x = _fused_product(grad_z, w.t().contiguous(), None, None, None, 1.0, False, form)
-        elif bf16:
-            grad_x = _Bf16InputLinear._mm(grad_z, w.t())
-        else:
-            grad_x = torch.mm(grad_z, w.t())
+    grad_x = input_gradient(grad_z, w, form) if want_x else None
     return grad_x, grad_w, grad_bias
 
 
