@@ -148,6 +148,39 @@ def test_train_step_matches_cpu_autograd(gemm, tol, fuse, linear_first, shape):
         assert float((p.detach() - b).abs().max()) <= 5 * 0.01 * 1.01
 
 
+@pytest.mark.parametrize("gemm", ["fp32", "bf16", "bf16x3"])
+@pytest.mark.parametrize("packed_activations", [False, True])
+def test_default_train_step_calls_no_library_product(gemm, packed_activations, monkeypatch):
+    """At the widths of the full train-step workload every dense product of the step -- layer products, weight
+    gradients, input gradients (the last layer's inner width 172 included) -- runs in libgnnagg's kernels: the step
+    goes through with torch's matrix products taken away."""
+    dev = "cuda:0"
+    n, dims, part_args = _SHAPES["c5_widths"]
+    part = synthetic.partition_edges(n, *part_args, seed=3, device=dev)
+    graph = synthetic.build_partition_graph(part, max(dims), True, exchange=synthetic.SeededHaloExchange(5), device=dev)
+    torch.manual_seed(0)
+    model = gcn.GCN(dims, gemm=gemm, packed_activations=packed_activations).to(dev)
+    opt = torch.optim.Adam(model.parameters(), lr=0.01)
+    gen = torch.Generator(device=dev).manual_seed(1)
+    x = torch.randn(n, dims[0], device=dev, generator=gen)
+    labels = torch.randint(0, dims[-1], (n,), device=dev, generator=gen)
+    train_idx = torch.randperm(n, device=dev, generator=gen)[: n // 10]
+    masks = gcn.make_dropout_masks(n, dims, 0.5, 7, dev)
+    want = float(gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks))
+
+    def taken_away(*a, **k):
+        raise AssertionError("a BLAS-library product inside the train step")
+
+    for name in ("mm", "addmm", "matmul", "bmm", "baddbmm", "einsum"):
+        monkeypatch.setattr(torch, name, taken_away)
+    monkeypatch.setattr(torch.Tensor, "__matmul__", taken_away)
+    monkeypatch.setattr(torch.nn.functional, "linear", taken_away)
+    for every_node in (False, True):
+        loss = float(gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks,
+                                    restrict_last_layer=not every_node))
+        assert np.isfinite(loss) and abs(loss - want) < 0.5
+
+
 @pytest.mark.parametrize("rows,feat", [(1000, 256), (333, 47), (64, 4), (1, 1)])
 @pytest.mark.parametrize("with_mask", [True, False])
 @pytest.mark.parametrize("with_div", [True, False])
