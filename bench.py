@@ -645,7 +645,8 @@ def run_c4(args, graph, setup_s):
     fp32_splits = graph.comm_splits
     graph.comm_splits = CommSplits(fp32_splits.recv_splits, fp32_splits.send_splits, world, 2)
     graph.comm_buf_for_quantization = CommBufferForQuantization(graph.comm_splits, feat, 2, device=dev)
-    graph.exchange_quantized = synthetic.SeededQuantizedHaloExchange(args.seed + 6)
+    graph.exchange_quantized = synthetic.PregeneratedQuantizedHaloExchange(args.seed + 6)
+    graph.fuse_dequantize = False   # the reference's form: a dequantise pass of its own into the fp32 buffer
     for _ in range(2):
         Aggregator.apply(graph, xr, 0, 2, True, True).backward(g)
     torch.cuda.synchronize()
@@ -655,7 +656,7 @@ def run_c4(args, graph, setup_s):
         o.backward(g)
     torch.cuda.synchronize()
     int2_both_ms = (time.perf_counter() - t0) * 1e3 / steps
-    # ... and with the received rows aggregated straight from the packed bytes (no dequantise pass)
+    # ... and with the received rows aggregated straight from the packed bytes (no dequantise pass; the default)
     graph.fuse_dequantize = True
     for _ in range(2):
         Aggregator.apply(graph, xr, 0, 2, True, True).backward(g)
@@ -679,7 +680,6 @@ def run_c4(args, graph, setup_s):
     codec.append({"op": "post-aggregation A_from@recv straight from the int2 bytes -> out", "bits": 2,
                   "rows_visited": m.sparse_size(0) - m.get_plan().info()["empty_rows"], "nnz": m.nnz(), "feat": feat,
                   "ms": round(e0.elapsed_time(e1) / steps, 4)})
-    graph.fuse_dequantize = False
     graph.comm_splits, graph.comm_buf_for_quantization, graph.exchange_quantized = fp32_splits, None, None
     # ... and as bf16 (num_bits=16): the two conversion passes per direction around a seeded stand-in
     from gnn_benchmark_amd.aggregator import _convert

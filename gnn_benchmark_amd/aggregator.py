@@ -145,10 +145,10 @@ def _quantize_and_exchange(graph, num_bits: int, tag: str, direction: str):
 
 
 def _fused_dequantize(graph, feat_len: int) -> bool:
-    """``graph.fuse_dequantize = True`` asks for the received rows to be aggregated straight from
-    the packed bytes (same values, no fp32 pass over the buffer; the fp32 buffer is then NOT
-    filled, unlike aggregator.py:85-88).  Needs a width that is a multiple of 4."""
-    return bool(getattr(graph, "fuse_dequantize", False)) and feat_len % 4 == 0
+    """Whether the received rows of a quantised exchange are aggregated straight from the packed bytes (the default:
+    same values, no fp32 pass over the buffer; the fp32 buffer is then NOT filled, unlike aggregator.py:85-88).
+    ``graph.fuse_dequantize = False`` keeps the dequantise pass of its own.  Needs a width that is a multiple of 4."""
+    return getattr(graph, "fuse_dequantize", True) is not False and feat_len % 4 == 0
 
 
 def _dequantize_received(graph, num_bits: int, direction: str) -> None:

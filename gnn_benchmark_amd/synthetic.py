@@ -280,6 +280,30 @@ class SeededQuantizedHaloExchange:
         return None
 
 
+class PregeneratedQuantizedHaloExchange(SeededQuantizedHaloExchange):
+    """The same seeded packed rows and parameters, drawn once per (tag, shape) and kept on the device; a later call
+    copies them into the receiving buffers (a device copy of the packed bytes, 1/16 of the fp32 rows at 2 bits) instead
+    of running the random-number kernels inside a timed step."""
+
+    def __init__(self, seed: int = 0):
+        super().__init__(seed)
+        self._kept = {}
+
+    def __call__(self, comm_splits, qbuf, tag: str, direction: str):
+        data = qbuf.quantized_recv_data_buf if direction == "forward" else qbuf.quantized_send_data_buf
+        params = qbuf.quantized_recv_params_buf_fp32 if direction == "forward" else qbuf.quantized_send_params_buf_fp32
+        key = (tag, tuple(data.shape), tuple(params.shape), str(data.device))
+        kept = self._kept.get(key)
+        if kept is None:
+            super().__call__(comm_splits, qbuf, tag, direction)
+            self._kept[key] = (data.clone(), params.clone())
+        else:
+            data.copy_(kept[0])
+            params.copy_(kept[1])
+            self.calls.append(tag)
+        return None
+
+
 class SeededBf16HaloExchange:
     """bf16 counterpart of SeededHaloExchange: fills the bf16 staging copy the aggregator widens."""
 

@@ -307,6 +307,7 @@ def test_quantised_exchange_world_matches_oracle(seed, sizes, bits):
         gr.exchange = lambda *a: (_ for _ in ()).throw(AssertionError("fp32 exchange used in a quantised run"))
         gr.exchange_quantized = PlayedQuantizedExchange((dev(fwd_data[r]), dev(fwd_params[r])),
                                                         (dev(bwd_data[r]), dev(bwd_params[r])))
+        gr.fuse_dequantize = False   # the reference's form: the received rows dequantised into the fp32 buffer
         xr = dev(x[sl[r]]).requires_grad_()
         out = Aggregator.apply(gr, xr, 1, bits, True, True)
         qb = gr.comm_buf_for_quantization
@@ -326,10 +327,10 @@ def test_quantised_exchange_world_matches_oracle(seed, sizes, bits):
             assert np.abs(out.detach().cpu().numpy() - want[sl[r]]).max() < 0.5
             assert np.abs(xr.grad.cpu().numpy() - want_t[sl[r]]).max() < 0.5
 
-    # the same run aggregating straight from the packed bytes: same outputs, bit for bit
+    # the same run aggregating straight from the packed bytes (the default): same outputs, bit for bit
     for r in range(W):
         gr, o = graphs[r], oracle_ranks[r]
-        gr.fuse_dequantize = True
+        del gr.fuse_dequantize
         gr.exchange_quantized = PlayedQuantizedExchange((dev(fwd_data[r]), dev(fwd_params[r])),
                                                         (dev(bwd_data[r]), dev(bwd_params[r])))
         gr.comm_buf.recv_buf.fill_(float("nan"))  # must not be read
@@ -633,6 +634,36 @@ def test_pregenerated_bf16_halo_rows_equal_the_seeded_ones(is_pre_delay):
         assert len(results[0]) == len(other)
         for a, b in zip(results[0], other):
             assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_pregenerated_quantized_halo_rows_equal_the_seeded_ones(fused):
+    """And for the int2 exchange: packed rows and parameters kept on the device and copied in give what drawing them
+    in every call gives, whether the received rows are aggregated from the packed bytes or dequantised first."""
+    from gnn_benchmark_amd import synthetic
+
+    n = 30_000
+    part = synthetic.partition_edges(n, 8, 5, 6.0, 1.8, 1500, 11_000, 70_000, seed=14, device="cuda")
+    results = []
+    for exchange_quantized in (synthetic.SeededQuantizedHaloExchange(9), synthetic.PregeneratedQuantizedHaloExchange(9)):
+        graph = synthetic.build_partition_graph(part, 96, True, exchange=synthetic.SeededHaloExchange(1), bits=2,
+                                                exchange_quantized=exchange_quantized, device="cuda")
+        graph.fuse_dequantize = fused
+        gen = torch.Generator(device="cuda").manual_seed(3)
+        seen = []
+        for call in range(3):
+            for layer, feat in ((0, 64), (1, 96)):
+                x = torch.randn(n, feat, device="cuda", generator=gen, requires_grad=True)
+                g = torch.randn(n, feat, device="cuda", generator=gen)
+                out = Aggregator.apply(graph, x, layer, 2, True, True)
+                out.backward(g)
+                seen += [out.detach().clone(), x.grad.clone()]
+        torch.cuda.synchronize()
+        assert exchange_quantized.calls == ["forward0", "backward0", "forward1", "backward1"] * 3
+        results.append(seen)
+    assert len(results[0]) == len(results[1])
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
 
 
 def test_bad_indices_raise_instead_of_reading_out_of_bounds():
