@@ -646,7 +646,8 @@ def run_c4(args, graph, setup_s):
     graph.comm_splits = CommSplits(fp32_splits.recv_splits, fp32_splits.send_splits, world, 2)
     graph.comm_buf_for_quantization = CommBufferForQuantization(graph.comm_splits, feat, 2, device=dev)
     graph.exchange_quantized = synthetic.PregeneratedQuantizedHaloExchange(args.seed + 6)
-    graph.fuse_dequantize = False   # the reference's form: a dequantise pass of its own into the fp32 buffer
+    # the reference's form: the outgoing rows quantised out of the fp32 buffer, the received ones dequantised into it
+    graph.fuse_dequantize = graph.fuse_quantize = False
     for _ in range(2):
         Aggregator.apply(graph, xr, 0, 2, True, True).backward(g)
     torch.cuda.synchronize()
@@ -656,8 +657,9 @@ def run_c4(args, graph, setup_s):
         o.backward(g)
     torch.cuda.synchronize()
     int2_both_ms = (time.perf_counter() - t0) * 1e3 / steps
-    # ... and with the received rows aggregated straight from the packed bytes (no dequantise pass; the default)
-    graph.fuse_dequantize = True
+    # ... and as it runs by default: the products in front of the exchange write the packed rows themselves, the
+    # products behind it aggregate straight from the packed bytes (no quantise pass, no dequantise pass)
+    graph.fuse_dequantize = graph.fuse_quantize = True
     for _ in range(2):
         Aggregator.apply(graph, xr, 0, 2, True, True).backward(g)
     torch.cuda.synchronize()
@@ -680,6 +682,25 @@ def run_c4(args, graph, setup_s):
     codec.append({"op": "post-aggregation A_from@recv straight from the int2 bytes -> out", "bits": 2,
                   "rows_visited": m.sparse_size(0) - m.get_plan().info()["empty_rows"], "nnz": m.nnz(), "feat": feat,
                   "ms": round(e0.elapsed_time(e1) / steps, 4)})
+    from gnn_benchmark_amd import computation_ops
+
+    m = graph.adj_t_pre_post_aggr_to
+    rp, cidx, vals = m.csr()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for i in range(steps + 2):
+        if i == 2:
+            e0.record()
+        computation_ops.spmm_quantize_for_all_procs(rp, cidx, vals, x, qb.quantized_send_data_buf,
+                                                    qb.quantized_send_params_buf_fp32, qb.quantized_work_range_per_proc,
+                                                    world, 2)
+    e1.record()
+    e1.synchronize()
+    ms = e0.elapsed_time(e1) / steps
+    gathered = m.nnz() * (4.0 * feat + 12.0) + m.sparse_size(0) * (8.0 + 8.0 + feat / 4.0)
+    codec.append({"op": "pre-aggregation A_to@X straight into the int2 bytes (natural row order, int64 column indices)",
+                  "bits": 2, "rows": m.sparse_size(0), "nnz": m.nnz(), "feat": feat, "ms": round(ms, 4),
+                  "bytes_model": gathered, "gbs_model": round(gathered / (ms * 1e-3) / 1e9, 1),
+                  "frac_model": round(gathered / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)})
     graph.comm_splits, graph.comm_buf_for_quantization, graph.exchange_quantized = fp32_splits, None, None
     # ... and as bf16 (num_bits=16): the two conversion passes per direction around a seeded stand-in
     from gnn_benchmark_amd.aggregator import _convert
@@ -748,8 +769,8 @@ def run_c4(args, graph, setup_s):
             "aggregator_forward_backward_ms": round(both_ms, 3),
             "aggregator_forward_backward_ms_bf16_exchange": round(bf16_both_ms, 3),
             "aggregator_forward_backward_ms_bf16_exchange_separate_copies": round(bf16_unfused_ms, 3),
-            "aggregator_forward_backward_ms_int2_exchange": round(int2_both_ms, 3),
-            "aggregator_forward_backward_ms_int2_exchange_fused_dequantize": round(int2_fused_ms, 3)}
+            "aggregator_forward_backward_ms_int2_exchange": round(int2_fused_ms, 3),
+            "aggregator_forward_backward_ms_int2_exchange_separate_codec_passes": round(int2_both_ms, 3)}
 
 
 def cpu_time_codec(x_host, bits, reps=2):

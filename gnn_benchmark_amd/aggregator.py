@@ -127,18 +127,44 @@ def _convert(src: torch.Tensor, dst: torch.Tensor) -> None:
             raise RuntimeError("Input mismatch: bf16 staging converts float32 <-> bfloat16 only")
 
 
-def _quantize_and_exchange(graph, num_bits: int, tag: str, direction: str):
-    """Pack the outgoing rows per peer rank and hand the bytes to the exchange
+def _outgoing_quantized(graph, direction: str):
+    """(fp32 rows, packed bytes, parameters, per-rank row prefix) of the outgoing side of a quantised exchange."""
+    qbuf = graph.comm_buf_for_quantization
+    if direction == "forward":
+        return (graph.comm_buf.send_buf, qbuf.quantized_send_data_buf, qbuf.quantized_send_params_buf_fp32,
+                qbuf.quantized_work_range_per_proc)
+    return (graph.comm_buf.recv_buf, qbuf.quantized_recv_data_buf, qbuf.quantized_recv_params_buf_fp32,
+            qbuf.dequantized_work_range_per_proc)
+
+
+def _product_into_packed_rows(graph, csr, dense: torch.Tensor, num_bits: int, direction: str) -> bool:
+    """The product in front of a quantised exchange writing the packed bytes and parameters itself
+    (``computation_ops.spmm_quantize_for_all_procs``: same bytes as the product followed by the quantise pass, without the
+    fp32 rows; the fp32 buffer is then NOT filled).  The default; ``graph.fuse_quantize = False`` keeps the two passes.
+    ``csr``: (rowptr, col, value) of the matrix whose rows are the outgoing rows.  False when nothing was done."""
+    if getattr(graph, "fuse_quantize", True) is False or dense.dtype != torch.float32 or csr[2] is None:
+        return False
+    _, data, params, work_range = _outgoing_quantized(graph, direction)
+    if csr[0].numel() - 1 == 0:
+        return False
+    world = len(graph.comm_splits.send_splits)
+    return computation_ops.spmm_quantize_for_all_procs(csr[0], csr[1], csr[2], dense, data, params, work_range, world,
+                                                        num_bits)
+
+
+def _transposed_csr(m: SparseTensor):
+    s = m.storage
+    return s.colptr(), s.row_T(), s.value_T()
+
+
+def _quantize_and_exchange(graph, num_bits: int, tag: str, direction: str, already_packed: bool = False):
+    """Pack the outgoing rows per peer rank (unless the product wrote them packed) and hand the bytes to the exchange
     (communicator.py:241-311)."""
     qbuf = graph.comm_buf_for_quantization
     world = len(graph.comm_splits.send_splits)
-    if direction == "forward":
-        outgoing, data, params, work_range = (graph.comm_buf.send_buf, qbuf.quantized_send_data_buf,
-                                              qbuf.quantized_send_params_buf_fp32, qbuf.quantized_work_range_per_proc)
-    else:
-        outgoing, data, params, work_range = (graph.comm_buf.recv_buf, qbuf.quantized_recv_data_buf,
-                                              qbuf.quantized_recv_params_buf_fp32,
-                                              qbuf.dequantized_work_range_per_proc)
+    if already_packed:
+        return graph.exchange_quantized(graph.comm_splits, qbuf, tag, direction)
+    outgoing, data, params, work_range = _outgoing_quantized(graph, direction)
     if outgoing.size(0) != 0:
         computation_ops.quantize_tensor_for_all_procs(outgoing, data, params, work_range, world, num_bits)
     return graph.exchange_quantized(graph.comm_splits, qbuf, tag, direction)
@@ -248,12 +274,17 @@ def _forward(ctx, graph, feats, layer, num_bits: int, is_pre_delay: bool, is_tra
 
     half_fused = half and isinstance(feats, _DenseFeatures) and _bf16_in_the_products(graph, feats, feat_len)
     if exchange is not None:
-        if is_pre_delay:  # pre-aggregation: send_buf = A_to @ X (straight into the bf16 staging rows when they travel)
-            feats.product(graph.adj_t_pre_post_aggr_to, graph.comm_buf.send_buf_fp16 if half_fused else send_buf, False)
+        packed_by_product = False
+        if is_pre_delay:  # pre-aggregation: send_buf = A_to @ X (straight into the rows that travel, bf16 or packed)
+            if quantized and isinstance(feats, _DenseFeatures) and send_buf.size(0) != 0:
+                packed_by_product = _product_into_packed_rows(graph, graph.adj_t_pre_post_aggr_to.csr(), feats.feat,
+                                                              num_bits, "forward")
+            if not packed_by_product:
+                feats.product(graph.adj_t_pre_post_aggr_to, graph.comm_buf.send_buf_fp16 if half_fused else send_buf, False)
         else:  # raw boundary rows (as bf16 at once when they travel so)
             feats.gather(graph.idx_nodes_send_to_others, graph.comm_buf.send_buf_fp16 if half_fused else send_buf)
         if quantized:
-            comm_handle = _quantize_and_exchange(graph, num_bits, f"forward{layer}", "forward")
+            comm_handle = _quantize_and_exchange(graph, num_bits, f"forward{layer}", "forward", packed_by_product)
         elif half:
             if not half_fused:
                 _convert(send_buf, graph.comm_buf.send_buf_fp16)
@@ -418,17 +449,22 @@ def _backward(ctx, local_out_grad, out=None, accumulate: bool = False):
     half_fused = half and not quantized and _bf16_in_the_products(graph, local_out_grad, feat_len)
     # the outgoing halo gradients: straight into the bf16 staging rows when they travel as bf16
     remote_nodes_grad_buf = graph.comm_buf.recv_buf_fp16 if half_fused else graph.comm_buf.recv_buf
+    packed_by_product = False
     if remote_nodes_grad_buf.size(0) != 0:
-        if support is not None:
+        remote = graph.adj_t_pre_post_aggr_from if is_pre_delay else graph.remote_adj_t
+        if quantized:  # straight into the packed rows that travel
+            csr = support.remote_T.csr() if support is not None else _transposed_csr(remote)
+            packed_by_product = _product_into_packed_rows(graph, csr, local_out_grad, num_bits, "backward")
+        if packed_by_product:
+            pass
+        elif support is not None:
             SPMM_forward(support.remote_T, local_out_grad, remote_nodes_grad_buf, accumulate=False)
-        elif is_pre_delay:
-            SPMM_backward(graph.adj_t_pre_post_aggr_from, local_out_grad, remote_nodes_grad_buf, accumulate=False)
         else:
-            SPMM_backward(graph.remote_adj_t, local_out_grad, remote_nodes_grad_buf, accumulate=False)
+            SPMM_backward(remote, local_out_grad, remote_nodes_grad_buf, accumulate=False)
 
     comm_handle = None
     if quantized:
-        comm_handle = _quantize_and_exchange(graph, num_bits, layer, "backward")
+        comm_handle = _quantize_and_exchange(graph, num_bits, layer, "backward", packed_by_product)
     elif half:  # the buffers swap roles on the way back (communicator.py:121-126)
         if not half_fused:
             _convert(remote_nodes_grad_buf, graph.comm_buf.recv_buf_fp16)

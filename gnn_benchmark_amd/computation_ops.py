@@ -134,6 +134,45 @@ def quantize_tensor_for_all_procs(input: torch.Tensor, output: torch.Tensor, qua
             num_procs, rows, packed_rows, input.size(1), bits, _lib.current_stream(dev)))
 
 
+def spmm_quantize_for_all_procs(rowptr: torch.Tensor, col: torch.Tensor, value: torch.Tensor, mat: torch.Tensor,
+                                output: torch.Tensor, quantized_params: torch.Tensor,
+                                work_range_per_proc: torch.Tensor, num_procs: int, bits: int) -> bool:
+    """``quantize_tensor_for_all_procs(A @ mat, output, ...)`` in one pass: the rows of the product are quantised out
+    of the registers they were summed in, bytes and parameters equal to the two calls' (aggregator.py:44-49 then
+    communicator.py:281-311).  ``rowptr`` / ``col`` int64 and ``value`` float32 are A's CSR arrays.  Returns False,
+    with nothing done, for operands the one-pass kernel does not take (width no multiple of 4 or above 512, rows of
+    ``mat`` off 16-byte boundaries): the caller then runs the two calls."""
+    _require(bits in (2, 4, 8), "bits must be 2, 4 or 8")
+    for t, name in ((rowptr, "rowptr"), (col, "col"), (value, "value"), (mat, "dense operand"), (output, "packed buffer"),
+                    (quantized_params, "quantisation parameters")):
+        _require_hip(t, name, mat.device if mat.is_cuda else None)
+    dev = mat.device
+    rows = rowptr.numel() - 1
+    feat = mat.size(1) if mat.dim() == 2 else -1
+    _require(rowptr.dtype == torch.int64 and col.dtype == torch.int64 and value.dtype == torch.float32
+             and rowptr.is_contiguous() and col.is_contiguous() and value.is_contiguous()
+             and value.numel() == col.numel(), "CSR arrays must be contiguous int64 / int64 / float32")
+    _require(mat.dtype == torch.float32 and mat.dim() == 2 and mat.stride(1) == 1 and mat.stride(0) >= feat,
+             "dense operand must be float32 2-D with contiguous rows")
+    _require(output.dtype == torch.uint8 and output.is_contiguous(), "packed buffer must be contiguous uint8")
+    _require(quantized_params.dtype == torch.float32 and quantized_params.is_contiguous()
+             and quantized_params.dim() == 2 and quantized_params.size(0) >= rows and quantized_params.size(1) == 2,
+             "parameters must be contiguous float32 [rows, 2]")
+    _require(work_range_per_proc.numel() == num_procs + 1, "work range must hold num_procs + 1 entries")
+    rows_d, packed_d, packed_rows, covered = _packed_range(work_range_per_proc, bits, dev)
+    _require(covered == rows, "work range does not cover the product's rows")
+    _require(output.numel() >= packed_rows * feat, "packed buffer too small")
+    if feat % 4 != 0 or feat > 512 or mat.stride(0) % 4 != 0 or mat.data_ptr() % 16 != 0 or output.data_ptr() % 4 != 0:
+        return False
+    _lib.check_index(col, mat.size(0), what="column indices of the sparse matrix")
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().gnnagg_spmm_csr_quantize_segments_f32(
+            _lib.ptr(rowptr), _lib.ptr(col), _lib.ptr(value), _lib.ptr(mat), mat.stride(0), _lib.ptr(output),
+            _lib.ptr(quantized_params), _lib.ptr(rows_d), _lib.ptr(packed_d), num_procs, rows, packed_rows, feat, bits,
+            _lib.current_stream(dev)))
+    return True
+
+
 def dequantize_tensor_for_all_procs(input: torch.Tensor, output: torch.Tensor, dequantized_params: torch.Tensor,
                                     work_range_per_proc: torch.Tensor, num_procs: int, bits: int) -> None:
     """Inverse of ``quantize_tensor_for_all_procs`` (quantization_arm.cpp:437-479):

@@ -354,6 +354,115 @@ __global__ __launch_bounds__(256) void dequantize_segments_kernel(const uint8_t 
     }
 }
 
+// ---- a product whose result rows leave quantised: packed = quantize(A @ X), segment by segment
+//
+// The pre-aggregation in front of a quantised exchange (model/layers/aggregator.py:44-49 followed by
+// communicator/communicator.py:281-311) as one pass: a lane group owns one packed row at a time, computes the 8/bits
+// fp32 rows that share its bytes one after the other -- each row the same single FMA chain over its stored elements,
+// in their order, that the product kernels run -- and quantises every finished row out of its registers with the
+// functions of the codec above, so parameters and bytes equal those of product-then-quantise while the fp32 rows are
+// never written or read back.  Rows are walked in their natural order (the bytes of a packed row belong to
+// consecutive rows); LPR lanes x NCH loads x 4 floats cover a row.
+template <int BITS, int LPR, int NCH>
+__global__ __launch_bounds__(256) void spmm_quantize_segments_kernel(
+    const int64_t *__restrict__ rowptr, const int64_t *__restrict__ col, const float *__restrict__ val,
+    const float *__restrict__ x, int ldx, uint8_t *__restrict__ packed, float *__restrict__ params,
+    const int32_t *__restrict__ row_range, const int32_t *__restrict__ packed_range, int segments, int rows,
+    int packed_rows, int feat) {
+    constexpr int EPB = 8 / BITS;
+    constexpr int GPB = 256 / LPR;
+    constexpr int U = NCH == 1 ? 8 : 4;  // gathers in flight per lane group
+    extern __shared__ int32_t range_lds[];
+    const int32_t *rr, *pr;
+    stage_ranges(row_range, packed_range, segments, range_lds, rr, pr);
+
+    const int lig = (int)threadIdx.x & (LPR - 1);
+    const int group = (int)threadIdx.x / LPR;
+    int foff[NCH];
+    bool fok[NCH];
+#pragma unroll
+    for (int k = 0; k < NCH; ++k) {
+        const int f = (k * LPR + lig) * 4;
+        fok[k] = f < feat;
+        foff[k] = fok[k] ? f : 0;  // lanes past the row keep a valid address; their values are never used
+    }
+
+    // Whole lane groups leave together, and no barrier follows the staging above.
+    for (int it = 0; it < kCodecIters; ++it) {
+        const int g = (int)(((int64_t)blockIdx.x * kCodecIters + it) * GPB + group);
+        if (g >= packed_rows) break;
+        const RowGroup rg = locate_group<EPB>(rr, pr, segments, g, rows, packed_rows);
+        // the extents of the group's rows: lane k holds rowptr[first + k], k <= count
+        const int64_t ext = lig <= rg.count && rg.count > 0 ? rowptr[rg.first + lig] : 0;
+        uint32_t word[NCH];
+#pragma unroll
+        for (int k = 0; k < NCH; ++k) word[k] = 0;
+        for (int r = 0; r < rg.count; ++r) {
+            const int64_t begin = __shfl(ext, r, LPR), end = __shfl(ext, r + 1, LPR);
+            f4 acc[NCH];
+#pragma unroll
+            for (int k = 0; k < NCH; ++k) acc[k] = f4{0.0f, 0.0f, 0.0f, 0.0f};
+            for (int64_t e0 = begin; e0 < end; e0 += LPR) {
+                const int n = (int)(end - e0 < LPR ? end - e0 : LPR);
+                // one coalesced fetch of up to LPR (column, value) pairs, handed round below
+                const int64_t c_mine = lig < n ? col[e0 + lig] : 0;
+                const float v_mine = lig < n ? val[e0 + lig] : 0.0f;
+                for (int j0 = 0; j0 < n; j0 += U) {
+                    f4 xv[U][NCH];
+                    float vv[U];
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        // a surplus gather reads row 0 (a valid address); its result never enters the chain
+                        const int64_t cc = j0 + u < n ? __shfl(c_mine, j0 + u, LPR) : 0;
+                        vv[u] = __shfl(v_mine, j0 + u < n ? j0 + u : 0, LPR);
+                        const float *xr = x + (size_t)cc * (size_t)ldx;
+#pragma unroll
+                        for (int k = 0; k < NCH; ++k) xv[u][k] = *reinterpret_cast<const f4 *>(xr + foff[k]);
+                    }
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        if (j0 + u < n) {
+#pragma unroll
+                            for (int k = 0; k < NCH; ++k) {
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) acc[k][e] = __builtin_fmaf(vv[u], xv[u][k][e], acc[k][e]);
+                            }
+                        }
+                    }
+                }
+            }
+            // the finished row: parameters, then its codes into the bytes it shares
+            float lo = INFINITY, hi = -INFINITY;
+#pragma unroll
+            for (int k = 0; k < NCH; ++k) {
+                if (fok[k]) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        lo = fminf(lo, acc[k][e]);
+                        hi = fmaxf(hi, acc[k][e]);
+                    }
+                }
+            }
+            group_min_max<LPR>(lo, hi);
+            float zp, scale;
+            params_of(lo, hi, BITS, zp, scale);
+            const float inv = __builtin_amdgcn_rcpf(scale);
+            if (lig == 0) *reinterpret_cast<float2 *>(params + (size_t)(rg.first + r) * 2) = make_float2(zp, scale);
+#pragma unroll
+            for (int k = 0; k < NCH; ++k) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    word[k] |= ((quantize_one_fast(acc[k][e], zp, scale, inv) << ((EPB - r - 1) * BITS)) & 0xFFu) << (8 * e);
+            }
+        }
+        if (rg.count > 0) {
+#pragma unroll
+            for (int k = 0; k < NCH; ++k)
+                if (fok[k]) *reinterpret_cast<uint32_t *>(packed + (size_t)g * (size_t)feat + foff[k]) = word[k];
+        }
+    }
+}
+
 // ---- mixed bits: one wavefront per row, width read from params[row][0]
 
 __global__ __launch_bounds__(256) void quantize_mixed_kernel(const float *__restrict__ x, uint8_t *__restrict__ data,
@@ -555,6 +664,42 @@ extern "C" int gnnagg_quantize_segments_f32(const float *x, uint8_t *packed, flo
     }
     GNNAGG_Q(2) GNNAGG_Q(4) GNNAGG_Q(8)
 #undef GNNAGG_Q
+    GNNAGG_HIP(hipGetLastError());
+    return GNNAGG_OK;
+}
+
+extern "C" int gnnagg_spmm_csr_quantize_segments_f32(const int64_t *rowptr, const int64_t *col, const float *value,
+                                                     const float *mat, int64_t mat_stride, uint8_t *packed,
+                                                     float *params, const int32_t *row_range,
+                                                     const int32_t *packed_range, int64_t segments, int64_t rows,
+                                                     int64_t packed_rows, int64_t feat, int bits, void *stream) {
+    const int rc = check_segments(mat, packed, params, row_range, packed_range, segments, rows, packed_rows, feat, bits);
+    if (rc != GNNAGG_OK || rows == 0 || feat == 0) return rc;
+    GNNAGG_REQUIRE(rowptr && col && value, "null rowptr/col/value");
+    GNNAGG_REQUIRE(mat_stride >= feat && mat_stride < (int64_t(1) << 31), "row stride %lld must be at least the width %lld "
+                   "and below 2^31", (long long)mat_stride, (long long)feat);
+    if (feat % 4 != 0 || feat > 512 || mat_stride % 4 != 0 || !aligned16(mat) || !aligned4(packed))
+        return fail(GNNAGG_ERR_UNSUPPORTED, "the product with quantised result rows takes widths that are multiples of 4 "
+                    "up to 512 (got %lld), rows of the dense operand on 16-byte boundaries and a 4-byte aligned result",
+                    (long long)feat);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const size_t lds = range_lds_bytes((int)segments);
+    const int nvec = (int)(feat / 4);
+#define GNNAGG_PQ(B, LPR, NCH)                                                                                       \
+    hipLaunchKernelGGL((spmm_quantize_segments_kernel<B, LPR, NCH>),                                                 \
+                       dim3(grid_for(packed_rows, (256 / LPR) * kCodecIters)), dim3(256), lds, st, rowptr, col, value, \
+                       mat, (int)mat_stride, packed, params, row_range, packed_range, (int)segments, (int)rows,      \
+                       (int)packed_rows, (int)feat)
+#define GNNAGG_PQ_BITS(B)                             \
+    if (bits == B) {                                  \
+        if (nvec <= 16) GNNAGG_PQ(B, 16, 1);          \
+        else if (nvec <= 32) GNNAGG_PQ(B, 32, 1);     \
+        else if (nvec <= 64) GNNAGG_PQ(B, 64, 1);     \
+        else GNNAGG_PQ(B, 64, 2);                     \
+    }
+    GNNAGG_PQ_BITS(2) GNNAGG_PQ_BITS(4) GNNAGG_PQ_BITS(8)
+#undef GNNAGG_PQ_BITS
+#undef GNNAGG_PQ
     GNNAGG_HIP(hipGetLastError());
     return GNNAGG_OK;
 }

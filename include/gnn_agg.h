@@ -420,6 +420,20 @@ int gnnagg_quantize_segments_f32(const float *x, uint8_t *packed, float *params,
 int gnnagg_dequantize_segments_f32(const uint8_t *packed, const float *params, float *out, const int32_t *row_range,
                                    const int32_t *packed_range, int64_t segments, int64_t rows, int64_t packed_rows,
                                    int64_t feat, int bits, void *stream);
+/* Pre-aggregation straight into the packed bytes: packed / params = quantize(A @ mat), every segment on its own --
+ * `send_buf += A_to @ X` followed by `quantize_tensor_for_all_procs(send_buf, ...)` (model/layers/aggregator.py:44-49,
+ * communicator/communicator.py:281-311; backward: :144-149 with the buffers' roles swapped) as one pass.  A is given as
+ * CSR arrays (rowptr int64 [rows + 1], col int64, value fp32; the transposed arrays for the gradient direction), mat
+ * fp32 with row stride mat_stride; the other arguments are gnnagg_quantize_segments_f32's.  Every result row is the
+ * single FMA chain over its stored elements, in their order, that gnnagg_plan_spmm_f32 runs, and is quantised by the
+ * same arithmetic, so parameters and bytes equal those of the two calls bit for bit while the fp32 rows are never
+ * written or read.  feat a multiple of 4 up to 512, mat rows on 16-byte boundaries (GNNAGG_ERR_UNSUPPORTED otherwise:
+ * use the two calls).  Column indices are not range-checked here (gnnagg_check_index).  No allocation, no host
+ * synchronisation. */
+int gnnagg_spmm_csr_quantize_segments_f32(const int64_t *rowptr, const int64_t *col, const float *value,
+                                          const float *mat, int64_t mat_stride, uint8_t *packed, float *params,
+                                          const int32_t *row_range, const int32_t *packed_range, int64_t segments,
+                                          int64_t rows, int64_t packed_rows, int64_t feat, int bits, void *stream);
 /* Post-aggregation straight from the packed bytes: gnnagg_plan_spmm_f32 whose dense operand
  * row c is given quantised -- packed / params as written by gnnagg_quantize_segments_f32 (or
  * received from a peer), row_code int32 [rows of the operand] = packed_row * 8 + position of

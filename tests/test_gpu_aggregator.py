@@ -307,7 +307,9 @@ def test_quantised_exchange_world_matches_oracle(seed, sizes, bits):
         gr.exchange = lambda *a: (_ for _ in ()).throw(AssertionError("fp32 exchange used in a quantised run"))
         gr.exchange_quantized = PlayedQuantizedExchange((dev(fwd_data[r]), dev(fwd_params[r])),
                                                         (dev(bwd_data[r]), dev(bwd_params[r])))
-        gr.fuse_dequantize = False   # the reference's form: the received rows dequantised into the fp32 buffer
+        # the reference's form: the outgoing rows summed into the fp32 buffer and quantised from there, the received
+        # rows dequantised into the fp32 buffer
+        gr.fuse_dequantize = gr.fuse_quantize = False
         xr = dev(x[sl[r]]).requires_grad_()
         out = Aggregator.apply(gr, xr, 1, bits, True, True)
         qb = gr.comm_buf_for_quantization
@@ -327,23 +329,33 @@ def test_quantised_exchange_world_matches_oracle(seed, sizes, bits):
             assert np.abs(out.detach().cpu().numpy() - want[sl[r]]).max() < 0.5
             assert np.abs(xr.grad.cpu().numpy() - want_t[sl[r]]).max() < 0.5
 
-    # the same run aggregating straight from the packed bytes (the default): same outputs, bit for bit
+    # the same run as it runs by default -- the products in front of the exchange writing the packed rows themselves,
+    # the products behind it aggregating straight from the packed bytes: same bytes sent, same outputs, bit for bit,
+    # and the fp32 boundary buffers neither written nor read
     for r in range(W):
         gr, o = graphs[r], oracle_ranks[r]
-        del gr.fuse_dequantize
+        del gr.fuse_dequantize, gr.fuse_quantize
         gr.exchange_quantized = PlayedQuantizedExchange((dev(fwd_data[r]), dev(fwd_params[r])),
                                                         (dev(bwd_data[r]), dev(bwd_params[r])))
-        gr.comm_buf.recv_buf.fill_(float("nan"))  # must not be read
+        qb = gr.comm_buf_for_quantization
+        gr.comm_buf.recv_buf.fill_(float("nan"))
         gr.comm_buf.send_buf.fill_(float("nan"))
+        qb.quantized_send_data_buf.fill_(0x5A)
+        qb.quantized_recv_data_buf.fill_(0x5A)
         xr = dev(x[sl[r]]).requires_grad_()
         out = Aggregator.apply(gr, xr, 1, bits, True, True)
+        assert np.array_equal(qb.quantized_send_data_buf.cpu().numpy(), q_send[r][0])
+        assert np.array_equal(qb.quantized_send_params_buf_fp32.cpu().numpy(), q_send[r][1])
         o_out = oagg.forward_out(o["local"], o["a_from"], np.ascontiguousarray(x[sl[r]]), recv[r])
         assert np.array_equal(out.detach().cpu().numpy(), o_out)
-        gr.comm_buf.send_buf.fill_(float("nan"))
         out.backward(dev(g[sl[r]]))
+        assert np.array_equal(qb.quantized_recv_data_buf.cpu().numpy(), q_back[r][0])
+        assert np.array_equal(qb.quantized_recv_params_buf_fp32.cpu().numpy(), q_back[r][1])
         o_dx = oagg.backward_out(o["local"], o["a_to"], np.ascontiguousarray(g[sl[r]]), incoming[r])
         assert np.array_equal(xr.grad.cpu().numpy(), o_dx)
-        gr.fuse_dequantize = False
+        for buf in (gr.comm_buf.recv_buf, gr.comm_buf.send_buf):
+            assert buf.numel() == 0 or bool(torch.isnan(buf).all())
+        gr.fuse_dequantize = gr.fuse_quantize = False
 
     # outside training the forward exchange carries fp32 rows (communicator.py:64-65)
     gr = graphs[0]

@@ -251,6 +251,70 @@ def test_aggregation_straight_from_packed_bytes_equals_dequantise_then_aggregate
     assert torch.equal(got3, want3)
 
 
+@pytest.mark.parametrize("bits", [2, 4, 8])
+@pytest.mark.parametrize("feat", [4, 48, 64, 100, 128, 132, 256, 260, 512])
+def test_product_with_quantised_result_rows_equals_product_then_quantise(bits, feat):
+    """``spmm_quantize_for_all_procs`` (the pre-aggregation writing the packed bytes itself) against ``SPMM_forward``
+    followed by ``quantize_tensor_for_all_procs``: bytes and parameters bit for bit -- ragged matrix with long rows
+    (several index chunks) and empty rows, segments whose heights are no multiples of the rows a byte holds, an empty
+    segment, a dense operand that is a column block of a wider array -- and against the oracle's bytes."""
+    from gnn_benchmark_amd import SPMM_forward
+    from gnn_benchmark_amd import computation_ops as ops
+    from gnn_benchmark_amd.data_manager import CommBufferForQuantization, CommSplits
+    from gnn_benchmark_amd.sparse_tensor import SparseTensor
+    from tests.gpu_util import skewed_csr
+
+    rng = np.random.default_rng(1000 * bits + feat)
+    send_rows, local = 703, 450
+    rowptr, col, val = skewed_csr(send_rows, local, seed=feat + bits)
+    adj = SparseTensor(rowptr=dev(rowptr), col=dev(col), value=dev(val), sparse_sizes=(send_rows, local), is_sorted=True)
+    splits = [121, 0, 78, 504]
+    cs = CommSplits([5, 5, 5, 5], splits, 4, bits)
+    for strided in (False, True):
+        wide = dev(_rows(rng, local, feat + 8))
+        x = wide[:, 4:4 + feat] if strided else wide[:, :feat].contiguous()
+        two = CommBufferForQuantization(cs, feat, bits, device="cuda")
+        one = CommBufferForQuantization(cs, feat, bits, device="cuda")
+        for q in (one, two):   # whatever neither path writes stays equal
+            q.quantized_send_data_buf.fill_(0xAB)
+            q.quantized_send_params_buf_fp32.fill_(-7.0)
+        send = torch.empty(send_rows, feat, device="cuda")
+        SPMM_forward(adj, x, send, accumulate=False)
+        ops.quantize_tensor_for_all_procs(send, two.quantized_send_data_buf, two.quantized_send_params_buf_fp32,
+                                          two.quantized_work_range_per_proc, 4, bits)
+        rp, c, v = adj.csr()
+        done = ops.spmm_quantize_for_all_procs(rp, c, v, x, one.quantized_send_data_buf,
+                                               one.quantized_send_params_buf_fp32, one.quantized_work_range_per_proc, 4,
+                                               bits)
+        assert done
+        assert torch.equal(one.quantized_send_params_buf_fp32, two.quantized_send_params_buf_fp32)
+        assert torch.equal(one.quantized_send_data_buf, two.quantized_send_data_buf)
+        o_bytes, o_params = oq.quantize_segments(send.cpu().numpy(), splits, bits)
+        assert np.array_equal(one.quantized_send_data_buf.cpu().numpy().reshape(-1)[:o_bytes.size], o_bytes.reshape(-1))
+        assert np.array_equal(one.quantized_send_params_buf_fp32.cpu().numpy(), o_params)
+
+
+def test_product_with_quantised_result_rows_leaves_other_widths_to_the_two_calls():
+    from gnn_benchmark_amd import computation_ops as ops
+    from gnn_benchmark_amd.data_manager import CommBufferForQuantization, CommSplits
+
+    cs = CommSplits([1], [3], 1, 2)
+    rp = torch.tensor([0, 1, 2, 2], device="cuda")
+    c = torch.tensor([0, 1], device="cuda")
+    v = torch.ones(2, device="cuda")
+    for feat in (6, 516):
+        q = CommBufferForQuantization(cs, feat, 2, device="cuda")
+        before = q.quantized_send_data_buf.clone()
+        assert not ops.spmm_quantize_for_all_procs(rp, c, v, torch.ones(2, feat, device="cuda"), q.quantized_send_data_buf,
+                                                   q.quantized_send_params_buf_fp32, q.quantized_work_range_per_proc, 1, 2)
+        assert torch.equal(q.quantized_send_data_buf, before)
+    q = CommBufferForQuantization(cs, 8, 2, device="cuda")
+    with pytest.raises(RuntimeError, match="outside"):   # a column index beyond the dense operand's rows
+        ops.spmm_quantize_for_all_procs(rp, torch.tensor([0, 2], device="cuda"), v, torch.ones(2, 8, device="cuda"),
+                                        q.quantized_send_data_buf, q.quantized_send_params_buf_fp32,
+                                        q.quantized_work_range_per_proc, 1, 2)
+
+
 def test_quantised_aggregation_error_behaviour():
     from gnn_benchmark_amd.data_manager import CommBufferForQuantization, CommSplits
     from gnn_benchmark_amd.sparse_tensor import SparseTensor
