@@ -392,46 +392,23 @@ __global__ __launch_bounds__(256) void spmm_quantize_segments_kernel(
         const int g = (int)(((int64_t)blockIdx.x * kCodecIters + it) * GPB + group);
         if (g >= packed_rows) break;
         const RowGroup rg = locate_group<EPB>(rr, pr, segments, g, rows, packed_rows);
-        // the extents of the group's rows: lane k holds rowptr[first + k], k <= count
-        const int64_t ext = lig <= rg.count && rg.count > 0 ? rowptr[rg.first + lig] : 0;
+        if (rg.count == 0) continue;
+        // the extents of the group's rows: lane k holds rowptr[first + k], k <= count.  The rows are consecutive, so
+        // their stored elements are one stretch [begin, end) of the index arrays, walked below as one stream with up
+        // to U gathers in flight whatever row they belong to; a row is closed when the stream passes its end.
+        const int64_t ext = lig <= rg.count ? rowptr[rg.first + lig] : 0;
+        const int64_t begin = __shfl(ext, 0, LPR), end = __shfl(ext, rg.count, LPR);
         uint32_t word[NCH];
+        f4 acc[NCH];
 #pragma unroll
-        for (int k = 0; k < NCH; ++k) word[k] = 0;
-        for (int r = 0; r < rg.count; ++r) {
-            const int64_t begin = __shfl(ext, r, LPR), end = __shfl(ext, r + 1, LPR);
-            f4 acc[NCH];
-#pragma unroll
-            for (int k = 0; k < NCH; ++k) acc[k] = f4{0.0f, 0.0f, 0.0f, 0.0f};
-            for (int64_t e0 = begin; e0 < end; e0 += LPR) {
-                const int n = (int)(end - e0 < LPR ? end - e0 : LPR);
-                // one coalesced fetch of up to LPR (column, value) pairs, handed round below
-                const int64_t c_mine = lig < n ? col[e0 + lig] : 0;
-                const float v_mine = lig < n ? val[e0 + lig] : 0.0f;
-                for (int j0 = 0; j0 < n; j0 += U) {
-                    f4 xv[U][NCH];
-                    float vv[U];
-#pragma unroll
-                    for (int u = 0; u < U; ++u) {
-                        // a surplus gather reads row 0 (a valid address); its result never enters the chain
-                        const int64_t cc = j0 + u < n ? __shfl(c_mine, j0 + u, LPR) : 0;
-                        vv[u] = __shfl(v_mine, j0 + u < n ? j0 + u : 0, LPR);
-                        const float *xr = x + (size_t)cc * (size_t)ldx;
-#pragma unroll
-                        for (int k = 0; k < NCH; ++k) xv[u][k] = *reinterpret_cast<const f4 *>(xr + foff[k]);
-                    }
-#pragma unroll
-                    for (int u = 0; u < U; ++u) {
-                        if (j0 + u < n) {
-#pragma unroll
-                            for (int k = 0; k < NCH; ++k) {
-#pragma unroll
-                                for (int e = 0; e < 4; ++e) acc[k][e] = __builtin_fmaf(vv[u], xv[u][k][e], acc[k][e]);
-                            }
-                        }
-                    }
-                }
-            }
-            // the finished row: parameters, then its codes into the bytes it shares
+        for (int k = 0; k < NCH; ++k) {
+            word[k] = 0;
+            acc[k] = f4{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+        int r = 0;
+        int64_t row_end = __shfl(ext, 1, LPR);
+        // the finished row r: parameters, then its codes into the bytes it shares
+        auto close_row = [&]() {
             float lo = INFINITY, hi = -INFINITY;
 #pragma unroll
             for (int k = 0; k < NCH; ++k) {
@@ -453,13 +430,47 @@ __global__ __launch_bounds__(256) void spmm_quantize_segments_kernel(
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
                     word[k] |= ((quantize_one_fast(acc[k][e], zp, scale, inv) << ((EPB - r - 1) * BITS)) & 0xFFu) << (8 * e);
+                acc[k] = f4{0.0f, 0.0f, 0.0f, 0.0f};
+            }
+            ++r;
+            row_end = __shfl(ext, r + 1 <= rg.count ? r + 1 : rg.count, LPR);
+        };
+        for (int64_t e0 = begin; e0 < end; e0 += LPR) {
+            const int n = (int)(end - e0 < LPR ? end - e0 : LPR);
+            // one coalesced fetch of up to LPR (column, value) pairs, handed round below
+            const int64_t c_mine = lig < n ? col[e0 + lig] : 0;
+            const float v_mine = lig < n ? val[e0 + lig] : 0.0f;
+            for (int j0 = 0; j0 < n; j0 += U) {
+                f4 xv[U][NCH];
+                float vv[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    // a surplus gather reads row 0 (a valid address); its result never enters a chain
+                    const int64_t cc = j0 + u < n ? __shfl(c_mine, j0 + u, LPR) : 0;
+                    vv[u] = __shfl(v_mine, j0 + u < n ? j0 + u : 0, LPR);
+                    const float *xr = x + (size_t)cc * (size_t)ldx;
+#pragma unroll
+                    for (int k = 0; k < NCH; ++k) xv[u][k] = *reinterpret_cast<const f4 *>(xr + foff[k]);
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    if (j0 + u < n) {
+                        if constexpr (EPB > 1) {
+                            while (e0 + j0 + u >= row_end) close_row();  // (rows without elements close at once)
+                        }
+#pragma unroll
+                        for (int k = 0; k < NCH; ++k) {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) acc[k][e] = __builtin_fmaf(vv[u], xv[u][k][e], acc[k][e]);
+                        }
+                    }
+                }
             }
         }
-        if (rg.count > 0) {
+        while (r < rg.count) close_row();
 #pragma unroll
-            for (int k = 0; k < NCH; ++k)
-                if (fok[k]) *reinterpret_cast<uint32_t *>(packed + (size_t)g * (size_t)feat + foff[k]) = word[k];
-        }
+        for (int k = 0; k < NCH; ++k)
+            if (fok[k]) *reinterpret_cast<uint32_t *>(packed + (size_t)g * (size_t)feat + foff[k]) = word[k];
     }
 }
 
