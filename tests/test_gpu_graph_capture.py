@@ -2,8 +2,8 @@
 record them into a HIP graph (here through torch.cuda.CUDAGraph, whose capture stream the library
 picks up as the current stream) and replay it.  One graph holds the plan SpMM with a very long row
 (block-per-row kernel on the plan's side stream, forked and joined with events), the transposed
-product, the strided product, the products with bf16 rows, the row gather, the codec, the bf16 conversions, both fused
-epilogues, the weight gradient, and the one-kernel dense layer with its one-pass gradient; it is replayed several times, with eager work and host
+product, the strided product, the products with bf16 rows, the product with quantised result rows, the row gather (fp32
+and bf16 rows), the codec, the bf16 conversions, both fused epilogues, the weight gradient, and the one-kernel dense layer with its one-pass gradient; it is replayed several times, with eager work and host
 synchronisation in between, and every replay must reproduce the eager results bit for bit."""
 import numpy as np
 import pytest
@@ -39,6 +39,7 @@ def test_entry_points_replay_from_a_hip_graph(monkeypatch):
     div = torch.randint(1, 9, (n,), device="cuda", generator=gen).float()
     work_range = torch.tensor([0, 1000, 1000, n], dtype=torch.int32)
     packed_rows = sum(-(-s // (8 // bits)) for s in (1000, 0, n - 1000))
+    csr_arrays = src.csr()
 
     def work():
         out = torch.empty(n, feat, device="cuda")
@@ -72,9 +73,16 @@ def test_entry_points_replay_from_a_hip_graph(monkeypatch):
         SPMM_forward(src, x, rounded, accumulate=False)               # bf16 result rows (a 16-bit exchange's send side)
         widened = torch.empty(n, feat, device="cuda")
         SPMM_backward(src, rounded, widened, accumulate=False)        # bf16 operand rows (its receive side)
+        rows16 = torch.empty(index.numel(), feat, dtype=torch.bfloat16, device="cuda")
+        _gather_rows(act, index, rows16)                               # the gather storing bf16 rows
+        packed1 = torch.empty((packed_rows, feat), dtype=torch.uint8, device="cuda")
+        params1 = torch.empty((n, 2), device="cuda")
+        assert ops.spmm_quantize_for_all_procs(csr_arrays[0], csr_arrays[1], csr_arrays[2], x, packed1, params1,
+                                               work_range, 3, bits)  # a quantised exchange's send side in one pass
         # (the left half of `cat` is scratch for a following layer and is never written here)
         return [out, dx, wide, cat[:, feat:], act, w, rows, packed, params, back, wire, layer.detach(), x_in.grad,
-                w_in.grad, b_in.grad, layer3.detach(), x3.grad, w3.grad, b3.grad, rounded, widened]
+                w_in.grad, b_in.grad, layer3.detach(), x3.grad, w3.grad, b3.grad, rounded, widened, rows16, packed1,
+                params1]
 
     eager = [t.clone() for t in work()]
     torch.cuda.synchronize()
