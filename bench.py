@@ -959,7 +959,46 @@ def run_c4_raw_halo(args, part):
         bf16_ms[fused] = (time.perf_counter() - t0) * 1e3 / steps
     graph.fuse_bf16_staging = True
     graph.comm_buf, graph.exchange_bf16 = fp32_buf, None
+    # ... and as int2 (num_bits=2): the gather and the gradient product writing the packed rows themselves and the
+    # products behind the exchange reading them (the default), or the reference's passes each on its own
+    from gnn_benchmark_amd import computation_ops
+    from gnn_benchmark_amd.data_manager import CommBufferForQuantization, CommSplits
+
+    world = len(graph.comm_splits.send_splits)
+    fp32_splits = graph.comm_splits
+    graph.comm_buf.resize_buffer(fp32_splits, feat, 32)
+    graph.comm_splits = CommSplits(fp32_splits.recv_splits, fp32_splits.send_splits, world, 2)
+    qb = graph.comm_buf_for_quantization = CommBufferForQuantization(graph.comm_splits, feat, 2, device=dev)
+    graph.exchange_quantized = synthetic.PregeneratedQuantizedHaloExchange(args.seed + 6)
+    for i in range(steps + 2):
+        if i == 2:
+            e0.record()
+        computation_ops.gather_quantize_for_all_procs(x, idx, qb.quantized_send_data_buf, qb.quantized_send_params_buf_fp32,
+                                                      qb.quantized_work_range_per_proc, world, 2)
+    e1.record()
+    e1.synchronize()
+    ms = e0.elapsed_time(e1) / steps
+    gq_bytes = idx.numel() * (8.0 + 4.0 * feat + feat / 4.0 + 8.0)
+    ops.append({"op": "gather boundary rows X[idx] -> int2 bytes + parameters", "rows": int(idx.numel()), "feat": feat,
+                "ms": round(ms, 4), "gbs_model": round(gq_bytes / (ms * 1e-3) / 1e9, 1),
+                "frac_of_hbm_peak": round(gq_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)})
+    int2_ms = {}
+    for fused in (True, False):
+        graph.fuse_quantize = graph.fuse_dequantize = fused
+        for _ in range(2):
+            Aggregator.apply(graph, xr, 0, 2, False, True).backward(g)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            o = Aggregator.apply(graph, xr, 0, 2, False, True)
+            o.backward(g)
+        torch.cuda.synchronize()
+        int2_ms[fused] = (time.perf_counter() - t0) * 1e3 / steps
+    graph.fuse_quantize = graph.fuse_dequantize = True
+    graph.comm_splits, graph.comm_buf_for_quantization, graph.exchange_quantized = fp32_splits, None, None
     return {"workload": "the c4 partition with raw boundary rows (is_pre_delay=False)", "feat": feat,
+            "aggregator_forward_backward_ms_int2_exchange": round(int2_ms[True], 3),
+            "aggregator_forward_backward_ms_int2_exchange_separate_codec_passes": round(int2_ms[False], 3),
             "send_rows": int(idx.numel()), "halo_rows": int(graph.remote_adj_t.sparse_size(1)), "setup_s": round(setup_s, 2),
             "ops": ops, "aggregator_forward_ms": round(fwd_ms, 3), "aggregator_forward_backward_ms": round(both_ms, 3),
             "aggregator_forward_backward_ms_bf16_exchange": round(bf16_ms[True], 3),

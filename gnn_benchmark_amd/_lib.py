@@ -58,6 +58,7 @@ EXPORTS = (
     "gnnagg_plan_spmm_packed_f32",
     "gnnagg_quantize_segments_f32",
     "gnnagg_spmm_csr_quantize_segments_f32",
+    "gnnagg_gather_quantize_segments_f32",
     "gnnagg_dequantize_segments_f32",
     "gnnagg_plan_spmm_quantized_f32",
     "gnnagg_plan_spmm_bf16_f32",
@@ -197,6 +198,8 @@ def lib() -> ctypes.CDLL:
     L.gnnagg_plan_spmm_packed_f32.argtypes = [vp, vp, vp, vp, vp, i64, i32, vp]
     L.gnnagg_quantize_segments_f32.restype = i32
     L.gnnagg_quantize_segments_f32.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp]
+    L.gnnagg_gather_quantize_segments_f32.restype = i32
+    L.gnnagg_gather_quantize_segments_f32.argtypes = [vp, i64, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp]
     L.gnnagg_spmm_csr_quantize_segments_f32.restype = i32
     L.gnnagg_spmm_csr_quantize_segments_f32.argtypes = [vp, vp, vp, vp, i64, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp]
     L.gnnagg_dequantize_segments_f32.restype = i32

@@ -281,6 +281,13 @@ def _forward(ctx, graph, feats, layer, num_bits: int, is_pre_delay: bool, is_tra
                                                               num_bits, "forward")
             if not packed_by_product:
                 feats.product(graph.adj_t_pre_post_aggr_to, graph.comm_buf.send_buf_fp16 if half_fused else send_buf, False)
+        elif (quantized and isinstance(feats, _DenseFeatures) and send_buf.size(0) != 0
+              and getattr(graph, "fuse_quantize", True) is not False and feats.feat.is_contiguous()):
+            # raw boundary rows quantised as they are gathered (the fp32 send rows are not written)
+            _, data, params, work_range = _outgoing_quantized(graph, "forward")
+            computation_ops.gather_quantize_for_all_procs(feats.feat, graph.idx_nodes_send_to_others, data, params,
+                                                          work_range, len(graph.comm_splits.send_splits), num_bits)
+            packed_by_product = True
         else:  # raw boundary rows (as bf16 at once when they travel so)
             feats.gather(graph.idx_nodes_send_to_others, graph.comm_buf.send_buf_fp16 if half_fused else send_buf)
         if quantized:

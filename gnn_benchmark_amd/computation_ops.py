@@ -134,6 +134,36 @@ def quantize_tensor_for_all_procs(input: torch.Tensor, output: torch.Tensor, qua
             num_procs, rows, packed_rows, input.size(1), bits, _lib.current_stream(dev)))
 
 
+def gather_quantize_for_all_procs(src: torch.Tensor, index: torch.Tensor, output: torch.Tensor,
+                                  quantized_params: torch.Tensor, work_range_per_proc: torch.Tensor, num_procs: int,
+                                  bits: int) -> None:
+    """``quantize_tensor_for_all_procs(src[index], output, ...)`` in one pass (aggregator.py:51 then
+    communicator.py:281-311): the raw boundary rows are quantised as they are gathered, same bytes and parameters,
+    without the gathered fp32 rows being written."""
+    _require(bits in (2, 4, 8), "bits must be 2, 4 or 8")
+    _require_hip(src, "source rows")
+    dev = src.device
+    for t, name in ((index, "index"), (output, "packed buffer"), (quantized_params, "quantisation parameters")):
+        _require_hip(t, name, dev)
+    rows = index.numel()
+    _require(src.dtype == torch.float32 and src.dim() == 2 and src.is_contiguous(),
+             "source rows must be contiguous float32 2-D")
+    _require(index.dtype == torch.int64 and index.is_contiguous(), "index must be contiguous int64")
+    _require(output.dtype == torch.uint8 and output.is_contiguous(), "packed buffer must be contiguous uint8")
+    _require(quantized_params.dtype == torch.float32 and quantized_params.is_contiguous()
+             and quantized_params.dim() == 2 and quantized_params.size(0) >= rows and quantized_params.size(1) == 2,
+             "parameters must be contiguous float32 [rows, 2]")
+    _require(work_range_per_proc.numel() == num_procs + 1, "work range must hold num_procs + 1 entries")
+    rows_d, packed_d, packed_rows, covered = _packed_range(work_range_per_proc, bits, dev)
+    _require(covered == rows, "work range does not cover the index list")
+    _require(output.numel() >= packed_rows * src.size(1), "packed buffer too small")
+    _lib.check_index(index, src.size(0), what="boundary row list (idx_nodes_send_to_others)")
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().gnnagg_gather_quantize_segments_f32(
+            _lib.ptr(src), src.size(0), _lib.ptr(index), _lib.ptr(output), _lib.ptr(quantized_params), _lib.ptr(rows_d),
+            _lib.ptr(packed_d), num_procs, rows, packed_rows, src.size(1), bits, _lib.current_stream(dev)))
+
+
 def spmm_quantize_for_all_procs(rowptr: torch.Tensor, col: torch.Tensor, value: torch.Tensor, mat: torch.Tensor,
                                 output: torch.Tensor, quantized_params: torch.Tensor,
                                 work_range_per_proc: torch.Tensor, num_procs: int, bits: int) -> bool:

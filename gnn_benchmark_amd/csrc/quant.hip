@@ -157,7 +157,8 @@ __global__ __launch_bounds__(256) void quantize_segments_kernel(const float *__r
                                                                 float *__restrict__ params,
                                                                 const int32_t *__restrict__ row_range,
                                                                 const int32_t *__restrict__ packed_range, int segments,
-                                                                int rows, int packed_rows, int feat) {
+                                                                int rows, int packed_rows, int feat,
+                                                                const int64_t *__restrict__ index, int64_t src_rows) {
     constexpr int EPB = 8 / BITS;
     constexpr int GPL = kRowsPerLaneGroup / EPB;
     constexpr int KEEP = NV > 0 ? NV : 1;
@@ -169,6 +170,16 @@ __global__ __launch_bounds__(256) void quantize_segments_kernel(const float *__r
 
     const int l = (int)threadIdx.x & (G - 1);
     const int nvec = (feat + VEC - 1) / VEC;  // VEC == 4 implies feat % 4 == 0
+    // where fp32 row r of the buffer lies: in x itself, or (index given: the gather of raw boundary rows folded in)
+    // at row index[r] of x -- an index outside x is never dereferenced, row 0 is read in its place
+    auto row_at = [&](int r) -> const float * {
+        size_t at = (size_t)r;
+        if (index) {
+            const int64_t i = index[r];
+            at = (uint64_t)i < (uint64_t)src_rows ? (size_t)i : 0;
+        }
+        return x + at * (size_t)feat;
+    };
 
     struct Slice {
         int g0;
@@ -189,7 +200,7 @@ __global__ __launch_bounds__(256) void quantize_segments_kernel(const float *__r
 #pragma unroll
                 for (int k = 0; k < EPB; ++k) {
                     // a row the group does not have reads row 0 instead (never used): loads without branches
-                    const float *row = x + (size_t)(k < sl.rg[u].count ? sl.rg[u].first + k : 0) * (size_t)feat;
+                    const float *row = row_at(k < sl.rg[u].count ? sl.rg[u].first + k : 0);
 #pragma unroll
                     for (int j = 0; j < KEEP; ++j) {
                         const int v = l + G * j;
@@ -221,7 +232,7 @@ __global__ __launch_bounds__(256) void quantize_segments_kernel(const float *__r
                             }
                         }
                     } else {
-                        const float *row = x + (size_t)(sl.rg[u].first + k) * (size_t)feat;
+                        const float *row = row_at(sl.rg[u].first + k);
                         for (int v = l; v < nvec; v += G) {
                             const QVec<VEC> t = QVec<VEC>::load(row + (size_t)v * VEC);
 #pragma unroll
@@ -253,7 +264,7 @@ __global__ __launch_bounds__(256) void quantize_segments_kernel(const float *__r
                     if (k < sl.rg[u].count) {
                         QVec<VEC> t;
                         if (NV > 0) t = sl.held[u][k][j];
-                        else t = QVec<VEC>::load(x + (size_t)(sl.rg[u].first + k) * (size_t)feat + (size_t)v * VEC);
+                        else t = QVec<VEC>::load(row_at(sl.rg[u].first + k) + (size_t)v * VEC);
 #pragma unroll
                         for (int e = 0; e < VEC; ++e)
                             byte[e] |= quantize_one_fast(t.get(e), zp[u][k], scale[u][k], inv[u][k])
@@ -547,6 +558,8 @@ struct SegArgs {
     const int32_t *row_range, *packed_range;
     int segments, rows, packed_rows, feat;
     hipStream_t st;
+    const int64_t *index = nullptr;  // quantise: fp32 row r is row index[r] of the source (a gather folded in)
+    int64_t src_rows = 0;
 };
 
 // packed rows handled by one lane group
@@ -564,13 +577,16 @@ void launch_quantize(const float *x, uint8_t *packed, float *params, const SegAr
     const size_t lds = range_lds_bytes(a.segments);
     if (nvec <= G)
         hipLaunchKernelGGL((quantize_segments_kernel<BITS, VEC, G, 1>), dim3(blocks), dim3(256), lds, a.st, x, packed,
-                           params, a.row_range, a.packed_range, a.segments, a.rows, a.packed_rows, a.feat);
+                           params, a.row_range, a.packed_range, a.segments, a.rows, a.packed_rows, a.feat, a.index,
+                           a.src_rows);
     else if (nvec <= 4 * G)
         hipLaunchKernelGGL((quantize_segments_kernel<BITS, VEC, G, 4>), dim3(blocks), dim3(256), lds, a.st, x, packed,
-                           params, a.row_range, a.packed_range, a.segments, a.rows, a.packed_rows, a.feat);
+                           params, a.row_range, a.packed_range, a.segments, a.rows, a.packed_rows, a.feat, a.index,
+                           a.src_rows);
     else
         hipLaunchKernelGGL((quantize_segments_kernel<BITS, VEC, G, 0>), dim3(blocks), dim3(256), lds, a.st, x, packed,
-                           params, a.row_range, a.packed_range, a.segments, a.rows, a.packed_rows, a.feat);
+                           params, a.row_range, a.packed_range, a.segments, a.rows, a.packed_rows, a.feat, a.index,
+                           a.src_rows);
 }
 
 template <int BITS, int VEC>
@@ -672,6 +688,30 @@ extern "C" int gnnagg_quantize_segments_f32(const float *x, uint8_t *packed, flo
     if (bits == B) {                                                     \
         if (v4) launch_quantize_g<B, 4>(x, packed, params, a);           \
         else launch_quantize_g<B, 1>(x, packed, params, a);              \
+    }
+    GNNAGG_Q(2) GNNAGG_Q(4) GNNAGG_Q(8)
+#undef GNNAGG_Q
+    GNNAGG_HIP(hipGetLastError());
+    return GNNAGG_OK;
+}
+
+extern "C" int gnnagg_gather_quantize_segments_f32(const float *src, int64_t src_rows, const int64_t *index,
+                                                   uint8_t *packed, float *params, const int32_t *row_range,
+                                                   const int32_t *packed_range, int64_t segments, int64_t rows,
+                                                   int64_t packed_rows, int64_t feat, int bits, void *stream) {
+    const int rc = check_segments(src, packed, params, row_range, packed_range, segments, rows, packed_rows, feat, bits);
+    if (rc != GNNAGG_OK || rows == 0 || feat == 0) return rc;
+    GNNAGG_REQUIRE(index, "null index");
+    GNNAGG_REQUIRE(src_rows > 0, "rows are asked of a source without rows");
+    SegArgs a{row_range, packed_range, (int)segments, (int)rows, (int)packed_rows, (int)feat,
+              static_cast<hipStream_t>(stream)};
+    a.index = index;
+    a.src_rows = src_rows;
+    const bool v4 = feat % 4 == 0 && aligned16(src) && aligned4(packed);
+#define GNNAGG_Q(B)                                                      \
+    if (bits == B) {                                                     \
+        if (v4) launch_quantize_g<B, 4>(src, packed, params, a);         \
+        else launch_quantize_g<B, 1>(src, packed, params, a);            \
     }
     GNNAGG_Q(2) GNNAGG_Q(4) GNNAGG_Q(8)
 #undef GNNAGG_Q

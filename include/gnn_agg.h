@@ -420,6 +420,16 @@ int gnnagg_quantize_segments_f32(const float *x, uint8_t *packed, float *params,
 int gnnagg_dequantize_segments_f32(const uint8_t *packed, const float *params, float *out, const int32_t *row_range,
                                    const int32_t *packed_range, int64_t segments, int64_t rows, int64_t packed_rows,
                                    int64_t feat, int bits, void *stream);
+/* Raw boundary rows straight into the packed bytes: gnnagg_quantize_segments_f32 whose fp32 row r is row index[r] of
+ * src -- `torch.index_select(local_nodes_feat, 0, idx_nodes_send_to_others, out=send_buf)` followed by
+ * `quantize_tensor_for_all_procs(send_buf, ...)` (model/layers/aggregator.py:51, communicator/communicator.py:281-311) as
+ * one pass; same bytes and parameters, the gathered fp32 rows never written.  src fp32 [src_rows, feat] contiguous,
+ * index int64 [rows]; an index outside [0, src_rows) is never dereferenced (row 0 is read in its place; raising for
+ * it is gnnagg_check_index's part).  No allocation, no host synchronisation. */
+int gnnagg_gather_quantize_segments_f32(const float *src, int64_t src_rows, const int64_t *index, uint8_t *packed,
+                                        float *params, const int32_t *row_range, const int32_t *packed_range,
+                                        int64_t segments, int64_t rows, int64_t packed_rows, int64_t feat, int bits,
+                                        void *stream);
 /* Pre-aggregation straight into the packed bytes: packed / params = quantize(A @ mat), every segment on its own --
  * `send_buf += A_to @ X` followed by `quantize_tensor_for_all_procs(send_buf, ...)` (model/layers/aggregator.py:44-49,
  * communicator/communicator.py:281-311; backward: :144-149 with the buffers' roles swapped) as one pass.  A is given as

@@ -533,6 +533,69 @@ def test_raw_halo_bf16_exchange_matches_oracle(seed, sizes, fused):
         assert_close(xr.grad, o_dx, "raw halo gradient vs oracle, bf16 rows")
 
 
+@pytest.mark.parametrize("bits", [2, 8])
+@pytest.mark.parametrize("seed,sizes", [(8, (300, 450, 250)), (9, (600, 1, 400, 330))])
+def test_raw_halo_quantised_exchange_matches_oracle(seed, sizes, bits):
+    """The raw-halo mode with packed rows on the wire (aggregator.py:51, :83-88, :180-199): the bytes and parameters
+    every rank sends equal the oracle codec's over the gathered rows / the outgoing gradient rows, output and gradient
+    equal the oracle pipeline fed with what the peers' bytes decode to -- in the reference's form (gather, quantise,
+    dequantise as passes of their own) and as it runs by default (the gather and the gradient product writing the
+    packed bytes themselves, the products behind the exchange reading them)."""
+    from oracle import quantization as oq
+
+    w = World(seed, sizes, mean_deg=8.0)
+    W, F = w.world, 40
+    graphs = _build_raw_graphs(w, F, bits=bits)
+    rng = np.random.default_rng(seed + 400)
+    x = (rng.standard_normal((w.n, F)) * rng.uniform(1e-2, 1e2, (w.n, 1))).astype(np.float32)
+    g = rng.standard_normal((w.n, F)).astype(np.float32)
+    sl = [slice(int(w.begins[r]), int(w.begins[r + 1])) for r in range(W)]
+    csr = [(_csr_np(gr.local_adj_t) + [gr.local_adj_t.sparse_sizes()], _csr_np(gr.remote_adj_t) + [gr.remote_adj_t.sparse_sizes()])
+           for gr in graphs]
+    idx = [gr.idx_nodes_send_to_others.cpu().numpy() for gr in graphs]
+    send_splits = [gr.comm_splits.send_splits for gr in graphs]
+    recv_splits = [gr.comm_splits.recv_splits for gr in graphs]
+    send_packed = [gr.comm_splits.send_splits_int2 for gr in graphs]
+    recv_packed = [gr.comm_splits.recv_splits_int2 for gr in graphs]
+    o_send = [oagg.forward_send_raw(idx[r], x[sl[r]]) for r in range(W)]
+    o_back = [oagg.backward_recv(csr[r][1], np.ascontiguousarray(g[sl[r]])) for r in range(W)]
+    q_send = [oq.quantize_segments(o_send[r], send_splits[r], bits) for r in range(W)]
+    q_back = [oq.quantize_segments(o_back[r], recv_splits[r], bits) for r in range(W)]
+    fwd_data = host_exchange([q[0] for q in q_send], send_packed, recv_packed)
+    fwd_params = host_exchange([oq.params_over_the_wire(q[1]) for q in q_send], send_splits, recv_splits)
+    bwd_data = host_exchange([q[0] for q in q_back], recv_packed, send_packed)
+    bwd_params = host_exchange([oq.params_over_the_wire(q[1]) for q in q_back], recv_splits, send_splits)
+    recv = host_exchange([oagg.quantized_wire(o_send[r], send_splits[r], bits) for r in range(W)], send_splits, recv_splits)
+    incoming = host_exchange([oagg.quantized_wire(o_back[r], recv_splits[r], bits) for r in range(W)], recv_splits,
+                             send_splits)
+    for fused in (False, True):
+        for r in range(W):
+            gr = graphs[r]
+            gr.exchange = lambda *a: (_ for _ in ()).throw(AssertionError("fp32 exchange used in a quantised run"))
+            gr.exchange_quantized = PlayedQuantizedExchange((dev(fwd_data[r]), dev(fwd_params[r])),
+                                                            (dev(bwd_data[r]), dev(bwd_params[r])))
+            gr.fuse_quantize = gr.fuse_dequantize = fused
+            qb = gr.comm_buf_for_quantization
+            qb.quantized_send_data_buf.fill_(0x5A)
+            qb.quantized_recv_data_buf.fill_(0x5A)
+            gr.comm_buf.send_buf.fill_(float("nan"))
+            gr.comm_buf.recv_buf.fill_(float("nan"))
+            xr = dev(x[sl[r]]).requires_grad_()
+            out = Aggregator.apply(gr, xr, 1, bits, False, True)
+            assert np.array_equal(qb.quantized_send_data_buf.cpu().numpy(), q_send[r][0])
+            assert np.array_equal(qb.quantized_send_params_buf_fp32.cpu().numpy(), q_send[r][1])
+            o_out = oagg.forward_out(csr[r][0], csr[r][1], np.ascontiguousarray(x[sl[r]]), recv[r])
+            assert np.array_equal(out.detach().cpu().numpy(), o_out)
+            out.backward(dev(g[sl[r]]))
+            assert np.array_equal(qb.quantized_recv_data_buf.cpu().numpy(), q_back[r][0])
+            assert np.array_equal(qb.quantized_recv_params_buf_fp32.cpu().numpy(), q_back[r][1])
+            o_dx = oagg.backward_out_raw(csr[r][0], idx[r], np.ascontiguousarray(g[sl[r]]), incoming[r])
+            assert_close(xr.grad, o_dx, "raw halo gradient vs oracle, quantised rows")
+            if fused:   # the fp32 boundary buffers are neither written nor read
+                for buf in (gr.comm_buf.recv_buf, gr.comm_buf.send_buf):
+                    assert buf.numel() == 0 or bool(torch.isnan(buf).all())
+
+
 @pytest.mark.parametrize("feat", [4, 8, 20, 40, 128, 132, 256, 604, 1028])
 @pytest.mark.parametrize("count", [0, 1, 3, 64, 1000, 4099])
 def test_row_gather_into_bf16_rows_equals_gather_then_copy(feat, count):

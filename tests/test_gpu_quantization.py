@@ -315,6 +315,38 @@ def test_product_with_quantised_result_rows_leaves_other_widths_to_the_two_calls
                                         q.quantized_work_range_per_proc, 1, 2)
 
 
+@pytest.mark.parametrize("bits", [2, 4, 8])
+@pytest.mark.parametrize("feat", [1, 3, 16, 47, 128, 130, 256, 602, 1028, 2052])
+def test_gather_folded_into_the_quantise_pass_equals_gather_then_quantise(bits, feat):
+    """``gather_quantize_for_all_procs`` (raw boundary rows quantised as they are gathered) against
+    ``src[index]`` followed by ``quantize_tensor_for_all_procs``: bytes and parameters bit for bit, repeated and
+    unsorted indices, ragged segments, every width class of the quantise kernel."""
+    from gnn_benchmark_amd import computation_ops as ops
+    from gnn_benchmark_amd.data_manager import CommBufferForQuantization, CommSplits
+
+    rng = np.random.default_rng(10 * feat + bits)
+    src = dev(_rows(rng, 333, feat))
+    splits = [121, 0, 78, 504]
+    index = torch.from_numpy(rng.integers(0, 333, sum(splits))).cuda()
+    cs = CommSplits([5, 5, 5, 5], splits, 4, bits)
+    one = CommBufferForQuantization(cs, feat, bits, device="cuda")
+    two = CommBufferForQuantization(cs, feat, bits, device="cuda")
+    for q in (one, two):
+        q.quantized_send_data_buf.fill_(0xAB)
+        q.quantized_send_params_buf_fp32.fill_(-7.0)
+    ops.quantize_tensor_for_all_procs(src[index].contiguous(), two.quantized_send_data_buf,
+                                      two.quantized_send_params_buf_fp32, two.quantized_work_range_per_proc, 4, bits)
+    ops.gather_quantize_for_all_procs(src, index, one.quantized_send_data_buf, one.quantized_send_params_buf_fp32,
+                                      one.quantized_work_range_per_proc, 4, bits)
+    assert torch.equal(one.quantized_send_params_buf_fp32, two.quantized_send_params_buf_fp32)
+    assert torch.equal(one.quantized_send_data_buf, two.quantized_send_data_buf)
+    with pytest.raises(RuntimeError, match="outside"):
+        bad = index.clone()
+        bad[5] = 333
+        ops.gather_quantize_for_all_procs(src, bad, one.quantized_send_data_buf, one.quantized_send_params_buf_fp32,
+                                          one.quantized_work_range_per_proc, 4, bits)
+
+
 def test_quantised_aggregation_error_behaviour():
     from gnn_benchmark_amd.data_manager import CommBufferForQuantization, CommSplits
     from gnn_benchmark_amd.sparse_tensor import SparseTensor
