@@ -137,12 +137,19 @@ def _outgoing_quantized(graph, direction: str):
             qbuf.dequantized_work_range_per_proc)
 
 
-def _product_into_packed_rows(graph, csr, dense: torch.Tensor, num_bits: int, direction: str) -> bool:
+# the one-pass kernel gives a row to one lane group from its first element to its last; a matrix with a longer row than
+# this goes through the product kernels (which spread such rows) and the quantise pass instead
+_ONE_PASS_MAX_ROW_LEN = 4096
+
+
+def _product_into_packed_rows(graph, plan, csr, dense: torch.Tensor, num_bits: int, direction: str) -> bool:
     """The product in front of a quantised exchange writing the packed bytes and parameters itself
     (``computation_ops.spmm_quantize_for_all_procs``: same bytes as the product followed by the quantise pass, without the
     fp32 rows; the fp32 buffer is then NOT filled).  The default; ``graph.fuse_quantize = False`` keeps the two passes.
-    ``csr``: (rowptr, col, value) of the matrix whose rows are the outgoing rows.  False when nothing was done."""
-    if getattr(graph, "fuse_quantize", True) is False or dense.dtype != torch.float32 or csr[2] is None:
+    ``csr``: (rowptr, col, value) of the matrix whose rows are the outgoing rows, ``plan`` its plan.  False when
+    nothing was done."""
+    if (getattr(graph, "fuse_quantize", True) is False or dense.dtype != torch.float32 or csr[2] is None
+            or plan.max_row_len > _ONE_PASS_MAX_ROW_LEN):
         return False
     _, data, params, work_range = _outgoing_quantized(graph, direction)
     if csr[0].numel() - 1 == 0:
@@ -277,8 +284,9 @@ def _forward(ctx, graph, feats, layer, num_bits: int, is_pre_delay: bool, is_tra
         packed_by_product = False
         if is_pre_delay:  # pre-aggregation: send_buf = A_to @ X (straight into the rows that travel, bf16 or packed)
             if quantized and isinstance(feats, _DenseFeatures) and send_buf.size(0) != 0:
-                packed_by_product = _product_into_packed_rows(graph, graph.adj_t_pre_post_aggr_to.csr(), feats.feat,
-                                                              num_bits, "forward")
+                to = graph.adj_t_pre_post_aggr_to
+                packed_by_product = _product_into_packed_rows(graph, to.get_plan(), to.csr(), feats.feat, num_bits,
+                                                              "forward")
             if not packed_by_product:
                 feats.product(graph.adj_t_pre_post_aggr_to, graph.comm_buf.send_buf_fp16 if half_fused else send_buf, False)
         elif (quantized and isinstance(feats, _DenseFeatures) and send_buf.size(0) != 0
@@ -460,8 +468,11 @@ def _backward(ctx, local_out_grad, out=None, accumulate: bool = False):
     if remote_nodes_grad_buf.size(0) != 0:
         remote = graph.adj_t_pre_post_aggr_from if is_pre_delay else graph.remote_adj_t
         if quantized:  # straight into the packed rows that travel
-            csr = support.remote_T.csr() if support is not None else _transposed_csr(remote)
-            packed_by_product = _product_into_packed_rows(graph, csr, local_out_grad, num_bits, "backward")
+            if support is not None:
+                plan, csr = support.remote_T.get_plan(), support.remote_T.csr()
+            else:
+                plan, csr = remote.get_plan_for_transpose(), _transposed_csr(remote)
+            packed_by_product = _product_into_packed_rows(graph, plan, csr, local_out_grad, num_bits, "backward")
         if packed_by_product:
             pass
         elif support is not None:

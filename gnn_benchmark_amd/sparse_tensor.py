@@ -52,6 +52,14 @@ class SpmmPlan:
                 "short_rows", "short_rows_per_group", "long_rows", "long_thresh")
         return dict(zip(keys, [int(x) for x in buf]))
 
+    @property
+    def max_row_len(self) -> int:
+        """Stored elements of the matrix's longest row (fixed when the plan was built)."""
+        hit = getattr(self, "_max_row_len", None)
+        if hit is None:
+            hit = self._max_row_len = self.info()["max_row_len"]
+        return hit
+
     def profile(self, enable: bool = True) -> None:
         """Record HIP events around the next SpMM calls (benchmark use)."""
         _lib.check(_lib.lib().gnnagg_plan_profile(self._handle, 1 if enable else 0))

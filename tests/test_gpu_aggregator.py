@@ -741,6 +741,36 @@ def test_pregenerated_quantized_halo_rows_equal_the_seeded_ones(fused):
         assert torch.equal(a, b)
 
 
+def test_quantised_run_with_a_very_long_outgoing_row_takes_the_two_passes(monkeypatch):
+    """A matrix with a row longer than the one-pass kernel's limit goes through the product kernels and the quantise
+    pass (they spread such a row over many lane groups); bytes, outputs and gradients are the same either way."""
+    from gnn_benchmark_amd import aggregator, computation_ops, synthetic
+
+    n = 30_000
+    part = synthetic.partition_edges(n, 8, 5, 6.0, 1.8, 1500, 11_000, 70_000, seed=15, device="cuda")
+    results = []
+    for limit in (aggregator._ONE_PASS_MAX_ROW_LEN, 2):
+        monkeypatch.setattr(aggregator, "_ONE_PASS_MAX_ROW_LEN", limit)
+        calls = []
+        real = computation_ops.spmm_quantize_for_all_procs
+        monkeypatch.setattr(computation_ops, "spmm_quantize_for_all_procs", lambda *a: calls.append(1) or real(*a))
+        graph = synthetic.build_partition_graph(part, 64, True, exchange=synthetic.SeededHaloExchange(1), bits=2,
+                                                exchange_quantized=synthetic.SeededQuantizedHaloExchange(9), device="cuda")
+        assert graph.adj_t_pre_post_aggr_to.get_plan().max_row_len > 2
+        gen = torch.Generator(device="cuda").manual_seed(3)
+        x = torch.randn(n, 64, device="cuda", generator=gen, requires_grad=True)
+        g = torch.randn(n, 64, device="cuda", generator=gen)
+        out = Aggregator.apply(graph, x, 0, 2, True, True)
+        sent = graph.comm_buf_for_quantization.quantized_send_data_buf.clone()
+        out.backward(g)
+        results.append((out.detach().clone(), x.grad.clone(), sent,
+                        graph.comm_buf_for_quantization.quantized_recv_data_buf.clone()))
+        assert len(calls) == (2 if limit > 2 else 0)
+        monkeypatch.setattr(computation_ops, "spmm_quantize_for_all_procs", real)
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
+
+
 def test_bad_indices_raise_instead_of_reading_out_of_bounds():
     """torch.index_select raises on an index outside its source (the reference's gather); so do the gather, the
     plan-less operator (column indices) and the aggregation straight from packed bytes (row codes) -- the lists are
