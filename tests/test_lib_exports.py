@@ -57,6 +57,23 @@ def test_argument_errors_without_gpu_work():
     assert L.gnnagg_dropout_layernorm_relu_backward_f32(256, 128, 256, None, 1.0, 256, 256, 1e-5, 256, None, 4, 128, None) == _lib.ERR_INVALID
     assert b"partial" in L.gnnagg_last_error()
     assert L.gnnagg_issue_probe(1, 1, None, None) == _lib.ERR_INVALID   # null sink
+    # the producers that write the exchange format themselves: argument checks before any launch (fake operands)
+    fake = 256
+    assert L.gnnagg_spmm_csr_quantize_segments_f32(fake, fake, fake, fake, 128, fake, fake, fake, fake, 1, 8, 2, 128, 3,
+                                                   None) == _lib.ERR_INVALID
+    assert b"bits" in L.gnnagg_last_error()
+    assert L.gnnagg_spmm_csr_quantize_segments_f32(None, fake, fake, fake, 128, fake, fake, fake, fake, 1, 8, 2, 128, 2,
+                                                   None) == _lib.ERR_INVALID   # null rowptr
+    assert L.gnnagg_spmm_csr_quantize_segments_f32(fake, fake, fake, fake, 64, fake, fake, fake, fake, 1, 8, 2, 128, 2,
+                                                   None) == _lib.ERR_INVALID   # row stride below the width
+    assert L.gnnagg_spmm_csr_quantize_segments_f32(fake, fake, fake, fake, 516, fake, fake, fake, fake, 1, 8, 2, 516, 2,
+                                                   None) == _lib.ERR_UNSUPPORTED   # wider than the kernel's rows
+    assert L.gnnagg_spmm_csr_quantize_segments_f32(None, None, None, None, 0, None, None, None, None, 1, 0, 0, 128, 2,
+                                                   None) == _lib.OK   # no rows
+    assert L.gnnagg_gather_quantize_segments_f32(fake, 5, None, fake, fake, fake, fake, 1, 8, 2, 128, 2,
+                                                 None) == _lib.ERR_INVALID   # null index
+    assert L.gnnagg_gather_quantize_segments_f32(fake, 0, fake, fake, fake, fake, fake, 1, 8, 2, 128, 2,
+                                                 None) == _lib.ERR_INVALID   # rows asked of an empty source
 
 
 def test_product_refuses_cpu_tensors():
