@@ -1140,6 +1140,32 @@ def run_c5_sage(args, graph):
         out["train_step_ms" + tag], out["loss" + tag] = ms, losses
         del model, opt, g
         torch.cuda.empty_cache()
+    # the same step (degrees folded) with the boundary rows travelling as bf16 / as int2 -- the widths the reference's
+    # own runs exchange at (`--num_bits=2 --is_pre_delay=true`); the rows a peer would have sent stand ready on the device
+    from gnn_benchmark_amd import synthetic
+    from gnn_benchmark_amd.data_manager import CommBuffer, CommBufferForQuantization, CommSplits
+
+    world = len(graph.comm_splits.send_splits)
+    fp32_splits, fp32_buf = folded.comm_splits, folded.comm_buf
+    for tag, bits in (("_folded_degrees_bf16_exchange", 16), ("_folded_degrees_int2_exchange", 2)):
+        if bits == 16:
+            folded.comm_buf = CommBuffer(fp32_splits, hidden, 16, device=dev)
+            synthetic.PregeneratedHaloExchange.attach(folded)
+            folded.exchange_bf16 = synthetic.PregeneratedBf16HaloExchange(args.seed + 7)
+        else:
+            folded.comm_splits = CommSplits(fp32_splits.recv_splits, fp32_splits.send_splits, world, 2)
+            folded.comm_buf_for_quantization = CommBufferForQuantization(folded.comm_splits, hidden, 2, device=dev)
+            folded.exchange_quantized = synthetic.PregeneratedQuantizedHaloExchange(args.seed + 6)
+        torch.manual_seed(args.seed)
+        model = sage.DistSAGE(dims[0], hidden, dims[-1], num_layers=len(dims) - 1, dropout=0.5, num_bits=bits,
+                              is_pre_delay=True).to(dev)
+        opt = torch.optim.Adam(model.parameters(), lr=0.01)
+        ms, losses = timed(lambda: sage.train_step(model, opt, folded, staged, labels, train_idx, masks, True))
+        out["train_step_ms" + tag], out["loss" + tag] = ms, losses
+        del model, opt
+        folded.comm_splits, folded.comm_buf = fp32_splits, fp32_buf
+        folded.exchange_bf16 = folded.exchange_quantized = folded.comm_buf_for_quantization = None
+        torch.cuda.empty_cache()
     del folded
     torch.cuda.empty_cache()
 
