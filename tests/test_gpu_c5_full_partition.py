@@ -132,3 +132,65 @@ def test_packed_activations_equal_the_dense_ones(workload):
 def test_packed_bf16x3_agrees_with_the_fp32_products(workload):
     _, step = workload
     _assert_same_step(step(gemm="bf16x3", packed=True), step(), "bf16x3 packed")
+
+
+@pytest.mark.parametrize("bits", [16, 2])
+def test_boundary_rows_in_their_exchange_format_at_full_size(workload, bits):
+    """``Aggregator`` forward + backward at F = 128 on the full partition with the boundary rows travelling as bf16 /
+    as int2: the products that write and read the exchange format themselves (the default) give the bytes, the output
+    and the gradient of the reference's separate passes, bit for bit -- 3 M send rows, 3 M halo rows, 20 M boundary
+    elements each way."""
+    from gnn_benchmark_amd import Aggregator
+    from gnn_benchmark_amd.data_manager import CommBuffer, CommBufferForQuantization, CommSplits
+
+    graph, _ = workload
+    dev = "cuda:0"
+    feat = 128
+    gen = torch.Generator(device=dev).manual_seed(11)
+    x = torch.randn(NODES, feat, device=dev, generator=gen)
+    g = torch.randn(NODES, feat, device=dev, generator=gen)
+    kept = (graph.comm_splits, graph.comm_buf)
+    world = len(graph.comm_splits.send_splits)
+    try:
+        if bits == 16:
+            graph.comm_buf = CommBuffer(graph.comm_splits, feat, 16, device=dev)
+            graph.exchange_bf16 = synthetic.SeededBf16HaloExchange(21)
+            options = ("fuse_bf16_staging",)
+        else:
+            graph.comm_splits = CommSplits(kept[0].recv_splits, kept[0].send_splits, world, 2)
+            graph.comm_buf_for_quantization = CommBufferForQuantization(graph.comm_splits, feat, 2, device=dev)
+            graph.exchange_quantized = synthetic.SeededQuantizedHaloExchange(22)
+            options = ("fuse_quantize", "fuse_dequantize")
+        seen = []
+        for fused in (True, False):
+            for name in options:
+                setattr(graph, name, fused)
+            xr = x.clone().requires_grad_()
+            out = Aggregator.apply(graph, xr, 0, bits, True, True)
+            if bits == 16:
+                sent = graph.comm_buf.send_buf_fp16.clone()
+            else:
+                qb = graph.comm_buf_for_quantization
+                sent = torch.cat([qb.quantized_send_data_buf.reshape(-1),
+                                  qb.quantized_send_params_buf_fp32.reshape(-1).view(torch.uint8)])
+            out.backward(g)
+            if bits == 16:
+                back = graph.comm_buf.recv_buf_fp16.clone()
+            else:
+                back = torch.cat([qb.quantized_recv_data_buf.reshape(-1),
+                                  qb.quantized_recv_params_buf_fp32.reshape(-1).view(torch.uint8)])
+            seen.append((out.detach(), xr.grad, sent, back))
+            del xr, out
+        for a, b in zip(*seen):
+            if a.dtype == torch.bfloat16:
+                a, b = a.view(torch.int16), b.view(torch.int16)
+            elif a.dtype == torch.float32:
+                assert bool(torch.isfinite(a).all())
+            assert torch.equal(a, b)
+    finally:
+        graph.comm_splits, graph.comm_buf = kept
+        graph.exchange_bf16 = graph.exchange_quantized = graph.comm_buf_for_quantization = None
+        for name in ("fuse_bf16_staging", "fuse_quantize", "fuse_dequantize"):
+            if name in graph.__dict__:
+                delattr(graph, name)
+        torch.cuda.empty_cache()
