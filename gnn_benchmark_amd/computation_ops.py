@@ -171,7 +171,7 @@ def spmm_quantize_for_all_procs(rowptr: torch.Tensor, col: torch.Tensor, value: 
     of the registers they were summed in, bytes and parameters equal to the two calls' (aggregator.py:44-49 then
     communicator.py:281-311).  ``rowptr`` / ``col`` int64 and ``value`` float32 are A's CSR arrays.  Returns False,
     with nothing done, for operands the one-pass kernel does not take (width no multiple of 4 or above 512, rows of
-    ``mat`` off 16-byte boundaries): the caller then runs the two calls."""
+    ``mat`` off 16-byte boundaries, a matrix without stored elements): the caller then runs the two calls."""
     _require(bits in (2, 4, 8), "bits must be 2, 4 or 8")
     for t, name in ((rowptr, "rowptr"), (col, "col"), (value, "value"), (mat, "dense operand"), (output, "packed buffer"),
                     (quantized_params, "quantisation parameters")):
@@ -192,7 +192,8 @@ def spmm_quantize_for_all_procs(rowptr: torch.Tensor, col: torch.Tensor, value: 
     rows_d, packed_d, packed_rows, covered = _packed_range(work_range_per_proc, bits, dev)
     _require(covered == rows, "work range does not cover the product's rows")
     _require(output.numel() >= packed_rows * feat, "packed buffer too small")
-    if feat % 4 != 0 or feat > 512 or mat.stride(0) % 4 != 0 or mat.data_ptr() % 16 != 0 or output.data_ptr() % 4 != 0:
+    if (feat % 4 != 0 or feat > 512 or mat.stride(0) % 4 != 0 or mat.data_ptr() % 16 != 0 or output.data_ptr() % 4 != 0
+            or col.numel() == 0 or rows == 0):
         return False
     _lib.check_index(col, mat.size(0), what="column indices of the sparse matrix")
     with torch.cuda.device(dev):

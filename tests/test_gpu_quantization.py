@@ -309,6 +309,10 @@ def test_product_with_quantised_result_rows_leaves_other_widths_to_the_two_calls
                                                    q.quantized_send_params_buf_fp32, q.quantized_work_range_per_proc, 1, 2)
         assert torch.equal(q.quantized_send_data_buf, before)
     q = CommBufferForQuantization(cs, 8, 2, device="cuda")
+    none = torch.zeros(0, dtype=torch.int64, device="cuda")   # a matrix without stored elements
+    assert not ops.spmm_quantize_for_all_procs(torch.zeros(4, dtype=torch.int64, device="cuda"), none, v[:0],
+                                               torch.ones(2, 8, device="cuda"), q.quantized_send_data_buf,
+                                               q.quantized_send_params_buf_fp32, q.quantized_work_range_per_proc, 1, 2)
     with pytest.raises(RuntimeError, match="outside"):   # a column index beyond the dense operand's rows
         ops.spmm_quantize_for_all_procs(rp, torch.tensor([0, 2], device="cuda"), v, torch.ones(2, 8, device="cuda"),
                                         q.quantized_send_data_buf, q.quantized_send_params_buf_fp32,
