@@ -61,6 +61,7 @@ EXPORTS = (
     "gnnagg_gather_quantize_segments_f32",
     "gnnagg_dequantize_segments_f32",
     "gnnagg_plan_spmm_quantized_f32",
+    "gnnagg_plan_spmm_quantized_elements_f32",
     "gnnagg_plan_spmm_bf16_f32",
     "gnnagg_quantize_mixed_f32",
     "gnnagg_dequantize_mixed_f32",
@@ -206,6 +207,8 @@ def lib() -> ctypes.CDLL:
     L.gnnagg_dequantize_segments_f32.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp]
     L.gnnagg_plan_spmm_quantized_f32.restype = i32
     L.gnnagg_plan_spmm_quantized_f32.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i32, i32, vp]
+    L.gnnagg_plan_spmm_quantized_elements_f32.restype = i32
+    L.gnnagg_plan_spmm_quantized_elements_f32.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i32, i32, vp]
     L.gnnagg_plan_spmm_bf16_f32.restype = i32
     L.gnnagg_plan_spmm_bf16_f32.argtypes = [vp, vp, vp, i32, i64, vp, i32, i64, i64, i32, vp]
     L.gnnagg_quantize_mixed_f32.restype = i32

@@ -695,9 +695,9 @@ extern "C" int gnnagg_plan_spmm_packed_f32(gnnagg_plan *plan, const float *value
     return GNNAGG_OK;
 }
 
-extern "C" int gnnagg_plan_spmm_quantized_f32(gnnagg_plan *plan, const float *value, const uint8_t *packed,
-                                              const float *params, const int32_t *row_code, float *out,
-                                              int64_t out_stride, int64_t feat, int bits, int accumulate, void *stream) {
+static int plan_spmm_quantized(gnnagg_plan *plan, const float *value, const uint8_t *packed, const float *params,
+                               const int32_t *row_code, const int64_t *elem_code, float *out, int64_t out_stride,
+                               int64_t feat, int bits, int accumulate, void *stream) {
     GNNAGG_REQUIRE(plan, "null plan");
     GNNAGG_REQUIRE(bits == 2 || bits == 4 || bits == 8, "bits must be 2, 4 or 8 (got %d)", bits);
     GNNAGG_REQUIRE(feat >= 0, "negative feature width");
@@ -707,7 +707,8 @@ extern "C" int gnnagg_plan_spmm_quantized_f32(gnnagg_plan *plan, const float *va
         return fail(GNNAGG_ERR_UNSUPPORTED, "quantised source rows need a width that is a multiple of 4 (got %lld)",
                     (long long)feat);
     GNNAGG_REQUIRE(out, "null out");
-    GNNAGG_REQUIRE(plan->nnz == 0 || (value && packed && params && row_code), "null value/packed/params/row_code");
+    GNNAGG_REQUIRE(plan->nnz == 0 || (value && packed && params && (row_code || elem_code)),
+                   "null value/packed/params/row codes");
     GNNAGG_REQUIRE(out_stride >= feat && out_stride % 4 == 0 && out_stride < (int64_t(1) << 31),
                    "output row stride %lld must be a multiple of 4, at least the width and below 2^31",
                    (long long)out_stride);
@@ -721,7 +722,7 @@ extern "C" int gnnagg_plan_spmm_quantized_f32(gnnagg_plan *plan, const float *va
         const Shape s = pick_shape(4, feat - f_base);
         SpmmArgs a{};
         a.task = plan->task;  // every row runs in the lane-group kernel, the very longest included
-        a.col = plan->col32;
+        a.col = elem_code ? static_cast<const void *>(elem_code) : static_cast<const void *>(plan->col32);
         a.val = value;
         a.qdata = packed;
         a.qparams = params;
@@ -734,10 +735,28 @@ extern "C" int gnnagg_plan_spmm_quantized_f32(gnnagg_plan *plan, const float *va
         a.accumulate = accumulate;
         a.ntasks = plan->rows - (accumulate ? plan->nempty : 0);
         a.head_tasks = plan->nlong;
-        GNNAGG_HIP((dispatch_shape<4, int32_t, kRowsPlanned, kSrcQuant>(s, a, regions, st)));
+        if (elem_code) GNNAGG_HIP((dispatch_shape<4, int64_t, kRowsPlanned, kSrcQuant>(s, a, regions, st)));
+        else GNNAGG_HIP((dispatch_shape<4, int32_t, kRowsPlanned, kSrcQuant>(s, a, regions, st)));
         f_base += s.width();
     }
     return GNNAGG_OK;
+}
+
+extern "C" int gnnagg_plan_spmm_quantized_f32(gnnagg_plan *plan, const float *value, const uint8_t *packed,
+                                              const float *params, const int32_t *row_code, float *out,
+                                              int64_t out_stride, int64_t feat, int bits, int accumulate, void *stream) {
+    GNNAGG_REQUIRE(plan == nullptr || plan->nnz == 0 || row_code, "null row_code");
+    return plan_spmm_quantized(plan, value, packed, params, row_code, nullptr, out, out_stride, feat, bits, accumulate,
+                               stream);
+}
+
+extern "C" int gnnagg_plan_spmm_quantized_elements_f32(gnnagg_plan *plan, const float *value, const uint8_t *packed,
+                                                       const float *params, const int64_t *elem_code, float *out,
+                                                       int64_t out_stride, int64_t feat, int bits, int accumulate,
+                                                       void *stream) {
+    GNNAGG_REQUIRE(plan == nullptr || plan->nnz == 0 || elem_code, "null elem_code");
+    return plan_spmm_quantized(plan, value, packed, params, nullptr, elem_code, out, out_stride, feat, bits, accumulate,
+                               stream);
 }
 
 extern "C" int gnnagg_plan_spmm_bf16_f32(gnnagg_plan *plan, const float *value, const void *mat, int mat_is_bf16,

@@ -264,8 +264,18 @@ __device__ __forceinline__ void gather_fma(FVec<VEC> (&acc)[NCH], IdxT c_l, floa
         float zp[UU], sc[UU];
         int shift[UU];
         int code[UU];
+        if constexpr (sizeof(IdxT) == 8) {
+            // 64-bit index elements carry the row code next to the column (code << 32 | column): translated once per
+            // matrix, so that the bytes can be asked for as soon as the index chunk has arrived
 #pragma unroll
-        for (int u = 0; u < UU; ++u) code[u] = a.qcode[cc[u]];
+            for (int u = 0; u < UU; ++u) {
+                code[u] = (int)(cc[u] >> 32);
+                cc[u] &= 0xffffffffll;
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < UU; ++u) code[u] = a.qcode[cc[u]];
+        }
 #pragma unroll
         for (int u = 0; u < UU; ++u) {
             const float2 p = *reinterpret_cast<const float2 *>(a.qparams + 2 * (size_t)cc[u]);

@@ -43,7 +43,23 @@ def SPMM_backward(src: SparseTensor, other: torch.Tensor, out: torch.Tensor, acc
     return out, None
 
 
-def _spmm_quantized(plan, value, packed, params, row_code, out, bits, accumulate, operand_rows):
+def _element_codes(plan, col: torch.Tensor, row_code: torch.Tensor) -> torch.Tensor:
+    """``(row_code[col[e]] << 32) | col[e]`` per stored element, built once per (matrix, code table) and kept on the
+    plan: with it the kernel can ask for a row's bytes as soon as the index chunk has arrived.  The entry keeps the
+    code table alive, so its address cannot pass to another tensor while the entry exists; an in-place change bumps
+    ``_version``."""
+    cache = plan.__dict__.setdefault("_element_codes", {})
+    key = (row_code.data_ptr(), row_code._version, int(row_code.numel()))
+    hit = cache.get(key)
+    if hit is None:
+        if len(cache) >= 4:
+            cache.clear()
+        codes = (row_code[col].to(torch.int64) << 32) | col
+        hit = cache[key] = (row_code, codes.contiguous())
+    return hit[1]
+
+
+def _spmm_quantized(plan, value, packed, params, row_code, out, bits, accumulate, operand_rows, col=None):
     if not all(t.is_cuda for t in (value, packed, params, row_code, out)):
         raise RuntimeError("quantised SpMM operands must be GPU (HIP) tensors; there is no CPU path")
     feat = out.size(1) if out.dim() == 2 else -1
@@ -55,10 +71,19 @@ def _spmm_quantized(plan, value, packed, params, row_code, out, bits, accumulate
                            "parameters, int32 [rows] row codes and a float32 [*, F] output with contiguous rows")
     # the kernel addresses byte row (row_code >> 3) of the packed buffer: checked once per code tensor and buffer height
     _lib.check_index(row_code, packed.size(0), shift=3, what="row codes of the packed buffer")
+    L = _lib.lib()
     with torch.cuda.device(out.device):
-        _lib.check(_lib.lib().gnnagg_plan_spmm_quantized_f32(
-            plan._handle, _lib.ptr(value.contiguous()), _lib.ptr(packed), _lib.ptr(params), _lib.ptr(row_code),
-            _lib.ptr(out), _row_stride(out), feat, int(bits), 1 if accumulate else 0, _lib.current_stream(out.device)))
+        if col is not None and col.numel() > 0:
+            codes = _element_codes(plan, col, row_code)
+            _lib.check(L.gnnagg_plan_spmm_quantized_elements_f32(
+                plan._handle, _lib.ptr(value.contiguous()), _lib.ptr(packed), _lib.ptr(params), _lib.ptr(codes),
+                _lib.ptr(out), _row_stride(out), feat, int(bits), 1 if accumulate else 0,
+                _lib.current_stream(out.device)))
+        else:
+            _lib.check(L.gnnagg_plan_spmm_quantized_f32(
+                plan._handle, _lib.ptr(value.contiguous()), _lib.ptr(packed), _lib.ptr(params), _lib.ptr(row_code),
+                _lib.ptr(out), _row_stride(out), feat, int(bits), 1 if accumulate else 0,
+                _lib.current_stream(out.device)))
 
 
 def SPMM_forward_quantized(src: SparseTensor, packed: torch.Tensor, params: torch.Tensor, row_code: torch.Tensor,
@@ -67,12 +92,12 @@ def SPMM_forward_quantized(src: SparseTensor, packed: torch.Tensor, params: torc
     ``SPMM_forward`` whose dense operand is a boundary buffer still in its exchange format
     (``CommBufferForQuantization``: packed bytes, per-row parameters, ``*_row_code``).  Equal,
     bit for bit, to dequantising first."""
-    _, _, value = src.csr()
+    _, col, value = src.csr()
     if value is None:
         raise RuntimeError("Input mismatch: the sparse matrix has no values")
     if out.size(0) < src.sparse_size(0):
         raise RuntimeError("Input mismatch: out has fewer rows than the sparse matrix")
-    _spmm_quantized(src.get_plan(), value, packed, params, row_code, out, bits, accumulate, src.sparse_size(1))
+    _spmm_quantized(src.get_plan(), value, packed, params, row_code, out, bits, accumulate, src.sparse_size(1), col)
     return None
 
 
@@ -85,5 +110,5 @@ def SPMM_backward_quantized(src: SparseTensor, packed: torch.Tensor, params: tor
     if out.size(0) < src.sparse_size(1):
         raise RuntimeError("Input mismatch: out has fewer rows than the sparse matrix has columns")
     _spmm_quantized(src.get_plan_for_transpose(), value_T, packed, params, row_code, out, bits, accumulate,
-                    src.sparse_size(0))
+                    src.sparse_size(0), src.storage.row_T())
     return out, None

@@ -456,6 +456,13 @@ int gnnagg_spmm_csr_quantize_segments_f32(const int64_t *rowptr, const int64_t *
 int gnnagg_plan_spmm_quantized_f32(gnnagg_plan *plan, const float *value, const uint8_t *packed, const float *params,
                                    const int32_t *row_code, float *out, int64_t out_stride, int64_t feat, int bits,
                                    int accumulate, void *stream);
+/* The same product with the row codes translated once per matrix: elem_code int64 [nnz], entry e =
+ * (row_code[col[e]] << 32) | col[e] in the order of the CSR arrays the plan was made from (the caller builds it once
+ * per matrix and code table).  The kernel then asks for a row's bytes as soon as its index chunk has arrived -- two
+ * dependent loads per gather instead of three; same result bit for bit. */
+int gnnagg_plan_spmm_quantized_elements_f32(gnnagg_plan *plan, const float *value, const uint8_t *packed,
+                                            const float *params, const int64_t *elem_code, float *out,
+                                            int64_t out_stride, int64_t feat, int bits, int accumulate, void *stream);
 
 /* The pre- and post-aggregation of a 16-bit exchange (communicator.py:111-137) without the two tensor copies around
  * it: gnnagg_plan_spmm_strided_f32 whose dense operand rows and / or result rows are bf16.

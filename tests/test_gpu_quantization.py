@@ -233,6 +233,13 @@ def test_aggregation_straight_from_packed_bytes_equals_dequantise_then_aggregate
     SPMM_forward_quantized(adj, qbuf.quantized_recv_data_buf, qbuf.quantized_recv_params_buf_fp32, qbuf.recv_row_code,
                            got2, bits, accumulate=False)
     assert torch.equal(got2, want2)
+    # the same product looking each row's code up per gather (row codes not translated per element beforehand)
+    from gnn_benchmark_amd.spmm_kernel import _spmm_quantized
+
+    got2b = torch.empty_like(out0)
+    _spmm_quantized(adj.get_plan(), adj.csr()[2], qbuf.quantized_recv_data_buf, qbuf.quantized_recv_params_buf_fp32,
+                    qbuf.recv_row_code, got2b, bits, False, halo)
+    assert torch.equal(got2b, want2)
     # transposed: the operand has one row per ROW of the matrix
     adj_t = SparseTensor(rowptr=dev(rowptr), col=dev(col), value=dev(val), sparse_sizes=(rows_a, halo), is_sorted=True)
     cs_t = CommSplits([1, 1, 1, 1], [300, 0, 399, 1], 4, bits)
