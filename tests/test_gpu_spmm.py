@@ -501,6 +501,16 @@ def test_more_than_2_to_31_stored_elements():
     assert torch.equal(out, want)
     tail = out[-3:].clone()  # the rows whose elements start beyond 2^31
     assert rowptr[-4] > 2 ** 31 and torch.equal(tail, want[-3:])
+    # the product that quantises its result rows walks the same arrays with 64-bit offsets: F = 4 (two more columns
+    # of the same kind), int8 codes and parameters equal to quantising the exact sums
+    x4 = torch.cat((x, x + 2.0), dim=1).contiguous()
+    want4 = torch.cat((want, want + 2.0 * per_row), dim=1).contiguous()
+    work_range = torch.tensor([0, rows // 3, rows], dtype=torch.int32)
+    one, two = (torch.empty(rows, 4, dtype=torch.uint8, device="cuda") for _ in range(2))
+    p_one, p_two = (torch.empty(rows, 2, device="cuda") for _ in range(2))
+    assert computation_ops.spmm_quantize_for_all_procs(rowptr, col, val, x4, one, p_one, work_range, 2, 8)
+    computation_ops.quantize_tensor_for_all_procs(want4, two, p_two, work_range, 2, 8)
+    assert torch.equal(one, two) and torch.equal(p_one, p_two)
 
 
 def test_dense_operands_beyond_2_to_31_floats():
