@@ -1067,9 +1067,40 @@ def run_c5(args, graph):
         out[f"loss_{tag}"] = [round(v, 5) for v in losses + [float(loss)]]
         del model, opt
     del folded
+    from gnn_benchmark_amd import synthetic
+    from gnn_benchmark_amd.data_manager import CommBuffer, CommBufferForQuantization, CommSplits
+
+    # the default step with the boundary rows of every layer travelling as bf16 / as int2 (the reference's runs
+    # exchange at `--num_bits=2`); the rows a peer would have sent stand ready on the device
+    world = len(graph.comm_splits.send_splits)
+    fp32_splits, fp32_buf = graph.comm_splits, graph.comm_buf
+    for bits in (16, 2):
+        if bits == 16:
+            graph.comm_buf = CommBuffer(fp32_splits, max(dims), 16, device=dev)
+            synthetic.PregeneratedHaloExchange.attach(graph)
+            graph.exchange_bf16 = synthetic.PregeneratedBf16HaloExchange(args.seed + 7)
+        else:
+            graph.comm_splits = CommSplits(fp32_splits.recv_splits, fp32_splits.send_splits, world, 2)
+            graph.comm_buf_for_quantization = CommBufferForQuantization(graph.comm_splits, max(dims), 2, device=dev)
+            graph.exchange_quantized = synthetic.PregeneratedQuantizedHaloExchange(args.seed + 6)
+        torch.manual_seed(args.seed)
+        model = gcn.GCN(dims, num_bits=bits).to(dev)
+        opt = torch.optim.Adam(model.parameters(), lr=0.01)
+        losses = [float(gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks)) for _ in range(2)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            loss = gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks)
+        torch.cuda.synchronize()
+        tag = "fp32_gemm_bf16_exchange" if bits == 16 else "fp32_gemm_int2_exchange"
+        out[f"train_step_ms_{tag}"] = round((time.perf_counter() - t0) * 1e3 / steps, 2)
+        out[f"loss_{tag}"] = [round(v, 5) for v in losses + [float(loss)]]
+        del model, opt
+        graph.comm_splits, graph.comm_buf = fp32_splits, fp32_buf
+        graph.exchange_bf16 = graph.exchange_quantized = graph.comm_buf_for_quantization = None
+        torch.cuda.empty_cache()
     # the same default step with the stand-in exchange drawing its rows inside the step (random-number kernels in
     # the timed region, which a real exchange would not run): how much of a step that was
-    from gnn_benchmark_amd import synthetic
 
     kept = graph.exchange
     graph.exchange = synthetic.SeededHaloExchange(kept.seed, std=kept.std, backward_std=kept.backward_std)

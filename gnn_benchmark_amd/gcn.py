@@ -427,11 +427,12 @@ class _BiasReluDropoutPacked(torch.autograd.Function):
 
 
 class GCNLayer(torch.nn.Module):
-    def __init__(self, in_channels: int, out_channels: int, gemm: str = "fp32"):
+    def __init__(self, in_channels: int, out_channels: int, gemm: str = "fp32", num_bits: int = 32):
         super().__init__()
         if gemm not in _FORMS:
             raise ValueError("gemm must be 'fp32', 'bf16' or 'bf16x3'")
         self.gemm = gemm
+        self.num_bits = num_bits  # width of the boundary rows on the wire (``Aggregator``'s fourth argument)
         self.linear_first = False
         self.fuse = True  # use the fused layer kernels where they apply
         self.weight = torch.nn.Parameter(torch.empty(in_channels, out_channels))
@@ -451,11 +452,11 @@ class GCNLayer(torch.nn.Module):
         product comes first, A (x W): the same up to rounding, and the aggregation, its backward
         and the boundary rows then have the output width."""
         if isinstance(x, tuple):
-            agg = AggregatorPacked.apply(graph, x[0], x[1], layer, 32, is_pre_delay, self.training)
+            agg = AggregatorPacked.apply(graph, x[0], x[1], layer, self.num_bits, is_pre_delay, self.training)
             return self._product(agg)
         if self.linear_first:
-            return Aggregator.apply(graph, self._product(x), layer, 32, is_pre_delay, self.training)
-        return self._product(Aggregator.apply(graph, x, layer, 32, is_pre_delay, self.training))
+            return Aggregator.apply(graph, self._product(x), layer, self.num_bits, is_pre_delay, self.training)
+        return self._product(Aggregator.apply(graph, x, layer, self.num_bits, is_pre_delay, self.training))
 
     def fused(self, graph, x, layer: int, is_pre_delay: bool, keep_bits, scale: float, relu: bool,
               pack_out: bool = False):
@@ -468,9 +469,9 @@ class GCNLayer(torch.nn.Module):
         if not fused_layer_supported(probe, self.weight.size(0), self.weight.size(1)):
             return None
         if isinstance(x, tuple):
-            agg = AggregatorPacked.apply(graph, x[0], x[1], layer, 32, is_pre_delay, self.training)
+            agg = AggregatorPacked.apply(graph, x[0], x[1], layer, self.num_bits, is_pre_delay, self.training)
         else:
-            agg = Aggregator.apply(graph, x, layer, 32, is_pre_delay, self.training)
+            agg = Aggregator.apply(graph, x, layer, self.num_bits, is_pre_delay, self.training)
         agg = _kernel_ready(agg)
         row_div = _row_divisors(graph)
         row_div = None if row_div is None else row_div.reshape(-1)
@@ -490,9 +491,9 @@ class GCNLayer(torch.nn.Module):
 
 class GCN(torch.nn.Module):
     def __init__(self, dims: Sequence[int], gemm: str = "fp32", dropout: float = 0.5, packed_activations: bool = False,
-                 linear_first_when_narrowing: bool = False, fused_layers: bool = True):
+                 linear_first_when_narrowing: bool = False, fused_layers: bool = True, num_bits: int = 32):
         super().__init__()
-        self.layers = torch.nn.ModuleList([GCNLayer(dims[i], dims[i + 1], gemm) for i in range(len(dims) - 1)])
+        self.layers = torch.nn.ModuleList([GCNLayer(dims[i], dims[i + 1], gemm, num_bits) for i in range(len(dims) - 1)])
         for layer in self.layers:  # one-kernel layers where they apply (fp32 products, dense activations)
             layer.fuse = fused_layers
         if linear_first_when_narrowing:  # a layer with fewer outputs than inputs aggregates its outputs

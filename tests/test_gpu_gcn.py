@@ -181,6 +181,40 @@ def test_default_train_step_calls_no_library_product(gemm, packed_activations, m
         assert np.isfinite(loss) and abs(loss - want) < 0.5
 
 
+@pytest.mark.parametrize("num_bits", [2, 16])
+@pytest.mark.parametrize("packed_activations", [False, True])
+def test_train_step_with_narrow_boundary_rows(num_bits, packed_activations):
+    """``GCN(num_bits=2 / 16)``: the boundary rows of every layer travel as int2 / bf16.  The products that write and
+    read the exchange format themselves (the default) give, step after step, the losses and parameters of the
+    reference's separate codec passes bit for bit; and the loss of the first step stays close to the fp32 exchange's
+    (the stand-in delivers other rows, so only roughly)."""
+    dev = "cuda:0"
+    n, dims, part_args = _SHAPES["c5_widths"]
+    part = synthetic.partition_edges(n, *part_args, seed=3, device=dev)
+    gen = torch.Generator(device=dev).manual_seed(1)
+    x = torch.randn(n, dims[0], device=dev, generator=gen)
+    labels = torch.randint(0, dims[-1], (n,), device=dev, generator=gen)
+    train_idx = torch.randperm(n, device=dev, generator=gen)[: n // 10]
+    masks = gcn.make_dropout_masks(n, dims, 0.5, 7, dev)
+    runs = []
+    for fused in (True, False):
+        graph = synthetic.build_partition_graph(part, max(dims), True, exchange=synthetic.SeededHaloExchange(5),
+                                                bits=num_bits, exchange_quantized=synthetic.SeededQuantizedHaloExchange(9),
+                                                exchange_bf16=synthetic.SeededBf16HaloExchange(9), device=dev)
+        graph.fuse_quantize = graph.fuse_dequantize = graph.fuse_bf16_staging = fused
+        torch.manual_seed(0)
+        model = gcn.GCN(dims, packed_activations=packed_activations, num_bits=num_bits).to(dev)
+        opt = torch.optim.Adam(model.parameters(), lr=0.01)
+        losses = [float(gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks)) for _ in range(3)]
+        hook = graph.exchange_quantized if num_bits == 2 else graph.exchange_bf16
+        assert len(hook.calls) == 3 * 5 and not graph.exchange.calls  # 3 layers forward, 2 backward (layer 0 needs none)
+        runs.append((losses, [p.detach().clone() for p in model.parameters()]))
+    assert runs[0][0] == runs[1][0] and all(np.isfinite(runs[0][0]))
+    for a, b in zip(runs[0][1], runs[1][1]):
+        assert torch.equal(a, b)
+    assert 4.0 < runs[0][0][0] < 7.0
+
+
 @pytest.mark.parametrize("rows,feat", [(1000, 256), (333, 47), (64, 4), (1, 1)])
 @pytest.mark.parametrize("with_mask", [True, False])
 @pytest.mark.parametrize("with_div", [True, False])
