@@ -1,5 +1,6 @@
 """Seeded random sweep over shapes the hand-picked cases do not name: every SpMM path
-(plan, plan-less, transposed) and the row-packed codec, bit for bit against the oracle; packed
+(plan, plan-less, transposed), the row-packed codec and the producers that write it themselves, bit for bit against the
+oracle; packed
 and strided operands bit for bit against the dense / contiguous product; the fused LayerNorm
 pass against torch's fp64 ops (5e-5 absolute on outputs, 2e-4 relative on gradients)."""
 import numpy as np
@@ -85,6 +86,51 @@ def test_random_shapes_match_oracle_bit_for_bit(seed):
         ops.dequantize_tensor_for_all_procs(packed, back, dev(wire), work_range, nseg, bits)
         want_back = oq.dequantize_segments(want_packed, wire, splits, bits)
         assert np.array_equal(back.cpu().numpy().view(np.uint32), want_back.view(np.uint32)), ("dequantised", what, bits)
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_products_and_gathers_that_write_the_exchange_format(seed):
+    """The pre-aggregation writing packed int2 / int4 / int8 rows itself and the gather folded into the quantise pass:
+    bytes and parameters equal the oracle codec over the oracle product (over the gathered rows), bit for bit --
+    ragged segments, empty and several-chunk rows, strided operands, every lane-group shape of the kernels."""
+    rng = np.random.default_rng(7000 + seed)
+    for case in range(20):
+        bits = int(rng.choice([2, 4, 8]))
+        feat = int(rng.choice([4, 8, 36, 64, 68, 100, 128, 132, 256, 260, 512]))
+        rows = int(rng.choice([1, 2, 3, 5, 17, 64, 255, 1000]))
+        cols = int(rng.choice([1, 7, 300, 5000]))
+        kind = rng.random(rows)
+        deg = np.where(kind < 0.2, 0, np.where(kind < 0.9, rng.integers(1, 12, rows), rng.integers(30, 300, rows)))
+        rowptr = np.concatenate(([0], np.cumsum(deg))).astype(np.int64)
+        nnz = int(rowptr[-1])
+        col = rng.integers(0, cols, nnz).astype(np.int64)
+        val = rng.standard_normal(nnz).astype(np.float32)
+        nseg = int(rng.choice([1, 2, 4, 9]))
+        splits = np.diff(np.concatenate(([0], np.sort(rng.integers(0, rows + 1, nseg - 1)), [rows]))).tolist()
+        work_range = torch.tensor(np.concatenate(([0], np.cumsum(splits))).astype(np.int32))
+        wide = (rng.standard_normal((cols, feat + 8)) * rng.uniform(0.01, 30, (cols, 1))).astype(np.float32)
+        strided = bool(rng.integers(0, 2))
+        x_host = np.ascontiguousarray(wide[:, 4:4 + feat] if strided else wide[:, :feat])
+        wide_d = dev(wide)
+        x = wide_d[:, 4:4 + feat] if strided else wide_d[:, :feat].contiguous()
+        what = dict(seed=seed, case=case, bits=bits, feat=feat, rows=rows, cols=cols, nnz=nnz, nseg=nseg, strided=strided)
+        per = 8 // bits
+        packed_rows = sum(-(-int(v) // per) for v in splits)
+        if nnz:
+            send = ospmm.spmm(rowptr, col, val, x_host, np.zeros((rows, feat), np.float32))
+            o_bytes, o_params = oq.quantize_segments(send, splits, bits)
+            got = torch.full((packed_rows, feat), 0xAB, dtype=torch.uint8, device="cuda")
+            params = torch.full((rows, 2), -7.0, device="cuda")
+            assert ops.spmm_quantize_for_all_procs(dev(rowptr), dev(col), dev(val), x, got, params, work_range, nseg, bits), what
+            assert np.array_equal(got.cpu().numpy(), o_bytes), what
+            assert np.array_equal(params.cpu().numpy().view(np.uint32), o_params.view(np.uint32)), what
+        index = rng.integers(0, cols, rows).astype(np.int64)
+        o_bytes, o_params = oq.quantize_segments(x_host[index], splits, bits)
+        got = torch.full((packed_rows, feat), 0xAB, dtype=torch.uint8, device="cuda")
+        params = torch.full((rows, 2), -7.0, device="cuda")
+        ops.gather_quantize_for_all_procs(dev(x_host), dev(index), got, params, work_range, nseg, bits)
+        assert np.array_equal(got.cpu().numpy(), o_bytes), what
+        assert np.array_equal(params.cpu().numpy().view(np.uint32), o_params.view(np.uint32)), what
 
 
 @pytest.mark.parametrize("seed", range(4))
