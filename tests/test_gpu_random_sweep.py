@@ -1,8 +1,7 @@
 """Seeded random sweep over shapes the hand-picked cases do not name: every SpMM path
 (plan, plan-less, transposed), the row-packed codec and the producers that write it themselves, bit for bit against the
-oracle; packed
-and strided operands bit for bit against the dense / contiguous product; the fused LayerNorm
-pass against torch's fp64 ops (5e-5 absolute on outputs, 2e-4 relative on gradients)."""
+oracle; packed and strided operands bit for bit against the dense / contiguous product; the fused LayerNorm pass against
+torch's fp64 ops (5e-5 absolute on outputs, 2e-4 relative on gradients)."""
 import numpy as np
 import pytest
 import torch
