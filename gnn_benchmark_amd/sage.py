@@ -317,8 +317,10 @@ class DistSAGEConvGrad(torch.nn.Module):
         # linear_first: apply lin_neigh before aggregating (same result up to rounding; the
         # aggregation and the exchange then run at out_channels)
         self.linear_first = linear_first
-        # gemm "bf16x3": the layer's dense products in libgnnagg's kernels with every fp32 operand as three bf16
-        # pieces (fp32 accuracy on the bf16 matrix units); "fp32": the BLAS library's products
+        # gemm "bf16x3": all of the layer's dense products in libgnnagg's kernels with every fp32 operand as three bf16
+        # pieces (fp32 accuracy on the bf16 matrix units); "fp32": the stacked product and the input-gradient product
+        # likewise (plain products, for which that form is the fastest fp32-accurate one), the weight gradients with the
+        # fp32 matrix instruction
         if gemm not in ("fp32", "bf16x3"):
             raise ValueError("gemm must be 'fp32' or 'bf16x3'")
         self.gemm = gemm
