@@ -6,20 +6,27 @@ A^T @ G on a seeded power-law graph of 2.45 M nodes / ~122 M stored elements wit
 GCN-normalised fp32 values and a 2.45 M x 100 fp32 dense operand.  One "step" is one
 forward plus one backward, with every input already resident in HBM.
 
-Prints ONE JSON line.  ``value`` is the FLOP rate of the whole step (2 * nnz * F per
-product).  ``roofline`` prices the dominant kernel (the forward's row kernel) against
-the 8 TB/s HBM peak with the no-reuse gather byte model
+Prints ONE compact JSON line on stdout (a few KB), last.  ``value`` is the FLOP rate of the whole
+step (2 * nnz * F per product).  ``roofline`` prices the dominant kernel (the forward's row
+kernel) against the 8 TB/s HBM peak with the no-reuse gather byte model
     bytes = nnz*(8+4) + (rows+1)*8 + nnz*F*4 + 2*rows*F*4
 over the rows / stored elements that launch covers, divided by its duration measured
 with HIP events on the launch stream inside the timed region.  ``cpu_baseline`` is the
 reference's own compiled operator (or the C port of it when that cannot run on the
-host) timed on this machine's cores on the same matrices.
+host) timed on this machine's cores on the same matrices.  ``parity`` is the gate in front of
+the number: the GPU results of the headline operands (and, when c4 runs, of a seeded row sample
+of the partition's pipeline) against that CPU operator, rel 1e-5 / abs 1e-6; a failure exits
+non-zero and prints no value.  ``targets`` summarises the partition workload: the six products of
+the pipeline as a fraction of the HBM peak, and the train steps.
 
-``extra`` carries the other workloads, run after the timed headline: c1 (the single-rank 2-layer GCN
-forward + backward, with the same step on the host cores beside it), c2 at F=128/256,
-c3 (dense-degree mean aggregation, F=602/256), c4 (one partition of a 16-way split:
-pre-aggregation, local SpMM, post-aggregation, F=128) and c5 (3-layer GCN train step and the
-reference's 3-layer SAGE model on the c4 partition).  ``--only headline`` skips them.
+The other workloads run after the timed headline: c1 (the single-rank 2-layer GCN forward +
+backward, with the same step on the host cores beside it), c2 at other widths, c3 (dense-degree
+mean aggregation, F=602/256), c4 (one partition of a 16-way split: pre-aggregation, local SpMM,
+post-aggregation, F=128) and c5 (3-layer GCN train step and the reference's 3-layer SAGE model
+on the c4 partition).  Their full reports do not go into the stdout line: each is written, as
+soon as its workload has finished, as one JSON line to stderr and into the side file
+``--extra-out`` (default gpurun_out/bench_extra.json), so a late failure loses nothing.
+``--only headline`` skips them.
 """
 import argparse
 import json
@@ -32,6 +39,69 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak
+MAX_LINE_BYTES = 6000   # the stdout line stays a few KB: everything else goes to the side file and stderr
+
+
+def _finite(obj):
+    """`obj` with non-finite floats replaced by their names (strict JSON has no NaN / Infinity)."""
+    if isinstance(obj, float):
+        return obj if obj == obj and abs(obj) != float("inf") else str(obj)
+    if isinstance(obj, dict):
+        return {k: _finite(v) for k, v in obj.items()}
+    if isinstance(obj, (list, tuple)):
+        return [_finite(v) for v in obj]
+    return obj
+
+
+class ExtraSink:
+    """Full reports of the workloads besides the headline: each goes to stderr as one JSON line and into the side
+    file (rewritten whole, atomically) the moment its workload has finished."""
+
+    def __init__(self, path):
+        self.path, self.data, self.keys, self.failed = path, {}, [], None
+
+    def put(self, key, value):
+        value = _finite(value)
+        self.data[key] = value
+        self.keys.append(key)
+        print(json.dumps({"extra": key, "report": value}, allow_nan=False), file=sys.stderr, flush=True)
+        if self.path:
+            try:
+                os.makedirs(os.path.dirname(os.path.abspath(self.path)), exist_ok=True)
+                with open(self.path + ".tmp", "w") as f:
+                    json.dump(self.data, f, allow_nan=False, indent=1)
+                os.replace(self.path + ".tmp", self.path)
+            except OSError as e:  # a read-only tree: stderr still has everything
+                self.failed = str(e)
+        return value
+
+    def where(self):
+        if not self.path or self.failed:
+            return "stderr only" + (f" ({self.failed})" if self.failed else "")
+        return os.path.relpath(self.path, ROOT)
+
+
+def c4_targets(c4):
+    """The compact summary of the partition workload for the stdout line: per product of the pipeline, as the
+    Aggregator runs it, [ms, fraction of the HBM peak on the model bytes, the same on the measured bytes (or null)];
+    and the whole autograd.Function."""
+    short = {"pre-aggregation A_to@X -> send_buf": "pre", "local A_local@X -> out": "local",
+             "post-aggregation A_from@recv_buf -> out": "post", "pre-aggregation transposed": "pre_T",
+             "local transposed": "local_T", "post-aggregation transposed": "post_T"}
+    products = {}
+    for op in c4["ops"]:
+        if not op.get("as_run_by_aggregator"):
+            continue
+        name = next((v for k, v in short.items() if op["op"].startswith(k)), None)
+        if name is not None:
+            products[name] = [op["ms"], op["frac_model"], op.get("frac_measured")]
+    out = {"products_ms_fracmodel_fracmeasured": products, "feat": c4["feat"],
+           "min_frac_model": min((v[1] for v in products.values()), default=None)}
+    for k in ("aggregator_forward_ms", "aggregator_forward_backward_ms", "aggregator_forward_ms_one_launch",
+              "aggregator_forward_backward_ms_one_launch", "aggregator_forward_backward_ms_int2_exchange"):
+        if k in c4:
+            out[k] = c4[k]
+    return out
 
 # HBM-side traffic of ONE launch, measured with rocprofv3 --pmc on this file's own workloads (default sizes and
 # seed): bytes read = 32 / 64 / 128-byte read requests of the L2 to the memory side, counted by size
@@ -194,8 +264,56 @@ def cpu_description(kind, threads):
             "protocol": "median of 5 timed calls after 2 warm-ups, OpenMP threads = the host share given to this job"}
 
 
-def cpu_baseline_spmm(src, x_host, g_host):
-    """Forward + transposed backward of the headline workload on the host cores."""
+PARITY_REL, PARITY_ABS = 1e-5, 1e-6  # the gate's tolerance: |gpu - cpu| <= ABS + REL * |cpu|
+
+
+def parity_excess(got, want):
+    """(worst |got - want| - (ABS + REL * |want|), bit-identical?) of two fp32 arrays, in slabs."""
+    import numpy as np
+
+    assert got.shape == want.shape, (got.shape, want.shape)
+    worst, same = -PARITY_ABS, True
+    step = max(1, (1 << 24) // max(1, got.shape[1]))
+    for lo in range(0, got.shape[0], step):
+        a, b = got[lo:lo + step].astype(np.float64), want[lo:lo + step].astype(np.float64)
+        if not np.isfinite(a).all():
+            return float("inf"), False
+        worst = max(worst, float((np.abs(a - b) - (PARITY_ABS + PARITY_REL * np.abs(b))).max(initial=-1.0)))
+        same = same and bool(np.array_equal(got[lo:lo + step], want[lo:lo + step]))
+    return worst, same
+
+
+class ParityGate:
+    """Collects the comparisons of GPU results with the CPU operator; `record` exits the process (status 4, nothing
+    on stdout) on the first one outside the tolerance -- no number is printed for results that differ."""
+
+    def __init__(self, enabled):
+        self.enabled, self.cases, self.kind = enabled, {}, None
+
+    def record(self, name, got, want, what):
+        excess, same = parity_excess(got, want)
+        self.cases[name] = {"what": what, "max_excess": float(f"{excess:.3e}"), "bit_identical": same,
+                            "pass": excess <= 0.0}
+        print(json.dumps({"parity": name, **self.cases[name]}), file=sys.stderr, flush=True)
+        if not excess <= 0.0:
+            print(f"bench.py: parity gate FAILED for {name} ({what}): worst excess over abs {PARITY_ABS} + rel "
+                  f"{PARITY_REL} is {excess:.3e}; no number is reported", file=sys.stderr, flush=True)
+            sys.exit(4)
+
+    def report(self):
+        if not self.enabled:
+            return {"checked": False}
+        return {"checked": bool(self.cases), "tolerance": f"abs {PARITY_ABS} + rel {PARITY_REL}",
+                "against": f"CPU operator ({self.kind})",
+                "max_excess": max((c["max_excess"] for c in self.cases.values()), default=None),
+                "bit_identical": all(c["bit_identical"] for c in self.cases.values()),
+                "cases": {k: [c["max_excess"], c["bit_identical"]] for k, c in self.cases.items()}}
+
+
+def cpu_baseline_spmm(src, x_host, g_host, gate=None, gpu_results=None, timed=True):
+    """Forward + transposed backward of the headline workload on the host cores.  The first, fresh pair of results
+    (onto zeros) is what the parity gate compares the GPU's `gpu_results` = (A @ X, A^T @ G) with, as the reference's
+    own test does (tests/test_spmm.py:93-115); the timed calls follow."""
     import numpy as np
 
     from oracle import spmm as ospmm
@@ -218,6 +336,13 @@ def cpu_baseline_spmm(src, x_host, g_host):
         run(rowptr, col, val, x_host, out_f, rs_f)
         run(colptr, row_t, val_t, g_host, out_b, rs_b)
 
+    if gate is not None and gate.enabled:
+        step()
+        gate.kind = f"{kind}, {threads} threads"
+        gate.record("c2_forward", gpu_results[0], out_f, f"A@X, all {rows} rows, F={feat}")
+        gate.record("c2_backward", gpu_results[1], out_b, f"A^T@G, all {cols} rows, F={feat}")
+    if not timed:
+        return None
     sec = cpu_median_seconds(step)
     flops = 2 * 2.0 * col.shape[0] * feat
     r = {"value": round(flops / sec / 1e9, 3), "unit": "GFLOP/s"}
@@ -225,6 +350,42 @@ def cpu_baseline_spmm(src, x_host, g_host):
     r["sample"] = f"the whole workload: 1 forward + 1 transposed backward per step, F={feat} (7 steps, about 2 s)"
     r["ms_per_step"] = round(sec * 1e3, 2)
     return r
+
+
+def parity_rows_of_pipeline(gate, graph, x, out, recv_buf, n_sample, seed):
+    """Gate for the partition workload: rows of `out` = A_local @ x + A_from @ recv_buf (the Aggregator's forward)
+    for a seeded sample of rows plus the 64 longest, against the CPU operator run on those rows' own slices of the
+    two matrices -- local elements first, then the received ones, the order the reference accumulates in
+    (model/layers/aggregator.py:67-104)."""
+    import numpy as np
+    import torch
+
+    from oracle import spmm as ospmm
+
+    threads = ospmm.max_threads()
+    run, kind = cpu_operator(threads)
+    gate.kind = gate.kind or f"{kind}, {threads} threads"
+    rp_l = graph.local_adj_t.csr()[0]
+    deg = (rp_l[1:] - rp_l[:-1]).cpu().numpy()
+    n = deg.shape[0]
+    pick = np.unique(np.concatenate([np.argsort(deg)[-64:], np.random.default_rng(seed).integers(0, n, n_sample)]))
+    want = np.zeros((pick.shape[0], x.shape[1]), dtype=np.float32)
+    for m, operand in ((graph.local_adj_t, x), (graph.adj_t_pre_post_aggr_from, recv_buf)):
+        rowptr, col, val = m.csr()
+        rp = rowptr.cpu().numpy()
+        lens = rp[pick + 1] - rp[pick]
+        take = torch.from_numpy(np.concatenate([np.arange(rp[r], rp[r + 1]) for r in pick] + [np.zeros(0, np.int64)]))
+        take = take.to(col.device)
+        sub_ptr = np.concatenate(([0], np.cumsum(lens))).astype(np.int64)
+        sub_col, sub_val = col[take].cpu().numpy(), val[take].cpu().numpy()
+        # only the operand rows the sample touches travel to the host
+        used, inverse = np.unique(sub_col, return_inverse=True)
+        operand_host = operand[torch.from_numpy(used).to(operand.device)].cpu().numpy()
+        rs = ospmm.distribute_work_for_row(sub_ptr, np.ones(sub_col.shape[0], np.float32), threads)
+        run(sub_ptr, inverse.astype(np.int64), sub_val, operand_host, want, rs)
+    got = out[torch.from_numpy(pick).to(out.device)].cpu().numpy()
+    gate.record("c4_aggregator_forward_rows", got, want,
+                f"A_local@X + A_from@recv_buf, {pick.shape[0]} sampled rows incl. the 64 longest, F={x.shape[1]}")
 
 
 def cpu_time_product(rowptr, col, val, x_host, rows):
@@ -317,7 +478,7 @@ def spmm_kernel_name(feat, planned=True):
     return f"gnnagg::spmm_tasks_kernel<{vec},{lpr},{nch},{'int' if planned else 'long'},{1 if planned else 0},0>"
 
 
-def run_c2(args):
+def run_c2(args, gate, sink):
     import torch
 
     from gnn_benchmark_amd import synthetic
@@ -353,15 +514,31 @@ def run_c2(args):
                      "kernel_ms": r["kernel_ms"], "kernel_ms_median": r["kernel_ms_median"],
                      "kernel_ms_min": r["kernel_ms_min"], "bytes_per_launch": r["kernel_bytes"]},
     }
-    extra = {"c2": [r]}
+    sink.put("c2_headline", r)
+    # the gate (and the CPU baseline) on the headline operands themselves: one fresh product each way
+    gpu_results = None
+    if gate.enabled:
+        rows, cols = src.sparse_sizes()
+        fresh_f = torch.zeros(rows, args.feat, device=dev)
+        fresh_b = torch.zeros(cols, args.feat, device=dev)
+        src.get_plan().spmm(src.csr()[2], x, fresh_f, True)
+        src.get_plan_for_transpose().spmm(src.storage.value_T(), gr, fresh_b, True)
+        gpu_results = (fresh_f.cpu().numpy(), fresh_b.cpu().numpy())
+        del fresh_f, fresh_b
+    line["cpu_baseline"] = None
+    if gate.enabled or not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline_spmm(src, x.cpu().numpy(), gr.cpu().numpy(), gate, gpu_results,
+                                                 timed=not args.no_cpu_baseline)
+    del gpu_results
     if "c2" in args.extras:
         # the hidden widths of c4 / c5, c5's class count (172) and two narrow widths whose rows are not whole
         # 16-byte vectors or 64-byte multiples (class counts 40 and 47)
+        widths = [r]
         for f in (128, 256, 172, 40, 47):
             if f != args.feat:
-                extra["c2"].append(spmm_pair(src, f, max(3, args.steps // 4), 2, gen, args, "c2")[0])
-    line["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline_spmm(src, x.cpu().numpy(), gr.cpu().numpy())
-    return line, extra
+                widths.append(spmm_pair(src, f, max(3, args.steps // 4), 2, gen, args, "c2")[0])
+        sink.put("c2", widths)
+    return line
 
 
 def run_c1(args):
@@ -456,9 +633,27 @@ def run_c1(args):
     return r
 
 
+def load_probes():
+    """ctypes handle of bench_probes/libbenchprobes.so (built by __graft_entry__.build(); built here when missing)."""
+    import ctypes
+    import subprocess
+
+    here = os.path.join(ROOT, "bench_probes")
+    path = os.path.join(here, "libbenchprobes.so")
+    if not os.path.exists(path):
+        subprocess.check_call(["make", "-C", here, "libbenchprobes.so"], stdout=subprocess.DEVNULL)
+    L = ctypes.CDLL(path)
+    vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+    L.bench_probe_memory.restype = i32
+    L.bench_probe_memory.argtypes = [i32, vp, vp, vp, i64, i64, i64, vp]
+    L.bench_probe_issue.restype = i32
+    L.bench_probe_issue.argtypes = [i32, i32, vp, vp]
+    return L
+
+
 def run_ceilings(args):
     """What the memory system delivers, in this run, for plain kernels with the access mixes of the aggregation
-    path (`gnnagg_memory_probe`): streams, uniformly random 512-byte row gathers with nothing written, and the
+    path (bench_probes/libbenchprobes.so, `bench_probe_memory`; asked for with `--only ceilings`): streams, uniformly random 512-byte row gathers with nothing written, and the
     same gathers mixed with the row writes / row read-modify-writes of the boundary products (7 gathers per row
     written: the pre-aggregation's mix; 3 per row read and written: the post-aggregation's; 15: the local product's
     on a graph without hub rows).  Sizes of the c4 partition at F=128: 7 M source rows, 20 M gathers."""
@@ -472,16 +667,19 @@ def run_ceilings(args):
     src = torch.randn(rows, feat, device=dev, generator=gen)
     dst = torch.zeros(rows, feat, device=dev)
     index = torch.randint(0, rows, (gathers,), device=dev, generator=gen, dtype=torch.int32)
-    L = _lib.lib()
+    L = load_probes()
     stream = _lib.current_stream(dev)
+
+    def check(rc):
+        if rc != 0:
+            raise RuntimeError(f"libbenchprobes returned {rc} (1 bad argument, 2 HIP error, 3 unsupported row width)")
 
     def timed(kind, count, per_row, nbytes, reps=10):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         for i in range(reps + 2):
             if i == 2:
                 e0.record()
-            _lib.check(L.gnnagg_memory_probe(kind, _lib.ptr(src), _lib.ptr(index), _lib.ptr(dst), count, feat, per_row,
-                                             stream))
+            check(L.bench_probe_memory(kind, _lib.ptr(src), _lib.ptr(index), _lib.ptr(dst), count, feat, per_row, stream))
         e1.record()
         e1.synchronize()
         ms = e0.elapsed_time(e1) / reps
@@ -500,13 +698,13 @@ def run_ceilings(args):
         nbytes = results * per_row * (row_b + 4.0) + (results * row_b if kind >= 4 else 0) + (results * row_b if kind == 5 else 0)
         out[name] = timed(kind, results, per_row, nbytes)
 
-    # matrix pipe and vector ALU of a SIMD, fed by different waves (`gnnagg_issue_probe`): alone and together
+    # matrix pipe and vector ALU of a SIMD, fed by different waves (`bench_probe_issue`): alone and together
     def issue(mfma_rounds, valu_rounds, reps=5):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         for i in range(reps + 2):
             if i == 2:
                 e0.record()
-            _lib.check(L.gnnagg_issue_probe(mfma_rounds, valu_rounds, _lib.ptr(dst), stream))
+            check(L.bench_probe_issue(mfma_rounds, valu_rounds, _lib.ptr(dst), stream))
         e1.record()
         e1.synchronize()
         return e0.elapsed_time(e1) / reps
@@ -568,7 +766,7 @@ def build_c4(args):
     return part, graph, time.perf_counter() - t0
 
 
-def run_c4(args, graph, setup_s):
+def run_c4(args, graph, setup_s, gate=None):
     import torch
 
     from gnn_benchmark_amd import Aggregator
@@ -635,6 +833,11 @@ def run_c4(args, graph, setup_s):
         o.backward(g)
     torch.cuda.synchronize()
     both_ms = (time.perf_counter() - t0) * 1e3 / steps
+    if gate is not None and gate.enabled:
+        with torch.no_grad():
+            o = Aggregator.apply(graph, x, 0, 32, True, True)
+        parity_rows_of_pipeline(gate, graph, x, o, graph.comm_buf.recv_buf, 4000, args.seed + 11)
+    del o
     graph.comm_buf.resize_buffer(graph.comm_splits, feat, 32)  # (the buffer's own tensors again, not delivered rows)
     codec = run_c4_codec(graph, feat, steps, gen, cpu=not args.no_cpu_baseline)
     # the same autograd.Function with the boundary rows travelling as int2 (seeded packed rows)
@@ -1247,8 +1450,16 @@ def main():
     ap.add_argument("--only", default="", help="'headline' = headline workload only; or a comma list of the extra "
                                                 "workloads to add: c1 (single-rank 2-layer GCN), c2 (F=128/256 and "
                                                 "the plan-less operator), c3, c4, c5 (GCN and SAGE train steps; "
-                                                "c5sage: the SAGE one alone).  Default: c1,c2,c3,c4,c5")
+                                                "c5sage: the SAGE one alone; "
+                                                "ceilings: plain-kernel probes of the memory system).  Default: "
+                                                "c1,c2,c3,c4,c5")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-parity-gate", action="store_true",
+                    help="skip the comparison of the GPU results with the CPU operator in front of the number "
+                         "(the line then says parity.checked = false)")
+    ap.add_argument("--extra-out", default=os.path.join(ROOT, "gpurun_out", "bench_extra.json"),
+                    help="side file for the full reports of the workloads besides the headline (also written to "
+                         "stderr, one JSON line per workload as it finishes)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy 3 times (a kernel of known traffic for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -1271,31 +1482,48 @@ def main():
             b.copy_(a)
         torch.cuda.synchronize()
         del a, b
-    line, extra = run_c2(args)
+    gate = ParityGate(not args.no_parity_gate)
+    sink = ExtraSink(args.extra_out)
+    line = run_c2(args, gate, sink)
     torch.cuda.empty_cache()
+    targets = {}
     if "c1" in args.extras:
-        extra["c1"] = run_c1(args)
+        sink.put("c1", run_c1(args))
         torch.cuda.empty_cache()
-    if "c4" in args.extras or "ceilings" in args.extras:
-        extra["memory_ceilings"] = run_ceilings(args)
+    if "ceilings" in args.extras:
+        sink.put("memory_ceilings", run_ceilings(args))
         torch.cuda.empty_cache()
     if "c3" in args.extras:
-        extra["c3"] = run_c3(args)
+        sink.put("c3", run_c3(args))
         torch.cuda.empty_cache()
     if any(k in args.extras for k in ("c4", "c5", "c5sage")):
         _part, graph, setup_s = build_c4(args)
         if "c4" in args.extras:
-            extra["c4"] = run_c4(args, graph, setup_s)
+            c4 = sink.put("c4", run_c4(args, graph, setup_s, gate))
+            targets["c4"] = c4_targets(c4)
             torch.cuda.empty_cache()
-            extra["c4_raw_halo"] = run_c4_raw_halo(args, _part)
+            sink.put("c4_raw_halo", run_c4_raw_halo(args, _part))
             torch.cuda.empty_cache()
         if "c5" in args.extras:
-            extra["c5"] = run_c5(args, graph)
+            c5 = sink.put("c5", run_c5(args, graph))
+            targets["c5_gcn_train_step_ms"] = {k[len("train_step_ms_"):]: c5[k] for k in (
+                "train_step_ms_fp32_gemm", "train_step_ms_bf16_gemm", "train_step_ms_bf16x3_gemm",
+                "train_step_ms_fp32_gemm_all_nodes_through_last_layer", "train_step_ms_fp32_gemm_int2_exchange")
+                if k in c5}
             torch.cuda.empty_cache()
         if "c5" in args.extras or "c5sage" in args.extras:
-            extra["c5_sage"] = run_c5_sage(args, graph)
-    line["extra"] = extra
-    print(json.dumps(line), flush=True)
+            c5s = sink.put("c5_sage", run_c5_sage(args, graph))
+            targets["c5_sage_train_step_ms"] = {
+                (k[len("train_step_ms_"):] if len(k) > len("train_step_ms") else "default"): c5s[k] for k in (
+                    "train_step_ms", "train_step_ms_folded_degrees", "train_step_ms_folded_degrees_int2_exchange",
+                    "train_step_ms_torch_ops_around_aggregator") if k in c5s}
+    line["parity"] = gate.report()
+    line["targets"] = targets
+    line["extra_file"] = sink.where()
+    line["extra_keys"] = sorted(sink.keys)
+    text = json.dumps(line, allow_nan=False, separators=(",", ":"))
+    assert len(text) < MAX_LINE_BYTES, len(text)
+    print(text, flush=True)
 
 
 if __name__ == "__main__":

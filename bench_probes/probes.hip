@@ -1,9 +1,37 @@
-// Memory-system probes: plain kernels with the access mixes of the aggregation path and nothing else, so that a
-// benchmark can put the rate of a product kernel next to what the machine delivers for the same mix of row gathers,
-// row reads and row writes in the same run.  Measurement aids; nothing in the product path calls them.
-#include "common.h"
+// Memory-system probes of the benchmark (libbenchprobes.so, loaded by bench.py for `--only ceilings` and by nothing
+// else): plain kernels with the access mixes of the aggregation path and nothing else, so that a benchmark can put
+// the rate of a product kernel next to what the machine delivers for the same mix of row gathers, row reads and row
+// writes in the same run.  Not part of libgnnagg.so and not part of its ABI.  Return codes: 0 ok, 1 bad argument,
+// 2 HIP error, 3 unsupported row width.
+//
+//   bench_probe_memory(kind, src, index, dst, count, row_floats, per_row, stream)
+//     kind 0  read `count` floats of src as a stream (dst: 4 writable bytes, never written for finite data)
+//     kind 1  write `count` floats of dst as a stream
+//     kind 2  copy `count` floats from src to dst
+//     kind 3  `count` result rows, each the sum of `per_row` rows of src gathered through index[count * per_row]
+//             (int32 row numbers of src); the results are dropped: reads only
+//     kind 4  the same, every result row written to dst[count, row_floats]
+//     kind 5  the same, every result row added onto the row dst holds: one row read and one written per result
+//     row_floats (kinds 3-5): 64, 128 or 256; src and dst 16-byte aligned; count a multiple of 4 for kinds 0-2.
+//   bench_probe_issue(mfma_rounds, valu_rounds, sink, stream)
+//     one block of eight waves per compute unit: waves 0-3 (one per SIMD) issue `mfma_rounds` x 8 independent
+//     v_mfma_f32_32x32x16_bf16, waves 4-7 run `valu_rounds` x 8 rounds of the vector-ALU sequence that cuts a pair of
+//     fp32 values into bf16 pieces.  Timing (mfma, 0), (0, valu) and (mfma, valu) shows whether the two pipes of a
+//     SIMD overlap when different waves feed them.  sink: 4 writable bytes, never written.
+// Both allocate nothing and do not synchronise with the host.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
 
-namespace gnnagg {
+#define PROBE_REQUIRE(cond) \
+    do {                    \
+        if (!(cond)) return 1; \
+    } while (0)
+#define PROBE_HIP(expr)                    \
+    do {                                   \
+        if ((expr) != hipSuccess) return 2; \
+    } while (0)
+
+namespace benchprobes {
 namespace {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -132,25 +160,24 @@ __global__ __launch_bounds__(512) void probe_issue_kernel(float *__restrict__ si
 }
 
 }  // namespace
-}  // namespace gnnagg
+}  // namespace benchprobes
 
-using namespace gnnagg;
+using namespace benchprobes;
 
-extern "C" int gnnagg_memory_probe(int kind, const float *src, const int32_t *index, float *dst, int64_t count,
+extern "C" int bench_probe_memory(int kind, const float *src, const int32_t *index, float *dst, int64_t count,
                                    int64_t row_floats, int64_t per_row, void *stream) {
-    GNNAGG_REQUIRE(kind >= 0 && kind <= 5, "probe kind %d outside 0..5", kind);
-    GNNAGG_REQUIRE(count >= 0 && count < (int64_t(1) << 40), "bad count");
-    if (count == 0) return GNNAGG_OK;
+    PROBE_REQUIRE(kind >= 0 && kind <= 5);
+    PROBE_REQUIRE(count >= 0 && count < (int64_t(1) << 40));
+    if (count == 0) return 0;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (kind <= 2) {  // streams over `count` floats
-        GNNAGG_REQUIRE(count % 4 == 0, "stream probes take a multiple of 4 floats");
-        GNNAGG_REQUIRE((kind == 1 || src) && (kind == 0 || dst), "null src/dst");
-        GNNAGG_REQUIRE(((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) == 0,
-                       "stream probes take 16-byte aligned arrays");
+        PROBE_REQUIRE(count % 4 == 0);
+        PROBE_REQUIRE((kind == 1 || src) && (kind == 0 || dst));
+        PROBE_REQUIRE(((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) == 0);
         const size_t n4 = (size_t)count / 4;
         const unsigned blocks = 32768;
         if (kind == 0) {
-            GNNAGG_REQUIRE(dst, "the read probe needs 4 writable bytes in dst (never written for finite data)");
+            PROBE_REQUIRE(dst);
             hipLaunchKernelGGL(probe_stream_read_kernel<8>, dim3(blocks), dim3(256), 0, st,
                                reinterpret_cast<const f32x4 *>(src), n4, dst);
         } else if (kind == 1) {
@@ -159,14 +186,13 @@ extern "C" int gnnagg_memory_probe(int kind, const float *src, const int32_t *in
             hipLaunchKernelGGL(probe_stream_copy_kernel, dim3(blocks), dim3(256), 0, st,
                                reinterpret_cast<const f32x4 *>(src), reinterpret_cast<f32x4 *>(dst), n4);
         }
-        GNNAGG_HIP(hipGetLastError());
-        return GNNAGG_OK;
+        PROBE_HIP(hipGetLastError());
+        return 0;
     }
     // row gathers: `count` result rows, each the sum of `per_row` gathered rows
-    GNNAGG_REQUIRE(src && index && dst, "null src/index/dst");
-    GNNAGG_REQUIRE(per_row >= 1 && per_row < (1 << 20), "gathers per result row outside 1 .. 2^20");
-    GNNAGG_REQUIRE(((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) == 0,
-                   "gather probes take 16-byte aligned arrays");
+    PROBE_REQUIRE(src && index && dst);
+    PROBE_REQUIRE(per_row >= 1 && per_row < (1 << 20));
+    PROBE_REQUIRE(((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) == 0);
     const int mode = kind - 3;
     const unsigned blocks = 65536;
     // in mode 0 the last 4 bytes of dst stand in for the sink (never written for finite data)
@@ -178,21 +204,19 @@ extern "C" int gnnagg_memory_probe(int kind, const float *src, const int32_t *in
     else if (row_floats == 256)
         hipLaunchKernelGGL(probe_gather_kernel<64>, dim3(blocks), dim3(256), 0, st, src, index, dst, count, (int)per_row, mode, sink);
     else
-        return fail(GNNAGG_ERR_UNSUPPORTED, "gather probes exist for rows of 64, 128 and 256 floats (got %lld)",
-                    (long long)row_floats);
-    GNNAGG_HIP(hipGetLastError());
-    return GNNAGG_OK;
+        return 3;
+    PROBE_HIP(hipGetLastError());
+    return 0;
 }
 
-extern "C" int gnnagg_issue_probe(int mfma_rounds, int valu_rounds, float *sink, void *stream) {
-    GNNAGG_REQUIRE(mfma_rounds >= 0 && valu_rounds >= 0 && mfma_rounds <= (1 << 20) && valu_rounds <= (1 << 20),
-                   "rounds outside 0 .. 2^20");
-    GNNAGG_REQUIRE(sink, "null sink");
+extern "C" int bench_probe_issue(int mfma_rounds, int valu_rounds, float *sink, void *stream) {
+    PROBE_REQUIRE(mfma_rounds >= 0 && valu_rounds >= 0 && mfma_rounds <= (1 << 20) && valu_rounds <= (1 << 20));
+    PROBE_REQUIRE(sink);
     int dev = 0, cus = 0;
-    GNNAGG_HIP(hipGetDevice(&dev));
-    GNNAGG_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    PROBE_HIP(hipGetDevice(&dev));
+    PROBE_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
     hipLaunchKernelGGL(probe_issue_kernel, dim3(cus > 0 ? cus : 256), dim3(512), 0, static_cast<hipStream_t>(stream), sink,
                        mfma_rounds, valu_rounds);
-    GNNAGG_HIP(hipGetLastError());
-    return GNNAGG_OK;
+    PROBE_HIP(hipGetLastError());
+    return 0;
 }

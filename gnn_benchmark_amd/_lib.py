@@ -12,7 +12,7 @@ _CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(_CSRC, "libgnnagg.so")
 
 OK, ERR_INVALID, ERR_HIP, ERR_UNSUPPORTED = 0, 1, 2, 3
-ABI_VERSION = 1
+ABI_VERSION = 3   # GNNAGG_ABI_VERSION of include/gnn_agg.h this binding was written against
 
 EXPORTS = (
     "gnnagg_abi_version",
@@ -23,6 +23,7 @@ EXPORTS = (
     "gnnagg_plan_destroy",
     "gnnagg_plan_spmm_f32",
     "gnnagg_plan_spmm_strided_f32",
+    "gnnagg_plan_spmm_two_sources_f32",
     "gnnagg_plan_info",
     "gnnagg_plan_profile",
     "gnnagg_plan_profile_read",
@@ -67,8 +68,6 @@ EXPORTS = (
     "gnnagg_dequantize_mixed_f32",
     "gnnagg_f32_to_bf16",
     "gnnagg_bf16_to_f32",
-    "gnnagg_memory_probe",
-    "gnnagg_issue_probe",
 )
 
 _lib = None
@@ -109,6 +108,10 @@ def lib() -> ctypes.CDLL:
     vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
     L.gnnagg_abi_version.restype = i32
     L.gnnagg_abi_version.argtypes = []
+    built = L.gnnagg_abi_version()
+    if built != ABI_VERSION:   # before any prototype is trusted: a stale library would be called with shifted arguments
+        raise RuntimeError(f"{LIB_PATH} has ABI version {built}, this binding was written against {ABI_VERSION} "
+                           "(include/gnn_agg.h changed since it was built): rebuild it (make -C gnn_benchmark_amd/csrc)")
     L.gnnagg_last_error.restype = ctypes.c_char_p
     L.gnnagg_last_error.argtypes = []
     L.gnnagg_spmm_csr_f32.restype = i32
@@ -123,6 +126,8 @@ def lib() -> ctypes.CDLL:
     L.gnnagg_plan_spmm_f32.argtypes = [vp, vp, vp, vp, i64, i32, vp]
     L.gnnagg_plan_spmm_strided_f32.restype = i32
     L.gnnagg_plan_spmm_strided_f32.argtypes = [vp, vp, vp, i64, vp, i64, i64, i32, vp]
+    L.gnnagg_plan_spmm_two_sources_f32.restype = i32
+    L.gnnagg_plan_spmm_two_sources_f32.argtypes = [vp, vp, vp, i64, i64, vp, i64, vp, i64, i64, i32, vp]
     L.gnnagg_plan_info.restype = i32
     L.gnnagg_plan_info.argtypes = [vp, ctypes.POINTER(i64)]
     L.gnnagg_plan_profile.restype = i32
@@ -215,12 +220,6 @@ def lib() -> ctypes.CDLL:
     L.gnnagg_quantize_mixed_f32.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp]
     L.gnnagg_dequantize_mixed_f32.restype = i32
     L.gnnagg_dequantize_mixed_f32.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp]
-    L.gnnagg_memory_probe.restype = i32
-    L.gnnagg_memory_probe.argtypes = [i32, vp, vp, vp, i64, i64, i64, vp]
-    L.gnnagg_issue_probe.restype = i32
-    L.gnnagg_issue_probe.argtypes = [i32, i32, vp, vp]
-    if L.gnnagg_abi_version() != ABI_VERSION:
-        raise RuntimeError("libgnnagg.so was built from a different include/gnn_agg.h; rebuild it")
     _lib = L
     return L
 

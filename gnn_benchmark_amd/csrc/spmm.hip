@@ -663,6 +663,57 @@ extern "C" int gnnagg_plan_spmm_strided_f32(gnnagg_plan *plan, const float *valu
     return plan_spmm(plan, value, mat, mat_stride, out, out_stride, feat, accumulate, stream);
 }
 
+extern "C" int gnnagg_plan_spmm_two_sources_f32(gnnagg_plan *plan, const float *value, const float *mat,
+                                                int64_t mat_stride, int64_t mat_rows, const float *mat2,
+                                                int64_t mat2_stride, float *out, int64_t out_stride, int64_t feat,
+                                                int accumulate, void *stream) {
+    GNNAGG_REQUIRE(plan, "null plan");
+    GNNAGG_REQUIRE(feat >= 0, "negative feature width");
+    GNNAGG_REQUIRE(mat_rows >= 0 && mat_rows <= plan->cols, "the first source holds %lld rows, the matrix has %lld columns",
+                   (long long)mat_rows, (long long)plan->cols);
+    if (plan->rows == 0 || feat == 0) return GNNAGG_OK;
+    if (int rc = check_feat(feat)) return rc;
+    GNNAGG_REQUIRE(out, "null out");
+    GNNAGG_REQUIRE(plan->nnz == 0 || (value && (mat || mat_rows == 0) && (mat2 || mat_rows == plan->cols)),
+                   "null value/mat/mat2");
+    GNNAGG_REQUIRE(mat_stride >= feat && mat2_stride >= feat && out_stride >= feat && mat_stride < (int64_t(1) << 31) &&
+                       mat2_stride < (int64_t(1) << 31) && out_stride < (int64_t(1) << 31),
+                   "row strides %lld / %lld / %lld must be at least the width %lld and below 2^31", (long long)mat_stride,
+                   (long long)mat2_stride, (long long)out_stride, (long long)feat);
+    // a source without rows is never addressed, but the surplus gathers of a row's last round read row 0 of the
+    // first source: point it at the second one's rows then
+    if (mat_rows == 0) mat = mat2;
+    if (mat_rows == plan->cols) mat2 = mat, mat2_stride = mat_stride;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int vec = std::min(pick_vec(feat, mat, out, mat_stride, out_stride), pick_vec(feat, mat2, out, mat2_stride, out_stride));
+    const Regions regions{plan->rows_per_group, plan->short_rows_per_group,
+                          plan->nshort + (accumulate ? 0 : plan->nempty)};
+    for (int64_t f_base = 0; f_base < feat;) {
+        const Shape s = pick_shape(vec, feat - f_base);
+        SpmmArgs a{};
+        a.task = plan->task;  // every row runs in the lane-group kernel, the very longest included
+        a.col = plan->col32;
+        a.val = value;
+        a.x = mat;
+        a.ldx = (int)mat_stride;
+        a.x2 = mat2;
+        a.ldx2 = (int)mat2_stride;
+        a.x_rows = (int)mat_rows;
+        a.dst = out;
+        a.ldd = (int)out_stride;
+        a.feat = (int)feat;
+        a.f_base = (int)f_base;
+        a.accumulate = accumulate;
+        a.ntasks = plan->rows - (accumulate ? plan->nempty : 0);
+        a.head_tasks = plan->nlong;
+        if (vec == 4) GNNAGG_HIP((dispatch_shape<4, int32_t, kRowsPlanned, kSrcDense2>(s, a, regions, st)));
+        else if (vec == 2) GNNAGG_HIP((dispatch_shape<2, int32_t, kRowsPlanned, kSrcDense2>(s, a, regions, st)));
+        else GNNAGG_HIP((dispatch_shape<1, int32_t, kRowsPlanned, kSrcDense2>(s, a, regions, st)));
+        f_base += s.width();
+    }
+    return GNNAGG_OK;
+}
+
 extern "C" int gnnagg_plan_spmm_packed_f32(gnnagg_plan *plan, const float *value, const float *y_packed,
                                            const uint32_t *header, float *out, int64_t feat, int accumulate,
                                            void *stream) {

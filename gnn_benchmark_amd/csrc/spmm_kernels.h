@@ -145,6 +145,9 @@ struct SpmmArgs {
     const void *col;          // IdxT [nnz]
     const float *val;         // [nnz]
     const float *x;           // dense operand [K, F] (packed source: non-zero values at the front of each row)
+    // two dense sources (kSrcDense2): columns [0, x_rows) are rows of x, columns x_rows + k are rows k of x2
+    const float *x2;
+    int x_rows, ldx2;         // ldx2: row stride of x2 in floats; 0 stands for F
     const uint32_t *hdr;      // packed source only: [K, hdr_words] row headers
     int hdr_words;
     // quantised source only (row-packed codec of the boundary buffers): byte rows [packed_rows, F] in
@@ -177,7 +180,8 @@ enum SourceKind : int {
     kSrcDense = 0,   // x[col, :] is a dense fp32 row
     kSrcPacked = 1,  // x[col, :] holds the row's non-zero values at its front, hdr[col, :] says which
     kSrcQuant = 2,   // row col is held quantised: qdata / qparams / qcode (boundary-buffer codec layout)
-    kSrcBf16 = 3     // x[col, :] is a bf16 row (x points at 16-bit values, ldx counts them): widened in the gather
+    kSrcBf16 = 3,    // x[col, :] is a bf16 row (x points at 16-bit values, ldx counts them): widened in the gather
+    kSrcDense2 = 4   // dense fp32 rows of two arrays: x[col, :] for col < x_rows, x2[col - x_rows, :] above
 };
 
 typedef float f32x4_unaligned __attribute__((ext_vector_type(4), aligned(4)));
@@ -235,7 +239,15 @@ __device__ __forceinline__ void gather_fma(FVec<VEC> (&acc)[NCH], IdxT c_l, floa
     for (int u = 0; u < UU; ++u) {
         cc[u] = group_bcast_idx<LPR>(c_l, j + u);
         vv[u] = __int_as_float(group_bcast<LPR>(__float_as_int(v_l), j + u));
-        xr[u] = x + (size_t)cc[u] * (size_t)ldx;
+        if constexpr (SRC == kSrcDense2) {
+            const bool second = cc[u] >= (int64_t)a.x_rows;
+            const float *__restrict__ from = second ? a.x2 : x;
+            const int64_t r = second ? cc[u] - (int64_t)a.x_rows : cc[u];
+            const int ld = second ? (a.ldx2 ? a.ldx2 : F) : ldx;
+            xr[u] = from + (size_t)r * (size_t)ld;
+        } else {
+            xr[u] = x + (size_t)cc[u] * (size_t)ldx;
+        }
     }
     FVec<VEC> xv[UU][NCH];
     if constexpr (SRC == kSrcPacked) {

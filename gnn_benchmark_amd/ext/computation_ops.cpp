@@ -11,6 +11,8 @@
 #include <c10/hip/HIPGuard.h>
 #include <c10/hip/HIPStream.h>
 
+#include <stdexcept>
+#include <string>
 #include <tuple>
 
 #include "gnn_agg.h"
@@ -63,6 +65,12 @@ std::tuple<torch::Tensor, torch::optional<torch::Tensor>> spmm_mi355x(
 }  // namespace
 
 PYBIND11_MODULE(computation_ops, m) {
+    // the library found at run time must be the one this module was compiled against: with another version of the
+    // header its entry points may take other arguments
+    if (gnnagg_abi_version() != GNNAGG_ABI_VERSION)
+        throw std::runtime_error("computation_ops was compiled against libgnnagg ABI version " +
+                                 std::to_string(GNNAGG_ABI_VERSION) + " but the library it loaded reports " +
+                                 std::to_string(gnnagg_abi_version()) + ": rebuild both (gnn_benchmark_amd/ext/build.sh)");
     m.doc() = "MI355X drop-in for the reference's computation_ops.spmm (libgnnagg.so underneath)";
     m.def("spmm", &spmm_mi355x);
 }

@@ -26,7 +26,11 @@ extern "C" {
 #define GNNAGG_ERR_HIP 2         /* a HIP runtime call failed */
 #define GNNAGG_ERR_UNSUPPORTED 3 /* sizes beyond what the kernels address (see each function) */
 
-#define GNNAGG_ABI_VERSION 1
+/* Raised whenever an exported prototype changes, an entry point goes away or the meaning of an argument changes
+ * (2: `src_rows` in the row gathers, `workspace_bytes` in the weight-gradient entry points, 12 values from
+ * gnnagg_plan_info; 3: the measurement probes left the library, gnnagg_plan_spmm_two_sources_f32 came).  Every binding compares it with
+ * gnnagg_abi_version() of the library it loaded before the first call. */
+#define GNNAGG_ABI_VERSION 3
 
 /* Version of this ABI (GNNAGG_ABI_VERSION of the built library).  No reference counterpart. */
 int gnnagg_abi_version(void);
@@ -128,6 +132,19 @@ int gnnagg_plan_spmm_f32(gnnagg_plan *plan, const float *value, const float *mat
  * writes the left one.  Results equal gnnagg_plan_spmm_f32 on contiguous copies bit for bit. */
 int gnnagg_plan_spmm_strided_f32(gnnagg_plan *plan, const float *value, const float *mat, int64_t mat_stride,
                                  float *out, int64_t out_stride, int64_t feat, int accumulate, void *stream);
+
+/* The same product with the dense operand in TWO arrays: column c of the matrix reads row c of mat for
+ * c < mat_rows and row c - mat_rows of mat2 above (plan->cols - mat_rows rows; strides in floats).  This is what
+ * lets the local aggregation and the aggregation of the received halo rows run as ONE launch, one FMA chain per
+ * output row: build the plan over [A_local | A_from] (every row: its local elements, then its halo elements with
+ * column + N_local -- the numbering the reference's raw-halo path gives halo nodes itself,
+ * data_manager/DataProcessor.py:29-60) and pass the layer input as mat and recv_buf as mat2.  Each output row is
+ * then written once instead of written by the local product and read and written again by the post-aggregation
+ * (model/layers/aggregator.py:67-70 then :102), with the same chain, hence the same bits.  Every row runs in the
+ * lane-group kernel (no block-per-row side launch).  Allocates nothing, no host synchronisation. */
+int gnnagg_plan_spmm_two_sources_f32(gnnagg_plan *plan, const float *value, const float *mat, int64_t mat_stride,
+                                     int64_t mat_rows, const float *mat2, int64_t mat2_stride, float *out,
+                                     int64_t out_stride, int64_t feat, int accumulate, void *stream);
 
 /* Host-side description of a plan, info[0..11] (host pointer):
  * rows, cols, nnz, rows handled by the block-per-row kernel (longer than the next
@@ -488,32 +505,6 @@ int gnnagg_dequantize_mixed_f32(const uint8_t *data, const int64_t *feat_range, 
  * allocate nothing, no host sync. */
 int gnnagg_f32_to_bf16(const float *x, uint16_t *y, int64_t count, void *stream);
 int gnnagg_bf16_to_f32(const uint16_t *x, float *y, int64_t count, void *stream);
-
-/* ---------------------------------------------------------------------------------
- * Memory-system probes: plain kernels with the access mixes of the aggregation path and nothing else, for
- * benchmarks that want the machine's own rate for a mix next to a product kernel's (a copy or a read stream is the
- * usual yardstick; row gathers mixed with row writes are what the boundary products do).  Nothing in the product
- * path calls them; no counterpart in the reference (its `#define PROFILE` timers, spmm.cpp:12, time the operator
- * only).  Allocate nothing, no host synchronisation.
- *   kind 0  read `count` floats of src as a stream (dst: 4 writable bytes, never written for finite data)
- *   kind 1  write `count` floats of dst as a stream
- *   kind 2  copy `count` floats from src to dst
- *   kind 3  `count` result rows, each the sum of `per_row` rows of src gathered through index[count * per_row]
- *           (int32 row numbers of src); the results are dropped: reads only
- *   kind 4  the same, every result row written to dst[count, row_floats]
- *   kind 5  the same, every result row added onto the row dst holds: one row read and one written per result
- * row_floats (kinds 3-5): 64, 128 or 256; src and dst 16-byte aligned; count a multiple of 4 for kinds 0-2.
- * ------------------------------------------------------------------------------- */
-int gnnagg_memory_probe(int kind, const float *src, const int32_t *index, float *dst, int64_t count,
-                        int64_t row_floats, int64_t per_row, void *stream);
-
-/* Issue probe.  One block of eight waves per compute unit: waves 0-3 (one per SIMD) issue `mfma_rounds` x 8
- * independent v_mfma_f32_32x32x16_bf16, waves 4-7 (one per SIMD) run `valu_rounds` x 8 rounds of the vector-ALU
- * sequence that cuts a pair of fp32 values into bf16 pieces (about 11 instructions a round).  Timing (mfma, 0),
- * (0, valu) and (mfma, valu) shows whether the two pipes of a SIMD overlap when different waves feed them; the
- * bf16 x 3 dense-layer kernels are designed around the answer.  No counterpart in the reference.  sink: 4 writable
- * bytes, never written.  Allocates nothing, no host synchronisation. */
-int gnnagg_issue_probe(int mfma_rounds, int valu_rounds, float *sink, void *stream);
 
 #ifdef __cplusplus
 }

@@ -22,6 +22,35 @@ def test_header_and_binding_agree():
     assert _declared() == sorted(_lib.EXPORTS)
 
 
+def _prototype_digest():
+    """sha256 over every exported prototype of the header, comments and white space taken out."""
+    import hashlib
+
+    with open(os.path.join(ROOT, "include", "gnn_agg.h")) as f:
+        text = f.read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    protos = re.findall(r"[A-Za-z_][A-Za-z0-9_ \*]*\bgnnagg_[a-z0-9_]+\s*\([^;{]*\)\s*;", text)
+    assert len(protos) == len(_declared())
+    canon = sorted(re.sub(r"\s+", " ", p).replace(" *", "*").replace("* ", "*").strip() for p in protos)
+    return hashlib.sha256("\n".join(canon).encode()).hexdigest()[:16]
+
+
+# GNNAGG_ABI_VERSION -> digest of the prototypes it stands for.  A changed, added or removed prototype changes the
+# digest: raise GNNAGG_ABI_VERSION (header) and ABI_VERSION (_lib.py) together and record the new pair here, so that a
+# library or extension module built from the old header is refused instead of being called with shifted arguments.
+ABI_DIGESTS = {3: "fb4f2a71dbecd71a"}
+
+
+def test_a_changed_prototype_needs_a_new_abi_version():
+    with open(os.path.join(ROOT, "include", "gnn_agg.h")) as f:
+        version = int(re.search(r"#define GNNAGG_ABI_VERSION (\d+)", f.read()).group(1))
+    assert version == _lib.ABI_VERSION
+    assert version in ABI_DIGESTS, "record the digest of the new ABI version in ABI_DIGESTS"
+    assert _prototype_digest() == ABI_DIGESTS[version], (
+        "an exported prototype changed: raise GNNAGG_ABI_VERSION / _lib.ABI_VERSION and record "
+        f"{{{version + 1}: '{_prototype_digest()}'}}")
+
+
 def test_library_exports_every_declared_symbol():
     if not os.path.exists(_lib.LIB_PATH):
         pytest.skip("libgnnagg.so not built yet (python -c 'import __graft_entry__ as g; g.build()')")
@@ -50,13 +79,9 @@ def test_argument_errors_without_gpu_work():
     assert L.gnnagg_check_index(None, 3, 5, 0, 10, None) == _lib.ERR_INVALID
     assert L.gnnagg_wgrad_f32(None, None, None, None, 0, 5, 8, 8, None) == _lib.ERR_INVALID   # null operands
     assert L.gnnagg_plan_create_ex(None, None, 1, 1, 0, None, None, None) == _lib.ERR_INVALID
-    assert L.gnnagg_memory_probe(9, None, None, None, 4, 128, 1, None) == _lib.ERR_INVALID
-    assert L.gnnagg_memory_probe(0, None, None, None, 0, 128, 1, None) == _lib.OK
-    assert L.gnnagg_issue_probe(-1, 0, None, None) == _lib.ERR_INVALID
     # a null partial-sums workspace is refused on the host, not dereferenced on the device (fake non-null operands)
     assert L.gnnagg_dropout_layernorm_relu_backward_f32(256, 128, 256, None, 1.0, 256, 256, 1e-5, 256, None, 4, 128, None) == _lib.ERR_INVALID
     assert b"partial" in L.gnnagg_last_error()
-    assert L.gnnagg_issue_probe(1, 1, None, None) == _lib.ERR_INVALID   # null sink
     # the producers that write the exchange format themselves: argument checks before any launch (fake operands)
     fake = 256
     assert L.gnnagg_spmm_csr_quantize_segments_f32(fake, fake, fake, fake, 128, fake, fake, fake, fake, 1, 8, 2, 128, 3,
