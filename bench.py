@@ -90,7 +90,7 @@ def c4_targets(c4):
              "local transposed": "local_T", "post-aggregation transposed": "post_T"}
     products = {}
     for op in c4["ops"]:
-        if not op.get("as_run_by_aggregator"):
+        if op.get("as_run_by_aggregator") is not True:
             continue
         name = next((v for k, v in short.items() if op["op"].startswith(k)), None)
         if name is not None:
@@ -837,7 +837,51 @@ def run_c4(args, graph, setup_s, gate=None):
         with torch.no_grad():
             o = Aggregator.apply(graph, x, 0, 32, True, True)
         parity_rows_of_pipeline(gate, graph, x, o, graph.comm_buf.recv_buf, 4000, args.seed + 11)
-    del o
+    # the same with the local and the received elements of every output row in ONE launch each way
+    # (graph.one_launch: [A_local | A_from] over (x ; recv_buf), [A_local^T | A_to^T] over (g ; send_buf))
+    from gnn_benchmark_amd.sparse_tensor import side_by_side
+
+    graph.one_launch = True
+    for _ in range(2):
+        o1 = Aggregator.apply(graph, xr, 0, 32, True, True)
+        o1.backward(g)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        o1 = Aggregator.apply(graph, xr, 0, 32, True, True)
+    torch.cuda.synchronize()
+    fwd1_ms = (time.perf_counter() - t0) * 1e3 / steps
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        o1 = Aggregator.apply(graph, xr, 0, 32, True, True)
+        o1.backward(g)
+    torch.cuda.synchronize()
+    both1_ms = (time.perf_counter() - t0) * 1e3 / steps
+    graph.one_launch = False
+    # the one-launch result against the three-launch one (`o`), every row: the same chains, so the same bits
+    one_launch_same_bits = bool(torch.equal(o1.detach(), o.detach()))
+    if not one_launch_same_bits and gate is not None and gate.enabled:
+        print("bench.py: the one-launch aggregation differs from the three-launch one; no number is reported",
+              file=sys.stderr, flush=True)
+        sys.exit(4)
+    del o, o1
+    for key, left, right, transposed, a1, a2, nm in (
+            ("local+post", graph.local_adj_t, graph.adj_t_pre_post_aggr_from, False, x, graph.comm_buf.recv_buf,
+             "local + post-aggregation in one launch [A_local | A_from]@(X ; recv_buf) -> out (overwriting)"),
+            ("local_T+pre_T", graph.local_adj_t, graph.adj_t_pre_post_aggr_to, True, g, graph.comm_buf.send_buf,
+             "local + pre-aggregation transposed in one launch [A_local^T | A_to^T]@(G ; send_buf) -> dX (overwriting)")):
+        m = side_by_side(left, right, transposed)
+        plan = m.get_plan()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for i in range(steps + 2):
+            if i == 2:
+                e0.record()
+            plan.spmm_two_sources(m.csr()[2], a1, a2, out, accumulate=False)
+        e1.record()
+        e1.synchronize()
+        ops.append(op_report(nm, m.nnz(), m.sparse_size(0), m.sparse_size(1), feat, e0.elapsed_time(e1) / steps,
+                             plan.info()["empty_rows"], False))
+        ops[-1]["as_run_by_aggregator"] = "one_launch"
     graph.comm_buf.resize_buffer(graph.comm_splits, feat, 32)  # (the buffer's own tensors again, not delivered rows)
     codec = run_c4_codec(graph, feat, steps, gen, cpu=not args.no_cpu_baseline)
     # the same autograd.Function with the boundary rows travelling as int2 (seeded packed rows)
@@ -970,6 +1014,9 @@ def run_c4(args, graph, setup_s, gate=None):
             "from_nnz": graph.adj_t_pre_post_aggr_from.nnz(), "to_nnz": graph.adj_t_pre_post_aggr_to.nnz(),
             "ops": ops, "aggregator_forward_ms": round(fwd_ms, 3),
             "aggregator_forward_backward_ms": round(both_ms, 3),
+            "aggregator_forward_ms_one_launch": round(fwd1_ms, 3),
+            "aggregator_forward_backward_ms_one_launch": round(both1_ms, 3),
+            "one_launch_same_bits": one_launch_same_bits,
             "aggregator_forward_backward_ms_bf16_exchange": round(bf16_both_ms, 3),
             "aggregator_forward_backward_ms_bf16_exchange_separate_copies": round(bf16_unfused_ms, 3),
             "aggregator_forward_backward_ms_int2_exchange": round(int2_fused_ms, 3),

@@ -41,6 +41,14 @@ What differs from the reference, on purpose:
   because an FMA chain started from a stored 0 equals one started from a register 0.
 * The backward ``index_add_`` (:197-199) runs as a deterministic SpMM with the
   selection matrix of ``idx_nodes_send_to_others``.
+* ``graph.one_launch = True`` (off by default) runs the local product and the product with
+  the received rows as ONE launch over ``[A_local | A_from]`` and the two dense operands
+  (``sparse_tensor.side_by_side``): every output row is one FMA chain -- local elements, then
+  received ones, the order of aggregator.py:70 then :102 -- written once, instead of written by
+  the local product and read and written again behind the exchange.  Same bits, fewer bytes;
+  the price is that the local product no longer runs while the exchange is in flight, so it
+  pays where the exchange is short next to the local product.  fp32 boundary rows and dense
+  features only; every other case runs the separate launches.
 
 ``AggregatorPacked`` is the same pipeline for local features handed over packed
 (``packed.py``: non-zero values at the front of each row plus a bitmap header); only the
@@ -50,7 +58,7 @@ two forward products that read the features differ.
 import torch
 
 from . import _lib, computation_ops, packed
-from .sparse_tensor import SparseTensor, _rows_are_dense
+from .sparse_tensor import SparseTensor, _rows_are_dense, side_by_side
 from .spmm_kernel import SPMM_backward, SPMM_backward_quantized, SPMM_forward, SPMM_forward_quantized
 
 
@@ -162,6 +170,16 @@ def _product_into_packed_rows(graph, plan, csr, dense: torch.Tensor, num_bits: i
 def _transposed_csr(m: SparseTensor):
     s = m.storage
     return s.colptr(), s.row_T(), s.value_T()
+
+
+def _transposed_matrix(m: SparseTensor) -> SparseTensor:
+    """``m^T`` as a matrix of its own over the transposed arrays of ``m`` (kept on ``m``)."""
+    hit = m.__dict__.get("_transposed_matrix")
+    if hit is None:
+        colptr, row_t, value_t = _transposed_csr(m)
+        hit = m.__dict__["_transposed_matrix"] = SparseTensor(
+            rowptr=colptr, col=row_t, value=value_t, sparse_sizes=(m.sparse_size(1), m.sparse_size(0)), is_sorted=True)
+    return hit
 
 
 def _quantize_and_exchange(graph, num_bits: int, tag: str, direction: str, already_packed: bool = False):
@@ -312,6 +330,18 @@ def _forward(ctx, graph, feats, layer, num_bits: int, is_pre_delay: bool, is_tra
         accumulate = False
     else:
         _check_result(out, graph.local_adj_t.sparse_size(0), feat_len, feats.device)
+    remote_adj = None
+    if exchange is not None:
+        remote_adj = graph.adj_t_pre_post_aggr_from if is_pre_delay else graph.remote_adj_t
+    one_launch = (getattr(graph, "one_launch", False) is True and remote_adj is not None and not quantized and not half
+                  and isinstance(feats, _DenseFeatures) and feats.feat.dtype == torch.float32
+                  and graph.comm_buf.recv_buf.size(0) != 0)
+    if one_launch:  # local elements, then received ones: one chain per output row, one launch
+        if comm_handle is not None:
+            comm_handle.wait()
+        both = side_by_side(graph.local_adj_t, remote_adj)
+        both.get_plan().spmm_two_sources(both.csr()[2], feats.feat, graph.comm_buf.recv_buf, out, accumulate)
+        return out
     feats.product(graph.local_adj_t, out, accumulate)
 
     if comm_handle is not None:
@@ -326,7 +356,7 @@ def _forward(ctx, graph, feats, layer, num_bits: int, is_pre_delay: bool, is_tra
     # (fused: the received bf16 rows are gathered as they are; recv_buf is not written)
     remote_nodes_feat = graph.comm_buf.recv_buf_fp16 if half_fused else graph.comm_buf.recv_buf
     if exchange is not None and remote_nodes_feat.size(0) != 0:
-        adj = graph.adj_t_pre_post_aggr_from if is_pre_delay else graph.remote_adj_t  # post-aggregation / raw halo
+        adj = remote_adj  # post-aggregation / raw halo
         if fused:
             qbuf = graph.comm_buf_for_quantization
             SPMM_forward_quantized(adj, qbuf.quantized_recv_data_buf, qbuf.quantized_recv_params_buf_fp32,
@@ -497,6 +527,19 @@ def _backward(ctx, local_out_grad, out=None, accumulate: bool = False):
     else:
         _check_result(out, graph.local_adj_t.sparse_size(-1), feat_len, local_out_grad.device)
         local_nodes_grad = out
+    one_launch = (getattr(graph, "one_launch", False) is True and exchange is not None and support is None
+                  and not quantized and not half and local_out_grad.dtype == torch.float32
+                  and graph.comm_buf.send_buf.size(0) != 0)
+    if one_launch:  # [A_local^T | A_to^T] over the gradient and the received gradient rows, one chain per row
+        if comm_handle is not None:
+            comm_handle.wait()
+        if is_pre_delay:
+            both = side_by_side(graph.local_adj_t, graph.adj_t_pre_post_aggr_to, transposed=True)
+        else:  # local^T next to the selection matrix of the boundary row list (itself untransposed)
+            both = side_by_side(_transposed_matrix(graph.local_adj_t), graph.send_scatter_adj_t())
+        both.get_plan().spmm_two_sources(both.csr()[2], local_out_grad, graph.comm_buf.send_buf, local_nodes_grad,
+                                         accumulate)
+        return local_nodes_grad
     if support is not None:
         SPMM_forward(support.local_T, local_out_grad, local_nodes_grad, accumulate=accumulate)
     else:

@@ -98,6 +98,29 @@ class SpmmPlan:
                     feat, 1 if accumulate else 0, _lib.current_stream(self.device)))
         return out
 
+    def spmm_two_sources(self, value: torch.Tensor, mat: torch.Tensor, mat2: torch.Tensor, out: torch.Tensor,
+                         accumulate: bool = True) -> torch.Tensor:
+        """``out (+)= A @ [mat ; mat2]`` with the dense operand in two arrays: column ``c`` reads row ``c`` of ``mat``
+        for ``c < mat.size(0)`` and row ``c - mat.size(0)`` of ``mat2`` above.  All float32, rows contiguous (column
+        blocks of wider tensors are read and written in place)."""
+        tensors = (value, mat, mat2, out)
+        if not all(t.is_cuda for t in tensors):
+            raise RuntimeError("value, mat, mat2 and out must be GPU (HIP) tensors; there is no CPU path")
+        if any(t.dtype != torch.float32 for t in tensors):
+            raise RuntimeError("Input mismatch: value/mat/mat2/out must be float32")
+        if not all(_rows_are_dense(t) for t in (mat, mat2, out)):
+            raise RuntimeError("Input mismatch: mat/mat2/out must be 2-D with contiguous rows")
+        feat = out.size(1)
+        if (value.numel() != self.nnz or mat.size(0) + mat2.size(0) < self.cols or mat.size(0) > self.cols
+                or out.size(0) < self.rows or mat.size(1) != feat or mat2.size(1) != feat):
+            raise RuntimeError("Input mismatch: operand shapes do not match the planned matrix")
+        with torch.cuda.device(self.device):
+            _lib.check(_lib.lib().gnnagg_plan_spmm_two_sources_f32(
+                self._handle, _lib.ptr(value.contiguous()), _lib.ptr(mat), _row_stride(mat), mat.size(0), _lib.ptr(mat2),
+                _row_stride(mat2), _lib.ptr(out), _row_stride(out), feat, 1 if accumulate else 0,
+                _lib.current_stream(self.device)))
+        return out
+
     def _spmm_bf16(self, value, mat, out, accumulate):
         """The product with bf16 rows on either side (the staging buffers of a 16-bit exchange): a bf16 ``mat`` is
         widened in the gather, a bf16 ``out`` receives the fp32 sums rounded to nearest even -- the same bits as the
@@ -333,3 +356,35 @@ class SparseTensor:
             s = self.storage
             self._plan_T = SpmmPlan(s.colptr(), s.row_T(), self.sparse_size(1), self.sparse_size(0))
         return self._plan_T
+
+
+def side_by_side(left: SparseTensor, right: SparseTensor, transposed: bool = False) -> SparseTensor:
+    """``[left | right]`` (``transposed``: ``[left^T | right^T]``) as one CSR: every row holds its elements of
+    ``left`` in their order, then its elements of ``right`` in theirs with the column moved up by the columns of
+    ``left``.  A product with it over the two dense operands stacked is, row by row, the FMA chain of the product
+    with ``left`` continued by the one with ``right``.  Built once per pair and kept on ``left``."""
+    cache = left.__dict__.setdefault("_side_by_side", {})
+    key = (id(right), bool(transposed))
+    hit = cache.get(key)
+    if hit is None:
+        parts = []
+        for m in (left, right):
+            row, col, value = m.coo()
+            if value is None:
+                raise RuntimeError("Input mismatch: the sparse matrix has no values")
+            parts.append((col, row, value) if transposed else (row, col, value))
+        rows = left.sparse_size(1 if transposed else 0)
+        if right.sparse_size(1 if transposed else 0) != rows:
+            raise RuntimeError("Input mismatch: the two matrices differ in their number of rows")
+        left_cols = left.sparse_size(0 if transposed else 1)
+        right_cols = right.sparse_size(0 if transposed else 1)
+        # (row, column) order with repeated pairs in input order: inside a row all of left's elements come before
+        # right's (their columns are smaller), each part in the order of its own (transposed) CSR
+        merged = SparseTensor(row=torch.cat([parts[0][0], parts[1][0]]),
+                              col=torch.cat([parts[0][1], parts[1][1] + left_cols]),
+                              value=torch.cat([parts[0][2], parts[1][2]]), sparse_sizes=(rows, left_cols + right_cols))
+        merged.first_source_rows = left_cols
+        if len(cache) >= 4:
+            cache.clear()
+        hit = cache[key] = (right, merged)   # holding `right` keeps its id its own
+    return hit[1]

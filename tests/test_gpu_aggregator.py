@@ -70,11 +70,16 @@ def _build_pre_graphs(w: World, feat, bits=32):
     return graphs
 
 
+@pytest.mark.parametrize("one_launch", [False, True])
 @pytest.mark.parametrize("seed,sizes", [(0, (300, 450, 250)), (1, (600, 1, 400, 330)), (2, (500, 0, 500))])
-def test_pre_post_world_matches_oracle_and_global_product(seed, sizes):
+def test_pre_post_world_matches_oracle_and_global_product(seed, sizes, one_launch):
+    """`one_launch`: local and received elements of every output row in one launch (`graph.one_launch`): same chains,
+    so the same bits as the oracle pipeline."""
     w = World(seed, sizes, mean_deg=8.0)
     W, F = w.world, 48
     graphs = _build_pre_graphs(w, F)
+    for gr in graphs:
+        gr.one_launch = one_launch
     oracle_ranks = build_pre_world(w)
     for r in range(W):
         _same_matrix(graphs[r].local_adj_t, oracle_ranks[r]["local"])
@@ -144,11 +149,14 @@ def _build_raw_graphs(w, F, bits=32):
     return graphs
 
 
+@pytest.mark.parametrize("one_launch", [False, True])
 @pytest.mark.parametrize("seed,sizes", [(4, (300, 450, 250)), (5, (600, 1, 400, 330))])
-def test_raw_halo_world_matches_oracle_and_global_product(seed, sizes):
+def test_raw_halo_world_matches_oracle_and_global_product(seed, sizes, one_launch):
     w = World(seed, sizes, mean_deg=8.0)
     W, F = w.world, 40
     graphs = _build_raw_graphs(w, F)
+    for gr in graphs:
+        gr.one_launch = one_launch
     rng = np.random.default_rng(seed)
     x = rng.standard_normal((w.n, F)).astype(np.float32)
     g = rng.standard_normal((w.n, F)).astype(np.float32)
@@ -182,6 +190,7 @@ def test_raw_halo_world_matches_oracle_and_global_product(seed, sizes):
         # product adds them per destination row in the same order: same chains
         o_dx = oagg.backward_out_raw(local, gr.idx_nodes_send_to_others.cpu().numpy(), np.ascontiguousarray(g[sl[r]]), incoming[r])
         assert_close(xr.grad, o_dx, "raw halo gradient vs oracle")
+        assert np.array_equal(xr.grad.cpu().numpy(), o_dx)
 
 
 def test_single_rank_world_and_autograd_contract():
