@@ -1276,7 +1276,8 @@ def run_c5(args, graph):
     # then with the narrowing last layer multiplying before it aggregates (A (x W) instead of (A x) W)
     folded = None
     # (layers with dense activations run as one libgnnagg kernel each way; "separate_kernels" is the
-    # same model with the BLAS product and the elementwise passes apart)
+    # same model with the product -- the same kernel, bare -- and the elementwise passes apart).
+    # `library_products_per_step`: dense products of one step that fell through to the BLAS library (0: none)
     for gemm, packed_activations, linear_first, fused in (
             ("fp32", False, False, True), ("fp32", False, False, False), ("bf16", False, False, True),
             ("fp32", True, False, True), ("bf16", True, False, True), ("fp32", False, True, True),
@@ -1306,6 +1307,7 @@ def run_c5(args, graph):
         opt = torch.optim.Adam(model.parameters(), lr=0.01)
         losses = [float(gcn.train_step(model, opt, g, x, labels, train_idx, True, masks, restrict)) for _ in range(2)]
         torch.cuda.synchronize()
+        fell_through = gcn.LIBRARY_PRODUCTS["count"]
         t0 = time.perf_counter()
         for _ in range(steps):
             loss = gcn.train_step(model, opt, g, x, labels, train_idx, True, masks, restrict)
@@ -1314,9 +1316,26 @@ def run_c5(args, graph):
                + ("_linear_first_when_narrowing" if linear_first else "") + ("" if fused else "_separate_kernels")
                + folded_tag + ("" if restrict else "_all_nodes_through_last_layer"))
         out[f"train_step_ms_{tag}"] = round((time.perf_counter() - t0) * 1e3 / steps, 2)
+        out["library_products_per_step"] = max(out.get("library_products_per_step", 0),
+                                               (gcn.LIBRARY_PRODUCTS["count"] - fell_through) // steps)
         out[f"loss_{tag}"] = [round(v, 5) for v in losses + [float(loss)]]
         del model, opt
     del folded
+    # the default step with the local and the received elements of every output row in one launch (graph.one_launch)
+    graph.one_launch = True
+    torch.manual_seed(args.seed)
+    model = gcn.GCN(dims).to(dev)
+    opt = torch.optim.Adam(model.parameters(), lr=0.01)
+    losses = [float(gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks)) for _ in range(2)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        loss = gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks)
+    torch.cuda.synchronize()
+    out["train_step_ms_fp32_gemm_one_launch_aggregation"] = round((time.perf_counter() - t0) * 1e3 / steps, 2)
+    out["loss_fp32_gemm_one_launch_aggregation"] = [round(v, 5) for v in losses + [float(loss)]]
+    graph.one_launch = False
+    del model, opt
     from gnn_benchmark_amd import synthetic
     from gnn_benchmark_amd.data_manager import CommBuffer, CommBufferForQuantization, CommSplits
 
@@ -1394,14 +1413,21 @@ def run_c5_sage(args, graph):
     masks = sage.make_dropout_masks(n, hidden, len(dims) - 1, 0.5, args.seed + 8, dev)
     out = {"layers": "DistSAGE %d->%d->%d->%d, LayerNorm, dropout 0.5" % tuple(dims), "steps": steps}
 
+    from gnn_benchmark_amd import gcn
+
     def timed(step):
         losses = [float(step()) for _ in range(2)]
         torch.cuda.synchronize()
+        fell_through = gcn.LIBRARY_PRODUCTS["count"]
         t0 = time.perf_counter()
         for _ in range(steps):
             loss = step()
         torch.cuda.synchronize()
-        return round((time.perf_counter() - t0) * 1e3 / steps, 2), [round(v, 5) for v in losses + [float(loss)]]
+        ms = round((time.perf_counter() - t0) * 1e3 / steps, 2)
+        # dense products of one step that fell through to the BLAS library (0: none), the most over the forms
+        out["library_products_per_step"] = max(out.get("library_products_per_step", 0),
+                                               (gcn.LIBRARY_PRODUCTS["count"] - fell_through) // steps)
+        return ms, [round(v, 5) for v in losses + [float(loss)]]
 
     staged = sage.stage_input(x)
     folded = None
@@ -1409,16 +1435,19 @@ def run_c5_sage(args, graph):
             ("", False, False, True, "fp32"), ("_folded_degrees", True, False, True, "fp32"),
             ("_folded_degrees_linear_first_when_narrowing", True, True, True, "fp32"),
             ("_folded_degrees_bf16x3_gemm", True, False, True, "bf16x3"),
-            ("_folded_degrees_all_nodes_through_last_layer", True, False, False, "fp32")):
+            ("_folded_degrees_all_nodes_through_last_layer", True, False, False, "fp32"),
+            ("_folded_degrees_one_launch_aggregation", True, False, True, "fp32")):
         if fold and folded is None:
             folded = sage.fold_in_degrees(graph)
         g = folded if fold else graph
+        g.one_launch = tag.endswith("one_launch_aggregation")
         torch.manual_seed(args.seed)
         model = sage.DistSAGE(dims[0], hidden, dims[-1], num_layers=len(dims) - 1, dropout=0.5, is_pre_delay=True,
                               linear_first_when_narrowing=linear_first, gemm=gemm).to(dev)
         opt = torch.optim.Adam(model.parameters(), lr=0.01)
         ms, losses = timed(lambda: sage.train_step(model, opt, g, staged, labels, train_idx, masks, restrict))
         out["train_step_ms" + tag], out["loss" + tag] = ms, losses
+        g.one_launch = False
         del model, opt, g
         torch.cuda.empty_cache()
     # the same step (degrees folded) with the boundary rows travelling as bf16 / as int2 -- the widths the reference's
@@ -1555,14 +1584,17 @@ def main():
             c5 = sink.put("c5", run_c5(args, graph))
             targets["c5_gcn_train_step_ms"] = {k[len("train_step_ms_"):]: c5[k] for k in (
                 "train_step_ms_fp32_gemm", "train_step_ms_bf16_gemm", "train_step_ms_bf16x3_gemm",
+                "train_step_ms_fp32_gemm_one_launch_aggregation",
                 "train_step_ms_fp32_gemm_all_nodes_through_last_layer", "train_step_ms_fp32_gemm_int2_exchange")
                 if k in c5}
+            targets["c5_gcn_train_step_ms"]["library_products"] = c5.get("library_products_per_step")
             torch.cuda.empty_cache()
         if "c5" in args.extras or "c5sage" in args.extras:
             c5s = sink.put("c5_sage", run_c5_sage(args, graph))
             targets["c5_sage_train_step_ms"] = {
                 (k[len("train_step_ms_"):] if len(k) > len("train_step_ms") else "default"): c5s[k] for k in (
-                    "train_step_ms", "train_step_ms_folded_degrees", "train_step_ms_folded_degrees_int2_exchange",
+                    "train_step_ms", "train_step_ms_folded_degrees", "train_step_ms_folded_degrees_one_launch_aggregation",
+                    "train_step_ms_folded_degrees_int2_exchange",
                     "train_step_ms_torch_ops_around_aggregator") if k in c5s}
     line["parity"] = gate.report()
     line["targets"] = targets

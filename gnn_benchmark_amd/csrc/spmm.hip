@@ -83,10 +83,17 @@ int64_t lay_out_blocks(SpmmArgs &args, int gpb, Regions r) {
     const int64_t head_blocks = (args.head_tasks + gpb - 1) / gpb;
     const int64_t mid_blocks = (args.tail_first - args.head_tasks + args.tasks_per_block - 1) / args.tasks_per_block;
     const int64_t tail_blocks = (tail + args.tail_tasks_per_block - 1) / args.tail_tasks_per_block;
-    if (head_blocks + mid_blocks + tail_blocks > 0x7fffffffll) return -1;
+    // rows in their natural order: the blocks that look for the long rows come first (args.scan_rows rows a group)
+    int64_t scan_blocks = 0;
+    if (args.long_len > 0 && args.scan_rows > 0)
+        scan_blocks = (args.ntasks + (int64_t)args.scan_rows * gpb - 1) / ((int64_t)args.scan_rows * gpb);
+    else
+        args.long_len = 0;
+    if (head_blocks + mid_blocks + tail_blocks + scan_blocks > 0x7fffffffll) return -1;
     args.head_blocks = (int)head_blocks;
     args.mid_blocks = (int)mid_blocks;
-    return head_blocks + mid_blocks + tail_blocks;
+    args.scan_blocks = (int)scan_blocks;
+    return head_blocks + mid_blocks + tail_blocks + scan_blocks;
 }
 
 template <int VEC, int LPR, int NCH, typename IdxT, int MODE, int SRC = kSrcDense>
@@ -321,6 +328,14 @@ extern "C" int gnnagg_abi_version(void) { return GNNAGG_ABI_VERSION; }
 
 extern "C" const char *gnnagg_last_error(void) { return last_error_slot().c_str(); }
 
+// the plan-less operator's own handling of long rows (see gnnagg_spmm_csr_f32)
+constexpr int64_t kScanMinRows = 16384;   // smaller matrices: one region, as they come
+// (measured on MI355X, 2.45 M rows / 122 M elements at F = 100 and 7 M rows / 102 M elements at F = 128, ms:
+//  no scanning 9.44 / 9.91; (length 256, 512 rows a group) 9.91 / 8.65; (256, 128) 7.93 / 8.68; (128, 128) 7.92 / 8.55;
+//  (64, 64) 8.01 / 8.43; (32, 64) 9.15 / 8.46 -- the plan's own launch takes 7.9 / 7.8)
+constexpr int kScanLongLen = 64;          // rows above this go to the scanning blocks
+constexpr int kScanRowsPerGroup = 64;     // rows of rowptr a scanning lane group walks
+
 static int check_feat(int64_t feat) {
     if (feat <= 0 || feat > (1 << 20))
         return fail(GNNAGG_ERR_UNSUPPORTED, "feature width %lld outside [1, 2^20]", (long long)feat);
@@ -352,6 +367,13 @@ extern "C" int gnnagg_spmm_csr_f32(const int64_t *rowptr, const int64_t *col, co
         a.feat = (int)feat;
         a.f_base = (int)f_base;
         a.accumulate = 1;
+        // No plan orders the rows by length here, so on a matrix of some size the launch's first blocks walk rowptr
+        // and run the rows above the plan's own long-row threshold themselves: the longest chains start at once,
+        // spread over the device, instead of wherever their row number puts them.  Allocates nothing.
+        if (sparse_rows >= kScanMinRows) {
+            a.long_len = kScanLongLen;
+            a.scan_rows = kScanRowsPerGroup;
+        }
         GNNAGG_HIP((dispatch_tasks<int64_t, kRowsNatural>(s, a, Regions{4, 4, 0}, st)));
         f_base += s.width();
     }

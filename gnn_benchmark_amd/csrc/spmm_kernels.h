@@ -121,6 +121,18 @@ __device__ __forceinline__ int64_t group_bcast_idx(int32_t v, int src) {
     return (int64_t)group_bcast<LPR>(v, src);
 }
 
+// Which lanes of the group hold `p` (bit i: the group's lane i); wave-uniform for a whole-wave group.
+template <int LPR>
+__device__ __forceinline__ uint64_t group_ballot(bool p) {
+    const uint64_t b = __builtin_amdgcn_ballot_w64(p);
+    if constexpr (LPR == 64) {
+        return b;
+    } else {
+        const int first = (int)__lane_id() & ~(LPR - 1);
+        return (b >> first) & ((uint64_t(1) << LPR) - 1);
+    }
+}
+
 __device__ __forceinline__ int64_t uniform_i64(int64_t v) {
     const int lo = __builtin_amdgcn_readfirstlane((int)(uint32_t)(v & 0xffffffffll));
     const int hi = __builtin_amdgcn_readfirstlane((int)(v >> 32));
@@ -174,6 +186,12 @@ struct SpmmArgs {
     int64_t tail_first;       // first task of the tail region (== ntasks: none)
     int mid_blocks;           // blocks of the middle region
     int tail_tasks_per_block;
+    // kRowsNatural only (no plan to order the rows by length): with long_len > 0 the first scan_blocks blocks walk
+    // rowptr, scan_rows rows per lane group, and run the rows of more than long_len elements they meet -- the longest
+    // chains start with the launch, spread over the whole device; the blocks behind them leave those rows out.
+    int long_len;
+    int scan_blocks;
+    int scan_rows;
 };
 
 enum SourceKind : int {
@@ -393,33 +411,53 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
         foff[k] = fok[k] ? f : a.f_base;
     }
 
+    // Rows without a plan: a scanner block's groups walk their stretch of rowptr for the long rows, LPR rows at a
+    // time; the other blocks take the remaining rows in their natural order.
+    bool scanner = false;
+    int64_t scan_next = 0, scan_end = 0;
+    int bid = (int)blockIdx.x;
+    if constexpr (MODE == kRowsNatural) {
+        scanner = bid < a.scan_blocks;
+        if (scanner) {
+            scan_next = ((int64_t)bid * GPB + group) * (int64_t)a.scan_rows;
+            scan_end = scan_next + a.scan_rows;
+            if (scan_end > a.ntasks) scan_end = a.ntasks;
+            if (scan_next >= scan_end) return;
+        }
+        bid -= a.scan_blocks;
+    }
+
     // Head region: one task per lane group, so that no group queues several of the
     // longest rows behind each other.  Blocks are dispatched in index order, hence the
     // longest rows start first and the short ones fill in behind them.
-    int64_t t0, t1;
-    if ((int)blockIdx.x < a.head_blocks) {
-        t0 = (int64_t)blockIdx.x * GPB;
-        t1 = t0 + GPB;
-        if (t1 > a.head_tasks) t1 = a.head_tasks;
-    } else if ((int)blockIdx.x < a.head_blocks + a.mid_blocks) {
-        t0 = a.head_tasks + (int64_t)((int)blockIdx.x - a.head_blocks) * a.tasks_per_block;
-        t1 = t0 + a.tasks_per_block;
-        if (t1 > a.tail_first) t1 = a.tail_first;
-    } else {
-        t0 = a.tail_first + (int64_t)((int)blockIdx.x - a.head_blocks - a.mid_blocks) * a.tail_tasks_per_block;
-        t1 = t0 + a.tail_tasks_per_block;
-        if (t1 > a.ntasks) t1 = a.ntasks;
+    int64_t t0 = 0, t1 = 0;
+    if (!scanner) {
+        if (bid < a.head_blocks) {
+            t0 = (int64_t)bid * GPB;
+            t1 = t0 + GPB;
+            if (t1 > a.head_tasks) t1 = a.head_tasks;
+        } else if (bid < a.head_blocks + a.mid_blocks) {
+            t0 = a.head_tasks + (int64_t)(bid - a.head_blocks) * a.tasks_per_block;
+            t1 = t0 + a.tasks_per_block;
+            if (t1 > a.tail_first) t1 = a.tail_first;
+        } else {
+            t0 = a.tail_first + (int64_t)(bid - a.head_blocks - a.mid_blocks) * a.tail_tasks_per_block;
+            t1 = t0 + a.tail_tasks_per_block;
+            if (t1 > a.ntasks) t1 = a.ntasks;
+        }
     }
     // this group's tasks: t0 + group + i * GPB, i < ntask  (ntask <= kMaxRowsPerGroup <= LPR)
     const int64_t tfirst = t0 + group;
-    if (tfirst >= t1) return;
-    int ntask = (int)((t1 - tfirst + GPB - 1) / GPB);
+    if (!scanner && tfirst >= t1) return;
+    int ntask = scanner ? 0 : (int)((t1 - tfirst + GPB - 1) / GPB);
     if constexpr (LPR == 64) ntask = __builtin_amdgcn_readfirstlane(ntask);
 
     // One coalesced fetch brings every descriptor of the group: lane i holds task i.
     int d_row = 0, d_len = 0;
     int64_t d_start = 0;
-    if (lig < ntask) {
+    // kRowsNatural: the group's lanes whose row is still to be done (a planned launch walks lanes 0 .. ntask-1)
+    uint64_t todo = 0;
+    if (!scanner && lig < ntask) {
         const int64_t t = tfirst + (int64_t)lig * GPB;
         if constexpr (MODE == kRowsPlanned) {
             const RowTask d = a.task[t];
@@ -432,87 +470,133 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
             d_len = (int)(a.rowptr[t + 1] - d_start);
         }
     }
-
-    // State of the row being accumulated and of the chunk of <= LPR (col, val) pairs held
-    // across the group's lanes.  The NEXT chunk -- of the same row, or the first chunk of
-    // the group's next row -- is always requested before the current chunk's gathers, so
-    // that the index stream never sits on the critical path.
-    int i = 0;
-    int row = group_bcast<LPR>(d_row, 0);
-    int64_t base = group_bcast_idx<LPR>(d_start, 0);
-    int64_t end = base + group_bcast<LPR>(d_len, 0);
-    IdxT c_l = 0;
-    float v_l = 0.0f;
-    if (base + lig < end) {
-        c_l = __builtin_nontemporal_load(col + base + lig);
-        v_l = __builtin_nontemporal_load(val + base + lig);
+    if constexpr (MODE == kRowsNatural) {
+        if (!scanner) {
+            // rows without elements keep their value when accumulating: not visited; long rows belong to the scanners
+            const bool mine = lig < ntask && (d_len > 0 || !a.accumulate) && !(a.long_len > 0 && d_len > a.long_len);
+            todo = group_ballot<LPR>(mine);
+            if (todo == 0) return;
+        }
     }
+
     const bool from_dst = a.accumulate != 0;
     const int ldd = a.ldd ? a.ldd : F;
-    float *dst = a.dst + (size_t)row * (size_t)ldd;
-    V acc[NCH];
+
+    for (;;) {  // one pass, except in a scanner block: one pass per stretch of LPR rows that holds long rows
+        if constexpr (MODE == kRowsNatural) {
+            if (scanner) {
+                todo = 0;
+                while (todo == 0 && scan_next < scan_end) {
+                    const int64_t r = scan_next + lig;
+                    d_len = 0;
+                    if (r < scan_end) {
+                        d_row = (int)r;
+                        d_start = a.rowptr[r];
+                        d_len = (int)(a.rowptr[r + 1] - d_start);
+                    }
+                    todo = group_ballot<LPR>(d_len > a.long_len);
+                    scan_next += LPR;
+                }
+                if (todo == 0) return;
+            }
+        }
+
+        // State of the row being accumulated and of the chunk of <= LPR (col, val) pairs held
+        // across the group's lanes.  The NEXT chunk -- of the same row, or the first chunk of
+        // the group's next row -- is always requested before the current chunk's gathers, so
+        // that the index stream never sits on the critical path.
+        int i = 0;
+        if constexpr (MODE == kRowsNatural) {
+            i = __builtin_ctzll(todo);
+            todo &= todo - 1;
+        }
+        int row = group_bcast<LPR>(d_row, i);
+        int64_t base = group_bcast_idx<LPR>(d_start, i);
+        int64_t end = base + group_bcast<LPR>(d_len, i);
+        IdxT c_l = 0;
+        float v_l = 0.0f;
+        if (base + lig < end) {
+            c_l = __builtin_nontemporal_load(col + base + lig);
+            v_l = __builtin_nontemporal_load(val + base + lig);
+        }
+        float *dst = a.dst + (size_t)row * (size_t)ldd;
+        V acc[NCH];
 #pragma unroll
-    for (int k = 0; k < NCH; ++k) {
-        acc[k] = V::zero();
-        if (from_dst && fok[k]) acc[k] = V::load_stream(dst + foff[k]);
-    }
-
-    while (true) {
-        const int64_t left = end - base;
-        const int cnt = left < LPR ? (int)left : LPR;
-
-        // where the next chunk comes from
-        int ni = i;
-        int nrow = row;
-        int64_t nbase = base + LPR, nend = end;
-        bool row_done = nbase >= end;
-        bool more = true;
-        if (row_done) {
-            ni = i + 1;
-            more = ni < ntask;
-            if (more) {
-                nrow = group_bcast<LPR>(d_row, ni);
-                nbase = group_bcast_idx<LPR>(d_start, ni);
-                nend = nbase + group_bcast<LPR>(d_len, ni);
-            }
-        }
-        IdxT nc = 0;
-        float nv = 0.0f;
-        if (more && nbase + lig < nend) {
-            nc = __builtin_nontemporal_load(col + nbase + lig);
-            nv = __builtin_nontemporal_load(val + nbase + lig);
+        for (int k = 0; k < NCH; ++k) {
+            acc[k] = V::zero();
+            if (from_dst && fok[k]) acc[k] = V::load_stream(dst + foff[k]);
         }
 
-        // full blocks of U gathers, then ONE more round for what is left (the smallest power of two of gathers
-        // that covers it, the surplus ones masked): a chunk of cnt elements costs ceil(cnt / U) dependent round trips
-        int j = 0;
-        for (; j + U <= cnt; j += U) gather_fma<U, VEC, LPR, NCH, SRC>(acc, c_l, v_l, j, a, foff);
-        const int rem = cnt - j;
-        if (rem > 0) {
-            if constexpr (U > 4) {
-                if (rem > 4) gather_fma<8, VEC, LPR, NCH, SRC, IdxT, true>(acc, c_l, v_l, j, a, foff, rem);
-            }
-            if constexpr (U > 2) {
-                if (rem > 2 && rem <= 4) gather_fma<4, VEC, LPR, NCH, SRC, IdxT, true>(acc, c_l, v_l, j, a, foff, rem);
-            }
-            if constexpr (U > 1) {
-                if (rem == 2) gather_fma<2, VEC, LPR, NCH, SRC, IdxT, false>(acc, c_l, v_l, j, a, foff);
-            }
-            if (rem == 1) gather_fma<1, VEC, LPR, NCH, SRC, IdxT, false>(acc, c_l, v_l, j, a, foff);
-        }
+        while (true) {
+            const int64_t left = end - base;
+            const int cnt = left < LPR ? (int)left : LPR;
 
-        if (row_done) {
-            if constexpr (VEC == 4) {
-                if (a.dst_bf16) {  // the result rows are bf16 (overwriting only): rounded once, here
-                    unsigned short *d16 = reinterpret_cast<unsigned short *>(a.dst) + (size_t)row * (size_t)ldd;
+            // where the next chunk comes from
+            int ni = i;
+            int nrow = row;
+            int64_t nbase = base + LPR, nend = end;
+            bool row_done = nbase >= end;
+            bool more = true;
+            if (row_done) {
+                if constexpr (MODE == kRowsNatural) {
+                    more = todo != 0;
+                    if (more) {
+                        ni = __builtin_ctzll(todo);
+                        todo &= todo - 1;
+                    }
+                } else {
+                    ni = i + 1;
+                    more = ni < ntask;
+                }
+                if (more) {
+                    nrow = group_bcast<LPR>(d_row, ni);
+                    nbase = group_bcast_idx<LPR>(d_start, ni);
+                    nend = nbase + group_bcast<LPR>(d_len, ni);
+                }
+            }
+            IdxT nc = 0;
+            float nv = 0.0f;
+            if (more && nbase + lig < nend) {
+                nc = __builtin_nontemporal_load(col + nbase + lig);
+                nv = __builtin_nontemporal_load(val + nbase + lig);
+            }
+
+            // full blocks of U gathers, then ONE more round for what is left (the smallest power of two of gathers
+            // that covers it, the surplus ones masked): a chunk of cnt elements costs ceil(cnt / U) dependent round trips
+            int j = 0;
+            for (; j + U <= cnt; j += U) gather_fma<U, VEC, LPR, NCH, SRC>(acc, c_l, v_l, j, a, foff);
+            const int rem = cnt - j;
+            if (rem > 0) {
+                if constexpr (U > 4) {
+                    if (rem > 4) gather_fma<8, VEC, LPR, NCH, SRC, IdxT, true>(acc, c_l, v_l, j, a, foff, rem);
+                }
+                if constexpr (U > 2) {
+                    if (rem > 2 && rem <= 4) gather_fma<4, VEC, LPR, NCH, SRC, IdxT, true>(acc, c_l, v_l, j, a, foff, rem);
+                }
+                if constexpr (U > 1) {
+                    if (rem == 2) gather_fma<2, VEC, LPR, NCH, SRC, IdxT, false>(acc, c_l, v_l, j, a, foff);
+                }
+                if (rem == 1) gather_fma<1, VEC, LPR, NCH, SRC, IdxT, false>(acc, c_l, v_l, j, a, foff);
+            }
+
+            if (row_done) {
+                if constexpr (VEC == 4) {
+                    if (a.dst_bf16) {  // the result rows are bf16 (overwriting only): rounded once, here
+                        unsigned short *d16 = reinterpret_cast<unsigned short *>(a.dst) + (size_t)row * (size_t)ldd;
 #pragma unroll
-                    for (int k = 0; k < NCH; ++k) {
-                        if (fok[k]) {
-                            typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-                            u32x2 r;
-                            r.x = (uint32_t)bf16_bits(acc[k].d.x) | ((uint32_t)bf16_bits(acc[k].d.y) << 16);
-                            r.y = (uint32_t)bf16_bits(acc[k].d.z) | ((uint32_t)bf16_bits(acc[k].d.w) << 16);
-                            __builtin_nontemporal_store(r, reinterpret_cast<u32x2 *>(d16 + foff[k]));
+                        for (int k = 0; k < NCH; ++k) {
+                            if (fok[k]) {
+                                typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+                                u32x2 r;
+                                r.x = (uint32_t)bf16_bits(acc[k].d.x) | ((uint32_t)bf16_bits(acc[k].d.y) << 16);
+                                r.y = (uint32_t)bf16_bits(acc[k].d.z) | ((uint32_t)bf16_bits(acc[k].d.w) << 16);
+                                __builtin_nontemporal_store(r, reinterpret_cast<u32x2 *>(d16 + foff[k]));
+                            }
+                        }
+                    } else {
+#pragma unroll
+                        for (int k = 0; k < NCH; ++k) {
+                            if (fok[k]) acc[k].store_stream(dst + foff[k]);
                         }
                     }
                 } else {
@@ -521,26 +605,26 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
                         if (fok[k]) acc[k].store_stream(dst + foff[k]);
                     }
                 }
-            } else {
+                if (!more) break;
+                dst = a.dst + (size_t)nrow * (size_t)ldd;
 #pragma unroll
                 for (int k = 0; k < NCH; ++k) {
-                    if (fok[k]) acc[k].store_stream(dst + foff[k]);
+                    acc[k] = V::zero();
+                    if (from_dst && fok[k]) acc[k] = V::load_stream(dst + foff[k]);
                 }
             }
-            if (!more) break;
-            dst = a.dst + (size_t)nrow * (size_t)ldd;
-#pragma unroll
-            for (int k = 0; k < NCH; ++k) {
-                acc[k] = V::zero();
-                if (from_dst && fok[k]) acc[k] = V::load_stream(dst + foff[k]);
-            }
+            i = ni;
+            row = nrow;
+            base = nbase;
+            end = nend;
+            c_l = nc;
+            v_l = nv;
         }
-        i = ni;
-        row = nrow;
-        base = nbase;
-        end = nend;
-        c_l = nc;
-        v_l = nv;
+        if constexpr (MODE == kRowsNatural) {
+            if (!scanner) return;
+        } else {
+            return;
+        }
     }
 }
 

@@ -6,19 +6,21 @@ order of self_benchmark/a64fx/model/layers/sageconv.py:65-93: ``out = Aggregator
 aggregation is this build's own definition of the workload: one weight matrix per layer
 (``Z = ((A X) W) / deg + b`` -- the degree normalisation is applied behind the dense
 product, where it fuses into the epilogue: D^-1 (A X) W == D^-1 ((A X) W)), ReLU, dropout
-with a precomputed seeded mask, log-softmax + NLL on the labelled nodes, Adam.  The
-forward and input-gradient products run on the matrix cores through the BLAS library
-behind ``torch.mm`` (fp32, or bf16 inputs with fp32 accumulation and fp32 output); the
-weight gradient -- a reduction over millions of rows into at most 256 x 256 outputs, the
-library's weakest shape -- runs in libgnnagg's own fp32 MFMA kernel.  With dense
-activations a layer whose widths the kernels take runs fused (``_FusedLayer``): the
-product (fp32, or bf16 inputs), the degree division, bias, ReLU and dropout are one libgnnagg
-kernel, and in the gradient direction the ReLU / dropout mask, the degree division, the bias
-gradient and the weight gradient are another; the fp32 input-gradient product stays with the
-BLAS library, the bf16-input one is the same libgnnagg product kernel.  ``gemm="bf16x3"`` keeps
-fp32 accuracy but feeds the matrix units every fp32 operand as three bf16 pieces (six bf16 MFMAs
-a product, a fraction of the fp32 MFMA's cycles): all three products of a fused layer run that
-way (where a layer is not fused, the weight gradient stays the fp32 kernel).
+with a precomputed seeded mask, log-softmax + NLL on the labelled nodes, Adam.  Every dense
+product runs on the matrix cores in libgnnagg's own kernels wherever they take the widths
+(inner width a multiple of 16 -- or padded to one for the input gradient --, at most 256 output
+columns per call): with dense activations a layer runs fused (``_FusedLayer``): the product
+(fp32, or bf16 inputs), the degree division, bias, ReLU and dropout are one kernel, and in the
+gradient direction the ReLU / dropout mask, the degree division, the bias gradient and the weight
+gradient are another, plus the input-gradient product (the same product kernel).  The forms
+that keep the product apart from the elementwise passes (``fused_layers=False``, a layer that
+multiplies first, packed activations in front of the product) call the same product kernel
+bare.  ``gemm="bf16x3"`` keeps fp32 accuracy but feeds the matrix units every fp32 operand as
+three bf16 pieces (six bf16 MFMAs a product, a fraction of the fp32 MFMA's cycles); plain
+``gemm="fp32"`` products (no epilogue) run that way too, where it is the fastest fp32-accurate
+form.  What the kernels do not take falls through to the BLAS library behind ``torch.mm`` --
+never silently: every such call goes through ``library_product``, which counts it
+(``LIBRARY_PRODUCTS``) and raises under ``forbid_library_products()``.
 """
 import contextlib
 from typing import List, Optional, Sequence
@@ -32,33 +34,75 @@ from .aggregator import Aggregator, AggregatorPacked
 from .sparse_tensor import _row_stride, _rows_are_dense
 
 
+# Dense products that libgnnagg's kernels do not take go to the BLAS library through this one door.  The counter says
+# how many did (a benchmark reports it per train step); ``forbid_library_products()`` turns every such call into an
+# error, for runs that must stay on the hand-written kernels.
+LIBRARY_PRODUCTS = {"count": 0, "forbidden": False}
+
+
+def library_product(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None, bf16_inputs: bool = False,
+                    out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``a @ b (+ bias)`` by the BLAS library (``bf16_inputs``: operands rounded to bf16, fp32 accumulation and
+    result), counted in ``LIBRARY_PRODUCTS``."""
+    if LIBRARY_PRODUCTS["forbidden"]:
+        raise RuntimeError("a dense product [%d, %d] @ [%d, %d] that libgnnagg's kernels do not take fell through to "
+                           "the BLAS library under forbid_library_products()" % (tuple(a.shape) + tuple(b.shape)))
+    LIBRARY_PRODUCTS["count"] += 1
+    if bf16_inputs:
+        y = torch.mm(a.to(torch.bfloat16), b.to(torch.bfloat16), out_dtype=torch.float32)
+        y = y if bias is None else y + bias
+        return y if out is None else out.copy_(y)
+    if bias is not None:
+        return torch.addmm(bias, a, b) if out is None else torch.addmm(bias, a, b, out=out)
+    return torch.mm(a, b) if out is None else torch.mm(a, b, out=out)
+
+
+@contextlib.contextmanager
+def forbid_library_products():
+    """Inside the block a dense product that would go to the BLAS library raises instead."""
+    previous = LIBRARY_PRODUCTS["forbidden"]
+    LIBRARY_PRODUCTS["forbidden"] = True
+    try:
+        yield
+    finally:
+        LIBRARY_PRODUCTS["forbidden"] = previous
+
+
+def plain_product(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor], form: int) -> torch.Tensor:
+    """``a @ b (+ bias)`` without an epilogue, in libgnnagg's product kernel where it takes the widths: operands
+    rounded to bf16 for ``BF16``, every operand as three bf16 pieces for ``FP32`` and ``BF16X3`` alike (fp32 accuracy;
+    for a plain product faster than the fp32 matrix instruction and than the BLAS library's fp32 product -- 7 M x 512
+    x 256: 10.8 ms against 14.8 and 12.9).  The BLAS library, counted, otherwise."""
+    if (a.is_cuda and a.dtype == torch.float32 and a.size(0) > 0
+            and _lib.lib().gnnagg_linear_shape_supported(a.size(1), b.size(1))):
+        return _fused_product(_kernel_ready(a), b.contiguous(), None if bias is None else bias.contiguous(), None, None,
+                              1.0, False, BF16 if form == BF16 else BF16X3)
+    return library_product(a, b, bias, bf16_inputs=form == BF16)
+
+
 class _Bf16InputLinear(torch.autograd.Function):
     """y = x @ w with x, w rounded to bf16, products accumulated in fp32, fp32 result; the
     input gradient is computed the same way.  The weight gradient stays in fp32: the
     hand-written kernel reads the fp32 operands as they are, which is faster than rounding
-    7 M-row operands to bf16 for the library's product, and more exact."""
-
-    @staticmethod
-    def _mm(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
-        return torch.mm(a.to(torch.bfloat16), b.to(torch.bfloat16), out_dtype=torch.float32)
+    7 M-row operands to bf16 first, and more exact."""
 
     @staticmethod
     def forward(ctx, x, w):
         ctx.save_for_backward(x, w)
-        return _Bf16InputLinear._mm(x, w)
+        return plain_product(x, w, None, BF16)
 
     @staticmethod
     def backward(ctx, g):
         x, w = ctx.saved_tensors
-        gx = _Bf16InputLinear._mm(g, w.t()) if ctx.needs_input_grad[0] else None
+        gx = input_gradient(g, w, BF16) if ctx.needs_input_grad[0] else None
         gw = weight_gradient(x, g) if ctx.needs_input_grad[1] else None
         return gx, gw
 
 
 def weight_gradient(x: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
-    """x^T @ g for tall-skinny fp32 operands through the library's MFMA kernel; falls back to
-    the BLAS library for shapes that kernel does not take (more than 256 columns).  Column
-    blocks of wider row-major tensors are read where they lie."""
+    """x^T @ g for tall-skinny fp32 operands through libgnnagg's MFMA kernel; the BLAS library (counted) for shapes
+    that kernel does not take (more than 256 columns).  Column blocks of wider row-major tensors are read where they
+    lie."""
     if not _rows_are_dense(x):
         x = x.contiguous()
     if not _rows_are_dense(g):
@@ -67,7 +111,7 @@ def weight_gradient(x: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
     L = _lib.lib()
     nbytes = int(L.gnnagg_wgrad_workspace_bytes(rows, fi, fo)) if x.is_cuda and x.dtype == torch.float32 else 0
     if nbytes == 0:
-        return torch.mm(x.t(), g)
+        return library_product(x.t(), g)
     out = torch.empty(fi, fo, dtype=torch.float32, device=x.device)
     workspace = torch.empty(nbytes // 4, dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
@@ -100,45 +144,23 @@ def weight_and_bias_gradient(x: torch.Tensor, g: torch.Tensor, form: int = 0):
 
 
 class _Fp32Linear(torch.autograd.Function):
-    """y = x @ w in fp32; the weight gradient (a reduction over millions of rows) runs in
-    the hand-written MFMA kernel, the two other products in the BLAS library."""
+    """y = x @ w to fp32 accuracy: the product and the input-gradient product in libgnnagg's product kernel (three
+    bf16 pieces an operand), the weight gradient (a reduction over millions of rows) in its fp32 MFMA kernel."""
 
     @staticmethod
     def forward(ctx, x, w):
         ctx.save_for_backward(x, w)
-        return torch.mm(x, w)
+        return plain_product(x, w, None, FP32)
 
     @staticmethod
     def backward(ctx, g):
         x, w = ctx.saved_tensors
-        gx = torch.mm(g, w.t()) if ctx.needs_input_grad[0] else None
+        gx = input_gradient(g, w, FP32) if ctx.needs_input_grad[0] else None
         gw = weight_gradient(x, g) if ctx.needs_input_grad[1] else None
         return gx, gw
 
 
-def _product_bf16x3(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
-    """a @ b with every fp32 operand fed to the matrix units as three bf16 pieces (fp32 accuracy); the BLAS library's
-    fp32 product for shapes the kernel does not take."""
-    if a.is_cuda and a.dtype == torch.float32 and _lib.lib().gnnagg_linear_shape_supported(a.size(1), b.size(1)):
-        return _fused_product(_kernel_ready(a), b.contiguous(), None, None, None, 1.0, False, BF16X3)
-    return torch.mm(a, b)
-
-
-class _Bf16x3Linear(torch.autograd.Function):
-    """y = x @ w, the product and the input-gradient product in the bf16 x 3 form of libgnnagg's product kernel; the
-    weight gradient in the fp32 MFMA kernel."""
-
-    @staticmethod
-    def forward(ctx, x, w):
-        ctx.save_for_backward(x, w)
-        return _product_bf16x3(x, w)
-
-    @staticmethod
-    def backward(ctx, g):
-        x, w = ctx.saved_tensors
-        gx = _product_bf16x3(g, w.t()) if ctx.needs_input_grad[0] else None
-        gw = weight_gradient(x, g) if ctx.needs_input_grad[1] else None
-        return gx, gw
+_Bf16x3Linear = _Fp32Linear   # a bare product has one fp32-accurate form: the two names run the same kernels
 
 
 def pack_keep_mask(keep: torch.Tensor) -> torch.Tensor:
@@ -198,23 +220,18 @@ def _fused_product(x, w, bias, keep_bits, row_div, scale, relu, form, out=None):
 
 
 def stacked_product(cat: torch.Tensor, weight: torch.Tensor, bias, form: int) -> torch.Tensor:
-    """cat @ weight (+ bias) in libgnnagg's product kernel with every operand as three bf16 pieces (fp32 accuracy: for
-    a plain product faster than the fp32 matrix instruction and than the BLAS library's fp32 product -- 7 M x 512 x 256:
-    10.8 ms against 14.8 and 12.9) where it takes the widths; the BLAS library's fp32 product otherwise."""
-    if (form in (FP32, BF16X3) and cat.is_cuda and cat.dtype == torch.float32 and cat.size(0) > 0
-            and _lib.lib().gnnagg_linear_shape_supported(cat.size(1), weight.size(1))):
-        return _fused_product(_kernel_ready(cat), weight.contiguous(), None if bias is None else bias.contiguous(),
-                              None, None, 1.0, False, BF16X3)
-    return torch.mm(cat, weight) if bias is None else torch.addmm(bias, cat, weight)
+    """cat @ weight (+ bias): ``plain_product`` (the SAGE layer's [A x | x] @ [W_neigh ; W_self])."""
+    return plain_product(cat, weight, bias, form)
 
 
-def input_gradient(g: torch.Tensor, weight: torch.Tensor, form: int) -> torch.Tensor:
+def input_gradient(g: torch.Tensor, weight: torch.Tensor, form: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """g @ weight^T, [rows, weight rows], through libgnnagg's product kernel: one call per block of at most 256 output
     columns, each writing its columns of the result.  ``form`` ``BF16`` rounds the operands to bf16; ``FP32`` and
     ``BF16X3`` both feed every operand as three bf16 pieces -- fp32 accuracy (errors at the level of the BLAS library's
     fp32 product), and for this plain product faster than the fp32 matrix instruction and than the library
     (7 M x 256 x 256: 5.8 ms against 8.0 and 7.0).  An inner width that is no multiple of 16 goes through a zero-padded
-    copy of ``g``.  The BLAS library's product only for what the kernel does not take."""
+    copy of ``g``.  ``out``: a [rows, weight rows] array with kernel-ready rows (a column block of a wider one is fine)
+    to write into.  The BLAS library's product, counted, only for what the kernel does not take."""
     wide, inner = weight.size(0), weight.size(1)
     blocks = [(c, min(c + 256, wide)) for c in range(0, wide, 256)]
     L = _lib.lib()
@@ -226,13 +243,15 @@ def input_gradient(g: torch.Tensor, weight: torch.Tensor, form: int) -> torch.Te
             weight = torch.nn.functional.pad(weight, (0, padded - inner))
         g = _kernel_ready(g)
         kernel_form = BF16 if form == BF16 else BF16X3
-        out = torch.empty(g.size(0), wide, dtype=torch.float32, device=g.device)
+        if out is None:
+            out = torch.empty(g.size(0), wide, dtype=torch.float32, device=g.device)
+        elif (out.shape != (g.size(0), wide) or out.dtype != torch.float32 or not _rows_are_dense(out)
+              or _row_stride(out) % 4 != 0 or out.data_ptr() % 16 != 0):
+            raise RuntimeError("Input mismatch: out must be float32 [rows, weight rows] with 16-byte aligned rows")
         for lo, hi in blocks:
             _fused_product(g, weight[lo:hi].t().contiguous(), None, None, None, 1.0, False, kernel_form, out=out[:, lo:hi])
         return out
-    if form == BF16:
-        return _Bf16InputLinear._mm(g, weight.t())
-    return torch.mm(g, weight.t())
+    return library_product(g, weight.t(), bf16_inputs=form == BF16, out=out)
 
 
 class _FusedLayer(torch.autograd.Function):

@@ -28,7 +28,8 @@ import torch
 import torch.nn.functional as F
 
 from . import _lib, aggregator
-from .gcn import _FORMS, _mean_nll, input_gradient, scored_rows, stacked_product, weight_and_bias_gradient, weight_gradient
+from .gcn import (_FORMS, _mean_nll, input_gradient, plain_product, scored_rows, stacked_product,
+                  weight_and_bias_gradient, weight_gradient)
 from .sparse_tensor import SparseTensor, _row_stride
 
 
@@ -244,14 +245,15 @@ class _SageConvLinearFirst(torch.autograd.Function):
     the reference sketches and leaves commented out, sageconv.py:67-71, :84)."""
 
     @staticmethod
-    def forward(ctx, graph, feats_in, weight, bias, layer, num_bits, is_pre_delay, is_training, normalize):
+    def forward(ctx, graph, feats_in, weight, bias, layer, num_bits, is_pre_delay, is_training, normalize, form=0):
         fi = weight.size(0) // 2
         ctx.staged = feats_in.size(1) == 2 * fi      # [N, 2 fi] with the features in the right half
         x = feats_in[:, fi:] if ctx.staged else feats_in
         folded = getattr(graph, "in_degrees_folded", False)
         ctx.divide = bool(normalize) and not folded
-        left = torch.mm(x, weight[:fi])                                   # x W_n
-        out = torch.mm(x, weight[fi:]) if bias is None else torch.addmm(bias, x, weight[fi:])
+        ctx.form = form
+        left = plain_product(x, weight[:fi], None, form)                  # x W_n
+        out = plain_product(x, weight[fi:], bias, form)                   # x W_s + b
         feats = aggregator._DenseFeatures(left)
         if ctx.divide:
             agg = aggregator._forward(ctx, graph, feats, layer, num_bits, is_pre_delay, is_training)
@@ -281,17 +283,18 @@ class _SageConvLinearFirst(torch.autograd.Function):
         elif want_b:
             grad_b = g.sum(dim=0)
         if ctx.needs_input_grad[1]:
+            # d/d x = (d/d (x W_n)) W_n^T + g W_s^T = [d/d (x W_n) | g] @ [W_n | W_s]^T: one product
+            both = torch.cat([grad_left, g], dim=1)
+            stacked = torch.cat([weight[:fi], weight[fi:]], dim=1)          # [fi, 2 fo]
             if ctx.staged:
                 # the gradient goes where the features were: the right half of an [N, 2 fi] array
                 # (its left half was scratch on the way forward: zero gradient, written as such)
                 grad_x = torch.empty(x.size(0), 2 * fi, dtype=torch.float32, device=x.device)
                 grad_x[:, :fi].zero_()
-                target = grad_x[:, fi:]
-                torch.mm(g, weight[fi:].t(), out=target)
-                target.addmm_(grad_left, weight[:fi].t())
+                input_gradient(both, stacked, ctx.form, out=grad_x[:, fi:])
             else:
-                grad_x = torch.addmm(torch.mm(g, weight[fi:].t()), grad_left, weight[:fi].t())
-        return None, grad_x, grad_w, grad_b, None, None, None, None, None
+                grad_x = input_gradient(both, stacked, ctx.form)
+        return None, grad_x, grad_w, grad_b, None, None, None, None, None, None
 
 
 class _LinearView:
@@ -377,7 +380,7 @@ class DistSAGEConvGrad(torch.nn.Module):
             if not local_nodes_feat.is_cuda or local_nodes_feat.dtype != torch.float32:
                 raise RuntimeError("Input mismatch: the features must be a float32 GPU (HIP) tensor")
             return _SageConvLinearFirst.apply(graph, local_nodes_feat, self.weight, self.bias, layer, self.num_bits,
-                                              self.is_pre_delay, self.training, self.normalize)
+                                              self.is_pre_delay, self.training, self.normalize, _FORMS[self.gemm])
         if width == self.in_channels:
             if local_nodes_feat.requires_grad:
                 raise RuntimeError("features that need a gradient must be handed over staged (stage_input)")

@@ -149,17 +149,22 @@ def test_train_step_matches_cpu_autograd(gemm, tol, fuse, linear_first, shape):
 
 
 @pytest.mark.parametrize("gemm", ["fp32", "bf16", "bf16x3"])
-@pytest.mark.parametrize("packed_activations", [False, True])
-def test_default_train_step_calls_no_library_product(gemm, packed_activations, monkeypatch):
+@pytest.mark.parametrize("packed_activations,linear_first,fused_layers",
+                         [(False, False, True), (True, False, True), (False, True, True), (False, False, False),
+                          (True, True, False)])
+def test_train_step_calls_no_library_product(gemm, packed_activations, linear_first, fused_layers, monkeypatch):
     """At the widths of the full train-step workload every dense product of the step -- layer products, weight
-    gradients, input gradients (the last layer's inner width 172 included) -- runs in libgnnagg's kernels: the step
-    goes through with torch's matrix products taken away."""
+    gradients, input gradients (the last layer's inner width 172 included) -- runs in libgnnagg's kernels, in the
+    default form and in the optional ones (the narrowing last layer multiplying first, the product kept apart from
+    the elementwise passes): the step goes through with torch's matrix products taken away and the door to the BLAS
+    library shut."""
     dev = "cuda:0"
     n, dims, part_args = _SHAPES["c5_widths"]
     part = synthetic.partition_edges(n, *part_args, seed=3, device=dev)
     graph = synthetic.build_partition_graph(part, max(dims), True, exchange=synthetic.SeededHaloExchange(5), device=dev)
     torch.manual_seed(0)
-    model = gcn.GCN(dims, gemm=gemm, packed_activations=packed_activations).to(dev)
+    model = gcn.GCN(dims, gemm=gemm, packed_activations=packed_activations,
+                    linear_first_when_narrowing=linear_first, fused_layers=fused_layers).to(dev)
     opt = torch.optim.Adam(model.parameters(), lr=0.01)
     gen = torch.Generator(device=dev).manual_seed(1)
     x = torch.randn(n, dims[0], device=dev, generator=gen)
@@ -175,10 +180,28 @@ def test_default_train_step_calls_no_library_product(gemm, packed_activations, m
         monkeypatch.setattr(torch, name, taken_away)
     monkeypatch.setattr(torch.Tensor, "__matmul__", taken_away)
     monkeypatch.setattr(torch.nn.functional, "linear", taken_away)
-    for every_node in (False, True):
-        loss = float(gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks,
-                                    restrict_last_layer=not every_node))
-        assert np.isfinite(loss) and abs(loss - want) < 0.5
+    before = gcn.LIBRARY_PRODUCTS["count"]
+    with gcn.forbid_library_products():
+        for every_node in (False, True):
+            loss = float(gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks,
+                                        restrict_last_layer=not every_node))
+            assert np.isfinite(loss) and abs(loss - want) < 0.5
+    assert gcn.LIBRARY_PRODUCTS["count"] == before
+
+
+def test_a_product_the_kernels_do_not_take_is_counted_or_refused():
+    """Widths outside the product kernel (inner width no multiple of 16) go to the BLAS library through the one
+    counted door, and raise under ``forbid_library_products()``."""
+    a = torch.randn(100, 20, device="cuda")
+    b = torch.randn(20, 24, device="cuda")
+    before = gcn.LIBRARY_PRODUCTS["count"]
+    y = gcn.plain_product(a, b, None, gcn.FP32)
+    assert gcn.LIBRARY_PRODUCTS["count"] == before + 1
+    assert torch.allclose(y, a @ b, rtol=1e-4, atol=1e-4)
+    with gcn.forbid_library_products():
+        with pytest.raises(RuntimeError, match="BLAS library"):
+            gcn.plain_product(a, b, None, gcn.FP32)
+    assert gcn.LIBRARY_PRODUCTS["forbidden"] is False
 
 
 @pytest.mark.parametrize("num_bits", [2, 16])

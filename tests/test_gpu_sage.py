@@ -204,17 +204,21 @@ def _cpu_mats(graph, is_pre_delay):
     return a_local, a_in, a_out_t
 
 
+@pytest.mark.parametrize("linear_first", [False, True])
 @pytest.mark.parametrize("gemm", ["fp32", "bf16x3"])
-def test_sage_train_step_calls_no_library_product(gemm, monkeypatch):
+def test_sage_train_step_calls_no_library_product(gemm, linear_first, monkeypatch):
     """At the widths of the full train-step workload (128 -> 256 -> 256 -> 172) every dense product of the SAGE step --
-    the stacked ``[A x | x] @ W``, the weight gradients of both halves, the input gradients -- runs in libgnnagg's
-    kernels: the step goes through with torch's matrix products taken away."""
+    the stacked ``[A x | x] @ W``, the weight gradients of both halves, the input gradients, and with ``linear_first``
+    the two products in front of the narrowing last layer's aggregation and its one input-gradient product (inner
+    width 344, padded) -- runs in libgnnagg's kernels: the step goes through with torch's matrix products taken away
+    and the door to the BLAS library shut."""
     dev_ = "cuda:0"
     n, dims = 20_000, [128, 256, 256, 172]
     part = synthetic.partition_edges(n, 16, 3, 6.8, 1.8, 2000, 8500, 57_000, seed=3, device=dev_)
     graph = synthetic.build_partition_graph(part, 256, True, exchange=synthetic.SeededHaloExchange(5), device=dev_)
     torch.manual_seed(0)
-    model = sage.DistSAGE(dims[0], dims[1], dims[-1], num_layers=3, dropout=0.5, is_pre_delay=True, gemm=gemm).to(dev_)
+    model = sage.DistSAGE(dims[0], dims[1], dims[-1], num_layers=3, dropout=0.5, is_pre_delay=True, gemm=gemm,
+                          linear_first_when_narrowing=linear_first).to(dev_)
     opt = torch.optim.Adam(model.parameters(), lr=0.01)
     gen = torch.Generator(device=dev_).manual_seed(1)
     x = torch.randn(n, dims[0], device=dev_, generator=gen)
@@ -223,6 +227,7 @@ def test_sage_train_step_calls_no_library_product(gemm, monkeypatch):
     masks = sage.make_dropout_masks(n, dims[1], 3, 0.5, 7, dev_)
     staged = sage.stage_input(x)
     want = float(sage.train_step(model, opt, graph, staged, labels, train_idx, masks))
+    from gnn_benchmark_amd import gcn
 
     def taken_away(*a, **k):
         raise AssertionError("a BLAS-library product inside the train step")
@@ -231,9 +236,10 @@ def test_sage_train_step_calls_no_library_product(gemm, monkeypatch):
         monkeypatch.setattr(torch, name, taken_away)
     monkeypatch.setattr(torch.Tensor, "__matmul__", taken_away)
     monkeypatch.setattr(torch.nn.functional, "linear", taken_away)
-    for every_node in (False, True):
-        loss = float(sage.train_step(model, opt, graph, staged, labels, train_idx, masks, not every_node))
-        assert np.isfinite(loss) and abs(loss - want) < 0.5
+    with gcn.forbid_library_products():
+        for every_node in (False, True):
+            loss = float(sage.train_step(model, opt, graph, staged, labels, train_idx, masks, not every_node))
+            assert np.isfinite(loss) and abs(loss - want) < 0.5
 
 
 @pytest.mark.parametrize("is_pre_delay", [True, False])
