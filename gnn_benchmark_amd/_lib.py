@@ -21,6 +21,7 @@ EXPORTS = (
     "gnnagg_plan_create",
     "gnnagg_plan_create_ex",
     "gnnagg_plan_destroy",
+    "gnnagg_plans_release",
     "gnnagg_plan_spmm_f32",
     "gnnagg_plan_spmm_strided_f32",
     "gnnagg_plan_spmm_two_sources_f32",
@@ -122,6 +123,8 @@ def lib() -> ctypes.CDLL:
     L.gnnagg_plan_create_ex.argtypes = [vp, vp, i64, i64, i64, ctypes.POINTER(PlanOptions), vp, ctypes.POINTER(vp)]
     L.gnnagg_plan_destroy.restype = i32
     L.gnnagg_plan_destroy.argtypes = [vp]
+    L.gnnagg_plans_release.restype = i32
+    L.gnnagg_plans_release.argtypes = []
     L.gnnagg_plan_spmm_f32.restype = i32
     L.gnnagg_plan_spmm_f32.argtypes = [vp, vp, vp, vp, i64, i32, vp]
     L.gnnagg_plan_spmm_strided_f32.restype = i32

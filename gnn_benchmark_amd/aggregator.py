@@ -135,6 +135,20 @@ def _convert(src: torch.Tensor, dst: torch.Tensor) -> None:
             raise RuntimeError("Input mismatch: bf16 staging converts float32 <-> bfloat16 only")
 
 
+def _poison_unfilled_rows(graph) -> None:
+    """Once per pair of boundary buffers, when a run first lets the products write / read the exchange format
+    themselves: the fp32 ``send_buf`` / ``recv_buf`` -- which the reference always fills (aggregator.py:85-88,
+    communicator.py:128, :137) and these runs no longer touch -- are set to NaN over their whole storage, so that a
+    hook or debugging code that still reads them sees at once that the rows are not there, instead of stale ones."""
+    buf = graph.comm_buf
+    if getattr(buf, "_fp32_rows_poisoned", False):
+        return
+    for t in (buf.send_buf, buf.recv_buf):
+        whole = torch.empty(0, dtype=t.dtype, device=t.device).set_(t.untyped_storage())
+        whole.fill_(float("nan"))
+    buf._fp32_rows_poisoned = True
+
+
 def _outgoing_quantized(graph, direction: str):
     """(fp32 rows, packed bytes, parameters, per-rank row prefix) of the outgoing side of a quantised exchange."""
     qbuf = graph.comm_buf_for_quantization
@@ -316,6 +330,8 @@ def _forward(ctx, graph, feats, layer, num_bits: int, is_pre_delay: bool, is_tra
             packed_by_product = True
         else:  # raw boundary rows (as bf16 at once when they travel so)
             feats.gather(graph.idx_nodes_send_to_others, graph.comm_buf.send_buf_fp16 if half_fused else send_buf)
+        if packed_by_product or half_fused:
+            _poison_unfilled_rows(graph)
         if quantized:
             comm_handle = _quantize_and_exchange(graph, num_bits, f"forward{layer}", "forward", packed_by_product)
         elif half:
@@ -347,6 +363,8 @@ def _forward(ctx, graph, feats, layer, num_bits: int, is_pre_delay: bool, is_tra
     if comm_handle is not None:
         comm_handle.wait()
     fused = quantized and _fused_dequantize(graph, feat_len) and out.stride(0) % 4 == 0
+    if fused:
+        _poison_unfilled_rows(graph)
     if quantized and not fused:
         _dequantize_received(graph, num_bits, "forward")
     half_fused = half_fused and out.stride(0) % 4 == 0
@@ -510,6 +528,8 @@ def _backward(ctx, local_out_grad, out=None, accumulate: bool = False):
         else:
             SPMM_backward(remote, local_out_grad, remote_nodes_grad_buf, accumulate=False)
 
+    if packed_by_product or half_fused:
+        _poison_unfilled_rows(graph)
     comm_handle = None
     if quantized:
         comm_handle = _quantize_and_exchange(graph, num_bits, layer, "backward", packed_by_product)
@@ -548,6 +568,8 @@ def _backward(ctx, local_out_grad, out=None, accumulate: bool = False):
     if comm_handle is not None:
         comm_handle.wait()
     fused = quantized and _fused_dequantize(graph, feat_len) and local_nodes_grad.stride(0) % 4 == 0
+    if fused:
+        _poison_unfilled_rows(graph)
     if quantized and not fused:
         _dequantize_received(graph, num_bits, "backward")
     half_fused = half_fused and local_nodes_grad.stride(0) % 4 == 0

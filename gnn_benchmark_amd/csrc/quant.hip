@@ -171,7 +171,10 @@ __global__ __launch_bounds__(256) void quantize_segments_kernel(const float *__r
     const int l = (int)threadIdx.x & (G - 1);
     const int nvec = (feat + VEC - 1) / VEC;  // VEC == 4 implies feat % 4 == 0
     // where fp32 row r of the buffer lies: in x itself, or (index given: the gather of raw boundary rows folded in)
-    // at row index[r] of x -- an index outside x is never dereferenced, row 0 is read in its place
+    // at row index[r] of x -- an index outside x is never dereferenced, row 0 is read in its place and the row's
+    // parameters are stored as NaN, so that whoever dequantises the row gets NaN (what the plain row gather stores
+    // for such an index)
+    auto row_is_bad = [&](int r) -> bool { return index && (uint64_t)index[r] >= (uint64_t)src_rows; };
     auto row_at = [&](int r) -> const float * {
         size_t at = (size_t)r;
         if (index) {
@@ -246,7 +249,8 @@ __global__ __launch_bounds__(256) void quantize_segments_kernel(const float *__r
                     params_of(lo, hi, BITS, zp[u][k], scale[u][k]);
                     inv[u][k] = __builtin_amdgcn_rcpf(scale[u][k]);
                     if (l == 0) {
-                        const float2 zs = make_float2(zp[u][k], scale[u][k]);
+                        float2 zs = make_float2(zp[u][k], scale[u][k]);
+                        if (row_is_bad(sl.rg[u].first + k)) zs = make_float2(NAN, NAN);
                         *reinterpret_cast<float2 *>(params + (size_t)(sl.rg[u].first + k) * 2) = zs;
                     }
                 }

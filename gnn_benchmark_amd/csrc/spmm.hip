@@ -435,6 +435,7 @@ extern "C" int gnnagg_plan_create_ex(const int64_t *rowptr, const int64_t *col, 
                        opt.short_rows_per_group >= 0 && opt.rows_per_group <= kMaxRowsPerGroup &&
                        opt.short_rows_per_group <= kMaxRowsPerGroup,
                    "plan options: thresholds must not be negative, rows per group lie in 0 .. %d", kMaxRowsPerGroup);
+    GNNAGG_REQUIRE(opt.reserved[0] == 0 && opt.reserved[1] == 0, "plan options: the reserved fields must be 0");
     GNNAGG_REQUIRE((opt.lanes_per_row == 0 && opt.loads_per_lane == 0) || shape_exists(opt.lanes_per_row, opt.loads_per_lane),
                    "plan options: no row kernel with %d lanes per row and %d loads per lane", opt.lanes_per_row,
                    opt.loads_per_lane);
@@ -549,6 +550,13 @@ extern "C" int gnnagg_plan_destroy(gnnagg_plan *plan) {
     if (!plan) return GNNAGG_OK;
     std::lock_guard<std::mutex> hold(retired_mutex);
     retired_plans.push_back(plan);
+    return GNNAGG_OK;
+}
+
+extern "C" int gnnagg_plans_release(void) {
+    int device = 0;
+    GNNAGG_HIP(hipGetDevice(&device));
+    free_retired_plans(device);
     return GNNAGG_OK;
 }
 

@@ -151,6 +151,15 @@ class SpmmPlan:
                 pass
 
 
+def release_plans(device=None) -> None:
+    """Free the device memory of the plans dropped so far on ``device`` (default: the current one).  A dropped plan
+    only queues its memory, so that a destructor in the middle of a step never synchronises; the queue is emptied by
+    the next plan creation on the device -- or here, at a moment the caller knows to be safe (this synchronises the
+    device): the end of graph set-up, between epochs."""
+    with torch.cuda.device(device):
+        _lib.check(_lib.lib().gnnagg_plans_release())
+
+
 def _rows_are_dense(t: torch.Tensor) -> bool:
     """2-D, unit stride along each row, rows not overlapping (a column block of a row-major tensor)."""
     return t.dim() == 2 and (t.size(1) <= 1 or t.stride(1) == 1) and (t.size(0) <= 1 or t.stride(0) >= t.size(1))

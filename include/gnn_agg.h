@@ -28,7 +28,7 @@ extern "C" {
 
 /* Raised whenever an exported prototype changes, an entry point goes away or the meaning of an argument changes
  * (2: `src_rows` in the row gathers, `workspace_bytes` in the weight-gradient entry points, 12 values from
- * gnnagg_plan_info; 3: the measurement probes left the library, gnnagg_plan_spmm_two_sources_f32 came).  Every binding compares it with
+ * gnnagg_plan_info; 3: the measurement probes left the library, gnnagg_plan_spmm_two_sources_f32 and gnnagg_plans_release came).  Every binding compares it with
  * gnnagg_abi_version() of the library it loaded before the first call. */
 #define GNNAGG_ABI_VERSION 3
 
@@ -110,6 +110,13 @@ int gnnagg_plan_create_ex(const int64_t *rowptr, const int64_t *col, int64_t row
  * end.  The plan's device memory is released by the next gnnagg_plan_create[_ex] on the same device (set-up work
  * that synchronises anyway), after a device synchronisation. */
 int gnnagg_plan_destroy(gnnagg_plan *plan);
+
+/* Releases, now, the device memory of every plan of the current device that was handed to gnnagg_plan_destroy
+ * (column indices narrowed to 32 bits and the row schedule: 4 bytes per stored element + 16 per row, about 0.5 GB
+ * for a 7 M-row / 100 M-element matrix).  Synchronises the device first, so call it where that is safe -- the end
+ * of graph set-up, between epochs -- and never while a stream is being captured.  A process that drops plans and
+ * creates no new one on that device would otherwise keep their memory until it ends.  No reference counterpart. */
+int gnnagg_plans_release(void);
 
 /* out (+)= A @ mat through a plan.  `value` is the fp32 [nnz] array in the CSR order
  * the plan was built from.  accumulate != 0: out += A@mat (the reference semantics,
@@ -441,8 +448,9 @@ int gnnagg_dequantize_segments_f32(const uint8_t *packed, const float *params, f
  * src -- `torch.index_select(local_nodes_feat, 0, idx_nodes_send_to_others, out=send_buf)` followed by
  * `quantize_tensor_for_all_procs(send_buf, ...)` (model/layers/aggregator.py:51, communicator/communicator.py:281-311) as
  * one pass; same bytes and parameters, the gathered fp32 rows never written.  src fp32 [src_rows, feat] contiguous,
- * index int64 [rows]; an index outside [0, src_rows) is never dereferenced (row 0 is read in its place; raising for
- * it is gnnagg_check_index's part).  No allocation, no host synchronisation. */
+ * index int64 [rows]; an index outside [0, src_rows) is never dereferenced (row 0 is read in its place and the row's
+ * two parameters are stored as NaN, so the row dequantises to NaN -- what gnnagg_gather_rows_f32 stores for such an
+ * index; raising for it is gnnagg_check_index's part).  No allocation, no host synchronisation. */
 int gnnagg_gather_quantize_segments_f32(const float *src, int64_t src_rows, const int64_t *index, uint8_t *packed,
                                         float *params, const int32_t *row_range, const int32_t *packed_range,
                                         int64_t segments, int64_t rows, int64_t packed_rows, int64_t feat, int bits,

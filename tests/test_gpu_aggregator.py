@@ -807,6 +807,23 @@ def test_bad_indices_raise_instead_of_reading_out_of_bounds():
     torch.cuda.synchronize()
     assert torch.equal(out[0], src[7]) and torch.equal(out[3], src[2]) and bool(torch.isnan(out[1:3]).all())
 
+    # ... and the gather that quantises: NaN parameters for the row of a bad index (it dequantises to NaN), the others
+    # as the checked path writes them
+    rr = torch.tensor([0, 4], dtype=torch.int32, device="cuda")
+    pr = torch.tensor([0, 1], dtype=torch.int32, device="cuda")
+    packed_bad = torch.zeros(1, 8, dtype=torch.uint8, device="cuda")
+    params_bad = torch.zeros(4, 2, device="cuda")
+    _lib.check(_lib.lib().gnnagg_gather_quantize_segments_f32(
+        _lib.ptr(src), 50, _lib.ptr(idx), _lib.ptr(packed_bad), _lib.ptr(params_bad), _lib.ptr(rr), _lib.ptr(pr), 1, 4,
+        1, 8, 2, _lib.current_stream(src.device)))
+    packed_ok = torch.zeros(1, 8, dtype=torch.uint8, device="cuda")
+    params_ok = torch.zeros(4, 2, device="cuda")
+    computation_ops.gather_quantize_for_all_procs(src, torch.tensor([7, 0, 0, 2], device="cuda"), packed_ok, params_ok,
+                                                  torch.tensor([0, 4], dtype=torch.int32), 1, 2)
+    torch.cuda.synchronize()
+    assert bool(torch.isnan(params_bad[1:3]).all()) and torch.equal(params_bad[[0, 3]], params_ok[[0, 3]])
+    assert torch.equal(packed_bad & 0xC3, packed_ok & 0xC3)   # the 2-bit fields of rows 0 and 3
+
     rowptr = torch.tensor([0, 2, 3], device="cuda")
     val = torch.ones(3, device="cuda")
     res = torch.zeros(2, 8, device="cuda")

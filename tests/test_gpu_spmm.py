@@ -712,3 +712,60 @@ def test_side_by_side_matrix_is_the_two_chains_joined():
         want_c = np.concatenate([lrt[lcp[r]:lcp[r + 1]], qrt[qcp[r]:qcp[r + 1]] + 400])
         want_v = np.concatenate([lvt[lcp[r]:lcp[r + 1]], qvt[qcp[r]:qcp[r + 1]]])
         assert np.array_equal(tc[tp[r]:tp[r + 1]], want_c) and np.array_equal(tv[tp[r]:tp[r + 1]], want_v)
+
+
+@pytest.mark.parametrize("feat", [1, 6, 100, 128, 256, 602])
+def test_plan_less_operator_with_its_long_rows_first_equals_the_plan(feat):
+    """From 16 384 rows on, the first blocks of the plan-less operator's launch walk rowptr and run the rows of more
+    than 64 elements, the others leave those rows out: every row is still done exactly once, by the same chain --
+    rows of every length around the threshold, very long ones, empty ones, a row count that ends inside a scanning
+    group's stretch, results onto random values."""
+    rows, cols = 16_384 + 777, 5000
+    rng = np.random.default_rng(feat)
+    deg = rng.poisson(5, rows)
+    deg[::11] = 0
+    deg[5::97] = rng.integers(60, 70, deg[5::97].shape[0])      # around the threshold
+    deg[[3, 9000, rows - 1, rows - 2]] = [4000, 900, 300, 65]
+    rowptr = np.concatenate(([0], np.cumsum(deg))).astype(np.int64)
+    col = rng.integers(0, cols, rowptr[-1]).astype(np.int64)
+    val = rng.standard_normal(rowptr[-1]).astype(np.float32)
+    x = dev(rng.standard_normal((cols, feat)).astype(np.float32))
+    out0 = dev(rng.standard_normal((rows, feat)).astype(np.float32))
+    want = out0.clone()
+    SpmmPlan(dev(rowptr), dev(col), rows, cols).spmm(dev(val), x, want)
+    got = out0.clone()
+    computation_ops.spmm(dev(rowptr), dev(col), dev(val), x, got, rows, EMPTY_I32, EMPTY_I32)
+    assert torch.equal(got, want)
+    # fewer sparse rows than the arrays hold: the rows behind stay as they are
+    got = out0.clone()
+    computation_ops.spmm(dev(rowptr), dev(col), dev(val), x, got, 16_500, EMPTY_I32, EMPTY_I32)
+    assert torch.equal(got[:16_500], want[:16_500]) and torch.equal(got[16_500:], out0[16_500:])
+    sample = [3, 9000, 5, 102, 16_499]
+    ref = _oracle(np.concatenate(([0], np.cumsum(deg[sample]))).astype(np.int64),
+                  np.concatenate([col[rowptr[r]:rowptr[r + 1]] for r in sample]),
+                  np.concatenate([val[rowptr[r]:rowptr[r + 1]] for r in sample]), x.cpu().numpy(),
+                  out0[sample].cpu().numpy())
+    assert np.array_equal(got[sample].cpu().numpy(), ref)
+
+
+def test_release_plans_gives_the_memory_of_dropped_plans_back():
+    """A dropped plan only queues its device memory (no synchronisation inside a step); ``release_plans`` frees the
+    queue at a moment the caller picks."""
+    from gnn_benchmark_amd.sparse_tensor import release_plans
+
+    a = random_csr(200_000, 4000, 0.005, seed=5)   # 4 M stored elements: 16 MB of narrowed columns + 3.2 MB of tasks
+    rowptr, col = dev(a.indptr.astype(np.int64)), dev(a.indices.astype(np.int64))
+    release_plans()
+    torch.cuda.synchronize()
+    free0 = torch.cuda.mem_get_info()[0]
+    plan = SpmmPlan(rowptr, col, 200_000, 4000)
+    torch.cuda.synchronize()
+    held = free0 - torch.cuda.mem_get_info()[0]
+    assert held >= 16_000_000
+    del plan
+    torch.cuda.synchronize()
+    queued = torch.cuda.mem_get_info()[0]
+    assert free0 - queued >= 16_000_000   # still held: only queued
+    release_plans()
+    # (the runtime may keep a pool chunk of its own: what must come back is the plan's arrays)
+    assert torch.cuda.mem_get_info()[0] - queued >= 16_000_000

