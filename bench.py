@@ -537,6 +537,19 @@ def run_c2(args, gate, sink):
         for f in (128, 256, 172, 40, 47):
             if f != args.feat:
                 widths.append(spmm_pair(src, f, max(3, args.steps // 4), 2, gen, args, "c2")[0])
+        # a width that is no multiple of 4 (4-byte loads) against the same rows padded by one zero column to 48
+        # (16-byte loads): the aggregation of a 47-class layer kept in 48-float rows; the first 47 columns of the
+        # result are the same bits
+        dev_rows, plan, val = src.sparse_size(0), src.get_plan(), src.csr()[2]
+        x48 = torch.zeros(dev_rows, 48, device=dev)
+        x48[:, :47].normal_(generator=gen)
+        o48 = torch.zeros(dev_rows, 48, device=dev)
+        x47, o47 = x48[:, :47].contiguous(), torch.zeros(dev_rows, 47, device=dev)
+        _, ms47 = time_plan(plan, val, x47, o47, 5, 2, accumulate=False)
+        _, ms48 = time_plan(plan, val, x48, o48, 5, 2, accumulate=False)
+        widths.append({"feat": 47, "padded_to": 48, "forward_ms": round(ms47, 4), "forward_ms_padded": round(ms48, 4),
+                       "same_bits": bool(torch.equal(o48[:, :47], o47))})
+        del x48, o48, x47, o47
         sink.put("c2", widths)
     return line
 
