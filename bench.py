@@ -128,7 +128,8 @@ MEASURED_TRAFFIC = {
     ("c4", "local_T", 128): (5.48742e+10, 3.58400e+09, _P), ("c4", "local_T_overwrite", 128): (5.12387e+10, 3.58400e+09, _P),
     ("c4", "post", 128): (1.43898e+10, 3.37825e+09, _P), ("c4", "post_overwrite", 128): (1.10093e+10, 3.58400e+09, _P),
     ("c4", "post_T", 128): (1.22983e+10, 1.55268e+09, _P), ("c4", "post_T_overwrite", 128): (1.07407e+10, 1.55268e+09, _P),
-    ("c4", "local_planless", 128): (5.58080e+10, 3.58400e+09, _P),
+    ("c4", "local_planless", 128): (5.50780e+10, 3.58400e+09, _P),
+    ("c4", "local+post", 128): (6.22570e+10, 3.58400e+09, _P), ("c4", "local_T+pre_T", 128): (6.22570e+10, 3.58400e+09, _P),
 }
 
 
@@ -893,7 +894,7 @@ def run_c4(args, graph, setup_s, gate=None):
         e1.record()
         e1.synchronize()
         ops.append(op_report(nm, m.nnz(), m.sparse_size(0), m.sparse_size(1), feat, e0.elapsed_time(e1) / steps,
-                             plan.info()["empty_rows"], False))
+                             plan.info()["empty_rows"], False, measured_traffic(args, "c4", key, feat)))
         ops[-1]["as_run_by_aggregator"] = "one_launch"
     graph.comm_buf.resize_buffer(graph.comm_splits, feat, 32)  # (the buffer's own tensors again, not delivered rows)
     codec = run_c4_codec(graph, feat, steps, gen, cpu=not args.no_cpu_baseline)
