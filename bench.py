@@ -98,7 +98,8 @@ def c4_targets(c4):
     out = {"products_ms_fracmodel_fracmeasured": products, "feat": c4["feat"],
            "min_frac_model": min((v[1] for v in products.values()), default=None)}
     for k in ("aggregator_forward_ms", "aggregator_forward_backward_ms", "aggregator_forward_ms_one_launch",
-              "aggregator_forward_backward_ms_one_launch", "aggregator_forward_backward_ms_int2_exchange"):
+              "aggregator_forward_backward_ms_one_launch", "aggregator_forward_backward_ms_int2_exchange",
+              "aggregator_forward_backward_ms_int2_exchange_one_launch"):
         if k in c4:
             out[k] = c4[k]
     return out
@@ -930,6 +931,18 @@ def run_c4(args, graph, setup_s, gate=None):
         o.backward(g)
     torch.cuda.synchronize()
     int2_fused_ms = (time.perf_counter() - t0) * 1e3 / steps
+    # ... and with one launch for the local elements and the received ones, gathered straight from the packed bytes
+    graph.one_launch = True
+    for _ in range(2):
+        Aggregator.apply(graph, xr, 0, 2, True, True).backward(g)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        o = Aggregator.apply(graph, xr, 0, 2, True, True)
+        o.backward(g)
+    torch.cuda.synchronize()
+    int2_one_launch_ms = (time.perf_counter() - t0) * 1e3 / steps
+    graph.one_launch = False
     from gnn_benchmark_amd.spmm_kernel import SPMM_forward_quantized
 
     qb, m = graph.comm_buf_for_quantization, graph.adj_t_pre_post_aggr_from
@@ -980,6 +993,17 @@ def run_c4(args, graph, setup_s, gate=None):
         o.backward(g)
     torch.cuda.synchronize()
     bf16_both_ms = (time.perf_counter() - t0) * 1e3 / steps
+    graph.one_launch = True   # one launch for the local elements and the received bf16 rows
+    for _ in range(2):
+        Aggregator.apply(graph, xr, 0, 16, True, True).backward(g)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        o = Aggregator.apply(graph, xr, 0, 16, True, True)
+        o.backward(g)
+    torch.cuda.synchronize()
+    bf16_one_launch_ms = (time.perf_counter() - t0) * 1e3 / steps
+    graph.one_launch = False
     # ... and with the two tensor copies around the exchange as passes of their own (the reference's form)
     graph.fuse_bf16_staging = False
     for _ in range(2):
@@ -1034,6 +1058,8 @@ def run_c4(args, graph, setup_s, gate=None):
             "aggregator_forward_backward_ms_bf16_exchange": round(bf16_both_ms, 3),
             "aggregator_forward_backward_ms_bf16_exchange_separate_copies": round(bf16_unfused_ms, 3),
             "aggregator_forward_backward_ms_int2_exchange": round(int2_fused_ms, 3),
+            "aggregator_forward_backward_ms_int2_exchange_one_launch": round(int2_one_launch_ms, 3),
+            "aggregator_forward_backward_ms_bf16_exchange_one_launch": round(bf16_one_launch_ms, 3),
             "aggregator_forward_backward_ms_int2_exchange_separate_codec_passes": round(int2_both_ms, 3)}
 
 
@@ -1357,7 +1383,8 @@ def run_c5(args, graph):
     # exchange at `--num_bits=2`); the rows a peer would have sent stand ready on the device
     world = len(graph.comm_splits.send_splits)
     fp32_splits, fp32_buf = graph.comm_splits, graph.comm_buf
-    for bits in (16, 2):
+    for bits, one_launch in ((16, False), (2, False), (2, True)):
+        graph.one_launch = one_launch
         if bits == 16:
             graph.comm_buf = CommBuffer(fp32_splits, max(dims), 16, device=dev)
             synthetic.PregeneratedHaloExchange.attach(graph)
@@ -1375,10 +1402,12 @@ def run_c5(args, graph):
         for _ in range(steps):
             loss = gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks)
         torch.cuda.synchronize()
-        tag = "fp32_gemm_bf16_exchange" if bits == 16 else "fp32_gemm_int2_exchange"
+        tag = ("fp32_gemm_bf16_exchange" if bits == 16 else "fp32_gemm_int2_exchange") + (
+            "_one_launch_aggregation" if one_launch else "")
         out[f"train_step_ms_{tag}"] = round((time.perf_counter() - t0) * 1e3 / steps, 2)
         out[f"loss_{tag}"] = [round(v, 5) for v in losses + [float(loss)]]
         del model, opt
+        graph.one_launch = False
         graph.comm_splits, graph.comm_buf = fp32_splits, fp32_buf
         graph.exchange_bf16 = graph.exchange_quantized = graph.comm_buf_for_quantization = None
         torch.cuda.empty_cache()
@@ -1471,7 +1500,9 @@ def run_c5_sage(args, graph):
 
     world = len(graph.comm_splits.send_splits)
     fp32_splits, fp32_buf = folded.comm_splits, folded.comm_buf
-    for tag, bits in (("_folded_degrees_bf16_exchange", 16), ("_folded_degrees_int2_exchange", 2)):
+    for tag, bits in (("_folded_degrees_bf16_exchange", 16), ("_folded_degrees_int2_exchange", 2),
+                      ("_folded_degrees_int2_exchange_one_launch_aggregation", 2)):
+        folded.one_launch = tag.endswith("one_launch_aggregation")
         if bits == 16:
             folded.comm_buf = CommBuffer(fp32_splits, hidden, 16, device=dev)
             synthetic.PregeneratedHaloExchange.attach(folded)
@@ -1487,6 +1518,7 @@ def run_c5_sage(args, graph):
         ms, losses = timed(lambda: sage.train_step(model, opt, folded, staged, labels, train_idx, masks, True))
         out["train_step_ms" + tag], out["loss" + tag] = ms, losses
         del model, opt
+        folded.one_launch = False
         folded.comm_splits, folded.comm_buf = fp32_splits, fp32_buf
         folded.exchange_bf16 = folded.exchange_quantized = folded.comm_buf_for_quantization = None
         torch.cuda.empty_cache()
@@ -1599,7 +1631,8 @@ def main():
             targets["c5_gcn_train_step_ms"] = {k[len("train_step_ms_"):]: c5[k] for k in (
                 "train_step_ms_fp32_gemm", "train_step_ms_bf16_gemm", "train_step_ms_bf16x3_gemm",
                 "train_step_ms_fp32_gemm_one_launch_aggregation",
-                "train_step_ms_fp32_gemm_all_nodes_through_last_layer", "train_step_ms_fp32_gemm_int2_exchange")
+                "train_step_ms_fp32_gemm_all_nodes_through_last_layer", "train_step_ms_fp32_gemm_int2_exchange",
+                "train_step_ms_fp32_gemm_int2_exchange_one_launch_aggregation")
                 if k in c5}
             targets["c5_gcn_train_step_ms"]["library_products"] = c5.get("library_products_per_step")
             torch.cuda.empty_cache()
@@ -1609,6 +1642,7 @@ def main():
                 (k[len("train_step_ms_"):] if len(k) > len("train_step_ms") else "default"): c5s[k] for k in (
                     "train_step_ms", "train_step_ms_folded_degrees", "train_step_ms_folded_degrees_one_launch_aggregation",
                     "train_step_ms_folded_degrees_int2_exchange",
+                    "train_step_ms_folded_degrees_int2_exchange_one_launch_aggregation",
                     "train_step_ms_torch_ops_around_aggregator") if k in c5s}
     line["parity"] = gate.report()
     line["targets"] = targets

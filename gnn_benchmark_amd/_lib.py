@@ -12,7 +12,7 @@ _CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(_CSRC, "libgnnagg.so")
 
 OK, ERR_INVALID, ERR_HIP, ERR_UNSUPPORTED = 0, 1, 2, 3
-ABI_VERSION = 3   # GNNAGG_ABI_VERSION of include/gnn_agg.h this binding was written against
+ABI_VERSION = 4   # GNNAGG_ABI_VERSION of include/gnn_agg.h this binding was written against
 
 EXPORTS = (
     "gnnagg_abi_version",
@@ -25,6 +25,8 @@ EXPORTS = (
     "gnnagg_plan_spmm_f32",
     "gnnagg_plan_spmm_strided_f32",
     "gnnagg_plan_spmm_two_sources_f32",
+    "gnnagg_plan_spmm_dense_then_bf16_f32",
+    "gnnagg_plan_spmm_dense_then_quantized_f32",
     "gnnagg_plan_info",
     "gnnagg_plan_profile",
     "gnnagg_plan_profile_read",
@@ -131,6 +133,10 @@ def lib() -> ctypes.CDLL:
     L.gnnagg_plan_spmm_strided_f32.argtypes = [vp, vp, vp, i64, vp, i64, i64, i32, vp]
     L.gnnagg_plan_spmm_two_sources_f32.restype = i32
     L.gnnagg_plan_spmm_two_sources_f32.argtypes = [vp, vp, vp, i64, i64, vp, i64, vp, i64, i64, i32, vp]
+    L.gnnagg_plan_spmm_dense_then_bf16_f32.restype = i32
+    L.gnnagg_plan_spmm_dense_then_bf16_f32.argtypes = [vp, vp, vp, vp, i64, i64, vp, i64, vp, i64, i64, i32, vp]
+    L.gnnagg_plan_spmm_dense_then_quantized_f32.restype = i32
+    L.gnnagg_plan_spmm_dense_then_quantized_f32.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp, vp, i32, vp, i64, i64, i32, vp]
     L.gnnagg_plan_info.restype = i32
     L.gnnagg_plan_info.argtypes = [vp, ctypes.POINTER(i64)]
     L.gnnagg_plan_profile.restype = i32

@@ -47,8 +47,9 @@ What differs from the reference, on purpose:
   received ones, the order of aggregator.py:70 then :102 -- written once, instead of written by
   the local product and read and written again behind the exchange.  Same bits, fewer bytes;
   the price is that the local product no longer runs while the exchange is in flight, so it
-  pays where the exchange is short next to the local product.  fp32 boundary rows and dense
-  features only; every other case runs the separate launches.
+  pays where the exchange is short next to the local product.  Received rows are read in the
+  format they arrived in (fp32, bf16, packed); dense features only (packed features and the
+  row-restricted backward run the separate launches).
 
 ``AggregatorPacked`` is the same pipeline for local features handed over packed
 (``packed.py``: non-zero values at the front of each row plus a bitmap header); only the
@@ -230,6 +231,38 @@ def _dequantize_received(graph, num_bits: int, direction: str) -> None:
         computation_ops.dequantize_tensor_for_all_procs(data, incoming, params, work_range, world, num_bits)
 
 
+def _kernel_rows(t: torch.Tensor) -> bool:
+    """fp32 rows as the two-format launches take them: 16-byte aligned, row stride a multiple of 4 floats."""
+    return t.data_ptr() % 16 == 0 and (t.size(0) <= 1 or t.stride(0) % 4 == 0)
+
+
+def _one_launch_product(graph, both: SparseTensor, dense: torch.Tensor, result: torch.Tensor, accumulate: bool,
+                        num_bits: int, direction: str, quantized: bool, half: bool, half_fused: bool, feat_len: int):
+    """``result (+)= both @ (dense ; received rows)`` in one launch (``graph.one_launch``), the received rows read in
+    the format they arrived in -- fp32, bf16 or packed -- where the products read exchange formats themselves
+    (``fuse_dequantize`` / ``fuse_bf16_staging``), after the reference's dequantise / copy pass otherwise."""
+    buf, qbuf = graph.comm_buf, graph.comm_buf_for_quantization if quantized else None
+    plan, value = both.get_plan(), both.csr()[2]
+    formats_ok = feat_len % 4 == 0 and _kernel_rows(dense) and _kernel_rows(result)
+    if quantized:
+        if _fused_dequantize(graph, feat_len) and formats_ok:
+            _poison_unfilled_rows(graph)
+            if direction == "forward":
+                second = (qbuf.quantized_recv_data_buf, qbuf.quantized_recv_params_buf_fp32, qbuf.recv_row_code, num_bits)
+            else:
+                second = (qbuf.quantized_send_data_buf, qbuf.quantized_send_params_buf_fp32, qbuf.send_row_code, num_bits)
+            plan.spmm_dense_then(value, both.first_counts, dense, second, result, accumulate)
+            return
+        _dequantize_received(graph, num_bits, direction)
+    elif half:
+        rows16 = buf.recv_buf_fp16 if direction == "forward" else buf.send_buf_fp16
+        if half_fused and formats_ok:
+            plan.spmm_dense_then(value, both.first_counts, dense, rows16, result, accumulate)
+            return
+        _convert(rows16, buf.recv_buf if direction == "forward" else buf.send_buf)
+    plan.spmm_two_sources(value, dense, buf.recv_buf if direction == "forward" else buf.send_buf, result, accumulate)
+
+
 class _DenseFeatures:
     """The local features as the forward pipeline reads them: two products and a row gather."""
 
@@ -349,14 +382,15 @@ def _forward(ctx, graph, feats, layer, num_bits: int, is_pre_delay: bool, is_tra
     remote_adj = None
     if exchange is not None:
         remote_adj = graph.adj_t_pre_post_aggr_from if is_pre_delay else graph.remote_adj_t
-    one_launch = (getattr(graph, "one_launch", False) is True and remote_adj is not None and not quantized and not half
+    one_launch = (getattr(graph, "one_launch", False) is True and remote_adj is not None
                   and isinstance(feats, _DenseFeatures) and feats.feat.dtype == torch.float32
                   and graph.comm_buf.recv_buf.size(0) != 0)
     if one_launch:  # local elements, then received ones: one chain per output row, one launch
         if comm_handle is not None:
             comm_handle.wait()
         both = side_by_side(graph.local_adj_t, remote_adj)
-        both.get_plan().spmm_two_sources(both.csr()[2], feats.feat, graph.comm_buf.recv_buf, out, accumulate)
+        _one_launch_product(graph, both, feats.feat, out, accumulate, num_bits, "forward", quantized,
+                            half, half_fused, feat_len)
         return out
     feats.product(graph.local_adj_t, out, accumulate)
 
@@ -548,8 +582,7 @@ def _backward(ctx, local_out_grad, out=None, accumulate: bool = False):
         _check_result(out, graph.local_adj_t.sparse_size(-1), feat_len, local_out_grad.device)
         local_nodes_grad = out
     one_launch = (getattr(graph, "one_launch", False) is True and exchange is not None and support is None
-                  and not quantized and not half and local_out_grad.dtype == torch.float32
-                  and graph.comm_buf.send_buf.size(0) != 0)
+                  and local_out_grad.dtype == torch.float32 and graph.comm_buf.send_buf.size(0) != 0)
     if one_launch:  # [A_local^T | A_to^T] over the gradient and the received gradient rows, one chain per row
         if comm_handle is not None:
             comm_handle.wait()
@@ -557,8 +590,8 @@ def _backward(ctx, local_out_grad, out=None, accumulate: bool = False):
             both = side_by_side(graph.local_adj_t, graph.adj_t_pre_post_aggr_to, transposed=True)
         else:  # local^T next to the selection matrix of the boundary row list (itself untransposed)
             both = side_by_side(_transposed_matrix(graph.local_adj_t), graph.send_scatter_adj_t())
-        both.get_plan().spmm_two_sources(both.csr()[2], local_out_grad, graph.comm_buf.send_buf, local_nodes_grad,
-                                         accumulate)
+        _one_launch_product(graph, both, local_out_grad, local_nodes_grad, accumulate, num_bits, "backward", quantized,
+                            half, half_fused, feat_len)
         return local_nodes_grad
     if support is not None:
         SPMM_forward(support.local_T, local_out_grad, local_nodes_grad, accumulate=accumulate)

@@ -744,6 +744,85 @@ extern "C" int gnnagg_plan_spmm_two_sources_f32(gnnagg_plan *plan, const float *
     return GNNAGG_OK;
 }
 
+// Local elements from dense fp32 rows, the rest of every row from a second source still in its exchange format.
+static int plan_spmm_dense_then(gnnagg_plan *plan, const float *value, const int32_t *split, const float *mat,
+                                int64_t mat_stride, int64_t mat_rows, const void *rows16, int64_t rows16_stride,
+                                const uint8_t *packed, const float *params, const int32_t *row_code, int bits, float *out,
+                                int64_t out_stride, int64_t feat, int accumulate, void *stream) {
+    GNNAGG_REQUIRE(plan, "null plan");
+    GNNAGG_REQUIRE(feat >= 0, "negative feature width");
+    GNNAGG_REQUIRE(mat_rows >= 0 && mat_rows <= plan->cols, "the first source holds %lld rows, the matrix has %lld columns",
+                   (long long)mat_rows, (long long)plan->cols);
+    if (plan->rows == 0 || feat == 0) return GNNAGG_OK;
+    if (int rc = check_feat(feat)) return rc;
+    if (feat % 4 != 0)
+        return fail(GNNAGG_ERR_UNSUPPORTED, "rows in an exchange format need a width that is a multiple of 4 (got %lld)",
+                    (long long)feat);
+    GNNAGG_REQUIRE(out && split, "null out/split");
+    const bool quant = packed != nullptr;
+    GNNAGG_REQUIRE(plan->nnz == 0 || (value && mat && (quant ? (params && row_code) : rows16 != nullptr)),
+                   "null value/mat/second source");
+    if (quant) GNNAGG_REQUIRE(bits == 2 || bits == 4 || bits == 8, "bits must be 2, 4 or 8 (got %d)", bits);
+    GNNAGG_REQUIRE(mat_stride >= feat && mat_stride % 4 == 0 && mat_stride < (int64_t(1) << 31) && out_stride >= feat &&
+                       out_stride % 4 == 0 && out_stride < (int64_t(1) << 31) &&
+                       (quant || (rows16_stride >= feat && rows16_stride % 4 == 0 && rows16_stride < (int64_t(1) << 31))),
+                   "row strides must be multiples of 4, at least the width and below 2^31");
+    GNNAGG_REQUIRE((reinterpret_cast<uintptr_t>(mat) & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0 &&
+                       (reinterpret_cast<uintptr_t>(rows16) & 7) == 0 && (reinterpret_cast<uintptr_t>(packed) & 3) == 0 &&
+                       (reinterpret_cast<uintptr_t>(params) & 7) == 0,
+                   "fp32 rows must be 16-byte aligned, bf16 rows and parameters 8-byte aligned, packed bytes 4-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const Regions regions{plan->rows_per_group, plan->short_rows_per_group,
+                          plan->nshort + (accumulate ? 0 : plan->nempty)};
+    for (int64_t f_base = 0; f_base < feat;) {
+        const Shape s = pick_shape(4, feat - f_base);
+        SpmmArgs a{};
+        a.task = plan->task;  // every row runs in the lane-group kernel, the very longest included
+        a.col = plan->col32;
+        a.val = value;
+        a.split = split;
+        a.x = mat;
+        a.ldx = (int)mat_stride;
+        a.x_rows = (int)mat_rows;
+        a.x2 = static_cast<const float *>(rows16);
+        a.ldx2 = (int)rows16_stride;
+        a.qdata = packed;
+        a.qparams = params;
+        a.qcode = row_code;
+        a.qbits = bits;
+        a.dst = out;
+        a.ldd = (int)out_stride;
+        a.feat = (int)feat;
+        a.f_base = (int)f_base;
+        a.accumulate = accumulate;
+        a.ntasks = plan->rows - (accumulate ? plan->nempty : 0);
+        a.head_tasks = plan->nlong;
+        if (quant) GNNAGG_HIP((dispatch_shape<4, int32_t, kRowsPlanned, kSrcDenseThenQuant>(s, a, regions, st)));
+        else GNNAGG_HIP((dispatch_shape<4, int32_t, kRowsPlanned, kSrcDenseThenBf16>(s, a, regions, st)));
+        f_base += s.width();
+    }
+    return GNNAGG_OK;
+}
+
+extern "C" int gnnagg_plan_spmm_dense_then_bf16_f32(gnnagg_plan *plan, const float *value, const int32_t *split,
+                                                    const float *mat, int64_t mat_stride, int64_t mat_rows,
+                                                    const uint16_t *mat2_bf16, int64_t mat2_stride, float *out,
+                                                    int64_t out_stride, int64_t feat, int accumulate, void *stream) {
+    GNNAGG_REQUIRE(plan == nullptr || plan->nnz == 0 || mat2_bf16, "null mat2_bf16");
+    return plan_spmm_dense_then(plan, value, split, mat, mat_stride, mat_rows, mat2_bf16, mat2_stride, nullptr, nullptr,
+                                nullptr, 0, out, out_stride, feat, accumulate, stream);
+}
+
+extern "C" int gnnagg_plan_spmm_dense_then_quantized_f32(gnnagg_plan *plan, const float *value, const int32_t *split,
+                                                         const float *mat, int64_t mat_stride, int64_t mat_rows,
+                                                         const uint8_t *packed, const float *params,
+                                                         const int32_t *row_code, int bits, float *out,
+                                                         int64_t out_stride, int64_t feat, int accumulate, void *stream) {
+    GNNAGG_REQUIRE(plan == nullptr || plan->nnz == 0 || packed, "null packed");
+    return plan_spmm_dense_then(plan, value, split, mat, mat_stride, mat_rows, nullptr, feat, packed, params, row_code,
+                                bits, out, out_stride, feat, accumulate, stream);
+}
+
 extern "C" int gnnagg_plan_spmm_packed_f32(gnnagg_plan *plan, const float *value, const float *y_packed,
                                            const uint32_t *header, float *out, int64_t feat, int accumulate,
                                            void *stream) {

@@ -160,6 +160,10 @@ struct SpmmArgs {
     // two dense sources (kSrcDense2): columns [0, x_rows) are rows of x, columns x_rows + k are rows k of x2
     const float *x2;
     int x_rows, ldx2;         // ldx2: row stride of x2 in floats; 0 stands for F
+    // a dense fp32 source followed by a second source in its exchange format (kSrcDenseThenBf16: x2 points at bf16
+    // rows, ldx2 counts 16-bit values; kSrcDenseThenQuant: qdata / qparams / qcode): the first split[row] stored
+    // elements of a row read x, the rest read row (column - x_rows) of the second source
+    const int32_t *split;     // [rows]
     const uint32_t *hdr;      // packed source only: [K, hdr_words] row headers
     int hdr_words;
     // quantised source only (row-packed codec of the boundary buffers): byte rows [packed_rows, F] in
@@ -199,7 +203,10 @@ enum SourceKind : int {
     kSrcPacked = 1,  // x[col, :] holds the row's non-zero values at its front, hdr[col, :] says which
     kSrcQuant = 2,   // row col is held quantised: qdata / qparams / qcode (boundary-buffer codec layout)
     kSrcBf16 = 3,    // x[col, :] is a bf16 row (x points at 16-bit values, ldx counts them): widened in the gather
-    kSrcDense2 = 4   // dense fp32 rows of two arrays: x[col, :] for col < x_rows, x2[col - x_rows, :] above
+    kSrcDense2 = 4,  // dense fp32 rows of two arrays: x[col, :] for col < x_rows, x2[col - x_rows, :] above
+    // the first split[row] elements of a row gather dense fp32 rows of x, the others rows of a second source:
+    kSrcDenseThenBf16 = 5,   // ... bf16 rows (x2)
+    kSrcDenseThenQuant = 6   // ... quantised rows (qdata / qparams / qcode)
 };
 
 typedef float f32x4_unaligned __attribute__((ext_vector_type(4), aligned(4)));
@@ -244,18 +251,25 @@ __device__ __forceinline__ FVec<4> expand_packed(uint32_t nib, const f32x4_unali
 // instead of a cascade of ever shorter dependent ones; the lanes past the row's end hold column 0 with value 0, so the
 // surplus gathers read row 0 of x (a valid, hot address) -- and only the first `valid` results enter the chain (selected,
 // not multiplied by zero: row 0 of x may hold anything).
-template <int UU, int VEC, int LPR, int NCH, int SRC, typename IdxT, bool TAIL = false>
+// SECOND: the elements belong to the second source of a two-format launch (x2 / ldx2, or the quantised buffers):
+// their column counts from x_rows.  CLAMP: the surplus gathers of a TAIL round must not use what the lanes behind the
+// stretch hold (elements of the other source, whose columns mean something else): they read row 0.
+template <int UU, int VEC, int LPR, int NCH, int SRC, typename IdxT, bool TAIL = false, bool SECOND = false, bool CLAMP = false>
 __device__ __forceinline__ void gather_fma(FVec<VEC> (&acc)[NCH], IdxT c_l, float v_l, int j, const SpmmArgs &a,
                                            const int (&foff)[NCH], int valid = UU) {
-    const float *__restrict__ x = a.x;
+    const float *__restrict__ x = SECOND ? a.x2 : a.x;
     const int F = a.feat;
-    const int ldx = a.ldx ? a.ldx : F;
+    const int ldx = SECOND ? (a.ldx2 ? a.ldx2 : F) : (a.ldx ? a.ldx : F);
     const float *xr[UU];
     float vv[UU];
     int64_t cc[UU];
 #pragma unroll
     for (int u = 0; u < UU; ++u) {
         cc[u] = group_bcast_idx<LPR>(c_l, j + u);
+        if constexpr (SECOND) cc[u] -= (int64_t)a.x_rows;
+        if constexpr (TAIL && CLAMP) {
+            if (u >= valid) cc[u] = 0;
+        }
         vv[u] = __int_as_float(group_bcast<LPR>(__float_as_int(v_l), j + u));
         if constexpr (SRC == kSrcDense2) {
             const bool second = cc[u] >= (int64_t)a.x_rows;
@@ -384,10 +398,33 @@ struct UnrollFor {
 
 constexpr int kMaxRowsPerGroup = 16;  // a group's task descriptors live one per lane
 
+// Elements [j0, j1) of the chunk held in (c_l, v_l): full blocks of U gathers, then ONE more round for what is left
+// (the smallest power of two of gathers that covers it, the surplus ones masked): ceil((j1 - j0) / U) dependent
+// round trips.
+template <int VEC, int LPR, int NCH, int SRC, typename IdxT, bool SECOND = false, bool CLAMP = false>
+__device__ __forceinline__ void gather_rounds(FVec<VEC> (&acc)[NCH], IdxT c_l, float v_l, int j0, int j1,
+                                              const SpmmArgs &a, const int (&foff)[NCH]) {
+    constexpr int U = UnrollFor<VEC, NCH>::value;
+    int j = j0;
+    for (; j + U <= j1; j += U) gather_fma<U, VEC, LPR, NCH, SRC, IdxT, false, SECOND, CLAMP>(acc, c_l, v_l, j, a, foff);
+    const int rem = j1 - j;
+    if (rem > 0) {
+        if constexpr (U > 4) {
+            if (rem > 4) gather_fma<8, VEC, LPR, NCH, SRC, IdxT, true, SECOND, CLAMP>(acc, c_l, v_l, j, a, foff, rem);
+        }
+        if constexpr (U > 2) {
+            if (rem > 2 && rem <= 4) gather_fma<4, VEC, LPR, NCH, SRC, IdxT, true, SECOND, CLAMP>(acc, c_l, v_l, j, a, foff, rem);
+        }
+        if constexpr (U > 1) {
+            if (rem == 2) gather_fma<2, VEC, LPR, NCH, SRC, IdxT, false, SECOND, CLAMP>(acc, c_l, v_l, j, a, foff);
+        }
+        if (rem == 1) gather_fma<1, VEC, LPR, NCH, SRC, IdxT, false, SECOND, CLAMP>(acc, c_l, v_l, j, a, foff);
+    }
+}
+
 template <int VEC, int LPR, int NCH, typename IdxT, int MODE, int SRC = kSrcDense>
 __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
     constexpr int GPB = 256 / LPR;  // groups per 256-thread block
-    constexpr int U = UnrollFor<VEC, NCH>::value;
     typedef FVec<VEC> V;
 
     const int lane = (int)threadIdx.x & 63;
@@ -455,6 +492,7 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
     // One coalesced fetch brings every descriptor of the group: lane i holds task i.
     int d_row = 0, d_len = 0;
     int64_t d_start = 0;
+    int d_split = 0;  // two-format launches: the row's leading elements that read the dense source
     // kRowsNatural: the group's lanes whose row is still to be done (a planned launch walks lanes 0 .. ntask-1)
     uint64_t todo = 0;
     if (!scanner && lig < ntask) {
@@ -464,6 +502,7 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
             d_row = d.row;
             d_len = d.len;
             d_start = d.start;
+            if constexpr (SRC == kSrcDenseThenBf16 || SRC == kSrcDenseThenQuant) d_split = a.split[d.row];
         } else {
             d_row = (int)t;
             d_start = a.rowptr[t];
@@ -513,6 +552,8 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
         int row = group_bcast<LPR>(d_row, i);
         int64_t base = group_bcast_idx<LPR>(d_start, i);
         int64_t end = base + group_bcast<LPR>(d_len, i);
+        int64_t first_end = base;  // (two-format launches) where the row's elements of the second source begin
+        if constexpr (SRC == kSrcDenseThenBf16 || SRC == kSrcDenseThenQuant) first_end = base + group_bcast<LPR>(d_split, i);
         IdxT c_l = 0;
         float v_l = 0.0f;
         if (base + lig < end) {
@@ -534,7 +575,7 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
             // where the next chunk comes from
             int ni = i;
             int nrow = row;
-            int64_t nbase = base + LPR, nend = end;
+            int64_t nbase = base + LPR, nend = end, nfirst_end = first_end;
             bool row_done = nbase >= end;
             bool more = true;
             if (row_done) {
@@ -552,6 +593,8 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
                     nrow = group_bcast<LPR>(d_row, ni);
                     nbase = group_bcast_idx<LPR>(d_start, ni);
                     nend = nbase + group_bcast<LPR>(d_len, ni);
+                    if constexpr (SRC == kSrcDenseThenBf16 || SRC == kSrcDenseThenQuant)
+                        nfirst_end = nbase + group_bcast<LPR>(d_split, ni);
                 }
             }
             IdxT nc = 0;
@@ -561,22 +604,15 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
                 nv = __builtin_nontemporal_load(val + nbase + lig);
             }
 
-            // full blocks of U gathers, then ONE more round for what is left (the smallest power of two of gathers
-            // that covers it, the surplus ones masked): a chunk of cnt elements costs ceil(cnt / U) dependent round trips
-            int j = 0;
-            for (; j + U <= cnt; j += U) gather_fma<U, VEC, LPR, NCH, SRC>(acc, c_l, v_l, j, a, foff);
-            const int rem = cnt - j;
-            if (rem > 0) {
-                if constexpr (U > 4) {
-                    if (rem > 4) gather_fma<8, VEC, LPR, NCH, SRC, IdxT, true>(acc, c_l, v_l, j, a, foff, rem);
-                }
-                if constexpr (U > 2) {
-                    if (rem > 2 && rem <= 4) gather_fma<4, VEC, LPR, NCH, SRC, IdxT, true>(acc, c_l, v_l, j, a, foff, rem);
-                }
-                if constexpr (U > 1) {
-                    if (rem == 2) gather_fma<2, VEC, LPR, NCH, SRC, IdxT, false>(acc, c_l, v_l, j, a, foff);
-                }
-                if (rem == 1) gather_fma<1, VEC, LPR, NCH, SRC, IdxT, false>(acc, c_l, v_l, j, a, foff);
+            if constexpr (SRC == kSrcDenseThenBf16 || SRC == kSrcDenseThenQuant) {
+                // the chunk's elements in front of the row's split read the dense source, the others the second one
+                const int64_t ahead = first_end - base;
+                const int cnt_a = ahead <= 0 ? 0 : (ahead < cnt ? (int)ahead : cnt);
+                gather_rounds<VEC, LPR, NCH, kSrcDense, IdxT, false, true>(acc, c_l, v_l, 0, cnt_a, a, foff);
+                gather_rounds<VEC, LPR, NCH, SRC == kSrcDenseThenBf16 ? kSrcBf16 : kSrcQuant, IdxT, true, true>(
+                    acc, c_l, v_l, cnt_a, cnt, a, foff);
+            } else {
+                gather_rounds<VEC, LPR, NCH, SRC, IdxT>(acc, c_l, v_l, 0, cnt, a, foff);
             }
 
             if (row_done) {
@@ -617,6 +653,7 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
             row = nrow;
             base = nbase;
             end = nend;
+            first_end = nfirst_end;
             c_l = nc;
             v_l = nv;
         }

@@ -121,6 +121,48 @@ class SpmmPlan:
                 _lib.current_stream(self.device)))
         return out
 
+    def spmm_dense_then(self, value: torch.Tensor, split: torch.Tensor, mat: torch.Tensor, second, out: torch.Tensor,
+                        accumulate: bool = True) -> torch.Tensor:
+        """``out (+)= A @ [mat ; second]`` where the rows of the second operand are still in an exchange format: the
+        first ``split[r]`` stored elements of row r gather float32 rows of ``mat`` (columns below ``mat.size(0)``), the
+        others rows of ``second`` -- a bfloat16 ``[rows, F]`` tensor, or a tuple ``(packed uint8 [packed rows, F],
+        params float32 [rows, 2], row_code int32 [rows], bits)`` as ``SPMM_forward_quantized`` takes them."""
+        if not all(t.is_cuda for t in (value, split, mat, out)):
+            raise RuntimeError("value, split, mat and out must be GPU (HIP) tensors; there is no CPU path")
+        feat = out.size(1) if out.dim() == 2 else -1
+        if (value.dtype != torch.float32 or mat.dtype != torch.float32 or out.dtype != torch.float32
+                or split.dtype != torch.int32 or not split.is_contiguous() or split.numel() != self.rows
+                or not _rows_are_dense(mat) or not _rows_are_dense(out) or mat.size(1) != feat
+                or value.numel() != self.nnz or out.size(0) < self.rows or mat.size(0) > self.cols):
+            raise RuntimeError("Input mismatch: value/mat/out must be float32 with contiguous rows, split int32 [rows], "
+                               "shapes matching the planned matrix")
+        second_rows = self.cols - mat.size(0)
+        L = _lib.lib()
+        with torch.cuda.device(self.device):
+            if isinstance(second, torch.Tensor):
+                if (second.dtype != torch.bfloat16 or not second.is_cuda or not _rows_are_dense(second)
+                        or second.size(0) < second_rows or second.size(1) != feat):
+                    raise RuntimeError("Input mismatch: the second source must be bfloat16 [rows, F] with contiguous rows")
+                _lib.check(L.gnnagg_plan_spmm_dense_then_bf16_f32(
+                    self._handle, _lib.ptr(value.contiguous()), _lib.ptr(split), _lib.ptr(mat), _row_stride(mat),
+                    mat.size(0), _lib.ptr(second), _row_stride(second), _lib.ptr(out), _row_stride(out), feat,
+                    1 if accumulate else 0, _lib.current_stream(self.device)))
+            else:
+                packed, params, row_code, bits = second
+                if (packed.dtype != torch.uint8 or not packed.is_contiguous() or packed.dim() != 2 or packed.size(1) != feat
+                        or params.dtype != torch.float32 or not params.is_contiguous() or params.dim() != 2
+                        or params.size(0) < second_rows or params.size(1) != 2 or row_code.dtype != torch.int32
+                        or not row_code.is_contiguous() or row_code.numel() < second_rows
+                        or not all(t.is_cuda for t in (packed, params, row_code))):
+                    raise RuntimeError("Input mismatch: quantised second source needs uint8 [packed rows, F] bytes, "
+                                       "float32 [rows, 2] parameters and int32 [rows] row codes on the GPU")
+                _lib.check_index(row_code, packed.size(0), shift=3, what="row codes of the packed buffer")
+                _lib.check(L.gnnagg_plan_spmm_dense_then_quantized_f32(
+                    self._handle, _lib.ptr(value.contiguous()), _lib.ptr(split), _lib.ptr(mat), _row_stride(mat),
+                    mat.size(0), _lib.ptr(packed), _lib.ptr(params), _lib.ptr(row_code), int(bits), _lib.ptr(out),
+                    _row_stride(out), feat, 1 if accumulate else 0, _lib.current_stream(self.device)))
+        return out
+
     def _spmm_bf16(self, value, mat, out, accumulate):
         """The product with bf16 rows on either side (the staging buffers of a 16-bit exchange): a bf16 ``mat`` is
         widened in the gather, a bf16 ``out`` receives the fp32 sums rounded to nearest even -- the same bits as the
@@ -393,6 +435,9 @@ def side_by_side(left: SparseTensor, right: SparseTensor, transposed: bool = Fal
                               col=torch.cat([parts[0][1], parts[1][1] + left_cols]),
                               value=torch.cat([parts[0][2], parts[1][2]]), sparse_sizes=(rows, left_cols + right_cols))
         merged.first_source_rows = left_cols
+        # per row: how many of its leading stored elements come from `left`
+        ptr = left.storage.colptr() if transposed else left.csr()[0]
+        merged.first_counts = (ptr[1:] - ptr[:-1]).to(torch.int32).contiguous()
         if len(cache) >= 4:
             cache.clear()
         hit = cache[key] = (right, merged)   # holding `right` keeps its id its own

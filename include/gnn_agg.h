@@ -28,9 +28,9 @@ extern "C" {
 
 /* Raised whenever an exported prototype changes, an entry point goes away or the meaning of an argument changes
  * (2: `src_rows` in the row gathers, `workspace_bytes` in the weight-gradient entry points, 12 values from
- * gnnagg_plan_info; 3: the measurement probes left the library, gnnagg_plan_spmm_two_sources_f32 and gnnagg_plans_release came).  Every binding compares it with
+ * gnnagg_plan_info; 3: the measurement probes left the library, gnnagg_plan_spmm_two_sources_f32 and gnnagg_plans_release came; 4: the two gnnagg_plan_spmm_dense_then_* entry points came).  Every binding compares it with
  * gnnagg_abi_version() of the library it loaded before the first call. */
-#define GNNAGG_ABI_VERSION 3
+#define GNNAGG_ABI_VERSION 4
 
 /* Version of this ABI (GNNAGG_ABI_VERSION of the built library).  No reference counterpart. */
 int gnnagg_abi_version(void);
@@ -152,6 +152,25 @@ int gnnagg_plan_spmm_strided_f32(gnnagg_plan *plan, const float *value, const fl
 int gnnagg_plan_spmm_two_sources_f32(gnnagg_plan *plan, const float *value, const float *mat, int64_t mat_stride,
                                      int64_t mat_rows, const float *mat2, int64_t mat2_stride, float *out,
                                      int64_t out_stride, int64_t feat, int accumulate, void *stream);
+
+/* The one-launch product when the received rows are still in their exchange format (a 16-bit or quantised
+ * exchange): the plan is over [A_local | A_from] as above, `split` int32 [rows] says how many of a row's leading
+ * stored elements belong to A_local; those gather fp32 rows of mat, the others rows (column - mat_rows) of the
+ * second source -- bf16 rows (mat2_bf16, stride in 16-bit values; what gnnagg_plan_spmm_bf16_f32 gathers), or the
+ * packed bytes / parameters / row codes gnnagg_plan_spmm_quantized_f32 gathers.  Every output row is the FMA chain
+ * of the local product continued by the one of the product from the exchange format, hence the same bits as those
+ * two calls (model/layers/aggregator.py:70 then :85-104; backward :170 then :180-199).  feat a multiple of 4, fp32
+ * rows 16-byte aligned.  A matrix whose rows all have split == their length is a plain product.  Allocate nothing,
+ * no host synchronisation. */
+int gnnagg_plan_spmm_dense_then_bf16_f32(gnnagg_plan *plan, const float *value, const int32_t *split, const float *mat,
+                                         int64_t mat_stride, int64_t mat_rows, const uint16_t *mat2_bf16,
+                                         int64_t mat2_stride, float *out, int64_t out_stride, int64_t feat,
+                                         int accumulate, void *stream);
+int gnnagg_plan_spmm_dense_then_quantized_f32(gnnagg_plan *plan, const float *value, const int32_t *split,
+                                              const float *mat, int64_t mat_stride, int64_t mat_rows,
+                                              const uint8_t *packed, const float *params, const int32_t *row_code,
+                                              int bits, float *out, int64_t out_stride, int64_t feat, int accumulate,
+                                              void *stream);
 
 /* Host-side description of a plan, info[0..11] (host pointer):
  * rows, cols, nnz, rows handled by the block-per-row kernel (longer than the next

@@ -275,9 +275,10 @@ class PlayedQuantizedExchange:
         return None
 
 
+@pytest.mark.parametrize("one_launch", [False, True])
 @pytest.mark.parametrize("bits", [2, 4, 8])
 @pytest.mark.parametrize("seed,sizes", [(0, (300, 450, 250)), (1, (600, 1, 400, 330))])
-def test_quantised_exchange_world_matches_oracle(seed, sizes, bits):
+def test_quantised_exchange_world_matches_oracle(seed, sizes, bits, one_launch):
     """Pre/post-aggregation with the boundary rows travelling as packed int2 / int4 / int8: every
     rank's buffers, output and gradient are bit-identical to the oracle pipeline (oracle codec
     between oracle SpMMs), and the result stays within the codec's error of the exact product."""
@@ -286,6 +287,8 @@ def test_quantised_exchange_world_matches_oracle(seed, sizes, bits):
     w = World(seed, sizes, mean_deg=8.0)
     W, F = w.world, 48
     graphs = _build_pre_graphs(w, F, bits=bits)
+    for gr_ in graphs:   # local and received elements of every output row in one launch: the same bits
+        gr_.one_launch = one_launch
     oracle_ranks = build_pre_world(w)
     rng = np.random.default_rng(seed + 100)
     x = rng.standard_normal((w.n, F)).astype(np.float32)
@@ -430,9 +433,10 @@ class PlayedBf16Exchange:
         return None
 
 
+@pytest.mark.parametrize("one_launch", [False, True])
 @pytest.mark.parametrize("fused", [True, False])
 @pytest.mark.parametrize("seed,sizes", [(0, (300, 450, 250)), (1, (600, 1, 400, 330))])
-def test_bf16_exchange_world_matches_oracle(seed, sizes, fused):
+def test_bf16_exchange_world_matches_oracle(seed, sizes, fused, one_launch):
     """Boundary rows travelling as bf16 (num_bits=16, communicator.py:111-137): what every rank
     stages for sending equals the oracle's rows rounded to bf16 bit for bit, and output and gradient
     equal the oracle pipeline fed with the rounded rows -- with the two tensor copies around the exchange as passes
@@ -443,6 +447,8 @@ def test_bf16_exchange_world_matches_oracle(seed, sizes, fused):
     w = World(seed, sizes, mean_deg=8.0)
     W, F = w.world, 40
     graphs = _build_pre_graphs(w, F, bits=16)
+    for gr_ in graphs:   # local and received elements of every output row in one launch: the same bits
+        gr_.one_launch = one_launch
     oracle_ranks = build_pre_world(w)
     rng = np.random.default_rng(seed + 200)
     x = (rng.standard_normal((w.n, F)) * rng.uniform(1e-3, 1e3, (w.n, 1))).astype(np.float32)
@@ -497,9 +503,10 @@ def test_bf16_exchange_world_matches_oracle(seed, sizes, fused):
         Aggregator.apply(graphs[1], dev(x[sl[1]]), 0, 16, True, True)
 
 
+@pytest.mark.parametrize("one_launch", [False, True])
 @pytest.mark.parametrize("fused", [True, False])
 @pytest.mark.parametrize("seed,sizes", [(6, (300, 450, 250)), (7, (600, 1, 400, 330))])
-def test_raw_halo_bf16_exchange_matches_oracle(seed, sizes, fused):
+def test_raw_halo_bf16_exchange_matches_oracle(seed, sizes, fused, one_launch):
     """The raw-halo mode with 16-bit rows on the wire (aggregator.py:51 then communicator.py:111-137): the staged rows
     are the gathered boundary rows rounded to bf16, bit for bit, whether the gather writes them as bf16 itself (the
     default) or the tensor copy follows it; output and gradient equal the oracle pipeline fed with the rounded rows."""
@@ -508,6 +515,8 @@ def test_raw_halo_bf16_exchange_matches_oracle(seed, sizes, fused):
     w = World(seed, sizes, mean_deg=8.0)
     W, F = w.world, 40
     graphs = _build_raw_graphs(w, F, bits=16)
+    for gr_ in graphs:   # local and received elements of every output row in one launch: the same bits
+        gr_.one_launch = one_launch
     rng = np.random.default_rng(seed + 300)
     x = (rng.standard_normal((w.n, F)) * rng.uniform(1e-3, 1e3, (w.n, 1))).astype(np.float32)
     g = rng.standard_normal((w.n, F)).astype(np.float32)
@@ -542,9 +551,10 @@ def test_raw_halo_bf16_exchange_matches_oracle(seed, sizes, fused):
         assert_close(xr.grad, o_dx, "raw halo gradient vs oracle, bf16 rows")
 
 
+@pytest.mark.parametrize("one_launch", [False, True])
 @pytest.mark.parametrize("bits", [2, 8])
 @pytest.mark.parametrize("seed,sizes", [(8, (300, 450, 250)), (9, (600, 1, 400, 330))])
-def test_raw_halo_quantised_exchange_matches_oracle(seed, sizes, bits):
+def test_raw_halo_quantised_exchange_matches_oracle(seed, sizes, bits, one_launch):
     """The raw-halo mode with packed rows on the wire (aggregator.py:51, :83-88, :180-199): the bytes and parameters
     every rank sends equal the oracle codec's over the gathered rows / the outgoing gradient rows, output and gradient
     equal the oracle pipeline fed with what the peers' bytes decode to -- in the reference's form (gather, quantise,
@@ -555,6 +565,8 @@ def test_raw_halo_quantised_exchange_matches_oracle(seed, sizes, bits):
     w = World(seed, sizes, mean_deg=8.0)
     W, F = w.world, 40
     graphs = _build_raw_graphs(w, F, bits=bits)
+    for gr_ in graphs:   # local and received elements of every output row in one launch: the same bits
+        gr_.one_launch = one_launch
     rng = np.random.default_rng(seed + 400)
     x = (rng.standard_normal((w.n, F)) * rng.uniform(1e-2, 1e2, (w.n, 1))).astype(np.float32)
     g = rng.standard_normal((w.n, F)).astype(np.float32)

@@ -178,7 +178,9 @@ def test_boundary_rows_in_their_exchange_format_at_full_size(workload, bits):
             graph.exchange_quantized = synthetic.SeededQuantizedHaloExchange(22)
             options = ("fuse_quantize", "fuse_dequantize")
         seen = []
-        for fused in (True, False):
+        # the third pass: the default products again, local and received elements of every output row in one launch
+        for fused, one_launch in ((True, False), (False, False), (True, True)):
+            graph.one_launch = one_launch
             for name in options:
                 setattr(graph, name, fused)
             xr = x.clone().requires_grad_()
@@ -197,13 +199,15 @@ def test_boundary_rows_in_their_exchange_format_at_full_size(workload, bits):
                                   qb.quantized_recv_params_buf_fp32.reshape(-1).view(torch.uint8)])
             seen.append((out.detach(), xr.grad, sent, back))
             del xr, out
-        for a, b in zip(*seen):
-            if a.dtype == torch.bfloat16:
-                a, b = a.view(torch.int16), b.view(torch.int16)
-            elif a.dtype == torch.float32:
-                assert bool(torch.isfinite(a).all())
-            assert torch.equal(a, b)
+        for other in seen[1:]:
+            for a, b in zip(seen[0], other):
+                if a.dtype == torch.bfloat16:
+                    a, b = a.view(torch.int16), b.view(torch.int16)
+                elif a.dtype == torch.float32:
+                    assert bool(torch.isfinite(a).all())
+                assert torch.equal(a, b)
     finally:
+        graph.one_launch = False
         graph.comm_splits, graph.comm_buf = kept
         graph.exchange_bf16 = graph.exchange_quantized = graph.comm_buf_for_quantization = None
         for name in ("fuse_bf16_staging", "fuse_quantize", "fuse_dequantize"):
@@ -346,10 +350,13 @@ def test_sage_one_launch_aggregation_gives_the_same_step(sage_workload):
 
 def test_sage_int2_exchange_in_the_products_equals_the_separate_codec_passes(sage_workload):
     """The boundary rows of every layer travelling as int2 (the reference's runs: --num_bits=2 --is_pre_delay=true):
-    the products that write and read the packed rows themselves against quantise / dequantise passes of their own."""
+    the products that write and read the packed rows themselves against quantise / dequantise passes of their own, and
+    against the one launch per aggregation that gathers the received rows straight from the packed bytes."""
     loss, grads, updated = sage_workload(fold=True, bits=2, fused_codec=True)
-    ref_loss, ref_grads, ref_updated = sage_workload(fold=True, bits=2, fused_codec=False)
     assert loss == loss and 4.5 < loss < 6.5
-    assert loss == ref_loss
-    for a, b in zip(grads + updated, ref_grads + ref_updated):
-        assert torch.equal(a, b)
+    for other in (sage_workload(fold=True, bits=2, fused_codec=False),
+                  sage_workload(fold=True, bits=2, fused_codec=True, one_launch=True)):
+        ref_loss, ref_grads, ref_updated = other
+        assert loss == ref_loss
+        for a, b in zip(grads + updated, ref_grads + ref_updated):
+            assert torch.equal(a, b)

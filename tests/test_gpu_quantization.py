@@ -427,3 +427,69 @@ def test_reference_recipe_all_procs_against_per_segment_loop_and_torch(bits):
         diff = (back.cpu() - ref).abs()
         assert bool((diff <= s_cpu.view(-1, 1) * (1 + 1e-4) + 1e-6).all())
         assert float((diff > 1e-6 + 1e-5 * ref.abs()).float().mean()) < 0.02
+
+
+@pytest.mark.parametrize("feat", [4, 48, 128, 256, 604])
+@pytest.mark.parametrize("kind", ["bf16", 2, 8])
+def test_one_launch_over_dense_rows_and_rows_in_their_exchange_format(kind, feat):
+    """``SpmmPlan.spmm_dense_then``: a plan over [L | R], the first elements of every row gathering fp32 rows, the
+    others bf16 rows or packed int2 / int8 rows -- bit-equal to the product with L followed by the product with R
+    from the exchange format (accumulating and overwriting), for local parts that end before, at and behind the
+    boundaries of the 32- / 64-element index chunks, rows with only local or only received elements and empty rows."""
+    from gnn_benchmark_amd import SPMM_forward
+    from gnn_benchmark_amd import computation_ops as ops
+    from gnn_benchmark_amd.data_manager import CommBufferForQuantization, CommSplits
+    from gnn_benchmark_amd.sparse_tensor import SparseTensor, side_by_side
+    from gnn_benchmark_amd.spmm_kernel import SPMM_forward_quantized
+
+    rng = np.random.default_rng(7 * feat + (0 if kind == "bf16" else kind))
+    rows, local_cols, halo = 600, 500, 333
+
+    def ragged(cols, lens):
+        rowptr = np.concatenate(([0], np.cumsum(lens))).astype(np.int64)
+        col = np.concatenate([np.sort(rng.integers(0, cols, n)) for n in lens] + [np.zeros(0, np.int64)]).astype(np.int64)
+        val = rng.standard_normal(rowptr[-1]).astype(np.float32)
+        return SparseTensor(rowptr=dev(rowptr), col=dev(col), value=dev(val), sparse_sizes=(rows, cols), is_sorted=True)
+
+    len_l = rng.poisson(6, rows)
+    len_r = rng.poisson(3, rows)
+    edges = [0, 1, 7, 8, 9, 31, 32, 33, 63, 64, 65, 96, 127, 128, 129, 300]
+    for i, n in enumerate(edges):       # local lengths around the chunk boundaries, with and without received elements
+        len_l[3 * i], len_r[3 * i] = n, 5
+        len_l[3 * i + 1], len_r[3 * i + 1] = n, 0
+        len_l[3 * i + 2], len_r[3 * i + 2] = n, 70
+    len_l[100:110], len_r[100:110] = 0, 0
+    left, right = ragged(local_cols, len_l), ragged(halo, len_r)
+    both = side_by_side(left, right)
+    assert np.array_equal(both.first_counts.cpu().numpy(), len_l)
+    x = dev(_rows(rng, local_cols, feat))
+    recv = dev(_rows(rng, halo, feat))
+    if kind == "bf16":
+        second = recv.to(torch.bfloat16)
+
+        def from_format(out):
+            SPMM_forward(right, second, out)
+    else:
+        cs = CommSplits([100, 0, 33, 200], [5, 5, 5, 5], 4, kind)
+        qbuf = CommBufferForQuantization(cs, feat, kind, device="cuda")
+        ops.quantize_tensor_for_all_procs(recv, qbuf.quantized_recv_data_buf, qbuf.quantized_recv_params_buf_fp32,
+                                          qbuf.dequantized_work_range_per_proc, 4, kind)
+        second = (qbuf.quantized_recv_data_buf, qbuf.quantized_recv_params_buf_fp32, qbuf.recv_row_code, kind)
+
+        def from_format(out):
+            SPMM_forward_quantized(right, second[0], second[1], second[2], out, kind)
+    out0 = dev(rng.standard_normal((rows, feat)).astype(np.float32))
+    for accumulate in (True, False):
+        want, got = out0.clone(), out0.clone()
+        SPMM_forward(left, x, want, accumulate=accumulate)
+        from_format(want)
+        both.get_plan().spmm_dense_then(both.csr()[2], both.first_counts, x, second, got, accumulate)
+        assert torch.equal(got, want), (kind, feat, accumulate)
+    # operands that are column blocks of wider arrays
+    wide_x = torch.zeros(local_cols, feat + 8, device="cuda")
+    wide_x[:, 4:4 + feat] = x
+    wide_out = torch.zeros(rows, 2 * feat, device="cuda")
+    both.get_plan().spmm_dense_then(both.csr()[2], both.first_counts, wide_x[:, 4:4 + feat], second, wide_out[:, feat:], False)
+    assert torch.equal(wide_out[:, feat:], want) and not wide_out[:, :feat].any()
+    with pytest.raises(RuntimeError, match="Input mismatch"):
+        both.get_plan().spmm_dense_then(both.csr()[2], both.first_counts[:-1], x, second, got, False)
