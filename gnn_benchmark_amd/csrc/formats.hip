@@ -1,11 +1,11 @@
 // Sparse-format construction on the device (setup-time): COO -> CSR, CSR -> transposed
 // CSR, and the boundary-row gather.  gfx950 only.
-#include <hipcub/hipcub.hpp>
 
 #include <algorithm>
 #include <type_traits>
 
 #include "common.h"
+#include "sort.h"
 
 namespace gnnagg {
 namespace {
@@ -157,16 +157,14 @@ hipError_t launch_gather_rows(const float *src, int64_t src_rows, const int64_t 
     return hipGetLastError();
 }
 
-int sort_keys(uint64_t *key_in, uint64_t *key_out, uint32_t *idx_in, uint32_t *idx_out, int64_t n, int bits,
-              hipStream_t st) {
-    size_t tmp_bytes = 0;
-    GNNAGG_HIP(hipcub::DeviceRadixSort::SortPairs(nullptr, tmp_bytes, key_in, key_out, idx_in, idx_out, (int)n, 0,
-                                                  bits, st));
-    DevBuf<char> tmp;
-    GNNAGG_HIP(tmp.alloc(std::max<size_t>(tmp_bytes, 1)));
-    GNNAGG_HIP(hipcub::DeviceRadixSort::SortPairs(tmp.p, tmp_bytes, key_in, key_out, idx_in, idx_out, (int)n, 0, bits,
-                                                  st));
-    GNNAGG_HIP(hipStreamSynchronize(st));
+// stable sort of the (key, position) pairs by the low `bits` bits of the key; where the result lies comes back in
+// *key_sorted / *idx_sorted (one of the two array pairs)
+int sort_keys(uint64_t *key_a, uint64_t *key_b, uint32_t *idx_a, uint32_t *idx_b, int64_t n, int bits, hipStream_t st,
+              uint64_t **key_sorted, uint32_t **idx_sorted) {
+    bool in_b = false;
+    if (int rc = sort_pairs_u64(key_a, key_b, idx_a, idx_b, n, bits, st, &in_b)) return rc;
+    *key_sorted = in_b ? key_b : key_a;
+    *idx_sorted = in_b ? idx_b : idx_a;
     return GNNAGG_OK;
 }
 
@@ -213,11 +211,14 @@ extern "C" int gnnagg_coo_to_csr(const int64_t *row, const int64_t *col, const f
     GNNAGG_HIP(hipMemcpyAsync(&h_bad, bad.p, sizeof(unsigned int), hipMemcpyDeviceToHost, st));
     GNNAGG_HIP(hipStreamSynchronize(st));
     GNNAGG_REQUIRE(!h_bad, "a row/col index lies outside [0,%lld) x [0,%lld)", (long long)rows, (long long)cols);
-    if (int rc = sort_keys(key_in.p, key_out.p, idx_in.p, idx_out.p, nnz, col_bits + row_bits, st)) return rc;
-    hipLaunchKernelGGL(unpack_sorted_kernel, dim3(grid_for(nnz, 256)), dim3(256), 0, st, key_out.p, idx_out.p, value,
+    uint64_t *key_sorted = nullptr;
+    uint32_t *idx_sorted = nullptr;
+    if (int rc = sort_keys(key_in.p, key_out.p, idx_in.p, idx_out.p, nnz, col_bits + row_bits, st, &key_sorted, &idx_sorted))
+        return rc;
+    hipLaunchKernelGGL(unpack_sorted_kernel, dim3(grid_for(nnz, 256)), dim3(256), 0, st, key_sorted, idx_sorted, value,
                        nnz, col_bits, col_out, value_out);
     GNNAGG_HIP(hipGetLastError());
-    hipLaunchKernelGGL(major_ptr_kernel, dim3(grid_for(rows + 1, 256)), dim3(256), 0, st, key_out.p, nnz, col_bits, rows,
+    hipLaunchKernelGGL(major_ptr_kernel, dim3(grid_for(rows + 1, 256)), dim3(256), 0, st, key_sorted, nnz, col_bits, rows,
                        rowptr);
     GNNAGG_HIP(hipGetLastError());
     GNNAGG_HIP(hipStreamSynchronize(st));
@@ -263,11 +264,14 @@ extern "C" int gnnagg_csr_transpose(const int64_t *rowptr, const int64_t *col, c
     GNNAGG_REQUIRE(!h_bad, "a column index lies outside [0,%lld)", (long long)cols);
     // (col, row) keys are unique per stored position up to repeated entries; the radix
     // sort is stable, so repeated (row, col) pairs keep their CSR order.
-    if (int rc = sort_keys(key_in.p, key_out.p, idx_in.p, idx_out.p, nnz, col_bits + row_bits, st)) return rc;
-    hipLaunchKernelGGL(unpack_sorted_kernel, dim3(grid_for(nnz, 256)), dim3(256), 0, st, key_out.p, idx_out.p, value,
+    uint64_t *key_sorted = nullptr;
+    uint32_t *idx_sorted = nullptr;
+    if (int rc = sort_keys(key_in.p, key_out.p, idx_in.p, idx_out.p, nnz, col_bits + row_bits, st, &key_sorted, &idx_sorted))
+        return rc;
+    hipLaunchKernelGGL(unpack_sorted_kernel, dim3(grid_for(nnz, 256)), dim3(256), 0, st, key_sorted, idx_sorted, value,
                        nnz, row_bits, row_t, value_t);
     GNNAGG_HIP(hipGetLastError());
-    hipLaunchKernelGGL(major_ptr_kernel, dim3(grid_for(cols + 1, 256)), dim3(256), 0, st, key_out.p, nnz, row_bits, cols,
+    hipLaunchKernelGGL(major_ptr_kernel, dim3(grid_for(cols + 1, 256)), dim3(256), 0, st, key_sorted, nnz, row_bits, cols,
                        colptr);
     GNNAGG_HIP(hipGetLastError());
     GNNAGG_HIP(hipStreamSynchronize(st));

@@ -1,0 +1,378 @@
+// Set-up time sorting and run detection on the device, hand-written for gfx950 (64-lane waves): a stable LSD radix
+// sort of (key, 32-bit payload) pairs, an exclusive scan, and the run structure of a sorted list (unique values,
+// counts, inverse).  They serve the format builders (COO -> CSR, CSR -> transposed CSR), the plan's ordering of rows
+// by length, and the index-map builders of data_manager/DataProcessor.py, which the reference writes as per-edge
+// Python loops over sorted lists (self_benchmark/a64fx/data_manager/DataProcessor.py:39-53, :238-246, :434-444).
+//
+// Radix sort, one pass per 8 bits of key, least significant first; a pass is three launches:
+//   1. histogram: a block counts the digits of its tile of kTile keys (LDS atomics) into hist[digit][block];
+//   2. exclusive scan of hist in (digit, block) order: where each block's keys of each digit start in the output;
+//   3. scatter: the block walks its tile again, 256 keys a round in input order; a key's place is the block's start
+//      for its digit + the keys of that digit in earlier rounds + those in lower waves of this round + those in
+//      lower lanes of its wave (eight ballots give the lanes that hold the same digit).  Equal keys therefore keep
+//      their input order: the sort is stable, which is what makes repeated (row, col) pairs keep their order and
+//      what the reference's known-answer vectors need of its argsort.
+#include "sort.h"
+
+#include <algorithm>
+
+namespace gnnagg {
+namespace {
+
+constexpr int kRadixBits = 8;
+constexpr int kBins = 1 << kRadixBits;
+constexpr int kKeysPerThread = 16;
+constexpr int kTile = 256 * kKeysPerThread;
+
+// ------------------------------------------------------------------ exclusive scan of uint32 (sums below 2^32)
+constexpr int kScanPerThread = 8;
+constexpr int kScanTile = 256 * kScanPerThread;
+
+__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v) {
+    const int lane = (int)__lane_id();
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t up = (uint32_t)__shfl_up((int)v, d, 64);
+        if (lane >= d) v += up;
+    }
+    return v;
+}
+
+// sum of the block's values in front of this thread's; *total: the block's sum (valid in every thread)
+__device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t mine, uint32_t *total) {
+    __shared__ uint32_t wave_sum[4];
+    const int lane = (int)threadIdx.x & 63, wave = (int)threadIdx.x >> 6;
+    const uint32_t incl = wave_inclusive_scan(mine);
+    if (lane == 63) wave_sum[wave] = incl;
+    __syncthreads();
+    uint32_t before = 0, all = 0;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        if (w < wave) before += wave_sum[w];
+        all += wave_sum[w];
+    }
+    __syncthreads();
+    *total = all;
+    return before + incl - mine;
+}
+
+__global__ __launch_bounds__(256) void scan_tile_sums_kernel(const uint32_t *__restrict__ in, int64_t n,
+                                                             uint32_t *__restrict__ tile_sum) {
+    const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanPerThread;
+    uint32_t s = 0;
+#pragma unroll
+    for (int k = 0; k < kScanPerThread; ++k)
+        if (base + k < n) s += in[base + k];
+    uint32_t total;
+    (void)block_exclusive_scan(s, &total);
+    if (threadIdx.x == 0) tile_sum[blockIdx.x] = total;
+}
+
+// one block: exclusive scan of the tile sums in place, 256 at a time with a running carry
+__global__ __launch_bounds__(256) void scan_sums_kernel(uint32_t *__restrict__ tile_sum, int64_t tiles) {
+    uint32_t carry = 0;
+    for (int64_t base = 0; base < tiles; base += 256) {
+        const int64_t i = base + threadIdx.x;
+        const uint32_t v = i < tiles ? tile_sum[i] : 0;
+        uint32_t total;
+        const uint32_t before = block_exclusive_scan(v, &total);
+        if (i < tiles) tile_sum[i] = carry + before;
+        carry += total;
+    }
+}
+
+// (in and out may be the same array: a block reads its tile before it writes it)
+__global__ __launch_bounds__(256) void scan_apply_kernel(const uint32_t *in, int64_t n,
+                                                         const uint32_t *__restrict__ tile_before, uint32_t *out) {
+    const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanPerThread;
+    uint32_t v[kScanPerThread];
+    uint32_t s = 0;
+#pragma unroll
+    for (int k = 0; k < kScanPerThread; ++k) {
+        v[k] = base + k < n ? in[base + k] : 0;
+        s += v[k];
+    }
+    uint32_t total;
+    uint32_t run = tile_before[blockIdx.x] + block_exclusive_scan(s, &total);
+#pragma unroll
+    for (int k = 0; k < kScanPerThread; ++k) {
+        if (base + k < n) out[base + k] = run;
+        run += v[k];
+    }
+}
+
+}  // namespace
+
+// out[i] = in[0] + ... + in[i - 1] (in == out is fine).  Allocates the tile sums; enqueues on `st`.
+int exclusive_scan_u32(const uint32_t *in, uint32_t *out, int64_t n, hipStream_t st) {
+    if (n <= 0) return GNNAGG_OK;
+    const int64_t tiles = (n + kScanTile - 1) / kScanTile;
+    GNNAGG_REQUIRE(tiles < (int64_t(1) << 31), "scan of more than 2^42 values");
+    DevBuf<uint32_t> sums;
+    GNNAGG_HIP(sums.alloc((size_t)tiles));
+    hipLaunchKernelGGL(scan_tile_sums_kernel, dim3((unsigned)tiles), dim3(256), 0, st, in, n, sums.p);
+    GNNAGG_HIP(hipGetLastError());
+    hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(256), 0, st, sums.p, tiles);
+    GNNAGG_HIP(hipGetLastError());
+    hipLaunchKernelGGL(scan_apply_kernel, dim3((unsigned)tiles), dim3(256), 0, st, in, n, sums.p, out);
+    GNNAGG_HIP(hipGetLastError());
+    GNNAGG_HIP(hipStreamSynchronize(st));  // the tile sums are released on scope exit
+    return GNNAGG_OK;
+}
+
+namespace {
+
+// ------------------------------------------------------------------ radix sort
+template <typename KeyT>
+__global__ __launch_bounds__(256) void radix_histogram_kernel(const KeyT *__restrict__ key, int64_t n, int shift,
+                                                              uint32_t *__restrict__ hist, int64_t blocks) {
+    __shared__ uint32_t bins[kBins];
+    bins[threadIdx.x] = 0;
+    __syncthreads();
+    const int64_t base = (int64_t)blockIdx.x * kTile + threadIdx.x;
+#pragma unroll
+    for (int r = 0; r < kKeysPerThread; ++r) {
+        const int64_t i = base + (int64_t)r * 256;
+        if (i < n) atomicAdd(&bins[(int)((key[i] >> shift) & (kBins - 1))], 1u);
+    }
+    __syncthreads();
+    hist[(int64_t)threadIdx.x * blocks + blockIdx.x] = bins[threadIdx.x];
+}
+
+template <typename KeyT>
+__global__ __launch_bounds__(256) void radix_scatter_kernel(const KeyT *__restrict__ key_in,
+                                                            const uint32_t *__restrict__ val_in, int64_t n, int shift,
+                                                            const uint32_t *__restrict__ start, int64_t blocks,
+                                                            KeyT *__restrict__ key_out, uint32_t *__restrict__ val_out) {
+    __shared__ uint32_t place[kBins];         // where the block's next key of each digit goes
+    __shared__ uint32_t in_wave[4][kBins];    // this round: keys of each digit in each wave
+    const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    place[tid] = start[(int64_t)tid * blocks + blockIdx.x];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) in_wave[w][tid] = 0;
+    const int64_t base = (int64_t)blockIdx.x * kTile + tid;
+    KeyT k[kKeysPerThread];
+    uint32_t v[kKeysPerThread];
+#pragma unroll
+    for (int r = 0; r < kKeysPerThread; ++r) {
+        const int64_t i = base + (int64_t)r * 256;
+        k[r] = i < n ? key_in[i] : KeyT(0);
+        v[r] = i < n ? val_in[i] : 0u;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < kKeysPerThread; ++r) {
+        const bool live = base + (int64_t)r * 256 < n;  // a tile's dead keys are its last ones: whole trailing lanes
+        const int digit = (int)((k[r] >> shift) & (kBins - 1));
+        // the lanes of this wave that hold a live key of the same digit
+        uint64_t same = __builtin_amdgcn_ballot_w64(live);
+#pragma unroll
+        for (int b = 0; b < kRadixBits; ++b) {
+            const uint64_t has = __builtin_amdgcn_ballot_w64(((digit >> b) & 1) != 0);
+            same &= ((digit >> b) & 1) ? has : ~has;
+        }
+        const uint32_t below = (uint32_t)__popcll(same & ((uint64_t(1) << lane) - 1));
+        if (live && below == 0) in_wave[wave][digit] = (uint32_t)__popcll(same);  // the digit's first lane
+        __syncthreads();
+        if (live) {
+            uint32_t at = place[digit] + below;
+#pragma unroll
+            for (int w = 0; w < 3; ++w)
+                if (w < wave) at += in_wave[w][digit];
+            key_out[at] = k[r];
+            val_out[at] = v[r];
+        }
+        __syncthreads();
+        // digit `tid`: move its place past this round's keys, clear the round's counts
+        place[tid] += in_wave[0][tid] + in_wave[1][tid] + in_wave[2][tid] + in_wave[3][tid];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) in_wave[w][tid] = 0;
+        __syncthreads();
+    }
+}
+
+template <typename KeyT>
+int radix_sort_pairs(KeyT *key_a, KeyT *key_b, uint32_t *val_a, uint32_t *val_b, int64_t n, int bits, hipStream_t st,
+                     bool *result_in_b) {
+    *result_in_b = false;
+    if (n <= 0 || bits <= 0) return GNNAGG_OK;
+    GNNAGG_REQUIRE(n < (int64_t(1) << 32), "radix sort of more than 2^32-1 pairs");
+    const int64_t blocks = (n + kTile - 1) / kTile;
+    DevBuf<uint32_t> hist;
+    GNNAGG_HIP(hist.alloc((size_t)(blocks * kBins)));
+    KeyT *kin = key_a, *kout = key_b;
+    uint32_t *vin = val_a, *vout = val_b;
+    for (int shift = 0; shift < bits; shift += kRadixBits) {
+        hipLaunchKernelGGL((radix_histogram_kernel<KeyT>), dim3((unsigned)blocks), dim3(256), 0, st, kin, n, shift,
+                           hist.p, blocks);
+        GNNAGG_HIP(hipGetLastError());
+        if (int rc = exclusive_scan_u32(hist.p, hist.p, blocks * kBins, st)) return rc;
+        hipLaunchKernelGGL((radix_scatter_kernel<KeyT>), dim3((unsigned)blocks), dim3(256), 0, st, kin, vin, n, shift,
+                           hist.p, blocks, kout, vout);
+        GNNAGG_HIP(hipGetLastError());
+        std::swap(kin, kout);
+        std::swap(vin, vout);
+        *result_in_b = !*result_in_b;
+    }
+    GNNAGG_HIP(hipStreamSynchronize(st));  // the histogram is released on scope exit
+    return GNNAGG_OK;
+}
+
+}  // namespace
+
+int sort_pairs_u64(uint64_t *key_a, uint64_t *key_b, uint32_t *val_a, uint32_t *val_b, int64_t n, int bits,
+                   hipStream_t st, bool *result_in_b) {
+    return radix_sort_pairs<uint64_t>(key_a, key_b, val_a, val_b, n, bits, st, result_in_b);
+}
+
+int sort_pairs_u32(uint32_t *key_a, uint32_t *key_b, uint32_t *val_a, uint32_t *val_b, int64_t n, int bits,
+                   hipStream_t st, bool *result_in_b) {
+    return radix_sort_pairs<uint32_t>(key_a, key_b, val_a, val_b, n, bits, st, result_in_b);
+}
+
+namespace {
+
+// ------------------------------------------------------------------ argsort / runs of a sorted list
+__global__ __launch_bounds__(256) void argsort_prepare_kernel(const int64_t *__restrict__ x, int64_t n,
+                                                              uint64_t *__restrict__ key, uint32_t *__restrict__ idx,
+                                                              unsigned long long *__restrict__ max_key,
+                                                              unsigned int *__restrict__ negative) {
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    unsigned long long m = 0;
+    bool neg = false;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
+        const int64_t v = x[i];
+        neg |= v < 0;
+        key[i] = (uint64_t)v;
+        idx[i] = (uint32_t)i;
+        if (v > 0 && (unsigned long long)v > m) m = (unsigned long long)v;
+    }
+    if (m) atomicMax(max_key, m);
+    if (neg) atomicOr(negative, 1u);
+}
+
+__global__ __launch_bounds__(256) void argsort_finish_kernel(const uint64_t *__restrict__ key,
+                                                             const uint32_t *__restrict__ idx, int64_t n,
+                                                             int64_t *__restrict__ perm, int64_t *__restrict__ sorted) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    perm[i] = (int64_t)idx[i];
+    if (sorted) sorted[i] = (int64_t)key[i];
+}
+
+// flag[i] = 1 where a run starts: i == 0, x[i] != x[i - 1], or i is one of the forced starts
+__global__ __launch_bounds__(256) void run_flags_kernel(const int64_t *__restrict__ x, int64_t n,
+                                                        uint32_t *__restrict__ flag) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    flag[i] = (i == 0 || x[i] != x[i - 1]) ? 1u : 0u;
+}
+
+__global__ __launch_bounds__(256) void force_starts_kernel(const int64_t *__restrict__ starts, int64_t count, int64_t n,
+                                                           uint32_t *__restrict__ flag) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= count) return;
+    const int64_t s = starts[i];
+    if (s >= 0 && s < n) flag[s] = 1u;
+}
+
+// before[i] = runs that start in front of position i (exclusive scan of the flags).  The run of position i is
+// before[i] + flag[i] - 1; a run's first position writes its value, and its start for the counts.
+__global__ __launch_bounds__(256) void run_outputs_kernel(const int64_t *__restrict__ x, const uint32_t *__restrict__ flag,
+                                                          const uint32_t *__restrict__ before, int64_t n,
+                                                          int64_t *__restrict__ uniq, int64_t *__restrict__ inverse,
+                                                          int64_t *__restrict__ run_start) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const int64_t run = (int64_t)before[i] + (int64_t)flag[i] - 1;
+    if (inverse) inverse[i] = run;
+    if (flag[i]) {
+        if (uniq) uniq[run] = x[i];
+        if (run_start) run_start[run] = i;
+    }
+}
+
+__global__ __launch_bounds__(256) void run_counts_kernel(const int64_t *__restrict__ run_start, int64_t runs, int64_t n,
+                                                         int64_t *__restrict__ counts) {
+    const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (r >= runs) return;
+    counts[r] = (r + 1 < runs ? run_start[r + 1] : n) - run_start[r];
+}
+
+}  // namespace
+}  // namespace gnnagg
+
+using namespace gnnagg;
+
+extern "C" int gnnagg_argsort_i64(const int64_t *x, int64_t n, int64_t *perm, int64_t *sorted, void *stream) {
+    GNNAGG_REQUIRE(n >= 0, "negative size");
+    if (n == 0) return GNNAGG_OK;
+    GNNAGG_REQUIRE(x && perm, "null x/perm");
+    if (n >= (int64_t(1) << 32)) return fail(GNNAGG_ERR_UNSUPPORTED, "argsort of more than 2^32-1 values");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    DevBuf<uint64_t> key_a, key_b;
+    DevBuf<uint32_t> idx_a, idx_b;
+    DevBuf<unsigned long long> flags;  // [0] the largest key, [1] whether a key was negative
+    GNNAGG_HIP(key_a.alloc((size_t)n));
+    GNNAGG_HIP(key_b.alloc((size_t)n));
+    GNNAGG_HIP(idx_a.alloc((size_t)n));
+    GNNAGG_HIP(idx_b.alloc((size_t)n));
+    GNNAGG_HIP(flags.alloc(2));
+    GNNAGG_HIP(hipMemsetAsync(flags.p, 0, 2 * sizeof(unsigned long long), st));
+    const unsigned grid = (unsigned)std::min<int64_t>((n + 255) / 256, 256 * 32);
+    hipLaunchKernelGGL(argsort_prepare_kernel, dim3(grid), dim3(256), 0, st, x, n, key_a.p, idx_a.p, flags.p,
+                       reinterpret_cast<unsigned int *>(flags.p + 1));
+    GNNAGG_HIP(hipGetLastError());
+    unsigned long long h[2] = {0, 0};
+    GNNAGG_HIP(hipMemcpyAsync(h, flags.p, sizeof(h), hipMemcpyDeviceToHost, st));
+    GNNAGG_HIP(hipStreamSynchronize(st));
+    GNNAGG_REQUIRE((h[1] & 0xffffffffull) == 0, "argsort takes non-negative keys (node ids, positions)");
+    const int bits = h[0] ? ceil_log2_u64(h[0] + 1) : 1;
+    bool in_b = false;
+    if (int rc = sort_pairs_u64(key_a.p, key_b.p, idx_a.p, idx_b.p, n, bits, st, &in_b)) return rc;
+    hipLaunchKernelGGL(argsort_finish_kernel, dim3(grid_for(n, 256)), dim3(256), 0, st, in_b ? key_b.p : key_a.p,
+                       in_b ? idx_b.p : idx_a.p, n, perm, sorted);
+    GNNAGG_HIP(hipGetLastError());
+    GNNAGG_HIP(hipStreamSynchronize(st));
+    return GNNAGG_OK;
+}
+
+extern "C" int gnnagg_runs_i64(const int64_t *x, int64_t n, const int64_t *forced_starts, int64_t forced_count,
+                               int64_t *uniq, int64_t *inverse, int64_t *counts, int64_t *runs_out, void *stream) {
+    GNNAGG_REQUIRE(n >= 0 && forced_count >= 0, "negative size");
+    GNNAGG_REQUIRE(runs_out, "null runs_out");
+    *runs_out = 0;
+    if (n == 0) return GNNAGG_OK;
+    GNNAGG_REQUIRE(x, "null x");
+    GNNAGG_REQUIRE(forced_count == 0 || forced_starts, "null forced_starts");
+    if (n >= (int64_t(1) << 32)) return fail(GNNAGG_ERR_UNSUPPORTED, "run detection over more than 2^32-1 values");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    DevBuf<uint32_t> flag, before;
+    DevBuf<int64_t> run_start;
+    GNNAGG_HIP(flag.alloc((size_t)n));
+    GNNAGG_HIP(before.alloc((size_t)n));
+    GNNAGG_HIP(run_start.alloc((size_t)n));
+    hipLaunchKernelGGL(run_flags_kernel, dim3(grid_for(n, 256)), dim3(256), 0, st, x, n, flag.p);
+    GNNAGG_HIP(hipGetLastError());
+    if (forced_count > 0) {
+        hipLaunchKernelGGL(force_starts_kernel, dim3(grid_for(forced_count, 256)), dim3(256), 0, st, forced_starts,
+                           forced_count, n, flag.p);
+        GNNAGG_HIP(hipGetLastError());
+    }
+    if (int rc = exclusive_scan_u32(flag.p, before.p, n, st)) return rc;
+    uint32_t last[2] = {0, 0};
+    GNNAGG_HIP(hipMemcpyAsync(&last[0], before.p + (n - 1), sizeof(uint32_t), hipMemcpyDeviceToHost, st));
+    GNNAGG_HIP(hipMemcpyAsync(&last[1], flag.p + (n - 1), sizeof(uint32_t), hipMemcpyDeviceToHost, st));
+    GNNAGG_HIP(hipStreamSynchronize(st));
+    const int64_t runs = (int64_t)last[0] + (int64_t)last[1];
+    hipLaunchKernelGGL(run_outputs_kernel, dim3(grid_for(n, 256)), dim3(256), 0, st, x, flag.p, before.p, n, uniq, inverse,
+                       run_start.p);
+    GNNAGG_HIP(hipGetLastError());
+    if (counts) {
+        hipLaunchKernelGGL(run_counts_kernel, dim3(grid_for(runs, 256)), dim3(256), 0, st, run_start.p, runs, n, counts);
+        GNNAGG_HIP(hipGetLastError());
+    }
+    GNNAGG_HIP(hipStreamSynchronize(st));
+    *runs_out = runs;
+    return GNNAGG_OK;
+}

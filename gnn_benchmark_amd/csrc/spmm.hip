@@ -1,7 +1,5 @@
 // Host side of the SpMM entry points: launch-shape selection, the direct (plan-less)
 // path, and the cached degree-binned plan.  gfx950 only.
-#include <hipcub/hipcub.hpp>
-
 #include <algorithm>
 #include <atomic>
 #include <mutex>
@@ -10,6 +8,7 @@
 #include <vector>
 
 #include "common.h"
+#include "sort.h"
 #include "spmm_kernels.h"
 
 namespace gnnagg {
@@ -504,17 +503,15 @@ extern "C" int gnnagg_plan_create_ex(const int64_t *rowptr, const int64_t *col, 
             GNNAGG_HIP(hipGetLastError());
         }
         // stable sort of the rows by class: ascending row id inside a class
-        size_t tmp_bytes = 0;
-        GNNAGG_HIP(hipcub::DeviceRadixSort::SortPairs(nullptr, tmp_bytes, key_in.p, key_out.p, row_in.p, perm.p,
-                                                      (int)rows, 0, kClassBits, st));
-        DevBuf<char> tmp;
-        GNNAGG_HIP(tmp.alloc(std::max<size_t>(tmp_bytes, 1)));
-        GNNAGG_HIP(hipcub::DeviceRadixSort::SortPairs(tmp.p, tmp_bytes, key_in.p, key_out.p, row_in.p, perm.p,
-                                                      (int)rows, 0, kClassBits, st));
+        bool in_b = false;
+        if (int rc = sort_pairs_u32(key_in.p, key_out.p, reinterpret_cast<uint32_t *>(row_in.p),
+                                    reinterpret_cast<uint32_t *>(perm.p), rows, kClassBits, st, &in_b))
+            return rc;
+        const int32_t *order = in_b ? perm.p : row_in.p;
         GNNAGG_HIP(hipMemcpyAsync(&h_out, d_out.p, sizeof(ClassifyOut), hipMemcpyDeviceToHost, st));
         GNNAGG_HIP(hipStreamSynchronize(st));
         if (!h_out.bad_rowptr && h_out.max_deg < (1ull << 31)) {  // row lengths are only meaningful for a monotone rowptr
-            hipLaunchKernelGGL(build_tasks_kernel, dim3(grid_for(rows, 256)), dim3(256), 0, st, rowptr, perm.p,
+            hipLaunchKernelGGL(build_tasks_kernel, dim3(grid_for(rows, 256)), dim3(256), 0, st, rowptr, order,
                                (int)rows, p->task);
             GNNAGG_HIP(hipGetLastError());
             GNNAGG_HIP(hipStreamSynchronize(st));  // perm is released on scope exit

@@ -13,17 +13,17 @@ Where the reference calls a setup-time collective (``dist.all_to_all`` at :77, :
 a caller-supplied callable instead; no process group is needed.
 
 Sorting.  The reference uses ``torch.argsort`` (tie order unspecified); a stable sort
-is used here, which reproduces every known-answer vector of the reference's tests.
+is used here, which reproduces every known-answer vector of the reference's tests.  The
+sort, unique and run-numbering steps go through ``device_ops``: libgnnagg's own radix-sort
+and run kernels for GPU tensors, torch host ops of the same meaning for CPU tensors.
 """
 from typing import Callable, List, Optional
 
 import torch
 
 from ..sparse_tensor import SparseTensor
-
-
-def _stable_argsort(x: torch.Tensor) -> torch.Tensor:
-    return torch.sort(x, stable=True).indices
+from . import device_ops
+from .device_ops import stable_argsort as _stable_argsort
 
 
 def _as_i64(x, device=None) -> torch.Tensor:
@@ -61,7 +61,7 @@ class DataProcessor(object):
         src = remote_edges_list[0]
         dev = src.device
         begins = _as_i64(num_nodes_on_each_subgraph, dev)
-        uniq, inverse = torch.unique_consecutive(src, return_inverse=True)
+        uniq, inverse, _ = device_ops.runs(src, want_counts=False)
         owner = torch.bucketize(uniq, begins[1:world_size + 1].contiguous(), right=True)
         counts = torch.bincount(owner, minlength=world_size)[:world_size].to(torch.int64)
         ranges = torch.zeros(world_size + 1, dtype=torch.int64, device=dev)
@@ -113,13 +113,16 @@ class DataProcessorForPreAggresive(object):
     @staticmethod
     def get_degrees(nodes_list):
         """{node id: occurrences}.  Reference: DataProcessor.py:125-131."""
-        uniq, counts = torch.unique(nodes_list, return_counts=True)
+        if nodes_list.is_cuda and nodes_list.numel():
+            ordered = nodes_list[_stable_argsort(nodes_list)]
+            uniq, _, counts = device_ops.runs(ordered, want_inverse=False)
+        else:
+            uniq, counts = torch.unique(nodes_list, return_counts=True)
         return dict(zip(uniq.tolist(), counts.tolist()))
 
     @staticmethod
     def _occurrences_per_entry(nodes: torch.Tensor) -> torch.Tensor:
-        _, inverse, counts = torch.unique(nodes, return_inverse=True, return_counts=True)
-        return counts[inverse]
+        return device_ops.occurrences_per_entry(nodes)
 
     @staticmethod
     def decide_pre_or_post_aggr(src_in_remote_edges, dst_in_remote_edges, is_pre, is_post):
@@ -140,7 +143,7 @@ class DataProcessorForPreAggresive(object):
         stored as [firsts | seconds].  Reference: DataProcessor.py:252-279."""
         src_in_pre = src_in_remote_edges[pre_aggr_edge_idx]
         dst_in_pre = dst_in_remote_edges[pre_aggr_edge_idx]
-        src_in_post = torch.unique(src_in_remote_edges[post_aggr_edge_idx], sorted=True)
+        src_in_post = device_ops.unique_sorted(src_in_remote_edges[post_aggr_edge_idx])
         src_to_send = torch.cat((src_in_pre, src_in_post), dim=0)
         dst_to_send = torch.cat((dst_in_pre, src_in_post), dim=0)
         order = _stable_argsort(dst_to_send)
@@ -156,13 +159,14 @@ class DataProcessorForPreAggresive(object):
         Reference: DataProcessor.py:283-326."""
         src_in_post = src_in_remote_edges[post_aggr_edge_idx]
         dst_in_post = dst_in_remote_edges[post_aggr_edge_idx]
-        pre_dst = torch.unique(dst_in_remote_edges[pre_aggr_edge_idx], sorted=True)
+        pre_dst = device_ops.unique_sorted(dst_in_remote_edges[pre_aggr_edge_idx])
         src_from_recv = torch.cat((src_in_post, pre_dst), dim=0)
         dst_from_recv = torch.cat((dst_in_post, pre_dst), dim=0)
         order = _stable_argsort(src_from_recv)
         src_from_recv = src_from_recv[order]
         dst_from_recv = dst_from_recv[order]
-        recv_splits_for_data_exchange.append(int(torch.unique_consecutive(src_from_recv).shape[0]))
+        recv_splits_for_data_exchange.append(
+            int(device_ops.runs(src_from_recv, want_inverse=False, want_counts=False)[0].shape[0]))
         remote_edges_for_aggr_on_recv[0] = torch.cat((remote_edges_for_aggr_on_recv[0], src_from_recv), dim=0)
         remote_edges_for_aggr_on_recv[1] = torch.cat((remote_edges_for_aggr_on_recv[1], dst_from_recv), dim=0)
         begin_edge_on_each_partition_from[cur_rank + 1] = (
@@ -207,7 +211,7 @@ class DataProcessorForPreAggresive(object):
             packed = remote_edges_recv_from_graph_exchange[i]
             n = int(packed.shape[0] / 2)
             src, dst = packed[:n], packed[n:]
-            send_splits_for_data_exchange.append(int(torch.unique(dst).shape[0]))
+            send_splits_for_data_exchange.append(int(device_ops.unique_sorted(dst).shape[0]))
             srcs.append(src)
             dsts.append(dst)
             begin_edge_on_each_partition_to[i + 1] = begin_edge_on_each_partition_to[i] + dst.shape[0]
@@ -245,14 +249,10 @@ class DataProcessorForPreAggresive(object):
         if n == 0:
             return 0
         dev = remote_nodes_list.device
-        is_new = torch.ones(n, dtype=torch.bool, device=dev)
-        is_new[1:] = remote_nodes_list[1:] != remote_nodes_list[:-1]
         starts = _as_i64(begin_edge_on_each_partition, dev)[:-1]
-        starts = starts[(starts >= 0) & (starts < n)]
-        is_new[starts] = True
-        new_ids = torch.cumsum(is_new.to(torch.int64), 0) - 1
+        values, new_ids, _ = device_ops.runs(remote_nodes_list, forced_starts=starts, want_counts=False)
         remote_nodes_list.copy_(new_ids)
-        return int(new_ids[-1].item()) + 1
+        return int(values.shape[0])
 
     @staticmethod
     def transform_edge_index_to_sparse_tensor(local_edges_list, remote_edges_list_pre_post_aggr_from,

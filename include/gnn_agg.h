@@ -28,9 +28,9 @@ extern "C" {
 
 /* Raised whenever an exported prototype changes, an entry point goes away or the meaning of an argument changes
  * (2: `src_rows` in the row gathers, `workspace_bytes` in the weight-gradient entry points, 12 values from
- * gnnagg_plan_info; 3: the measurement probes left the library, gnnagg_plan_spmm_two_sources_f32 and gnnagg_plans_release came; 4: the two gnnagg_plan_spmm_dense_then_* entry points came).  Every binding compares it with
+ * gnnagg_plan_info; 3: the measurement probes left the library, gnnagg_plan_spmm_two_sources_f32 and gnnagg_plans_release came; 4: the two gnnagg_plan_spmm_dense_then_* entry points came; 5: gnnagg_argsort_i64 and gnnagg_runs_i64 came).  Every binding compares it with
  * gnnagg_abi_version() of the library it loaded before the first call. */
-#define GNNAGG_ABI_VERSION 4
+#define GNNAGG_ABI_VERSION 5
 
 /* Version of this ABI (GNNAGG_ABI_VERSION of the built library).  No reference counterpart. */
 int gnnagg_abi_version(void);
@@ -214,6 +214,28 @@ int gnnagg_csr_transpose(const int64_t *rowptr, const int64_t *col, const float 
  * ------------------------------------------------------------------------------- */
 int gnnagg_coo_to_csr(const int64_t *row, const int64_t *col, const float *value, int64_t nnz, int64_t rows,
                       int64_t cols, int64_t *rowptr, int64_t *col_out, float *value_out, void *stream);
+
+/* ---------------------------------------------------------------------------------
+ * Sorting and run detection for the index-map builders (set-up time; both allocate temporaries and SYNCHRONISE the
+ * stream).  The reference walks sorted edge lists with per-edge Python loops
+ * (data_manager/DataProcessor.py:39-53 halo renumbering, :238-246 pre/post decision, :434-444 buffer-row
+ * renumbering) after `torch.argsort` (:21, :259, :306) and `torch.unique` (:127); on the device the same maps are
+ * a stable sort plus the run structure of the sorted list.
+ *
+ * gnnagg_argsort_i64: perm int64 [n] such that x[perm] is ascending, equal keys in their input order (a stable
+ * radix sort, 8 bits a pass over the bits the largest key needs); sorted (may be NULL) receives x[perm].  Keys must
+ * be non-negative (GNNAGG_ERR_INVALID otherwise); n < 2^32.
+ *
+ * gnnagg_runs_i64: the runs of equal neighbours of x (a sorted list, or any list: torch.unique_consecutive).  A
+ * run also starts at every position listed in forced_starts (int64 [forced_count], positions outside [0, n) are
+ * ignored; NULL with 0): the per-rank segments of data_manager/DataProcessor.py:432-445, across which equality is
+ * not carried.  Outputs, each may be NULL: uniq int64 [runs] the value of each run, inverse int64 [n] the run of
+ * each position, counts int64 [runs] the length of each run (all three arrays sized n by the caller); *runs_out
+ * (host) the number of runs.
+ * ------------------------------------------------------------------------------- */
+int gnnagg_argsort_i64(const int64_t *x, int64_t n, int64_t *perm, int64_t *sorted, void *stream);
+int gnnagg_runs_i64(const int64_t *x, int64_t n, const int64_t *forced_starts, int64_t forced_count, int64_t *uniq,
+                    int64_t *inverse, int64_t *counts, int64_t *runs_out, void *stream);
 
 /* ---------------------------------------------------------------------------------
  * Boundary-row gather, out[i,:] = src[index[i],:].  Replaces

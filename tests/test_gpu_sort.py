@@ -1,0 +1,68 @@
+"""The hand-written set-up kernels of csrc/sort.hip through the C ABI: stable radix argsort and the run structure of
+a list, against torch's host ops; and the index-map steps built on them (``data_manager.device_ops``)."""
+import numpy as np
+import pytest
+import torch
+
+from gnn_benchmark_amd.data_manager import device_ops
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("n", [0, 1, 2, 63, 64, 255, 256, 257, 4095, 4096, 4097, 8193, 100_003, 1_000_003])
+@pytest.mark.parametrize("span", [1, 5, 300, 70_000, 1 << 33, (1 << 62) + 12345])
+def test_argsort_is_the_stable_ascending_order(n, span):
+    """Few distinct keys (long runs of equal keys: stability), keys of 1 .. 8 radix passes, sizes around the tile and
+    round boundaries of the scatter kernel."""
+    rng = np.random.default_rng(n + span % 1000)
+    x = torch.from_numpy(rng.integers(0, span, n, dtype=np.int64))
+    want = torch.sort(x, stable=True).indices
+    got = device_ops.stable_argsort(x.cuda())
+    assert got.dtype == torch.int64 and torch.equal(got.cpu(), want)
+
+
+def test_argsort_takes_sorted_reversed_and_constant_input_and_refuses_negative_keys():
+    n = 300_000
+    for x in (torch.arange(n), torch.arange(n).flip(0), torch.zeros(n, dtype=torch.int64),
+              torch.full((n,), (1 << 40) + 7, dtype=torch.int64), torch.arange(n) // 7):
+        assert torch.equal(device_ops.stable_argsort(x.cuda()).cpu(), torch.sort(x, stable=True).indices)
+    with pytest.raises(RuntimeError, match="non-negative"):
+        device_ops.stable_argsort(torch.tensor([3, -1, 2]).cuda())
+
+
+@pytest.mark.parametrize("n", [1, 2, 255, 2048, 2049, 100_003, 3_000_001])
+@pytest.mark.parametrize("distinct", [1, 3, 1000, 10 ** 9])
+def test_runs_equal_unique_consecutive(n, distinct):
+    rng = np.random.default_rng(n % 977 + distinct % 13)
+    x = torch.from_numpy(np.sort(rng.integers(0, distinct, n, dtype=np.int64)))
+    values, inverse, counts = torch.unique_consecutive(x, return_inverse=True, return_counts=True)
+    got = device_ops.runs(x.cuda())
+    assert torch.equal(got[0].cpu(), values) and torch.equal(got[1].cpu(), inverse) and torch.equal(got[2].cpu(), counts)
+    # unsorted input: runs of equal neighbours, not distinct values
+    y = torch.from_numpy(rng.integers(0, 3, n, dtype=np.int64))
+    values, inverse, counts = torch.unique_consecutive(y, return_inverse=True, return_counts=True)
+    got = device_ops.runs(y.cuda())
+    assert torch.equal(got[0].cpu(), values) and torch.equal(got[1].cpu(), inverse) and torch.equal(got[2].cpu(), counts)
+    only = device_ops.runs(y.cuda(), want_inverse=False, want_counts=False)
+    assert only[1] is None and only[2] is None and torch.equal(only[0].cpu(), values)
+
+
+def test_runs_with_forced_starts_equal_the_host_form():
+    """Segments across which equality is not carried (the per-rank restart of remap_remote_nodes_id)."""
+    rng = np.random.default_rng(3)
+    x = torch.from_numpy(np.sort(rng.integers(0, 50, 5000, dtype=np.int64)))
+    starts = torch.tensor([0, 17, 17, 2500, 4999, 5000, -3, 99999])
+    want = device_ops.runs(x, forced_starts=starts)          # host tensors: the torch form
+    got = device_ops.runs(x.cuda(), forced_starts=starts)
+    for a, b in zip(got, want):
+        assert torch.equal(a.cpu(), b)
+    assert int(want[0].shape[0]) > int(torch.unique_consecutive(x).shape[0])
+
+
+@pytest.mark.parametrize("n", [1, 1000, 250_000])
+def test_unique_and_occurrences_equal_torch(n):
+    rng = np.random.default_rng(n)
+    x = torch.from_numpy(rng.integers(0, max(2, n // 5), n, dtype=np.int64))
+    assert torch.equal(device_ops.unique_sorted(x.cuda()).cpu(), torch.unique(x, sorted=True))
+    _, inverse, counts = torch.unique(x, return_inverse=True, return_counts=True)
+    assert torch.equal(device_ops.occurrences_per_entry(x.cuda()).cpu(), counts[inverse])
