@@ -7,11 +7,11 @@
 // Radix sort, one pass per 8 bits of key, least significant first; a pass is three launches:
 //   1. histogram: a block counts the digits of its tile of kTile keys (LDS atomics) into hist[digit][block];
 //   2. exclusive scan of hist in (digit, block) order: where each block's keys of each digit start in the output;
-//   3. scatter: the block walks its tile again, 256 keys a round in input order; a key's place is the block's start
-//      for its digit + the keys of that digit in earlier rounds + those in lower waves of this round + those in
-//      lower lanes of its wave (eight ballots give the lanes that hold the same digit).  Equal keys therefore keep
-//      their input order: the sort is stable, which is what makes repeated (row, col) pairs keep their order and
-//      what the reference's known-answer vectors need of its argsort.
+//   3. scatter: the block ranks its tile's keys by digit, in input order (per-wave LDS counters; eight ballots give
+//      the lanes of a wave that hold the same digit), brings them to their place in the tile through LDS, and writes
+//      the tile out digit by digit, so that a digit's keys leave as one run of neighbouring addresses.  Equal keys
+//      keep their input order: the sort is stable, which is what makes repeated (row, col) pairs keep their order
+//      and what the reference's known-answer vectors need of its argsort.
 #include "sort.h"
 
 #include <algorithm>
@@ -21,8 +21,9 @@ namespace {
 
 constexpr int kRadixBits = 8;
 constexpr int kBins = 1 << kRadixBits;
-constexpr int kKeysPerThread = 16;
+constexpr int kKeysPerThread = 32;
 constexpr int kTile = 256 * kKeysPerThread;
+constexpr int kXcds = 8;  // gfx950: eight accelerator dies, each with its own L2
 
 // ------------------------------------------------------------------ exclusive scan of uint32 (sums below 2^32)
 constexpr int kScanPerThread = 8;
@@ -103,19 +104,31 @@ __global__ __launch_bounds__(256) void scan_apply_kernel(const uint32_t *in, int
 
 }  // namespace
 
-// out[i] = in[0] + ... + in[i - 1] (in == out is fine).  Allocates the tile sums; enqueues on `st`.
+namespace {
+
+int64_t scan_tiles(int64_t n) { return (n + kScanTile - 1) / kScanTile; }
+
+// the scan with the caller's array for the tile sums (scan_tiles(n) entries); enqueues only
+int exclusive_scan_into(const uint32_t *in, uint32_t *out, int64_t n, uint32_t *tile_sums, hipStream_t st) {
+    const int64_t tiles = scan_tiles(n);
+    hipLaunchKernelGGL(scan_tile_sums_kernel, dim3((unsigned)tiles), dim3(256), 0, st, in, n, tile_sums);
+    GNNAGG_HIP(hipGetLastError());
+    hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(256), 0, st, tile_sums, tiles);
+    GNNAGG_HIP(hipGetLastError());
+    hipLaunchKernelGGL(scan_apply_kernel, dim3((unsigned)tiles), dim3(256), 0, st, in, n, tile_sums, out);
+    GNNAGG_HIP(hipGetLastError());
+    return GNNAGG_OK;
+}
+
+}  // namespace
+
+// out[i] = in[0] + ... + in[i - 1] (in == out is fine).  Allocates the tile sums; returns when the scan is done.
 int exclusive_scan_u32(const uint32_t *in, uint32_t *out, int64_t n, hipStream_t st) {
     if (n <= 0) return GNNAGG_OK;
-    const int64_t tiles = (n + kScanTile - 1) / kScanTile;
-    GNNAGG_REQUIRE(tiles < (int64_t(1) << 31), "scan of more than 2^42 values");
+    GNNAGG_REQUIRE(scan_tiles(n) < (int64_t(1) << 31), "scan of more than 2^42 values");
     DevBuf<uint32_t> sums;
-    GNNAGG_HIP(sums.alloc((size_t)tiles));
-    hipLaunchKernelGGL(scan_tile_sums_kernel, dim3((unsigned)tiles), dim3(256), 0, st, in, n, sums.p);
-    GNNAGG_HIP(hipGetLastError());
-    hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(256), 0, st, sums.p, tiles);
-    GNNAGG_HIP(hipGetLastError());
-    hipLaunchKernelGGL(scan_apply_kernel, dim3((unsigned)tiles), dim3(256), 0, st, in, n, sums.p, out);
-    GNNAGG_HIP(hipGetLastError());
+    GNNAGG_HIP(sums.alloc((size_t)scan_tiles(n)));
+    if (int rc = exclusive_scan_into(in, out, n, sums.p, st)) return rc;
     GNNAGG_HIP(hipStreamSynchronize(st));  // the tile sums are released on scope exit
     return GNNAGG_OK;
 }
@@ -139,32 +152,47 @@ __global__ __launch_bounds__(256) void radix_histogram_kernel(const KeyT *__rest
     hist[(int64_t)threadIdx.x * blocks + blockIdx.x] = bins[threadIdx.x];
 }
 
+// One pass's scatter.  A block takes its tile in index order, wave w the keys [w * kTile / 4, (w + 1) * kTile / 4) in
+// rounds of 64.  (1) Each wave ranks its keys against its own LDS counters, no block barrier: a key's rank in its wave
+// is the counter of its digit + the lower lanes of this round that hold the same digit (eight ballots).  (2) From the
+// four waves' counters: where each digit starts in the tile, and where each wave's keys of it do.  (3) The keys go to
+// their place in the tile through LDS, so that (4) thread t writes position t + 256 j of the sorted tile: keys of one
+// digit leave as one run of neighbouring addresses (kTile / 256 keys on average) instead of one by one.  (5) The
+// payloads take the same way through the same LDS array, to the addresses step 4 kept.
 template <typename KeyT>
 __global__ __launch_bounds__(256) void radix_scatter_kernel(const KeyT *__restrict__ key_in,
                                                             const uint32_t *__restrict__ val_in, int64_t n, int shift,
                                                             const uint32_t *__restrict__ start, int64_t blocks,
                                                             KeyT *__restrict__ key_out, uint32_t *__restrict__ val_out) {
-    __shared__ uint32_t place[kBins];         // where the block's next key of each digit goes
-    __shared__ uint32_t in_wave[4][kBins];    // this round: keys of each digit in each wave
+    __shared__ KeyT sorted[kTile];
+    __shared__ uint32_t count[4][kBins];  // per wave: keys of each digit so far; after step 2: where they start
+    __shared__ uint32_t out_base[kBins];  // output address of the digit's first key of this tile - its place in the tile
     const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    place[tid] = start[(int64_t)tid * blocks + blockIdx.x];
+    // Workgroups go to the eight XCDs in turn; each XCD gets a stretch of neighbouring tiles, so that the runs two
+    // neighbouring tiles write to one digit's region, which adjoin, meet in one L2 instead of two.
+    const int64_t per_xcd = (int64_t)(gridDim.x / kXcds);
+    const int64_t tile = (int64_t)(blockIdx.x % kXcds) * per_xcd + (int64_t)(blockIdx.x / kXcds);
+    if (tile >= blocks) return;
+    const int64_t tile_base = tile * kTile;
+    const int live_keys = (int)std::min<int64_t>(kTile, n - tile_base);
 #pragma unroll
-    for (int w = 0; w < 4; ++w) in_wave[w][tid] = 0;
-    const int64_t base = (int64_t)blockIdx.x * kTile + tid;
+    for (int w = 0; w < 4; ++w) count[w][tid] = 0;
     KeyT k[kKeysPerThread];
     uint32_t v[kKeysPerThread];
+    uint32_t rank[kKeysPerThread];
+    const int mine = wave * (kTile / 4) + lane;  // this thread's key of round r: tile position mine + 64 r
 #pragma unroll
     for (int r = 0; r < kKeysPerThread; ++r) {
-        const int64_t i = base + (int64_t)r * 256;
-        k[r] = i < n ? key_in[i] : KeyT(0);
-        v[r] = i < n ? val_in[i] : 0u;
+        const int at = mine + 64 * r;
+        k[r] = at < live_keys ? key_in[tile_base + at] : KeyT(0);
+        v[r] = at < live_keys ? val_in[tile_base + at] : 0u;
     }
     __syncthreads();
+    uint32_t *my_count = count[wave];
 #pragma unroll
     for (int r = 0; r < kKeysPerThread; ++r) {
-        const bool live = base + (int64_t)r * 256 < n;  // a tile's dead keys are its last ones: whole trailing lanes
+        const bool live = mine + 64 * r < live_keys;  // dead keys are the tile's last ones
         const int digit = (int)((k[r] >> shift) & (kBins - 1));
-        // the lanes of this wave that hold a live key of the same digit
         uint64_t same = __builtin_amdgcn_ballot_w64(live);
 #pragma unroll
         for (int b = 0; b < kRadixBits; ++b) {
@@ -172,22 +200,53 @@ __global__ __launch_bounds__(256) void radix_scatter_kernel(const KeyT *__restri
             same &= ((digit >> b) & 1) ? has : ~has;
         }
         const uint32_t below = (uint32_t)__popcll(same & ((uint64_t(1) << lane) - 1));
-        if (live && below == 0) in_wave[wave][digit] = (uint32_t)__popcll(same);  // the digit's first lane
-        __syncthreads();
-        if (live) {
-            uint32_t at = place[digit] + below;
+        // the wave's LDS accesses execute in program order: this read sees the last round's update
+        const uint32_t before = my_count[digit];
+        __builtin_amdgcn_wave_barrier();
+        if (live && below == 0) my_count[digit] = before + (uint32_t)__popcll(same);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        rank[r] = before + below;
+    }
+    __syncthreads();
+    {   // digit `tid`
+        const uint32_t c0 = count[0][tid], c1 = count[1][tid], c2 = count[2][tid], c3 = count[3][tid];
+        uint32_t total;
+        const uint32_t first = block_exclusive_scan(c0 + c1 + c2 + c3, &total);
+        count[0][tid] = first;
+        count[1][tid] = first + c0;
+        count[2][tid] = first + c0 + c1;
+        count[3][tid] = first + c0 + c1 + c2;
+        out_base[tid] = start[(int64_t)tid * blocks + tile] - first;
+    }
+    __syncthreads();
 #pragma unroll
-            for (int w = 0; w < 3; ++w)
-                if (w < wave) at += in_wave[w][digit];
-            key_out[at] = k[r];
-            val_out[at] = v[r];
+    for (int r = 0; r < kKeysPerThread; ++r) {
+        const int digit = (int)((k[r] >> shift) & (kBins - 1));
+        rank[r] += my_count[digit];  // now the key's place in the sorted tile
+        if (mine + 64 * r < live_keys) sorted[rank[r]] = k[r];
+    }
+    __syncthreads();
+    uint32_t to[kKeysPerThread];
+#pragma unroll
+    for (int j = 0; j < kKeysPerThread; ++j) {
+        const int p = tid + 256 * j;
+        if (p < live_keys) {
+            const KeyT key = sorted[p];
+            to[j] = out_base[(int)((key >> shift) & (kBins - 1))] + (uint32_t)p;
+            key_out[to[j]] = key;
         }
-        __syncthreads();
-        // digit `tid`: move its place past this round's keys, clear the round's counts
-        place[tid] += in_wave[0][tid] + in_wave[1][tid] + in_wave[2][tid] + in_wave[3][tid];
+    }
+    __syncthreads();
+    uint32_t *sorted_val = reinterpret_cast<uint32_t *>(sorted);
 #pragma unroll
-        for (int w = 0; w < 4; ++w) in_wave[w][tid] = 0;
-        __syncthreads();
+    for (int r = 0; r < kKeysPerThread; ++r)
+        if (mine + 64 * r < live_keys) sorted_val[rank[r]] = v[r];
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kKeysPerThread; ++j) {
+        const int p = tid + 256 * j;
+        if (p < live_keys) val_out[to[j]] = sorted_val[p];
     }
 }
 
@@ -198,23 +257,25 @@ int radix_sort_pairs(KeyT *key_a, KeyT *key_b, uint32_t *val_a, uint32_t *val_b,
     if (n <= 0 || bits <= 0) return GNNAGG_OK;
     GNNAGG_REQUIRE(n < (int64_t(1) << 32), "radix sort of more than 2^32-1 pairs");
     const int64_t blocks = (n + kTile - 1) / kTile;
-    DevBuf<uint32_t> hist;
+    DevBuf<uint32_t> hist, sums;
     GNNAGG_HIP(hist.alloc((size_t)(blocks * kBins)));
+    GNNAGG_HIP(sums.alloc((size_t)scan_tiles(blocks * kBins)));
     KeyT *kin = key_a, *kout = key_b;
     uint32_t *vin = val_a, *vout = val_b;
     for (int shift = 0; shift < bits; shift += kRadixBits) {
         hipLaunchKernelGGL((radix_histogram_kernel<KeyT>), dim3((unsigned)blocks), dim3(256), 0, st, kin, n, shift,
                            hist.p, blocks);
         GNNAGG_HIP(hipGetLastError());
-        if (int rc = exclusive_scan_u32(hist.p, hist.p, blocks * kBins, st)) return rc;
-        hipLaunchKernelGGL((radix_scatter_kernel<KeyT>), dim3((unsigned)blocks), dim3(256), 0, st, kin, vin, n, shift,
+        if (int rc = exclusive_scan_into(hist.p, hist.p, blocks * kBins, sums.p, st)) return rc;
+        const int64_t scatter_grid = (blocks + kXcds - 1) / kXcds * kXcds;
+        hipLaunchKernelGGL((radix_scatter_kernel<KeyT>), dim3((unsigned)scatter_grid), dim3(256), 0, st, kin, vin, n, shift,
                            hist.p, blocks, kout, vout);
         GNNAGG_HIP(hipGetLastError());
         std::swap(kin, kout);
         std::swap(vin, vout);
         *result_in_b = !*result_in_b;
     }
-    GNNAGG_HIP(hipStreamSynchronize(st));  // the histogram is released on scope exit
+    GNNAGG_HIP(hipStreamSynchronize(st));  // the histogram and the tile sums are released on scope exit
     return GNNAGG_OK;
 }
 

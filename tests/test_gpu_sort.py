@@ -9,7 +9,8 @@ from gnn_benchmark_amd.data_manager import device_ops
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("n", [0, 1, 2, 63, 64, 255, 256, 257, 4095, 4096, 4097, 8193, 100_003, 1_000_003])
+@pytest.mark.parametrize("n", [0, 1, 2, 63, 64, 255, 256, 257, 2047, 2048, 2049, 4097, 8191, 8192, 8193, 16385, 65_537,
+                               100_003, 1_000_003])
 @pytest.mark.parametrize("span", [1, 5, 300, 70_000, 1 << 33, (1 << 62) + 12345])
 def test_argsort_is_the_stable_ascending_order(n, span):
     """Few distinct keys (long runs of equal keys: stability), keys of 1 .. 8 radix passes, sizes around the tile and
