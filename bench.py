@@ -769,16 +769,26 @@ def build_c4(args):
                                      local_mean_out_degree=6.8, zipf_s=1.8, max_degree=15000,
                                      num_halo_nodes=int(args.c4_nodes * 3 / 7),
                                      num_remote_edges=int(args.c4_nodes * 20 / 7), seed=args.seed + 4, device=dev)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
     # stand-in rows on the scale of real ones: features O(0.1), gradients of a mean loss O(1e-7)
     # (the seeded rows are drawn once per layer and direction and kept on the device; a step points the boundary
     # buffers at them -- no random-number work, and no other work of the stand-in, inside a timed step)
     exchange = synthetic.PregeneratedHaloExchange(args.seed + 4, std=0.1, backward_std=1e-7)
     graph = synthetic.build_partition_graph(part, 256, True, exchange=exchange, device=dev)
+    torch.cuda.synchronize()
+    t2 = time.perf_counter()
     for m in (graph.local_adj_t, graph.adj_t_pre_post_aggr_from, graph.adj_t_pre_post_aggr_to):
         m.get_plan()
         m.get_plan_for_transpose()
     torch.cuda.synchronize()
-    return part, graph, time.perf_counter() - t0
+    t3 = time.perf_counter()
+    # what the set-up time is made of: the synthetic edge lists (not part of the path), the index-map builders with
+    # the three matrices and the buffers (the reference's DataProcessor loops), the six degree-ordered plans with the
+    # transposed arrays behind three of them
+    setup = {"total": round(t3 - t0, 3), "synthetic_edge_lists": round(t1 - t0, 3),
+             "index_maps_matrices_buffers": round(t2 - t1, 3), "plans_and_transposed_arrays": round(t3 - t2, 3)}
+    return part, graph, setup
 
 
 def run_c4(args, graph, setup_s, gate=None):
@@ -1047,7 +1057,8 @@ def run_c4(args, graph, setup_s, gate=None):
                       "gbs": round(src.numel() * 6.0 / (ms * 1e-3) / 1e9, 1),
                       "frac_of_hbm_peak": round(src.numel() * 6.0 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)})
     graph.comm_buf, graph.exchange_bf16 = fp32_buf, None
-    return {"partition": f"rank 3 of 16, {n} local nodes", "feat": feat, "setup_s": round(setup_s, 2), "codec": codec,
+    return {"partition": f"rank 3 of 16, {n} local nodes", "feat": feat, "setup_s": round(setup_s["total"], 2),
+            "setup_breakdown_s": setup_s, "codec": codec,
             "local_nnz": graph.local_adj_t.nnz(), "halo_rows": int(recv_buf.size(0)), "send_rows": int(send_buf.size(0)),
             "from_nnz": graph.adj_t_pre_post_aggr_from.nnz(), "to_nnz": graph.adj_t_pre_post_aggr_to.nnz(),
             "ops": ops, "aggregator_forward_ms": round(fwd_ms, 3),
@@ -1361,21 +1372,23 @@ def run_c5(args, graph):
         out[f"loss_{tag}"] = [round(v, 5) for v in losses + [float(loss)]]
         del model, opt
     del folded
-    # the default step with the local and the received elements of every output row in one launch (graph.one_launch)
+    # the default step with the local and the received elements of every output row in one launch (graph.one_launch),
+    # in each form of the dense products
     graph.one_launch = True
-    torch.manual_seed(args.seed)
-    model = gcn.GCN(dims).to(dev)
-    opt = torch.optim.Adam(model.parameters(), lr=0.01)
-    losses = [float(gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks)) for _ in range(2)]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        loss = gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks)
-    torch.cuda.synchronize()
-    out["train_step_ms_fp32_gemm_one_launch_aggregation"] = round((time.perf_counter() - t0) * 1e3 / steps, 2)
-    out["loss_fp32_gemm_one_launch_aggregation"] = [round(v, 5) for v in losses + [float(loss)]]
+    for gemm in ("fp32", "bf16x3", "bf16"):
+        torch.manual_seed(args.seed)
+        model = gcn.GCN(dims, gemm=gemm).to(dev)
+        opt = torch.optim.Adam(model.parameters(), lr=0.01)
+        losses = [float(gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks)) for _ in range(2)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            loss = gcn.train_step(model, opt, graph, x, labels, train_idx, True, masks)
+        torch.cuda.synchronize()
+        out[f"train_step_ms_{gemm}_gemm_one_launch_aggregation"] = round((time.perf_counter() - t0) * 1e3 / steps, 2)
+        out[f"loss_{gemm}_gemm_one_launch_aggregation"] = [round(v, 5) for v in losses + [float(loss)]]
+        del model, opt
     graph.one_launch = False
-    del model, opt
     from gnn_benchmark_amd import synthetic
     from gnn_benchmark_amd.data_manager import CommBuffer, CommBufferForQuantization, CommSplits
 
@@ -1630,7 +1643,7 @@ def main():
             c5 = sink.put("c5", run_c5(args, graph))
             targets["c5_gcn_train_step_ms"] = {k[len("train_step_ms_"):]: c5[k] for k in (
                 "train_step_ms_fp32_gemm", "train_step_ms_bf16_gemm", "train_step_ms_bf16x3_gemm",
-                "train_step_ms_fp32_gemm_one_launch_aggregation",
+                "train_step_ms_fp32_gemm_one_launch_aggregation", "train_step_ms_bf16x3_gemm_one_launch_aggregation",
                 "train_step_ms_fp32_gemm_all_nodes_through_last_layer", "train_step_ms_fp32_gemm_int2_exchange",
                 "train_step_ms_fp32_gemm_int2_exchange_one_launch_aggregation")
                 if k in c5}

@@ -12,7 +12,7 @@ _CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(_CSRC, "libgnnagg.so")
 
 OK, ERR_INVALID, ERR_HIP, ERR_UNSUPPORTED = 0, 1, 2, 3
-ABI_VERSION = 5   # GNNAGG_ABI_VERSION of include/gnn_agg.h this binding was written against
+ABI_VERSION = 6   # GNNAGG_ABI_VERSION of include/gnn_agg.h this binding was written against
 
 EXPORTS = (
     "gnnagg_abi_version",
@@ -32,7 +32,9 @@ EXPORTS = (
     "gnnagg_plan_profile_read",
     "gnnagg_csr_transpose",
     "gnnagg_coo_to_csr",
+    "gnnagg_argsort_workspace_bytes",
     "gnnagg_argsort_i64",
+    "gnnagg_runs_workspace_bytes",
     "gnnagg_runs_i64",
     "gnnagg_gather_rows_f32",
     "gnnagg_gather_rows_f32_bf16",
@@ -150,9 +152,12 @@ def lib() -> ctypes.CDLL:
     L.gnnagg_coo_to_csr.restype = i32
     L.gnnagg_coo_to_csr.argtypes = [vp, vp, vp, i64, i64, i64, vp, vp, vp, vp]
     L.gnnagg_argsort_i64.restype = i32
-    L.gnnagg_argsort_i64.argtypes = [vp, i64, vp, vp, vp]
+    L.gnnagg_argsort_i64.argtypes = [vp, i64, vp, vp, vp, i64, vp]
     L.gnnagg_runs_i64.restype = i32
-    L.gnnagg_runs_i64.argtypes = [vp, i64, vp, i64, vp, vp, vp, ctypes.POINTER(i64), vp]
+    L.gnnagg_runs_i64.argtypes = [vp, i64, vp, i64, vp, vp, vp, ctypes.POINTER(i64), vp, i64, vp]
+    for name in ("gnnagg_argsort_workspace_bytes", "gnnagg_runs_workspace_bytes"):
+        getattr(L, name).restype = i64
+        getattr(L, name).argtypes = [i64]
     L.gnnagg_gather_rows_f32.restype = i32
     L.gnnagg_gather_rows_f32.argtypes = [vp, i64, vp, vp, i64, i64, vp]
     L.gnnagg_gather_rows_f32_bf16.restype = i32

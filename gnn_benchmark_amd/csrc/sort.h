@@ -7,12 +7,14 @@
 namespace gnnagg {
 
 // Stable ascending sort of n pairs by the low `bits` bits of the key, 8 bits a pass, ping-pong between the (a) and
-// (b) arrays: the input is in (key_a, val_a); *result_in_b says where the sorted pairs ended up.  Allocates its
-// histogram, synchronises `st` before it returns.
+// (b) arrays: the input is in (key_a, val_a); *result_in_b says where the sorted pairs ended up.  `workspace`:
+// sort_pairs_workspace_bytes(n) bytes of device memory (the histograms), 256-byte aligned -- the call then only
+// enqueues on `st`; nullptr: the call allocates them and synchronises `st` before it returns.
+size_t sort_pairs_workspace_bytes(int64_t n);
 int sort_pairs_u64(uint64_t *key_a, uint64_t *key_b, uint32_t *val_a, uint32_t *val_b, int64_t n, int bits,
-                   hipStream_t st, bool *result_in_b);
+                   hipStream_t st, bool *result_in_b, void *workspace = nullptr);
 int sort_pairs_u32(uint32_t *key_a, uint32_t *key_b, uint32_t *val_a, uint32_t *val_b, int64_t n, int bits,
-                   hipStream_t st, bool *result_in_b);
+                   hipStream_t st, bool *result_in_b, void *workspace = nullptr);
 
 // out[i] = in[0] + ... + in[i - 1] for sums below 2^32 (in == out is fine).  Synchronises `st` before it returns.
 int exclusive_scan_u32(const uint32_t *in, uint32_t *out, int64_t n, hipStream_t st);

@@ -250,50 +250,67 @@ __global__ __launch_bounds__(256) void radix_scatter_kernel(const KeyT *__restri
     }
 }
 
+size_t align_up(size_t bytes) { return (bytes + 255) & ~size_t(255); }
+
+size_t sort_hist_bytes(int64_t n) { return align_up((size_t)((n + kTile - 1) / kTile) * kBins * sizeof(uint32_t)); }
+size_t sort_sums_bytes(int64_t n) {
+    return align_up((size_t)scan_tiles((n + kTile - 1) / kTile * kBins) * sizeof(uint32_t));
+}
+
 template <typename KeyT>
 int radix_sort_pairs(KeyT *key_a, KeyT *key_b, uint32_t *val_a, uint32_t *val_b, int64_t n, int bits, hipStream_t st,
-                     bool *result_in_b) {
+                     bool *result_in_b, void *workspace) {
     *result_in_b = false;
     if (n <= 0 || bits <= 0) return GNNAGG_OK;
     GNNAGG_REQUIRE(n < (int64_t(1) << 32), "radix sort of more than 2^32-1 pairs");
     const int64_t blocks = (n + kTile - 1) / kTile;
-    DevBuf<uint32_t> hist, sums;
-    GNNAGG_HIP(hist.alloc((size_t)(blocks * kBins)));
-    GNNAGG_HIP(sums.alloc((size_t)scan_tiles(blocks * kBins)));
+    DevBuf<char> own;
+    if (!workspace) {
+        GNNAGG_HIP(own.alloc(sort_pairs_workspace_bytes(n)));
+        workspace = own.p;
+    }
+    uint32_t *hist = static_cast<uint32_t *>(workspace);
+    uint32_t *sums = reinterpret_cast<uint32_t *>(static_cast<char *>(workspace) + sort_hist_bytes(n));
     KeyT *kin = key_a, *kout = key_b;
     uint32_t *vin = val_a, *vout = val_b;
     for (int shift = 0; shift < bits; shift += kRadixBits) {
         hipLaunchKernelGGL((radix_histogram_kernel<KeyT>), dim3((unsigned)blocks), dim3(256), 0, st, kin, n, shift,
-                           hist.p, blocks);
+                           hist, blocks);
         GNNAGG_HIP(hipGetLastError());
-        if (int rc = exclusive_scan_into(hist.p, hist.p, blocks * kBins, sums.p, st)) return rc;
+        if (int rc = exclusive_scan_into(hist, hist, blocks * kBins, sums, st)) return rc;
         const int64_t scatter_grid = (blocks + kXcds - 1) / kXcds * kXcds;
         hipLaunchKernelGGL((radix_scatter_kernel<KeyT>), dim3((unsigned)scatter_grid), dim3(256), 0, st, kin, vin, n, shift,
-                           hist.p, blocks, kout, vout);
+                           hist, blocks, kout, vout);
         GNNAGG_HIP(hipGetLastError());
         std::swap(kin, kout);
         std::swap(vin, vout);
         *result_in_b = !*result_in_b;
     }
-    GNNAGG_HIP(hipStreamSynchronize(st));  // the histogram and the tile sums are released on scope exit
+    if (own.p) GNNAGG_HIP(hipStreamSynchronize(st));  // its own workspace is released on scope exit
     return GNNAGG_OK;
 }
 
 }  // namespace
 
+size_t sort_pairs_workspace_bytes(int64_t n) { return n > 0 ? sort_hist_bytes(n) + sort_sums_bytes(n) : 0; }
+
 int sort_pairs_u64(uint64_t *key_a, uint64_t *key_b, uint32_t *val_a, uint32_t *val_b, int64_t n, int bits,
-                   hipStream_t st, bool *result_in_b) {
-    return radix_sort_pairs<uint64_t>(key_a, key_b, val_a, val_b, n, bits, st, result_in_b);
+                   hipStream_t st, bool *result_in_b, void *workspace) {
+    return radix_sort_pairs<uint64_t>(key_a, key_b, val_a, val_b, n, bits, st, result_in_b, workspace);
 }
 
 int sort_pairs_u32(uint32_t *key_a, uint32_t *key_b, uint32_t *val_a, uint32_t *val_b, int64_t n, int bits,
-                   hipStream_t st, bool *result_in_b) {
-    return radix_sort_pairs<uint32_t>(key_a, key_b, val_a, val_b, n, bits, st, result_in_b);
+                   hipStream_t st, bool *result_in_b, void *workspace) {
+    return radix_sort_pairs<uint32_t>(key_a, key_b, val_a, val_b, n, bits, st, result_in_b, workspace);
 }
 
 namespace {
 
 // ------------------------------------------------------------------ argsort / runs of a sorted list
+__global__ void fill_u32_kernel(uint32_t *p, int count, uint32_t v) {
+    if ((int)threadIdx.x < count) p[threadIdx.x] = v;
+}
+
 __global__ __launch_bounds__(256) void argsort_prepare_kernel(const int64_t *__restrict__ x, int64_t n,
                                                               uint64_t *__restrict__ key, uint32_t *__restrict__ idx,
                                                               unsigned long long *__restrict__ max_key,
@@ -365,41 +382,79 @@ __global__ __launch_bounds__(256) void run_counts_kernel(const int64_t *__restri
 
 using namespace gnnagg;
 
-extern "C" int gnnagg_argsort_i64(const int64_t *x, int64_t n, int64_t *perm, int64_t *sorted, void *stream) {
+namespace {
+
+// The temporaries of one call, carved out of the caller's workspace or, without one, out of one allocation of the
+// call's own (released when the call returns, which then has to wait for its kernels).
+struct Carver {
+    char *at = nullptr;
+    DevBuf<char> own;
+    int open(void *workspace, int64_t workspace_bytes, size_t need) {
+        if (workspace) {
+            GNNAGG_REQUIRE(workspace_bytes >= (int64_t)need, "workspace smaller than the *_workspace_bytes of this size");
+            GNNAGG_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 15) == 0, "workspace not 16-byte aligned");
+            at = static_cast<char *>(workspace);
+        } else {
+            GNNAGG_HIP(own.alloc(need));
+            at = own.p;
+        }
+        return GNNAGG_OK;
+    }
+    template <typename T>
+    T *take(size_t count) {
+        T *p = reinterpret_cast<T *>(at);
+        at += align_up(count * sizeof(T));
+        return p;
+    }
+};
+
+size_t argsort_bytes(int64_t n) {
+    return 2 * align_up((size_t)n * 8) + 2 * align_up((size_t)n * 4) + align_up(16) + sort_pairs_workspace_bytes(n);
+}
+size_t runs_bytes(int64_t n) {
+    return 2 * align_up((size_t)n * 4) + align_up((size_t)n * 8) + align_up((size_t)scan_tiles(n) * 4);
+}
+
+}  // namespace
+
+extern "C" int64_t gnnagg_argsort_workspace_bytes(int64_t n) { return n > 0 ? (int64_t)argsort_bytes(n) : 0; }
+extern "C" int64_t gnnagg_runs_workspace_bytes(int64_t n) { return n > 0 ? (int64_t)runs_bytes(n) : 0; }
+
+extern "C" int gnnagg_argsort_i64(const int64_t *x, int64_t n, int64_t *perm, int64_t *sorted, void *workspace,
+                                  int64_t workspace_bytes, void *stream) {
     GNNAGG_REQUIRE(n >= 0, "negative size");
     if (n == 0) return GNNAGG_OK;
     GNNAGG_REQUIRE(x && perm, "null x/perm");
     if (n >= (int64_t(1) << 32)) return fail(GNNAGG_ERR_UNSUPPORTED, "argsort of more than 2^32-1 values");
     hipStream_t st = static_cast<hipStream_t>(stream);
-    DevBuf<uint64_t> key_a, key_b;
-    DevBuf<uint32_t> idx_a, idx_b;
-    DevBuf<unsigned long long> flags;  // [0] the largest key, [1] whether a key was negative
-    GNNAGG_HIP(key_a.alloc((size_t)n));
-    GNNAGG_HIP(key_b.alloc((size_t)n));
-    GNNAGG_HIP(idx_a.alloc((size_t)n));
-    GNNAGG_HIP(idx_b.alloc((size_t)n));
-    GNNAGG_HIP(flags.alloc(2));
-    GNNAGG_HIP(hipMemsetAsync(flags.p, 0, 2 * sizeof(unsigned long long), st));
+    Carver ws;
+    if (int rc = ws.open(workspace, workspace_bytes, argsort_bytes(n))) return rc;
+    uint64_t *key_a = ws.take<uint64_t>((size_t)n), *key_b = ws.take<uint64_t>((size_t)n);
+    uint32_t *idx_a = ws.take<uint32_t>((size_t)n), *idx_b = ws.take<uint32_t>((size_t)n);
+    unsigned long long *flags = ws.take<unsigned long long>(2);  // [0] the largest key, [1] whether a key was negative
+    void *sort_ws = ws.take<char>(sort_pairs_workspace_bytes(n));
     const unsigned grid = (unsigned)std::min<int64_t>((n + 255) / 256, 256 * 32);
-    hipLaunchKernelGGL(argsort_prepare_kernel, dim3(grid), dim3(256), 0, st, x, n, key_a.p, idx_a.p, flags.p,
-                       reinterpret_cast<unsigned int *>(flags.p + 1));
+    hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(64), 0, st, reinterpret_cast<uint32_t *>(flags), 4, 0u);
+    hipLaunchKernelGGL(argsort_prepare_kernel, dim3(grid), dim3(256), 0, st, x, n, key_a, idx_a, flags,
+                       reinterpret_cast<unsigned int *>(flags + 1));
     GNNAGG_HIP(hipGetLastError());
     unsigned long long h[2] = {0, 0};
-    GNNAGG_HIP(hipMemcpyAsync(h, flags.p, sizeof(h), hipMemcpyDeviceToHost, st));
+    GNNAGG_HIP(hipMemcpyAsync(h, flags, sizeof(h), hipMemcpyDeviceToHost, st));
     GNNAGG_HIP(hipStreamSynchronize(st));
     GNNAGG_REQUIRE((h[1] & 0xffffffffull) == 0, "argsort takes non-negative keys (node ids, positions)");
     const int bits = h[0] ? ceil_log2_u64(h[0] + 1) : 1;
     bool in_b = false;
-    if (int rc = sort_pairs_u64(key_a.p, key_b.p, idx_a.p, idx_b.p, n, bits, st, &in_b)) return rc;
-    hipLaunchKernelGGL(argsort_finish_kernel, dim3(grid_for(n, 256)), dim3(256), 0, st, in_b ? key_b.p : key_a.p,
-                       in_b ? idx_b.p : idx_a.p, n, perm, sorted);
+    if (int rc = sort_pairs_u64(key_a, key_b, idx_a, idx_b, n, bits, st, &in_b, sort_ws)) return rc;
+    hipLaunchKernelGGL(argsort_finish_kernel, dim3(grid_for(n, 256)), dim3(256), 0, st, in_b ? key_b : key_a,
+                       in_b ? idx_b : idx_a, n, perm, sorted);
     GNNAGG_HIP(hipGetLastError());
-    GNNAGG_HIP(hipStreamSynchronize(st));
+    if (ws.own.p) GNNAGG_HIP(hipStreamSynchronize(st));
     return GNNAGG_OK;
 }
 
 extern "C" int gnnagg_runs_i64(const int64_t *x, int64_t n, const int64_t *forced_starts, int64_t forced_count,
-                               int64_t *uniq, int64_t *inverse, int64_t *counts, int64_t *runs_out, void *stream) {
+                               int64_t *uniq, int64_t *inverse, int64_t *counts, int64_t *runs_out, void *workspace,
+                               int64_t workspace_bytes, void *stream) {
     GNNAGG_REQUIRE(n >= 0 && forced_count >= 0, "negative size");
     GNNAGG_REQUIRE(runs_out, "null runs_out");
     *runs_out = 0;
@@ -408,32 +463,32 @@ extern "C" int gnnagg_runs_i64(const int64_t *x, int64_t n, const int64_t *force
     GNNAGG_REQUIRE(forced_count == 0 || forced_starts, "null forced_starts");
     if (n >= (int64_t(1) << 32)) return fail(GNNAGG_ERR_UNSUPPORTED, "run detection over more than 2^32-1 values");
     hipStream_t st = static_cast<hipStream_t>(stream);
-    DevBuf<uint32_t> flag, before;
-    DevBuf<int64_t> run_start;
-    GNNAGG_HIP(flag.alloc((size_t)n));
-    GNNAGG_HIP(before.alloc((size_t)n));
-    GNNAGG_HIP(run_start.alloc((size_t)n));
-    hipLaunchKernelGGL(run_flags_kernel, dim3(grid_for(n, 256)), dim3(256), 0, st, x, n, flag.p);
+    Carver ws;
+    if (int rc = ws.open(workspace, workspace_bytes, runs_bytes(n))) return rc;
+    uint32_t *flag = ws.take<uint32_t>((size_t)n), *before = ws.take<uint32_t>((size_t)n);
+    int64_t *run_start = ws.take<int64_t>((size_t)n);
+    uint32_t *sums = ws.take<uint32_t>((size_t)scan_tiles(n));
+    hipLaunchKernelGGL(run_flags_kernel, dim3(grid_for(n, 256)), dim3(256), 0, st, x, n, flag);
     GNNAGG_HIP(hipGetLastError());
     if (forced_count > 0) {
         hipLaunchKernelGGL(force_starts_kernel, dim3(grid_for(forced_count, 256)), dim3(256), 0, st, forced_starts,
-                           forced_count, n, flag.p);
+                           forced_count, n, flag);
         GNNAGG_HIP(hipGetLastError());
     }
-    if (int rc = exclusive_scan_u32(flag.p, before.p, n, st)) return rc;
+    if (int rc = exclusive_scan_into(flag, before, n, sums, st)) return rc;
     uint32_t last[2] = {0, 0};
-    GNNAGG_HIP(hipMemcpyAsync(&last[0], before.p + (n - 1), sizeof(uint32_t), hipMemcpyDeviceToHost, st));
-    GNNAGG_HIP(hipMemcpyAsync(&last[1], flag.p + (n - 1), sizeof(uint32_t), hipMemcpyDeviceToHost, st));
-    GNNAGG_HIP(hipStreamSynchronize(st));
+    GNNAGG_HIP(hipMemcpyAsync(&last[0], before + (n - 1), sizeof(uint32_t), hipMemcpyDeviceToHost, st));
+    GNNAGG_HIP(hipMemcpyAsync(&last[1], flag + (n - 1), sizeof(uint32_t), hipMemcpyDeviceToHost, st));
+    GNNAGG_HIP(hipStreamSynchronize(st));  // the number of runs sizes the last launch and is what the call returns
     const int64_t runs = (int64_t)last[0] + (int64_t)last[1];
-    hipLaunchKernelGGL(run_outputs_kernel, dim3(grid_for(n, 256)), dim3(256), 0, st, x, flag.p, before.p, n, uniq, inverse,
-                       run_start.p);
+    hipLaunchKernelGGL(run_outputs_kernel, dim3(grid_for(n, 256)), dim3(256), 0, st, x, flag, before, n, uniq, inverse,
+                       run_start);
     GNNAGG_HIP(hipGetLastError());
     if (counts) {
-        hipLaunchKernelGGL(run_counts_kernel, dim3(grid_for(runs, 256)), dim3(256), 0, st, run_start.p, runs, n, counts);
+        hipLaunchKernelGGL(run_counts_kernel, dim3(grid_for(runs, 256)), dim3(256), 0, st, run_start, runs, n, counts);
         GNNAGG_HIP(hipGetLastError());
     }
-    GNNAGG_HIP(hipStreamSynchronize(st));
+    if (ws.own.p) GNNAGG_HIP(hipStreamSynchronize(st));
     *runs_out = runs;
     return GNNAGG_OK;
 }

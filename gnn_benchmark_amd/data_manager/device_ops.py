@@ -15,15 +15,23 @@ def _on_gpu(x: torch.Tensor) -> bool:
     return x.is_cuda and x.dtype == torch.int64 and x.dim() == 1
 
 
+def _workspace(nbytes: int, device) -> torch.Tensor:
+    """The kernels' temporaries, from torch's caching allocator (a call with no workspace allocates from the driver)."""
+    return torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=device)
+
+
 def stable_argsort(x: torch.Tensor) -> torch.Tensor:
     """Positions that put ``x`` in ascending order, equal values in their input order."""
     if not _on_gpu(x) or x.numel() == 0:
         return torch.sort(x, stable=True).indices
     x = x.contiguous()
     perm = torch.empty_like(x)
+    L = _lib.lib()
+    nbytes = int(L.gnnagg_argsort_workspace_bytes(x.numel()))
+    workspace = _workspace(nbytes, x.device)
     with torch.cuda.device(x.device):
-        _lib.check(_lib.lib().gnnagg_argsort_i64(_lib.ptr(x), x.numel(), _lib.ptr(perm), None,
-                                                 _lib.current_stream(x.device)))
+        _lib.check(L.gnnagg_argsort_i64(_lib.ptr(x), x.numel(), _lib.ptr(perm), None, _lib.ptr(workspace), nbytes,
+                                        _lib.current_stream(x.device)))
     return perm
 
 
@@ -50,10 +58,13 @@ def runs(x: torch.Tensor, forced_starts: Optional[torch.Tensor] = None, want_val
     counts = torch.empty_like(x) if want_counts else None
     forced = None if forced_starts is None else forced_starts.to(device=x.device, dtype=torch.int64).contiguous()
     found = ctypes.c_int64(0)
+    L = _lib.lib()
+    nbytes = int(L.gnnagg_runs_workspace_bytes(n))
+    workspace = _workspace(nbytes, x.device)
     with torch.cuda.device(x.device):
-        _lib.check(_lib.lib().gnnagg_runs_i64(_lib.ptr(x), n, _lib.ptr(forced), 0 if forced is None else forced.numel(),
-                                              _lib.ptr(values), _lib.ptr(inverse), _lib.ptr(counts), ctypes.byref(found),
-                                              _lib.current_stream(x.device)))
+        _lib.check(L.gnnagg_runs_i64(_lib.ptr(x), n, _lib.ptr(forced), 0 if forced is None else forced.numel(),
+                                     _lib.ptr(values), _lib.ptr(inverse), _lib.ptr(counts), ctypes.byref(found),
+                                     _lib.ptr(workspace), nbytes, _lib.current_stream(x.device)))
     k = int(found.value)
     return (None if values is None else values[:k], inverse, None if counts is None else counts[:k])
 

@@ -28,9 +28,10 @@ extern "C" {
 
 /* Raised whenever an exported prototype changes, an entry point goes away or the meaning of an argument changes
  * (2: `src_rows` in the row gathers, `workspace_bytes` in the weight-gradient entry points, 12 values from
- * gnnagg_plan_info; 3: the measurement probes left the library, gnnagg_plan_spmm_two_sources_f32 and gnnagg_plans_release came; 4: the two gnnagg_plan_spmm_dense_then_* entry points came; 5: gnnagg_argsort_i64 and gnnagg_runs_i64 came).  Every binding compares it with
+ * gnnagg_plan_info; 3: the measurement probes left the library, gnnagg_plan_spmm_two_sources_f32 and gnnagg_plans_release came; 4: the two gnnagg_plan_spmm_dense_then_* entry points came; 5: gnnagg_argsort_i64 and gnnagg_runs_i64 came; 6: both take a workspace, gnnagg_argsort_workspace_bytes and
+ * gnnagg_runs_workspace_bytes came).  Every binding compares it with
  * gnnagg_abi_version() of the library it loaded before the first call. */
-#define GNNAGG_ABI_VERSION 5
+#define GNNAGG_ABI_VERSION 6
 
 /* Version of this ABI (GNNAGG_ABI_VERSION of the built library).  No reference counterpart. */
 int gnnagg_abi_version(void);
@@ -216,8 +217,10 @@ int gnnagg_coo_to_csr(const int64_t *row, const int64_t *col, const float *value
                       int64_t cols, int64_t *rowptr, int64_t *col_out, float *value_out, void *stream);
 
 /* ---------------------------------------------------------------------------------
- * Sorting and run detection for the index-map builders (set-up time; both allocate temporaries and SYNCHRONISE the
- * stream).  The reference walks sorted edge lists with per-edge Python loops
+ * Sorting and run detection for the index-map builders (set-up time).  `workspace`: device memory of at least
+ * gnnagg_*_workspace_bytes(n) bytes, 16-byte aligned, for the call's temporaries; NULL: the call allocates them itself
+ * and waits for its kernels before it returns.  gnnagg_argsort_i64 waits for the stream once either way (the
+ * largest key decides the number of passes), gnnagg_runs_i64 too (the number of runs).  The reference walks sorted edge lists with per-edge Python loops
  * (data_manager/DataProcessor.py:39-53 halo renumbering, :238-246 pre/post decision, :434-444 buffer-row
  * renumbering) after `torch.argsort` (:21, :259, :306) and `torch.unique` (:127); on the device the same maps are
  * a stable sort plus the run structure of the sorted list.
@@ -233,9 +236,13 @@ int gnnagg_coo_to_csr(const int64_t *row, const int64_t *col, const float *value
  * each position, counts int64 [runs] the length of each run (all three arrays sized n by the caller); *runs_out
  * (host) the number of runs.
  * ------------------------------------------------------------------------------- */
-int gnnagg_argsort_i64(const int64_t *x, int64_t n, int64_t *perm, int64_t *sorted, void *stream);
+int64_t gnnagg_argsort_workspace_bytes(int64_t n);
+int gnnagg_argsort_i64(const int64_t *x, int64_t n, int64_t *perm, int64_t *sorted, void *workspace,
+                       int64_t workspace_bytes, void *stream);
+int64_t gnnagg_runs_workspace_bytes(int64_t n);
 int gnnagg_runs_i64(const int64_t *x, int64_t n, const int64_t *forced_starts, int64_t forced_count, int64_t *uniq,
-                    int64_t *inverse, int64_t *counts, int64_t *runs_out, void *stream);
+                    int64_t *inverse, int64_t *counts, int64_t *runs_out, void *workspace, int64_t workspace_bytes,
+                    void *stream);
 
 /* ---------------------------------------------------------------------------------
  * Boundary-row gather, out[i,:] = src[index[i],:].  Replaces

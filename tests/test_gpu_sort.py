@@ -67,3 +67,31 @@ def test_unique_and_occurrences_equal_torch(n):
     assert torch.equal(device_ops.unique_sorted(x.cuda()).cpu(), torch.unique(x, sorted=True))
     _, inverse, counts = torch.unique(x, return_inverse=True, return_counts=True)
     assert torch.equal(device_ops.occurrences_per_entry(x.cuda()).cpu(), counts[inverse])
+
+
+def test_calls_without_a_workspace_allocate_their_own_and_a_short_workspace_is_refused():
+    import ctypes
+
+    from gnn_benchmark_amd import _lib
+
+    L = _lib.lib()
+    n = 50_001
+    x = torch.from_numpy(np.random.default_rng(5).integers(0, 900, n, dtype=np.int64)).cuda()
+    perm, ordered = torch.empty_like(x), torch.empty_like(x)
+    stream = _lib.current_stream(x.device)
+    _lib.check(L.gnnagg_argsort_i64(_lib.ptr(x), n, _lib.ptr(perm), _lib.ptr(ordered), None, 0, stream))
+    assert torch.equal(perm, device_ops.stable_argsort(x)) and torch.equal(ordered, x[perm])
+    values, counts = torch.empty_like(x), torch.empty_like(x)
+    found = ctypes.c_int64(0)
+    _lib.check(L.gnnagg_runs_i64(_lib.ptr(ordered), n, None, 0, _lib.ptr(values), None, _lib.ptr(counts),
+                                 ctypes.byref(found), None, 0, stream))
+    want_values, want_counts = torch.unique_consecutive(ordered, return_counts=True)
+    k = int(found.value)
+    assert k == want_values.numel()
+    assert torch.equal(values[:k], want_values) and torch.equal(counts[:k], want_counts)
+    short = torch.empty(int(L.gnnagg_argsort_workspace_bytes(n)) - 256, dtype=torch.uint8, device="cuda")
+    with pytest.raises(_lib.GnnAggError, match="workspace"):
+        _lib.check(L.gnnagg_argsort_i64(_lib.ptr(x), n, _lib.ptr(perm), None, _lib.ptr(short), short.numel(), stream))
+    with pytest.raises(_lib.GnnAggError, match="workspace"):
+        _lib.check(L.gnnagg_runs_i64(_lib.ptr(ordered), n, None, 0, _lib.ptr(values), None, None, ctypes.byref(found),
+                                     _lib.ptr(short), 64, stream))

@@ -38,7 +38,7 @@ def _prototype_digest():
 # GNNAGG_ABI_VERSION -> digest of the prototypes it stands for.  A changed, added or removed prototype changes the
 # digest: raise GNNAGG_ABI_VERSION (header) and ABI_VERSION (_lib.py) together and record the new pair here, so that a
 # library or extension module built from the old header is refused instead of being called with shifted arguments.
-ABI_DIGESTS = {5: "d8a30016c7791f4b"}
+ABI_DIGESTS = {6: "d32bfa6402ead32b"}
 
 
 def test_a_changed_prototype_needs_a_new_abi_version():
