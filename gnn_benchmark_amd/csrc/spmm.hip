@@ -185,15 +185,17 @@ hipError_t launch_long_rows(const LongArgs &a, int64_t nrows, hipStream_t st) {
     int chunk = kLongMaxChunk;
     if (chunk * vpr > 256 * kLongLoads) chunk = 256 * kLongLoads / vpr;
     if (chunk * tile > kLongTileFloats) chunk = kLongTileFloats / tile;
+    chunk &= ~3;  // the chain reads a chunk's elements four at a time, 16-byte aligned
     args.chunk = chunk;
     const unsigned tiles = (unsigned)((a.feat + tile - 1) / tile);
     const int slots = chunk * vpr;  // vectors of a whole chunk; 256 threads fetch them in NL rounds
     const dim3 grid((unsigned)nrows, tiles);
+    const dim3 block((unsigned)(kLongFetchThreads + 64 * ((tile + 63) / 64)));  // fetch waves + one chain wave per 64 features
     if (VEC == 4 && slots > 1024 && a.feat % tile == 0 && tile >= 16 && (tile & (tile - 1)) == 0) {
         // every tile has the same power-of-two width: the instance that knows it at compile time
 #define GNNAGG_LONG_FIXED(W)                                                                                     \
     if (tile == W)                                                                                               \
-        hipLaunchKernelGGL((spmm_long_rows_kernel<4, 8, W>), grid, dim3(256), kLongSmemBytes, st, args)
+        hipLaunchKernelGGL((spmm_long_rows_kernel<4, 8, W>), grid, block, kLongSmemBytes, st, args)
         GNNAGG_LONG_FIXED(16);
         GNNAGG_LONG_FIXED(32);
         GNNAGG_LONG_FIXED(64);
@@ -202,10 +204,10 @@ hipError_t launch_long_rows(const LongArgs &a, int64_t nrows, hipStream_t st) {
 #undef GNNAGG_LONG_FIXED
         return hipGetLastError();
     }
-    if (slots <= 256) hipLaunchKernelGGL((spmm_long_rows_kernel<VEC, 1>), grid, dim3(256), kLongSmemBytes, st, args);
-    else if (slots <= 512) hipLaunchKernelGGL((spmm_long_rows_kernel<VEC, 2>), grid, dim3(256), kLongSmemBytes, st, args);
-    else if (slots <= 1024) hipLaunchKernelGGL((spmm_long_rows_kernel<VEC, 4>), grid, dim3(256), kLongSmemBytes, st, args);
-    else hipLaunchKernelGGL((spmm_long_rows_kernel<VEC, 8>), grid, dim3(256), kLongSmemBytes, st, args);
+    if (slots <= 256) hipLaunchKernelGGL((spmm_long_rows_kernel<VEC, 1>), grid, block, kLongSmemBytes, st, args);
+    else if (slots <= 512) hipLaunchKernelGGL((spmm_long_rows_kernel<VEC, 2>), grid, block, kLongSmemBytes, st, args);
+    else if (slots <= 1024) hipLaunchKernelGGL((spmm_long_rows_kernel<VEC, 4>), grid, block, kLongSmemBytes, st, args);
+    else hipLaunchKernelGGL((spmm_long_rows_kernel<VEC, 8>), grid, block, kLongSmemBytes, st, args);
     return hipGetLastError();
 }
 

@@ -43,6 +43,7 @@ struct FVec<1> {
     __device__ __forceinline__ void store_stream(float *p) const { __builtin_nontemporal_store(d, p); }
     __device__ __forceinline__ void fma(float a, const FVec &x) { d = __builtin_fmaf(a, x.d, d); }
     __device__ __forceinline__ void add(const FVec &x) { d += x.d; }
+    __device__ __forceinline__ float at(int) const { return d; }
 };
 
 template <>
@@ -67,6 +68,7 @@ struct FVec<2> {
         d.x += x.d.x;
         d.y += x.d.y;
     }
+    __device__ __forceinline__ float at(int i) const { return d[i]; }
 };
 
 template <>
@@ -95,6 +97,7 @@ struct FVec<4> {
         d.z += x.d.z;
         d.w += x.d.w;
     }
+    __device__ __forceinline__ float at(int i) const { return d[i]; }
 };
 
 // Lane-to-lane hand-over of a 32-bit word inside a group of LPR lanes.  For LPR == 64
@@ -667,27 +670,42 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
 
 
 // ---------------------------------------------------------------------------------------
-// Very long rows.  One 256-thread block per (row, feature tile of 16 .. 256 floats).  The
-// row's chain must stay sequential (bit-identical results), so what is parallelised is the
-// FETCH: all four waves gather a chunk of dense rows at once (up to 8 vector loads per thread
-// and chunk), while the threads that own a feature each run the FMA chain over an earlier
-// chunk out of LDS, in CSR order.  A row advances by one chunk per memory round trip, so the
-// chunk is made as long as a 32 KB tile buffer allows -- 32 rows of 256 floats, 512 rows of
-// 16 -- and with few such rows the host cuts them into narrow feature tiles (every feature's
-// chain is its own), which also spreads one row's fetch over several compute units.
-// kLongDepth chunks are in flight in registers; the (col, val) pairs come in super-chunks of
-// kLongDepth chunks, two super-chunks ahead.
+// Very long rows.  One block per (row, feature tile of 16 .. 256 floats): four FETCH waves and,
+// behind them, one CHAIN wave per 64 features of the tile.  The row's chain must stay
+// sequential (bit-identical results), so what is parallelised is the fetch: the fetch waves
+// gather a chunk of dense rows at once (up to 8 vector loads per thread and chunk) and land it
+// in LDS, while in the chain waves the lane that owns a feature runs the FMA chain over the
+// chunk landed before, in CSR order, and does nothing else.  A chunk lies TRANSPOSED in LDS --
+// tile[feature][element of the chunk] -- so that the owner of a feature reads four consecutive
+// elements with one 16-byte LDS read, and the four matrix values that go with them with
+// another (the same address in every lane): 1.5 instructions per stored element, of which only
+// the FMA is on the chain.  Measured in one wave on this part: 1.9 ns per element for the bare
+// chain, 3.7 ns with these reads (sixteen and sixteen requested ahead of their 64 FMAs), 3.9 ns
+// with the matrix value handed round by v_readlane instead, 5.8 ns with a 4-byte LDS read per
+// element on top of that.  A row advances by one chunk per memory round trip, so the chunk is
+// made as long as a tile buffer allows -- 32 rows of 256 floats, 512 rows of 16 -- and with few
+// such rows the host cuts them into narrow feature tiles (every feature's chain is its own),
+// which also spreads one row's fetch over several compute units.  kLongDepth chunks are in
+// flight in registers; the (col, val) pairs come in super-chunks of kLongDepth chunks, two
+// super-chunks ahead.
 // ---------------------------------------------------------------------------------------
-constexpr int kLongTileFloats = 8192;  // floats per LDS tile buffer (32 KB), two buffers
+constexpr int kLongTileFloats = 8192;  // most floats of one chunk (tile width x rows of the chunk)
 constexpr int kLongMaxChunk = 512;     // most dense rows gathered per chunk
+constexpr int kLongRowPad = 4;         // floats between the feature rows of a tile buffer: lanes f, f + 1, ... read
+                                       // 16 bytes each at a stride of chunk + 4 floats, 16 lanes covering all banks
+constexpr int kLongFeatTile = 256;     // most features per block
+constexpr int kLongFetchThreads = 256; // the fetch waves of a block; behind them one chain wave per 64 features
+// floats of one tile buffer: width x (chunk + pad) <= kLongTileFloats + kLongFeatTile * kLongRowPad, and four
+// floats behind them where the fetch slots past a chunk's rows land
+constexpr int kLongDump = kLongTileFloats + kLongFeatTile * kLongRowPad;
+constexpr int kLongBufFloats = kLongDump + 4;
 constexpr int kLongLoads = 8;          // most vector loads per thread and chunk
 constexpr int kLongDepth = 2;          // chunks in flight
-constexpr int kLongFeatTile = 256;     // most features per block
 constexpr int kLongMinFeatTile = 16;   // fewest: one 64-byte piece of every gathered row
 constexpr int kLongPairs = kLongDepth * kLongMaxChunk / 256;  // (col, val) pairs per thread and super-chunk
 // dynamic LDS: two tile buffers, then three (col, val) super-chunk buffers
 constexpr size_t kLongSmemBytes =
-    2 * kLongTileFloats * sizeof(float) + 3 * kLongDepth * kLongMaxChunk * (sizeof(int) + sizeof(float));
+    2 * kLongBufFloats * sizeof(float) + 3 * kLongDepth * kLongMaxChunk * (sizeof(int) + sizeof(float));
 
 struct LongArgs {
     const RowTask *task;  // rows handled: task[0 .. gridDim.x)
@@ -698,39 +716,59 @@ struct LongArgs {
     int feat;        // F
     int ldx, ldd;    // row strides of x and dst in floats; 0 stands for F
     int tile;        // features per block (a multiple of VEC, <= kLongFeatTile)
-    int chunk;       // dense rows per chunk: chunk * min(F, 256) <= kLongTileFloats, chunk * (tile / VEC) <= 2048
+    int chunk;       // dense rows per chunk, a multiple of 4: chunk * tile <= kLongTileFloats, chunk * (tile / VEC) <= 2048
     int accumulate;
 };
 
-// The chain over one whole chunk of CC stored elements for the feature a thread owns: the CC values of
-// its column are requested from LDS back to back (independent reads, fully pipelined) and the CC matrix
-// values come in with ONE read per lane and are handed to the whole wave lane by lane (v_readlane, so the
-// multiplier of every FMA is a scalar); what remains sequential is the FMA chain itself.
-// FW: the tile's width when the host knows it (the LDS offsets are then immediates), 0: take `fw`.
-template <int CC, int FW>
-__device__ __forceinline__ float chain_whole_chunk(const float *tb, const float *vb, int fw, float acc) {
-    static_assert(CC <= 64, "one matrix value per lane");
-    float xs[CC];
+// The chain over `cnt` stored elements for the feature a thread owns: tb = the feature's row of the tile buffer
+// (element j of the chunk at tb[j]), vb = the matrix values of the chunk; both 16-byte aligned.  Sixteen 16-byte
+// reads of each are requested back to back ahead of their 64 FMAs.
+__device__ __forceinline__ float chain_over_chunk(const float *tb, const float *vb, int cnt, float acc) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    // the matrix values sit at the same address for every lane; kept in a vector register all the same, so that
+    // the sixteen reads of a round are one base and sixteen immediates instead of sixteen scalar adds and moves
+    int same = 0;
+    asm volatile("" : "+v"(same));
+    vb += same;
+    int j = 0;
+    for (; j + 64 <= cnt; j += 64) {
+        f4 xs[16], vs[16];
 #pragma unroll
-    for (int j = 0; j < CC; ++j) xs[j] = tb[j * (FW ? FW : fw)];
-    const int lane = (int)__lane_id();
-    const int vl = __float_as_int(vb[lane < CC ? lane : 0]);
+        for (int q = 0; q < 16; ++q) {
+            xs[q] = *reinterpret_cast<const f4 *>(tb + j + 4 * q);
+            vs[q] = *reinterpret_cast<const f4 *>(vb + j + 4 * q);
+        }
 #pragma unroll
-    for (int j = 0; j < CC; ++j) acc = __builtin_fmaf(__int_as_float(__builtin_amdgcn_readlane(vl, j)), xs[j], acc);
+        for (int q = 0; q < 16; ++q) {
+            acc = __builtin_fmaf(vs[q].x, xs[q].x, acc);
+            acc = __builtin_fmaf(vs[q].y, xs[q].y, acc);
+            acc = __builtin_fmaf(vs[q].z, xs[q].z, acc);
+            acc = __builtin_fmaf(vs[q].w, xs[q].w, acc);
+        }
+    }
+    for (; j + 4 <= cnt; j += 4) {
+        const f4 x = *reinterpret_cast<const f4 *>(tb + j);
+        const f4 v = *reinterpret_cast<const f4 *>(vb + j);
+        acc = __builtin_fmaf(v.x, x.x, acc);
+        acc = __builtin_fmaf(v.y, x.y, acc);
+        acc = __builtin_fmaf(v.z, x.z, acc);
+        acc = __builtin_fmaf(v.w, x.w, acc);
+    }
+    for (; j < cnt; ++j) acc = __builtin_fmaf(vb[j], tb[j], acc);
     return acc;
 }
 
 // NL: vector loads per thread and chunk, the smallest of 1, 2, 4, 8 with NL * 256 >= chunk * (tile / VEC).
 // FW: the width of EVERY tile of the launch when that is one of 16 .. 256 and divides F, else 0.
 template <int VEC, int NL, int FW = 0>
-__global__ __launch_bounds__(256) void spmm_long_rows_kernel(const LongArgs a) {
+__global__ __launch_bounds__(kLongFetchThreads + kLongFeatTile) void spmm_long_rows_kernel(const LongArgs a) {
     typedef FVec<VEC> V;
     constexpr int D = kLongDepth;
     constexpr int kSuper = D * kLongMaxChunk;  // index pairs per super-chunk buffer
     extern __shared__ __attribute__((aligned(16))) unsigned char long_smem[];
-    float(*tile)[kLongTileFloats] = reinterpret_cast<float(*)[kLongTileFloats]>(long_smem);
-    int(*s_col)[kSuper] = reinterpret_cast<int(*)[kSuper]>(long_smem + 2 * kLongTileFloats * sizeof(float));
-    float(*s_val)[kSuper] = reinterpret_cast<float(*)[kSuper]>(long_smem + 2 * kLongTileFloats * sizeof(float) +
+    float(*tile)[kLongBufFloats] = reinterpret_cast<float(*)[kLongBufFloats]>(long_smem);
+    int(*s_col)[kSuper] = reinterpret_cast<int(*)[kSuper]>(long_smem + 2 * kLongBufFloats * sizeof(float));
+    float(*s_val)[kSuper] = reinterpret_cast<float(*)[kSuper]>(long_smem + 2 * kLongBufFloats * sizeof(float) +
                                                                3 * kSuper * sizeof(int));
 
     const int t = (int)threadIdx.x;
@@ -747,14 +785,20 @@ __global__ __launch_bounds__(256) void spmm_long_rows_kernel(const LongArgs a) {
     const int32_t *__restrict__ col = a.col + d.start;
     const float *__restrict__ val = a.val + d.start;
 
-    // fixed (dense row in chunk, vector in row) slots of this thread; slot e lands at float e * VEC of a
-    // tile buffer (= row e / vpr, vector e % vpr), always inside the buffer
+    // fixed (dense row in chunk, vector in row) slots of this thread: slot e is row e / vpr, vector e % vpr; its
+    // VEC floats land in the feature rows sv .. sv + VEC - 1 of a tile buffer at element sj
+    const int stride = C + kLongRowPad;  // floats between the feature rows of a tile buffer (C is a multiple of 4)
     int sj[NL], sv[NL];
+    int land_at[NL], land_step[NL];  // where the slot's first float lands, and how far apart its floats do
 #pragma unroll
     for (int s = 0; s < NL; ++s) {
         const int e = t + s * 256;
         sj[s] = e / vpr;
         sv[s] = (e - sj[s] * vpr) * VEC;
+        // a slot past the chunk's rows fetches a repeat of the last row: it lands behind the tile, where nobody
+        // reads (no branch around the stores: with one, the compiler waits for every load in flight instead)
+        land_at[s] = sj[s] < C ? sv[s] * stride + sj[s] : kLongDump;
+        land_step[s] = sj[s] < C ? stride : 0;
     }
 
     auto chunk_len = [&](int k) { const int left = d.len - k * C; return left < C ? left : C; };
@@ -771,9 +815,37 @@ __global__ __launch_bounds__(256) void spmm_long_rows_kernel(const LongArgs a) {
         }
     };
     auto land = [&](int k, const V(&g)[NL]) {
+        float *tb = tile[k & 1];
 #pragma unroll
-        for (int s = 0; s < NL; ++s) g[s].store(&tile[k & 1][(t + s * 256) * VEC]);
+        for (int s = 0; s < NL; ++s) {
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) tb[land_at[s] + i * land_step[s]] = g[s].at(i);
+        }
     };
+
+    float *dst = a.dst + (size_t)d.row * (size_t)(a.ldd ? a.ldd : F) + f0;
+
+    // Threads 256 and up are the chain waves, one lane per feature of the tile; they fetch nothing.  Both kinds of
+    // wave pass the same barriers: two in the prologue, one per chunk.
+    if (t >= 256) {
+        const int f = t - 256;
+        const bool own = f < fw;
+        __syncthreads();
+        __syncthreads();
+        float acc = 0.0f;
+        if (own && a.accumulate) acc = __builtin_nontemporal_load(dst + f);
+        const float *mine = &tile[0][(own ? f : 0) * stride];
+        for (int k = 0; k < nchunks; ++k) {
+            // the chain over chunk k, in CSR order, out of LDS, while the fetch waves land chunk k + 1; lanes past
+            // the tile's width sit it out (an LDS read costs by the lanes that take part)
+            if (own)
+                acc = chain_over_chunk(mine + (k & 1) * kLongBufFloats, &s_val[(k / D) % 3][(k % D) * C], chunk_len(k),
+                                       acc);
+            __syncthreads();
+        }
+        if (own) __builtin_nontemporal_store(acc, dst + f);
+        return;
+    }
 
     // prologue: index pairs of super-chunks 0 and 1, dense rows of chunks 0 .. D-1, chunk 0 landed
 #pragma unroll
@@ -794,12 +866,6 @@ __global__ __launch_bounds__(256) void spmm_long_rows_kernel(const LongArgs a) {
     for (int u = 0; u < D; ++u) request(u < nchunks ? u : nchunks - 1, g[u]);
     land(0, g[0]);
     __syncthreads();
-
-    float *dst = a.dst + (size_t)d.row * (size_t)(a.ldd ? a.ldd : F) + f0;
-    float acc = 0.0f;
-    const bool own = t < fw;
-    const bool wave_owns = (t & ~63) < fw;  // the same for the 64 lanes of a wave
-    if (own && a.accumulate) acc = __builtin_nontemporal_load(dst + t);
 
     for (int kb = 0; kb < nchunks; kb += D) {
         // index pairs of the super-chunk after the next one: requested now, stored at the end
@@ -822,22 +888,7 @@ __global__ __launch_bounds__(256) void spmm_long_rows_kernel(const LongArgs a) {
             // (1) chunk k left its registers for LDS in the step before: request chunk k + D into them
             //     (past the row's end: the last chunk once more, never landed where it is read)
             request(k + D < nchunks ? k + D : nchunks - 1, g[u]);
-            // (2) the chain over chunk k, in CSR order, out of LDS (whole waves take part: a lane past the
-            //     tile's width computes a value nobody stores)
-            if (wave_owns) {
-                const int cnt = chunk_len(k);
-                const float *tb = &tile[k & 1][t];
-                const float *vb = &s_val[super % 3][u * C];
-                int j = 0;
-                for (; j + 64 <= cnt; j += 64) acc = chain_whole_chunk<64, FW>(tb + j * fw, vb + j, fw, acc);
-                if (j + 32 <= cnt) {
-                    acc = chain_whole_chunk<32, FW>(tb + j * fw, vb + j, fw, acc);
-                    j += 32;
-                }
-#pragma unroll 8
-                for (; j < cnt; ++j) acc = __builtin_fmaf(vb[j], tb[j * fw], acc);
-            }
-            // (3) land chunk k + 1 (requested D - 1 steps ago) in the other tile buffer
+            // (2) land chunk k + 1 (requested D - 1 steps ago) in the tile buffer the chain waves are not reading
             land(k + 1, g[(u + 1) % D]);
             if (u == D - 1) {
 #pragma unroll
@@ -849,7 +900,6 @@ __global__ __launch_bounds__(256) void spmm_long_rows_kernel(const LongArgs a) {
             __syncthreads();
         }
     }
-    if (own) __builtin_nontemporal_store(acc, dst + t);
 }
 
 }  // namespace gnnagg
