@@ -66,6 +66,16 @@ struct DevBuf {
     }
 };
 
+// the largest of the 64 lanes' values, in every lane (all lanes of the wave must call it)
+__device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const unsigned long long o = __shfl_xor(v, off, 64);
+        v = o > v ? o : v;
+    }
+    return v;
+}
+
 inline int ceil_log2_u64(uint64_t x) {  // smallest b with 2^b >= x (x >= 1)
     int b = 0;
     while ((uint64_t(1) << b) < x) ++b;

@@ -325,8 +325,13 @@ __global__ __launch_bounds__(256) void argsort_prepare_kernel(const int64_t *__r
         idx[i] = (uint32_t)i;
         if (v > 0 && (unsigned long long)v > m) m = (unsigned long long)v;
     }
-    if (m) atomicMax(max_key, m);
-    if (neg) atomicOr(negative, 1u);
+    // one atomic per wave, not per thread: all of them land on one address
+    m = wave_max_u64(m);
+    const bool any_neg = __builtin_amdgcn_ballot_w64(neg) != 0;
+    if ((threadIdx.x & 63) == 0) {
+        if (m) atomicMax(max_key, m);
+        if (any_neg) atomicOr(negative, 1u);
+    }
 }
 
 __global__ __launch_bounds__(256) void argsort_finish_kernel(const uint64_t *__restrict__ key,

@@ -249,19 +249,32 @@ __global__ __launch_bounds__(256) void classify_rows_kernel(const int64_t *__res
     if (threadIdx.x == 0) smax = 0;
     __syncthreads();
     const int r = (int)blockIdx.x * 256 + (int)threadIdx.x;
+    int c = -1;  // the row's class; -1: no row, or a row whose rowptr runs backwards
+    unsigned long long longest = 0;
     if (r < rows) {
         const int64_t d = rowptr[r + 1] - rowptr[r];
         if (d < 0) {
             atomicOr(&out->bad_rowptr, 1u);
             key[r] = (uint32_t)kEmptyClass;
         } else {
-            const int c = degree_class(d);
+            c = degree_class(d);
             key[r] = (uint32_t)c;
-            atomicAdd(&hist[c], 1u);
-            atomicMax(&smax, (unsigned long long)d);
+            longest = (unsigned long long)d;
         }
         rowid[r] = r;
     }
+    // per wave one LDS atomic per class that occurs in it (its lanes found by ballots over the class's bits) and one
+    // for the longest row, instead of one of each per row onto a handful of addresses
+    uint64_t same = __builtin_amdgcn_ballot_w64(c >= 0);
+#pragma unroll
+    for (int b = 0; b < kClassBits; ++b) {
+        const uint64_t has = __builtin_amdgcn_ballot_w64(((c >> b) & 1) != 0);
+        same &= ((c >> b) & 1) ? has : ~has;
+    }
+    const int lane = (int)threadIdx.x & 63;
+    if (c >= 0 && (same & ((uint64_t(1) << lane) - 1)) == 0) atomicAdd(&hist[c], (unsigned int)__popcll(same));
+    longest = wave_max_u64(longest);
+    if (lane == 0 && longest) atomicMax(&smax, longest);
     __syncthreads();
     if (threadIdx.x < kNumClasses && hist[threadIdx.x])
         atomicAdd(&out->class_count[threadIdx.x], (unsigned long long)hist[threadIdx.x]);
