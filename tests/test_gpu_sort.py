@@ -95,3 +95,20 @@ def test_calls_without_a_workspace_allocate_their_own_and_a_short_workspace_is_r
     with pytest.raises(_lib.GnnAggError, match="workspace"):
         _lib.check(L.gnnagg_runs_i64(_lib.ptr(ordered), n, None, 0, _lib.ptr(values), None, None, ctypes.byref(found),
                                      _lib.ptr(short), 64, stream))
+
+
+@pytest.mark.parametrize("n,distinct", [(50_000_000, 1_000_003), (120_000_000, 1 << 46)])
+def test_argsort_at_the_size_of_a_partitions_edge_list_is_sorted_stable_and_a_permutation(n, distinct):
+    """Size-independent properties at the scale of config 4's edge lists (10^8 keys): the keys come out in
+    non-decreasing order, equal keys in their input order, and every position occurs exactly once."""
+    gen = torch.Generator(device="cuda").manual_seed(n % 1000)
+    x = torch.randint(0, distinct, (n,), device="cuda", generator=gen, dtype=torch.int64)
+    perm = device_ops.stable_argsort(x)
+    ordered = x[perm]
+    step = ordered[1:] - ordered[:-1]
+    assert bool((step >= 0).all())
+    assert bool((perm[1:][step == 0] > perm[:-1][step == 0]).all())          # stable
+    del step, ordered
+    seen = torch.zeros(n, dtype=torch.int8, device="cuda")
+    seen[perm] = 1
+    assert int(seen.sum(dtype=torch.int64)) == n and int(perm.min()) == 0 and int(perm.max()) == n - 1
