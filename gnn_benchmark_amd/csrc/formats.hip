@@ -51,27 +51,56 @@ __global__ __launch_bounds__(256) void major_ptr_kernel(const uint64_t *__restri
     ptr[r] = lo;
 }
 
-// key = col << row_bits | row for every stored element of a CSR matrix (row found by
-// binary search in rowptr); idx = position.
+// key = col << row_bits | row for every stored element of a CSR matrix; idx = position.  The row of element e is the
+// last row r with rowptr[r] <= e.  A block owns 256 consecutive elements: two threads find the rows of its first and
+// last element by binary search in rowptr, the block copies that stretch of rowptr to LDS (when it is at most kSpan
+// rows: rows without elements can make it long) and every thread searches there instead of in memory.
+constexpr int kSpan = 1024;
+
+__device__ __forceinline__ int64_t last_row_at_or_before(const int64_t *__restrict__ rowptr, int64_t lo, int64_t hi,
+                                                         int64_t e) {
+    while (hi - lo > 1) {  // invariant: rowptr[lo] <= e, and hi is past the answer
+        const int64_t mid = (lo + hi) >> 1;
+        if (rowptr[mid] <= e) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
 __global__ __launch_bounds__(256) void pack_transposed_keys_kernel(const int64_t *__restrict__ rowptr,
                                                                    const int64_t *__restrict__ col, int64_t rows,
                                                                    int64_t cols, int64_t nnz, int row_bits,
                                                                    uint64_t *__restrict__ key,
                                                                    uint32_t *__restrict__ idx,
                                                                    unsigned int *__restrict__ bad) {
-    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    __shared__ int64_t s_ptr[kSpan];
+    __shared__ int64_t s_first, s_last;
+    const int64_t e0 = (int64_t)blockIdx.x * 256;
+    const int64_t e = e0 + threadIdx.x;
+    if (threadIdx.x == 0) s_first = last_row_at_or_before(rowptr, 0, rows, e0);
+    if (threadIdx.x == 64) s_last = last_row_at_or_before(rowptr, 0, rows, e0 + 255 < nnz ? e0 + 255 : nnz - 1);
+    __syncthreads();
+    const int64_t first = s_first, last = s_last;
+    const int span = last - first + 1 <= kSpan ? (int)(last - first + 1) : 0;  // 0: too long for LDS
+    for (int i = (int)threadIdx.x; i < span; i += 256) s_ptr[i] = rowptr[first + i];
+    __syncthreads();
     if (e >= nnz) return;
-    int64_t lo = 0, hi = rows;  // last row with rowptr[row] <= e
-    while (hi - lo > 1) {
-        const int64_t mid = (lo + hi) >> 1;
-        if (rowptr[mid] <= e) lo = mid; else hi = mid;
+    int64_t row;
+    if (span) {
+        int lo = 0, hi = span;
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (s_ptr[mid] <= e) lo = mid; else hi = mid;
+        }
+        row = first + lo;
+    } else {
+        row = last_row_at_or_before(rowptr, first, last + 1, e);
     }
     const int64_t c = col[e];
     if (c < 0 || c >= cols) {
         atomicOr(bad, 1u);
         key[e] = 0;
     } else {
-        key[e] = ((uint64_t)c << row_bits) | (uint64_t)lo;
+        key[e] = ((uint64_t)c << row_bits) | (uint64_t)row;
     }
     idx[e] = (uint32_t)e;
 }
