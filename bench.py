@@ -25,7 +25,7 @@ mean aggregation, F=602/256), c4 (one partition of a 16-way split: pre-aggregati
 post-aggregation, F=128) and c5 (3-layer GCN train step and the reference's 3-layer SAGE model
 on the c4 partition).  Their full reports do not go into the stdout line: each is written, as
 soon as its workload has finished, as one JSON line to stderr and into the side file
-``--extra-out`` (default gpurun_out/bench_extra.json), so a late failure loses nothing.
+``--extra-out`` (default bench_out/bench_extra.json), so a late failure loses nothing.
 ``--only headline`` skips them.
 """
 import argparse
@@ -1592,7 +1592,7 @@ def main():
     ap.add_argument("--no-parity-gate", action="store_true",
                     help="skip the comparison of the GPU results with the CPU operator in front of the number "
                          "(the line then says parity.checked = false)")
-    ap.add_argument("--extra-out", default=os.path.join(ROOT, "gpurun_out", "bench_extra.json"),
+    ap.add_argument("--extra-out", default=os.path.join(ROOT, "bench_out", "bench_extra.json"),
                     help="side file for the full reports of the workloads besides the headline (also written to "
                          "stderr, one JSON line per workload as it finishes)")
     ap.add_argument("--copy-calibration", action="store_true",
