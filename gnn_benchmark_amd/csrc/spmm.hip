@@ -170,15 +170,31 @@ hipError_t enable_long_rows_lds() {
     return e;
 }
 
+// What a stored element costs a row of the block-per-row kernel, by tile width (ns, measured on a 200 000-element
+// row): the chain itself does not depend on the width, but a wider tile means a shorter chunk (a tile buffer holds
+// 8192 floats), and with two chunks in flight a short chunk no longer covers the memory round trip.
+struct LongTileCost { int tile; double ns_per_element; };
+constexpr LongTileCost kLongTileCosts[] = {{16, 6.0}, {32, 7.5}, {64, 12.5}, {128, 34.0}, {256, 70.0}};
+constexpr double kComputeUnits = 256.0;
+
 template <int VEC>
-hipError_t launch_long_rows(const LongArgs &a, int64_t nrows, hipStream_t st) {
+hipError_t launch_long_rows(const LongArgs &a, int64_t nrows, int64_t longest, int64_t elems, hipStream_t st) {
     LongArgs args = a;
-    // What bounds a row is the rate at which ONE compute unit can fetch its dense rows, so with few
-    // such rows each is cut along the features into more blocks (each feature's chain is its own),
-    // down to 16 features = one 64-byte piece per stored element; a narrower tile also means a longer
-    // chunk (more stored elements per memory round trip).
+    // Every feature's chain is its own, so a row can be cut along the features into tiles of 16 .. 256 floats, one
+    // block each.  The launch lasts as long as the longest row's block, or as long as all blocks take on all compute
+    // units (rows are handed out longest first): the tile width is the one for which the larger of the two is smallest.
     int tile = kLongFeatTile;
-    while (tile > kLongMinFeatTile && nrows * ((a.feat + tile / 2 - 1) / (tile / 2)) <= 512) tile /= 2;
+    double best = 0.0;
+    for (const LongTileCost &c : kLongTileCosts) {
+        const double tiles = (double)((a.feat + c.tile - 1) / c.tile);
+        const double longest_row = (double)longest * c.ns_per_element;
+        const double all_rows = (double)elems * tiles * c.ns_per_element / kComputeUnits;
+        const double lasts = std::max(longest_row, all_rows);
+        if (best == 0.0 || lasts < best) {
+            best = lasts;
+            tile = c.tile;
+        }
+    }
     if (tile > a.feat) tile = a.feat;
     args.tile = tile;
     const int vpr = tile / VEC;
@@ -189,7 +205,9 @@ hipError_t launch_long_rows(const LongArgs &a, int64_t nrows, hipStream_t st) {
     args.chunk = chunk;
     const unsigned tiles = (unsigned)((a.feat + tile - 1) / tile);
     const int slots = chunk * vpr;  // vectors of a whole chunk; 256 threads fetch them in NL rounds
-    const dim3 grid((unsigned)nrows, tiles);
+    args.tiles = (int)tiles;
+    if (nrows * (int64_t)tiles >= (int64_t(1) << 31)) return hipErrorInvalidValue;
+    const dim3 grid((unsigned)(nrows * (int64_t)tiles));
     const dim3 block((unsigned)(kLongFetchThreads + 64 * ((tile + 63) / 64)));  // fetch waves + one chain wave per 64 features
     if (VEC == 4 && slots > 1024 && a.feat % tile == 0 && tile >= 16 && (tile & (tile - 1)) == 0) {
         // every tile has the same power-of-two width: the instance that knows it at compile time
@@ -317,6 +335,7 @@ struct gnnagg_plan {
     int64_t rows = 0, cols = 0, nnz = 0;
     int huge_thresh = 0;      // rows longer than this run in the block-per-row kernel
     int64_t nhuge = 0;        // such rows (the first nhuge tasks)
+    int64_t huge_elems = 0;   // upper bound of the stored elements in them (class counts x the classes' upper ends)
     int long_thresh = 0;      // rows longer than this get a lane group of their own (head region)
     int64_t nlong = 0;        // such rows, the huge ones included (the first nlong tasks)
     int64_t nempty = 0;       // rows with no stored element (the last nempty entries of perm)
@@ -543,7 +562,12 @@ extern "C" int gnnagg_plan_create_ex(const int64_t *rowptr, const int64_t *col, 
     const int thresh_class = degree_class(p->long_thresh);
     for (int c = 0; c < thresh_class; ++c) p->nlong += (int64_t)h_out.class_count[c];
     const int huge_class = degree_class(p->huge_thresh);
-    for (int c = 0; c < huge_class; ++c) p->nhuge += (int64_t)h_out.class_count[c];
+    for (int c = 0; c < huge_class; ++c) {
+        p->nhuge += (int64_t)h_out.class_count[c];
+        // class c holds the rows of ceil(log2(length)) == kEmptyClass - 1 - c
+        const int64_t upper = std::min<int64_t>(int64_t(1) << (kEmptyClass - 1 - c), p->max_deg);
+        p->huge_elems += (int64_t)h_out.class_count[c] * upper;
+    }
     for (int c = degree_class(kShortRowLen); c < kEmptyClass; ++c) p->nshort += (int64_t)h_out.class_count[c];
     if (p->long_thresh < kShortRowLen) p->nshort = 0;  // (such rows sit in the head region then)
     if (p->nhuge > 0) {
@@ -651,9 +675,9 @@ int plan_spmm(gnnagg_plan *plan, const float *value, const float *mat, int64_t l
         la.ldx = (int)ldx;
         la.ldd = (int)ldd;
         la.accumulate = accumulate;
-        if (vec == 4) GNNAGG_HIP(launch_long_rows<4>(la, plan->nhuge, plan->side));
-        else if (vec == 2) GNNAGG_HIP(launch_long_rows<2>(la, plan->nhuge, plan->side));
-        else GNNAGG_HIP(launch_long_rows<1>(la, plan->nhuge, plan->side));
+        if (vec == 4) GNNAGG_HIP(launch_long_rows<4>(la, plan->nhuge, plan->max_deg, plan->huge_elems, plan->side));
+        else if (vec == 2) GNNAGG_HIP(launch_long_rows<2>(la, plan->nhuge, plan->max_deg, plan->huge_elems, plan->side));
+        else GNNAGG_HIP(launch_long_rows<1>(la, plan->nhuge, plan->max_deg, plan->huge_elems, plan->side));
         GNNAGG_HIP(hipEventRecord(plan->join, plan->side));
     }
     for (int64_t f_base = 0; f_base < feat;) {

@@ -708,7 +708,7 @@ constexpr size_t kLongSmemBytes =
     2 * kLongBufFloats * sizeof(float) + 3 * kLongDepth * kLongMaxChunk * (sizeof(int) + sizeof(float));
 
 struct LongArgs {
-    const RowTask *task;  // rows handled: task[0 .. gridDim.x)
+    const RowTask *task;  // rows handled: task[0 .. gridDim.x / tiles)
     const int32_t *col;
     const float *val;
     const float *x;
@@ -716,6 +716,7 @@ struct LongArgs {
     int feat;        // F
     int ldx, ldd;    // row strides of x and dst in floats; 0 stands for F
     int tile;        // features per block (a multiple of VEC, <= kLongFeatTile)
+    int tiles;       // tiles per row: the grid is rows x tiles blocks, block b = row b / tiles, tile b % tiles
     int chunk;       // dense rows per chunk, a multiple of 4: chunk * tile <= kLongTileFloats, chunk * (tile / VEC) <= 2048
     int accumulate;
 };
@@ -772,10 +773,14 @@ __global__ __launch_bounds__(kLongFetchThreads + kLongFeatTile) void spmm_long_r
                                                                3 * kSuper * sizeof(int));
 
     const int t = (int)threadIdx.x;
-    const RowTask d = a.task[blockIdx.x];
+    // blocks are handed out in the order of their index: the tiles of one row next to each other, rows in the order
+    // of the schedule (longest first), so that the longest row's blocks all start at once
+    const int row_of_block = (int)(blockIdx.x / (unsigned)a.tiles);
+    const int tile_of_block = (int)(blockIdx.x % (unsigned)a.tiles);
+    const RowTask d = a.task[row_of_block];
     const int F = a.feat;
     const int ldx = a.ldx ? a.ldx : F;
-    const int f0 = (int)blockIdx.y * a.tile;
+    const int f0 = tile_of_block * a.tile;
     const int fw = FW ? FW : (F - f0 < a.tile ? F - f0 : a.tile);    // width of this tile (multiple of VEC)
     const int vpr = fw / VEC;                                        // vectors per gathered row
     const int C = a.chunk;
