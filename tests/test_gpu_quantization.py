@@ -493,3 +493,73 @@ def test_one_launch_over_dense_rows_and_rows_in_their_exchange_format(kind, feat
     assert torch.equal(wide_out[:, feat:], want) and not wide_out[:, :feat].any()
     with pytest.raises(RuntimeError, match="Input mismatch"):
         both.get_plan().spmm_dense_then(both.csr()[2], both.first_counts[:-1], x, second, got, False)
+
+
+@pytest.mark.parametrize("bits", [2, 4, 8])
+def test_compiled_module_codec_functions_match_oracle_and_golden_bytes(bits):
+    """The codec functions of the compiled pybind11 module ``computation_ops`` (gnn_benchmark_amd/ext), called with the
+    reference's positional arguments (self_benchmark/a64fx/model/ops/src/quantization_arm.h; quantizer.py:18-90):
+    the oracle's bytes and parameters for ragged segments, the whole-buffer form, and the mixed-width golden bytes of
+    self_benchmark/a64fx/tests/test_quantizer.py:81."""
+    from gnn_benchmark_amd import ext
+
+    mod = ext.load()
+    rng = np.random.default_rng(77 + bits)
+    feat = 130
+    splits = [5, 0, 13, 1, 8, 0, 4, 7]
+    rows = sum(splits)
+    x = _rows(rng, rows, feat)
+    want_packed, want_params = oq.quantize_segments(x, splits, bits)
+    work_range = torch.tensor(np.concatenate(([0], np.cumsum(splits))), dtype=torch.int32)
+    packed = torch.full(want_packed.shape, 0xAB, dtype=torch.uint8, device="cuda")
+    params = torch.full((rows, 2), -7.0, device="cuda")
+    for _ in range(2):  # the second call finds the range's device copies again
+        assert mod.quantize_tensor_for_all_procs(dev(x), packed, params, work_range, len(splits), bits) is None
+    assert np.array_equal(params.cpu().numpy(), want_params) and np.array_equal(packed.cpu().numpy(), want_packed)
+    back = torch.full((rows, feat), 9.0, device="cuda")
+    mod.dequantize_tensor_for_all_procs(packed, back, params, work_range, len(splits), bits)
+    want_back = oq.dequantize_segments(want_packed, want_params, splits, bits)
+    assert np.array_equal(back.cpu().numpy().view(np.uint32), want_back.view(np.uint32))
+    work_range[2] += 1  # changed in place: a new prefix, no stale copy
+    work_range[2] -= 1
+    mod.dequantize_tensor_for_all_procs(packed, back, params, work_range, len(splits), bits)
+    assert np.array_equal(back.cpu().numpy().view(np.uint32), want_back.view(np.uint32))
+
+    one_packed, one_params = oq.quantize_segments(x, [rows], bits)
+    packed1 = torch.zeros(one_packed.shape, dtype=torch.uint8, device="cuda")
+    params1 = torch.zeros((rows, 2), device="cuda")
+    mod.quantize_tensor(dev(x), packed1, params1, bits)
+    assert np.array_equal(packed1.cpu().numpy(), one_packed) and np.array_equal(params1.cpu().numpy(), one_params)
+    back1 = torch.zeros((rows, feat), device="cuda")
+    mod.dequantize_tensor(packed1, back1, params1, bits)
+    assert np.array_equal(back1.cpu().numpy().view(np.uint32),
+                          oq.dequantize_segments(one_packed, one_params, [rows], bits).view(np.uint32))
+
+    with pytest.raises(RuntimeError, match="GPU"):
+        mod.quantize_tensor(torch.zeros(4, 8), packed1, params1, bits)
+    with pytest.raises(RuntimeError, match="bits"):
+        mod.quantize_tensor(dev(x), packed1, params1, 3)
+    with pytest.raises(RuntimeError, match="work range"):
+        mod.quantize_tensor_for_all_procs(dev(x), packed, params, work_range[:-1], len(splits), bits)
+
+
+def test_compiled_module_mixed_width_functions_on_the_reference_golden_bytes():
+    from gnn_benchmark_amd import ext
+    from gnn_benchmark_amd.quantizer import QuantizerForMixedBits
+
+    mod = ext.load()
+    x = torch.tensor([[0.2, 0.1, 0.3], [0.4, 0.5, 0.6], [0.7, 0.8, 0.9], [1.0, 1.1, 1.2], [0.3, 0.1, 0.7]],
+                     device="cuda")
+    bits = torch.tensor([8, 4, 2, 4, 4], device="cuda")
+    params = torch.empty((5, 3), device="cuda")
+    params[:, 0] = bits
+    feat_range = QuantizerForMixedBits.get_quantized_nodes_feat_range(5, 3, bits)
+    data = torch.empty(int(feat_range[-1]), dtype=torch.uint8, device="cuda")
+    mod.quantize_tensor_v1(x, data, feat_range, params)
+    assert data.tolist() == [127, 0, 255, 7, 240, 44, 8, 240, 80, 240]   # tests/test_quantizer.py:81
+    back = torch.empty_like(x)
+    mod.dequantize_tensor_v1(data, back, feat_range, params)
+    assert bool(((back - x).abs() <= params[:, 2:3] * 0.5 + 1e-6).all())
+    params[2, 0] = 3.0
+    with pytest.raises(RuntimeError, match="bit width"):
+        mod.quantize_tensor_v1(x, data, feat_range, params)

@@ -153,13 +153,23 @@ def test_compiled_extension_module_keeps_the_reference_signature():
         mod.spmm(*args)
     with pytest.raises(TypeError):
         mod.spmm(*args[:7])
+    # the codec functions the trainer's quantizer calls, with the positional arguments of
+    # self_benchmark/a64fx/model/ops/src/quantization_arm.h (bound at model/ops/src/ops.cpp:12-18)
+    for name, tensors in (("quantize_tensor", 3), ("dequantize_tensor", 3), ("quantize_tensor_v1", 4),
+                          ("dequantize_tensor_v1", 4), ("quantize_tensor_for_all_procs", 4),
+                          ("dequantize_tensor_for_all_procs", 4)):
+        doc = getattr(mod, name).__doc__
+        assert doc.count("torch.Tensor") == tensors and "-> None" in doc, doc
+    with pytest.raises(RuntimeError, match="GPU"):
+        mod.quantize_tensor(torch.ones(2, 4), torch.zeros(4, dtype=torch.uint8), torch.zeros(2, 2), 2)
 
 
 def test_reference_build_and_drop_in_module_stay_apart_in_one_process(reference_op):
     """pybind11 keeps one module object per module name in a process, so the checker's build of the reference's
     module carries its own name: loaded in either order, it and the product's ``computation_ops`` are two modules
-    (the reference's binds the quantisation kernels too, the drop-in refuses CPU tensors; the tests of the oracle
-    call the reference's ``spmm`` on CPU tensors in this same process)."""
+    (the reference's build binds the x86 flavour of the quantisation kernels, the drop-in the flavour the trainer's
+    quantizer calls, and refuses CPU tensors; the tests of the oracle call the reference's ``spmm`` on CPU tensors in
+    this same process)."""
     import torch
 
     from gnn_benchmark_amd import ext
@@ -170,7 +180,7 @@ def test_reference_build_and_drop_in_module_stay_apart_in_one_process(reference_
         pytest.skip("the extension module is not built yet (gnn_benchmark_amd/ext/build.sh)")
     assert mod is not reference_op
     assert mod.__name__ == "computation_ops" and reference_op.__name__ == "reference_computation_ops"
-    assert hasattr(reference_op, "quantize_tensor") and not hasattr(mod, "quantize_tensor")
+    assert hasattr(reference_op, "quantize_tensor_v2_torch") and not hasattr(mod, "quantize_tensor_v2_torch")
     empty = torch.empty(0, dtype=torch.int32)
     with pytest.raises(RuntimeError, match="GPU"):   # the drop-in has no CPU path (the reference's module computes)
         mod.spmm(torch.tensor([0, 1]), torch.tensor([0]), torch.ones(1), torch.ones(1, 4), torch.zeros(1, 4), 1, empty,
