@@ -165,25 +165,24 @@ hipError_t enable_long_rows_lds() {
     if (e == hipSuccess) e = allow_long_rows_lds_fixed_width<16>();
     if (e == hipSuccess) e = allow_long_rows_lds_fixed_width<32>();
     if (e == hipSuccess) e = allow_long_rows_lds_fixed_width<64>();
-    if (e == hipSuccess) e = allow_long_rows_lds_fixed_width<128>();
-    if (e == hipSuccess) e = allow_long_rows_lds_fixed_width<256>();
     return e;
 }
 
 // What a stored element costs a row of the block-per-row kernel, by tile width (ns, measured on a 200 000-element
 // row): the chain itself does not depend on the width, but a wider tile means a shorter chunk (a tile buffer holds
-// 8192 floats), and with two chunks in flight a short chunk no longer covers the memory round trip.
+// 6144 floats), and with two chunks in flight a short chunk no longer covers the memory round trip.  Two blocks
+// share a compute unit; they slow each other down by about what the second one adds, so the model counts one.
 struct LongTileCost { int tile; double ns_per_element; };
-constexpr LongTileCost kLongTileCosts[] = {{16, 6.0}, {32, 7.5}, {64, 12.5}, {128, 34.0}, {256, 70.0}};
+constexpr LongTileCost kLongTileCosts[] = {{16, 5.5}, {32, 6.8}, {64, 14.7}};
 constexpr double kComputeUnits = 256.0;
 
 template <int VEC>
 hipError_t launch_long_rows(const LongArgs &a, int64_t nrows, int64_t longest, int64_t elems, hipStream_t st) {
     LongArgs args = a;
-    // Every feature's chain is its own, so a row can be cut along the features into tiles of 16 .. 256 floats, one
+    // Every feature's chain is its own, so a row can be cut along the features into tiles of 16 .. 64 floats, one
     // block each.  The launch lasts as long as the longest row's block, or as long as all blocks take on all compute
     // units (rows are handed out longest first): the tile width is the one for which the larger of the two is smallest.
-    int tile = kLongFeatTile;
+    int tile = kLongTileCosts[0].tile;
     double best = 0.0;
     for (const LongTileCost &c : kLongTileCosts) {
         const double tiles = (double)((a.feat + c.tile - 1) / c.tile);
@@ -208,7 +207,7 @@ hipError_t launch_long_rows(const LongArgs &a, int64_t nrows, int64_t longest, i
     args.tiles = (int)tiles;
     if (nrows * (int64_t)tiles >= (int64_t(1) << 31)) return hipErrorInvalidValue;
     const dim3 grid((unsigned)(nrows * (int64_t)tiles));
-    const dim3 block((unsigned)(kLongFetchThreads + 64 * ((tile + 63) / 64)));  // fetch waves + one chain wave per 64 features
+    const dim3 block((unsigned)(kLongFetchThreads + 64));  // fetch waves + the chain wave
     if (VEC == 4 && slots > 1024 && a.feat % tile == 0 && tile >= 16 && (tile & (tile - 1)) == 0) {
         // every tile has the same power-of-two width: the instance that knows it at compile time
 #define GNNAGG_LONG_FIXED(W)                                                                                     \
@@ -217,8 +216,6 @@ hipError_t launch_long_rows(const LongArgs &a, int64_t nrows, int64_t longest, i
         GNNAGG_LONG_FIXED(16);
         GNNAGG_LONG_FIXED(32);
         GNNAGG_LONG_FIXED(64);
-        GNNAGG_LONG_FIXED(128);
-        GNNAGG_LONG_FIXED(256);
 #undef GNNAGG_LONG_FIXED
         return hipGetLastError();
     }
@@ -335,7 +332,7 @@ struct gnnagg_plan {
     int64_t rows = 0, cols = 0, nnz = 0;
     int huge_thresh = 0;      // rows longer than this run in the block-per-row kernel
     int64_t nhuge = 0;        // such rows (the first nhuge tasks)
-    int64_t huge_elems = 0;   // upper bound of the stored elements in them (class counts x the classes' upper ends)
+    int64_t huge_elems = 0;   // the stored elements in them (exact for up to 65536 such rows, else the class counts x the classes' upper ends)
     int long_thresh = 0;      // rows longer than this get a lane group of their own (head region)
     int64_t nlong = 0;        // such rows, the huge ones included (the first nlong tasks)
     int64_t nempty = 0;       // rows with no stored element (the last nempty entries of perm)
@@ -571,6 +568,13 @@ extern "C" int gnnagg_plan_create_ex(const int64_t *rowptr, const int64_t *col, 
     for (int c = degree_class(kShortRowLen); c < kEmptyClass; ++c) p->nshort += (int64_t)h_out.class_count[c];
     if (p->long_thresh < kShortRowLen) p->nshort = 0;  // (such rows sit in the head region then)
     if (p->nhuge > 0) {
+        // the elements in those rows exactly, when the rows are few enough to look at (they head the schedule)
+        if (p->nhuge <= 65536) {
+            std::vector<RowTask> head((size_t)p->nhuge);
+            GNNAGG_HIP(hipMemcpy(head.data(), p->task, head.size() * sizeof(RowTask), hipMemcpyDeviceToHost));
+            p->huge_elems = 0;
+            for (const RowTask &t : head) p->huge_elems += t.len;
+        }
         GNNAGG_HIP(enable_long_rows_lds());
         GNNAGG_HIP(hipStreamCreateWithFlags(&p->side, hipStreamNonBlocking));
         GNNAGG_HIP(hipEventCreateWithFlags(&p->fork, hipEventDisableTiming));

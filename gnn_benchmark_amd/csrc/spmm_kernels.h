@@ -670,11 +670,11 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
 
 
 // ---------------------------------------------------------------------------------------
-// Very long rows.  One block per (row, feature tile of 16 .. 256 floats): four FETCH waves and,
-// behind them, one CHAIN wave per 64 features of the tile.  The row's chain must stay
+// Very long rows.  One block per (row, feature tile of 16 .. 64 floats): four FETCH waves and,
+// behind them, one CHAIN wave.  The row's chain must stay
 // sequential (bit-identical results), so what is parallelised is the fetch: the fetch waves
 // gather a chunk of dense rows at once (up to 8 vector loads per thread and chunk) and land it
-// in LDS, while in the chain waves the lane that owns a feature runs the FMA chain over the
+// in LDS, while in the chain wave the lane that owns a feature runs the FMA chain over the
 // chunk landed before, in CSR order, and does nothing else.  A chunk lies TRANSPOSED in LDS --
 // tile[feature][element of the chunk] -- so that the owner of a feature reads four consecutive
 // elements with one 16-byte LDS read, and the four matrix values that go with them with
@@ -683,18 +683,19 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
 // chain, 3.7 ns with these reads (sixteen and sixteen requested ahead of their 64 FMAs), 3.9 ns
 // with the matrix value handed round by v_readlane instead, 5.8 ns with a 4-byte LDS read per
 // element on top of that.  A row advances by one chunk per memory round trip, so the chunk is
-// made as long as a tile buffer allows -- 32 rows of 256 floats, 512 rows of 16 -- and with few
-// such rows the host cuts them into narrow feature tiles (every feature's chain is its own),
-// which also spreads one row's fetch over several compute units.  kLongDepth chunks are in
+// made as long as a tile buffer allows -- 128 rows of 64 floats, 512 rows of 16 -- and the host
+// cuts the rows into narrow feature tiles (every feature's chain is its own), which also
+// spreads one row's fetch over several compute units.  kLongDepth chunks are in
 // flight in registers; the (col, val) pairs come in super-chunks of kLongDepth chunks, two
 // super-chunks ahead.
 // ---------------------------------------------------------------------------------------
-constexpr int kLongTileFloats = 8192;  // most floats of one chunk (tile width x rows of the chunk)
-constexpr int kLongMaxChunk = 512;     // most dense rows gathered per chunk
+constexpr int kLongTileFloats = 6144;  // most floats of one chunk (tile width x rows of the chunk)
+constexpr int kLongMaxChunk = 384;     // most dense rows gathered per chunk
 constexpr int kLongRowPad = 4;         // floats between the feature rows of a tile buffer: lanes f, f + 1, ... read
                                        // 16 bytes each at a stride of chunk + 4 floats, 16 lanes covering all banks
-constexpr int kLongFeatTile = 256;     // most features per block
-constexpr int kLongFetchThreads = 256; // the fetch waves of a block; behind them one chain wave per 64 features
+constexpr int kLongFeatTile = 64;      // most features per block: one chain wave (wider tiles mean shorter chunks, which
+                                       // two chunks in flight no longer cover: 34 ns per element at 128 floats, 70 at 256)
+constexpr int kLongFetchThreads = 256; // the fetch waves of a block; behind them the chain wave
 // floats of one tile buffer: width x (chunk + pad) <= kLongTileFloats + kLongFeatTile * kLongRowPad, and four
 // floats behind them where the fetch slots past a chunk's rows land
 constexpr int kLongDump = kLongTileFloats + kLongFeatTile * kLongRowPad;
@@ -830,7 +831,7 @@ __global__ __launch_bounds__(kLongFetchThreads + kLongFeatTile) void spmm_long_r
 
     float *dst = a.dst + (size_t)d.row * (size_t)(a.ldd ? a.ldd : F) + f0;
 
-    // Threads 256 and up are the chain waves, one lane per feature of the tile; they fetch nothing.  Both kinds of
+    // Threads 256 and up are the chain wave, one lane per feature of the tile; it fetches nothing.  Both kinds of
     // wave pass the same barriers: two in the prologue, one per chunk.
     if (t >= 256) {
         const int f = t - 256;
@@ -893,7 +894,7 @@ __global__ __launch_bounds__(kLongFetchThreads + kLongFeatTile) void spmm_long_r
             // (1) chunk k left its registers for LDS in the step before: request chunk k + D into them
             //     (past the row's end: the last chunk once more, never landed where it is read)
             request(k + D < nchunks ? k + D : nchunks - 1, g[u]);
-            // (2) land chunk k + 1 (requested D - 1 steps ago) in the tile buffer the chain waves are not reading
+            // (2) land chunk k + 1 (requested D - 1 steps ago) in the tile buffer the chain wave is not reading
             land(k + 1, g[(u + 1) % D]);
             if (u == D - 1) {
 #pragma unroll
