@@ -683,7 +683,7 @@ __global__ __launch_bounds__(256) void spmm_tasks_kernel(const SpmmArgs a) {
 // chain, 3.7 ns with these reads (sixteen and sixteen requested ahead of their 64 FMAs), 3.9 ns
 // with the matrix value handed round by v_readlane instead, 5.8 ns with a 4-byte LDS read per
 // element on top of that.  A row advances by one chunk per memory round trip, so the chunk is
-// made as long as a tile buffer allows -- 128 rows of 64 floats, 512 rows of 16 -- and the host
+// made as long as a tile buffer allows -- 96 rows of 64 floats, 384 rows of 16 -- and the host
 // cuts the rows into narrow feature tiles (every feature's chain is its own), which also
 // spreads one row's fetch over several compute units.  kLongDepth chunks are in
 // flight in registers; the (col, val) pairs come in super-chunks of kLongDepth chunks, two
