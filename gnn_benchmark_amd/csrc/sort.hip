@@ -325,12 +325,20 @@ __global__ __launch_bounds__(256) void argsort_prepare_kernel(const int64_t *__r
         idx[i] = (uint32_t)i;
         if (v > 0 && (unsigned long long)v > m) m = (unsigned long long)v;
     }
-    // one atomic per wave, not per thread: all of them land on one address
+    // one atomic per block, not per thread: all of them land on one address
+    __shared__ unsigned long long wave_m[4];
+    __shared__ unsigned int wave_neg[4];
     m = wave_max_u64(m);
     const bool any_neg = __builtin_amdgcn_ballot_w64(neg) != 0;
     if ((threadIdx.x & 63) == 0) {
+        wave_m[threadIdx.x >> 6] = m;
+        wave_neg[threadIdx.x >> 6] = any_neg ? 1u : 0u;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 4; ++w) m = wave_m[w] > m ? wave_m[w] : m;
         if (m) atomicMax(max_key, m);
-        if (any_neg) atomicOr(negative, 1u);
+        if (wave_neg[0] | wave_neg[1] | wave_neg[2] | wave_neg[3]) atomicOr(negative, 1u);
     }
 }
 
@@ -438,7 +446,7 @@ extern "C" int gnnagg_argsort_i64(const int64_t *x, int64_t n, int64_t *perm, in
     uint32_t *idx_a = ws.take<uint32_t>((size_t)n), *idx_b = ws.take<uint32_t>((size_t)n);
     unsigned long long *flags = ws.take<unsigned long long>(2);  // [0] the largest key, [1] whether a key was negative
     void *sort_ws = ws.take<char>(sort_pairs_workspace_bytes(n));
-    const unsigned grid = (unsigned)std::min<int64_t>((n + 255) / 256, 256 * 32);
+    const unsigned grid = (unsigned)std::min<int64_t>((n + 255) / 256, 256 * 4);
     hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(64), 0, st, reinterpret_cast<uint32_t *>(flags), 4, 0u);
     hipLaunchKernelGGL(argsort_prepare_kernel, dim3(grid), dim3(256), 0, st, x, n, key_a, idx_a, flags,
                        reinterpret_cast<unsigned int *>(flags + 1));
