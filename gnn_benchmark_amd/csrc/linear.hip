@@ -889,6 +889,22 @@ __global__ __launch_bounds__(256) void pack_keep_bits_kernel(const uint8_t *__re
     bits[i] = w;
 }
 
+// the same for rows of whole words on a 16-byte boundary: the word's 32 bytes arrive as two 16-byte loads
+__global__ __launch_bounds__(256) void pack_keep_bits_aligned_kernel(const uint4 *__restrict__ keep,
+                                                                     uint32_t *__restrict__ bits, int64_t total) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const uint4 lo = keep[2 * i], hi = keep[2 * i + 1];
+    const uint32_t part[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    uint32_t w = 0;
+#pragma unroll
+    for (int p = 0; p < 8; ++p)
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+            if ((part[p] >> (8 * b)) & 0xffu) w |= 1u << (4 * p + b);
+    bits[i] = w;
+}
+
 }  // namespace
 }  // namespace gnnagg
 
@@ -904,8 +920,13 @@ extern "C" int gnnagg_pack_keep_bits(const void *keep, uint32_t *bits, int64_t r
     GNNAGG_REQUIRE(keep && bits, "null keep/bits");
     const int words = (int)((feat + 31) / 32);
     const int64_t total = rows * words;
-    hipLaunchKernelGGL(pack_keep_bits_kernel, dim3(grid_for(total, 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
-                       static_cast<const uint8_t *>(keep), bits, (int)feat, words, total);
+    if (feat % 32 == 0 && reinterpret_cast<uintptr_t>(keep) % 16 == 0)
+        hipLaunchKernelGGL(pack_keep_bits_aligned_kernel, dim3(grid_for(total, 256)), dim3(256), 0,
+                           static_cast<hipStream_t>(stream), static_cast<const uint4 *>(keep), bits, total);
+    else
+        hipLaunchKernelGGL(pack_keep_bits_kernel, dim3(grid_for(total, 256)), dim3(256), 0,
+                           static_cast<hipStream_t>(stream), static_cast<const uint8_t *>(keep), bits, (int)feat, words,
+                           total);
     GNNAGG_HIP(hipGetLastError());
     return GNNAGG_OK;
 }

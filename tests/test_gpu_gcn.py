@@ -636,3 +636,23 @@ def test_layer_kernels_walk_several_tiles_per_block(form, rows, k, n):
     # no bias, no mask, no divisor, no ReLU: the bare product (what the input-gradient product runs)
     bare = gcn._fused_product(x, w, None, None, None, 1.0, False, form)
     assert bool(((bare.double() - xs @ ws).abs() <= 1e-5 * (xs.abs() @ ws.abs()).clamp(min=1.0)).all())
+
+
+@pytest.mark.parametrize("feat", [32, 64, 256, 172, 47, 1])
+def test_keep_bits_are_the_mask_bytes_little_end_first(feat):
+    """``gcn.pack_keep_mask``: bit q of word w of a row is mask byte 32 w + q (any non-zero byte counts); widths of
+    whole words on a 16-byte boundary take the 16-byte-load kernel, others and unaligned views the byte one."""
+    rng = np.random.default_rng(feat)
+    rows = 1003
+    keep = rng.integers(0, 2, (rows, feat)).astype(np.uint8) * rng.integers(1, 255, (rows, feat)).astype(np.uint8)
+    words = (feat + 31) // 32
+    padded = np.zeros((rows, words * 32), dtype=np.uint8)
+    padded[:, :feat] = keep != 0
+    want = np.packbits(padded.reshape(rows, words, 32), axis=2, bitorder="little").view(np.uint32).reshape(rows, words)
+    got = gcn.pack_keep_mask(torch.from_numpy(keep).cuda())
+    assert np.array_equal(got.cpu().numpy().view(np.uint32).reshape(rows, words), want)
+    if feat % 32 == 0:  # the same rows one byte off the 16-byte boundary
+        shifted = torch.empty(rows * feat + 1, dtype=torch.uint8, device="cuda")[1:].view(rows, feat)
+        shifted.copy_(torch.from_numpy(keep))
+        got = gcn.pack_keep_mask(shifted)
+        assert np.array_equal(got.cpu().numpy().view(np.uint32).reshape(rows, words), want)
