@@ -269,10 +269,10 @@ __global__ __launch_bounds__(256) void classify_rows_kernel(const int64_t *__res
     __syncthreads();
     const int lane = (int)threadIdx.x & 63;
     unsigned long long longest = 0;
-    const int stride = (int)gridDim.x * 256;
+    const int64_t stride = (int64_t)gridDim.x * 256;
     // (every thread of a block makes the same number of rounds: the ballots below want whole waves)
-    for (int base = (int)blockIdx.x * 256; base < rows; base += stride) {
-        const int r = base + (int)threadIdx.x;
+    for (int64_t base = (int64_t)blockIdx.x * 256; base < rows; base += stride) {
+        const int64_t r = base + (int64_t)threadIdx.x;
         int c = -1;  // the row's class; -1: no row, or a row whose rowptr runs backwards
         if (r < rows) {
             const int64_t d = rowptr[r + 1] - rowptr[r];
@@ -284,7 +284,7 @@ __global__ __launch_bounds__(256) void classify_rows_kernel(const int64_t *__res
                 key[r] = (uint32_t)c;
                 if ((unsigned long long)d > longest) longest = (unsigned long long)d;
             }
-            rowid[r] = r;
+            rowid[r] = (int32_t)r;
         }
         // per wave one LDS atomic per class that occurs in it (its lanes found by ballots over the class's bits)
         uint64_t same = __builtin_amdgcn_ballot_w64(c >= 0);
